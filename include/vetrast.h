@@ -1,0 +1,210 @@
+/*
+ * vetrast — C ABI of the MI355X (gfx950) blending point rasterizer.
+ *
+ * This header is the whole drop-in boundary: plain pointers, sizes and PODs, no torch or HIP types.
+ * All `device` pointers are hipMalloc'ed (or torch-allocated) memory on the GPU the context was created
+ * on; all `host` pointers are ordinary host memory that only has to stay valid for the duration of the call.
+ * Every entry point returns 0 on success or a negative vetrast_status, never aborts, never allocates device
+ * memory behind the caller's back (the caller owns inputs, outputs and the workspace) and, unless stated
+ * otherwise, only enqueues work on the given stream (pass the hipStream_t as `void*`, NULL = default stream).
+ *
+ * The reference has no C ABI; its seam is the libtorch function
+ *   std::vector<torch::Tensor> BlendPointCloud(NeuralRenderInfo*)          src/lib/rendering/PointRenderer.h:53
+ *   torch::autograd::PointRender::forward / ::backward                      src/lib/rendering/PointRenderer.h:39-47
+ * implemented by BlendPointCloudForward / BlendPointCloudBackward            src/lib/rendering/PointRenderer.cu:657,1111
+ * The entry points below are what a libtorch shim with that signature binds (see vet_amd/torch_ext).
+ */
+#ifndef VETRAST_H
+#define VETRAST_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define VETRAST_MAX_LAYERS 5   /* max_layers, src/lib/rendering/RenderConstants.h:33 */
+#define VETRAST_MAX_CHANNELS 4 /* CUDA_KERNEL_ASSERT(num_texture_channels <= 4), src/lib/rendering/RenderForward.cu:1322 */
+
+typedef enum vetrast_status
+{
+    VETRAST_OK                  = 0,
+    VETRAST_ERR_INVALID_ARG     = -1, /* null pointer, size out of range, misaligned workspace */
+    VETRAST_ERR_WORKSPACE_SMALL = -2, /* workspace_bytes below vetrast_forward_workspace_bytes() */
+    VETRAST_ERR_HIP             = -3, /* a HIP runtime call failed; see vetrast_last_hip_error() */
+    VETRAST_ERR_UNSUPPORTED     = -4, /* a reference feature outside the blending path (OCam, normals, ...) */
+    VETRAST_ERR_BAD_INPUT_DATA  = -5  /* device-side check failed (non-zero distortion), from vetrast_query_device_flags */
+} vetrast_status;
+
+/* Camera model tag of a view. Mirrors enum CameraModel, src/lib/data/SceneData.h:30-35.
+ * Only PINHOLE_DISTORTION with all eight distortion coefficients equal to zero is implemented. */
+#define VETRAST_CAMERA_PINHOLE_DISTORTION 0
+#define VETRAST_CAMERA_OCAM 1
+#define VETRAST_CAMERA_SPHERICAL 2
+
+/* One view of the batch. Mirrors struct ReducedImageInfo, src/lib/data/SceneData.h:39-50, field by field
+ * (the Eigen members are spelled out as floats). The reference passes it by value as a kernel argument
+ * (CountingPrepassMulti, src/lib/rendering/RenderForward.cu:807); so does this library. */
+typedef struct vetrast_view
+{
+    int32_t w, h;              /* full-resolution size of layer 0; must be equal for all views of a call */
+    int32_t image_index;       /* row of poses_se3 / pose gradient */
+    int32_t camera_index;      /* row of intrinsics / intrinsics gradient */
+    int32_t camera_model_type; /* VETRAST_CAMERA_* */
+    float crop_transform[5];   /* fx, fy, cx, cy, s of IntrinsicsPinholef crop_transform */
+    float crop_rotation[4];    /* r00, r01, r10, r11 (row-major; Eigen stores the 2x2 column-major) */
+} vetrast_view;
+
+/* Scalar parameters of the path. Mirrors the RenderParams fields the blending path reads
+ * (src/lib/data/Settings.h:19-93, copied into DeviceRenderParams at src/lib/rendering/RenderConstants.h:105-126). */
+typedef struct vetrast_params
+{
+    int32_t num_texture_channels;         /* C, 1..4 */
+    int32_t num_layers;                   /* L, 1..5  (NeuralRenderInfo::num_layers) */
+    int32_t debug_max_list_length;        /* K; <= 0 means no cut (reference default -1) */
+    int32_t use_environment_map;          /* 0: the background colour is blended behind the last fragment */
+    int32_t need_point_gradient;          /* backward: compute the position gradient */
+    int32_t viewer_only;                  /* with it, points with confidence < stability_cutoff_value are skipped */
+    float stability_cutoff_value;
+    int32_t drop_out_points_by_radius;    /* stop descending layers once the splat radius falls below the threshold */
+    float drop_out_radius_threshold;
+    int32_t output_background_mask;       /* forward also writes out_mask = (weight == 0 ? mask_value : 1) */
+    float output_background_mask_value;
+    int32_t check_normal;                 /* must be 0 (needs saiga's UnpackNormal10Bit) */
+    /* Two switches for behaviours of the reference that are accidents of its implementation: */
+    int32_t quirk_background_confidence_leak; /* 1: the background pseudo-fragment also adds its alpha gradient to
+                                                 grad_confidence[0], as src/lib/rendering/RenderBackward.cu:1157 does */
+    int32_t point_gradient_normalization;     /* 0: leave sums and counts; 1: row i / count i;
+                                                 2: literal reference (vec3 stride over the [N,4] buffer,
+                                                 src/lib/rendering/PointRenderer.cu:1278-1279) */
+} vetrast_params;
+
+typedef struct vetrast_ctx vetrast_ctx;
+
+/* Per-kernel timing scopes, named after the reference's CudaTimerSystem scopes
+ * (src/lib/rendering/PointRenderer.cu:249,770,791,843,872,886,1222,1252). */
+typedef enum vetrast_scope
+{
+    VETRAST_SCOPE_PREPARE = 0,      /* "Build Cache": zero-fill, view preparation, descriptor interleave */
+    VETRAST_SCOPE_COUNT,            /* "CountingPass" */
+    VETRAST_SCOPE_SCAN,             /* "CreateAndAllocateBuffers" (prefix scan; no allocation here) */
+    VETRAST_SCOPE_FILL,             /* "CollectionPass" */
+    VETRAST_SCOPE_SORT,             /* "SortingPass" */
+    VETRAST_SCOPE_BLEND,            /* "BlendingPass" */
+    VETRAST_SCOPE_BACKWARD_PREPARE, /* "Prepare Backward": zero-fill of gradient buffers */
+    VETRAST_SCOPE_BACKWARD_BLEND,   /* "BlendBackwards" */
+    VETRAST_SCOPE_BACKWARD_POST,    /* "Post Process Gradient" */
+    VETRAST_SCOPE_COUNT_
+} vetrast_scope;
+
+/* Byte offsets of the arrays inside the forward workspace, so that a caller (or a test) can read the
+ * per-pixel fragment lists. Pixels of all layers are numbered consecutively: q = layer_pixel_base[l] + y*w_l + x. */
+typedef struct vetrast_workspace_layout
+{
+    int32_t layer_w[VETRAST_MAX_LAYERS];
+    int32_t layer_h[VETRAST_MAX_LAYERS];
+    int64_t layer_pixel_base[VETRAST_MAX_LAYERS + 1]; /* [L] = total pixel count P of one view */
+    int64_t fragment_capacity;                        /* N * L, the per-view upper bound on fragments */
+    size_t total_bytes;
+    /* per-view arrays: offset of view b = base + b * stride */
+    size_t offsets_base, offsets_stride;     /* uint32 [P+1]: exclusive scan of per-pixel counts; [P] = fragments of the view */
+    size_t fragments_base, fragments_stride; /* uint64 [N*L]: (depth_bits << 32) | point_id, per pixel ascending; only the
+                                                first min(count, K) entries of a pixel's list are sorted and meaningful */
+    size_t transmittance_base, transmittance_stride; /* float [N*L]: transmittance in front of each kept fragment */
+    size_t weight_base, weight_stride;       /* float [P]: final transmittance per pixel (the reference's `weight` image) */
+    /* shared by all views */
+    size_t packed_base;    /* float [N][8]: descriptor (4, zero padded), confidence, 3 pad */
+    size_t slots_base;     /* uint32 [L][N]: per (layer, point) arrival rank inside its pixel, 0xFFFFFFFF = no fragment */
+    size_t views_base;     /* prepared per-view camera constants */
+    size_t scan_partials_base;
+    size_t flags_base;     /* uint32 [4] device status flags */
+} vetrast_workspace_layout;
+
+/* Arguments of the forward pass. Replaces the inputs PointRender::forward receives
+ * (src/lib/rendering/RenderInfo.cpp:25-29,34-43) plus what it reads through info->scene. */
+typedef struct vetrast_forward_args
+{
+    int32_t num_points; /* N */
+    int32_t num_views;  /* B = info->images.size() */
+    int32_t num_poses;  /* F, rows of poses_se3 */
+    int32_t num_cameras;
+    const float* position;    /* device [N,4] x,y,z,drop-out radius (t_position, src/lib/rendering/NeuralPointCloudCuda.h:193-224) */
+    const int32_t* index;     /* device [N] texture index of a point (t_index) or NULL for the identity */
+    const float* texture;     /* device [C,N] planar descriptors */
+    const float* confidence;  /* device [N] (the reference's [1,N]) already in (0,1) */
+    const float* background;  /* device [C] */
+    const float* dropout;     /* device [B,N], a point is skipped in view b where the value == 1; NULL = none */
+    const double* poses_se3;  /* device [F,8] world->camera: unit quaternion x,y,z,w, translation, 1 pad
+                                 (src/lib/data/NeuralStructure.cpp:15-28) */
+    const float* intrinsics;  /* device [num_cameras,13]: fx,fy,cx,cy,s,k1..k6,p1,p2 (src/lib/data/NeuralStructure.cpp:65-99) */
+    const vetrast_view* views; /* host [B] */
+    vetrast_params params;
+    int32_t save_for_backward; /* also store the per-fragment transmittance the backward pass reads */
+    float* out[VETRAST_MAX_LAYERS];      /* device, layer l: [B,C,h_l,w_l] contiguous NCHW; fully overwritten */
+    float* out_mask[VETRAST_MAX_LAYERS]; /* device, layer l: [B,1,h_l,w_l]; only with output_background_mask */
+    void* workspace;                     /* device, 256-byte aligned */
+    size_t workspace_bytes;
+} vetrast_forward_args;
+
+/* Arguments of the backward pass. Replaces BlendPointCloudBackward's inputs and its seven returned tensors
+ * (src/lib/rendering/PointRenderer.cu:1111-1323). The workspace and `out` must be those of the matching forward call
+ * (made with save_for_backward = 1) and unchanged since; this is the saved state of
+ * src/lib/rendering/PointRenderer.cu:1027-1059. */
+typedef struct vetrast_backward_args
+{
+    vetrast_forward_args fwd;                      /* same values as passed to vetrast_forward */
+    const float* grad_out[VETRAST_MAX_LAYERS];     /* device, layer l: [B,C,h_l,w_l] upstream gradient */
+    float* grad_texture;     /* device [C,N]; overwritten */
+    float* grad_confidence;  /* device [N]; overwritten */
+    float* grad_background;  /* device [C]; overwritten */
+    float* grad_points;      /* device [N,4] or NULL (points do not require grad); xyz sums (w stays 0); overwritten */
+    float* grad_point_count; /* device [N]; number of fragments that contributed to a point; required with grad_points */
+} vetrast_backward_args;
+
+/* Create / destroy a context bound to the current HIP device. The context owns only a few HIP events. */
+int vetrast_create(vetrast_ctx** out_ctx);
+void vetrast_destroy(vetrast_ctx* ctx);
+
+/* Layer pyramid by repeated integer halving (src/lib/rendering/PointRenderer.cu:351-381). Pure host arithmetic. */
+int vetrast_layer_sizes(int32_t w, int32_t h, int32_t num_layers, int32_t* layer_w, int32_t* layer_h);
+
+/* Size and layout of the workspace a forward call with these dimensions needs. Pure host arithmetic. The reference
+ * sizes its fragment buffers from a device->host read of the scan total (src/lib/rendering/PointRenderer.cu:811-821);
+ * here the buffer has the upper bound N*L entries per view instead, so no read-back is needed. */
+int vetrast_workspace_layout_for(int32_t num_points, int32_t num_views, int32_t num_layers, int32_t w, int32_t h,
+                                 vetrast_workspace_layout* layout);
+size_t vetrast_forward_workspace_bytes(int32_t num_points, int32_t num_views, int32_t num_layers, int32_t w, int32_t h);
+
+/* Forward: project, count, scan, fill, per-pixel sort by (depth bits, point id), top-K cut, front-to-back blend.
+ * Replaces BlendPointCloudForward in FULL_BLEND mode (src/lib/rendering/PointRenderer.cu:657-1069). */
+int vetrast_forward(vetrast_ctx* ctx, const vetrast_forward_args* args, void* stream);
+
+/* Backward: gradients to descriptors, confidence, background and point positions.
+ * Replaces BlendPointCloudBackward in FULL_BLEND mode (src/lib/rendering/PointRenderer.cu:1111-1323). */
+int vetrast_backward(vetrast_ctx* ctx, const vetrast_backward_args* args, void* stream);
+
+/* Blocking: waits for the stream, then reads the device flag word of the workspace. Returns VETRAST_OK or
+ * VETRAST_ERR_BAD_INPUT_DATA (a camera with non-zero distortion coefficients was used; the reference's saiga
+ * distortion model is not available, so such input is flagged instead of guessed). */
+int vetrast_query_device_flags(vetrast_ctx* ctx, const void* workspace, const vetrast_workspace_layout* layout,
+                               void* stream);
+
+/* Per-kernel timing, the counterpart of NeuralRenderInfo::timer_system (src/lib/rendering/PointRenderer.h:32).
+ * With profiling enabled every launch is bracketed by HIP events on the call's stream; vetrast_scope_times
+ * synchronises on them and returns, per scope, the summed kernel time in milliseconds and the number of launches
+ * since the last vetrast_reset_scope_times. */
+int vetrast_set_profiling(vetrast_ctx* ctx, int32_t enabled);
+int vetrast_reset_scope_times(vetrast_ctx* ctx);
+int vetrast_scope_times(vetrast_ctx* ctx, float* ms /* [VETRAST_SCOPE_COUNT_] */,
+                        int32_t* launches /* [VETRAST_SCOPE_COUNT_] */);
+const char* vetrast_scope_name(int32_t scope);
+
+const char* vetrast_status_string(int status);
+/* hipError_t value of the last failed HIP call of this context (0 if none). */
+int vetrast_last_hip_error(const vetrast_ctx* ctx);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* VETRAST_H */

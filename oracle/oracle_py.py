@@ -1,0 +1,138 @@
+"""ctypes wrapper of the CPU oracle (oracle/libvetrast_oracle.so) — TEST INFRASTRUCTURE ONLY.
+
+Imported by tests/, __graft_entry__.smoke() and bench.py's cpu_baseline leg; the product (vet_amd/) never imports it.
+The argument structs are the ctypes mirrors of include/vetrast.h from vet_amd.abi, filled with host pointers.
+"""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+from vet_amd import abi
+from vet_amd.rasterizer import fill_forward_args, make_params, make_views
+from vet_amd.synthetic import Scene
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "libvetrast_oracle.so")
+_lib = None
+
+
+def build():
+    subprocess.run(["make", "-C", HERE, "-B", "libvetrast_oracle.so"], check=True)
+    return LIB_PATH
+
+
+def load():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise OSError(f"{LIB_PATH} is missing: run `make -C oracle`")
+        lib = C.CDLL(LIB_PATH)
+        lib.vetref_forward.restype = C.c_int
+        lib.vetref_forward.argtypes = [C.POINTER(abi.ForwardArgs), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
+                                       C.c_int]
+        lib.vetref_backward.restype = C.c_int
+        lib.vetref_backward.argtypes = [C.POINTER(abi.BackwardArgs), C.c_void_p, C.c_void_p, C.c_int]
+        lib.vetref_prepare_view.restype = C.c_int
+        lib.vetref_prepare_view.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p]
+        lib.vetref_project_point.restype = C.c_int
+        lib.vetref_project_point.argtypes = [C.c_void_p, C.POINTER(abi.View), C.c_void_p, C.c_void_p]
+        _lib = lib
+    return _lib
+
+
+def _addr(a):
+    return None if a is None else a.ctypes.data
+
+
+class OracleForward:
+    """Result of the oracle's forward pass (numpy arrays) plus everything backward needs."""
+
+    def __init__(self, scene: Scene, params: abi.Params, num_threads=1):
+        self.scene, self.params = scene, params
+        self.views = make_views(scene)
+        B, Cn, N, L = len(scene.views), scene.num_channels, scene.num_points, scene.num_layers
+        self.sizes = scene.layer_sizes()
+        self.P = sum(w * h for w, h in self.sizes)
+        self.cap = N * L
+        self.out = [np.zeros((B, Cn, h, w), np.float32) for (w, h) in self.sizes]
+        self.out_mask = [np.zeros((B, 1, h, w), np.float32) if params.output_background_mask else None
+                         for (w, h) in self.sizes]
+        self.offsets = np.zeros((B, self.P + 1), np.uint32)
+        self.fragments = np.zeros((B, max(self.cap, 1)), np.uint64)
+        self.transmittance = np.zeros((B, max(self.cap, 1)), np.float32)
+        self.weight = np.zeros((B, self.P), np.float32)
+        self.inputs = {k: (None if getattr(scene, k) is None else np.ascontiguousarray(getattr(scene, k)))
+                       for k in ("position", "index", "texture", "confidence", "background", "dropout", "poses_se3",
+                                 "intrinsics")}
+        a = abi.ForwardArgs()
+        fill_forward_args(a, scene, params, self.views, lambda n: _addr(self.inputs[n]))
+        a.save_for_backward = 1
+        for l in range(L):
+            a.out[l] = _addr(self.out[l])
+            a.out_mask[l] = _addr(self.out_mask[l])
+        self.args = a
+        self.status = load().vetref_forward(C.byref(a), _addr(self.offsets), _addr(self.fragments),
+                                            _addr(self.transmittance), _addr(self.weight), num_threads)
+
+    def layer_base(self, l):
+        return sum(w * h for w, h in self.sizes[:l])
+
+    def pixel_list(self, b, l, x, y):
+        q = self.layer_base(l) + y * self.sizes[l][0] + x
+        o0, o1 = int(self.offsets[b, q]), int(self.offsets[b, q + 1])
+        return self.fragments[b, o0:o1]
+
+
+def forward(scene: Scene, params: abi.Params = None, num_threads=1, **overrides) -> OracleForward:
+    params = params or make_params(scene, **overrides)
+    res = OracleForward(scene, params, num_threads)
+    if res.status != 0:
+        raise abi.VetrastError(res.status, "oracle forward")
+    return res
+
+
+def backward(fwd: OracleForward, grad_out, want_points=True, num_threads=1, **param_overrides):
+    scene = fwd.scene
+    N, Cn = scene.num_points, scene.num_channels
+    g = abi.BackwardArgs()
+    C.memmove(C.byref(g.fwd), C.byref(fwd.args), C.sizeof(abi.ForwardArgs))
+    for k, v in param_overrides.items():
+        setattr(g.fwd.params, k, v)
+    go = [np.ascontiguousarray(t, dtype=np.float32) for t in grad_out]
+    for l, t in enumerate(go):
+        g.grad_out[l] = _addr(t)
+    res = {
+        "texture": np.zeros((Cn, N), np.float32),
+        "confidence": np.zeros((N,), np.float32),
+        "background": np.zeros((Cn,), np.float32),
+    }
+    g.grad_texture = _addr(res["texture"])
+    g.grad_confidence = _addr(res["confidence"])
+    g.grad_background = _addr(res["background"])
+    if want_points:
+        res["points"] = np.zeros((N, 4), np.float32)
+        res["point_count"] = np.zeros((N,), np.float32)
+        g.grad_points = _addr(res["points"])
+        g.grad_point_count = _addr(res["point_count"])
+    st = load().vetref_backward(C.byref(g), _addr(fwd.offsets), _addr(fwd.fragments), num_threads)
+    if st != 0:
+        raise abi.VetrastError(st, "oracle backward")
+    return res
+
+
+def prepare_view(pose8, intrinsics13):
+    out = np.zeros(17, np.float32)
+    p = np.ascontiguousarray(pose8, np.float64)
+    k = np.ascontiguousarray(intrinsics13, np.float32)
+    load().vetref_prepare_view(_addr(p), _addr(k), _addr(out))
+    return out
+
+
+def project_point(prepared17, view: abi.View, position4):
+    out = np.zeros(4, np.float32)
+    m = np.ascontiguousarray(prepared17, np.float32)
+    p = np.ascontiguousarray(position4, np.float32)
+    ok = load().vetref_project_point(_addr(m), C.byref(view), _addr(p), _addr(out))
+    return bool(ok), out

@@ -1,0 +1,572 @@
+// CPU oracle of the blending point rasterizer — TEST INFRASTRUCTURE ONLY (see vetrast_oracle.h).
+//
+// Scalar restatement of the reference's FULL_BLEND path. Every function names the reference lines it follows
+// (paths relative to the reference's src/lib/). Build with -ffp-contract=off: the canonical arithmetic has no
+// fused multiply-add, every operation is rounded on its own, in the order written here.
+#include "vetrast_oracle.h"
+
+#include <algorithm>
+#include <cmath>
+#include <cstring>
+#include <vector>
+
+#ifdef _OPENMP
+#    include <omp.h>
+#endif
+
+namespace
+{
+struct Prepared
+{
+    float r[9];  // row-major rotation, world -> camera
+    float t[3];
+    float fx, fy, cx, cy, s;
+};
+
+struct Layers
+{
+    int L;
+    int w[VETRAST_MAX_LAYERS], h[VETRAST_MAX_LAYERS];
+    int64_t base[VETRAST_MAX_LAYERS + 1];
+};
+
+// Layer pyramid: repeated integer halving. rendering/PointRenderer.cu:351-381
+Layers make_layers(int w, int h, int L)
+{
+    Layers ly;
+    ly.L       = L;
+    ly.base[0] = 0;
+    for (int l = 0; l < L; ++l)
+    {
+        ly.w[l]        = w;
+        ly.h[l]        = h;
+        ly.base[l + 1] = ly.base[l] + (int64_t)w * h;
+        w /= 2;
+        h /= 2;
+    }
+    return ly;
+}
+
+// Pose: the reference keeps Sophus::SE3d (unit quaternion x,y,z,w + translation) and casts it to float per use
+// (rendering/RenderConstants.h:78, data/NeuralStructure.cpp:15-28). Canon: rotation matrix from the quaternion in
+// double (the usual 2xy-2wz form), then one rounding to float.
+Prepared prepare(const double* q, const float* intr)
+{
+    Prepared p;
+    const double x = q[0], y = q[1], z = q[2], w = q[3];
+    const double tx = 2.0 * x, ty = 2.0 * y, tz = 2.0 * z;
+    const double twx = tx * w, twy = ty * w, twz = tz * w;
+    const double txx = tx * x, txy = ty * x, txz = tz * x;
+    const double tyy = ty * y, tyz = tz * y, tzz = tz * z;
+    p.r[0] = (float)(1.0 - (tyy + tzz));
+    p.r[1] = (float)(txy - twz);
+    p.r[2] = (float)(txz + twy);
+    p.r[3] = (float)(txy + twz);
+    p.r[4] = (float)(1.0 - (txx + tzz));
+    p.r[5] = (float)(tyz - twx);
+    p.r[6] = (float)(txz - twy);
+    p.r[7] = (float)(tyz + twx);
+    p.r[8] = (float)(1.0 - (txx + tyy));
+    p.t[0] = (float)q[4];
+    p.t[1] = (float)q[5];
+    p.t[2] = (float)q[6];
+    p.fx   = intr[0];
+    p.fy   = intr[1];
+    p.cx   = intr[2];
+    p.cy   = intr[3];
+    p.s    = intr[4];
+    return p;
+}
+
+bool distortion_is_zero(const float* intr)
+{
+    for (int k = 5; k < 13; ++k)
+        if (intr[k] != 0.f) return false;
+    return true;
+}
+
+struct Projected
+{
+    float ipx, ipy, z, radius;
+};
+
+// ProjPoint + ProjectPointPinhole + rotateCropAroundCenter. rendering/RenderForward.cu:110-158,
+// rendering/PointRendererHelper.h:184-218. Zero distortion only, so distortNormalizedPoint is the identity.
+// Returns false when the point is rejected (z == 0 after the clamp, RenderForward.cu:852).
+bool project(const Prepared& c, const vetrast_view& v, const float* p4, Projected& o)
+{
+    const float x = p4[0], y = p4[1], zz = p4[2];
+    const float vx = ((c.r[0] * x + c.r[1] * y) + c.r[2] * zz) + c.t[0];
+    const float vy = ((c.r[3] * x + c.r[4] * y) + c.r[5] * zz) + c.t[1];
+    const float vz = ((c.r[6] * x + c.r[7] * y) + c.r[8] * zz) + c.t[2];
+    float z        = std::fmax(vz, 0.f);  // PointRendererHelper.h:191-192
+    if (!(z > 0.f)) return false;        // z == 0 (also NaN)
+    const float nx = vx / vz;             // DivideByZ, PointRendererHelper.h:205
+    const float ny = vy / vz;
+    const float u  = (c.fx * nx + c.s * ny) + c.cx;  // K.normalizedToImage, PointRendererHelper.h:214
+    const float w  = c.fy * ny + c.cy;
+    const float* k = v.crop_transform;
+    float ipx      = (k[0] * u + k[4] * w) + k[2];  // crop_transform.normalizedToImage, RenderForward.cu:155
+    float ipy      = k[1] * w + k[3];
+    const float ccx = (float)(v.w / 2), ccy = (float)(v.h / 2);  // integer halves, RenderForward.cu:156
+    const float dx = ipx - ccx, dy = ipy - ccy;
+    const float rx = v.crop_rotation[0] * dx + v.crop_rotation[1] * dy;  // RenderForward.cu:110-116
+    const float ry = v.crop_rotation[2] * dx + v.crop_rotation[3] * dy;
+    o.ipx          = rx + ccx;
+    o.ipy          = ry + ccy;
+    o.z            = z;
+    o.radius       = ((c.fx * k[0]) * p4[3]) / z;  // RenderForward.cu:132
+    return true;
+}
+
+inline uint32_t float_bits(float f)
+{
+    uint32_t u;
+    std::memcpy(&u, &f, 4);
+    return u;
+}
+
+// Visits the pixel a point lands in, layer by layer. The loop of CountingPrepassMulti / CollectMulti:
+// rendering/RenderForward.cu:855-903 and :1075-1096. __float2int_rn = round half to even = rintf in the default mode.
+template <class F>
+inline void for_each_layer_pixel(const Projected& pr, const Layers& ly, const vetrast_params& prm, F&& fn)
+{
+    float ipx = pr.ipx, ipy = pr.ipy, radius = pr.radius;
+    for (int l = 0; l < ly.L; ++l, radius *= 0.5f, ipx *= 0.5f, ipy *= 0.5f)
+    {
+        if (prm.drop_out_points_by_radius && radius < prm.drop_out_radius_threshold) break;
+        const float fx = std::rint(ipx), fy = std::rint(ipy);
+        // inImage2(y, x): 0 <= x < w and 0 <= y < h
+        if (!(fx >= 0.f && fx < (float)ly.w[l] && fy >= 0.f && fy < (float)ly.h[l])) continue;
+        fn(l, (int)fx, (int)fy);
+    }
+}
+
+struct Scene
+{
+    const vetrast_forward_args* a;
+    Layers ly;
+    int64_t P;
+    int64_t cap;
+    std::vector<Prepared> cams;
+};
+
+int validate(const vetrast_forward_args* a)
+{
+    if (!a || !a->position || !a->texture || !a->confidence || !a->background || !a->poses_se3 || !a->intrinsics ||
+        !a->views)
+        return VETRAST_ERR_INVALID_ARG;
+    const vetrast_params& p = a->params;
+    if (a->num_points < 0 || a->num_views < 1) return VETRAST_ERR_INVALID_ARG;
+    if (p.num_layers < 1 || p.num_layers > VETRAST_MAX_LAYERS) return VETRAST_ERR_INVALID_ARG;
+    if (p.num_texture_channels < 1 || p.num_texture_channels > VETRAST_MAX_CHANNELS) return VETRAST_ERR_INVALID_ARG;
+    if (p.check_normal) return VETRAST_ERR_UNSUPPORTED;
+    for (int b = 0; b < a->num_views; ++b)
+    {
+        const vetrast_view& v = a->views[b];
+        if (v.camera_model_type != VETRAST_CAMERA_PINHOLE_DISTORTION) return VETRAST_ERR_UNSUPPORTED;
+        if (v.w != a->views[0].w || v.h != a->views[0].h || v.w < 1 || v.h < 1) return VETRAST_ERR_INVALID_ARG;
+        if (v.image_index < 0 || v.image_index >= a->num_poses) return VETRAST_ERR_INVALID_ARG;
+        if (v.camera_index < 0 || v.camera_index >= a->num_cameras) return VETRAST_ERR_INVALID_ARG;
+        if (!distortion_is_zero(a->intrinsics + 13 * (size_t)v.camera_index)) return VETRAST_ERR_BAD_INPUT_DATA;
+    }
+    return VETRAST_OK;
+}
+
+Scene make_scene(const vetrast_forward_args* a)
+{
+    Scene s;
+    s.a   = a;
+    s.ly  = make_layers(a->views[0].w, a->views[0].h, a->params.num_layers);
+    s.P   = s.ly.base[s.ly.L];
+    s.cap = (int64_t)a->num_points * a->params.num_layers;
+    for (int b = 0; b < a->num_views; ++b)
+    {
+        const vetrast_view& v = a->views[b];
+        s.cams.push_back(prepare(a->poses_se3 + 8 * (size_t)v.image_index, a->intrinsics + 13 * (size_t)v.camera_index));
+    }
+    return s;
+}
+
+// Point skipping shared by the counting and the collection pass: rendering/RenderForward.cu:829-833,168-176.
+inline bool point_skipped(const vetrast_forward_args* a, int b, int i)
+{
+    if (a->dropout && a->dropout[(size_t)b * a->num_points + i] == 1.f) return true;
+    const int ti = a->index ? a->index[i] : i;
+    if (a->params.viewer_only && a->confidence[ti] < a->params.stability_cutoff_value) return true;
+    return false;
+}
+
+// compute_blend / compute_new_alphadest. rendering/PointBlending.h:90-94,116-119
+inline float compute_blend(float alpha_dest, float alpha_s, float color, float color_dest)
+{
+    return alpha_dest * alpha_s * color + color_dest;  // (alpha_dest*alpha_s)*color, then + dest; no contraction
+}
+inline float compute_new_alphadest(float alphadest_old, float alpha_s)
+{
+    return (1 - alpha_s) * alphadest_old;
+}
+
+inline void atomic_add(float* p, float v, bool parallel)
+{
+    if (parallel)
+    {
+#pragma omp atomic
+        *p += v;
+    }
+    else
+        *p += v;
+}
+
+}  // namespace
+
+extern "C" int vetref_prepare_view(const double* pose8, const float* intrinsics13, float* out17)
+{
+    Prepared p = prepare(pose8, intrinsics13);
+    for (int r = 0; r < 3; ++r)
+    {
+        for (int c = 0; c < 3; ++c) out17[4 * r + c] = p.r[3 * r + c];
+        out17[4 * r + 3] = p.t[r];
+    }
+    out17[12] = p.fx;
+    out17[13] = p.fy;
+    out17[14] = p.cx;
+    out17[15] = p.cy;
+    out17[16] = p.s;
+    return 0;
+}
+
+extern "C" int vetref_project_point(const float* m, const vetrast_view* view, const float* position4, float* ip_z_r)
+{
+    Prepared p;
+    for (int r = 0; r < 3; ++r)
+    {
+        for (int c = 0; c < 3; ++c) p.r[3 * r + c] = m[4 * r + c];
+        p.t[r] = m[4 * r + 3];
+    }
+    p.fx = m[12];
+    p.fy = m[13];
+    p.cx = m[14];
+    p.cy = m[15];
+    p.s  = m[16];
+    Projected o;
+    if (!project(p, *view, position4, o)) return 0;
+    ip_z_r[0] = o.ipx;
+    ip_z_r[1] = o.ipy;
+    ip_z_r[2] = o.z;
+    ip_z_r[3] = o.radius;
+    return 1;
+}
+
+// Forward pass. Host sequence of BlendPointCloudForward, rendering/PointRenderer.cu:768-899:
+// counting pass, exclusive scan, collection pass, per-pixel sort, blend.
+extern "C" int vetref_forward(const vetrast_forward_args* a, uint32_t* offsets, uint64_t* fragments,
+                              float* transmittance, float* weight, int num_threads)
+{
+    int st = validate(a);
+    if (st != VETRAST_OK) return st;
+    if (!offsets || !fragments || !weight) return VETRAST_ERR_INVALID_ARG;
+    for (int l = 0; l < a->params.num_layers; ++l)
+        if (!a->out[l]) return VETRAST_ERR_INVALID_ARG;
+    Scene s                  = make_scene(a);
+    const int N              = a->num_points;
+    const int C              = a->params.num_texture_channels;
+    const int K              = a->params.debug_max_list_length;
+    const vetrast_params& pr = a->params;
+    const bool par           = num_threads > 1;
+#ifdef _OPENMP
+    omp_set_num_threads(num_threads > 0 ? num_threads : 1);
+#endif
+
+    for (int b = 0; b < a->num_views; ++b)
+    {
+        const Prepared& cam   = s.cams[b];
+        const vetrast_view& v = a->views[b];
+        uint32_t* off         = offsets + (size_t)b * (s.P + 1);
+        uint64_t* frag        = fragments + (size_t)b * s.cap;
+        float* wgt            = weight + (size_t)b * s.P;
+        std::vector<uint32_t> count((size_t)s.P, 0u), cursor((size_t)s.P, 0u);
+
+        // CountingPrepassMulti<L,false>, rendering/RenderForward.cu:806-905 (the depth atomicMin image is not
+        // read by FULL_BLEND and is not produced here).
+#pragma omp parallel for schedule(static) if (par)
+        for (int i = 0; i < N; ++i)
+        {
+            if (point_skipped(a, b, i)) continue;
+            Projected p;
+            if (!project(cam, v, a->position + 4 * (size_t)i, p)) continue;
+            for_each_layer_pixel(p, s.ly, pr, [&](int l, int x, int y) {
+                uint32_t* c = &count[(size_t)(s.ly.base[l] + (int64_t)y * s.ly.w[l] + x)];
+                if (par)
+                    __atomic_fetch_add(c, 1u, __ATOMIC_RELAXED);
+                else
+                    ++*c;
+            });
+        }
+
+        // thrust::exclusive_scan per layer, rendering/PointRenderer.cu:799-813. The layers are concatenated here,
+        // so a layer's list positions are shifted by the fragments of the finer layers; list contents are the same.
+        uint32_t run = 0;
+        for (int64_t q = 0; q < s.P; ++q)
+        {
+            off[q] = run;
+            run += count[(size_t)q];
+        }
+        off[s.P] = run;
+
+        // CollectMulti<L,false>, rendering/RenderForward.cu:1011-1096: slot = scan[pixel] + atomicAdd(counter, 1),
+        // record = (depth bits, point id).
+#pragma omp parallel for schedule(static) if (par)
+        for (int i = 0; i < N; ++i)
+        {
+            if (point_skipped(a, b, i)) continue;
+            Projected p;
+            if (!project(cam, v, a->position + 4 * (size_t)i, p)) continue;
+            const uint64_t key = ((uint64_t)float_bits(p.z) << 32) | (uint32_t)i;
+            for_each_layer_pixel(p, s.ly, pr, [&](int l, int x, int y) {
+                const size_t q = (size_t)(s.ly.base[l] + (int64_t)y * s.ly.w[l] + x);
+                uint32_t slot;
+                if (par)
+                    slot = __atomic_fetch_add(&cursor[q], 1u, __ATOMIC_RELAXED);
+                else
+                    slot = cursor[q]++;
+                frag[off[q] + slot] = key;
+            });
+        }
+
+        // SortMulti, rendering/RenderForward.cu:1277-1300 and rendering/AlphaListSort.cu:23-32: ascending depth per
+        // pixel list. The reference leaves equal depths in arrival order; the point id in the low key bits makes
+        // the order total. BlendMulti, rendering/RenderForward.cu:1303-1357.
+        for (int l = 0; l < s.ly.L; ++l)
+        {
+            const int lw = s.ly.w[l], lh = s.ly.h[l];
+            float* out = a->out[l] + (size_t)b * C * lw * lh;
+#pragma omp parallel for schedule(dynamic, 8) if (par)
+            for (int y = 0; y < lh; ++y)
+                for (int x = 0; x < lw; ++x)
+                {
+                    const size_t q   = (size_t)(s.ly.base[l] + (int64_t)y * lw + x);
+                    const uint32_t o = off[q];
+                    const int n      = (int)(off[q + 1] - o);
+                    std::sort(frag + o, frag + o + n);
+                    int size_of_chunk = n;
+                    if (K > 0) size_of_chunk = std::min(K, size_of_chunk);  // RenderForward.cu:1317-1318
+                    float alpha_dest = 1.f;
+                    float color_out[VETRAST_MAX_CHANNELS];
+                    for (int ci = 0; ci < C; ++ci) color_out[ci] = 0.f;
+                    for (int i = 0; i < size_of_chunk; ++i)
+                    {
+                        const int point_id      = (int)(uint32_t)frag[o + i];
+                        const int texture_index = a->index ? a->index[point_id] : point_id;
+                        const float conf        = a->confidence[texture_index];
+                        if (transmittance) transmittance[(size_t)b * s.cap + o + i] = alpha_dest;
+                        for (int ci = 0; ci < C; ++ci)
+                        {
+                            const float color = a->texture[(size_t)ci * N + texture_index];
+                            color_out[ci]     = compute_blend(alpha_dest, conf, color, color_out[ci]);
+                        }
+                        alpha_dest = compute_new_alphadest(alpha_dest, conf);
+                    }
+                    for (int ci = 0; ci < C; ++ci)
+                    {
+                        if (!pr.use_environment_map)
+                            color_out[ci] = compute_blend(alpha_dest, 1.f, a->background[ci], color_out[ci]);
+                        out[((size_t)ci * lh + y) * lw + x] = color_out[ci];
+                    }
+                    wgt[q] = alpha_dest;  // atomicAdd onto a zeroed image, RenderForward.cu:1355-1356
+                    // CreateMask, rendering/PointRenderer.cu:216-235
+                    if (pr.output_background_mask && a->out_mask[l])
+                        a->out_mask[l][((size_t)b * lh + y) * lw + x] =
+                            (alpha_dest == 0.f) ? pr.output_background_mask_value : 1.f;
+                }
+        }
+    }
+    return VETRAST_OK;
+}
+
+// Backward pass. BlendBackwards2<C>, rendering/RenderBackward.cu:1083-1513, followed literally including the O(n^2)
+// inner loop; host part rendering/PointRenderer.cu:1111-1323 (zeroed gradient buffers, NormalizeGradient).
+extern "C" int vetref_backward(const vetrast_backward_args* g, const uint32_t* offsets, const uint64_t* fragments,
+                               int num_threads)
+{
+    const vetrast_forward_args* a = &g->fwd;
+    int st                        = validate(a);
+    if (st != VETRAST_OK) return st;
+    if (!g->grad_texture || !g->grad_confidence || !g->grad_background) return VETRAST_ERR_INVALID_ARG;
+    if (g->grad_points && !g->grad_point_count) return VETRAST_ERR_INVALID_ARG;
+    Scene s                  = make_scene(a);
+    const int N              = a->num_points;
+    const int C              = a->params.num_texture_channels;
+    const int K              = a->params.debug_max_list_length;
+    const vetrast_params& pr = a->params;
+    const bool par           = num_threads > 1;
+#ifdef _OPENMP
+    omp_set_num_threads(num_threads > 0 ? num_threads : 1);
+#endif
+    // zeros_like of every gradient tensor, rendering/PointRenderer.cu:267-277
+    std::fill(g->grad_texture, g->grad_texture + (size_t)C * N, 0.f);
+    std::fill(g->grad_confidence, g->grad_confidence + N, 0.f);
+    std::fill(g->grad_background, g->grad_background + C, 0.f);
+    if (g->grad_points)
+    {
+        std::fill(g->grad_points, g->grad_points + (size_t)4 * N, 0.f);
+        std::fill(g->grad_point_count, g->grad_point_count + N, 0.f);
+    }
+    const bool need_point_gradients = pr.need_point_gradient && g->grad_points;
+
+    for (int b = 0; b < a->num_views; ++b)
+    {
+        const Prepared& cam   = s.cams[b];
+        const vetrast_view& v = a->views[b];
+        const uint32_t* off   = offsets + (size_t)b * (s.P + 1);
+        const uint64_t* frag  = fragments + (size_t)b * s.cap;
+        for (int l = 0; l < s.ly.L; ++l)
+        {
+            const int lw = s.ly.w[l], lh = s.ly.h[l];
+            const size_t plane = (size_t)lw * lh;
+            const float* G     = g->grad_out[l] + (size_t)b * C * plane;
+            const float* I     = a->out[l] + (size_t)b * C * plane;
+#pragma omp parallel for schedule(dynamic, 8) if (par)
+            for (int gy = 0; gy < lh; ++gy)
+                for (int gx = 0; gx < lw; ++gx)
+                {
+                    const size_t q             = (size_t)(s.ly.base[l] + (int64_t)gy * lw + gx);
+                    const uint32_t offset      = off[q];
+                    int size_of_chunk          = (int)(off[q + 1] - offset);
+                    if (K > 0) size_of_chunk   = std::min(K, size_of_chunk);  // RenderBackward.cu:1098-1100
+                    auto sample_point_id       = [&](int pos) { return (int)(uint32_t)frag[pos]; };
+                    auto sample_texture_index  = [&](int pos) {
+                        const int id = sample_point_id(pos);
+                        return a->index ? a->index[id] : id;
+                    };
+                    // ---- value gradients, RenderBackward.cu:1118-1181
+                    {
+                        float alpha_dest = 1.f;
+                        const int list_size = pr.use_environment_map ? size_of_chunk : size_of_chunk + 1;
+                        for (int i = 0; i < list_size; ++i)
+                        {
+                            const bool is_foreground = i != size_of_chunk;
+                            int texture_index        = 0;
+                            if (is_foreground) texture_index = sample_texture_index(offset + i);
+                            float confidence_val = 1.f;
+                            if (is_foreground) confidence_val = a->confidence[texture_index];
+                            float colors[VETRAST_MAX_CHANNELS], grad_in[VETRAST_MAX_CHANNELS];
+                            for (int ci = 0; ci < C; ++ci)
+                                colors[ci] = is_foreground ? a->texture[(size_t)ci * N + texture_index]
+                                                           : a->background[ci];
+                            float g_alpha = 0;
+                            for (int ci = 0; ci < C; ++ci)
+                            {
+                                grad_in[ci]   = G[ci * plane + (size_t)gy * lw + gx];
+                                float g_col   = alpha_dest * confidence_val * grad_in[ci];
+                                float* target = is_foreground ? &g->grad_texture[(size_t)ci * N + texture_index]
+                                                              : &g->grad_background[ci];
+                                atomic_add(target, g_col, par);
+                                g_alpha += colors[ci] * grad_in[ci];
+                            }
+                            g_alpha *= alpha_dest;
+                            // The reference adds this unguarded, so the background element leaks into index 0
+                            // (RenderBackward.cu:1130-1131,1157); kept behind a switch.
+                            if (is_foreground || pr.quirk_background_confidence_leak)
+                                atomic_add(&g->grad_confidence[texture_index], g_alpha, par);
+                            for (int j = 0; j < i; ++j)
+                            {
+                                const int texture_index_iter    = sample_texture_index(offset + j);
+                                const float confidence_val_iter = a->confidence[texture_index_iter];
+                                float g_iter                    = 0;
+                                for (int ci = 0; ci < C; ++ci)
+                                {
+                                    const float epsilon = 1e-9;
+                                    float g_alpha_iter  = (grad_in[ci] * colors[ci] * alpha_dest * confidence_val /
+                                                          (1 - confidence_val_iter + epsilon));
+                                    g_iter -= g_alpha_iter;
+                                }
+                                atomic_add(&g->grad_confidence[texture_index_iter], g_iter, par);
+                            }
+                            alpha_dest = compute_new_alphadest(alpha_dest, confidence_val);
+                        }
+                    }
+                    if (!need_point_gradients) continue;
+                    // ---- position gradient heuristic, RenderBackward.cu:1185-1408
+                    // distanceFromEdge(y, x) = min(x, y, w-1-x, h-1-y)
+                    const int edge = std::min(std::min(gx, gy), std::min(lw - 1 - gx, lh - 1 - gy));
+                    if (!(edge > 2)) continue;
+                    for (int i = 0; i < size_of_chunk; ++i)
+                    {
+                        const int point_id      = sample_point_id(offset + i);
+                        const int texture_index = a->index ? a->index[point_id] : point_id;
+                        float dR_dpx = 0, dR_dpy = 0;
+                        for (int ci = 0; ci < C; ++ci)
+                        {
+                            const float T_p   = a->texture[(size_t)ci * N + texture_index];
+                            const float* Ic   = I + ci * plane;
+                            const float* Gc   = G + ci * plane;
+                            const size_t ctr  = (size_t)gy * lw + gx;
+                            const float I_px0 = Ic[ctr - 1], I_px1 = Ic[ctr + 1];
+                            const float I_py0 = Ic[ctr - lw], I_py1 = Ic[ctr + lw];
+                            const float G_px0 = Gc[ctr - 1], G_px1 = Gc[ctr + 1];
+                            const float G_py0 = Gc[ctr - lw], G_py1 = Gc[ctr + lw];
+                            float dI_dp_at_px0 = -(T_p - I_px0) * G_px0;  // RenderBackward.cu:1364-1371
+                            float dI_dp_at_px1 = (T_p - I_px1) * G_px1;
+                            float dI_dp_at_py0 = -(T_p - I_py0) * G_py0;
+                            float dI_dp_at_py1 = (T_p - I_py1) * G_py1;
+                            dR_dpx += 0.5f * (dI_dp_at_px0 + dI_dp_at_px1);
+                            dR_dpy += 0.5f * (dI_dp_at_py0 + dI_dp_at_py1);
+                        }
+                        const float gxp = dR_dpx / float(C), gyp = dR_dpy / float(C);  // :1374
+                        // crop_transform.scale(0.5^layer): all five coefficients, RenderBackward.cu:1381-1385
+                        const float scale = powf(0.5f, float(l));
+                        const float cfx = v.crop_transform[0] * scale, cfy = v.crop_transform[1] * scale,
+                                    cs = v.crop_transform[4] * scale;
+                        // ProjectPointPinholeBackward, rendering/PointRendererHelper.h:317-372 (zero distortion:
+                        // J_p_dis = I); J_point = R, J_p_div = [1/z 0 -x/z^2; 0 1/z -y/z^2].
+                        const float* p4 = a->position + 4 * (size_t)point_id;
+                        const float px = p4[0], py = p4[1], pz = p4[2];
+                        const float vx = ((cam.r[0] * px + cam.r[1] * py) + cam.r[2] * pz) + cam.t[0];
+                        const float vy = ((cam.r[3] * px + cam.r[4] * py) + cam.r[5] * pz) + cam.t[1];
+                        const float vz = ((cam.r[6] * px + cam.r[7] * py) + cam.r[8] * pz) + cam.t[2];
+                        float gp[3] = {0.f, 0.f, 0.f};
+                        if (vz > 0.f)
+                        {
+                            const float ar = v.crop_rotation[0] * gxp + v.crop_rotation[2] * gyp;  // J_rot^T grad
+                            const float br = v.crop_rotation[1] * gxp + v.crop_rotation[3] * gyp;
+                            const float a2 = cfx * ar;            // J_p_K2^T
+                            const float b2 = cs * ar + cfy * br;
+                            const float d0 = cam.fx * a2;         // J_p_K1^T
+                            const float d1 = cam.s * a2 + cam.fy * b2;
+                            const float iz = 1.f / vz;
+                            const float e0 = iz * d0, e1 = iz * d1;
+                            const float e2 = (-vx * iz * iz) * d0 + (-vy * iz * iz) * d1;
+                            gp[0]          = (cam.r[0] * e0 + cam.r[3] * e1) + cam.r[6] * e2;  // R^T
+                            gp[1]          = (cam.r[1] * e0 + cam.r[4] * e1) + cam.r[7] * e2;
+                            gp[2]          = (cam.r[2] * e0 + cam.r[5] * e1) + cam.r[8] * e2;
+                        }
+                        for (int k = 0; k < 3; ++k) atomic_add(&g->grad_points[4 * (size_t)point_id + k], gp[k], par);
+                        atomic_add(&g->grad_point_count[point_id], 1.f, par);  // RenderBackward.cu:1407
+                    }
+                }
+        }
+    }
+
+    // NormalizeGradient<float,3>, rendering/PointRenderer.cu:1072-1090,1273-1280
+    if (g->grad_points && pr.point_gradient_normalization == 1)
+    {
+        for (int i = 0; i < N; ++i)
+        {
+            const float c = g->grad_point_count[i];
+            if (c > 0)
+                for (int k = 0; k < 3; ++k) g->grad_points[4 * (size_t)i + k] /= c;
+        }
+    }
+    else if (g->grad_points && pr.point_gradient_normalization == 2)
+    {
+        // literal: the [N,4] buffer is addressed as N vec3, so flat elements 3i..3i+2 are divided by count[i]
+        for (int i = 0; i < N; ++i)
+        {
+            const float c = g->grad_point_count[i];
+            if (c > 0)
+                for (int k = 0; k < 3; ++k) g->grad_points[3 * (size_t)i + k] /= c;
+        }
+    }
+    return VETRAST_OK;
+}

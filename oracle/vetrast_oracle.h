@@ -1,0 +1,53 @@
+/*
+ * CPU oracle of the blending point rasterizer — TEST INFRASTRUCTURE ONLY.
+ *
+ * A plain scalar restatement of the reference's FULL_BLEND path (lfranke/VET, src/lib/rendering). It exists to
+ * check the GPU library and to be timed as the CPU baseline; nothing that ships may call it. Only tests/,
+ * __graft_entry__.smoke() and bench.py's cpu_baseline leg load this library.
+ *
+ * Argument structs are the PODs of include/vetrast.h, with every `device` pointer replaced by a host pointer and
+ * the workspace ignored; saved state goes to explicit caller-allocated arrays instead:
+ *   offsets       uint32 [B][P+1]   exclusive scan of per-pixel counts, pixels of all layers concatenated
+ *   fragments     uint64 [B][N*L]   (depth_bits << 32) | point_id; every pixel list fully sorted ascending
+ *   transmittance float  [B][N*L]   transmittance in front of fragment i for i < min(count, K)
+ *   weight        float  [B][P]     final transmittance per pixel
+ *
+ * Parity status of the pieces (what pins each is in tests/test_oracle_*.py):
+ *   projection        pinned by the reference's own host restatements of the pinhole model
+ *                     (src/lib/data/SceneData.cpp:28-36,1020-1049) for zero distortion and by brute-force checks;
+ *                     the bit pattern of saiga's TransformPoint / DivideByZ is PARITY UNPINNED (saiga is not vendored)
+ *   count/scan/fill   pinned by brute force and by the reference's own invariant counters == counts
+ *   sort              pinned against a generic sort of (depth, id) pairs; the id tie-break refines the reference's
+ *                     depth-only order
+ *   blend             pinned by closed forms (empty pixel, one fragment, n equal fragments, partition of unity)
+ *   value gradients   pinned by double-precision central differences of an independent numpy blend
+ *   position gradient literal restatement; the heuristic is checked on hand-computed cases, the projection Jacobian
+ *                     by finite differences; saiga's operator order inside the Jacobians is PARITY UNPINNED
+ *   distortion != 0, check_normal, OCam, spherical: not implemented (rejected), PARITY UNPINNED
+ */
+#ifndef VETRAST_ORACLE_H
+#define VETRAST_ORACLE_H
+
+#include "../include/vetrast.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Prepared per-view camera constants: 12 floats world->camera (R row-major | t as 4th column per row),
+ * then fx,fy,cx,cy,s. Exposed so that tests can pin the quaternion conversion. */
+int vetref_prepare_view(const double* pose8, const float* intrinsics13, float* out17);
+
+/* Project one point for one prepared view; returns 0 if rejected (z == 0). ip_z_r = {ip.x, ip.y, z, radius_px}. */
+int vetref_project_point(const float* prepared17, const vetrast_view* view, const float* position4, float* ip_z_r);
+
+int vetref_forward(const vetrast_forward_args* args, uint32_t* offsets, uint64_t* fragments, float* transmittance,
+                   float* weight, int num_threads);
+
+int vetref_backward(const vetrast_backward_args* args, const uint32_t* offsets, const uint64_t* fragments,
+                    int num_threads);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

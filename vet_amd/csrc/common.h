@@ -1,0 +1,112 @@
+// Shared declarations of the gfx950 blending point rasterizer (internal; the public boundary is include/vetrast.h).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/vetrast.h"
+
+namespace vetrast
+{
+constexpr int kBlock          = 256;          // threads per workgroup = 4 wave64
+constexpr int kWave           = 64;
+constexpr uint32_t kNoSlot    = 0xFFFFFFFFu;
+constexpr uint64_t kInfKey    = ~0ull;        // sorts behind every real (depth bits, point id) key
+constexpr int kScanPerThread  = 16;
+constexpr int kScanPerBlock   = kBlock * kScanPerThread;  // 4096 counts per workgroup
+constexpr int kPackedFloats   = 8;            // interleaved record: 4 descriptor floats, confidence, 3 pad
+
+// Camera constants of one view, written by prepare_views_kernel and read (uniformly) by every other kernel.
+// Counterpart of what the reference pulls per thread out of d_render_params.Pose()/PinholeIntrinsics() and the
+// by-value ReducedImageInfo (src/lib/rendering/RenderForward.cu:117-158).
+struct DeviceView
+{
+    float r[9];  // world -> camera rotation, row-major
+    float t[3];
+    float fx, fy, cx, cy, s;  // K
+    float crop[5];            // fx, fy, cx, cy, s of the crop transform
+    float rot[4];             // crop rotation r00 r01 r10 r11
+    float ccx, ccy;           // (w/2, h/2) with integer halving
+    float pad[4];
+};
+static_assert(sizeof(DeviceView) == 32 * 4, "DeviceView is 32 floats");
+
+// Pixels of all layers of one view are numbered consecutively: q = base[l] + y * w[l] + x.
+struct LayerTable
+{
+    int L;
+    int w[VETRAST_MAX_LAYERS];
+    int h[VETRAST_MAX_LAYERS];
+    uint32_t base[VETRAST_MAX_LAYERS + 1];
+};
+
+// Launch descriptor shared by the forward kernels of one view.
+struct ViewPass
+{
+    const float4* position;
+    const int32_t* index;
+    const float* confidence;
+    const float* dropout;  // already offset to this view, or null
+    const DeviceView* view;
+    LayerTable ly;
+    int N;
+    int drop_by_radius;
+    float radius_threshold;
+    int viewer_only;
+    float stability_cutoff;
+};
+
+struct Projected
+{
+    float ipx, ipy, z, radius;
+};
+
+// Projection of one point: rigid transform, clamp z, divide, K, crop transform, rotation about the crop centre.
+// Follows ProjPoint / ProjectPointPinhole / rotateCropAroundCenter (src/lib/rendering/RenderForward.cu:110-158,
+// src/lib/rendering/PointRendererHelper.h:184-218) for zero distortion. Every operation is rounded on its own
+// (the file is compiled with -ffp-contract=off) so that the CPU check of the same formula agrees bit for bit.
+__device__ __forceinline__ bool project_point(const DeviceView& c, const float4 p, Projected& o)
+{
+    const float vx = ((c.r[0] * p.x + c.r[1] * p.y) + c.r[2] * p.z) + c.t[0];
+    const float vy = ((c.r[3] * p.x + c.r[4] * p.y) + c.r[5] * p.z) + c.t[1];
+    const float vz = ((c.r[6] * p.x + c.r[7] * p.y) + c.r[8] * p.z) + c.t[2];
+    const float z  = fmaxf(vz, 0.f);
+    if (!(z > 0.f)) return false;
+    const float nx  = vx / vz;
+    const float ny  = vy / vz;
+    const float u   = (c.fx * nx + c.s * ny) + c.cx;
+    const float v   = c.fy * ny + c.cy;
+    const float ipx = (c.crop[0] * u + c.crop[4] * v) + c.crop[2];
+    const float ipy = c.crop[1] * v + c.crop[3];
+    const float dx = ipx - c.ccx, dy = ipy - c.ccy;
+    const float rx = c.rot[0] * dx + c.rot[1] * dy;
+    const float ry = c.rot[2] * dx + c.rot[3] * dy;
+    o.ipx          = rx + c.ccx;
+    o.ipy          = ry + c.ccy;
+    o.z            = z;
+    o.radius       = ((c.fx * c.crop[0]) * p.w) / z;
+    return true;
+}
+
+// Pixel of layer l for a projected point, or -1. The caller halves ipx/ipy/radius between layers
+// (src/lib/rendering/RenderForward.cu:856,888-891); rintf is round-half-even like __float2int_rn.
+__device__ __forceinline__ int64_t layer_pixel(const LayerTable& ly, int l, float ipx, float ipy)
+{
+    const float fx = rintf(ipx), fy = rintf(ipy);
+    if (!(fx >= 0.f && fx < (float)ly.w[l] && fy >= 0.f && fy < (float)ly.h[l])) return -1;
+    return (int64_t)ly.base[l] + (int64_t)(int)fy * ly.w[l] + (int)fx;
+}
+
+__device__ __forceinline__ int layer_of_pixel(const LayerTable& ly, uint32_t q)
+{
+    int l = 0;
+#pragma unroll
+    for (int k = 1; k < VETRAST_MAX_LAYERS; ++k)
+        if (k < ly.L && q >= ly.base[k]) l = k;
+    return l;
+}
+
+// ---- host-side launchers (one per source file) -------------------------------------------------------------
+struct ForwardLaunch;
+struct BackwardLaunch;
+
+}  // namespace vetrast

@@ -1,0 +1,301 @@
+// Forward kernels: zero fill, view preparation, descriptor interleave, project+count, scan, fill, blend.
+#pragma once
+#include "common.h"
+
+namespace vetrast
+{
+// Plain fill kernel (used instead of hipMemsetAsync so that callers may capture the launches in a HIP graph).
+__global__ void __launch_bounds__(kBlock) fill_u32_kernel(uint32_t* __restrict__ dst, size_t n, uint32_t value)
+{
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) dst[i] = value;
+}
+
+// 16-byte wide variant for the big buffers; n4 counts uint4 elements.
+__global__ void __launch_bounds__(kBlock) fill_u128_kernel(uint4* __restrict__ dst, size_t n4, uint32_t value)
+{
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    const uint4 v       = make_uint4(value, value, value, value);
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += stride) dst[i] = v;
+}
+
+struct ViewSource
+{
+    int image_index, camera_index, w, h;
+    float crop[5];
+    float rot[4];
+};
+
+struct PrepareViewsArgs
+{
+    ViewSource src[16];
+};
+
+// One thread per view: pose (unit quaternion + translation, double) -> 3x4 float matrix, intrinsics row -> K.
+// The reference casts the SE3d to float in every thread (src/lib/rendering/RenderConstants.h:78); here the rotation
+// matrix is formed once, in double, and rounded once. Non-zero distortion coefficients raise flag bit 0.
+__global__ void prepare_views_kernel(PrepareViewsArgs args, int first_view, int num_views,
+                                     const double* __restrict__ poses_se3, const float* __restrict__ intrinsics,
+                                     DeviceView* __restrict__ views, uint32_t* __restrict__ flags)
+{
+    const int k = threadIdx.x;
+    if (k >= num_views) return;
+    const ViewSource& s = args.src[k];
+    const double* q     = poses_se3 + 8 * (size_t)s.image_index;
+    const float* in     = intrinsics + 13 * (size_t)s.camera_index;
+    DeviceView v;
+    const double x = q[0], y = q[1], z = q[2], w = q[3];
+    const double tx = 2.0 * x, ty = 2.0 * y, tz = 2.0 * z;
+    const double twx = tx * w, twy = ty * w, twz = tz * w;
+    const double txx = tx * x, txy = ty * x, txz = tz * x;
+    const double tyy = ty * y, tyz = tz * y, tzz = tz * z;
+    v.r[0] = (float)(1.0 - (tyy + tzz));
+    v.r[1] = (float)(txy - twz);
+    v.r[2] = (float)(txz + twy);
+    v.r[3] = (float)(txy + twz);
+    v.r[4] = (float)(1.0 - (txx + tzz));
+    v.r[5] = (float)(tyz - twx);
+    v.r[6] = (float)(txz - twy);
+    v.r[7] = (float)(tyz + twx);
+    v.r[8] = (float)(1.0 - (txx + tyy));
+    v.t[0] = (float)q[4];
+    v.t[1] = (float)q[5];
+    v.t[2] = (float)q[6];
+    v.fx   = in[0];
+    v.fy   = in[1];
+    v.cx   = in[2];
+    v.cy   = in[3];
+    v.s    = in[4];
+    bool distorted = false;
+    for (int j = 5; j < 13; ++j) distorted |= (in[j] != 0.f);
+    if (distorted) atomicOr(flags, 1u);
+    for (int j = 0; j < 5; ++j) v.crop[j] = s.crop[j];
+    for (int j = 0; j < 4; ++j) v.rot[j] = s.rot[j];
+    v.ccx = (float)(s.w / 2);
+    v.ccy = (float)(s.h / 2);
+    for (int j = 0; j < 4; ++j) v.pad[j] = 0.f;
+    views[first_view + k] = v;
+}
+
+// Planar descriptors [C,N] + confidence [N] -> one 32-byte record per texture index, so that a fragment costs a single
+// aligned gather instead of C+1 gathers from planes megabytes apart (the reference's BlendMulti reads
+// d_texture.in_texture(ci, idx) per channel, src/lib/rendering/RenderForward.cu:1338-1342).
+template <int C>
+__global__ void __launch_bounds__(kBlock) pack_descriptors_kernel(const float* __restrict__ texture,
+                                                                   const float* __restrict__ confidence,
+                                                                   float4* __restrict__ packed, int N)
+{
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= N) return;
+    float t[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int ci = 0; ci < C; ++ci) t[ci] = texture[(size_t)ci * N + i];
+    packed[2 * (size_t)i]     = make_float4(t[0], t[1], t[2], t[3]);
+    packed[2 * (size_t)i + 1] = make_float4(confidence[i], 0.f, 0.f, 0.f);
+}
+
+__device__ __forceinline__ bool point_is_skipped(const ViewPass& a, int i)
+{
+    if (a.dropout && a.dropout[i] == 1.f) return true;
+    if (a.viewer_only)
+    {
+        const int ti = a.index ? a.index[i] : i;
+        if (a.confidence[ti] < a.stability_cutoff) return true;
+    }
+    return false;
+}
+
+// Project every point and count it in the pixel it rounds to, in every layer. The returning atomic hands each
+// (point, layer) its arrival rank inside the pixel, which the fill pass turns into a buffer position without a second
+// atomic. Counterpart of CountingPrepassMulti<L,false> (src/lib/rendering/RenderForward.cu:806-905).
+__global__ void __launch_bounds__(kBlock) count_kernel(ViewPass a, uint32_t* __restrict__ counts,
+                                                        uint32_t* __restrict__ slots)
+{
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= a.N) return;
+    if (point_is_skipped(a, i)) return;
+    Projected p;
+    if (!project_point(*a.view, a.position[i], p)) return;
+    float ipx = p.ipx, ipy = p.ipy, radius = p.radius;
+    for (int l = 0; l < a.ly.L; ++l, radius *= 0.5f, ipx *= 0.5f, ipy *= 0.5f)
+    {
+        if (a.drop_by_radius && radius < a.radius_threshold) break;
+        const int64_t q = layer_pixel(a.ly, l, ipx, ipy);
+        if (q < 0) continue;
+        slots[(size_t)l * a.N + i] = atomicAdd(&counts[q], 1u);
+    }
+}
+
+// ---- exclusive scan of the per-pixel counts, in place, in two launches -------------------------------------------
+// Launch 1: one partial sum per 4096 counts. Launch 2: every workgroup adds up the partials in front of it (a few
+// hundred values, cache resident), then scans its own 4096 counts. No workgroup waits for another one.
+// Counterpart of thrust::exclusive_scan + the two .item<int>() read-backs (src/lib/rendering/PointRenderer.cu:799-813);
+// the total lands at counts[P] because the array is zero padded behind P.
+__device__ __forceinline__ uint32_t wave_inclusive_scan(uint32_t v, int lane)
+{
+#pragma unroll
+    for (int d = 1; d < kWave; d <<= 1)
+    {
+        const uint32_t o = __shfl_up(v, d, kWave);
+        if (lane >= d) v += o;
+    }
+    return v;
+}
+
+__device__ __forceinline__ uint32_t block_reduce_sum(uint32_t v, uint32_t* lds4)
+{
+#pragma unroll
+    for (int d = kWave / 2; d >= 1; d >>= 1) v += __shfl_xor(v, d, kWave);
+    const int wave = threadIdx.x / kWave;
+    if ((threadIdx.x & (kWave - 1)) == 0) lds4[wave] = v;
+    __syncthreads();
+    const uint32_t total = lds4[0] + lds4[1] + lds4[2] + lds4[3];
+    __syncthreads();
+    return total;
+}
+
+__global__ void __launch_bounds__(kBlock) scan_partials_kernel(const uint4* __restrict__ counts4,
+                                                                uint32_t* __restrict__ partials)
+{
+    __shared__ uint32_t lds4[4];
+    const uint4* src = counts4 + (size_t)blockIdx.x * (kScanPerBlock / 4);
+    uint32_t sum     = 0;
+#pragma unroll
+    for (int k = 0; k < kScanPerThread / 4; ++k)
+    {
+        const uint4 v = src[k * kBlock + threadIdx.x];
+        sum += (v.x + v.y) + (v.z + v.w);
+    }
+    const uint32_t total = block_reduce_sum(sum, lds4);
+    if (threadIdx.x == 0) partials[blockIdx.x] = total;
+}
+
+__global__ void __launch_bounds__(kBlock) scan_apply_kernel(uint4* __restrict__ counts4,
+                                                             const uint32_t* __restrict__ partials)
+{
+    __shared__ uint32_t lds4[4];
+    __shared__ uint32_t wave_tot[4];
+    uint32_t before = 0;
+    for (int k = threadIdx.x; k < (int)blockIdx.x; k += kBlock) before += partials[k];
+    const uint32_t block_base = block_reduce_sum(before, lds4);
+
+    // thread t owns the 16 consecutive counts [16 t, 16 t + 16) of this workgroup's 4096
+    uint4* mine = counts4 + (size_t)blockIdx.x * (kScanPerBlock / 4) + threadIdx.x * (kScanPerThread / 4);
+    uint4 v[kScanPerThread / 4];
+    uint32_t sum = 0;
+#pragma unroll
+    for (int k = 0; k < kScanPerThread / 4; ++k)
+    {
+        v[k] = mine[k];
+        sum += (v[k].x + v[k].y) + (v[k].z + v[k].w);
+    }
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    const uint32_t incl = wave_inclusive_scan(sum, lane);
+    if (lane == kWave - 1) wave_tot[wave] = incl;
+    __syncthreads();
+    uint32_t run = block_base + (incl - sum);
+    for (int k = 0; k < wave; ++k) run += wave_tot[k];
+#pragma unroll
+    for (int k = 0; k < kScanPerThread / 4; ++k)
+    {
+        uint4 o;
+        o.x = run;
+        run += v[k].x;
+        o.y = run;
+        run += v[k].y;
+        o.z = run;
+        run += v[k].z;
+        o.w = run;
+        run += v[k].w;
+        mine[k] = o;
+    }
+}
+
+// Second projection of every point; writes its 64-bit record (depth bits, point id) at scan[pixel] + rank.
+// Counterpart of CollectMulti<L,false> (src/lib/rendering/RenderForward.cu:1011-1096), which draws the rank from a
+// second atomic counter image and stores depth and id in two separate rows.
+__global__ void __launch_bounds__(kBlock) fill_kernel(ViewPass a, const uint32_t* __restrict__ offsets,
+                                                       const uint32_t* __restrict__ slots,
+                                                       uint64_t* __restrict__ fragments, uint32_t capacity)
+{
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= a.N) return;
+    if (point_is_skipped(a, i)) return;
+    Projected p;
+    if (!project_point(*a.view, a.position[i], p)) return;
+    const uint64_t key = ((uint64_t)__float_as_uint(p.z) << 32) | (uint32_t)i;
+    float ipx = p.ipx, ipy = p.ipy, radius = p.radius;
+    for (int l = 0; l < a.ly.L; ++l, radius *= 0.5f, ipx *= 0.5f, ipy *= 0.5f)
+    {
+        if (a.drop_by_radius && radius < a.radius_threshold) break;
+        const int64_t q = layer_pixel(a.ly, l, ipx, ipy);
+        if (q < 0) continue;
+        const uint32_t pos = offsets[q] + slots[(size_t)l * a.N + i];
+        if (pos < capacity) fragments[pos] = key;  // always true when count and fill agree; guards the store
+    }
+}
+
+struct BlendPass
+{
+    const uint32_t* offsets;
+    const uint64_t* fragments;
+    const int32_t* index;
+    const float4* packed;
+    const float* background;
+    float* transmittance;  // per fragment, null unless the backward pass will run
+    float* weight;         // per pixel
+    float* out[VETRAST_MAX_LAYERS];       // already offset to this view
+    float* out_mask[VETRAST_MAX_LAYERS];  // already offset to this view, or null
+    LayerTable ly;
+    uint32_t P;
+    int N;
+    int K;
+    int use_environment_map;
+    float mask_value;
+};
+
+// One thread per pixel walks the sorted list front to back: out += (T*c)*t, T = (1-c)*T, in exactly this order, then
+// the background behind the last fragment. Counterpart of BlendMulti (src/lib/rendering/RenderForward.cu:1303-1357)
+// and CreateMask (src/lib/rendering/PointRenderer.cu:216-235). Pixels of all layers are served by one launch.
+template <int C>
+__global__ void __launch_bounds__(kBlock) blend_kernel(BlendPass a)
+{
+    const uint32_t q = blockIdx.x * blockDim.x + threadIdx.x;
+    if (q >= a.P) return;
+    const uint32_t off = a.offsets[q];
+    uint32_t n         = a.offsets[q + 1] - off;
+    if (a.K > 0) n = min(n, (uint32_t)a.K);
+    float T = 1.f;
+    float color[C];
+#pragma unroll
+    for (int ci = 0; ci < C; ++ci) color[ci] = 0.f;
+    const uint64_t* list = a.fragments + off;
+    for (uint32_t i = 0; i < n; ++i)
+    {
+        const int id = (int)(uint32_t)list[i];
+        if ((uint32_t)id >= (uint32_t)a.N) break;  // cannot happen for a list the fill pass wrote; guards the gather
+        const int ti = a.index ? a.index[id] : id;
+        if ((uint32_t)ti >= (uint32_t)a.N) break;  // texture index out of range (the reference asserts here)
+        const float4 t4 = a.packed[2 * (size_t)ti];
+        const float c   = a.packed[2 * (size_t)ti + 1].x;
+        if (a.transmittance) a.transmittance[off + i] = T;
+        const float t[4] = {t4.x, t4.y, t4.z, t4.w};
+        const float Tc   = T * c;
+#pragma unroll
+        for (int ci = 0; ci < C; ++ci) color[ci] = Tc * t[ci] + color[ci];
+        T = (1.f - c) * T;
+    }
+    const int l          = layer_of_pixel(a.ly, q);
+    const size_t plane   = (size_t)a.ly.w[l] * a.ly.h[l];
+    const uint32_t local = q - a.ly.base[l];
+#pragma unroll
+    for (int ci = 0; ci < C; ++ci)
+    {
+        if (!a.use_environment_map) color[ci] = (T * 1.f) * a.background[ci] + color[ci];
+        a.out[l][ci * plane + local] = color[ci];
+    }
+    a.weight[q] = T;
+    if (a.out_mask[l]) a.out_mask[l][local] = (T == 0.f) ? a.mask_value : 1.f;
+}
+
+}  // namespace vetrast

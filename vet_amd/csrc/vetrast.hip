@@ -1,0 +1,591 @@
+// C ABI of the gfx950 blending point rasterizer: argument checks, workspace layout and the launch sequence.
+// Host-side counterpart of BlendPointCloudForward / BlendPointCloudBackward and PointRendererCache
+// (src/lib/rendering/PointRenderer.cu:238-470,657-1069,1111-1323 of the reference), without its per-layer
+// device->host reads, per-frame allocations and __constant__ uploads.
+#include <hip/hip_runtime.h>
+
+#include <cstring>
+#include <new>
+#include <vector>
+
+#include "backward_kernels.h"
+#include "common.h"
+#include "forward_kernels.h"
+#include "sort_kernels.h"
+
+using namespace vetrast;
+
+struct vetrast_ctx
+{
+    int device         = 0;
+    int profiling      = 0;
+    int last_hip_error = 0;
+    struct Span
+    {
+        int scope;
+        hipEvent_t start, stop;
+    };
+    std::vector<Span> spans;             // recorded since the last reset
+    std::vector<hipEvent_t> free_events;  // recycled events
+    float acc_ms[VETRAST_SCOPE_COUNT_]      = {};
+    int32_t acc_launches[VETRAST_SCOPE_COUNT_] = {};
+};
+
+namespace
+{
+constexpr size_t kAlign = 256;
+inline size_t align_up(size_t v, size_t a)
+{
+    return (v + a - 1) / a * a;
+}
+
+#define VET_HIP(ctx, expr)                               \
+    do                                                   \
+    {                                                    \
+        hipError_t e_ = (expr);                          \
+        if (e_ != hipSuccess)                            \
+        {                                                \
+            if (ctx) (ctx)->last_hip_error = (int)e_;    \
+            return VETRAST_ERR_HIP;                      \
+        }                                                \
+    } while (0)
+
+// Brackets the launches of one scope with events when profiling is on.
+struct ScopeTimer
+{
+    vetrast_ctx* ctx;
+    hipStream_t stream;
+    int scope;
+    hipEvent_t start = nullptr, stop = nullptr;
+    bool on          = false;
+    ScopeTimer(vetrast_ctx* c, hipStream_t s, int sc) : ctx(c), stream(s), scope(sc)
+    {
+        if (!ctx->profiling) return;
+        start = take();
+        stop  = take();
+        if (!start || !stop) return;
+        on = hipEventRecord(start, stream) == hipSuccess;
+    }
+    ~ScopeTimer()
+    {
+        if (!on) return;
+        (void)hipEventRecord(stop, stream);
+        ctx->spans.push_back({scope, start, stop});
+    }
+    hipEvent_t take()
+    {
+        if (!ctx->free_events.empty())
+        {
+            hipEvent_t e = ctx->free_events.back();
+            ctx->free_events.pop_back();
+            return e;
+        }
+        hipEvent_t e = nullptr;
+        if (hipEventCreate(&e) != hipSuccess) return nullptr;
+        return e;
+    }
+};
+
+inline int grid_for(size_t n, int block = kBlock)
+{
+    return (int)((n + block - 1) / block);
+}
+
+LayerTable make_layer_table(int w, int h, int L)
+{
+    LayerTable t;
+    std::memset(&t, 0, sizeof(t));
+    t.L          = L;
+    uint32_t run = 0;
+    for (int l = 0; l < L; ++l)
+    {
+        t.w[l]    = w;
+        t.h[l]    = h;
+        t.base[l] = run;
+        run += (uint32_t)w * (uint32_t)h;
+        w /= 2;
+        h /= 2;
+    }
+    for (int l = L; l <= VETRAST_MAX_LAYERS; ++l) t.base[l] = run;
+    return t;
+}
+
+int check_dims(int64_t N, int B, int L, int w, int h)
+{
+    if (N < 0 || B < 1 || L < 1 || L > VETRAST_MAX_LAYERS || w < 1 || h < 1) return VETRAST_ERR_INVALID_ARG;
+    if ((w >> (L - 1)) < 1 || (h >> (L - 1)) < 1) return VETRAST_ERR_INVALID_ARG;  // coarsest layer must not be empty
+    // fragment positions and pixel numbers are 32-bit
+    if (N * L >= (int64_t)0xFFFFFFF0ll) return VETRAST_ERR_INVALID_ARG;
+    int64_t P = 0;
+    int lw = w, lh = h;
+    for (int l = 0; l < L; ++l, lw /= 2, lh /= 2) P += (int64_t)lw * lh;
+    if (P + kScanPerBlock >= (int64_t)0x7FFFFFFFll) return VETRAST_ERR_INVALID_ARG;
+    return VETRAST_OK;
+}
+
+int validate_forward(const vetrast_forward_args* a, vetrast_workspace_layout* lay)
+{
+    if (!a) return VETRAST_ERR_INVALID_ARG;
+    const vetrast_params& p = a->params;
+    if (!a->position || !a->texture || !a->confidence || !a->background || !a->poses_se3 || !a->intrinsics ||
+        !a->views || !a->workspace)
+        return VETRAST_ERR_INVALID_ARG;
+    if (a->num_views < 1 || a->num_poses < 1 || a->num_cameras < 1) return VETRAST_ERR_INVALID_ARG;
+    if (p.num_texture_channels < 1 || p.num_texture_channels > VETRAST_MAX_CHANNELS) return VETRAST_ERR_INVALID_ARG;
+    if (p.check_normal) return VETRAST_ERR_UNSUPPORTED;
+    const int w = a->views[0].w, h = a->views[0].h;
+    int st = check_dims(a->num_points, a->num_views, p.num_layers, w, h);
+    if (st != VETRAST_OK) return st;
+    for (int b = 0; b < a->num_views; ++b)
+    {
+        const vetrast_view& v = a->views[b];
+        if (v.camera_model_type != VETRAST_CAMERA_PINHOLE_DISTORTION) return VETRAST_ERR_UNSUPPORTED;
+        if (v.w != w || v.h != h) return VETRAST_ERR_INVALID_ARG;
+        if (v.image_index < 0 || v.image_index >= a->num_poses) return VETRAST_ERR_INVALID_ARG;
+        if (v.camera_index < 0 || v.camera_index >= a->num_cameras) return VETRAST_ERR_INVALID_ARG;
+    }
+    for (int l = 0; l < p.num_layers; ++l)
+    {
+        if (!a->out[l]) return VETRAST_ERR_INVALID_ARG;
+        if (p.output_background_mask && !a->out_mask[l]) return VETRAST_ERR_INVALID_ARG;
+    }
+    if (((uintptr_t)a->workspace % kAlign) != 0 || ((uintptr_t)a->position % 16) != 0) return VETRAST_ERR_INVALID_ARG;
+    st = vetrast_workspace_layout_for(a->num_points, a->num_views, p.num_layers, w, h, lay);
+    if (st != VETRAST_OK) return st;
+    if (a->workspace_bytes < lay->total_bytes) return VETRAST_ERR_WORKSPACE_SMALL;
+    return VETRAST_OK;
+}
+
+template <class T>
+inline T* ws_ptr(void* ws, size_t off)
+{
+    return reinterpret_cast<T*>(static_cast<char*>(ws) + off);
+}
+
+ViewPass make_view_pass(const vetrast_forward_args* a, const vetrast_workspace_layout& lay, const LayerTable& ly, int b)
+{
+    ViewPass vp;
+    vp.position         = reinterpret_cast<const float4*>(a->position);
+    vp.index            = a->index;
+    vp.confidence       = a->confidence;
+    vp.dropout          = a->dropout ? a->dropout + (size_t)b * a->num_points : nullptr;
+    vp.view             = ws_ptr<DeviceView>(a->workspace, lay.views_base) + b;
+    vp.ly               = ly;
+    vp.N                = a->num_points;
+    vp.drop_by_radius   = a->params.drop_out_points_by_radius;
+    vp.radius_threshold = a->params.drop_out_radius_threshold;
+    vp.viewer_only      = a->params.viewer_only;
+    vp.stability_cutoff = a->params.stability_cutoff_value;
+    return vp;
+}
+
+}  // namespace
+
+extern "C" {
+
+int vetrast_create(vetrast_ctx** out_ctx)
+{
+    if (!out_ctx) return VETRAST_ERR_INVALID_ARG;
+    *out_ctx         = nullptr;
+    vetrast_ctx* ctx = new (std::nothrow) vetrast_ctx();
+    if (!ctx) return VETRAST_ERR_INVALID_ARG;
+    hipError_t e = hipGetDevice(&ctx->device);
+    if (e != hipSuccess)
+    {
+        delete ctx;
+        return VETRAST_ERR_HIP;
+    }
+    *out_ctx = ctx;
+    return VETRAST_OK;
+}
+
+void vetrast_destroy(vetrast_ctx* ctx)
+{
+    if (!ctx) return;
+    for (auto& s : ctx->spans)
+    {
+        (void)hipEventDestroy(s.start);
+        (void)hipEventDestroy(s.stop);
+    }
+    for (auto e : ctx->free_events) (void)hipEventDestroy(e);
+    delete ctx;
+}
+
+int vetrast_layer_sizes(int32_t w, int32_t h, int32_t num_layers, int32_t* layer_w, int32_t* layer_h)
+{
+    if (!layer_w || !layer_h || num_layers < 1 || num_layers > VETRAST_MAX_LAYERS || w < 1 || h < 1)
+        return VETRAST_ERR_INVALID_ARG;
+    for (int l = 0; l < num_layers; ++l)
+    {
+        layer_w[l] = w;
+        layer_h[l] = h;
+        w /= 2;
+        h /= 2;
+    }
+    return VETRAST_OK;
+}
+
+int vetrast_workspace_layout_for(int32_t N, int32_t B, int32_t L, int32_t w, int32_t h, vetrast_workspace_layout* lay)
+{
+    if (!lay) return VETRAST_ERR_INVALID_ARG;
+    int st = check_dims(N, B, L, w, h);
+    if (st != VETRAST_OK) return st;
+    std::memset(lay, 0, sizeof(*lay));
+    LayerTable t = make_layer_table(w, h, L);
+    for (int l = 0; l < L; ++l)
+    {
+        lay->layer_w[l] = t.w[l];
+        lay->layer_h[l] = t.h[l];
+    }
+    for (int l = 0; l <= VETRAST_MAX_LAYERS; ++l) lay->layer_pixel_base[l] = t.base[l < L ? l : L];
+    const size_t P         = t.base[L];
+    const size_t Ppad      = align_up(P + 1, kScanPerBlock);
+    const size_t cap       = (size_t)N * L;
+    lay->fragment_capacity = (int64_t)cap;
+    size_t at              = 0;
+    lay->flags_base        = at;
+    at += kAlign;
+    lay->offsets_base   = at;
+    lay->offsets_stride = Ppad * sizeof(uint32_t);
+    at += lay->offsets_stride * B;
+    lay->scan_partials_base = at;
+    at += align_up((Ppad / kScanPerBlock) * sizeof(uint32_t), kAlign);
+    lay->views_base = at;
+    at += align_up((size_t)B * sizeof(DeviceView), kAlign);
+    lay->packed_base = at;
+    at += align_up((size_t)N * kPackedFloats * sizeof(float), kAlign);
+    lay->slots_base = at;
+    at += align_up(cap * sizeof(uint32_t), kAlign);
+    lay->weight_base   = at;
+    lay->weight_stride = align_up(P * sizeof(float), kAlign);
+    at += lay->weight_stride * B;
+    lay->fragments_base   = at;
+    lay->fragments_stride = align_up(cap * sizeof(uint64_t), kAlign);
+    at += lay->fragments_stride * B;
+    lay->transmittance_base   = at;
+    lay->transmittance_stride = align_up(cap * sizeof(float), kAlign);
+    at += lay->transmittance_stride * B;
+    lay->total_bytes = align_up(at, kAlign);
+    return VETRAST_OK;
+}
+
+size_t vetrast_forward_workspace_bytes(int32_t N, int32_t B, int32_t L, int32_t w, int32_t h)
+{
+    vetrast_workspace_layout lay;
+    if (vetrast_workspace_layout_for(N, B, L, w, h, &lay) != VETRAST_OK) return 0;
+    return lay.total_bytes;
+}
+
+int vetrast_forward(vetrast_ctx* ctx, const vetrast_forward_args* a, void* stream_)
+{
+    if (!ctx) return VETRAST_ERR_INVALID_ARG;
+    vetrast_workspace_layout lay;
+    int st = validate_forward(a, &lay);
+    if (st != VETRAST_OK) return st;
+    hipStream_t stream      = (hipStream_t)stream_;
+    const vetrast_params& p = a->params;
+    const int N = a->num_points, B = a->num_views, L = p.num_layers, C = p.num_texture_channels;
+    const LayerTable ly = make_layer_table(a->views[0].w, a->views[0].h, L);
+    const uint32_t P    = ly.base[L];
+    const size_t Ppad   = lay.offsets_stride / sizeof(uint32_t);
+    void* ws            = a->workspace;
+    uint32_t* flags     = ws_ptr<uint32_t>(ws, lay.flags_base);
+    float4* packed      = ws_ptr<float4>(ws, lay.packed_base);
+    uint32_t* slots     = ws_ptr<uint32_t>(ws, lay.slots_base);
+    uint32_t* partials  = ws_ptr<uint32_t>(ws, lay.scan_partials_base);
+    DeviceView* views   = ws_ptr<DeviceView>(ws, lay.views_base);
+
+    {
+        ScopeTimer tm(ctx, stream, VETRAST_SCOPE_PREPARE);
+        // per-pixel counters of all views (contiguous) start at zero; InitializeData, PointRenderer.cu:402-470
+        const size_t n4 = Ppad * B / 4;
+        hipLaunchKernelGGL(fill_u128_kernel, dim3(std::min(grid_for(n4), 4096)), dim3(kBlock), 0, stream,
+                           ws_ptr<uint4>(ws, lay.offsets_base), n4, 0u);
+        hipLaunchKernelGGL(fill_u32_kernel, dim3(1), dim3(kWave), 0, stream, flags, (size_t)4, 0u);
+        for (int first = 0; first < B; first += 16)
+        {
+            PrepareViewsArgs pv;
+            const int cnt = std::min(16, B - first);
+            for (int k = 0; k < cnt; ++k)
+            {
+                const vetrast_view& v = a->views[first + k];
+                ViewSource& s         = pv.src[k];
+                s.image_index         = v.image_index;
+                s.camera_index        = v.camera_index;
+                s.w                   = v.w;
+                s.h                   = v.h;
+                for (int j = 0; j < 5; ++j) s.crop[j] = v.crop_transform[j];
+                for (int j = 0; j < 4; ++j) s.rot[j] = v.crop_rotation[j];
+            }
+            hipLaunchKernelGGL(prepare_views_kernel, dim3(1), dim3(kWave), 0, stream, pv, first, cnt, a->poses_se3,
+                               a->intrinsics, views, flags);
+        }
+        if (N > 0)
+        {
+            const dim3 g(grid_for(N)), blk(kBlock);
+            switch (C)
+            {
+                case 1: hipLaunchKernelGGL(pack_descriptors_kernel<1>, g, blk, 0, stream, a->texture, a->confidence, packed, N); break;
+                case 2: hipLaunchKernelGGL(pack_descriptors_kernel<2>, g, blk, 0, stream, a->texture, a->confidence, packed, N); break;
+                case 3: hipLaunchKernelGGL(pack_descriptors_kernel<3>, g, blk, 0, stream, a->texture, a->confidence, packed, N); break;
+                default: hipLaunchKernelGGL(pack_descriptors_kernel<4>, g, blk, 0, stream, a->texture, a->confidence, packed, N); break;
+            }
+        }
+    }
+
+    for (int b = 0; b < B; ++b)
+    {
+        const ViewPass vp   = make_view_pass(a, lay, ly, b);
+        uint32_t* offsets   = ws_ptr<uint32_t>(ws, lay.offsets_base + lay.offsets_stride * b);
+        uint64_t* fragments = ws_ptr<uint64_t>(ws, lay.fragments_base + lay.fragments_stride * b);
+        float* trans        = ws_ptr<float>(ws, lay.transmittance_base + lay.transmittance_stride * b);
+        float* weight       = ws_ptr<float>(ws, lay.weight_base + lay.weight_stride * b);
+        if (N > 0)
+        {
+            ScopeTimer tm(ctx, stream, VETRAST_SCOPE_COUNT);
+            hipLaunchKernelGGL(count_kernel, dim3(grid_for(N)), dim3(kBlock), 0, stream, vp, offsets, slots);
+        }
+        {
+            ScopeTimer tm(ctx, stream, VETRAST_SCOPE_SCAN);
+            const int blocks = (int)(Ppad / kScanPerBlock);
+            hipLaunchKernelGGL(scan_partials_kernel, dim3(blocks), dim3(kBlock), 0, stream,
+                               reinterpret_cast<const uint4*>(offsets), partials);
+            hipLaunchKernelGGL(scan_apply_kernel, dim3(blocks), dim3(kBlock), 0, stream,
+                               reinterpret_cast<uint4*>(offsets), partials);
+        }
+        if (N > 0)
+        {
+            ScopeTimer tm(ctx, stream, VETRAST_SCOPE_FILL);
+            hipLaunchKernelGGL(fill_kernel, dim3(grid_for(N)), dim3(kBlock), 0, stream, vp, offsets, slots, fragments,
+                               (uint32_t)lay.fragment_capacity);
+        }
+        if (N > 0)
+        {
+            ScopeTimer tm(ctx, stream, VETRAST_SCOPE_SORT);
+            hipLaunchKernelGGL(sort_lists_kernel, dim3(grid_for(P)), dim3(kBlock), 0, stream, offsets, fragments, P,
+                               p.debug_max_list_length);
+        }
+        {
+            ScopeTimer tm(ctx, stream, VETRAST_SCOPE_BLEND);
+            BlendPass bp;
+            bp.offsets             = offsets;
+            bp.fragments           = fragments;
+            bp.index               = a->index;
+            bp.packed              = packed;
+            bp.background          = a->background;
+            bp.transmittance       = a->save_for_backward ? trans : nullptr;
+            bp.weight              = weight;
+            bp.ly                  = ly;
+            bp.P                   = P;
+            bp.N                   = N;
+            bp.K                   = p.debug_max_list_length;
+            bp.use_environment_map = p.use_environment_map;
+            bp.mask_value          = p.output_background_mask_value;
+            for (int l = 0; l < VETRAST_MAX_LAYERS; ++l)
+            {
+                bp.out[l]      = nullptr;
+                bp.out_mask[l] = nullptr;
+                if (l >= L) continue;
+                const size_t plane = (size_t)ly.w[l] * ly.h[l];
+                bp.out[l]          = a->out[l] + (size_t)b * C * plane;
+                if (p.output_background_mask) bp.out_mask[l] = a->out_mask[l] + (size_t)b * plane;
+            }
+            const dim3 g(grid_for(P)), blk(kBlock);
+            switch (C)
+            {
+                case 1: hipLaunchKernelGGL(blend_kernel<1>, g, blk, 0, stream, bp); break;
+                case 2: hipLaunchKernelGGL(blend_kernel<2>, g, blk, 0, stream, bp); break;
+                case 3: hipLaunchKernelGGL(blend_kernel<3>, g, blk, 0, stream, bp); break;
+                default: hipLaunchKernelGGL(blend_kernel<4>, g, blk, 0, stream, bp); break;
+            }
+        }
+    }
+    VET_HIP(ctx, hipGetLastError());
+    return VETRAST_OK;
+}
+
+int vetrast_backward(vetrast_ctx* ctx, const vetrast_backward_args* g, void* stream_)
+{
+    if (!ctx || !g) return VETRAST_ERR_INVALID_ARG;
+    const vetrast_forward_args* a = &g->fwd;
+    vetrast_workspace_layout lay;
+    int st = validate_forward(a, &lay);
+    if (st != VETRAST_OK) return st;
+    if (!a->save_for_backward) return VETRAST_ERR_INVALID_ARG;
+    if (!g->grad_texture || !g->grad_confidence || !g->grad_background) return VETRAST_ERR_INVALID_ARG;
+    if (g->grad_points && !g->grad_point_count) return VETRAST_ERR_INVALID_ARG;
+    if (g->grad_points && ((uintptr_t)g->grad_points % 16) != 0) return VETRAST_ERR_INVALID_ARG;
+    const vetrast_params& p = a->params;
+    for (int l = 0; l < p.num_layers; ++l)
+        if (!g->grad_out[l]) return VETRAST_ERR_INVALID_ARG;
+    hipStream_t stream = (hipStream_t)stream_;
+    const int N = a->num_points, B = a->num_views, L = p.num_layers, C = p.num_texture_channels;
+    const LayerTable ly = make_layer_table(a->views[0].w, a->views[0].h, L);
+    const uint32_t P    = ly.base[L];
+    void* ws            = a->workspace;
+
+    {
+        // zeros_like of every gradient tensor, PointRenderer.cu:267-277
+        ScopeTimer tm(ctx, stream, VETRAST_SCOPE_BACKWARD_PREPARE);
+        auto zero = [&](float* ptr, size_t n) {
+            if (!ptr || n == 0) return;
+            hipLaunchKernelGGL(fill_u32_kernel, dim3(std::min(grid_for(n), 8192)), dim3(kBlock), 0, stream,
+                               reinterpret_cast<uint32_t*>(ptr), n, 0u);
+        };
+        zero(g->grad_texture, (size_t)C * N);
+        zero(g->grad_confidence, (size_t)N);
+        zero(g->grad_background, (size_t)C);
+        if (g->grad_points)
+        {
+            zero(g->grad_points, (size_t)4 * N);
+            zero(g->grad_point_count, (size_t)N);
+        }
+    }
+    for (int b = 0; b < B; ++b)
+    {
+        ScopeTimer tm(ctx, stream, VETRAST_SCOPE_BACKWARD_BLEND);
+        BackwardPass bp;
+        bp.offsets          = ws_ptr<uint32_t>(ws, lay.offsets_base + lay.offsets_stride * b);
+        bp.fragments        = ws_ptr<uint64_t>(ws, lay.fragments_base + lay.fragments_stride * b);
+        bp.transmittance    = ws_ptr<float>(ws, lay.transmittance_base + lay.transmittance_stride * b);
+        bp.weight           = ws_ptr<float>(ws, lay.weight_base + lay.weight_stride * b);
+        bp.index            = a->index;
+        bp.packed           = ws_ptr<float4>(ws, lay.packed_base);
+        bp.position         = reinterpret_cast<const float4*>(a->position);
+        bp.background       = a->background;
+        bp.view             = ws_ptr<DeviceView>(ws, lay.views_base) + b;
+        bp.grad_texture     = g->grad_texture;
+        bp.grad_confidence  = g->grad_confidence;
+        bp.grad_background  = g->grad_background;
+        bp.grad_points      = g->grad_points;
+        bp.grad_point_count = g->grad_point_count;
+        bp.ly               = ly;
+        bp.P                = P;
+        bp.N                = N;
+        bp.K                = p.debug_max_list_length;
+        bp.use_environment_map              = p.use_environment_map;
+        bp.need_point_gradient              = p.need_point_gradient;
+        bp.quirk_background_confidence_leak = p.quirk_background_confidence_leak;
+        for (int l = 0; l < VETRAST_MAX_LAYERS; ++l)
+        {
+            bp.grad_out[l] = nullptr;
+            bp.out[l]      = nullptr;
+            if (l >= L) continue;
+            const size_t plane = (size_t)ly.w[l] * ly.h[l];
+            bp.grad_out[l]     = g->grad_out[l] + (size_t)b * C * plane;
+            bp.out[l]          = a->out[l] + (size_t)b * C * plane;
+        }
+        const dim3 grid(grid_for(P)), blk(kBlock);
+        switch (C)
+        {
+            case 1: hipLaunchKernelGGL(blend_backward_kernel<1>, grid, blk, 0, stream, bp); break;
+            case 2: hipLaunchKernelGGL(blend_backward_kernel<2>, grid, blk, 0, stream, bp); break;
+            case 3: hipLaunchKernelGGL(blend_backward_kernel<3>, grid, blk, 0, stream, bp); break;
+            default: hipLaunchKernelGGL(blend_backward_kernel<4>, grid, blk, 0, stream, bp); break;
+        }
+    }
+    if (g->grad_points && p.point_gradient_normalization != 0 && N > 0)
+    {
+        ScopeTimer tm(ctx, stream, VETRAST_SCOPE_BACKWARD_POST);
+        hipLaunchKernelGGL(normalize_point_gradient_kernel, dim3(grid_for(N)), dim3(kBlock), 0, stream,
+                           g->grad_points, g->grad_point_count, N, p.point_gradient_normalization);
+    }
+    VET_HIP(ctx, hipGetLastError());
+    return VETRAST_OK;
+}
+
+int vetrast_query_device_flags(vetrast_ctx* ctx, const void* workspace, const vetrast_workspace_layout* layout,
+                               void* stream)
+{
+    if (!ctx || !workspace || !layout) return VETRAST_ERR_INVALID_ARG;
+    uint32_t flags[4] = {0, 0, 0, 0};
+    VET_HIP(ctx, hipStreamSynchronize((hipStream_t)stream));
+    VET_HIP(ctx, hipMemcpy(flags, static_cast<const char*>(workspace) + layout->flags_base, sizeof(flags),
+                           hipMemcpyDeviceToHost));
+    return (flags[0] & 1u) ? VETRAST_ERR_BAD_INPUT_DATA : VETRAST_OK;
+}
+
+int vetrast_set_profiling(vetrast_ctx* ctx, int32_t enabled)
+{
+    if (!ctx) return VETRAST_ERR_INVALID_ARG;
+    ctx->profiling = enabled ? 1 : 0;
+    return VETRAST_OK;
+}
+
+static int collect_spans(vetrast_ctx* ctx)
+{
+    for (auto& s : ctx->spans)
+    {
+        VET_HIP(ctx, hipEventSynchronize(s.stop));
+        float ms = 0.f;
+        VET_HIP(ctx, hipEventElapsedTime(&ms, s.start, s.stop));
+        ctx->acc_ms[s.scope] += ms;
+        ctx->acc_launches[s.scope] += 1;
+        ctx->free_events.push_back(s.start);
+        ctx->free_events.push_back(s.stop);
+    }
+    ctx->spans.clear();
+    return VETRAST_OK;
+}
+
+int vetrast_reset_scope_times(vetrast_ctx* ctx)
+{
+    if (!ctx) return VETRAST_ERR_INVALID_ARG;
+    int st = collect_spans(ctx);
+    for (int i = 0; i < VETRAST_SCOPE_COUNT_; ++i)
+    {
+        ctx->acc_ms[i]       = 0.f;
+        ctx->acc_launches[i] = 0;
+    }
+    return st;
+}
+
+int vetrast_scope_times(vetrast_ctx* ctx, float* ms, int32_t* launches)
+{
+    if (!ctx || !ms || !launches) return VETRAST_ERR_INVALID_ARG;
+    int st = collect_spans(ctx);
+    for (int i = 0; i < VETRAST_SCOPE_COUNT_; ++i)
+    {
+        ms[i]       = ctx->acc_ms[i];
+        launches[i] = ctx->acc_launches[i];
+    }
+    return st;
+}
+
+const char* vetrast_scope_name(int32_t scope)
+{
+    switch (scope)
+    {
+        case VETRAST_SCOPE_PREPARE: return "Build Cache";
+        case VETRAST_SCOPE_COUNT: return "CountingPass";
+        case VETRAST_SCOPE_SCAN: return "CreateAndAllocateBuffers";
+        case VETRAST_SCOPE_FILL: return "CollectionPass";
+        case VETRAST_SCOPE_SORT: return "SortingPass";
+        case VETRAST_SCOPE_BLEND: return "BlendingPass";
+        case VETRAST_SCOPE_BACKWARD_PREPARE: return "Prepare Backward";
+        case VETRAST_SCOPE_BACKWARD_BLEND: return "BlendBackwards";
+        case VETRAST_SCOPE_BACKWARD_POST: return "Post Process Gradient";
+        default: return "?";
+    }
+}
+
+const char* vetrast_status_string(int status)
+{
+    switch (status)
+    {
+        case VETRAST_OK: return "ok";
+        case VETRAST_ERR_INVALID_ARG: return "invalid argument";
+        case VETRAST_ERR_WORKSPACE_SMALL: return "workspace too small";
+        case VETRAST_ERR_HIP: return "HIP runtime error";
+        case VETRAST_ERR_UNSUPPORTED: return "feature outside the implemented blending path";
+        case VETRAST_ERR_BAD_INPUT_DATA: return "device-side input check failed (non-zero distortion)";
+        default: return "unknown status";
+    }
+}
+
+int vetrast_last_hip_error(const vetrast_ctx* ctx)
+{
+    return ctx ? ctx->last_hip_error : 0;
+}
+
+}  // extern "C"

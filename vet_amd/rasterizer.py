@@ -1,0 +1,223 @@
+"""Thin Python host over the C ABI (include/vetrast.h), with torch used only for device memory and streams.
+
+This is what tests and bench.py drive. It adds no arithmetic of its own and has no CPU path: without a GPU and the
+built HIP library every call raises.
+"""
+import ctypes as C
+from dataclasses import dataclass
+from typing import List, Optional
+
+import numpy as np
+import torch
+
+from . import abi
+from .synthetic import Scene
+
+
+def make_params(scene: Scene, **overrides) -> abi.Params:
+    """RenderParams of the blending path with the defaults the benchmark configurations use."""
+    p = abi.Params()
+    p.num_texture_channels = scene.num_channels
+    p.num_layers = scene.num_layers
+    p.debug_max_list_length = scene.max_list_length
+    p.use_environment_map = 0
+    p.need_point_gradient = 0
+    p.viewer_only = 0
+    p.stability_cutoff_value = 10000.0
+    p.drop_out_points_by_radius = 0
+    p.drop_out_radius_threshold = 0.6
+    p.output_background_mask = 0
+    p.output_background_mask_value = 0.0
+    p.check_normal = 0
+    p.quirk_background_confidence_leak = 0
+    p.point_gradient_normalization = 0
+    for k, v in {**scene.params, **overrides}.items():
+        if not hasattr(p, k):
+            raise AttributeError(f"vetrast_params has no field {k}")
+        setattr(p, k, v)
+    return p
+
+
+def make_views(scene: Scene):
+    arr = (abi.View * len(scene.views))()
+    for i, v in enumerate(scene.views):
+        arr[i].w, arr[i].h = v.w, v.h
+        arr[i].image_index, arr[i].camera_index = v.image_index, v.camera_index
+        arr[i].camera_model_type = v.camera_model_type
+        arr[i].crop_transform = (C.c_float * 5)(*v.crop_transform)
+        arr[i].crop_rotation = (C.c_float * 4)(*v.crop_rotation)
+    return arr
+
+
+def fill_forward_args(args: abi.ForwardArgs, scene: Scene, params: abi.Params, views, ptr):
+    """Common part for host (oracle) and device callers; `ptr(name)` returns the address of an input array or None."""
+    args.num_points = scene.num_points
+    args.num_views = len(scene.views)
+    args.num_poses = int(scene.poses_se3.shape[0])
+    args.num_cameras = int(scene.intrinsics.shape[0])
+    for name in ("position", "index", "texture", "confidence", "background", "dropout", "poses_se3", "intrinsics"):
+        setattr(args, name, ptr(name))
+    args.views = views
+    args.params = params
+
+
+@dataclass
+class ForwardResult:
+    out: List[torch.Tensor]
+    out_mask: List[Optional[torch.Tensor]]
+    workspace: torch.Tensor
+    layout: abi.WorkspaceLayout
+    args: abi.ForwardArgs
+    keep: tuple  # objects that must outlive `args`
+
+    def _view_array(self, base, stride, b, dtype, count):
+        nbytes = count * torch.empty((), dtype=dtype).element_size()
+        raw = self.workspace[base + stride * b: base + stride * b + nbytes]
+        return raw.view(dtype)
+
+    def total_pixels(self):
+        return int(self.layout.layer_pixel_base[self.args.params.num_layers])
+
+    def offsets(self, b=0):
+        """int64 numpy copy of the exclusive scan [P+1] of view b."""
+        P = self.total_pixels()
+        t = self._view_array(self.layout.offsets_base, self.layout.offsets_stride, b, torch.int32, P + 1)
+        return t.cpu().numpy().astype(np.int64) & 0xFFFFFFFF
+
+    def fragments(self, b=0):
+        """uint64 numpy copy of the fragment buffer of view b, cut to the number of fragments."""
+        total = int(self.offsets(b)[-1])
+        t = self._view_array(self.layout.fragments_base, self.layout.fragments_stride, b, torch.int64, total)
+        return t.cpu().numpy().view(np.uint64)
+
+    def transmittance(self, b=0):
+        total = int(self.offsets(b)[-1])
+        return self._view_array(self.layout.transmittance_base, self.layout.transmittance_stride, b, torch.float32,
+                                total).cpu().numpy()
+
+    def weight(self, b=0):
+        return self._view_array(self.layout.weight_base, self.layout.weight_stride, b, torch.float32,
+                                self.total_pixels()).cpu().numpy()
+
+
+class DeviceScene:
+    """Inputs of a Scene as torch tensors on the GPU."""
+
+    def __init__(self, scene: Scene, device="cuda:0"):
+        self.scene = scene
+        self.device = torch.device(device)
+        f = lambda a: None if a is None else torch.from_numpy(np.ascontiguousarray(a)).to(self.device)
+        self.position = f(scene.position)
+        self.index = f(scene.index)
+        self.texture = f(scene.texture)
+        self.confidence = f(scene.confidence)
+        self.background = f(scene.background)
+        self.dropout = f(scene.dropout)
+        self.poses_se3 = f(scene.poses_se3)
+        self.intrinsics = f(scene.intrinsics)
+
+    def ptr(self, name):
+        t = getattr(self, name)
+        return None if t is None else t.data_ptr()
+
+
+class Rasterizer:
+    """Owns a vetrast context; forward/backward enqueue on torch's current stream."""
+
+    def __init__(self):
+        if not torch.cuda.is_available():
+            raise RuntimeError("vet_amd.Rasterizer needs a GPU; there is no CPU path")
+        self.lib = abi.load_library()
+        h = C.c_void_p()
+        abi.check(self.lib.vetrast_create(C.byref(h)), "create")
+        self.ctx = h
+
+    def __del__(self):
+        try:
+            if getattr(self, "ctx", None):
+                self.lib.vetrast_destroy(self.ctx)
+                self.ctx = None
+        except Exception:
+            pass
+
+    @staticmethod
+    def _stream():
+        return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    def layout(self, scene: Scene) -> abi.WorkspaceLayout:
+        lay = abi.WorkspaceLayout()
+        v = scene.views[0]
+        abi.check(self.lib.vetrast_workspace_layout_for(scene.num_points, len(scene.views), scene.num_layers, v.w, v.h,
+                                                        C.byref(lay)), "workspace_layout_for")
+        return lay
+
+    def forward(self, dev: DeviceScene, params: abi.Params = None, save_for_backward=True, workspace=None,
+                out=None) -> ForwardResult:
+        scene = dev.scene
+        params = params or make_params(scene)
+        lay = self.layout(scene)
+        if workspace is None:
+            workspace = torch.empty(lay.total_bytes, dtype=torch.uint8, device=dev.device)
+        B, Cn = len(scene.views), scene.num_channels
+        sizes = scene.layer_sizes()
+        if out is None:
+            out = [torch.empty((B, Cn, h, w), dtype=torch.float32, device=dev.device) for (w, h) in sizes]
+        masks = [None] * len(sizes)
+        if params.output_background_mask:
+            masks = [torch.empty((B, 1, h, w), dtype=torch.float32, device=dev.device) for (w, h) in sizes]
+        args = abi.ForwardArgs()
+        views = make_views(scene)
+        fill_forward_args(args, scene, params, views, dev.ptr)
+        args.save_for_backward = 1 if save_for_backward else 0
+        for l in range(len(sizes)):
+            args.out[l] = out[l].data_ptr()
+            args.out_mask[l] = masks[l].data_ptr() if masks[l] is not None else None
+        args.workspace = workspace.data_ptr()
+        args.workspace_bytes = workspace.numel()
+        abi.check(self.lib.vetrast_forward(self.ctx, C.byref(args), self._stream()), "forward")
+        return ForwardResult(out, masks, workspace, lay, args, (views, dev, params))
+
+    def backward(self, fwd: ForwardResult, grad_out: List[torch.Tensor], want_points=True, **param_overrides):
+        dev = fwd.keep[1]
+        scene = dev.scene
+        N, Cn = scene.num_points, scene.num_channels
+        g = abi.BackwardArgs()
+        C.memmove(C.byref(g.fwd), C.byref(fwd.args), C.sizeof(abi.ForwardArgs))
+        for k, v in param_overrides.items():
+            setattr(g.fwd.params, k, v)
+        for l, t in enumerate(grad_out):
+            assert t.is_contiguous() and t.dtype == torch.float32
+            g.grad_out[l] = t.data_ptr()
+        res = {
+            "texture": torch.empty((Cn, N), dtype=torch.float32, device=dev.device),
+            "confidence": torch.empty((N,), dtype=torch.float32, device=dev.device),
+            "background": torch.empty((Cn,), dtype=torch.float32, device=dev.device),
+        }
+        g.grad_texture = res["texture"].data_ptr()
+        g.grad_confidence = res["confidence"].data_ptr()
+        g.grad_background = res["background"].data_ptr()
+        if want_points:
+            res["points"] = torch.empty((N, 4), dtype=torch.float32, device=dev.device)
+            res["point_count"] = torch.empty((N,), dtype=torch.float32, device=dev.device)
+            g.grad_points = res["points"].data_ptr()
+            g.grad_point_count = res["point_count"].data_ptr()
+        abi.check(self.lib.vetrast_backward(self.ctx, C.byref(g), self._stream()), "backward")
+        res["_args"] = g
+        return res
+
+    def check_device_flags(self, fwd: ForwardResult):
+        return self.lib.vetrast_query_device_flags(self.ctx, C.c_void_p(fwd.workspace.data_ptr()),
+                                                   C.byref(fwd.layout), self._stream())
+
+    # ---- per-kernel timing (the reference's timer_system) -------------------------------------------------------
+    def set_profiling(self, on: bool):
+        abi.check(self.lib.vetrast_set_profiling(self.ctx, 1 if on else 0), "set_profiling")
+
+    def reset_scope_times(self):
+        abi.check(self.lib.vetrast_reset_scope_times(self.ctx), "reset_scope_times")
+
+    def scope_times(self):
+        ms = (C.c_float * abi.SCOPE_COUNT)()
+        n = (C.c_int32 * abi.SCOPE_COUNT)()
+        abi.check(self.lib.vetrast_scope_times(self.ctx, ms, n), "scope_times")
+        return {abi.SCOPE_NAMES[i]: (float(ms[i]), int(n[i])) for i in range(abi.SCOPE_COUNT)}

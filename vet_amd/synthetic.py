@@ -1,0 +1,277 @@
+"""Seeded synthetic scenes for the rasterizer's five benchmark / parity configurations.
+
+All random numbers come from one in-repo counter-based generator (SplitMix64 finaliser over key + counter), evaluated
+on the host with numpy, so that the CPU check and the GPU path see identical bits. Uniforms use the top 24 bits, so
+they are exact in float32; normals are Box-Muller in float64, rounded once to float32.
+"""
+import math
+from dataclasses import dataclass, field
+from typing import List, Optional
+
+import numpy as np
+
+_GOLDEN = np.uint64(0x9E3779B97F4A7C15)
+_M1 = np.uint64(0xBF58476D1CE4E5B9)
+_M2 = np.uint64(0x94D049BB133111EB)
+_MASK = (1 << 64) - 1
+
+
+def _mix(z):
+    z = (z ^ (z >> np.uint64(30))) * _M1
+    z = (z ^ (z >> np.uint64(27))) * _M2
+    return z ^ (z >> np.uint64(31))
+
+
+def _fnv1a(tag: str) -> int:
+    h = 0xCBF29CE484222325
+    for ch in tag.encode():
+        h = ((h ^ ch) * 0x100000001B3) & _MASK
+    return h
+
+
+class Stream:
+    """Independent random stream per (seed, tag)."""
+
+    def __init__(self, seed: int, tag: str):
+        with np.errstate(over="ignore"):
+            k = np.array([(seed * 0x9E3779B97F4A7C15 + _fnv1a(tag)) & _MASK], dtype=np.uint64)
+            self.key = _mix(k)[0]
+        self.counter = 0
+
+    def u64(self, n: int) -> np.ndarray:
+        idx = np.arange(self.counter + 1, self.counter + n + 1, dtype=np.uint64)
+        self.counter += n
+        with np.errstate(over="ignore"):
+            return _mix(self.key + idx * _GOLDEN)
+
+    def uniform(self, n: int) -> np.ndarray:
+        """float64 in [0, 1) with 24 significant bits."""
+        return (self.u64(n) >> np.uint64(40)).astype(np.float64) / float(1 << 24)
+
+    def normal(self, n: int) -> np.ndarray:
+        u1 = ((self.u64(n) >> np.uint64(40)).astype(np.float64) + 1.0) / float(1 << 24)
+        u2 = (self.u64(n) >> np.uint64(40)).astype(np.float64) / float(1 << 24)
+        return np.sqrt(-2.0 * np.log(u1)) * np.cos(2.0 * math.pi * u2)
+
+
+def sigmoid(x):
+    return 1.0 / (1.0 + np.exp(-x))
+
+
+@dataclass
+class ViewSpec:
+    w: int
+    h: int
+    image_index: int = 0
+    camera_index: int = 0
+    camera_model_type: int = 0
+    crop_transform: tuple = (1.0, 1.0, 0.0, 0.0, 0.0)
+    crop_rotation: tuple = (1.0, 0.0, 0.0, 1.0)
+
+
+@dataclass
+class Scene:
+    """Host-side inputs of one render call (numpy, C-contiguous) in the layouts the C ABI expects."""
+    name: str
+    position: np.ndarray      # [N,4] f32
+    texture: np.ndarray       # [C,N] f32
+    confidence: np.ndarray    # [N] f32
+    background: np.ndarray    # [C] f32
+    poses_se3: np.ndarray     # [F,8] f64
+    intrinsics: np.ndarray    # [Ncam,13] f32
+    views: List[ViewSpec]
+    num_layers: int
+    max_list_length: int
+    seed: int
+    index: Optional[np.ndarray] = None    # [N] i32
+    dropout: Optional[np.ndarray] = None  # [B,N] f32
+    params: dict = field(default_factory=dict)
+
+    @property
+    def num_points(self):
+        return int(self.position.shape[0])
+
+    @property
+    def num_channels(self):
+        return int(self.texture.shape[0])
+
+    def layer_sizes(self):
+        w, h = self.views[0].w, self.views[0].h
+        out = []
+        for _ in range(self.num_layers):
+            out.append((w, h))
+            w //= 2
+            h //= 2
+        return out
+
+    def grad_out(self, seed_offset=0):
+        """Upstream gradient N(0,1) per output element, one array [B,C,h_l,w_l] per layer."""
+        res = []
+        B, Cn = len(self.views), self.num_channels
+        for l, (w, h) in enumerate(self.layer_sizes()):
+            st = Stream(self.seed + seed_offset, f"grad_out_{l}")
+            res.append(st.normal(B * Cn * h * w).astype(np.float32).reshape(B, Cn, h, w))
+        return res
+
+
+def _identity_pose(t):
+    return np.array([[0.0, 0.0, 0.0, 1.0, t[0], t[1], t[2], 0.0]], dtype=np.float64)
+
+
+def _intrinsics(fx, fy, cx, cy, s=0.0):
+    k = np.zeros((1, 13), dtype=np.float32)
+    k[0, :5] = [fx, fy, cx, cy, s]
+    return k
+
+
+def config1(num_points=20000, seed=0) -> Scene:
+    """Tiny case: uniform cube, 256x256, one layer, K=8, forward only."""
+    N = num_points
+    pos = np.empty((N, 4), dtype=np.float32)
+    pos[:, :3] = (Stream(seed, "position").uniform(3 * N).reshape(N, 3) - 0.5).astype(np.float32)
+    pos[:, 3] = 0.01
+    tex = Stream(seed, "texture").uniform(4 * N).reshape(4, N).astype(np.float32)
+    conf = sigmoid(Stream(seed, "confidence").normal(N)).astype(np.float32)
+    return Scene("config1_cube20k", pos, tex, conf, np.zeros(4, np.float32), _identity_pose((0, 0, 2.0)),
+                 _intrinsics(256, 256, 128, 128), [ViewSpec(256, 256)], num_layers=1, max_list_length=8, seed=seed)
+
+
+def _orthonormal_frame(n):
+    n = n / np.linalg.norm(n, axis=1, keepdims=True)
+    helper = np.where(np.abs(n[:, :1]) < 0.9, np.array([[1.0, 0.0, 0.0]]), np.array([[0.0, 1.0, 0.0]]))
+    u = np.cross(n, helper)
+    u /= np.linalg.norm(u, axis=1, keepdims=True)
+    v = np.cross(n, u)
+    return n, u, v
+
+
+def surface_points(seed, num_primitives, points_per_primitive, box=5.0, jitter=0.01, tag=""):
+    """Points on random plane patches and spheres inside [-box, box]^3 with N(0, jitter) noise, float64 [n,3]."""
+    Pn, M = num_primitives, points_per_primitive
+    st = Stream(seed, "primitives" + tag)
+    is_sphere = st.uniform(Pn) < 0.5
+    centre = (st.uniform(3 * Pn).reshape(Pn, 3) * 2.0 - 1.0) * box
+    normal = st.normal(3 * Pn).reshape(Pn, 3)
+    size = 0.5 + 1.5 * st.uniform(Pn)
+    n, u, v = _orthonormal_frame(normal)
+    sp = Stream(seed, "surface" + tag)
+    a = sp.uniform(Pn * M).reshape(Pn, M) * 2.0 - 1.0
+    b = sp.uniform(Pn * M).reshape(Pn, M) * 2.0 - 1.0
+    d = sp.normal(3 * Pn * M).reshape(Pn, M, 3)
+    d /= np.maximum(np.linalg.norm(d, axis=2, keepdims=True), 1e-12)
+    plane = centre[:, None, :] + size[:, None, None] * (a[..., None] * u[:, None, :] + b[..., None] * v[:, None, :])
+    sphere = centre[:, None, :] + (0.5 * size)[:, None, None] * d
+    pts = np.where(is_sphere[:, None, None], sphere, plane).reshape(Pn * M, 3)
+    pts += jitter * Stream(seed, "jitter" + tag).normal(3 * Pn * M).reshape(Pn * M, 3)
+    return pts
+
+
+def _descriptors(seed, N, channels=4, sigma=0.5):
+    tex = (sigma * Stream(seed, "texture").normal(channels * N)).reshape(channels, N).astype(np.float32)
+    conf = sigmoid(Stream(seed, "confidence").normal(N)).astype(np.float32)
+    bg = Stream(seed, "background").uniform(channels).astype(np.float32)
+    return tex, conf, bg
+
+
+def config2(num_points=2_000_000, seed=1, w=1920, h=1080, num_layers=4, K=16) -> Scene:
+    """SfM-like scene: points on 200 planes/spheres in a 10 m box, 1080p, fx=1000, 4 layers, K=16."""
+    prims = 200
+    per = max(1, num_points // prims)
+    N = prims * per
+    pos = np.empty((N, 4), dtype=np.float32)
+    pos[:, :3] = surface_points(seed, prims, per).astype(np.float32)
+    pos[:, 3] = 0.01
+    tex, conf, bg = _descriptors(seed, N)
+    scale = w / 1920.0
+    return Scene("config2_sfm", pos, tex, conf, bg, _identity_pose((0, 0, 4.5)),
+                 _intrinsics(1000 * scale, 1000 * scale, w / 2, h / 2), [ViewSpec(w, h)], num_layers=num_layers,
+                 max_list_length=K, seed=seed)
+
+
+def config3(num_points=2_000_000, seed=1, **kw) -> Scene:
+    """Config 2's scene with the backward pass: gradients to descriptors, confidence and xyz."""
+    s = config2(num_points=num_points, seed=seed, **kw)
+    s.name = "config3_sfm_fwd_bwd"
+    s.params["need_point_gradient"] = 1
+    return s
+
+
+def _random_poses(seed, B, extent=4.0):
+    st = Stream(seed, "poses")
+    q = st.normal(4 * B).reshape(B, 4)
+    q /= np.linalg.norm(q, axis=1, keepdims=True)
+    c = (st.uniform(3 * B).reshape(B, 3) * 2.0 - 1.0) * extent
+    poses = np.zeros((B, 8), dtype=np.float64)
+    for b in range(B):
+        x, y, z, w_ = q[b]
+        R = np.array([
+            [1 - 2 * (y * y + z * z), 2 * (x * y - w_ * z), 2 * (x * z + w_ * y)],
+            [2 * (x * y + w_ * z), 1 - 2 * (x * x + z * z), 2 * (y * z - w_ * x)],
+            [2 * (x * z - w_ * y), 2 * (y * z + w_ * x), 1 - 2 * (x * x + y * y)],
+        ])
+        poses[b, :4] = q[b]
+        poses[b, 4:7] = -R @ c[b]
+    return poses
+
+
+def config4(surface_points_n=4_000_000, sphere_points=500_000, seed=3, w=1920, h=1080, num_views=4, num_layers=4,
+            K=16) -> Scene:
+    """Surface points plus three nested environment spheres (r = 50/100/200 m), a batch of random views."""
+    prims = 400
+    per = max(1, surface_points_n // prims)
+    surf = surface_points(seed, prims, per)
+    shells = []
+    for k, r in enumerate((50.0, 100.0, 200.0)):
+        d = Stream(seed, f"sphere{k}").normal(3 * sphere_points).reshape(sphere_points, 3)
+        d /= np.maximum(np.linalg.norm(d, axis=1, keepdims=True), 1e-12)
+        shells.append(r * d)
+    xyz = np.concatenate([surf] + shells, axis=0)
+    N = xyz.shape[0]
+    pos = np.empty((N, 4), dtype=np.float32)
+    pos[:, :3] = xyz.astype(np.float32)
+    pos[:, 3] = 0.01
+    tex, conf, bg = _descriptors(seed, N)
+    scale = w / 1920.0
+    views = [ViewSpec(w, h, image_index=b) for b in range(num_views)]
+    s = Scene("config4_envspheres_batch", pos, tex, conf, bg, _random_poses(seed, num_views),
+              _intrinsics(1000 * scale, 1000 * scale, w / 2, h / 2), views, num_layers=num_layers, max_list_length=K,
+              seed=seed)
+    s.params["need_point_gradient"] = 1
+    return s
+
+
+def config5(num_points=10_000_000, seed=4, w=1920, h=1080, num_layers=4, K=16) -> Scene:
+    """Depth-complexity stress: a 1 m^3 cube of points filling the frustum."""
+    N = num_points
+    pos = np.empty((N, 4), dtype=np.float32)
+    xyz = Stream(seed, "position").uniform(3 * N).reshape(N, 3) - 0.5
+    xyz[:, 2] += 1.2
+    pos[:, :3] = xyz.astype(np.float32)
+    pos[:, 3] = 0.01
+    tex, conf, bg = _descriptors(seed, N)
+    scale = w / 1920.0
+    s = Scene("config5_depth_stress", pos, tex, conf, bg, _identity_pose((0, 0, 0)),
+              _intrinsics(1000 * scale, 1000 * scale, w / 2, h / 2), [ViewSpec(w, h)], num_layers=num_layers,
+              max_list_length=K, seed=seed)
+    s.params["need_point_gradient"] = 1
+    return s
+
+
+def tiny_scene(num_points=300, w=24, h=16, num_layers=3, K=4, seed=7, channels=4, num_views=1) -> Scene:
+    """A few hundred points on a small image: every pixel list is long enough to exercise sort and cut."""
+    N = num_points
+    st = Stream(seed, "tiny")
+    pos = np.empty((N, 4), dtype=np.float32)
+    pos[:, 0] = (st.uniform(N) * 2.4 - 1.2).astype(np.float32)
+    pos[:, 1] = (st.uniform(N) * 1.6 - 0.8).astype(np.float32)
+    pos[:, 2] = (st.uniform(N) * 2.0 - 0.5).astype(np.float32)
+    pos[:, 3] = (0.002 + 0.05 * st.uniform(N)).astype(np.float32)
+    tex = (0.5 * st.normal(channels * N)).reshape(channels, N).astype(np.float32)
+    conf = sigmoid(st.normal(N)).astype(np.float32)
+    bg = st.uniform(channels).astype(np.float32)
+    poses = _random_poses(seed, num_views, extent=0.2)
+    poses[:, :4] = [0, 0, 0, 1]
+    poses[:, 4:7] = np.array([[0.02 * b, -0.01 * b, 2.0 + 0.1 * b] for b in range(num_views)])
+    views = [ViewSpec(w, h, image_index=b) for b in range(num_views)]
+    return Scene("tiny", pos, tex, conf, bg, poses, _intrinsics(0.45 * w, 0.45 * w, w / 2.0, h / 2.0, 0.0), views,
+                 num_layers=num_layers, max_list_length=K, seed=seed)
