@@ -93,7 +93,8 @@ typedef enum vetrast_scope
     VETRAST_SCOPE_SORT,             /* "SortingPass" */
     VETRAST_SCOPE_BLEND,            /* "BlendingPass" */
     VETRAST_SCOPE_BACKWARD_PREPARE, /* "Prepare Backward": zero-fill of gradient buffers */
-    VETRAST_SCOPE_BACKWARD_BLEND,   /* "BlendBackwards" */
+    VETRAST_SCOPE_BACKWARD_BLEND,   /* "BlendBackwards", per-pixel part */
+    VETRAST_SCOPE_BACKWARD_GATHER,  /* "BlendBackwards", per-point sum of the stored fragment gradients */
     VETRAST_SCOPE_BACKWARD_POST,    /* "Post Process Gradient" */
     VETRAST_SCOPE_COUNT_
 } vetrast_scope;
@@ -119,6 +120,8 @@ typedef struct vetrast_workspace_layout
     size_t views_base;     /* prepared per-view camera constants */
     size_t scan_partials_base;
     size_t flags_base;     /* uint32 [4] device status flags */
+    size_t forward_only_bytes; /* a forward call with save_for_backward = 0 needs only this much */
+    size_t partial_base;   /* float [L][N][8]: backward scratch, gradient record of the fragment of point i in layer l */
 } vetrast_workspace_layout;
 
 /* Arguments of the forward pass. Replaces the inputs PointRender::forward receives

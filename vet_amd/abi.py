@@ -20,7 +20,7 @@ CAMERA_OCAM = 1
 CAMERA_SPHERICAL = 2
 
 SCOPE_NAMES = [
-    "PREPARE", "COUNT", "SCAN", "FILL", "SORT", "BLEND", "BACKWARD_PREPARE", "BACKWARD_BLEND", "BACKWARD_POST",
+    "PREPARE", "COUNT", "SCAN", "FILL", "SORT", "BLEND", "BACKWARD_PREPARE", "BACKWARD_BLEND", "BACKWARD_GATHER", "BACKWARD_POST",
 ]
 SCOPE_COUNT = len(SCOPE_NAMES)
 
@@ -69,6 +69,8 @@ class WorkspaceLayout(C.Structure):
         ("views_base", C.c_size_t),
         ("scan_partials_base", C.c_size_t),
         ("flags_base", C.c_size_t),
+        ("forward_only_bytes", C.c_size_t),
+        ("partial_base", C.c_size_t),
     ]
 
 

@@ -1,4 +1,11 @@
 // Backward kernels: gradients of the blend with respect to descriptors, confidence, background and point positions.
+//
+// A point lands in exactly one pixel per layer, so a fragment is identified by (layer, point id). The per-pixel kernel
+// therefore STORES each kept fragment's gradient contribution as one 32-byte record at partial[layer][point] instead
+// of adding it to the gradient tensors with global atomics, and a per-point kernel sums a point's (at most L) records
+// in a fixed order and writes the gradient tensors with plain coalesced stores. Device-scope float atomics, which the
+// reference issues per fragment and channel (src/lib/rendering/RenderBackward.cu:1152,1157,1177,1405-1407), were the
+// single largest cost on MI355X; without them the gradients are also reproducible run to run.
 #pragma once
 #include "common.h"
 
@@ -17,11 +24,9 @@ struct BackwardPass
     const DeviceView* view;
     const float* grad_out[VETRAST_MAX_LAYERS];  // already offset to this view
     const float* out[VETRAST_MAX_LAYERS];       // forward result, already offset to this view
-    float* grad_texture;     // [C,N]
-    float* grad_confidence;  // [N]
-    float* grad_background;  // [C]
-    float* grad_points;      // [N,4] or null
-    float* grad_point_count; // [N]
+    float4* partial;          // [L][N] records of 2 float4: (d tex0..3), (d conf, d x, d y, d z)
+    float* grad_background;   // [C]
+    float* grad_confidence;   // [N]; only touched for the background leak switch
     LayerTable ly;
     uint32_t P;
     int N;
@@ -36,6 +41,13 @@ __device__ __forceinline__ float wave_sum(float v)
 #pragma unroll
     for (int d = kWave / 2; d >= 1; d >>= 1) v += __shfl_xor(v, d, kWave);
     return v;
+}
+
+// Pixels closer than 3 to the border get no position gradient: distanceFromEdge(y, x) > 2,
+// src/lib/rendering/RenderBackward.cu:1187.
+__device__ __forceinline__ bool interior_pixel(int x, int y, int w, int h)
+{
+    return min(min(x, y), min(w - 1 - x, h - 1 - y)) > 2;
 }
 
 // One thread per pixel, all layers of a view in one launch. The list is walked back to front with the transmittance
@@ -91,8 +103,7 @@ __global__ void __launch_bounds__(kBlock) blend_backward_kernel(BackwardPass a)
         }
 
         // neighbour samples for the position heuristic, shared by every fragment of the pixel
-        const int edge      = min(min(gx, gy), min(lw - 1 - gx, lh - 1 - gy));
-        const bool do_point = a.need_point_gradient && a.grad_points && edge > 2 && n > 0;
+        const bool do_point = a.need_point_gradient && n > 0 && interior_pixel(gx, gy, lw, lh);
         float Ix0[C], Ix1[C], Iy0[C], Iy1[C], Gx0[C], Gx1[C], Gy0[C], Gy1[C];
         float cfx = 0.f, cfy = 0.f, cs = 0.f;
         if (do_point)
@@ -120,6 +131,7 @@ __global__ void __launch_bounds__(kBlock) blend_backward_kernel(BackwardPass a)
 
         const uint64_t* list = a.fragments + off;
         const float* Tlist   = a.transmittance + off;
+        float4* partial_l    = a.partial + 2 * (size_t)l * a.N;
         for (int j = (int)n - 1; j >= 0; --j)
         {
             const int id = (int)(uint32_t)list[j];
@@ -132,16 +144,18 @@ __global__ void __launch_bounds__(kBlock) blend_backward_kernel(BackwardPass a)
             const float t[4] = {t4.x, t4.y, t4.z, t4.w};
             float dot = 0.f, x = 0.f;
             const float Tc = T * c;
+            float gt[4]    = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int ci = 0; ci < C; ++ci)
             {
-                atomicAdd(&a.grad_texture[(size_t)ci * a.N + ti], Tc * g[ci]);
+                gt[ci] = Tc * g[ci];
                 dot += t[ci] * g[ci];
                 x += ((g[ci] * t[ci]) * T) * c;
             }
-            atomicAdd(&a.grad_confidence[ti], dot * T - S / ((1.f - c) + 1e-9f));
+            const float gconf = dot * T - S / ((1.f - c) + 1e-9f);
             S += x;
 
+            float gp0 = 0.f, gp1 = 0.f, gp2 = 0.f;
             if (do_point)
             {
                 float dR_dpx = 0.f, dR_dpy = 0.f;
@@ -161,7 +175,6 @@ __global__ void __launch_bounds__(kBlock) blend_backward_kernel(BackwardPass a)
                 const float vx = ((cam.r[0] * p.x + cam.r[1] * p.y) + cam.r[2] * p.z) + cam.t[0];
                 const float vy = ((cam.r[3] * p.x + cam.r[4] * p.y) + cam.r[5] * p.z) + cam.t[1];
                 const float vz = ((cam.r[6] * p.x + cam.r[7] * p.y) + cam.r[8] * p.z) + cam.t[2];
-                float gp0 = 0.f, gp1 = 0.f, gp2 = 0.f;
                 if (vz > 0.f)
                 {
                     const float ar = cam.rot[0] * gxp + cam.rot[2] * gyp;
@@ -177,12 +190,9 @@ __global__ void __launch_bounds__(kBlock) blend_backward_kernel(BackwardPass a)
                     gp1            = (cam.r[1] * e0 + cam.r[4] * e1) + cam.r[7] * e2;
                     gp2            = (cam.r[2] * e0 + cam.r[5] * e1) + cam.r[8] * e2;
                 }
-                float* gpt = a.grad_points + 4 * (size_t)id;
-                atomicAdd(gpt + 0, gp0);
-                atomicAdd(gpt + 1, gp1);
-                atomicAdd(gpt + 2, gp2);
-                atomicAdd(a.grad_point_count + id, 1.f);
             }
+            partial_l[2 * (size_t)id]     = make_float4(gt[0], gt[1], gt[2], gt[3]);
+            partial_l[2 * (size_t)id + 1] = make_float4(gconf, gp0, gp1, gp2);
         }
     }
 
@@ -201,6 +211,106 @@ __global__ void __launch_bounds__(kBlock) blend_backward_kernel(BackwardPass a)
         {
             const float s = wave_sum(leak);
             if (lane == 0 && s != 0.f) atomicAdd(&a.grad_confidence[0], s);
+        }
+    }
+}
+
+struct GatherPass
+{
+    ViewPass vp;
+    const uint32_t* offsets;
+    const uint64_t* fragments;
+    const float4* partial;
+    float* grad_texture;      // [C,N]
+    float* grad_confidence;   // [N]
+    float* grad_points;       // [N,4] or null
+    float* grad_point_count;  // [N]
+    int K;
+    int need_point_gradient;
+    int accumulate;  // 0: overwrite the gradient rows (first view), 1: add to them (further views)
+};
+
+// One thread per point: find the pixel the point fell into in every layer (the same projection as the count pass), decide
+// whether its fragment survived the top-K cut (its key is not larger than the K-th key of that pixel's sorted list), and
+// sum the stored records. With a texture index indirection several points may share a descriptor row; only then the
+// descriptor and confidence sums are added with atomics (onto rows the host zero-filled).
+template <int C>
+__global__ void __launch_bounds__(kBlock) gather_point_gradients_kernel(GatherPass a)
+{
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= a.vp.N) return;
+    float gt[C];
+#pragma unroll
+    for (int ci = 0; ci < C; ++ci) gt[ci] = 0.f;
+    float gc = 0.f, gx = 0.f, gy = 0.f, gz = 0.f, cnt = 0.f;
+    Projected p;
+    if (!point_is_skipped(a.vp, i) && project_point(*a.vp.view, a.vp.position[i], p))
+    {
+        const uint64_t key = ((uint64_t)__float_as_uint(p.z) << 32) | (uint32_t)i;
+        float ipx = p.ipx, ipy = p.ipy, radius = p.radius;
+        const LayerTable& ly = a.vp.ly;
+        for (int l = 0; l < ly.L; ++l, radius *= 0.5f, ipx *= 0.5f, ipy *= 0.5f)
+        {
+            if (a.vp.drop_by_radius && radius < a.vp.radius_threshold) break;
+            const float fx = rintf(ipx), fy = rintf(ipy);
+            if (!(fx >= 0.f && fx < (float)ly.w[l] && fy >= 0.f && fy < (float)ly.h[l])) continue;
+            const int x = (int)fx, y = (int)fy;
+            const uint32_t q   = ly.base[l] + (uint32_t)y * (uint32_t)ly.w[l] + (uint32_t)x;
+            const uint32_t off = a.offsets[q];
+            const uint32_t n   = a.offsets[q + 1] - off;
+            if (a.K > 0 && n > (uint32_t)a.K && key > a.fragments[off + a.K - 1]) continue;  // cut away
+            const float4 r0 = a.partial[2 * ((size_t)l * a.vp.N + i)];
+            const float4 r1 = a.partial[2 * ((size_t)l * a.vp.N + i) + 1];
+            const float r[4] = {r0.x, r0.y, r0.z, r0.w};
+#pragma unroll
+            for (int ci = 0; ci < C; ++ci) gt[ci] += r[ci];
+            gc += r1.x;
+            if (a.need_point_gradient && interior_pixel(x, y, ly.w[l], ly.h[l]))
+            {
+                gx += r1.y;
+                gy += r1.z;
+                gz += r1.w;
+                cnt += 1.f;
+            }
+        }
+    }
+    const int N = a.vp.N;
+    if (a.vp.index)
+    {
+        const int ti = a.vp.index[i];
+        if ((uint32_t)ti < (uint32_t)N)
+        {
+#pragma unroll
+            for (int ci = 0; ci < C; ++ci)
+                if (gt[ci] != 0.f) atomicAdd(&a.grad_texture[(size_t)ci * N + ti], gt[ci]);
+            if (gc != 0.f) atomicAdd(&a.grad_confidence[ti], gc);
+        }
+    }
+    else if (a.accumulate)
+    {
+#pragma unroll
+        for (int ci = 0; ci < C; ++ci) a.grad_texture[(size_t)ci * N + i] += gt[ci];
+        a.grad_confidence[i] += gc;
+    }
+    else
+    {
+#pragma unroll
+        for (int ci = 0; ci < C; ++ci) a.grad_texture[(size_t)ci * N + i] = gt[ci];
+        a.grad_confidence[i] = gc;
+    }
+    if (a.grad_points)
+    {
+        float4* gp = reinterpret_cast<float4*>(a.grad_points) + i;
+        if (a.accumulate)
+        {
+            const float4 o = *gp;
+            *gp            = make_float4(o.x + gx, o.y + gy, o.z + gz, 0.f);
+            a.grad_point_count[i] += cnt;
+        }
+        else
+        {
+            *gp                   = make_float4(gx, gy, gz, 0.f);
+            a.grad_point_count[i] = cnt;
         }
     }
 }

@@ -8,10 +8,10 @@
 #include <new>
 #include <vector>
 
-#include "backward_kernels.h"
 #include "common.h"
 #include "forward_kernels.h"
 #include "sort_kernels.h"
+#include "backward_kernels.h"
 
 using namespace vetrast;
 
@@ -152,7 +152,8 @@ int validate_forward(const vetrast_forward_args* a, vetrast_workspace_layout* la
     if (((uintptr_t)a->workspace % kAlign) != 0 || ((uintptr_t)a->position % 16) != 0) return VETRAST_ERR_INVALID_ARG;
     st = vetrast_workspace_layout_for(a->num_points, a->num_views, p.num_layers, w, h, lay);
     if (st != VETRAST_OK) return st;
-    if (a->workspace_bytes < lay->total_bytes) return VETRAST_ERR_WORKSPACE_SMALL;
+    const size_t need = a->save_for_backward ? lay->total_bytes : lay->forward_only_bytes;
+    if (a->workspace_bytes < need) return VETRAST_ERR_WORKSPACE_SMALL;
     return VETRAST_OK;
 }
 
@@ -265,6 +266,10 @@ int vetrast_workspace_layout_for(int32_t N, int32_t B, int32_t L, int32_t w, int
     lay->transmittance_base   = at;
     lay->transmittance_stride = align_up(cap * sizeof(float), kAlign);
     at += lay->transmittance_stride * B;
+    lay->forward_only_bytes = align_up(at, kAlign);
+    at                      = lay->forward_only_bytes;
+    lay->partial_base       = at;
+    at += align_up(cap * 8 * sizeof(float), kAlign);
     lay->total_bytes = align_up(at, kAlign);
     return VETRAST_OK;
 }
@@ -424,64 +429,97 @@ int vetrast_backward(vetrast_ctx* ctx, const vetrast_backward_args* g, void* str
     const uint32_t P    = ly.base[L];
     void* ws            = a->workspace;
 
+    // The gather kernel overwrites every gradient row in the first view, so the zeros_like fills of
+    // PointRenderer.cu:267-277 are only needed where rows are added to: with a texture index indirection (several
+    // points may share a row) or with the background leak switch (which adds into row 0 before the gather runs).
+    const bool add_to_rows = a->index != nullptr || p.quirk_background_confidence_leak != 0;
     {
-        // zeros_like of every gradient tensor, PointRenderer.cu:267-277
         ScopeTimer tm(ctx, stream, VETRAST_SCOPE_BACKWARD_PREPARE);
         auto zero = [&](float* ptr, size_t n) {
             if (!ptr || n == 0) return;
             hipLaunchKernelGGL(fill_u32_kernel, dim3(std::min(grid_for(n), 8192)), dim3(kBlock), 0, stream,
                                reinterpret_cast<uint32_t*>(ptr), n, 0u);
         };
-        zero(g->grad_texture, (size_t)C * N);
-        zero(g->grad_confidence, (size_t)N);
         zero(g->grad_background, (size_t)C);
-        if (g->grad_points)
+        if (add_to_rows || N == 0)
         {
-            zero(g->grad_points, (size_t)4 * N);
-            zero(g->grad_point_count, (size_t)N);
+            zero(g->grad_texture, (size_t)C * N);
+            zero(g->grad_confidence, (size_t)N);
+            if (g->grad_points)
+            {
+                zero(g->grad_points, (size_t)4 * N);
+                zero(g->grad_point_count, (size_t)N);
+            }
         }
     }
+    float4* partial = ws_ptr<float4>(ws, lay.partial_base);
     for (int b = 0; b < B; ++b)
     {
-        ScopeTimer tm(ctx, stream, VETRAST_SCOPE_BACKWARD_BLEND);
-        BackwardPass bp;
-        bp.offsets          = ws_ptr<uint32_t>(ws, lay.offsets_base + lay.offsets_stride * b);
-        bp.fragments        = ws_ptr<uint64_t>(ws, lay.fragments_base + lay.fragments_stride * b);
-        bp.transmittance    = ws_ptr<float>(ws, lay.transmittance_base + lay.transmittance_stride * b);
-        bp.weight           = ws_ptr<float>(ws, lay.weight_base + lay.weight_stride * b);
-        bp.index            = a->index;
-        bp.packed           = ws_ptr<float4>(ws, lay.packed_base);
-        bp.position         = reinterpret_cast<const float4*>(a->position);
-        bp.background       = a->background;
-        bp.view             = ws_ptr<DeviceView>(ws, lay.views_base) + b;
-        bp.grad_texture     = g->grad_texture;
-        bp.grad_confidence  = g->grad_confidence;
-        bp.grad_background  = g->grad_background;
-        bp.grad_points      = g->grad_points;
-        bp.grad_point_count = g->grad_point_count;
-        bp.ly               = ly;
-        bp.P                = P;
-        bp.N                = N;
-        bp.K                = p.debug_max_list_length;
-        bp.use_environment_map              = p.use_environment_map;
-        bp.need_point_gradient              = p.need_point_gradient;
-        bp.quirk_background_confidence_leak = p.quirk_background_confidence_leak;
-        for (int l = 0; l < VETRAST_MAX_LAYERS; ++l)
+        uint32_t* offsets   = ws_ptr<uint32_t>(ws, lay.offsets_base + lay.offsets_stride * b);
+        uint64_t* fragments = ws_ptr<uint64_t>(ws, lay.fragments_base + lay.fragments_stride * b);
         {
-            bp.grad_out[l] = nullptr;
-            bp.out[l]      = nullptr;
-            if (l >= L) continue;
-            const size_t plane = (size_t)ly.w[l] * ly.h[l];
-            bp.grad_out[l]     = g->grad_out[l] + (size_t)b * C * plane;
-            bp.out[l]          = a->out[l] + (size_t)b * C * plane;
+            ScopeTimer tm(ctx, stream, VETRAST_SCOPE_BACKWARD_BLEND);
+            BackwardPass bp;
+            bp.offsets          = offsets;
+            bp.fragments        = fragments;
+            bp.transmittance    = ws_ptr<float>(ws, lay.transmittance_base + lay.transmittance_stride * b);
+            bp.weight           = ws_ptr<float>(ws, lay.weight_base + lay.weight_stride * b);
+            bp.index            = a->index;
+            bp.packed           = ws_ptr<float4>(ws, lay.packed_base);
+            bp.position         = reinterpret_cast<const float4*>(a->position);
+            bp.background       = a->background;
+            bp.view             = ws_ptr<DeviceView>(ws, lay.views_base) + b;
+            bp.partial          = partial;
+            bp.grad_background  = g->grad_background;
+            bp.grad_confidence  = g->grad_confidence;
+            bp.ly               = ly;
+            bp.P                = P;
+            bp.N                = N;
+            bp.K                = p.debug_max_list_length;
+            bp.use_environment_map              = p.use_environment_map;
+            bp.need_point_gradient              = (p.need_point_gradient && g->grad_points) ? 1 : 0;
+            bp.quirk_background_confidence_leak = p.quirk_background_confidence_leak;
+            for (int l = 0; l < VETRAST_MAX_LAYERS; ++l)
+            {
+                bp.grad_out[l] = nullptr;
+                bp.out[l]      = nullptr;
+                if (l >= L) continue;
+                const size_t plane = (size_t)ly.w[l] * ly.h[l];
+                bp.grad_out[l]     = g->grad_out[l] + (size_t)b * C * plane;
+                bp.out[l]          = a->out[l] + (size_t)b * C * plane;
+            }
+            const dim3 grid(grid_for(P)), blk(kBlock);
+            switch (C)
+            {
+                case 1: hipLaunchKernelGGL(blend_backward_kernel<1>, grid, blk, 0, stream, bp); break;
+                case 2: hipLaunchKernelGGL(blend_backward_kernel<2>, grid, blk, 0, stream, bp); break;
+                case 3: hipLaunchKernelGGL(blend_backward_kernel<3>, grid, blk, 0, stream, bp); break;
+                default: hipLaunchKernelGGL(blend_backward_kernel<4>, grid, blk, 0, stream, bp); break;
+            }
         }
-        const dim3 grid(grid_for(P)), blk(kBlock);
-        switch (C)
+        if (N > 0)
         {
-            case 1: hipLaunchKernelGGL(blend_backward_kernel<1>, grid, blk, 0, stream, bp); break;
-            case 2: hipLaunchKernelGGL(blend_backward_kernel<2>, grid, blk, 0, stream, bp); break;
-            case 3: hipLaunchKernelGGL(blend_backward_kernel<3>, grid, blk, 0, stream, bp); break;
-            default: hipLaunchKernelGGL(blend_backward_kernel<4>, grid, blk, 0, stream, bp); break;
+            ScopeTimer tm(ctx, stream, VETRAST_SCOPE_BACKWARD_GATHER);
+            GatherPass gp;
+            gp.vp                  = make_view_pass(a, lay, ly, b);
+            gp.offsets             = offsets;
+            gp.fragments           = fragments;
+            gp.partial             = partial;
+            gp.grad_texture        = g->grad_texture;
+            gp.grad_confidence     = g->grad_confidence;
+            gp.grad_points         = g->grad_points;
+            gp.grad_point_count    = g->grad_point_count;
+            gp.K                   = p.debug_max_list_length;
+            gp.need_point_gradient = (p.need_point_gradient && g->grad_points) ? 1 : 0;
+            gp.accumulate          = (add_to_rows || b > 0) ? 1 : 0;
+            const dim3 grid(grid_for(N)), blk(kBlock);
+            switch (C)
+            {
+                case 1: hipLaunchKernelGGL(gather_point_gradients_kernel<1>, grid, blk, 0, stream, gp); break;
+                case 2: hipLaunchKernelGGL(gather_point_gradients_kernel<2>, grid, blk, 0, stream, gp); break;
+                case 3: hipLaunchKernelGGL(gather_point_gradients_kernel<3>, grid, blk, 0, stream, gp); break;
+                default: hipLaunchKernelGGL(gather_point_gradients_kernel<4>, grid, blk, 0, stream, gp); break;
+            }
         }
     }
     if (g->grad_points && p.point_gradient_normalization != 0 && N > 0)
@@ -564,6 +602,7 @@ const char* vetrast_scope_name(int32_t scope)
         case VETRAST_SCOPE_BLEND: return "BlendingPass";
         case VETRAST_SCOPE_BACKWARD_PREPARE: return "Prepare Backward";
         case VETRAST_SCOPE_BACKWARD_BLEND: return "BlendBackwards";
+        case VETRAST_SCOPE_BACKWARD_GATHER: return "BlendBackwards (per-point sum)";
         case VETRAST_SCOPE_BACKWARD_POST: return "Post Process Gradient";
         default: return "?";
     }
