@@ -122,6 +122,7 @@ typedef struct vetrast_workspace_layout
     size_t flags_base;     /* uint32 [4] device status flags */
     size_t forward_only_bytes; /* a forward call with save_for_backward = 0 needs only this much */
     size_t partial_base;   /* float [L][N][8]: backward scratch, gradient record of the fragment of point i in layer l */
+    size_t background_partial_base; /* float [ceil(P/256)][8]: backward scratch, per-workgroup background-gradient sums */
 } vetrast_workspace_layout;
 
 /* Arguments of the forward pass. Replaces the inputs PointRender::forward receives

@@ -71,6 +71,7 @@ class WorkspaceLayout(C.Structure):
         ("flags_base", C.c_size_t),
         ("forward_only_bytes", C.c_size_t),
         ("partial_base", C.c_size_t),
+        ("background_partial_base", C.c_size_t),
     ]
 
 

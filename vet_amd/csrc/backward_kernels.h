@@ -25,8 +25,7 @@ struct BackwardPass
     const float* grad_out[VETRAST_MAX_LAYERS];  // already offset to this view
     const float* out[VETRAST_MAX_LAYERS];       // forward result, already offset to this view
     float4* partial;          // [L][N] records of 2 float4: (d tex0..3), (d conf, d x, d y, d z)
-    float* grad_background;   // [C]
-    float* grad_confidence;   // [N]; only touched for the background leak switch
+    float* background_partial;  // [workgroups][8]: per-workgroup sums of d background[0..C) and of the leak term
     LayerTable ly;
     uint32_t P;
     int N;
@@ -196,22 +195,65 @@ __global__ void __launch_bounds__(kBlock) blend_backward_kernel(BackwardPass a)
         }
     }
 
-    // Every pixel adds to the same C background values: reduce over the wave first, one atomic per wave and channel
-    // (the reference issues one atomic per pixel and channel, src/lib/rendering/RenderBackward.cu:1150-1152).
-    if (!a.use_environment_map)
-    {
-        const int lane = threadIdx.x & (kWave - 1);
+    // Every pixel adds to the same C background values. Atomics on one address serialise (the reference issues one per
+    // pixel and channel, src/lib/rendering/RenderBackward.cu:1150-1152), so each workgroup reduces its 256 pixels and
+    // stores one row of partial sums; reduce_background_kernel adds the rows up.
+    __shared__ float red[kBlock / kWave][C + 1];
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
 #pragma unroll
-        for (int ci = 0; ci < C; ++ci)
-        {
-            const float s = wave_sum(bg_grad[ci]);
-            if (lane == 0 && s != 0.f) atomicAdd(&a.grad_background[ci], s);
-        }
-        if (a.quirk_background_confidence_leak)
-        {
-            const float s = wave_sum(leak);
-            if (lane == 0 && s != 0.f) atomicAdd(&a.grad_confidence[0], s);
-        }
+    for (int ci = 0; ci < C; ++ci)
+    {
+        const float s = wave_sum(bg_grad[ci]);
+        if (lane == 0) red[wave][ci] = s;
+    }
+    {
+        const float s = wave_sum(leak);
+        if (lane == 0) red[wave][C] = s;
+    }
+    __syncthreads();
+    if (threadIdx.x <= C)
+        a.background_partial[(size_t)blockIdx.x * kBackgroundRow + threadIdx.x] =
+            (red[0][threadIdx.x] + red[1][threadIdx.x]) + (red[2][threadIdx.x] + red[3][threadIdx.x]);
+}
+
+// Sums the per-workgroup background rows of one view (one workgroup, fixed order, so the result is reproducible) and
+// adds the background pseudo-fragment's alpha gradient to confidence row 0 when that switch of the reference's
+// behaviour is on (src/lib/rendering/RenderBackward.cu:1130-1131,1157).
+__global__ void __launch_bounds__(kBlock) reduce_background_kernel(const float* __restrict__ rows, int num_rows, int C,
+                                                                    float* __restrict__ grad_background,
+                                                                    float* __restrict__ grad_confidence, int add_leak,
+                                                                    int accumulate)
+{
+    __shared__ float red[kBlock / kWave][kBackgroundRow];
+    float acc[kBackgroundRow];
+#pragma unroll
+    for (int k = 0; k < kBackgroundRow; ++k) acc[k] = 0.f;
+    for (int r = threadIdx.x; r < num_rows; r += kBlock)
+    {
+        const float4 a0 = reinterpret_cast<const float4*>(rows)[2 * (size_t)r];
+        const float4 a1 = reinterpret_cast<const float4*>(rows)[2 * (size_t)r + 1];
+        acc[0] += a0.x;
+        acc[1] += a0.y;
+        acc[2] += a0.z;
+        acc[3] += a0.w;
+        acc[4] += a1.x;
+    }
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+#pragma unroll
+    for (int k = 0; k < 5; ++k)
+    {
+        const float s = wave_sum(acc[k]);
+        if (lane == 0) red[wave][k] = s;
+    }
+    __syncthreads();
+    if (threadIdx.x <= C)
+    {
+        const int k   = threadIdx.x;
+        const float s = (red[0][k] + red[1][k]) + (red[2][k] + red[3][k]);
+        if (k < C)
+            grad_background[k] = accumulate ? grad_background[k] + s : s;
+        else if (add_leak)
+            grad_confidence[0] += s;
     }
 }
 

@@ -13,6 +13,7 @@ constexpr uint32_t kNoSlot    = 0xFFFFFFFFu;
 constexpr uint64_t kInfKey    = ~0ull;        // sorts behind every real (depth bits, point id) key
 constexpr int kScanPerThread  = 16;
 constexpr int kScanPerBlock   = kBlock * kScanPerThread;  // 4096 counts per workgroup
+constexpr int kBackgroundRow  = 8;            // floats per workgroup row of background-gradient partial sums
 constexpr int kPackedFloats   = 8;            // interleaved record: 4 descriptor floats, confidence, 3 pad
 
 // Camera constants of one view, written by prepare_views_kernel and read (uniformly) by every other kernel.

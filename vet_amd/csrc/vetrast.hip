@@ -270,6 +270,8 @@ int vetrast_workspace_layout_for(int32_t N, int32_t B, int32_t L, int32_t w, int
     at                      = lay->forward_only_bytes;
     lay->partial_base       = at;
     at += align_up(cap * 8 * sizeof(float), kAlign);
+    lay->background_partial_base = at;
+    at += align_up(((P + kBlock - 1) / kBlock) * kBackgroundRow * sizeof(float), kAlign);
     lay->total_bytes = align_up(at, kAlign);
     return VETRAST_OK;
 }
@@ -429,10 +431,10 @@ int vetrast_backward(vetrast_ctx* ctx, const vetrast_backward_args* g, void* str
     const uint32_t P    = ly.base[L];
     void* ws            = a->workspace;
 
-    // The gather kernel overwrites every gradient row in the first view, so the zeros_like fills of
-    // PointRenderer.cu:267-277 are only needed where rows are added to: with a texture index indirection (several
-    // points may share a row) or with the background leak switch (which adds into row 0 before the gather runs).
-    const bool add_to_rows = a->index != nullptr || p.quirk_background_confidence_leak != 0;
+    // The per-point kernel overwrites every gradient row in the first view, so the zeros_like fills of
+    // PointRenderer.cu:267-277 are only needed where rows are added to with atomics: with a texture index
+    // indirection, where several points may share a row.
+    const bool add_to_rows = a->index != nullptr;
     {
         ScopeTimer tm(ctx, stream, VETRAST_SCOPE_BACKWARD_PREPARE);
         auto zero = [&](float* ptr, size_t n) {
@@ -440,8 +442,7 @@ int vetrast_backward(vetrast_ctx* ctx, const vetrast_backward_args* g, void* str
             hipLaunchKernelGGL(fill_u32_kernel, dim3(std::min(grid_for(n), 8192)), dim3(kBlock), 0, stream,
                                reinterpret_cast<uint32_t*>(ptr), n, 0u);
         };
-        zero(g->grad_background, (size_t)C);
-        if (add_to_rows || N == 0)
+        if (add_to_rows)
         {
             zero(g->grad_texture, (size_t)C * N);
             zero(g->grad_confidence, (size_t)N);
@@ -452,7 +453,8 @@ int vetrast_backward(vetrast_ctx* ctx, const vetrast_backward_args* g, void* str
             }
         }
     }
-    float4* partial = ws_ptr<float4>(ws, lay.partial_base);
+    float4* partial        = ws_ptr<float4>(ws, lay.partial_base);
+    float* background_rows = ws_ptr<float>(ws, lay.background_partial_base);
     for (int b = 0; b < B; ++b)
     {
         uint32_t* offsets   = ws_ptr<uint32_t>(ws, lay.offsets_base + lay.offsets_stride * b);
@@ -470,8 +472,7 @@ int vetrast_backward(vetrast_ctx* ctx, const vetrast_backward_args* g, void* str
             bp.background       = a->background;
             bp.view             = ws_ptr<DeviceView>(ws, lay.views_base) + b;
             bp.partial          = partial;
-            bp.grad_background  = g->grad_background;
-            bp.grad_confidence  = g->grad_confidence;
+            bp.background_partial = background_rows;
             bp.ly               = ly;
             bp.P                = P;
             bp.N                = N;
@@ -520,6 +521,14 @@ int vetrast_backward(vetrast_ctx* ctx, const vetrast_backward_args* g, void* str
                 case 3: hipLaunchKernelGGL(gather_point_gradients_kernel<3>, grid, blk, 0, stream, gp); break;
                 default: hipLaunchKernelGGL(gather_point_gradients_kernel<4>, grid, blk, 0, stream, gp); break;
             }
+        }
+        {
+            // after the per-point kernel: it overwrites confidence row 0, the leak term is added on top
+            ScopeTimer tm(ctx, stream, VETRAST_SCOPE_BACKWARD_GATHER);
+            hipLaunchKernelGGL(reduce_background_kernel, dim3(1), dim3(kBlock), 0, stream, background_rows,
+                               grid_for(P), C, g->grad_background, g->grad_confidence,
+                               (p.quirk_background_confidence_leak && !p.use_environment_map && N > 0) ? 1 : 0,
+                               b > 0 ? 1 : 0);
         }
     }
     if (g->grad_points && p.point_gradient_normalization != 0 && N > 0)
