@@ -1,0 +1,76 @@
+"""The libtorch shim (PointRender autograd Function with the reference's argument order) against the oracle.
+
+This is the check the reference's authors sketched in their disabled A/B harness (src/lib/models/Pipeline.cpp:167-219):
+render, reduce the outputs to a scalar, call backward, compare the gradients of the scene tensors.
+"""
+import numpy as np
+import pytest
+import torch
+
+from tests.helpers import max_rel_err
+from vet_amd import synthetic
+from vet_amd.rasterizer import make_params
+
+pytestmark = pytest.mark.gpu
+
+
+def _views(scene):
+    return [(v.w, v.h, v.image_index, v.camera_index, v.camera_model_type, *v.crop_transform, *v.crop_rotation)
+            for v in scene.views]
+
+
+@pytest.mark.parametrize("literal", [True, False], ids=["reference_literal", "clean"])
+def test_autograd_matches_oracle(literal, oracle):
+    from vet_amd import torch_ops
+
+    scene = synthetic.tiny_scene(num_points=5000, K=8, seed=31, num_views=2)
+    quirks = dict(quirk_background_confidence_leak=1 if literal else 0,
+                  point_gradient_normalization=2 if literal else 0)
+    params = make_params(scene, need_point_gradient=1, **quirks)
+    ref = oracle.forward(scene, params)
+    grad_out = scene.grad_out()
+    ref_g = oracle.backward(ref, grad_out)
+
+    cu = lambda a, rg=False: torch.from_numpy(np.ascontiguousarray(a)).cuda().requires_grad_(rg)
+    texture, background = cu(scene.texture, True), cu(scene.background, True)
+    points, confidence = cu(scene.position, True), cu(scene.confidence.reshape(1, -1), True)
+    tangents = torch.zeros((scene.poses_se3.shape[0], 6), dtype=torch.float64, device="cuda", requires_grad=True)
+    intrinsics = cu(scene.intrinsics, True)
+    outs = torch_ops.blend_point_cloud(texture, background, points, tangents, intrinsics, confidence,
+                                       cu(scene.poses_se3), None, _views(scene), scene.num_layers, train=False,
+                                       use_environment_map=0, need_point_gradient=1, drop_out_points_by_radius=0,
+                                       debug_max_list_length=scene.max_list_length, **quirks)
+    assert len(outs) == scene.num_layers
+    loss = 0
+    for l, o in enumerate(outs):
+        assert tuple(o.shape) == ref.out[l].shape
+        np.testing.assert_array_equal(o.detach().cpu().numpy(), ref.out[l])
+        loss = loss + (o * torch.from_numpy(grad_out[l]).cuda()).sum()
+    loss.backward()
+    assert max_rel_err(texture.grad.cpu().numpy(), ref_g["texture"]) <= 1e-4
+    assert max_rel_err(confidence.grad.cpu().numpy().reshape(-1), ref_g["confidence"]) <= 1e-4
+    assert max_rel_err(background.grad.cpu().numpy(), ref_g["background"]) <= 1e-4
+    assert max_rel_err(points.grad.cpu().numpy(), ref_g["points"]) <= 1e-4
+    assert tangents.grad is None and intrinsics.grad is None  # not computed on this path
+
+
+def test_no_grad_call_and_masks(oracle):
+    from vet_amd import torch_ops
+
+    scene = synthetic.tiny_scene(num_points=3000, K=8, seed=32)
+    params = make_params(scene, output_background_mask=1, output_background_mask_value=0.25)
+    ref = oracle.forward(scene, params)
+    cu = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
+    with torch.no_grad():
+        outs = torch_ops.blend_point_cloud(cu(scene.texture), cu(scene.background), cu(scene.position),
+                                           torch.zeros((1, 6), dtype=torch.float64, device="cuda"),
+                                           cu(scene.intrinsics), cu(scene.confidence.reshape(1, -1)),
+                                           cu(scene.poses_se3), None, _views(scene), scene.num_layers,
+                                           use_environment_map=0, drop_out_points_by_radius=0,
+                                           debug_max_list_length=scene.max_list_length, output_background_mask=1,
+                                           output_background_mask_value=0.25)
+    L = scene.num_layers
+    assert len(outs) == 2 * L
+    for l in range(L):
+        np.testing.assert_array_equal(outs[l].cpu().numpy(), ref.out[l])
+        np.testing.assert_array_equal(outs[L + l].cpu().numpy(), ref.out_mask[l])

@@ -37,7 +37,37 @@ def build_library(verbose=True):
     return LIB_PATH
 
 
+TORCH_EXT_PATH = os.path.join(LIB_DIR, "vetrast_torch.so")
+
+
+def build_torch_extension(verbose=True):
+    """libtorch shim (vet_amd/torch_ext) as a Python extension module vet_amd/lib/vetrast_torch.so, linked against
+    libvetrast.so. Plain host C++: g++ against the torch headers, no device code."""
+    import sysconfig
+
+    import torch
+    from torch.utils import cpp_extension
+
+    os.makedirs(LIB_DIR, exist_ok=True)
+    inc = cpp_extension.include_paths()
+    torch_lib = os.path.join(os.path.dirname(torch.__file__), "lib")
+    cmd = [os.environ.get("CXX", "g++"), "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-Wno-unused-function",
+           "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1", "-DTORCH_EXTENSION_NAME=vetrast_torch",
+           "-DTORCH_API_INCLUDE_EXTENSION_H", f"-D_GLIBCXX_USE_CXX11_ABI={int(torch._C._GLIBCXX_USE_CXX11_ABI)}"]
+    for i in inc + ["/opt/rocm/include", sysconfig.get_paths()["include"]]:
+        cmd += ["-isystem", i]
+    cmd += [os.path.join(HERE, "torch_ext", "point_render.cpp"), "-o", TORCH_EXT_PATH,
+            f"-L{torch_lib}", f"-L{LIB_DIR}", "-lvetrast", "-lc10", "-lc10_hip", "-ltorch_cpu", "-ltorch_hip", "-ltorch",
+            "-ltorch_python", "-Wl,-rpath,$ORIGIN", f"-Wl,-rpath,{torch_lib}"]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    subprocess.run(cmd, check=True)
+    return TORCH_EXT_PATH
+
+
 if __name__ == "__main__":
     build_library()
     print("built", LIB_PATH)
+    build_torch_extension()
+    print("built", TORCH_EXT_PATH)
     sys.exit(0)

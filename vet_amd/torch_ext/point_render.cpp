@@ -1,0 +1,335 @@
+// libtorch host side of the MI355X blending point rasterizer: autograd Function with the reference's argument order,
+// calling the C ABI of include/vetrast.h. See point_render.h for the reference lines each piece mirrors.
+#include "point_render.h"
+
+#include <c10/hip/HIPStream.h>
+#include <torch/extension.h>
+
+namespace vet_amd
+{
+namespace
+{
+void check_status(int st, const char* where)
+{
+    TORCH_CHECK(st == VETRAST_OK, "vetrast ", where, " failed: ", st, " (", vetrast_status_string(st), ")");
+}
+
+void* current_stream()
+{
+    return (void*)c10::hip::getCurrentHIPStream().stream();
+}
+
+vetrast_params to_abi_params(const RenderParams& p, int num_layers)
+{
+    vetrast_params q;
+    q.num_texture_channels             = p.num_texture_channels;
+    q.num_layers                       = num_layers;
+    q.debug_max_list_length            = p.debug_max_list_length;
+    q.use_environment_map              = p.use_environment_map ? 1 : 0;
+    q.need_point_gradient              = p.need_point_gradient ? 1 : 0;
+    q.viewer_only                      = p.viewer_only ? 1 : 0;
+    q.stability_cutoff_value           = p.stability_cutoff_value;
+    q.drop_out_points_by_radius        = p.drop_out_points_by_radius ? 1 : 0;
+    q.drop_out_radius_threshold        = p.drop_out_radius_threshold;
+    q.output_background_mask           = p.output_background_mask ? 1 : 0;
+    q.output_background_mask_value     = p.output_background_mask_value;
+    q.check_normal                     = p.check_normal ? 1 : 0;
+    q.quirk_background_confidence_leak = p.quirk_background_confidence_leak ? 1 : 0;
+    q.point_gradient_normalization     = p.point_gradient_normalization;
+    return q;
+}
+
+void check_f32_cuda(const torch::Tensor& t, const char* name)
+{
+    TORCH_CHECK(t.defined() && t.is_cuda() && t.scalar_type() == torch::kFloat32 && t.is_contiguous(), name,
+                " must be a contiguous float32 tensor on the GPU");
+}
+
+// Fills the part of the argument struct that forward and backward share. `info->images` must outlive the call.
+vetrast_forward_args make_forward_args(NeuralRenderInfo* info, const torch::Tensor& texture,
+                                       const torch::Tensor& background_color, const torch::Tensor& points,
+                                       const torch::Tensor& intrinsics, const torch::Tensor& confidence,
+                                       const torch::Tensor& dropout, const torch::Tensor& poses_se3,
+                                       const torch::Tensor& t_index)
+{
+    check_f32_cuda(texture, "texture");
+    check_f32_cuda(background_color, "background_color");
+    check_f32_cuda(points, "points");
+    check_f32_cuda(intrinsics, "intrinsics");
+    check_f32_cuda(confidence, "confidence");
+    TORCH_CHECK(points.dim() == 2 && points.size(1) == 4, "points must be [N,4]");  // PointRenderer.cu:532
+    TORCH_CHECK(texture.dim() == 2 && texture.size(1) == points.size(0), "texture must be [C,N]");
+    TORCH_CHECK(confidence.numel() == points.size(0), "confidence must be [1,N]");
+    TORCH_CHECK(intrinsics.dim() == 2 && intrinsics.size(1) == 13, "intrinsics must be [num_cameras,13]");
+    TORCH_CHECK(poses_se3.defined() && poses_se3.is_cuda() && poses_se3.scalar_type() == torch::kFloat64 &&
+                    poses_se3.is_contiguous() && poses_se3.dim() == 2 && poses_se3.size(1) == 8,
+                "poses_se3 must be a contiguous [F,8] float64 tensor on the GPU");
+    TORCH_CHECK(info->params.render_mode == 1, "only render_mode 1 (FULL_BLEND) is implemented");
+    TORCH_CHECK(!info->params.add_depth_to_network, "add_depth_to_network is not part of the blending path");
+    TORCH_CHECK(!info->images.empty(), "no views");
+
+    vetrast_forward_args a;
+    std::memset(&a, 0, sizeof(a));
+    a.num_points  = (int32_t)points.size(0);
+    a.num_views   = (int32_t)info->images.size();
+    a.num_poses   = (int32_t)poses_se3.size(0);
+    a.num_cameras = (int32_t)intrinsics.size(0);
+    a.position    = points.data_ptr<float>();
+    a.index       = nullptr;
+    if (t_index.defined())
+    {
+        TORCH_CHECK(t_index.is_cuda() && t_index.scalar_type() == torch::kInt32 && t_index.is_contiguous() &&
+                        t_index.numel() == points.size(0),
+                    "t_index must be a contiguous [N,1] int32 tensor on the GPU");
+        a.index = t_index.data_ptr<int32_t>();
+    }
+    a.texture    = texture.data_ptr<float>();
+    a.confidence = confidence.data_ptr<float>();
+    a.background = background_color.data_ptr<float>();
+    a.dropout    = dropout.defined() ? dropout.data_ptr<float>() : nullptr;
+    a.poses_se3  = poses_se3.data_ptr<double>();
+    a.intrinsics = intrinsics.data_ptr<float>();
+    a.views      = info->images.data();
+    RenderParams prm         = info->params;
+    prm.num_texture_channels = (int)texture.size(0);
+    a.params                 = to_abi_params(prm, info->num_layers);
+    return a;
+}
+
+}  // namespace
+
+PointRendererCache::PointRendererCache()
+{
+    check_status(vetrast_create(&ctx), "create");
+}
+
+PointRendererCache::~PointRendererCache()
+{
+    vetrast_destroy(ctx);
+}
+
+std::vector<torch::Tensor> BlendPointCloud(NeuralRenderInfo* info)
+{
+    TORCH_CHECK(info && info->scene && info->cache, "BlendPointCloud: scene and cache must be set");
+    torch::intrusive_ptr<NeuralRenderInfo> render_data = torch::make_intrusive<NeuralRenderInfo>(*info);
+    SceneTensors& s                                    = *render_data->scene;
+    return PointRender::apply(s.texture, s.background_color, s.t_position, s.tangent_poses, s.intrinsics,
+                              s.confidence_value_of_point, s.dynamic_refinement_t, torch::IValue(render_data));
+}
+
+torch::autograd::variable_list PointRender::forward(torch::autograd::AutogradContext* ctx, torch::Tensor texture,
+                                                    torch::Tensor background_color, torch::Tensor points,
+                                                    torch::Tensor pose_tangents, torch::Tensor intrinsics,
+                                                    torch::Tensor confidence, torch::Tensor dynamic_refinement,
+                                                    torch::IValue info_value)
+{
+    ctx->saved_data["render_info"] = info_value;
+    NeuralRenderInfo* info         = info_value.toCustomClass<NeuralRenderInfo>().get();
+    TORCH_CHECK(dynamic_refinement.dim() <= 1, "per-view point displacements are not implemented");
+
+    const int B = (int)info->images.size(), L = info->num_layers, C = (int)texture.size(0);
+    const int64_t N = points.size(0);
+    auto f32        = torch::TensorOptions().device(points.device()).dtype(torch::kFloat32);
+
+    // dropout mask per view, PointRenderer.cu:461-468 (the mask is 1 where a point is dropped)
+    torch::Tensor dropout;
+    if (info->train && info->params.dropout > 0) dropout = torch::empty({B, N}, f32).bernoulli_(info->params.dropout);
+
+    // side inputs read through info->scene; they are saved with the graph so that backward does not touch the scene
+    const torch::Tensor poses_se3 = info->scene->poses_se3;
+    const torch::Tensor t_index   = info->scene->t_index;
+    vetrast_forward_args a =
+        make_forward_args(info, texture, background_color, points, intrinsics, confidence, dropout, poses_se3, t_index);
+    vetrast_workspace_layout lay;
+    check_status(vetrast_workspace_layout_for(a.num_points, B, L, info->images[0].w, info->images[0].h, &lay), "layout");
+
+    const bool need_backward = ctx != nullptr && (texture.requires_grad() || background_color.requires_grad() ||
+                                                  points.requires_grad() || confidence.requires_grad());
+    auto u8 = torch::TensorOptions().device(points.device()).dtype(torch::kUInt8);
+    torch::Tensor workspace;
+    if (need_backward)
+        workspace = torch::empty({(int64_t)lay.total_bytes}, u8);  // saved for backward, like the reference's buffers
+    else
+    {
+        auto& ws = info->cache->eval_workspace;
+        if (!ws.defined() || ws.numel() < (int64_t)lay.forward_only_bytes || ws.device() != points.device())
+            ws = torch::empty({(int64_t)lay.forward_only_bytes}, u8);
+        workspace = ws;
+    }
+
+    std::vector<torch::Tensor> out(L), mask;
+    for (int l = 0; l < L; ++l)
+    {
+        out[l]   = torch::empty({B, C, lay.layer_h[l], lay.layer_w[l]}, f32);
+        a.out[l] = out[l].data_ptr<float>();
+    }
+    if (info->params.output_background_mask)
+    {
+        mask.resize(L);
+        for (int l = 0; l < L; ++l)
+        {
+            mask[l]       = torch::empty({B, 1, lay.layer_h[l], lay.layer_w[l]}, f32);
+            a.out_mask[l] = mask[l].data_ptr<float>();
+        }
+    }
+    a.workspace         = workspace.data_ptr();
+    a.workspace_bytes   = (size_t)workspace.numel();
+    a.save_for_backward = need_backward ? 1 : 0;
+    check_status(vetrast_forward(info->cache->ctx, &a, current_stream()), "forward");
+
+    if (need_backward)
+    {
+        // saved state: workspace (scan, sorted lists, transmittance, weight), outputs, dropout. PointRenderer.cu:1027-1059
+        std::vector<torch::Tensor> saved = {workspace, texture, background_color, points, intrinsics, confidence,
+                                            poses_se3};
+        saved.insert(saved.end(), out.begin(), out.end());
+        if (dropout.defined()) saved.push_back(dropout);
+        if (t_index.defined()) saved.push_back(t_index);
+        ctx->save_for_backward(saved);
+        ctx->saved_data["has_dropout"] = dropout.defined();
+        ctx->saved_data["has_index"]   = t_index.defined();
+        ctx->saved_data["points_need_grad"] = points.requires_grad();
+    }
+    // masks are not differentiable (the reference detaches them in RenderModule.cpp:74-102)
+    if (ctx) ctx->mark_non_differentiable(mask);
+    out.insert(out.end(), mask.begin(), mask.end());
+    return out;
+}
+
+torch::autograd::variable_list PointRender::backward(torch::autograd::AutogradContext* ctx,
+                                                     torch::autograd::variable_list grad_output)
+{
+    torch::IValue info_value = ctx->saved_data["render_info"];
+    NeuralRenderInfo* info   = info_value.toCustomClass<NeuralRenderInfo>().get();
+    const int L              = info->num_layers;
+    auto saved               = ctx->get_saved_variables();
+    const bool has_dropout   = ctx->saved_data["has_dropout"].toBool();
+    const bool has_index     = ctx->saved_data["has_index"].toBool();
+    constexpr int kFixed     = 7;
+    TORCH_CHECK((int)saved.size() == kFixed + L + (has_dropout ? 1 : 0) + (has_index ? 1 : 0),
+                "unexpected number of saved tensors");  // PointRenderer.cu:1163-1164
+    TORCH_CHECK((int)grad_output.size() >= L, "expected one upstream gradient per layer");  // PointRenderer.cu:1158-1159
+    torch::Tensor workspace = saved[0], texture = saved[1], background_color = saved[2], points = saved[3],
+                  intrinsics = saved[4], confidence = saved[5], poses_se3 = saved[6];
+    torch::Tensor dropout = has_dropout ? saved[kFixed + L] : torch::Tensor();
+    torch::Tensor t_index = has_index ? saved[kFixed + L + (has_dropout ? 1 : 0)] : torch::Tensor();
+
+    vetrast_backward_args g;
+    std::memset(&g, 0, sizeof(g));
+    g.fwd = make_forward_args(info, texture, background_color, points, intrinsics, confidence, dropout, poses_se3, t_index);
+    std::vector<torch::Tensor> grads(L);
+    for (int l = 0; l < L; ++l)
+    {
+        g.fwd.out[l] = saved[kFixed + l].data_ptr<float>();
+        TORCH_CHECK(grad_output[l].defined(), "upstream gradient of layer ", l, " is undefined");
+        TORCH_CHECK(grad_output[l].scalar_type() == torch::kFloat32, "upstream gradients must be float32");  // :1117
+        grads[l]      = grad_output[l].contiguous();
+        g.grad_out[l] = grads[l].data_ptr<float>();
+    }
+    g.fwd.workspace         = workspace.data_ptr();
+    g.fwd.workspace_bytes   = (size_t)workspace.numel();
+    g.fwd.save_for_backward = 1;
+
+    // zeros_like of each gradient tensor (PointRenderer.cu:267-277); the library overwrites them.
+    torch::Tensor g_texture    = torch::empty_like(texture);
+    torch::Tensor g_confidence = torch::empty_like(confidence);
+    torch::Tensor g_background = torch::empty_like(background_color);
+    torch::Tensor g_points, g_point_count;
+    g.grad_texture    = g_texture.data_ptr<float>();
+    g.grad_confidence = g_confidence.data_ptr<float>();
+    g.grad_background = g_background.data_ptr<float>();
+    if (ctx->saved_data["points_need_grad"].toBool())
+    {
+        g_points           = torch::empty_like(points);
+        g_point_count      = torch::empty({points.size(0)}, points.options());
+        g.grad_points      = g_points.data_ptr<float>();
+        g.grad_point_count = g_point_count.data_ptr<float>();
+    }
+    check_status(vetrast_backward(info->cache->ctx, &g, current_stream()), "backward");
+
+    // order: texture, background, points, pose_tangent, intrinsics, confidence, dynamic (PointRenderer.cu:1319-1322),
+    // plus one empty gradient for the IValue (RenderInfo.cpp:64). Pose and intrinsics gradients are not computed.
+    return {g_texture, g_background, g_points, torch::Tensor(), torch::Tensor(), g_confidence, torch::Tensor(),
+            torch::Tensor()};
+}
+
+}  // namespace vet_amd
+
+TORCH_LIBRARY(vet_amd, m)
+{
+    m.class_<vet_amd::NeuralRenderInfo>("NeuralRenderInfo").def(torch::init());
+}
+
+// ---- Python binding used by the tests: builds a NeuralRenderInfo from plain arguments and calls BlendPointCloud ----
+namespace
+{
+std::shared_ptr<vet_amd::PointRendererCache> g_cache;
+
+std::vector<torch::Tensor> blend_point_cloud(torch::Tensor texture, torch::Tensor background_color, torch::Tensor points,
+                                             torch::Tensor pose_tangents, torch::Tensor intrinsics,
+                                             torch::Tensor confidence, torch::Tensor poses_se3, torch::Tensor t_index,
+                                             std::vector<std::vector<double>> views, int num_layers, bool train,
+                                             pybind11::dict params)
+{
+    using namespace vet_amd;
+    if (!g_cache) g_cache = std::make_shared<PointRendererCache>();
+    SceneTensors scene;
+    scene.texture                   = texture;
+    scene.background_color          = background_color;
+    scene.t_position                = points;
+    scene.tangent_poses             = pose_tangents;
+    scene.intrinsics                = intrinsics;
+    scene.confidence_value_of_point = confidence;
+    scene.dynamic_refinement_t      = torch::zeros({1}, points.options());
+    scene.poses_se3                 = poses_se3;
+    if (t_index.defined() && t_index.numel() > 0) scene.t_index = t_index;
+
+    NeuralRenderInfo nri;
+    nri.scene      = &scene;
+    nri.num_layers = num_layers;
+    nri.train      = train;
+    nri.cache      = g_cache.get();
+    for (auto& v : views)
+    {
+        TORCH_CHECK(v.size() == 14, "a view is (w, h, image_index, camera_index, camera_model, crop[5], rot[4])");
+        ReducedImageInfo r;
+        r.w                 = (int)v[0];
+        r.h                 = (int)v[1];
+        r.image_index       = (int)v[2];
+        r.camera_index      = (int)v[3];
+        r.camera_model_type = (int)v[4];
+        for (int j = 0; j < 5; ++j) r.crop_transform[j] = (float)v[5 + j];
+        for (int j = 0; j < 4; ++j) r.crop_rotation[j] = (float)v[10 + j];
+        nri.images.push_back(r);
+    }
+    RenderParams& p = nri.params;
+    p.dropout       = 0.f;
+    for (auto item : params)
+    {
+        const std::string k = pybind11::cast<std::string>(item.first);
+        auto as_d           = [&] { return pybind11::cast<double>(item.second); };
+        if (k == "dropout") p.dropout = (float)as_d();
+        else if (k == "drop_out_radius_threshold") p.drop_out_radius_threshold = (float)as_d();
+        else if (k == "drop_out_points_by_radius") p.drop_out_points_by_radius = as_d() != 0;
+        else if (k == "output_background_mask") p.output_background_mask = as_d() != 0;
+        else if (k == "output_background_mask_value") p.output_background_mask_value = (float)as_d();
+        else if (k == "stability_cutoff_value") p.stability_cutoff_value = (float)as_d();
+        else if (k == "need_point_gradient") p.need_point_gradient = as_d() != 0;
+        else if (k == "use_environment_map") p.use_environment_map = as_d() != 0;
+        else if (k == "viewer_only") p.viewer_only = as_d() != 0;
+        else if (k == "debug_max_list_length") p.debug_max_list_length = (int)as_d();
+        else if (k == "quirk_background_confidence_leak") p.quirk_background_confidence_leak = as_d() != 0;
+        else if (k == "point_gradient_normalization") p.point_gradient_normalization = (int)as_d();
+        else if (k == "render_mode") p.render_mode = (int)as_d();
+        else TORCH_CHECK(false, "unknown RenderParams field ", k);
+    }
+    // the scene bundle only has to live for the duration of apply(): everything backward needs is saved in the graph
+    return BlendPointCloud(&nri);
+}
+}  // namespace
+
+PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
+{
+    m.def("blend_point_cloud", &blend_point_cloud,
+          "BlendPointCloud(NeuralRenderInfo*) of the reference, with the scene passed as tensors");
+}

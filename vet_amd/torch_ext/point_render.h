@@ -1,0 +1,100 @@
+// libtorch host side of the MI355X blending point rasterizer.
+//
+// Mirrors the reference's seam so that VET's pipeline can call it unchanged in spirit:
+//   std::vector<torch::Tensor> BlendPointCloud(NeuralRenderInfo* info)        src/lib/rendering/PointRenderer.h:53
+//   struct PointRender : torch::autograd::Function<PointRender>              src/lib/rendering/PointRenderer.h:39-47
+//   class NeuralRenderInfo : torch::CustomClassHolder                         src/lib/rendering/PointRenderer.h:23-34
+// Argument order, output list and the seven returned gradients are the reference's (src/lib/rendering/RenderInfo.cpp:18-67,
+// src/lib/rendering/PointRenderer.cu:1061-1068,1319-1322). All arithmetic happens behind the C ABI of include/vetrast.h.
+#pragma once
+#include <torch/torch.h>
+
+#include <memory>
+#include <vector>
+
+#include "../../include/vetrast.h"
+
+namespace vet_amd
+{
+// ReducedImageInfo (src/lib/data/SceneData.h:39-50) is the ABI's vetrast_view.
+using ReducedImageInfo = vetrast_view;
+
+// The RenderParams members the blending path reads (src/lib/data/Settings.h:19-93), same names and defaults.
+struct RenderParams
+{
+    bool check_normal                  = false;
+    float dropout                      = 0.25f;
+    float drop_out_radius_threshold    = 0.6f;
+    bool drop_out_points_by_radius     = true;
+    int num_texture_channels           = -1;
+    bool output_background_mask        = false;
+    float output_background_mask_value = 0.f;
+    bool add_depth_to_network          = false;  // not produced by FULL_BLEND in the reference either (depth images stay zero)
+    float stability_cutoff_value       = 10000.f;
+    bool need_point_gradient           = true;
+    bool use_environment_map           = true;
+    int render_mode                    = 1;  // FULL_BLEND; the other modes are not implemented
+    bool viewer_only                   = false;
+    int debug_max_list_length          = -1;
+    // Switches for two accidents of the reference implementation; the defaults reproduce it literally.
+    bool quirk_background_confidence_leak = true;   // src/lib/rendering/RenderBackward.cu:1157
+    int point_gradient_normalization      = 2;      // src/lib/rendering/PointRenderer.cu:1278-1279
+};
+
+// The tensors BlendPointCloud reads through info->scene (src/lib/rendering/RenderInfo.cpp:25-29 and
+// src/lib/data/NeuralScene.h:101-113): a plain bundle instead of the NeuralScene object.
+struct SceneTensors
+{
+    torch::Tensor texture;                    // scene->texture->texture                    [C,N] f32
+    torch::Tensor background_color;           // scene->texture->background_color           [C]   f32
+    torch::Tensor t_position;                 // scene->point_cloud_cuda->t_position        [N,4] f32
+    torch::Tensor tangent_poses;              // scene->poses->tangent_poses                [F,6] f64
+    torch::Tensor intrinsics;                 // scene->intrinsics->intrinsics              [Ncam,13] f32
+    torch::Tensor confidence_value_of_point;  // scene->texture->confidence_value_of_point  [1,N] f32
+    torch::Tensor dynamic_refinement_t;       // scene->dynamic_refinement_t                [1] dummy
+    torch::Tensor poses_se3;                  // scene->poses->poses_se3                    [F,8] f64
+    torch::Tensor t_index;                    // scene->point_cloud_cuda->t_index           [N,1] i32, may be undefined
+};
+
+// Owns the vetrast context and the workspace that is re-used between no-grad calls
+// (counterpart of PointRendererCache, src/lib/rendering/PointRenderer.h:112-248).
+class PointRendererCache
+{
+   public:
+    PointRendererCache();
+    ~PointRendererCache();
+    PointRendererCache(const PointRendererCache&)            = delete;
+    PointRendererCache& operator=(const PointRendererCache&) = delete;
+    vetrast_ctx* ctx = nullptr;
+    torch::Tensor eval_workspace;
+};
+
+class NeuralRenderInfo : public torch::CustomClassHolder
+{
+   public:
+    SceneTensors* scene = nullptr;
+    std::vector<ReducedImageInfo> images;
+    RenderParams params;
+    int num_layers           = 1;
+    bool train               = false;
+    int current_epoch        = 0;
+    void* timer_system       = nullptr;  // accepted for signature parity; per-kernel times come from vetrast_scope_times
+    PointRendererCache* cache = nullptr;
+};
+
+struct PointRender : public torch::autograd::Function<PointRender>
+{
+    static torch::autograd::variable_list forward(torch::autograd::AutogradContext* ctx, torch::Tensor texture,
+                                                  torch::Tensor background_color, torch::Tensor points,
+                                                  torch::Tensor pose_tangents, torch::Tensor intrinsics,
+                                                  torch::Tensor confidence, torch::Tensor dynamic_refinement,
+                                                  torch::IValue info);
+    static torch::autograd::variable_list backward(torch::autograd::AutogradContext* ctx,
+                                                   torch::autograd::variable_list grad_output);
+};
+
+// Render the scene into a batch of images; every image is a pyramid of layers: L tensors [B,C,h_l,w_l], then L masks
+// [B,1,h_l,w_l] if output_background_mask.
+std::vector<torch::Tensor> BlendPointCloud(NeuralRenderInfo* info);
+
+}  // namespace vet_amd

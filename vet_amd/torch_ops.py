@@ -1,0 +1,33 @@
+"""Loader of the libtorch shim (vet_amd/lib/vetrast_torch.so) for Python callers and tests."""
+import importlib.util
+import os
+
+import torch  # noqa: F401  (libtorch must be loaded before the extension)
+
+_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib", "vetrast_torch.so")
+_mod = None
+
+
+def load():
+    global _mod
+    if _mod is None:
+        if not os.path.exists(_PATH):
+            raise OSError(f"{_PATH} is missing: build it with `python -m vet_amd.build`")
+        spec = importlib.util.spec_from_file_location("vetrast_torch", _PATH)
+        _mod = importlib.util.module_from_spec(spec)
+        spec.loader.exec_module(_mod)
+    return _mod
+
+
+def blend_point_cloud(texture, background_color, points, pose_tangents, intrinsics, confidence, poses_se3, t_index,
+                      views, num_layers, train=False, **params):
+    """BlendPointCloud of the reference (src/lib/rendering/PointRenderer.h:53) on tensors; differentiable.
+
+    views: list of (w, h, image_index, camera_index, camera_model, crop fx,fy,cx,cy,s, rot r00,r01,r10,r11).
+    Returns L tensors [B,C,h_l,w_l], then L masks if output_background_mask.
+    """
+    if t_index is None:
+        t_index = torch.empty(0, dtype=torch.int32, device=points.device)
+    return load().blend_point_cloud(texture, background_color, points, pose_tangents, intrinsics, confidence, poses_se3,
+                                    t_index, [list(map(float, v)) for v in views], int(num_layers), bool(train),
+                                    {k: float(v) for k, v in params.items()})
