@@ -1,0 +1,46 @@
+"""Writes tests/golden/config1_oracle.npz: the CPU oracle's result for BASELINE config 1 (20 000 points uniform in the
+unit cube, 256x256, one layer, K=8, seed 0). The reference has no fixtures of its own and cannot run here, so this
+vector records the oracle (after it has been pinned by tests/test_oracle_pinning.py) and serves as a regression pin for
+the oracle and as a second, oracle-free check of the GPU path.
+
+    python tests/golden/make_config1_fixture.py
+"""
+import hashlib
+import os
+import sys
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+sys.path.insert(0, ROOT)
+
+from oracle import oracle_py  # noqa: E402
+from vet_amd import synthetic  # noqa: E402
+
+
+def sha(a):
+    return hashlib.sha256(np.ascontiguousarray(a).tobytes()).hexdigest()
+
+
+def main():
+    scene = synthetic.config1()
+    f = oracle_py.forward(scene)
+    counts = np.diff(f.offsets[0].astype(np.int64))
+    assert counts.max() < 256
+    total = int(f.offsets[0, -1])
+    out = f.out[0][0]
+    path = os.path.join(ROOT, "tests", "golden", "config1_oracle.npz")
+    np.savez_compressed(
+        path,
+        counts=counts.astype(np.uint8),                      # per-pixel fragment counts, row-major 256x256
+        fragments=f.fragments[0, :total],                    # every list fully sorted by (depth bits, point id)
+        out_rows=out[:, 96:160:4, :].copy(),                 # 16 image rows of the blended features, all channels
+        out_sha256=np.array(sha(out)),
+        weight_sha256=np.array(sha(f.weight[0])),
+        input_sha256=np.array([sha(scene.position), sha(scene.texture), sha(scene.confidence)]),
+    )
+    print("wrote", path, os.path.getsize(path), "bytes; fragments", total, "max list", counts.max())
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,127 @@
+"""Host-side checks that need no GPU: the C-ABI library loads, exports every symbol include/vetrast.h declares, and its
+pure-host functions (layer sizes, workspace layout, status strings, argument validation) behave."""
+import ctypes as C
+import os
+import re
+
+import pytest
+
+from vet_amd import abi, synthetic
+from vet_amd.rasterizer import fill_forward_args, make_params, make_views
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_functions():
+    text = open(os.path.join(ROOT, "include", "vetrast.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(vetrast_[a-z_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = abi.load_library()
+    names = declared_functions()
+    assert len(names) >= 14
+    assert sorted(abi.SYMBOLS) == names, "vet_amd/abi.py and include/vetrast.h disagree"
+    for n in names:
+        assert getattr(lib, n) is not None
+
+
+def test_struct_sizes_are_the_c_ones():
+    # sizes the C compiler gives the structs of include/vetrast.h (LP64)
+    assert C.sizeof(abi.View) == 5 * 4 + 9 * 4
+    assert C.sizeof(abi.Params) == 14 * 4
+    assert C.sizeof(abi.ForwardArgs) % 8 == 0
+    assert abi.BackwardArgs.grad_out.offset == C.sizeof(abi.ForwardArgs)
+
+
+def test_layer_sizes_halve_with_integer_division():
+    lib = abi.load_library()
+    w = (C.c_int32 * 5)()
+    h = (C.c_int32 * 5)()
+    assert lib.vetrast_layer_sizes(1920, 1080, 4, w, h) == 0
+    assert list(w)[:4] == [1920, 960, 480, 240] and list(h)[:4] == [1080, 540, 270, 135]
+    assert lib.vetrast_layer_sizes(25, 13, 3, w, h) == 0
+    assert list(w)[:3] == [25, 12, 6] and list(h)[:3] == [13, 6, 3]
+    assert lib.vetrast_layer_sizes(25, 13, 6, w, h) == abi.ERR_INVALID_ARG
+    assert lib.vetrast_layer_sizes(0, 13, 1, w, h) == abi.ERR_INVALID_ARG
+
+
+def test_workspace_layout_is_aligned_and_disjoint():
+    lib = abi.load_library()
+    lay = abi.WorkspaceLayout()
+    N, B, L, w, h = 2_000_000, 2, 4, 1920, 1080
+    assert lib.vetrast_workspace_layout_for(N, B, L, w, h, C.byref(lay)) == 0
+    P = 1920 * 1080 + 960 * 540 + 480 * 270 + 240 * 135
+    assert lay.layer_pixel_base[L] == P and lay.fragment_capacity == N * L
+    regions = [
+        ("flags", lay.flags_base, 16),
+        ("offsets", lay.offsets_base, lay.offsets_stride * B),
+        ("fragments", lay.fragments_base, lay.fragments_stride * B),
+        ("transmittance", lay.transmittance_base, lay.transmittance_stride * B),
+        ("weight", lay.weight_base, lay.weight_stride * B),
+        ("packed", lay.packed_base, N * 32),
+        ("slots", lay.slots_base, N * L * 4),
+        ("views", lay.views_base, B * 128),
+        ("partial", lay.partial_base, N * L * 32),
+        ("background_partial", lay.background_partial_base, (P + 255) // 256 * 32),
+    ]
+    assert lay.offsets_stride >= (P + 1) * 4 and lay.fragments_stride >= N * L * 8
+    for name, base, size in regions:
+        assert base % 256 == 0, name
+        assert base + size <= lay.total_bytes, name
+    ordered = sorted(regions, key=lambda r: r[1])
+    for (n0, b0, s0), (n1, b1, _) in zip(ordered, ordered[1:]):
+        assert b0 + s0 <= b1, (n0, n1)
+    assert lay.forward_only_bytes <= lay.partial_base < lay.total_bytes
+    assert lib.vetrast_forward_workspace_bytes(N, B, L, w, h) == lay.total_bytes
+    # invalid dimensions
+    assert lib.vetrast_workspace_layout_for(N, 0, L, w, h, C.byref(lay)) == abi.ERR_INVALID_ARG
+    assert lib.vetrast_workspace_layout_for(N, B, 6, w, h, C.byref(lay)) == abi.ERR_INVALID_ARG
+    assert lib.vetrast_workspace_layout_for(N, B, 5, 8, 8, C.byref(lay)) == abi.ERR_INVALID_ARG  # coarsest layer empty
+    assert lib.vetrast_workspace_layout_for(2_000_000_000, B, 4, w, h, C.byref(lay)) == abi.ERR_INVALID_ARG
+    assert lib.vetrast_forward_workspace_bytes(N, 0, L, w, h) == 0
+
+
+def test_status_and_scope_names():
+    lib = abi.load_library()
+    assert lib.vetrast_status_string(0) == b"ok"
+    for st in (abi.ERR_INVALID_ARG, abi.ERR_WORKSPACE_SMALL, abi.ERR_HIP, abi.ERR_UNSUPPORTED, abi.ERR_BAD_INPUT_DATA):
+        assert lib.vetrast_status_string(st) not in (b"ok", b"unknown status")
+    assert lib.vetrast_status_string(-99) == b"unknown status"
+    names = [lib.vetrast_scope_name(i).decode() for i in range(abi.SCOPE_COUNT)]
+    # the reference's CudaTimerSystem scope names (src/lib/rendering/PointRenderer.cu:770-886,1222,1252)
+    for want in ("CountingPass", "CollectionPass", "SortingPass", "BlendingPass", "BlendBackwards"):
+        assert want in names
+
+
+def test_null_arguments_are_refused_without_touching_a_gpu():
+    lib = abi.load_library()
+    assert lib.vetrast_create(None) == abi.ERR_INVALID_ARG
+    assert lib.vetrast_forward(None, None, None) == abi.ERR_INVALID_ARG
+    assert lib.vetrast_backward(None, None, None) == abi.ERR_INVALID_ARG
+    assert lib.vetrast_set_profiling(None, 1) == abi.ERR_INVALID_ARG
+    assert lib.vetrast_last_hip_error(None) == 0
+    lib.vetrast_destroy(None)  # no-op
+
+
+def test_product_path_has_no_cpu_fallback():
+    """Without a GPU the host wrapper must raise instead of computing anything on the CPU."""
+    import torch
+
+    from vet_amd.rasterizer import Rasterizer
+
+    if torch.cuda.is_available():
+        pytest.skip("GPU present")
+    with pytest.raises(RuntimeError):
+        Rasterizer()
+
+
+def test_product_sources_do_not_use_the_oracle():
+    """The oracle is test infrastructure: nothing under vet_amd/ may import, load or link it."""
+    pat = re.compile(r"from\s+oracle|import\s+oracle|oracle_py|libvetrast_oracle|vetref_|oracle/")
+    for dirpath, _, files in os.walk(os.path.join(ROOT, "vet_amd")):
+        for f in files:
+            if f.endswith((".py", ".h", ".hip", ".cpp")):
+                text = open(os.path.join(dirpath, f)).read()
+                assert not pat.search(text), os.path.join(dirpath, f)

@@ -265,7 +265,7 @@ def tiny_scene(num_points=300, w=24, h=16, num_layers=3, K=4, seed=7, channels=4
     pos[:, 0] = (st.uniform(N) * 2.4 - 1.2).astype(np.float32)
     pos[:, 1] = (st.uniform(N) * 1.6 - 0.8).astype(np.float32)
     pos[:, 2] = (st.uniform(N) * 2.0 - 0.5).astype(np.float32)
-    pos[:, 3] = (0.002 + 0.05 * st.uniform(N)).astype(np.float32)
+    pos[:, 3] = (0.05 + 1.0 * st.uniform(N)).astype(np.float32)  # splat radii of 0.2 .. 8 pixels at layer 0
     tex = (0.5 * st.normal(channels * N)).reshape(channels, N).astype(np.float32)
     conf = sigmoid(st.normal(N)).astype(np.float32)
     bg = st.uniform(channels).astype(np.float32)
