@@ -15,12 +15,6 @@
 
 namespace vetrast
 {
-__device__ __forceinline__ uint64_t shfl_xor_u64(uint64_t v, int mask)
-{
-    const uint32_t lo = __shfl_xor((uint32_t)v, mask, kWave);
-    const uint32_t hi = __shfl_xor((uint32_t)(v >> 32), mask, kWave);
-    return ((uint64_t)hi << 32) | lo;
-}
 __device__ __forceinline__ uint64_t shfl_u64(uint64_t v, int src)
 {
     const uint32_t lo = __shfl((uint32_t)v, src, kWave);
@@ -28,12 +22,68 @@ __device__ __forceinline__ uint64_t shfl_u64(uint64_t v, int src)
     return ((uint64_t)hi << 32) | lo;
 }
 
-// One compare-exchange stage: lanes whose bit `low_bit` is clear keep the smaller key of the pair.
-__device__ __forceinline__ uint64_t exchange(uint64_t key, int partner_xor, bool keep_min)
+// Value of lane (lane ^ M) for the xor patterns a 64-wide bitonic network needs. Inside a row of 16 lanes the exchange
+// is a DPP move (register to register, a few cycles); only the four patterns that cross rows go through the LDS
+// crossbar (ds_swizzle within 32 lanes, ds_bpermute across the halves).
+template <int CTRL>
+__device__ __forceinline__ uint32_t dpp_move(uint32_t v)
 {
-    const uint64_t other = shfl_xor_u64(key, partner_xor);
+    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, 0xF, 0xF, false);
+}
+
+template <int M>
+__device__ __forceinline__ uint32_t lane_xor(uint32_t v, int lane)
+{
+    if constexpr (M == 1) return dpp_move<0xB1>(v);         // quad_perm [1,0,3,2]
+    else if constexpr (M == 2) return dpp_move<0x4E>(v);    // quad_perm [2,3,0,1]
+    else if constexpr (M == 3) return dpp_move<0x1B>(v);    // quad_perm [3,2,1,0]
+    else if constexpr (M == 7) return dpp_move<0x141>(v);   // row_half_mirror
+    else if constexpr (M == 15) return dpp_move<0x140>(v);  // row_mirror
+    else if constexpr (M == 8) return dpp_move<0x128>(v);   // row_ror:8
+    else if constexpr (M == 4)
+    {
+        // banks (groups of 4 lanes) 0 and 2 read lane+4 (row_shl:4), banks 1 and 3 read lane-4 (row_shr:4)
+        int t = __builtin_amdgcn_update_dpp((int)v, (int)v, 0x104, 0xF, 0x5, false);
+        t     = __builtin_amdgcn_update_dpp(t, (int)v, 0x114, 0xF, 0xA, false);
+        return (uint32_t)t;
+    }
+    else if constexpr (M == 16) return (uint32_t)__builtin_amdgcn_ds_swizzle((int)v, 0x401F);  // xor 0x10, and 0x1F
+    else if constexpr (M == 31) return (uint32_t)__builtin_amdgcn_ds_swizzle((int)v, 0x7C1F);  // xor 0x1F, and 0x1F
+    else return (uint32_t)__builtin_amdgcn_ds_bpermute((lane ^ M) << 2, (int)v);               // 32, 63
+}
+
+// One compare-exchange stage with partner lane ^ M: lanes for which keep_min holds keep the smaller key of the pair.
+template <int M>
+__device__ __forceinline__ uint64_t exchange(uint64_t key, int lane, bool keep_min)
+{
+    const uint32_t lo    = lane_xor<M>((uint32_t)key, lane);
+    const uint32_t hi    = lane_xor<M>((uint32_t)(key >> 32), lane);
+    const uint64_t other = ((uint64_t)hi << 32) | lo;
     const bool take      = keep_min ? (other < key) : (other > key);
     return take ? other : key;
+}
+
+template <int K2, int J>
+__device__ __forceinline__ uint64_t halving_steps(uint64_t key, int lane)
+{
+    if constexpr (J >= 1)
+    {
+        key = exchange<J>(key, lane, (lane & J) == 0);
+        key = halving_steps<K2, (J >> 1)>(key, lane);
+    }
+    return key;
+}
+
+template <int K2, int MAXK>
+__device__ __forceinline__ uint64_t bitonic_stages(uint64_t key, int lane)
+{
+    if constexpr (K2 <= MAXK)
+    {
+        key = exchange<K2 - 1>(key, lane, (lane & (K2 >> 1)) == 0);  // mirror step inside every block of K2 lanes
+        key = halving_steps<K2, (K2 >> 2)>(key, lane);
+        key = bitonic_stages<K2 * 2, MAXK>(key, lane);
+    }
+    return key;
 }
 
 // Ascending bitonic sort of every aligned group of 2^LOG lanes (all-ascending form: a mirror step, then halving
@@ -41,22 +91,13 @@ __device__ __forceinline__ uint64_t exchange(uint64_t key, int partner_xor, bool
 template <int LOG>
 __device__ __forceinline__ uint64_t bitonic_sort_groups(uint64_t key, int lane)
 {
-#pragma unroll
-    for (int k = 2; k <= (1 << LOG); k <<= 1)
-    {
-        key = exchange(key, k - 1, (lane & (k >> 1)) == 0);
-#pragma unroll
-        for (int j = k >> 2; j >= 1; j >>= 1) key = exchange(key, j, (lane & j) == 0);
-    }
-    return key;
+    return bitonic_stages<2, (1 << LOG)>(key, lane);
 }
 
 // Halving steps only: sorts a bitonic sequence held by the 64 lanes.
 __device__ __forceinline__ uint64_t bitonic_merge64(uint64_t key, int lane)
 {
-#pragma unroll
-    for (int j = 32; j >= 1; j >>= 1) key = exchange(key, j, (lane & j) == 0);
-    return key;
+    return halving_steps<64, 32>(key, lane);
 }
 
 // Sort `count` lists of class LOG (2^(LOG-1) < n <= 2^LOG) found in the wave; src_lane[r] is the lane that owns the r-th.
@@ -147,19 +188,38 @@ __device__ __forceinline__ void sort_in_memory(uint64_t* list, uint32_t n, int l
     }
 }
 
+// How waves are dealt to pixels: layer l is served by waves [first_wave[l], first_wave[l+1]), each owning
+// pixels_per_wave[l] consecutive pixels (a power of two <= 64). Coarse layers carry the same number of fragments in far
+// fewer pixels, so they get fewer pixels per wave; otherwise a handful of waves would sort most of the frame alone.
+struct SortWaveMap
+{
+    int L;
+    uint32_t first_wave[VETRAST_MAX_LAYERS + 1];
+    uint32_t pixels_per_wave[VETRAST_MAX_LAYERS];
+    uint32_t pixel_base[VETRAST_MAX_LAYERS + 1];
+};
+
 __global__ void __launch_bounds__(kBlock) sort_lists_kernel(const uint32_t* __restrict__ offsets,
-                                                             uint64_t* __restrict__ fragments, uint32_t P, int K)
+                                                             uint64_t* __restrict__ fragments, SortWaveMap map, int K)
 {
     __shared__ uint8_t src_lane_all[kBlock / kWave][kWave];
     const int lane    = threadIdx.x & (kWave - 1);
     const int wave    = threadIdx.x / kWave;
     uint8_t* src_lane = src_lane_all[wave];
-    const uint32_t q  = blockIdx.x * blockDim.x + threadIdx.x;
+    const uint32_t gw = blockIdx.x * (kBlock / kWave) + wave;  // global wave number
+    int l             = 0;
+#pragma unroll
+    for (int k = 1; k < VETRAST_MAX_LAYERS; ++k)
+        if (k < map.L && gw >= map.first_wave[k]) l = k;
     uint32_t off = 0, n = 0;
-    if (q < P)
+    if (gw < map.first_wave[map.L] && (uint32_t)lane < map.pixels_per_wave[l])
     {
-        off = offsets[q];
-        n   = offsets[q + 1] - off;
+        const uint32_t q = map.pixel_base[l] + (gw - map.first_wave[l]) * map.pixels_per_wave[l] + lane;
+        if (q < map.pixel_base[l + 1])
+        {
+            off = offsets[q];
+            n   = offsets[q + 1] - off;
+        }
     }
     // class = ceil(log2(n)) for 2 <= n <= 64, 0 for n <= 1 (nothing to do), 7 for n > 64
     int cls = 0;

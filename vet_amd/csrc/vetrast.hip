@@ -163,6 +163,33 @@ inline T* ws_ptr(void* ws, size_t off)
     return reinterpret_cast<T*>(static_cast<char*>(ws) + off);
 }
 
+// Pixels per wave in the sort: about 128 fragments per wave if every point were visible in the layer (N / pixels is an
+// upper bound of the mean list length that needs no device read-back), between 4 and 64, a power of two.
+SortWaveMap make_sort_wave_map(const LayerTable& ly, int N)
+{
+    SortWaveMap m;
+    std::memset(&m, 0, sizeof(m));
+    m.L           = ly.L;
+    uint32_t wave = 0;
+    for (int l = 0; l < ly.L; ++l)
+    {
+        const uint32_t pixels = (uint32_t)ly.w[l] * (uint32_t)ly.h[l];
+        const double mean_len = (double)N / (double)pixels;
+        uint32_t ppw          = 64;
+        while (ppw > 4 && mean_len * ppw > 128.0) ppw >>= 1;
+        m.first_wave[l]      = wave;
+        m.pixels_per_wave[l] = ppw;
+        m.pixel_base[l]      = ly.base[l];
+        wave += (pixels + ppw - 1) / ppw;
+    }
+    for (int l = ly.L; l <= VETRAST_MAX_LAYERS; ++l)
+    {
+        m.first_wave[l] = wave;
+        m.pixel_base[l] = ly.base[ly.L];
+    }
+    return m;
+}
+
 ViewPass make_view_pass(const vetrast_forward_args* a, const vetrast_workspace_layout& lay, const LayerTable& ly, int b)
 {
     ViewPass vp;
@@ -369,8 +396,9 @@ int vetrast_forward(vetrast_ctx* ctx, const vetrast_forward_args* a, void* strea
         if (N > 0)
         {
             ScopeTimer tm(ctx, stream, VETRAST_SCOPE_SORT);
-            hipLaunchKernelGGL(sort_lists_kernel, dim3(grid_for(P)), dim3(kBlock), 0, stream, offsets, fragments, P,
-                               p.debug_max_list_length);
+            const SortWaveMap map = make_sort_wave_map(ly, N);
+            hipLaunchKernelGGL(sort_lists_kernel, dim3((map.first_wave[L] + kBlock / kWave - 1) / (kBlock / kWave)),
+                               dim3(kBlock), 0, stream, offsets, fragments, map, p.debug_max_list_length);
         }
         {
             ScopeTimer tm(ctx, stream, VETRAST_SCOPE_BLEND);
