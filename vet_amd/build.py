@@ -68,6 +68,7 @@ def build_torch_extension(verbose=True):
 if __name__ == "__main__":
     build_library()
     print("built", LIB_PATH)
-    build_torch_extension()
-    print("built", TORCH_EXT_PATH)
+    if "--lib-only" not in sys.argv:
+        build_torch_extension()
+        print("built", TORCH_EXT_PATH)
     sys.exit(0)

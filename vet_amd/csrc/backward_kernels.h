@@ -27,6 +27,7 @@ struct BackwardPass
     float4* partial;          // [L][N] records of 2 float4: (d tex0..3), (d conf, d x, d y, d z)
     float* background_partial;  // [workgroups][8]: per-workgroup sums of d background[0..C) and of the leak term
     LayerTable ly;
+    TileMap tiles;
     uint32_t P;
     int N;
     int K;
@@ -62,8 +63,9 @@ __device__ __forceinline__ bool interior_pixel(int x, int y, int w, int h)
 template <int C>
 __global__ void __launch_bounds__(kBlock) blend_backward_kernel(BackwardPass a)
 {
-    const uint32_t q  = blockIdx.x * blockDim.x + threadIdx.x;
-    const bool active = q < a.P;
+    const TilePixel px = tile_pixel(a.tiles, a.ly);
+    const uint32_t q   = px.q;
+    const bool active  = px.active;
     float bg_grad[C];
 #pragma unroll
     for (int ci = 0; ci < C; ++ci) bg_grad[ci] = 0.f;
@@ -71,11 +73,11 @@ __global__ void __launch_bounds__(kBlock) blend_backward_kernel(BackwardPass a)
 
     if (active)
     {
-        const int l          = layer_of_pixel(a.ly, q);
+        const int l          = px.l;
         const int lw = a.ly.w[l], lh = a.ly.h[l];
         const size_t plane   = (size_t)lw * lh;
-        const uint32_t local = q - a.ly.base[l];
-        const int gy = (int)(local / (uint32_t)lw), gx = (int)(local - (uint32_t)gy * lw);
+        const uint32_t local = px.local;
+        const int gy = px.y, gx = px.x;
         const float* G = a.grad_out[l];
         float g[C];
 #pragma unroll
@@ -122,7 +124,8 @@ __global__ void __launch_bounds__(kBlock) blend_backward_kernel(BackwardPass a)
                 Gy0[ci] = Gc[-lw];
                 Gy1[ci] = Gc[lw];
             }
-            const float scale = powf(0.5f, (float)l);
+            // crop_transform.scale(0.5^layer), RenderBackward.cu:1381-1385; 2^-l is exact
+            const float scale = __uint_as_float((uint32_t)(127 - l) << 23);
             cfx               = a.view->crop[0] * scale;
             cfy               = a.view->crop[1] * scale;
             cs                = a.view->crop[4] * scale;
@@ -131,67 +134,94 @@ __global__ void __launch_bounds__(kBlock) blend_backward_kernel(BackwardPass a)
         const uint64_t* list = a.fragments + off;
         const float* Tlist   = a.transmittance + off;
         float4* partial_l    = a.partial + 2 * (size_t)l * a.N;
-        for (int j = (int)n - 1; j >= 0; --j)
+        const DeviceView& cam = *a.view;
+        // Back to front in chunks of kBlendChunk fragments; all loads of a chunk (key, stored transmittance, descriptor
+        // record, position) are issued before its arithmetic, so a thread keeps several gathers in flight.
+        for (int top = (int)n - 1; top >= 0; top -= kBlendChunk)
         {
-            const int id = (int)(uint32_t)list[j];
-            if ((uint32_t)id >= (uint32_t)a.N) continue;  // guards the gathers; never true for a valid workspace
-            const int ti = a.index ? a.index[id] : id;
-            if ((uint32_t)ti >= (uint32_t)a.N) continue;
-            const float4 t4  = a.packed[2 * (size_t)ti];
-            const float c    = a.packed[2 * (size_t)ti + 1].x;
-            const float T    = Tlist[j];
-            const float t[4] = {t4.x, t4.y, t4.z, t4.w};
-            float dot = 0.f, x = 0.f;
-            const float Tc = T * c;
-            float gt[4]    = {0.f, 0.f, 0.f, 0.f};
+            int id[kBlendChunk], ti[kBlendChunk];
+            float T[kBlendChunk], c[kBlendChunk];
+            float4 t4[kBlendChunk], pos[kBlendChunk];
 #pragma unroll
-            for (int ci = 0; ci < C; ++ci)
+            for (int u = 0; u < kBlendChunk; ++u)
             {
-                gt[ci] = Tc * g[ci];
-                dot += t[ci] * g[ci];
-                x += ((g[ci] * t[ci]) * T) * c;
+                const int j = top - u;
+                id[u] = ti[u] = -1;
+                if (j >= 0)
+                {
+                    id[u] = (int)(uint32_t)list[j];
+                    T[u]  = Tlist[j];
+                    // guards the gathers; never false for a workspace the forward pass wrote
+                    if ((uint32_t)id[u] < (uint32_t)a.N) ti[u] = a.index ? a.index[id[u]] : id[u];
+                    if ((uint32_t)ti[u] >= (uint32_t)a.N) ti[u] = -1;
+                }
             }
-            const float gconf = dot * T - S / ((1.f - c) + 1e-9f);
-            S += x;
-
-            float gp0 = 0.f, gp1 = 0.f, gp2 = 0.f;
-            if (do_point)
+#pragma unroll
+            for (int u = 0; u < kBlendChunk; ++u)
             {
-                float dR_dpx = 0.f, dR_dpy = 0.f;
+                if (ti[u] >= 0)
+                {
+                    t4[u] = a.packed[2 * (size_t)ti[u]];
+                    c[u]  = a.packed[2 * (size_t)ti[u] + 1].x;
+                    if (do_point) pos[u] = a.position[id[u]];
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < kBlendChunk; ++u)
+            {
+                if (ti[u] < 0) continue;
+                const float t[4] = {t4[u].x, t4[u].y, t4[u].z, t4[u].w};
+                float dot = 0.f, x = 0.f;
+                const float Tc = T[u] * c[u];
+                float gt[4]    = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int ci = 0; ci < C; ++ci)
                 {
-                    const float d_x0 = -(t[ci] - Ix0[ci]) * Gx0[ci];
-                    const float d_x1 = (t[ci] - Ix1[ci]) * Gx1[ci];
-                    const float d_y0 = -(t[ci] - Iy0[ci]) * Gy0[ci];
-                    const float d_y1 = (t[ci] - Iy1[ci]) * Gy1[ci];
-                    dR_dpx += 0.5f * (d_x0 + d_x1);
-                    dR_dpy += 0.5f * (d_y0 + d_y1);
+                    gt[ci] = Tc * g[ci];
+                    dot += t[ci] * g[ci];
+                    x += ((g[ci] * t[ci]) * T[u]) * c[u];
                 }
-                const float gxp = dR_dpx / (float)C, gyp = dR_dpy / (float)C;
-                const DeviceView& cam = *a.view;
-                const float4 p        = a.position[id];
-                const float vx = ((cam.r[0] * p.x + cam.r[1] * p.y) + cam.r[2] * p.z) + cam.t[0];
-                const float vy = ((cam.r[3] * p.x + cam.r[4] * p.y) + cam.r[5] * p.z) + cam.t[1];
-                const float vz = ((cam.r[6] * p.x + cam.r[7] * p.y) + cam.r[8] * p.z) + cam.t[2];
-                if (vz > 0.f)
+                const float gconf = dot * T[u] - S / ((1.f - c[u]) + 1e-9f);
+                S += x;
+
+                float gp0 = 0.f, gp1 = 0.f, gp2 = 0.f;
+                if (do_point)
                 {
-                    const float ar = cam.rot[0] * gxp + cam.rot[2] * gyp;
-                    const float br = cam.rot[1] * gxp + cam.rot[3] * gyp;
-                    const float a2 = cfx * ar;
-                    const float b2 = cs * ar + cfy * br;
-                    const float d0 = cam.fx * a2;
-                    const float d1 = cam.s * a2 + cam.fy * b2;
-                    const float iz = 1.f / vz;
-                    const float e0 = iz * d0, e1 = iz * d1;
-                    const float e2 = (-vx * iz * iz) * d0 + (-vy * iz * iz) * d1;
-                    gp0            = (cam.r[0] * e0 + cam.r[3] * e1) + cam.r[6] * e2;
-                    gp1            = (cam.r[1] * e0 + cam.r[4] * e1) + cam.r[7] * e2;
-                    gp2            = (cam.r[2] * e0 + cam.r[5] * e1) + cam.r[8] * e2;
+                    float dR_dpx = 0.f, dR_dpy = 0.f;
+#pragma unroll
+                    for (int ci = 0; ci < C; ++ci)
+                    {
+                        const float d_x0 = -(t[ci] - Ix0[ci]) * Gx0[ci];
+                        const float d_x1 = (t[ci] - Ix1[ci]) * Gx1[ci];
+                        const float d_y0 = -(t[ci] - Iy0[ci]) * Gy0[ci];
+                        const float d_y1 = (t[ci] - Iy1[ci]) * Gy1[ci];
+                        dR_dpx += 0.5f * (d_x0 + d_x1);
+                        dR_dpy += 0.5f * (d_y0 + d_y1);
+                    }
+                    const float gxp = dR_dpx / (float)C, gyp = dR_dpy / (float)C;
+                    const float4 p = pos[u];
+                    const float vx = ((cam.r[0] * p.x + cam.r[1] * p.y) + cam.r[2] * p.z) + cam.t[0];
+                    const float vy = ((cam.r[3] * p.x + cam.r[4] * p.y) + cam.r[5] * p.z) + cam.t[1];
+                    const float vz = ((cam.r[6] * p.x + cam.r[7] * p.y) + cam.r[8] * p.z) + cam.t[2];
+                    if (vz > 0.f)
+                    {
+                        const float ar = cam.rot[0] * gxp + cam.rot[2] * gyp;
+                        const float br = cam.rot[1] * gxp + cam.rot[3] * gyp;
+                        const float a2 = cfx * ar;
+                        const float b2 = cs * ar + cfy * br;
+                        const float d0 = cam.fx * a2;
+                        const float d1 = cam.s * a2 + cam.fy * b2;
+                        const float iz = 1.f / vz;
+                        const float e0 = iz * d0, e1 = iz * d1;
+                        const float e2 = (-vx * iz * iz) * d0 + (-vy * iz * iz) * d1;
+                        gp0            = (cam.r[0] * e0 + cam.r[3] * e1) + cam.r[6] * e2;
+                        gp1            = (cam.r[1] * e0 + cam.r[4] * e1) + cam.r[7] * e2;
+                        gp2            = (cam.r[2] * e0 + cam.r[5] * e1) + cam.r[8] * e2;
+                    }
                 }
+                partial_l[2 * (size_t)id[u]]     = make_float4(gt[0], gt[1], gt[2], gt[3]);
+                partial_l[2 * (size_t)id[u] + 1] = make_float4(gconf, gp0, gp1, gp2);
             }
-            partial_l[2 * (size_t)id]     = make_float4(gt[0], gt[1], gt[2], gt[3]);
-            partial_l[2 * (size_t)id + 1] = make_float4(gconf, gp0, gp1, gp2);
         }
     }
 

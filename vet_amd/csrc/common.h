@@ -13,6 +13,7 @@ constexpr uint32_t kNoSlot    = 0xFFFFFFFFu;
 constexpr uint64_t kInfKey    = ~0ull;        // sorts behind every real (depth bits, point id) key
 constexpr int kScanPerThread  = 16;
 constexpr int kScanPerBlock   = kBlock * kScanPerThread;  // 4096 counts per workgroup
+constexpr int kBlendChunk     = 4;            // fragments a blend / backward thread prefetches at a time
 constexpr int kBackgroundRow  = 8;            // floats per workgroup row of background-gradient partial sums
 constexpr int kPackedFloats   = 8;            // interleaved record: 4 descriptor floats, confidence, 3 pad
 
@@ -106,8 +107,56 @@ __device__ __forceinline__ int layer_of_pixel(const LayerTable& ly, uint32_t q)
     return l;
 }
 
-// ---- host-side launchers (one per source file) -------------------------------------------------------------
-struct ForwardLaunch;
-struct BackwardLaunch;
+// Workgroup -> pixel mapping of the per-pixel kernels (blend, backward). A workgroup owns a 16x16 pixel tile (a wave
+// 16x4 of it), because the fragments of neighbouring pixels come from the same few 256-point blocks of the cloud and
+// their descriptor / position records then share cache lines. Workgroups are dealt round-robin to the 8 XCDs, each with
+// its own L2, so XCD k = b % 8 is given the k-th eighth of the tiles of EVERY layer (the coarse layers carry as many
+// fragments as the fine ones in far fewer tiles, so each XCD needs its share of each), coarsest layer first: every XCD
+// walks contiguous runs of tiles and finds in its L2 the lines the tile before (and the tile row above) brought in.
+constexpr int kTile = 16;
+constexpr int kXcds = 8;
+struct TileMap
+{
+    int L;
+    uint32_t tiles[VETRAST_MAX_LAYERS];    // tiles of layer l
+    uint32_t tiles_x[VETRAST_MAX_LAYERS];  // tiles per tile row of layer l
+    uint32_t chunk[VETRAST_MAX_LAYERS];    // tiles of layer l per XCD = ceil(tiles / 8)
+    uint32_t start[VETRAST_MAX_LAYERS];    // first per-XCD slot of layer l (slots run from the coarsest layer down)
+    uint32_t slots_per_xcd;                // sum of chunk[]
+};
+
+struct TilePixel
+{
+    bool active;
+    int l, x, y;
+    uint32_t q;      // pixel number over all layers
+    uint32_t local;  // y * w + x inside the layer
+};
+
+__device__ __forceinline__ TilePixel tile_pixel(const TileMap& tm, const LayerTable& ly)
+{
+    TilePixel r;
+    r.active = false;
+    r.l = r.x = r.y = 0;
+    r.q = r.local = 0;
+    const uint32_t b    = blockIdx.x;
+    const uint32_t xcd  = b % kXcds;
+    const uint32_t slot = b / kXcds;
+    int l               = 0;
+#pragma unroll
+    for (int k = 1; k < VETRAST_MAX_LAYERS; ++k)
+        if (k < tm.L && slot < tm.start[k - 1]) l = k;  // start[] decreases with l: start[L-1] = 0
+    const uint32_t t = xcd * tm.chunk[l] + (slot - tm.start[l]);
+    if (slot >= tm.slots_per_xcd || t >= tm.tiles[l]) return r;
+    const uint32_t ty = t / tm.tiles_x[l], tx = t - ty * tm.tiles_x[l];
+    r.l               = l;
+    r.x               = (int)(tx * kTile + (threadIdx.x & (kTile - 1)));
+    r.y               = (int)(ty * kTile + (threadIdx.x / kTile));
+    if (r.x >= ly.w[l] || r.y >= ly.h[l]) return r;
+    r.local  = (uint32_t)r.y * (uint32_t)ly.w[l] + (uint32_t)r.x;
+    r.q      = ly.base[l] + r.local;
+    r.active = true;
+    return r;
+}
 
 }  // namespace vetrast

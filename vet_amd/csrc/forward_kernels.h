@@ -247,6 +247,7 @@ struct BlendPass
     float* out[VETRAST_MAX_LAYERS];       // already offset to this view
     float* out_mask[VETRAST_MAX_LAYERS];  // already offset to this view, or null
     LayerTable ly;
+    TileMap tiles;
     uint32_t P;
     int N;
     int K;
@@ -256,12 +257,14 @@ struct BlendPass
 
 // One thread per pixel walks the sorted list front to back: out += (T*c)*t, T = (1-c)*T, in exactly this order, then
 // the background behind the last fragment. Counterpart of BlendMulti (src/lib/rendering/RenderForward.cu:1303-1357)
-// and CreateMask (src/lib/rendering/PointRenderer.cu:216-235). Pixels of all layers are served by one launch.
+// and CreateMask (src/lib/rendering/PointRenderer.cu:216-235). Pixels of all layers are served by one launch; the
+// reference also uses 16x16 workgroups (RenderForward.cu:1385), one launch per layer.
 template <int C>
 __global__ void __launch_bounds__(kBlock) blend_kernel(BlendPass a)
 {
-    const uint32_t q = blockIdx.x * blockDim.x + threadIdx.x;
-    if (q >= a.P) return;
+    const TilePixel px = tile_pixel(a.tiles, a.ly);
+    if (!px.active) return;
+    const uint32_t q   = px.q;
     const uint32_t off = a.offsets[q];
     uint32_t n         = a.offsets[q + 1] - off;
     if (a.K > 0) n = min(n, (uint32_t)a.K);
@@ -270,24 +273,53 @@ __global__ void __launch_bounds__(kBlock) blend_kernel(BlendPass a)
 #pragma unroll
     for (int ci = 0; ci < C; ++ci) color[ci] = 0.f;
     const uint64_t* list = a.fragments + off;
-    for (uint32_t i = 0; i < n; ++i)
+    // The list is walked in chunks of kBlendChunk fragments: all keys of a chunk are loaded first, then all descriptor
+    // records, and only then the (strictly sequential) blend arithmetic runs, so a thread keeps several gathers in
+    // flight instead of one dependent load chain per fragment.
+    for (uint32_t base = 0; base < n; base += kBlendChunk)
     {
-        const int id = (int)(uint32_t)list[i];
-        if ((uint32_t)id >= (uint32_t)a.N) break;  // cannot happen for a list the fill pass wrote; guards the gather
-        const int ti = a.index ? a.index[id] : id;
-        if ((uint32_t)ti >= (uint32_t)a.N) break;  // texture index out of range (the reference asserts here)
-        const float4 t4 = a.packed[2 * (size_t)ti];
-        const float c   = a.packed[2 * (size_t)ti + 1].x;
-        if (a.transmittance) a.transmittance[off + i] = T;
-        const float t[4] = {t4.x, t4.y, t4.z, t4.w};
-        const float Tc   = T * c;
+        int ti[kBlendChunk];
+        float4 t4[kBlendChunk];
+        float c[kBlendChunk];
 #pragma unroll
-        for (int ci = 0; ci < C; ++ci) color[ci] = Tc * t[ci] + color[ci];
-        T = (1.f - c) * T;
+        for (int u = 0; u < kBlendChunk; ++u)
+        {
+            ti[u] = -1;
+            if (base + u < n)
+            {
+                const int id = (int)(uint32_t)list[base + u];
+                // an id or texture index out of range cannot come from a list the fill pass wrote; such a fragment is
+                // skipped instead of gathered (the reference asserts on the texture index, RenderForward.cu:1335-1336)
+                if ((uint32_t)id < (uint32_t)a.N) ti[u] = a.index ? a.index[id] : id;
+                if ((uint32_t)ti[u] >= (uint32_t)a.N) ti[u] = -1;
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < kBlendChunk; ++u)
+        {
+            if (ti[u] >= 0)
+            {
+                t4[u] = a.packed[2 * (size_t)ti[u]];
+                c[u]  = a.packed[2 * (size_t)ti[u] + 1].x;
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < kBlendChunk; ++u)
+        {
+            if (ti[u] >= 0)
+            {
+                if (a.transmittance) a.transmittance[off + base + u] = T;
+                const float t[4] = {t4[u].x, t4[u].y, t4[u].z, t4[u].w};
+                const float Tc   = T * c[u];
+#pragma unroll
+                for (int ci = 0; ci < C; ++ci) color[ci] = Tc * t[ci] + color[ci];
+                T = (1.f - c[u]) * T;
+            }
+        }
     }
-    const int l          = layer_of_pixel(a.ly, q);
+    const int l          = px.l;
     const size_t plane   = (size_t)a.ly.w[l] * a.ly.h[l];
-    const uint32_t local = q - a.ly.base[l];
+    const uint32_t local = px.local;
 #pragma unroll
     for (int ci = 0; ci < C; ++ci)
     {

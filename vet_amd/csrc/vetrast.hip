@@ -190,6 +190,27 @@ SortWaveMap make_sort_wave_map(const LayerTable& ly, int N)
     return m;
 }
 
+TileMap make_tile_map(const LayerTable& ly)
+{
+    TileMap m;
+    std::memset(&m, 0, sizeof(m));
+    m.L = ly.L;
+    for (int l = 0; l < ly.L; ++l)
+    {
+        m.tiles_x[l] = (uint32_t)(ly.w[l] + kTile - 1) / kTile;
+        m.tiles[l]   = m.tiles_x[l] * ((uint32_t)(ly.h[l] + kTile - 1) / kTile);
+        m.chunk[l]   = (m.tiles[l] + kXcds - 1) / kXcds;
+    }
+    uint32_t slot = 0;
+    for (int l = ly.L - 1; l >= 0; --l)
+    {
+        m.start[l] = slot;
+        slot += m.chunk[l];
+    }
+    m.slots_per_xcd = slot;
+    return m;
+}
+
 ViewPass make_view_pass(const vetrast_forward_args* a, const vetrast_workspace_layout& lay, const LayerTable& ly, int b)
 {
     ViewPass vp;
@@ -298,7 +319,7 @@ int vetrast_workspace_layout_for(int32_t N, int32_t B, int32_t L, int32_t w, int
     lay->partial_base       = at;
     at += align_up(cap * 8 * sizeof(float), kAlign);
     lay->background_partial_base = at;
-    at += align_up(((P + kBlock - 1) / kBlock) * kBackgroundRow * sizeof(float), kAlign);
+    at += align_up((size_t)make_tile_map(t).slots_per_xcd * kXcds * kBackgroundRow * sizeof(float), kAlign);
     lay->total_bytes = align_up(at, kAlign);
     return VETRAST_OK;
 }
@@ -320,6 +341,7 @@ int vetrast_forward(vetrast_ctx* ctx, const vetrast_forward_args* a, void* strea
     const vetrast_params& p = a->params;
     const int N = a->num_points, B = a->num_views, L = p.num_layers, C = p.num_texture_channels;
     const LayerTable ly = make_layer_table(a->views[0].w, a->views[0].h, L);
+    const TileMap tiles = make_tile_map(ly);
     const uint32_t P    = ly.base[L];
     const size_t Ppad   = lay.offsets_stride / sizeof(uint32_t);
     void* ws            = a->workspace;
@@ -411,6 +433,7 @@ int vetrast_forward(vetrast_ctx* ctx, const vetrast_forward_args* a, void* strea
             bp.transmittance       = a->save_for_backward ? trans : nullptr;
             bp.weight              = weight;
             bp.ly                  = ly;
+            bp.tiles               = tiles;
             bp.P                   = P;
             bp.N                   = N;
             bp.K                   = p.debug_max_list_length;
@@ -425,7 +448,7 @@ int vetrast_forward(vetrast_ctx* ctx, const vetrast_forward_args* a, void* strea
                 bp.out[l]          = a->out[l] + (size_t)b * C * plane;
                 if (p.output_background_mask) bp.out_mask[l] = a->out_mask[l] + (size_t)b * plane;
             }
-            const dim3 g(grid_for(P)), blk(kBlock);
+            const dim3 g(tiles.slots_per_xcd * kXcds), blk(kBlock);
             switch (C)
             {
                 case 1: hipLaunchKernelGGL(blend_kernel<1>, g, blk, 0, stream, bp); break;
@@ -456,6 +479,7 @@ int vetrast_backward(vetrast_ctx* ctx, const vetrast_backward_args* g, void* str
     hipStream_t stream = (hipStream_t)stream_;
     const int N = a->num_points, B = a->num_views, L = p.num_layers, C = p.num_texture_channels;
     const LayerTable ly = make_layer_table(a->views[0].w, a->views[0].h, L);
+    const TileMap tiles = make_tile_map(ly);
     const uint32_t P    = ly.base[L];
     void* ws            = a->workspace;
 
@@ -502,6 +526,7 @@ int vetrast_backward(vetrast_ctx* ctx, const vetrast_backward_args* g, void* str
             bp.partial          = partial;
             bp.background_partial = background_rows;
             bp.ly               = ly;
+            bp.tiles            = tiles;
             bp.P                = P;
             bp.N                = N;
             bp.K                = p.debug_max_list_length;
@@ -517,7 +542,7 @@ int vetrast_backward(vetrast_ctx* ctx, const vetrast_backward_args* g, void* str
                 bp.grad_out[l]     = g->grad_out[l] + (size_t)b * C * plane;
                 bp.out[l]          = a->out[l] + (size_t)b * C * plane;
             }
-            const dim3 grid(grid_for(P)), blk(kBlock);
+            const dim3 grid(tiles.slots_per_xcd * kXcds), blk(kBlock);
             switch (C)
             {
                 case 1: hipLaunchKernelGGL(blend_backward_kernel<1>, grid, blk, 0, stream, bp); break;
@@ -554,7 +579,7 @@ int vetrast_backward(vetrast_ctx* ctx, const vetrast_backward_args* g, void* str
             // after the per-point kernel: it overwrites confidence row 0, the leak term is added on top
             ScopeTimer tm(ctx, stream, VETRAST_SCOPE_BACKWARD_GATHER);
             hipLaunchKernelGGL(reduce_background_kernel, dim3(1), dim3(kBlock), 0, stream, background_rows,
-                               grid_for(P), C, g->grad_background, g->grad_confidence,
+                               (int)(tiles.slots_per_xcd * kXcds), C, g->grad_background, g->grad_confidence,
                                (p.quirk_background_confidence_leak && !p.use_environment_map && N > 0) ? 1 : 0,
                                b > 0 ? 1 : 0);
         }

@@ -166,6 +166,36 @@ def surface_points(seed, num_primitives, points_per_primitive, box=5.0, jitter=0
     return pts
 
 
+def _spread_bits21(v):
+    """Spreads the low 21 bits of v so that two zero bits follow every bit (3-D Morton interleave)."""
+    v = v.astype(np.uint64) & np.uint64(0x1FFFFF)
+    v = (v | (v << np.uint64(32))) & np.uint64(0x1F00000000FFFF)
+    v = (v | (v << np.uint64(16))) & np.uint64(0x1F0000FF0000FF)
+    v = (v | (v << np.uint64(8))) & np.uint64(0x100F00F00F00F00F)
+    v = (v | (v << np.uint64(4))) & np.uint64(0x10C30C30C30C30C3)
+    v = (v | (v << np.uint64(2))) & np.uint64(0x1249249249249249)
+    return v
+
+
+def vet_preprocess_order(xyz, seed, block=256):
+    """The point order VET's scene preprocessing produces before the rasterizer ever sees a cloud:
+    ReorderMorton64() followed by RandomBlockShuffle(256) (src/lib/data/SceneData.cpp:105-106 of the reference).
+    Returns the permutation: 63-bit Morton order of the positions in their bounding box, then whole blocks of `block`
+    consecutive points shuffled with the seeded generator."""
+    xyz = np.asarray(xyz, dtype=np.float64)
+    lo, hi = xyz.min(axis=0), xyz.max(axis=0)
+    cell = np.floor((xyz - lo) / np.maximum(hi - lo, 1e-30) * ((1 << 21) - 1)).astype(np.uint64)
+    code = _spread_bits21(cell[:, 0]) | (_spread_bits21(cell[:, 1]) << np.uint64(1)) | (_spread_bits21(cell[:, 2]) << np.uint64(2))
+    order = np.argsort(code, kind="stable")
+    n = order.shape[0]
+    nb = (n + block - 1) // block
+    keys = Stream(seed, "block_shuffle").u64(nb)
+    block_perm = np.argsort(keys, kind="stable")
+    idx = (block_perm[:, None] * block + np.arange(block)[None, :]).reshape(-1)
+    idx = idx[idx < n]
+    return order[idx]
+
+
 def _descriptors(seed, N, channels=4, sigma=0.5):
     tex = (sigma * Stream(seed, "texture").normal(channels * N)).reshape(channels, N).astype(np.float32)
     conf = sigmoid(Stream(seed, "confidence").normal(N)).astype(np.float32)
@@ -173,13 +203,21 @@ def _descriptors(seed, N, channels=4, sigma=0.5):
     return tex, conf, bg
 
 
-def config2(num_points=2_000_000, seed=1, w=1920, h=1080, num_layers=4, K=16) -> Scene:
-    """SfM-like scene: points on 200 planes/spheres in a 10 m box, 1080p, fx=1000, 4 layers, K=16."""
+def config2(num_points=2_000_000, seed=1, w=1920, h=1080, num_layers=4, K=16, point_order="vet_preprocess") -> Scene:
+    """SfM-like scene: points on 200 planes/spheres in a 10 m box, 1080p, fx=1000, 4 layers, K=16.
+
+    point_order: "vet_preprocess" lists the points the way VET's loader hands them to the rasterizer (Morton order,
+    256-point blocks shuffled); "generated" keeps the generator's order (primitive by primitive, random inside)."""
     prims = 200
     per = max(1, num_points // prims)
     N = prims * per
     pos = np.empty((N, 4), dtype=np.float32)
-    pos[:, :3] = surface_points(seed, prims, per).astype(np.float32)
+    xyz = surface_points(seed, prims, per)
+    if point_order == "vet_preprocess":
+        xyz = xyz[vet_preprocess_order(xyz, seed)]
+    else:
+        assert point_order == "generated", point_order
+    pos[:, :3] = xyz.astype(np.float32)
     pos[:, 3] = 0.01
     tex, conf, bg = _descriptors(seed, N)
     scale = w / 1920.0
