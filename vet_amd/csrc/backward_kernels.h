@@ -19,12 +19,10 @@ struct BackwardPass
     const float* weight;         // per pixel: transmittance behind the last kept fragment
     const int32_t* index;
     const float4* packed;
-    const float4* position;
     const float* background;
-    const DeviceView* view;
     const float* grad_out[VETRAST_MAX_LAYERS];  // already offset to this view
     const float* out[VETRAST_MAX_LAYERS];       // forward result, already offset to this view
-    float4* partial;          // [L][N] records of 2 float4: (d tex0..3), (d conf, d x, d y, d z)
+    float4* partial;          // [L][N] records of 2 float4: (d tex0..3), (d conf, d image x, d image y, 0)
     float* background_partial;  // [workgroups][8]: per-workgroup sums of d background[0..C) and of the leak term
     LayerTable ly;
     TileMap tiles;
@@ -106,7 +104,6 @@ __global__ void __launch_bounds__(kBlock) blend_backward_kernel(BackwardPass a)
         // neighbour samples for the position heuristic, shared by every fragment of the pixel
         const bool do_point = a.need_point_gradient && n > 0 && interior_pixel(gx, gy, lw, lh);
         float Ix0[C], Ix1[C], Iy0[C], Iy1[C], Gx0[C], Gx1[C], Gy0[C], Gy1[C];
-        float cfx = 0.f, cfy = 0.f, cs = 0.f;
         if (do_point)
         {
             const float* I = a.out[l];
@@ -124,24 +121,18 @@ __global__ void __launch_bounds__(kBlock) blend_backward_kernel(BackwardPass a)
                 Gy0[ci] = Gc[-lw];
                 Gy1[ci] = Gc[lw];
             }
-            // crop_transform.scale(0.5^layer), RenderBackward.cu:1381-1385; 2^-l is exact
-            const float scale = __uint_as_float((uint32_t)(127 - l) << 23);
-            cfx               = a.view->crop[0] * scale;
-            cfy               = a.view->crop[1] * scale;
-            cs                = a.view->crop[4] * scale;
         }
 
         const uint64_t* list = a.fragments + off;
         const float* Tlist   = a.transmittance + off;
         float4* partial_l    = a.partial + 2 * (size_t)l * a.N;
-        const DeviceView& cam = *a.view;
         // Back to front in chunks of kBlendChunk fragments; all loads of a chunk (key, stored transmittance, descriptor
         // record, position) are issued before its arithmetic, so a thread keeps several gathers in flight.
         for (int top = (int)n - 1; top >= 0; top -= kBlendChunk)
         {
             int id[kBlendChunk], ti[kBlendChunk];
             float T[kBlendChunk], c[kBlendChunk];
-            float4 t4[kBlendChunk], pos[kBlendChunk];
+            float4 t4[kBlendChunk];
 #pragma unroll
             for (int u = 0; u < kBlendChunk; ++u)
             {
@@ -163,7 +154,6 @@ __global__ void __launch_bounds__(kBlock) blend_backward_kernel(BackwardPass a)
                 {
                     t4[u] = a.packed[2 * (size_t)ti[u]];
                     c[u]  = a.packed[2 * (size_t)ti[u] + 1].x;
-                    if (do_point) pos[u] = a.position[id[u]];
                 }
             }
 #pragma unroll
@@ -184,7 +174,7 @@ __global__ void __launch_bounds__(kBlock) blend_backward_kernel(BackwardPass a)
                 const float gconf = dot * T[u] - S / ((1.f - c[u]) + 1e-9f);
                 S += x;
 
-                float gp0 = 0.f, gp1 = 0.f, gp2 = 0.f;
+                float gp0 = 0.f, gp1 = 0.f;
                 if (do_point)
                 {
                     float dR_dpx = 0.f, dR_dpy = 0.f;
@@ -198,29 +188,11 @@ __global__ void __launch_bounds__(kBlock) blend_backward_kernel(BackwardPass a)
                         dR_dpx += 0.5f * (d_x0 + d_x1);
                         dR_dpy += 0.5f * (d_y0 + d_y1);
                     }
-                    const float gxp = dR_dpx / (float)C, gyp = dR_dpy / (float)C;
-                    const float4 p = pos[u];
-                    const float vx = ((cam.r[0] * p.x + cam.r[1] * p.y) + cam.r[2] * p.z) + cam.t[0];
-                    const float vy = ((cam.r[3] * p.x + cam.r[4] * p.y) + cam.r[5] * p.z) + cam.t[1];
-                    const float vz = ((cam.r[6] * p.x + cam.r[7] * p.y) + cam.r[8] * p.z) + cam.t[2];
-                    if (vz > 0.f)
-                    {
-                        const float ar = cam.rot[0] * gxp + cam.rot[2] * gyp;
-                        const float br = cam.rot[1] * gxp + cam.rot[3] * gyp;
-                        const float a2 = cfx * ar;
-                        const float b2 = cs * ar + cfy * br;
-                        const float d0 = cam.fx * a2;
-                        const float d1 = cam.s * a2 + cam.fy * b2;
-                        const float iz = 1.f / vz;
-                        const float e0 = iz * d0, e1 = iz * d1;
-                        const float e2 = (-vx * iz * iz) * d0 + (-vy * iz * iz) * d1;
-                        gp0            = (cam.r[0] * e0 + cam.r[3] * e1) + cam.r[6] * e2;
-                        gp1            = (cam.r[1] * e0 + cam.r[4] * e1) + cam.r[7] * e2;
-                        gp2            = (cam.r[2] * e0 + cam.r[5] * e1) + cam.r[8] * e2;
-                    }
+                    gp0 = dR_dpx / (float)C;  // image-space gradient of this fragment at the layer's resolution;
+                    gp1 = dR_dpy / (float)C;  // the per-point kernel pushes it through the projection Jacobian
                 }
                 partial_l[2 * (size_t)id[u]]     = make_float4(gt[0], gt[1], gt[2], gt[3]);
-                partial_l[2 * (size_t)id[u] + 1] = make_float4(gconf, gp0, gp1, gp2);
+                partial_l[2 * (size_t)id[u] + 1] = make_float4(gconf, gp0, gp1, 0.f);
             }
         }
     }
@@ -316,8 +288,14 @@ __global__ void __launch_bounds__(kBlock) gather_point_gradients_kernel(GatherPa
     for (int ci = 0; ci < C; ++ci) gt[ci] = 0.f;
     float gc = 0.f, gx = 0.f, gy = 0.f, gz = 0.f, cnt = 0.f;
     Projected p;
-    if (!point_is_skipped(a.vp, i) && project_point(*a.vp.view, a.vp.position[i], p))
+    const DeviceView& cam = *a.vp.view;
+    const float4 wp       = a.vp.position[i];
+    if (!point_is_skipped(a.vp, i) && project_point(cam, wp, p))
     {
+        // view-space position again, for the projection Jacobian (same expressions as project_point)
+        const float vx = ((cam.r[0] * wp.x + cam.r[1] * wp.y) + cam.r[2] * wp.z) + cam.t[0];
+        const float vy = ((cam.r[3] * wp.x + cam.r[4] * wp.y) + cam.r[5] * wp.z) + cam.t[1];
+        const float vz = ((cam.r[6] * wp.x + cam.r[7] * wp.y) + cam.r[8] * wp.z) + cam.t[2];
         const uint64_t key = ((uint64_t)__float_as_uint(p.z) << 32) | (uint32_t)i;
         float ipx = p.ipx, ipy = p.ipy, radius = p.radius;
         const LayerTable& ly = a.vp.ly;
@@ -339,9 +317,24 @@ __global__ void __launch_bounds__(kBlock) gather_point_gradients_kernel(GatherPa
             gc += r1.x;
             if (a.need_point_gradient && interior_pixel(x, y, ly.w[l], ly.h[l]))
             {
-                gx += r1.y;
-                gy += r1.z;
-                gz += r1.w;
+                // ProjectPointPinholeBackward (src/lib/rendering/PointRendererHelper.h:317-372) for zero distortion, with
+                // the crop transform scaled by 0.5^layer (src/lib/rendering/RenderBackward.cu:1381-1385; 2^-l is exact):
+                // crop rotation^T, crop K^T, K^T, divide-by-z Jacobian^T, R^T.
+                const float scale = __uint_as_float((uint32_t)(127 - l) << 23);
+                const float cfx = cam.crop[0] * scale, cfy = cam.crop[1] * scale, cs = cam.crop[4] * scale;
+                const float gxp = r1.y, gyp = r1.z;
+                const float ar = cam.rot[0] * gxp + cam.rot[2] * gyp;
+                const float br = cam.rot[1] * gxp + cam.rot[3] * gyp;
+                const float a2 = cfx * ar;
+                const float b2 = cs * ar + cfy * br;
+                const float d0 = cam.fx * a2;
+                const float d1 = cam.s * a2 + cam.fy * b2;
+                const float iz = 1.f / vz;
+                const float e0 = iz * d0, e1 = iz * d1;
+                const float e2 = (-vx * iz * iz) * d0 + (-vy * iz * iz) * d1;
+                gx += (cam.r[0] * e0 + cam.r[3] * e1) + cam.r[6] * e2;
+                gy += (cam.r[1] * e0 + cam.r[4] * e1) + cam.r[7] * e2;
+                gz += (cam.r[2] * e0 + cam.r[5] * e1) + cam.r[8] * e2;
                 cnt += 1.f;
             }
         }

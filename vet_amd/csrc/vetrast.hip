@@ -520,9 +520,7 @@ int vetrast_backward(vetrast_ctx* ctx, const vetrast_backward_args* g, void* str
             bp.weight           = ws_ptr<float>(ws, lay.weight_base + lay.weight_stride * b);
             bp.index            = a->index;
             bp.packed           = ws_ptr<float4>(ws, lay.packed_base);
-            bp.position         = reinterpret_cast<const float4*>(a->position);
             bp.background       = a->background;
-            bp.view             = ws_ptr<DeviceView>(ws, lay.views_base) + b;
             bp.partial          = partial;
             bp.background_partial = background_rows;
             bp.ly               = ly;
