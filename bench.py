@@ -1,16 +1,18 @@
 #!/usr/bin/env python3
 """Benchmark of the blending point rasterizer on one MI355X.
 
-One step = one forward + backward pass of the hot path over one frame of synthetic input (config 3: 2 M points on 200
-planes/spheres, 1920x1080, 4 layers, K=16, gradients to descriptors, confidence and xyz). Inputs, outputs and the
-workspace are resident in HBM before the timed region starts. Prints ONE JSON line.
+One step = one forward + backward pass of the hot path over one frame of synthetic input (BASELINE config 3: 2 M points
+on 200 planes/spheres, 1920x1080, 4 layers, K=16, gradients to descriptors, confidence and xyz). Inputs, outputs and
+the workspace are resident in HBM before the timed region starts. Prints ONE JSON line.
 
-  python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 2|3|5] [--no-cpu-baseline]
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 2|3|5] [--point-order vet_preprocess|generated]
+                  [--no-cpu-baseline] [--no-second-order]
 """
 import argparse
 import ctypes as C
 import json
 import os
+import re
 import sys
 import time
 
@@ -20,10 +22,12 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic_config3.md")
 
 
 def algorithmic_bytes(N, P, F, Fk, Cn):
-    """Compulsory bytes per view and pass, each datum counted once per producer and once per consumer (4-byte scalars).
+    """Compulsory bytes per view and kernel, each datum counted once per producer and once per consumer (4-byte scalars):
+    B_fwd = 32N + 36P + 24F + 28Fk, B_bwd = 32P + 116Fk + 40N for C = 4.
 
     N points, P pixels over all layers, F fragments, Fk fragments kept after the top-K cut.
     """
@@ -34,57 +38,43 @@ def algorithmic_bytes(N, P, F, Fk, Cn):
         "SORT": 16 * F,                               # records read and written
         "BLEND": 8 * Fk + (4 * Cn + 4) * Fk + 4 * P + 4 * Cn * P + 4 * P,  # lists, descriptor+confidence, offsets, out, weight
     }
-    # B_bwd = 32P + 116Fk + 40N for C = 4, split over the two backward kernels: the per-pixel kernel reads upstream
-    # grads and forward outputs (8CP), lists (8Fk), descriptor+confidence (4(C+1)Fk), positions (16Fk) and writes one
-    # half of the gradient read-modify-write (4(C+1+4)Fk); the per-point kernel reads that half back and writes the
-    # gradient rows (4(C+1+4+1)N, the term the reference spends on zero-filling them).
+    # The per-pixel kernel reads upstream grads and forward outputs (8CP), lists (8Fk), descriptor+confidence (4(C+1)Fk)
+    # and writes one half of the gradient read-modify-write (4(C+1+4)Fk); the per-point kernel reads positions (16Fk in the
+    # model), that half back, and writes the gradient rows (4(C+1+4+1)N, the term the reference spends on zero-filling).
     rmw_half = 4 * (Cn + 1 + 4) * Fk
     bwd = {
-        "BACKWARD_BLEND": 8 * Cn * P + 8 * Fk + (4 * Cn + 4) * Fk + 16 * Fk + rmw_half,
-        "BACKWARD_GATHER": rmw_half + 4 * (Cn + 1 + 4 + 1) * N,
+        "BACKWARD_BLEND": 8 * Cn * P + 8 * Fk + (4 * Cn + 4) * Fk + rmw_half,
+        "BACKWARD_GATHER": 16 * Fk + rmw_half + 4 * (Cn + 1 + 4 + 1) * N,
     }
     return fwd, bwd
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--config", type=int, default=3, choices=[2, 3, 5])
-    ap.add_argument("--points", type=int, default=None, help="override the point count (parity/debug runs)")
-    ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--cpu-threads", type=int, default=0, help="0 = min(16, available cores)")
-    args = ap.parse_args()
-    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
-        print("bench.py: this build runs the rasterizer on ONE GPU (views of a batch are rendered back to back); "
-              "--gpus N with N > 1 is not available", file=sys.stderr)
-        sys.exit(2)
+def measured_traffic():
+    """HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs, read from the committed summary
+    (rows `| SCOPE | fetch KiB | write KiB |`, already scaled by the copy-kernel calibration). Empty if absent."""
+    res = {}
+    if not os.path.exists(TRAFFIC_FILE):
+        return res
+    for line in open(TRAFFIC_FILE):
+        m = re.match(r"^\|\s*([A-Z_]+)\s*\|\s*([0-9.]+)\s*\|\s*([0-9.]+)\s*\|", line)
+        if m:
+            res[m.group(1)] = (float(m.group(2)) + float(m.group(3))) * 1024.0
+    return res
 
+
+def run_scene(scene, backward, steps, warmup, profile=True):
     import torch
 
-    from vet_amd import abi, synthetic
+    from vet_amd import abi
     from vet_amd.rasterizer import DeviceScene, Rasterizer, make_params
 
-    if not torch.cuda.is_available():
-        print("bench.py needs a GPU (there is no CPU path in the product)", file=sys.stderr)
-        sys.exit(2)
-
-    kw = {} if args.points is None else {"num_points": args.points}
-    if args.config == 2:
-        scene, backward = synthetic.config2(**kw), False
-    elif args.config == 3:
-        scene, backward = synthetic.config3(**kw), True
-    else:
-        scene, backward = synthetic.config5(**kw), True
     params = make_params(scene, need_point_gradient=1 if backward else 0)
     N, Cn, L = scene.num_points, scene.num_channels, scene.num_layers
-
     rast = Rasterizer()
     dev = DeviceScene(scene)
     lay = rast.layout(scene)
     workspace = torch.empty(lay.total_bytes, dtype=torch.uint8, device="cuda")
-    out = [torch.empty((1, Cn, h, w), dtype=torch.float32, device="cuda") for (w, h) in scene.layer_sizes()]
+    out = [torch.empty((len(scene.views), Cn, h, w), dtype=torch.float32, device="cuda") for (w, h) in scene.layer_sizes()]
     fwd = rast.forward(dev, params, save_for_backward=backward, workspace=workspace, out=out)
     torch.cuda.synchronize()
     off = fwd.offsets(0)
@@ -95,62 +85,108 @@ def main():
     Fk = int(np.minimum(counts, K).sum()) if K > 0 else F
     F_layers = [int(off[int(lay.layer_pixel_base[l + 1])] - off[int(lay.layer_pixel_base[l])]) for l in range(L)]
 
-    grad_out = [torch.from_numpy(g).cuda() for g in scene.grad_out()] if backward else None
     bargs = None
     if backward:
+        grad_out = [torch.from_numpy(g).cuda() for g in scene.grad_out()]
         first = rast.backward(fwd, grad_out)  # allocates the gradient tensors once; reused below
         bargs = first["_args"]
     stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
     lib, ctx = rast.lib, rast.ctx
 
-    def step():
-        abi.check(lib.vetrast_forward(ctx, C.byref(fwd.args), stream), "forward")
-        if backward:
-            abi.check(lib.vetrast_backward(ctx, C.byref(bargs), stream), "backward")
-
     def forward_only():
         abi.check(lib.vetrast_forward(ctx, C.byref(fwd.args), stream), "forward")
 
-    def timed(fn, warmup, steps):
-        for _ in range(warmup):
+    def step():
+        forward_only()
+        if backward:
+            abi.check(lib.vetrast_backward(ctx, C.byref(bargs), stream), "backward")
+
+    def timed(fn, nwarm, nsteps):
+        for _ in range(nwarm):
             fn()
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        for _ in range(steps):
+        for _ in range(nsteps):
             fn()
         torch.cuda.synchronize()
-        return (time.perf_counter() - t0) * 1e3 / steps
+        return (time.perf_counter() - t0) * 1e3 / nsteps
 
-    ms_step = timed(step, args.warmup, args.steps)
-    ms_fwd = timed(forward_only, 2, args.steps) if backward else ms_step
+    res = {"ms_step": timed(step, warmup, steps)}
+    res["ms_fwd"] = timed(forward_only, 2, steps) if backward else res["ms_step"]
+    res.update(N=N, P=P, F=F, Fk=Fk, F_layers=F_layers, K=K, Cn=Cn, L=L, params=params)
+    if profile:
+        # per-kernel times: HIP events recorded by the library on the launch stream around every scope
+        rast.set_profiling(True)
+        for _ in range(3):
+            step()
+        torch.cuda.synchronize()
+        rast.reset_scope_times()
+        prof_steps = max(5, min(steps, 20))
+        for _ in range(prof_steps):
+            step()
+        torch.cuda.synchronize()
+        scopes = rast.scope_times()
+        rast.set_profiling(False)
+        res["per_launch_ms"] = {k: (ms / n if n else 0.0) for k, (ms, n) in scopes.items()}
+        res["per_step_ms"] = {k: ms / prof_steps for k, (ms, n) in scopes.items()}
+    del workspace, out, fwd
+    torch.cuda.empty_cache()
+    return res
 
-    # ---- per-kernel times, HIP events on the launch stream ------------------------------------------------------
-    rast.set_profiling(True)
-    for _ in range(3):
-        step()
-    torch.cuda.synchronize()
-    rast.reset_scope_times()
-    prof_steps = max(5, min(args.steps, 20))
-    for _ in range(prof_steps):
-        step()
-    torch.cuda.synchronize()
-    scopes = rast.scope_times()
-    rast.set_profiling(False)
-    per_launch_ms = {k: (ms / n if n else 0.0) for k, (ms, n) in scopes.items()}
-    per_step_ms = {k: ms / prof_steps for k, (ms, n) in scopes.items()}
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--config", type=int, default=3, choices=[2, 3, 5])
+    ap.add_argument("--points", type=int, default=None, help="override the point count (debug runs)")
+    ap.add_argument("--point-order", default="vet_preprocess", choices=["vet_preprocess", "generated"])
+    ap.add_argument("--no-second-order", action="store_true", help="skip timing the other point order")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-threads", type=int, default=0, help="0 = min(16, available cores)")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build runs the rasterizer on ONE GPU (views of a batch are rendered back to back); "
+              "--gpus N with N > 1 is not available", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    from vet_amd import synthetic
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU (there is no CPU path in the product)", file=sys.stderr)
+        sys.exit(2)
+
+    kw = {"point_order": args.point_order}
+    if args.points is not None:
+        kw["num_points"] = args.points
+    make = {2: synthetic.config2, 3: synthetic.config3, 5: synthetic.config5}[args.config]
+    backward = args.config != 2
+    scene = make(**kw)
+    r = run_scene(scene, backward, args.steps, args.warmup)
+    N, P, F, Fk, Cn, L, K = r["N"], r["P"], r["F"], r["Fk"], r["Cn"], r["L"], r["K"]
+    ms_step, ms_fwd = r["ms_step"], r["ms_fwd"]
 
     fwd_b, bwd_b = algorithmic_bytes(N, P, F, Fk, Cn)
     alg = dict(fwd_b)
     if backward:
         alg.update(bwd_b)
+    traffic = measured_traffic() if (args.config == 3 and args.points is None and args.point_order == "vet_preprocess") else {}
     kernels = {}
     for k, nbytes in alg.items():
-        t = per_step_ms.get(k, 0.0)
+        t = r["per_step_ms"].get(k, 0.0)
         kernels[k] = {"ms": round(t, 5), "alg_MB": round(nbytes / 1e6, 3),
-                      "GBps": round(nbytes / 1e6 / t, 1) if t > 0 else None}
-    kernels["PREPARE"] = {"ms": round(per_step_ms.get("PREPARE", 0.0), 5), "alg_MB": 0.0, "GBps": None}
-    dominant = max(alg.keys(), key=lambda k: per_step_ms.get(k, 0.0))
-    dom_ms = per_step_ms[dominant]
+                      "GBps": round(nbytes / 1e6 / t, 1) if t > 0 else None,
+                      "frac": round(nbytes / 1e6 / t / HBM_PEAK_GBS, 4) if t > 0 else None}
+        if k in traffic:
+            kernels[k]["hbm_traffic_MB"] = round(traffic[k] / 1e6, 1)
+    for k in ("PREPARE", "BACKWARD_PREPARE", "BACKWARD_POST"):
+        if r["per_step_ms"].get(k, 0.0) > 0:
+            kernels[k] = {"ms": round(r["per_step_ms"][k], 5), "alg_MB": 0.0, "GBps": None, "frac": None}
+    dominant = max(alg.keys(), key=lambda k: r["per_step_ms"].get(k, 0.0))
+    dom_ms = r["per_launch_ms"][dominant]
     achieved = alg[dominant] / 1e6 / dom_ms if dom_ms > 0 else 0.0
     total_alg = sum(alg.values())
 
@@ -169,8 +205,10 @@ def main():
         "data": "synthetic",
         "config": {
             "workload": f"BASELINE config {args.config} ({scene.name}): N={N} points, {scene.views[0].w}x{scene.views[0].h}, "
-                        f"L={L} layers, K={K}, C={Cn}, B=1 view, " + ("forward+backward" if backward else "forward"),
-            "fragments_per_layer": F_layers, "fragments": F, "fragments_kept": Fk, "pixels": P,
+                        f"L={L} layers, K={K}, C={Cn}, B=1 view, " + ("forward+backward" if backward else "forward")
+                        + f", point order {args.point_order}",
+            "point_order": args.point_order,
+            "fragments_per_layer": r["F_layers"], "fragments": F, "fragments_kept": Fk, "pixels": P,
         },
         "forward_ms": round(ms_fwd, 5),
         "backward_ms": round(ms_step - ms_fwd, 5) if backward else None,
@@ -184,12 +222,20 @@ def main():
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBS, 4),
-            "traffic": None,
-            "avg_launch_ms": round(per_launch_ms[dominant], 5),
+            "traffic": int(traffic[dominant]) if dominant in traffic else None,
+            "avg_launch_ms": round(dom_ms, 5),
             "algorithmic_bytes_per_launch": alg[dominant],
         },
         "kernels": kernels,
     }
+
+    if not args.no_second_order:
+        # VET hands the rasterizer Morton-ordered clouds with shuffled 256-point blocks; the generator's raw order
+        # (random inside each primitive) is timed as well so that the effect of that order is visible.
+        other = "generated" if args.point_order == "vet_preprocess" else "vet_preprocess"
+        r2 = run_scene(make(**dict(kw, point_order=other)), backward, max(10, args.steps // 2), 5, profile=False)
+        result["other_point_order"] = {"point_order": other, "ms_per_step": round(r2["ms_step"], 5),
+                                       "forward_ms": round(r2["ms_fwd"], 5)}
 
     if not args.no_cpu_baseline:
         from oracle import oracle_py
@@ -200,16 +246,16 @@ def main():
 
         def cpu_step(threads):
             t0 = time.perf_counter()
-            f = oracle_py.forward(scene, params, num_threads=threads)
+            f = oracle_py.forward(scene, r["params"], num_threads=threads)
             t1 = time.perf_counter()
             if backward:
                 oracle_py.backward(f, cpu_grad_out, num_threads=threads)
             t2 = time.perf_counter()
             return (t2 - t0) * 1e3, (t1 - t0) * 1e3
 
-        single_ms, single_fwd = cpu_step(1)
+        single_ms, _ = cpu_step(1)
         runs = [cpu_step(cores) for _ in range(3)]
-        multi_ms = float(np.median([r[0] for r in runs]))
+        multi_ms = float(np.median([x[0] for x in runs]))
         result["cpu_baseline"] = {
             "value": round(multi_ms, 2),
             "unit": "ms",
@@ -218,7 +264,7 @@ def main():
             "sample": f"the same frame (config {args.config}, all {N} points): CPU oracle, median of 3 runs on {cores} "
                       f"threads; one run on 1 thread = {single_ms:.1f} ms",
             "single_thread_ms": round(single_ms, 2),
-            "forward_ms": round(float(np.median([r[1] for r in runs])), 2),
+            "forward_ms": round(float(np.median([x[1] for x in runs])), 2),
         }
     print(json.dumps(result))
 

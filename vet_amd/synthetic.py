@@ -253,7 +253,7 @@ def _random_poses(seed, B, extent=4.0):
 
 
 def config4(surface_points_n=4_000_000, sphere_points=500_000, seed=3, w=1920, h=1080, num_views=4, num_layers=4,
-            K=16) -> Scene:
+            K=16, point_order="vet_preprocess") -> Scene:
     """Surface points plus three nested environment spheres (r = 50/100/200 m), a batch of random views."""
     prims = 400
     per = max(1, surface_points_n // prims)
@@ -264,6 +264,8 @@ def config4(surface_points_n=4_000_000, sphere_points=500_000, seed=3, w=1920, h
         d /= np.maximum(np.linalg.norm(d, axis=1, keepdims=True), 1e-12)
         shells.append(r * d)
     xyz = np.concatenate([surf] + shells, axis=0)
+    if point_order == "vet_preprocess":
+        xyz = xyz[vet_preprocess_order(xyz, seed)]
     N = xyz.shape[0]
     pos = np.empty((N, 4), dtype=np.float32)
     pos[:, :3] = xyz.astype(np.float32)
@@ -278,12 +280,14 @@ def config4(surface_points_n=4_000_000, sphere_points=500_000, seed=3, w=1920, h
     return s
 
 
-def config5(num_points=10_000_000, seed=4, w=1920, h=1080, num_layers=4, K=16) -> Scene:
+def config5(num_points=10_000_000, seed=4, w=1920, h=1080, num_layers=4, K=16, point_order="vet_preprocess") -> Scene:
     """Depth-complexity stress: a 1 m^3 cube of points filling the frustum."""
     N = num_points
     pos = np.empty((N, 4), dtype=np.float32)
     xyz = Stream(seed, "position").uniform(3 * N).reshape(N, 3) - 0.5
     xyz[:, 2] += 1.2
+    if point_order == "vet_preprocess":
+        xyz = xyz[vet_preprocess_order(xyz, seed)]
     pos[:, :3] = xyz.astype(np.float32)
     pos[:, 3] = 0.01
     tex, conf, bg = _descriptors(seed, N)
