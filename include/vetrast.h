@@ -114,6 +114,7 @@ typedef struct vetrast_workspace_layout
                                                 first min(count, K) entries of a pixel's list are sorted and meaningful */
     size_t transmittance_base, transmittance_stride; /* float [N*L]: transmittance in front of each kept fragment */
     size_t weight_base, weight_stride;       /* float [P]: final transmittance per pixel (the reference's `weight` image) */
+    size_t cut_flags_base, cut_flags_stride; /* uint8 [P]: 1 where the top-K cut dropped fragments of the pixel */
     /* shared by all views */
     size_t packed_base;    /* float [N][8]: descriptor (4, zero padded), confidence, 3 pad */
     size_t slots_base;     /* uint32 [L][N]: per (layer, point) arrival rank inside its pixel, 0xFFFFFFFF = no fragment */

@@ -64,6 +64,7 @@ class WorkspaceLayout(C.Structure):
         ("fragments_base", C.c_size_t), ("fragments_stride", C.c_size_t),
         ("transmittance_base", C.c_size_t), ("transmittance_stride", C.c_size_t),
         ("weight_base", C.c_size_t), ("weight_stride", C.c_size_t),
+        ("cut_flags_base", C.c_size_t), ("cut_flags_stride", C.c_size_t),
         ("packed_base", C.c_size_t),
         ("slots_base", C.c_size_t),
         ("views_base", C.c_size_t),

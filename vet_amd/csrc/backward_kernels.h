@@ -230,15 +230,34 @@ __global__ void __launch_bounds__(kBlock) reduce_background_kernel(const float* 
     float acc[kBackgroundRow];
 #pragma unroll
     for (int k = 0; k < kBackgroundRow; ++k) acc[k] = 0.f;
-    for (int r = threadIdx.x; r < num_rows; r += kBlock)
+    // eight independent row loads per thread and trip: one workgroup has to pull in ~10^4 rows and would otherwise sit
+    // on one memory round trip per row
+    constexpr int kUnroll = 8;
+    for (int r0 = threadIdx.x; r0 < num_rows; r0 += kBlock * kUnroll)
     {
-        const float4 a0 = reinterpret_cast<const float4*>(rows)[2 * (size_t)r];
-        const float4 a1 = reinterpret_cast<const float4*>(rows)[2 * (size_t)r + 1];
-        acc[0] += a0.x;
-        acc[1] += a0.y;
-        acc[2] += a0.z;
-        acc[3] += a0.w;
-        acc[4] += a1.x;
+        float4 a0[kUnroll];
+        float a1[kUnroll];
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u)
+        {
+            const int r = r0 + u * kBlock;
+            a0[u]       = make_float4(0.f, 0.f, 0.f, 0.f);
+            a1[u]       = 0.f;
+            if (r < num_rows)
+            {
+                a0[u] = reinterpret_cast<const float4*>(rows)[2 * (size_t)r];
+                a1[u] = rows[(size_t)r * kBackgroundRow + 4];
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u)
+        {
+            acc[0] += a0[u].x;
+            acc[1] += a0[u].y;
+            acc[2] += a0[u].z;
+            acc[3] += a0[u].w;
+            acc[4] += a1[u];
+        }
     }
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
 #pragma unroll
@@ -264,6 +283,7 @@ struct GatherPass
     ViewPass vp;
     const uint32_t* offsets;
     const uint64_t* fragments;
+    const uint8_t* list_is_cut;  // per pixel, written by the sort
     const float4* partial;
     float* grad_texture;      // [C,N]
     float* grad_confidence;   // [N]
@@ -306,9 +326,7 @@ __global__ void __launch_bounds__(kBlock) gather_point_gradients_kernel(GatherPa
             if (!(fx >= 0.f && fx < (float)ly.w[l] && fy >= 0.f && fy < (float)ly.h[l])) continue;
             const int x = (int)fx, y = (int)fy;
             const uint32_t q   = ly.base[l] + (uint32_t)y * (uint32_t)ly.w[l] + (uint32_t)x;
-            const uint32_t off = a.offsets[q];
-            const uint32_t n   = a.offsets[q + 1] - off;
-            if (a.K > 0 && n > (uint32_t)a.K && key > a.fragments[off + a.K - 1]) continue;  // cut away
+            if (a.K > 0 && a.list_is_cut[q] && key > a.fragments[a.offsets[q] + a.K - 1]) continue;  // cut away
             const float4 r0 = a.partial[2 * ((size_t)l * a.vp.N + i)];
             const float4 r1 = a.partial[2 * ((size_t)l * a.vp.N + i) + 1];
             const float r[4] = {r0.x, r0.y, r0.z, r0.w};

@@ -39,6 +39,12 @@ __global__ void prepare_views_kernel(PrepareViewsArgs args, int first_view, int 
                                      DeviceView* __restrict__ views, uint32_t* __restrict__ flags)
 {
     const int k = threadIdx.x;
+    if (first_view == 0)
+    {
+        // the device flag word starts every call at zero
+        if (k < 4) flags[k] = 0u;
+        __syncthreads();
+    }
     if (k >= num_views) return;
     const ViewSource& s = args.src[k];
     const double* q     = poses_se3 + 8 * (size_t)s.image_index;

@@ -200,7 +200,8 @@ struct SortWaveMap
 };
 
 __global__ void __launch_bounds__(kBlock) sort_lists_kernel(const uint32_t* __restrict__ offsets,
-                                                             uint64_t* __restrict__ fragments, SortWaveMap map, int K)
+                                                             uint64_t* __restrict__ fragments,
+                                                             uint8_t* __restrict__ list_is_cut, SortWaveMap map, int K)
 {
     __shared__ uint8_t src_lane_all[kBlock / kWave][kWave];
     const int lane    = threadIdx.x & (kWave - 1);
@@ -219,6 +220,9 @@ __global__ void __launch_bounds__(kBlock) sort_lists_kernel(const uint32_t* __re
         {
             off = offsets[q];
             n   = offsets[q + 1] - off;
+            // one byte per pixel: does the top-K cut drop fragments here? The backward per-point kernel only has to look
+            // up the K-th key of a pixel where this is set (a few percent of the pixels at the fine layers).
+            list_is_cut[q] = (K > 0 && n > (uint32_t)K) ? 1 : 0;
         }
     }
     // class = ceil(log2(n)) for 2 <= n <= 64, 0 for n <= 1 (nothing to do), 7 for n > 64

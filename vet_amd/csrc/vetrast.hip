@@ -308,6 +308,9 @@ int vetrast_workspace_layout_for(int32_t N, int32_t B, int32_t L, int32_t w, int
     lay->weight_base   = at;
     lay->weight_stride = align_up(P * sizeof(float), kAlign);
     at += lay->weight_stride * B;
+    lay->cut_flags_base   = at;
+    lay->cut_flags_stride = align_up(P, kAlign);
+    at += lay->cut_flags_stride * B;
     lay->fragments_base   = at;
     lay->fragments_stride = align_up(cap * sizeof(uint64_t), kAlign);
     at += lay->fragments_stride * B;
@@ -357,7 +360,6 @@ int vetrast_forward(vetrast_ctx* ctx, const vetrast_forward_args* a, void* strea
         const size_t n4 = Ppad * B / 4;
         hipLaunchKernelGGL(fill_u128_kernel, dim3(std::min(grid_for(n4), 4096)), dim3(kBlock), 0, stream,
                            ws_ptr<uint4>(ws, lay.offsets_base), n4, 0u);
-        hipLaunchKernelGGL(fill_u32_kernel, dim3(1), dim3(kWave), 0, stream, flags, (size_t)4, 0u);
         for (int first = 0; first < B; first += 16)
         {
             PrepareViewsArgs pv;
@@ -420,7 +422,9 @@ int vetrast_forward(vetrast_ctx* ctx, const vetrast_forward_args* a, void* strea
             ScopeTimer tm(ctx, stream, VETRAST_SCOPE_SORT);
             const SortWaveMap map = make_sort_wave_map(ly, N);
             hipLaunchKernelGGL(sort_lists_kernel, dim3((map.first_wave[L] + kBlock / kWave - 1) / (kBlock / kWave)),
-                               dim3(kBlock), 0, stream, offsets, fragments, map, p.debug_max_list_length);
+                               dim3(kBlock), 0, stream, offsets, fragments,
+                               ws_ptr<uint8_t>(ws, lay.cut_flags_base + lay.cut_flags_stride * b), map,
+                               p.debug_max_list_length);
         }
         {
             ScopeTimer tm(ctx, stream, VETRAST_SCOPE_BLEND);
@@ -556,6 +560,7 @@ int vetrast_backward(vetrast_ctx* ctx, const vetrast_backward_args* g, void* str
             gp.vp                  = make_view_pass(a, lay, ly, b);
             gp.offsets             = offsets;
             gp.fragments           = fragments;
+            gp.list_is_cut         = ws_ptr<uint8_t>(ws, lay.cut_flags_base + lay.cut_flags_stride * b);
             gp.partial             = partial;
             gp.grad_texture        = g->grad_texture;
             gp.grad_confidence     = g->grad_confidence;
