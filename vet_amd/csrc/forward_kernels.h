@@ -114,22 +114,65 @@ __device__ __forceinline__ bool point_is_skipped(const ViewPass& a, int i)
 // Project every point and count it in the pixel it rounds to, in every layer. The returning atomic hands each
 // (point, layer) its arrival rank inside the pixel, which the fill pass turns into a buffer position without a second
 // atomic. Counterpart of CountingPrepassMulti<L,false> (src/lib/rendering/RenderForward.cu:806-905).
+//
+// Global atomics are the scarce resource here (MI355X retires about 26 G of them per second whatever their scope,
+// return mode or address spread), and VET hands over clouds in Morton order with 256-point blocks
+// (src/lib/data/SceneData.cpp:105-106), so the 256 points of a workgroup fall into few pixels of the coarse layers.
+// The workgroup therefore first counts its (pixel, layer) hits in an LDS hash table (LDS atomics), then issues ONE
+// global atomic per distinct pixel for the whole group, and every point's rank is group base + rank inside the group.
+constexpr int kCountTableBits = 11;  // 2048 entries for at most 256 points x 5 layers: load factor <= 0.63
+constexpr int kCountTable     = 1 << kCountTableBits;
+constexpr uint32_t kEmptyKey  = 0xFFFFFFFFu;
+
 __global__ void __launch_bounds__(kBlock) count_kernel(ViewPass a, uint32_t* __restrict__ counts,
                                                         uint32_t* __restrict__ slots)
 {
-    const int i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (i >= a.N) return;
-    if (point_is_skipped(a, i)) return;
-    Projected p;
-    if (!project_point(*a.view, a.position[i], p)) return;
-    float ipx = p.ipx, ipy = p.ipy, radius = p.radius;
-    for (int l = 0; l < a.ly.L; ++l, radius *= 0.5f, ipx *= 0.5f, ipy *= 0.5f)
+    __shared__ uint32_t t_key[kCountTable];
+    __shared__ uint32_t t_val[kCountTable];  // hits of the group in the pixel, then the group's base rank
+    for (int e = threadIdx.x; e < kCountTable; e += kBlock)
     {
-        if (a.drop_by_radius && radius < a.radius_threshold) break;
-        const int64_t q = layer_pixel(a.ly, l, ipx, ipy);
-        if (q < 0) continue;
-        slots[(size_t)l * a.N + i] = atomicAdd(&counts[q], 1u);
+        t_key[e] = kEmptyKey;
+        t_val[e] = 0u;
     }
+    __syncthreads();
+
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    uint32_t entry[VETRAST_MAX_LAYERS], rank[VETRAST_MAX_LAYERS];
+#pragma unroll
+    for (int l = 0; l < VETRAST_MAX_LAYERS; ++l) entry[l] = kEmptyKey;
+    Projected p;
+    if (i < a.N && !point_is_skipped(a, i) && project_point(*a.view, a.position[i], p))
+    {
+        float ipx = p.ipx, ipy = p.ipy, radius = p.radius;
+#pragma unroll
+        for (int l = 0; l < VETRAST_MAX_LAYERS; ++l, radius *= 0.5f, ipx *= 0.5f, ipy *= 0.5f)
+        {
+            if (l >= a.ly.L) break;
+            if (a.drop_by_radius && radius < a.radius_threshold) break;
+            const int64_t q64 = layer_pixel(a.ly, l, ipx, ipy);
+            if (q64 < 0) continue;
+            const uint32_t q = (uint32_t)q64;
+            uint32_t h       = (q * 2654435761u) >> (32 - kCountTableBits);
+            while (true)  // linear probing; the table can never fill up
+            {
+                const uint32_t old = atomicCAS(&t_key[h], kEmptyKey, q);
+                if (old == kEmptyKey || old == q) break;
+                h = (h + 1) & (kCountTable - 1);
+            }
+            entry[l] = h;
+            rank[l]  = atomicAdd(&t_val[h], 1u);
+        }
+    }
+    __syncthreads();
+    for (int e = threadIdx.x; e < kCountTable; e += kBlock)
+    {
+        const uint32_t q = t_key[e];
+        if (q != kEmptyKey) t_val[e] = atomicAdd(&counts[q], t_val[e]);
+    }
+    __syncthreads();
+#pragma unroll
+    for (int l = 0; l < VETRAST_MAX_LAYERS; ++l)
+        if (entry[l] != kEmptyKey) slots[(size_t)l * a.N + i] = t_val[entry[l]] + rank[l];
 }
 
 // ---- exclusive scan of the per-pixel counts, in place, in two launches -------------------------------------------
