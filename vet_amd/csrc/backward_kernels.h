@@ -48,47 +48,65 @@ __device__ __forceinline__ bool interior_pixel(int x, int y, int w, int h)
     return min(min(x, y), min(w - 1 - x, h - 1 - y)) > 2;
 }
 
-// One thread per pixel, all layers of a view in one launch. The list is walked back to front with the transmittance
-// T_j the forward pass stored, so the reference's inner loop over all fragments in front
-// (src/lib/rendering/RenderBackward.cu:1160-1178, n(n-1)/2 atomics per pixel) becomes a running suffix sum:
+// Per-pixel part of the backward pass; all layers of a view in one launch. Counterpart of BlendBackwards2<C>
+// (src/lib/rendering/RenderBackward.cu:1083-1513).
+//
+// Arithmetic. With the transmittance T_j the forward pass stored, the reference's inner loop over all fragments in
+// front (src/lib/rendering/RenderBackward.cu:1160-1178, n(n-1)/2 atomics per pixel) is a suffix sum:
 //   S_j         = sum_{i>j} sum_ci g[ci] * t_i[ci] * T_i * c_i          (the background counts as the last fragment)
 //   d conf_j    = T_j * (t_j . g)  -  S_j / (1 - c_j + 1e-9)
 //   d tex_j[ci] = T_j * c_j * g[ci]
-// which is the same sum in a different order. Position gradient: the neighbour-difference heuristic of
-// src/lib/rendering/RenderBackward.cu:1346-1377 pushed through the pinhole chain of
-// src/lib/rendering/PointRendererHelper.h:317-372 (zero distortion), J_point = R.
-// Counterpart of BlendBackwards2<C> (src/lib/rendering/RenderBackward.cu:1083-1513).
+// i.e. the same terms added in a different order. The position term is the neighbour-difference heuristic of
+// src/lib/rendering/RenderBackward.cu:1346-1377, stored as an image-space gradient; the per-point kernel applies the
+// projection Jacobian.
+//
+// Work distribution. A wave owns 16x4 pixels, but at the fine layers most pixels hold no or one fragment while a few
+// hold several, so one-thread-per-pixel loops leave most lanes idle. Instead the wave lays the kept fragments of its
+// 64 pixels out as one dense item list (in windows of 16 fragments per pixel), and every lane processes one FRAGMENT:
+// per-pixel data (upstream gradient, neighbour samples) is staged in LDS, the suffix sum is a segmented scan over the
+// lanes of a pixel plus a per-pixel carry, rounds run from the deepest fragments to the nearest.
+constexpr int kWindow     = 16;                 // fragments per pixel in one window
+constexpr int kWaveItems  = kWave * kWindow;    // item table of a wave
+
 template <int C>
 __global__ void __launch_bounds__(kBlock) blend_backward_kernel(BackwardPass a)
 {
+    constexpr int kWaves = kBlock / kWave;
+    __shared__ uint32_t s_off[kWaves][kWave];
+    __shared__ uint32_t s_base[kWaves][kWave];
+    __shared__ float s_carry[kWaves][kWave];
+    __shared__ float4 s_g[kWaves][kWave];
+    __shared__ float4 s_nb[kWaves][kWave][8];  // I(x-1), I(x+1), I(y-1), I(y+1), G(x-1), G(x+1), G(y-1), G(y+1)
+    __shared__ uint8_t s_point[kWaves][kWave];
+    __shared__ uint8_t s_item[kWaves][kWaveItems];
+    __shared__ float red[kWaves][C + 1];
+
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
     const TilePixel px = tile_pixel(a.tiles, a.ly);
-    const uint32_t q   = px.q;
-    const bool active  = px.active;
+    const int l        = px.l;
     float bg_grad[C];
 #pragma unroll
     for (int ci = 0; ci < C; ++ci) bg_grad[ci] = 0.f;
     float leak = 0.f;
+    uint32_t off = 0, n = 0;
 
-    if (active)
+    if (px.active)
     {
-        const int l          = px.l;
         const int lw = a.ly.w[l], lh = a.ly.h[l];
         const size_t plane   = (size_t)lw * lh;
         const uint32_t local = px.local;
-        const int gy = px.y, gx = px.x;
-        const float* G = a.grad_out[l];
-        float g[C];
+        const float* G       = a.grad_out[l];
+        float g[4]           = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int ci = 0; ci < C; ++ci) g[ci] = G[ci * plane + local];
-
-        const uint32_t off = a.offsets[q];
-        uint32_t n         = a.offsets[q + 1] - off;
+        off = a.offsets[px.q];
+        n   = a.offsets[px.q + 1] - off;
         if (a.K > 0) n = min(n, (uint32_t)a.K);
 
         float S = 0.f;
         if (!a.use_environment_map)
         {
-            const float Tn = a.weight[q];
+            const float Tn = a.weight[px.q];
             float dot      = 0.f;
 #pragma unroll
             for (int ci = 0; ci < C; ++ci)
@@ -100,108 +118,152 @@ __global__ void __launch_bounds__(kBlock) blend_backward_kernel(BackwardPass a)
             }
             if (a.quirk_background_confidence_leak) leak = dot * Tn;
         }
-
-        // neighbour samples for the position heuristic, shared by every fragment of the pixel
-        const bool do_point = a.need_point_gradient && n > 0 && interior_pixel(gx, gy, lw, lh);
-        float Ix0[C], Ix1[C], Iy0[C], Iy1[C], Gx0[C], Gx1[C], Gy0[C], Gy1[C];
+        const bool do_point = a.need_point_gradient && n > 0 && interior_pixel(px.x, px.y, lw, lh);
+        s_off[wave][lane]   = off;
+        s_carry[wave][lane] = S;
+        s_g[wave][lane]     = make_float4(g[0], g[1], g[2], g[3]);
+        s_point[wave][lane] = do_point ? 1 : 0;
         if (do_point)
         {
             const float* I = a.out[l];
+            float nb[8][4];
+#pragma unroll
+            for (int k = 0; k < 8; ++k)
+#pragma unroll
+                for (int ci = 0; ci < 4; ++ci) nb[k][ci] = 0.f;
 #pragma unroll
             for (int ci = 0; ci < C; ++ci)
             {
                 const float* Ic = I + ci * plane + local;
                 const float* Gc = G + ci * plane + local;
-                Ix0[ci] = Ic[-1];
-                Ix1[ci] = Ic[1];
-                Iy0[ci] = Ic[-lw];
-                Iy1[ci] = Ic[lw];
-                Gx0[ci] = Gc[-1];
-                Gx1[ci] = Gc[1];
-                Gy0[ci] = Gc[-lw];
-                Gy1[ci] = Gc[lw];
+                nb[0][ci] = Ic[-1];
+                nb[1][ci] = Ic[1];
+                nb[2][ci] = Ic[-lw];
+                nb[3][ci] = Ic[lw];
+                nb[4][ci] = Gc[-1];
+                nb[5][ci] = Gc[1];
+                nb[6][ci] = Gc[-lw];
+                nb[7][ci] = Gc[lw];
             }
+#pragma unroll
+            for (int k = 0; k < 8; ++k) s_nb[wave][lane][k] = make_float4(nb[k][0], nb[k][1], nb[k][2], nb[k][3]);
         }
+    }
 
-        const uint64_t* list = a.fragments + off;
-        const float* Tlist   = a.transmittance + off;
-        float4* partial_l    = a.partial + 2 * (size_t)l * a.N;
-        // Back to front in chunks of kBlendChunk fragments; all loads of a chunk (key, stored transmittance, descriptor
-        // record, position) are issued before its arithmetic, so a thread keeps several gathers in flight.
-        for (int top = (int)n - 1; top >= 0; top -= kBlendChunk)
+    // ---- fragments: windows of kWindow per pixel, deepest window first ------------------------------------------
+    uint32_t max_n = n;
+#pragma unroll
+    for (int d = kWave / 2; d >= 1; d >>= 1) max_n = max(max_n, (uint32_t)__shfl_xor((int)max_n, d, kWave));
+    float4* partial_l = a.partial + 2 * (size_t)l * a.N;
+    for (int jw = max_n == 0 ? -1 : (int)((max_n - 1) / kWindow) * kWindow; jw >= 0; jw -= kWindow)
+    {
+        const uint32_t nw = (n > (uint32_t)jw) ? min(n - (uint32_t)jw, (uint32_t)kWindow) : 0u;
+        uint32_t incl     = nw;
+#pragma unroll
+        for (int d = 1; d < kWave; d <<= 1)
         {
-            int id[kBlendChunk], ti[kBlendChunk];
-            float T[kBlendChunk], c[kBlendChunk];
-            float4 t4[kBlendChunk];
-#pragma unroll
-            for (int u = 0; u < kBlendChunk; ++u)
+            const uint32_t o = __shfl_up(incl, d, kWave);
+            if (lane >= d) incl += o;
+        }
+        const uint32_t base  = incl - nw;
+        const uint32_t total = __shfl(incl, kWave - 1, kWave);
+        s_base[wave][lane]   = base;
+        for (uint32_t j = 0; j < nw; ++j) s_item[wave][base + j] = (uint8_t)lane;
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+
+        for (int k0 = (int)((total - 1) / kWave) * kWave; total > 0 && k0 >= 0; k0 -= kWave)
+        {
+            const uint32_t k = (uint32_t)k0 + lane;
+            const bool valid = k < total;
+            const int p      = valid ? (int)s_item[wave][k] : -1;  // lane of the pixel this fragment belongs to
+            float x = 0.f, T = 0.f, c = 0.f, dot = 0.f;
+            float t[4] = {0.f, 0.f, 0.f, 0.f};
+            float4 g4  = make_float4(0.f, 0.f, 0.f, 0.f);
+            int id = -1, ti = -1;
+            if (valid)
             {
-                const int j = top - u;
-                id[u] = ti[u] = -1;
-                if (j >= 0)
-                {
-                    id[u] = (int)(uint32_t)list[j];
-                    T[u]  = Tlist[j];
-                    // guards the gathers; never false for a workspace the forward pass wrote
-                    if ((uint32_t)id[u] < (uint32_t)a.N) ti[u] = a.index ? a.index[id[u]] : id[u];
-                    if ((uint32_t)ti[u] >= (uint32_t)a.N) ti[u] = -1;
-                }
+                const uint32_t pos = s_off[wave][p] + (uint32_t)jw + (k - s_base[wave][p]);
+                id                 = (int)(uint32_t)a.fragments[pos];
+                T                  = a.transmittance[pos];
+                // guards the gathers; never false for a workspace the forward pass wrote
+                if ((uint32_t)id < (uint32_t)a.N) ti = a.index ? a.index[id] : id;
+                if ((uint32_t)ti >= (uint32_t)a.N) ti = -1;
+                g4 = s_g[wave][p];
             }
-#pragma unroll
-            for (int u = 0; u < kBlendChunk; ++u)
+            if (ti >= 0)
             {
-                if (ti[u] >= 0)
-                {
-                    t4[u] = a.packed[2 * (size_t)ti[u]];
-                    c[u]  = a.packed[2 * (size_t)ti[u] + 1].x;
-                }
-            }
-#pragma unroll
-            for (int u = 0; u < kBlendChunk; ++u)
-            {
-                if (ti[u] < 0) continue;
-                const float t[4] = {t4[u].x, t4[u].y, t4[u].z, t4[u].w};
-                float dot = 0.f, x = 0.f;
-                const float Tc = T[u] * c[u];
-                float gt[4]    = {0.f, 0.f, 0.f, 0.f};
+                const float4 t4 = a.packed[2 * (size_t)ti];
+                c               = a.packed[2 * (size_t)ti + 1].x;
+                t[0] = t4.x, t[1] = t4.y, t[2] = t4.z, t[3] = t4.w;
+                const float g[4] = {g4.x, g4.y, g4.z, g4.w};
 #pragma unroll
                 for (int ci = 0; ci < C; ++ci)
                 {
-                    gt[ci] = Tc * g[ci];
                     dot += t[ci] * g[ci];
-                    x += ((g[ci] * t[ci]) * T[u]) * c[u];
+                    x += ((g[ci] * t[ci]) * T) * c;
                 }
-                const float gconf = dot * T[u] - S / ((1.f - c[u]) + 1e-9f);
-                S += x;
-
+            }
+            // suffix sum over the fragments of the same pixel that sit in higher lanes of this round
+            float v = x;
+#pragma unroll
+            for (int d = 1; d < kWave; d <<= 1)
+            {
+                const float o = __shfl_down(v, d, kWave);
+                const int po  = __shfl_down(p, d, kWave);
+                if (lane + d < kWave && po == p) v += o;
+            }
+            const float vn = __shfl_down(v, 1, kWave);
+            const int pn   = __shfl_down(p, 1, kWave);
+            const int pp   = __shfl_up(p, 1, kWave);
+            float S        = (lane + 1 < kWave && pn == p) ? vn : 0.f;  // deeper fragments of this round
+            if (valid) S += s_carry[wave][p];                            // and of the rounds / windows before
+            if (valid && (lane == 0 || pp != p)) s_carry[wave][p] += v;  // one lane per pixel moves the carry on
+            if (ti >= 0)
+            {
+                const float g[4]  = {g4.x, g4.y, g4.z, g4.w};
+                const float Tc    = T * c;
+                const float gconf = dot * T - S / ((1.f - c) + 1e-9f);
                 float gp0 = 0.f, gp1 = 0.f;
-                if (do_point)
+                if (s_point[wave][p])
                 {
+                    float nb[8][4];
+#pragma unroll
+                    for (int q8 = 0; q8 < 8; ++q8)
+                    {
+                        const float4 w4 = s_nb[wave][p][q8];
+                        nb[q8][0] = w4.x, nb[q8][1] = w4.y, nb[q8][2] = w4.z, nb[q8][3] = w4.w;
+                    }
                     float dR_dpx = 0.f, dR_dpy = 0.f;
 #pragma unroll
                     for (int ci = 0; ci < C; ++ci)
                     {
-                        const float d_x0 = -(t[ci] - Ix0[ci]) * Gx0[ci];
-                        const float d_x1 = (t[ci] - Ix1[ci]) * Gx1[ci];
-                        const float d_y0 = -(t[ci] - Iy0[ci]) * Gy0[ci];
-                        const float d_y1 = (t[ci] - Iy1[ci]) * Gy1[ci];
+                        const float d_x0 = -(t[ci] - nb[0][ci]) * nb[4][ci];
+                        const float d_x1 = (t[ci] - nb[1][ci]) * nb[5][ci];
+                        const float d_y0 = -(t[ci] - nb[2][ci]) * nb[6][ci];
+                        const float d_y1 = (t[ci] - nb[3][ci]) * nb[7][ci];
                         dR_dpx += 0.5f * (d_x0 + d_x1);
                         dR_dpy += 0.5f * (d_y0 + d_y1);
                     }
                     gp0 = dR_dpx / (float)C;  // image-space gradient of this fragment at the layer's resolution;
                     gp1 = dR_dpy / (float)C;  // the per-point kernel pushes it through the projection Jacobian
                 }
-                partial_l[2 * (size_t)id[u]]     = make_float4(gt[0], gt[1], gt[2], gt[3]);
-                partial_l[2 * (size_t)id[u] + 1] = make_float4(gconf, gp0, gp1, 0.f);
+                float gt[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int ci = 0; ci < C; ++ci) gt[ci] = Tc * g[ci];
+                partial_l[2 * (size_t)id]     = make_float4(gt[0], gt[1], gt[2], gt[3]);
+                partial_l[2 * (size_t)id + 1] = make_float4(gconf, gp0, gp1, 0.f);
             }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
         }
     }
 
     // Every pixel adds to the same C background values. Atomics on one address serialise (the reference issues one per
     // pixel and channel, src/lib/rendering/RenderBackward.cu:1150-1152), so each workgroup reduces its 256 pixels and
     // stores one row of partial sums; reduce_background_kernel adds the rows up.
-    __shared__ float red[kBlock / kWave][C + 1];
-    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
 #pragma unroll
     for (int ci = 0; ci < C; ++ci)
     {
