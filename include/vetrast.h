@@ -78,6 +78,11 @@ typedef struct vetrast_params
     int32_t point_gradient_normalization;     /* 0: leave sums and counts; 1: row i / count i;
                                                  2: literal reference (vec3 stride over the [N,4] buffer,
                                                  src/lib/rendering/PointRenderer.cu:1278-1279) */
+    /* Pose / intrinsics gradients (only computed when the matching buffers of vetrast_backward_args are given): */
+    float K_gradient_factor;                  /* RenderParams::K_gradient_factor, src/lib/data/Settings.h:55 */
+    int32_t camera_gradient_normalization;    /* 0: leave sums and counts; 1: divide each pose / intrinsics row by its
+                                                 count as src/lib/rendering/PointRenderer.cu:1253-1308 does (the count
+                                                 grows by 1/1024 per fragment, so this is 1024 x the mean) */
 } vetrast_params;
 
 typedef struct vetrast_ctx vetrast_ctx;
@@ -123,7 +128,8 @@ typedef struct vetrast_workspace_layout
     size_t flags_base;     /* uint32 [4] device status flags */
     size_t forward_only_bytes; /* a forward call with save_for_backward = 0 needs only this much */
     size_t partial_base;   /* float [L][N][8]: backward scratch, gradient record of the fragment of point i in layer l */
-    size_t background_partial_base; /* float [ceil(P/256)][8]: backward scratch, per-workgroup background-gradient sums */
+    size_t background_partial_base; /* float [workgroups][8]: backward scratch, per-workgroup background-gradient sums */
+    size_t camera_partial_base;     /* double [ceil(N/256)][12]: backward scratch, per-workgroup pose / intrinsics sums */
 } vetrast_workspace_layout;
 
 /* Arguments of the forward pass. Replaces the inputs PointRender::forward receives
@@ -165,6 +171,14 @@ typedef struct vetrast_backward_args
     float* grad_background;  /* device [C]; overwritten */
     float* grad_points;      /* device [N,4] or NULL (points do not require grad); xyz sums (w stays 0); overwritten */
     float* grad_point_count; /* device [N]; number of fragments that contributed to a point; required with grad_points */
+    /* Optional camera gradients, accumulated over every fragment that gets a position gradient
+     * (src/lib/rendering/RenderBackward.cu:1418-1459). NULL = not wanted. */
+    double* grad_pose;           /* device [F,6]: d/d(se3 tangent: translation, rotation) of pose row image_index; overwritten */
+    float* grad_pose_count;      /* device [F]: fragments / 1024 per pose row; required with grad_pose */
+    float* grad_intrinsics;      /* device [num_cameras,13]: fx,fy,cx,cy scaled by K_gradient_factor; the skew column is
+                                    zeroed as in the reference, and the 8 distortion columns stay 0 (their Jacobian is in
+                                    saiga, which is not available); overwritten */
+    float* grad_intrinsics_count; /* device [num_cameras]: fragments / 1024 per camera row; required with grad_intrinsics */
 } vetrast_backward_args;
 
 /* Create / destroy a context bound to the current HIP device. The context owns only a few HIP events. */

@@ -93,7 +93,7 @@ def forward(scene: Scene, params: abi.Params = None, num_threads=1, **overrides)
     return res
 
 
-def backward(fwd: OracleForward, grad_out, want_points=True, num_threads=1, **param_overrides):
+def backward(fwd: OracleForward, grad_out, want_points=True, want_cameras=False, num_threads=1, **param_overrides):
     scene = fwd.scene
     N, Cn = scene.num_points, scene.num_channels
     g = abi.BackwardArgs()
@@ -116,6 +116,16 @@ def backward(fwd: OracleForward, grad_out, want_points=True, num_threads=1, **pa
         res["point_count"] = np.zeros((N,), np.float32)
         g.grad_points = _addr(res["points"])
         g.grad_point_count = _addr(res["point_count"])
+    if want_cameras:
+        F, ncam = int(scene.poses_se3.shape[0]), int(scene.intrinsics.shape[0])
+        res["pose"] = np.zeros((F, 6), np.float64)
+        res["pose_count"] = np.zeros((F,), np.float32)
+        res["intrinsics"] = np.zeros((ncam, 13), np.float32)
+        res["intrinsics_count"] = np.zeros((ncam,), np.float32)
+        g.grad_pose = _addr(res["pose"])
+        g.grad_pose_count = _addr(res["pose_count"])
+        g.grad_intrinsics = _addr(res["intrinsics"])
+        g.grad_intrinsics_count = _addr(res["intrinsics_count"])
     st = load().vetref_backward(C.byref(g), _addr(fwd.offsets), _addr(fwd.fragments), num_threads)
     if st != 0:
         raise abi.VetrastError(st, "oracle backward")

@@ -394,6 +394,8 @@ extern "C" int vetref_backward(const vetrast_backward_args* g, const uint32_t* o
     if (st != VETRAST_OK) return st;
     if (!g->grad_texture || !g->grad_confidence || !g->grad_background) return VETRAST_ERR_INVALID_ARG;
     if (g->grad_points && !g->grad_point_count) return VETRAST_ERR_INVALID_ARG;
+    if (g->grad_pose && !g->grad_pose_count) return VETRAST_ERR_INVALID_ARG;
+    if (g->grad_intrinsics && !g->grad_intrinsics_count) return VETRAST_ERR_INVALID_ARG;
     Scene s                  = make_scene(a);
     const int N              = a->num_points;
     const int C              = a->params.num_texture_channels;
@@ -403,6 +405,16 @@ extern "C" int vetref_backward(const vetrast_backward_args* g, const uint32_t* o
 #ifdef _OPENMP
     omp_set_num_threads(num_threads > 0 ? num_threads : 1);
 #endif
+    if (g->grad_pose)
+    {
+        std::fill(g->grad_pose, g->grad_pose + (size_t)6 * a->num_poses, 0.0);
+        std::fill(g->grad_pose_count, g->grad_pose_count + a->num_poses, 0.f);
+    }
+    if (g->grad_intrinsics)
+    {
+        std::fill(g->grad_intrinsics, g->grad_intrinsics + (size_t)13 * a->num_cameras, 0.f);
+        std::fill(g->grad_intrinsics_count, g->grad_intrinsics_count + a->num_cameras, 0.f);
+    }
     // zeros_like of every gradient tensor, rendering/PointRenderer.cu:267-277
     std::fill(g->grad_texture, g->grad_texture + (size_t)C * N, 0.f);
     std::fill(g->grad_confidence, g->grad_confidence + N, 0.f);
@@ -412,7 +424,7 @@ extern "C" int vetref_backward(const vetrast_backward_args* g, const uint32_t* o
         std::fill(g->grad_points, g->grad_points + (size_t)4 * N, 0.f);
         std::fill(g->grad_point_count, g->grad_point_count + N, 0.f);
     }
-    const bool need_point_gradients = pr.need_point_gradient && g->grad_points;
+    const bool need_point_gradients = pr.need_point_gradient && (g->grad_points || g->grad_pose || g->grad_intrinsics);
 
     for (int b = 0; b < a->num_views; ++b)
     {
@@ -526,6 +538,8 @@ extern "C" int vetref_backward(const vetrast_backward_args* g, const uint32_t* o
                         const float vy = ((cam.r[3] * px + cam.r[4] * py) + cam.r[5] * pz) + cam.t[1];
                         const float vz = ((cam.r[6] * px + cam.r[7] * py) + cam.r[8] * pz) + cam.t[2];
                         float gp[3] = {0.f, 0.f, 0.f};
+                        double gpose[6] = {0, 0, 0, 0, 0, 0};
+                        float gk[5]     = {0.f, 0.f, 0.f, 0.f, 0.f};
                         if (vz > 0.f)
                         {
                             const float ar = v.crop_rotation[0] * gxp + v.crop_rotation[2] * gyp;  // J_rot^T grad
@@ -540,12 +554,74 @@ extern "C" int vetref_backward(const vetrast_backward_args* g, const uint32_t* o
                             gp[0]          = (cam.r[0] * e0 + cam.r[3] * e1) + cam.r[6] * e2;  // R^T
                             gp[1]          = (cam.r[1] * e0 + cam.r[4] * e1) + cam.r[7] * e2;
                             gp[2]          = (cam.r[2] * e0 + cam.r[5] * e1) + cam.r[8] * e2;
+                            // J_pose^T e with J_pose = [I | -[view_p]x]: the tangent (translation, rotation) acts on
+                            // the left, pose <- exp(tangent) * pose (ApplyTangent, rendering/PointRenderer.cu:1325-1341)
+                            gpose[0] = e0;
+                            gpose[1] = e1;
+                            gpose[2] = e2;
+                            gpose[3] = vy * e2 - vz * e1;  // view_p x e
+                            gpose[4] = vz * e0 - vx * e2;
+                            gpose[5] = vx * e1 - vy * e0;
+                            // J_k_K1^T grad_p_k2: image = (fx*nx + s*ny + cx, fy*ny + cy), columns fx, fy, cx, cy, s
+                            const float nx = vx / vz, ny = vy / vz;
+                            gk[0] = nx * a2;
+                            gk[1] = ny * b2;
+                            gk[2] = a2;
+                            gk[3] = b2;
+                            gk[4] = ny * a2;
                         }
-                        for (int k = 0; k < 3; ++k) atomic_add(&g->grad_points[4 * (size_t)point_id + k], gp[k], par);
-                        atomic_add(&g->grad_point_count[point_id], 1.f, par);  // RenderBackward.cu:1407
+                        if (g->grad_points)
+                        {
+                            for (int k = 0; k < 3; ++k)
+                                atomic_add(&g->grad_points[4 * (size_t)point_id + k], gp[k], par);
+                            atomic_add(&g->grad_point_count[point_id], 1.f, par);  // RenderBackward.cu:1407
+                        }
+                        if (g->grad_pose)  // RenderBackward.cu:1418-1426
+                        {
+                            for (int k = 0; k < 6; ++k)
+                            {
+                                double* dst = &g->grad_pose[6 * (size_t)v.image_index + k];
+                                if (par)
+                                {
+#pragma omp atomic
+                                    *dst += gpose[k];
+                                }
+                                else
+                                    *dst += gpose[k];
+                            }
+                            atomic_add(&g->grad_pose_count[v.image_index], 1.f / 1024.f, par);
+                        }
+                        if (g->grad_intrinsics)  // RenderBackward.cu:1428-1459; g_k(4) *= 0 removes the skew
+                        {
+                            gk[4] *= 0;
+                            for (int k = 0; k < 5; ++k)
+                                atomic_add(&g->grad_intrinsics[13 * (size_t)v.camera_index + k],
+                                           pr.K_gradient_factor * gk[k], par);
+                            // the eight distortion columns need saiga's distortion Jacobian: left at zero
+                            atomic_add(&g->grad_intrinsics_count[v.camera_index], 1.f / 1024.f, par);
+                        }
                     }
                 }
         }
+    }
+
+    // NormalizeGradientDevTensor<double,6> and NormalizeGradient<float,13>, rendering/PointRenderer.cu:1253-1308
+    if (pr.camera_gradient_normalization)
+    {
+        if (g->grad_pose)
+            for (int i = 0; i < a->num_poses; ++i)
+            {
+                const float c = g->grad_pose_count[i];
+                if (c > 0)
+                    for (int k = 0; k < 6; ++k) g->grad_pose[6 * (size_t)i + k] /= c;
+            }
+        if (g->grad_intrinsics)
+            for (int i = 0; i < a->num_cameras; ++i)
+            {
+                const float c = g->grad_intrinsics_count[i];
+                if (c > 0)
+                    for (int k = 0; k < 13; ++k) g->grad_intrinsics[13 * (size_t)i + k] /= c;
+            }
     }
 
     // NormalizeGradient<float,3>, rendering/PointRenderer.cu:1072-1090,1273-1280

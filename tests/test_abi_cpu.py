@@ -30,7 +30,7 @@ def test_library_exports_every_declared_symbol():
 def test_struct_sizes_are_the_c_ones():
     # sizes the C compiler gives the structs of include/vetrast.h (LP64)
     assert C.sizeof(abi.View) == 5 * 4 + 9 * 4
-    assert C.sizeof(abi.Params) == 14 * 4
+    assert C.sizeof(abi.Params) == 16 * 4
     assert C.sizeof(abi.ForwardArgs) % 8 == 0
     assert abi.BackwardArgs.grad_out.offset == C.sizeof(abi.ForwardArgs)
 
@@ -65,6 +65,7 @@ def test_workspace_layout_is_aligned_and_disjoint():
         ("views", lay.views_base, B * 128),
         ("partial", lay.partial_base, N * L * 32),
         ("background_partial", lay.background_partial_base, (P + 255) // 256 * 32),
+        ("camera_partial", lay.camera_partial_base, (N + 255) // 256 * 96),
     ]
     assert lay.offsets_stride >= (P + 1) * 4 and lay.fragments_stride >= N * L * 8
     for name, base, size in regions:

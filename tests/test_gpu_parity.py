@@ -141,3 +141,34 @@ def test_backward_is_reproducible(rasterizer):
         runs.append({k: v.cpu().numpy() for k, v in g.items() if k != "_args"})
     for key in ("texture", "confidence", "points", "point_count"):
         np.testing.assert_array_equal(runs[0][key], runs[1][key])
+
+
+@pytest.mark.parametrize("normalize", [0, 1])
+def test_pose_and_intrinsics_gradients(normalize, rasterizer, oracle):
+    """Camera gradients: per-workgroup sums in double on the GPU against the oracle's per-fragment accumulation."""
+    scene = synthetic.tiny_scene(num_points=6000, K=8, seed=41, num_views=3)
+    scene.views[2].image_index = 0  # two views share a pose row: their sums add up
+    over = {"need_point_gradient": 1, "camera_gradient_normalization": normalize}
+    ref, dev, res, _ = _check_forward(scene, over, rasterizer, oracle)
+    grad_out = scene.grad_out()
+    want = oracle.backward(ref, grad_out, want_cameras=True)
+    got = rasterizer.backward(res, [torch.from_numpy(g).cuda() for g in grad_out], want_cameras=True)
+    torch.cuda.synchronize()
+    np.testing.assert_allclose(got["pose_count"].cpu().numpy(), want["pose_count"], rtol=1e-6)
+    np.testing.assert_allclose(got["intrinsics_count"].cpu().numpy(), want["intrinsics_count"], rtol=1e-6)
+    assert want["pose_count"][0] > want["pose_count"][1] > 0 and want["pose_count"][2] == 0
+    for key in ("pose", "intrinsics", "points", "texture"):
+        err = max_rel_err(got[key].cpu().numpy(), want[key])
+        print(f"  {key}: max rel err {err:.3e}", flush=True)
+        assert err <= GRAD_TOL, key
+
+
+def test_camera_gradients_without_point_gradient_buffer(rasterizer, oracle):
+    scene = synthetic.tiny_scene(num_points=3000, K=8, seed=42)
+    ref, dev, res, _ = _check_forward(scene, {"need_point_gradient": 1}, rasterizer, oracle)
+    grad_out = scene.grad_out()
+    want = oracle.backward(ref, grad_out, want_points=False, want_cameras=True)
+    got = rasterizer.backward(res, [torch.from_numpy(g).cuda() for g in grad_out], want_points=False, want_cameras=True)
+    torch.cuda.synchronize()
+    assert max_rel_err(got["pose"].cpu().numpy(), want["pose"]) <= GRAD_TOL
+    assert max_rel_err(got["intrinsics"].cpu().numpy(), want["intrinsics"]) <= GRAD_TOL

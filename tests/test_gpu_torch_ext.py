@@ -25,11 +25,12 @@ def test_autograd_matches_oracle(literal, oracle):
 
     scene = synthetic.tiny_scene(num_points=5000, K=8, seed=31, num_views=2)
     quirks = dict(quirk_background_confidence_leak=1 if literal else 0,
-                  point_gradient_normalization=2 if literal else 0)
+                  point_gradient_normalization=2 if literal else 0,
+                  camera_gradient_normalization=1 if literal else 0)
     params = make_params(scene, need_point_gradient=1, **quirks)
     ref = oracle.forward(scene, params)
     grad_out = scene.grad_out()
-    ref_g = oracle.backward(ref, grad_out)
+    ref_g = oracle.backward(ref, grad_out, want_cameras=True)
 
     cu = lambda a, rg=False: torch.from_numpy(np.ascontiguousarray(a)).cuda().requires_grad_(rg)
     texture, background = cu(scene.texture, True), cu(scene.background, True)
@@ -51,7 +52,11 @@ def test_autograd_matches_oracle(literal, oracle):
     assert max_rel_err(confidence.grad.cpu().numpy().reshape(-1), ref_g["confidence"]) <= 1e-4
     assert max_rel_err(background.grad.cpu().numpy(), ref_g["background"]) <= 1e-4
     assert max_rel_err(points.grad.cpu().numpy(), ref_g["points"]) <= 1e-4
-    assert tangents.grad is None and intrinsics.grad is None  # not computed on this path
+    # pose tangents [F,6] float64 and intrinsics [Ncam,13]: fx, fy, cx, cy columns (skew and distortion stay zero)
+    assert tangents.grad.dtype == torch.float64
+    assert max_rel_err(tangents.grad.cpu().numpy(), ref_g["pose"]) <= 1e-4
+    assert max_rel_err(intrinsics.grad.cpu().numpy(), ref_g["intrinsics"]) <= 1e-4
+    assert np.all(intrinsics.grad.cpu().numpy()[:, 4:] == 0)
 
 
 def test_no_grad_call_and_masks(oracle):

@@ -446,3 +446,85 @@ def test_threaded_oracle_agrees_with_single_thread(oracle):
     gb = oracle.backward(b, go, num_threads=4, need_point_gradient=1)
     for k in ("texture", "confidence", "points"):
         np.testing.assert_allclose(ga[k], gb[k], rtol=1e-4, atol=1e-5 * np.abs(ga[k]).max())
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+# pose and intrinsics gradients
+# ---------------------------------------------------------------------------------------------------------------------
+def project64_camera(p, R, t, K5, crop5, rot4, w, h):
+    v = R @ np.asarray(p[:3], dtype=np.float64) + t
+    n = v[:2] / v[2]
+    u = K5[0] * n[0] + K5[4] * n[1] + K5[2]
+    vv = K5[1] * n[1] + K5[3]
+    x = crop5[0] * u + crop5[4] * vv + crop5[2]
+    y = crop5[1] * vv + crop5[3]
+    c = np.array([w // 2, h // 2], dtype=np.float64)
+    M = np.array([[rot4[0], rot4[1]], [rot4[2], rot4[3]]], dtype=np.float64)
+    return M @ (np.array([x, y]) - c) + c
+
+
+def test_pose_and_intrinsics_gradients(oracle):
+    """Camera gradients = sum over fragments of J^T dR/dp, with J the finite-difference Jacobian of the float64
+    projection with respect to (a) the se3 tangent applied on the left, pose <- exp(tangent) * pose, as ApplyTangent does
+    (src/lib/rendering/PointRenderer.cu:1325-1341), order (translation, rotation), and (b) fx, fy, cx, cy (skew zeroed,
+    scaled by K_gradient_factor). Counts grow by 1/1024 per fragment."""
+    scene = synthetic.tiny_scene(num_points=500, w=24, h=16, num_layers=2, K=3, seed=19)
+    ang = -0.15
+    scene.views[0].crop_transform = (1.05, 0.95, 0.5, 1.0, 0.02)
+    scene.views[0].crop_rotation = (np.cos(ang), -np.sin(ang), np.sin(ang), np.cos(ang))
+    scene.intrinsics[0, 4] = 0.2
+    q = np.array([0.03, 0.04, -0.02, 1.0])
+    scene.poses_se3[0, :4] = q / np.linalg.norm(q)
+    params = make_params(scene, need_point_gradient=1, K_gradient_factor=0.5)
+    f = oracle.forward(scene, params)
+    go = scene.grad_out()
+    g = oracle.backward(f, go, want_cameras=True)
+    lists = lists_of(f)
+    tex = scene.texture.astype(np.float64)
+    v = scene.views[0]
+    crop32 = np.array(v.crop_transform, np.float32).astype(np.float64)
+    rot32 = np.array(v.crop_rotation, np.float32).astype(np.float64)
+    K5 = scene.intrinsics[0, :5].astype(np.float64)
+    R0 = Rotation.from_quat(scene.poses_se3[0, :4]).as_matrix()
+    t0 = scene.poses_se3[0, 4:7].copy()
+    want_pose, want_k, n_frag = np.zeros(6), np.zeros(5), 0
+    Cn = scene.num_channels
+    eps = 1e-6
+    for (l, x, y), ids in lists.items():
+        w, h = f.sizes[l]
+        if min(x, y, w - 1 - x, h - 1 - y) <= 2:
+            continue
+        I, G = f.out[l][0].astype(np.float64), go[l][0].astype(np.float64)
+        for i in ids:
+            t = tex[:, i]
+            dx = 0.5 * (-(t - I[:, y, x - 1]) * G[:, y, x - 1] + (t - I[:, y, x + 1]) * G[:, y, x + 1]).sum() / Cn
+            dy = 0.5 * (-(t - I[:, y - 1, x]) * G[:, y - 1, x] + (t - I[:, y + 1, x]) * G[:, y + 1, x]).sum() / Cn
+            grad = (0.5 ** l) * np.array([dx, dy])
+            p = scene.position[i].astype(np.float64)
+            for k in range(6):
+                xi = np.zeros(6)
+                ips = []
+                for sgn in (+1, -1):
+                    xi[:] = 0
+                    xi[k] = sgn * eps
+                    Rw = Rotation.from_rotvec(xi[3:]).as_matrix()
+                    ips.append(project64_camera(p, Rw @ R0, Rw @ t0 + xi[:3], K5, crop32, rot32, v.w, v.h))
+                want_pose[k] += grad @ ((ips[0] - ips[1]) / (2 * eps))
+            for k in range(4):  # fx, fy, cx, cy; the skew column is zeroed by the reference
+                Kp, Km = K5.copy(), K5.copy()
+                h_k = 1e-4
+                Kp[k] += h_k
+                Km[k] -= h_k
+                d = project64_camera(p, R0, t0, Kp, crop32, rot32, v.w, v.h) - project64_camera(p, R0, t0, Km, crop32, rot32, v.w, v.h)
+                want_k[k] += 0.5 * (grad @ (d / (2 * h_k)))
+            n_frag += 1
+    assert n_frag > 100
+    assert g["pose_count"][0] == pytest.approx(n_frag / 1024.0, rel=1e-5)
+    assert g["intrinsics_count"][0] == pytest.approx(n_frag / 1024.0, rel=1e-5)
+    np.testing.assert_allclose(g["pose"][0], want_pose, rtol=2e-3, atol=2e-4 * np.abs(want_pose).max())
+    np.testing.assert_allclose(g["intrinsics"][0, :5], want_k, rtol=2e-3, atol=2e-4 * np.abs(want_k).max())
+    assert np.all(g["intrinsics"][0, 4:] == 0)
+    # normalisation: every row divided by its count (1024 x the mean over fragments)
+    gn = oracle.backward(f, go, want_cameras=True, camera_gradient_normalization=1)
+    np.testing.assert_allclose(gn["pose"][0], g["pose"][0] / g["pose_count"][0], rtol=1e-6)
+    np.testing.assert_allclose(gn["intrinsics"][0], g["intrinsics"][0] / g["intrinsics_count"][0], rtol=1e-6)

@@ -50,6 +50,8 @@ class Params(C.Structure):
         ("check_normal", C.c_int32),
         ("quirk_background_confidence_leak", C.c_int32),
         ("point_gradient_normalization", C.c_int32),
+        ("K_gradient_factor", C.c_float),
+        ("camera_gradient_normalization", C.c_int32),
     ]
 
 
@@ -73,6 +75,7 @@ class WorkspaceLayout(C.Structure):
         ("forward_only_bytes", C.c_size_t),
         ("partial_base", C.c_size_t),
         ("background_partial_base", C.c_size_t),
+        ("camera_partial_base", C.c_size_t),
     ]
 
 
@@ -106,6 +109,10 @@ class BackwardArgs(C.Structure):
         ("grad_background", C.c_void_p),
         ("grad_points", C.c_void_p),
         ("grad_point_count", C.c_void_p),
+        ("grad_pose", C.c_void_p),
+        ("grad_pose_count", C.c_void_p),
+        ("grad_intrinsics", C.c_void_p),
+        ("grad_intrinsics_count", C.c_void_p),
     ]
 
 

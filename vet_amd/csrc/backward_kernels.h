@@ -351,10 +351,13 @@ struct GatherPass
     float* grad_confidence;   // [N]
     float* grad_points;       // [N,4] or null
     float* grad_point_count;  // [N]
+    double* camera_partial;   // [workgroups][kCameraRow] per-workgroup pose / intrinsics sums, or null
     int K;
     int need_point_gradient;
     int accumulate;  // 0: overwrite the gradient rows (first view), 1: add to them (further views)
 };
+
+constexpr int kCameraRow = 12;  // doubles per workgroup row: 6 pose tangent, fx, fy, cx, cy, fragment count, pad
 
 // One thread per point: find the pixel the point fell into in every layer (the same projection as the count pass), decide
 // whether its fragment survived the top-K cut (its key is not larger than the K-th key of that pixel's sorted list), and
@@ -363,16 +366,19 @@ struct GatherPass
 template <int C>
 __global__ void __launch_bounds__(kBlock) gather_point_gradients_kernel(GatherPass a)
 {
-    const int i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (i >= a.vp.N) return;
+    const int i      = blockIdx.x * blockDim.x + threadIdx.x;
+    const bool alive = i < a.vp.N;
     float gt[C];
 #pragma unroll
     for (int ci = 0; ci < C; ++ci) gt[ci] = 0.f;
     float gc = 0.f, gx = 0.f, gy = 0.f, gz = 0.f, cnt = 0.f;
+    float cam_sum[10];  // pose tangent (translation, rotation), fx, fy, cx, cy
+#pragma unroll
+    for (int k = 0; k < 10; ++k) cam_sum[k] = 0.f;
     Projected p;
     const DeviceView& cam = *a.vp.view;
-    const float4 wp       = a.vp.position[i];
-    if (!point_is_skipped(a.vp, i) && project_point(cam, wp, p))
+    const float4 wp       = alive ? a.vp.position[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+    if (alive && !point_is_skipped(a.vp, i) && project_point(cam, wp, p))
     {
         // view-space position again, for the projection Jacobian (same expressions as project_point)
         const float vx = ((cam.r[0] * wp.x + cam.r[1] * wp.y) + cam.r[2] * wp.z) + cam.t[0];
@@ -416,9 +422,44 @@ __global__ void __launch_bounds__(kBlock) gather_point_gradients_kernel(GatherPa
                 gy += (cam.r[1] * e0 + cam.r[4] * e1) + cam.r[7] * e2;
                 gz += (cam.r[2] * e0 + cam.r[5] * e1) + cam.r[8] * e2;
                 cnt += 1.f;
+                if (a.camera_partial)
+                {
+                    // pose: J_pose^T e with J_pose = [I | -[view_p]x] (tangent = translation, rotation; applied on the
+                    // left, src/lib/rendering/PointRenderer.cu:1325-1341); K: d image / d (fx, fy, cx, cy)
+                    // (src/lib/rendering/RenderBackward.cu:1418-1437, the skew column is zeroed there)
+                    cam_sum[0] += e0;
+                    cam_sum[1] += e1;
+                    cam_sum[2] += e2;
+                    cam_sum[3] += vy * e2 - vz * e1;
+                    cam_sum[4] += vz * e0 - vx * e2;
+                    cam_sum[5] += vx * e1 - vy * e0;
+                    cam_sum[6] += (vx / vz) * a2;
+                    cam_sum[7] += (vy / vz) * b2;
+                    cam_sum[8] += a2;
+                    cam_sum[9] += b2;
+                }
             }
         }
     }
+    if (a.camera_partial)
+    {
+        // workgroup sums in double, one row per workgroup; reduce_camera_kernel adds the rows of a view
+        __shared__ double cam_red[kBlock / kWave][kCameraRow];
+        const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+#pragma unroll
+        for (int k = 0; k < 11; ++k)
+        {
+            double v = (k < 10) ? (double)cam_sum[k] : (double)cnt;
+#pragma unroll
+            for (int d = kWave / 2; d >= 1; d >>= 1) v += __shfl_xor(v, d, kWave);
+            if (lane == 0) cam_red[wave][k] = v;
+        }
+        __syncthreads();
+        if (threadIdx.x < 11)
+            a.camera_partial[(size_t)blockIdx.x * kCameraRow + threadIdx.x] =
+                (cam_red[0][threadIdx.x] + cam_red[1][threadIdx.x]) + (cam_red[2][threadIdx.x] + cam_red[3][threadIdx.x]);
+    }
+    if (!alive) return;
     const int N = a.vp.N;
     if (a.vp.index)
     {
@@ -457,6 +498,82 @@ __global__ void __launch_bounds__(kBlock) gather_point_gradients_kernel(GatherPa
             *gp                   = make_float4(gx, gy, gz, 0.f);
             a.grad_point_count[i] = cnt;
         }
+    }
+}
+
+// Adds the per-workgroup camera rows of one view to the pose row image_index (double) and the intrinsics row
+// camera_index (fx, fy, cx, cy times K_gradient_factor; skew and distortion columns stay zero), and the fragment count
+// / 1024 to both count arrays, as src/lib/rendering/RenderBackward.cu:1418-1459 does per fragment with atomics.
+__global__ void __launch_bounds__(kBlock) reduce_camera_kernel(const double* __restrict__ rows, int num_rows,
+                                                                int image_index, int camera_index, float k_factor,
+                                                                double* __restrict__ grad_pose,
+                                                                float* __restrict__ grad_pose_count,
+                                                                float* __restrict__ grad_intrinsics,
+                                                                float* __restrict__ grad_intrinsics_count)
+{
+    __shared__ double red[kBlock / kWave][kCameraRow];
+    double acc[11];
+#pragma unroll
+    for (int k = 0; k < 11; ++k) acc[k] = 0.0;
+    for (int r = threadIdx.x; r < num_rows; r += kBlock)
+    {
+        const double* row = rows + (size_t)r * kCameraRow;
+#pragma unroll
+        for (int k = 0; k < 11; ++k) acc[k] += row[k];
+    }
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+#pragma unroll
+    for (int k = 0; k < 11; ++k)
+    {
+        double v = acc[k];
+#pragma unroll
+        for (int d = kWave / 2; d >= 1; d >>= 1) v += __shfl_xor(v, d, kWave);
+        if (lane == 0) red[wave][k] = v;
+    }
+    __syncthreads();
+    if (threadIdx.x < 11)
+    {
+        const int k    = threadIdx.x;
+        const double s = (red[0][k] + red[1][k]) + (red[2][k] + red[3][k]);
+        if (k < 6)
+        {
+            if (grad_pose) grad_pose[6 * (size_t)image_index + k] += s;
+        }
+        else if (k < 10)
+        {
+            if (grad_intrinsics)
+                grad_intrinsics[13 * (size_t)camera_index + (k - 6)] += (float)((double)k_factor * s);
+        }
+        else
+        {
+            const float c = (float)(s / 1024.0);
+            if (grad_pose) grad_pose_count[image_index] += c;
+            if (grad_intrinsics) grad_intrinsics_count[camera_index] += c;
+        }
+    }
+}
+
+// Rows divided by their counts: NormalizeGradientDevTensor<double,6> on the poses and NormalizeGradient<float,13> on the
+// intrinsics (src/lib/rendering/PointRenderer.cu:1092-1109,1253-1308).
+__global__ void __launch_bounds__(kBlock) normalize_camera_gradients_kernel(double* __restrict__ grad_pose,
+                                                                             const float* __restrict__ pose_count,
+                                                                             int num_poses,
+                                                                             float* __restrict__ grad_intrinsics,
+                                                                             const float* __restrict__ intrinsics_count,
+                                                                             int num_cameras)
+{
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (grad_pose && i < num_poses)
+    {
+        const float c = pose_count[i];
+        if (c > 0.f)
+            for (int k = 0; k < 6; ++k) grad_pose[6 * (size_t)i + k] = grad_pose[6 * (size_t)i + k] / c;
+    }
+    if (grad_intrinsics && i < num_cameras)
+    {
+        const float c = intrinsics_count[i];
+        if (c > 0.f)
+            for (int k = 0; k < 13; ++k) grad_intrinsics[13 * (size_t)i + k] = grad_intrinsics[13 * (size_t)i + k] / c;
     }
 }
 

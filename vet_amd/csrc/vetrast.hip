@@ -323,6 +323,8 @@ int vetrast_workspace_layout_for(int32_t N, int32_t B, int32_t L, int32_t w, int
     at += align_up(cap * 8 * sizeof(float), kAlign);
     lay->background_partial_base = at;
     at += align_up((size_t)make_tile_map(t).slots_per_xcd * kXcds * kBackgroundRow * sizeof(float), kAlign);
+    lay->camera_partial_base = at;
+    at += align_up(((size_t)N + kBlock - 1) / kBlock * kCameraRow * sizeof(double), kAlign);
     lay->total_bytes = align_up(at, kAlign);
     return VETRAST_OK;
 }
@@ -477,6 +479,8 @@ int vetrast_backward(vetrast_ctx* ctx, const vetrast_backward_args* g, void* str
     if (!g->grad_texture || !g->grad_confidence || !g->grad_background) return VETRAST_ERR_INVALID_ARG;
     if (g->grad_points && !g->grad_point_count) return VETRAST_ERR_INVALID_ARG;
     if (g->grad_points && ((uintptr_t)g->grad_points % 16) != 0) return VETRAST_ERR_INVALID_ARG;
+    if (g->grad_pose && !g->grad_pose_count) return VETRAST_ERR_INVALID_ARG;
+    if (g->grad_intrinsics && !g->grad_intrinsics_count) return VETRAST_ERR_INVALID_ARG;
     const vetrast_params& p = a->params;
     for (int l = 0; l < p.num_layers; ++l)
         if (!g->grad_out[l]) return VETRAST_ERR_INVALID_ARG;
@@ -498,6 +502,16 @@ int vetrast_backward(vetrast_ctx* ctx, const vetrast_backward_args* g, void* str
             hipLaunchKernelGGL(fill_u32_kernel, dim3(std::min(grid_for(n), 8192)), dim3(kBlock), 0, stream,
                                reinterpret_cast<uint32_t*>(ptr), n, 0u);
         };
+        if (g->grad_pose)
+        {
+            zero(reinterpret_cast<float*>(g->grad_pose), (size_t)12 * a->num_poses);
+            zero(g->grad_pose_count, (size_t)a->num_poses);
+        }
+        if (g->grad_intrinsics)
+        {
+            zero(g->grad_intrinsics, (size_t)13 * a->num_cameras);
+            zero(g->grad_intrinsics_count, (size_t)a->num_cameras);
+        }
         if (add_to_rows)
         {
             zero(g->grad_texture, (size_t)C * N);
@@ -509,6 +523,11 @@ int vetrast_backward(vetrast_ctx* ctx, const vetrast_backward_args* g, void* str
             }
         }
     }
+    // position, pose and intrinsics gradients all hang off the per-fragment image-space gradient
+    // (src/lib/rendering/RenderBackward.cu:1183, 1401-1459)
+    const bool want_camera         = p.need_point_gradient && (g->grad_pose || g->grad_intrinsics) && N > 0;
+    const bool want_image_gradient = p.need_point_gradient && (g->grad_points || g->grad_pose || g->grad_intrinsics);
+    double* camera_rows            = ws_ptr<double>(ws, lay.camera_partial_base);
     float4* partial        = ws_ptr<float4>(ws, lay.partial_base);
     float* background_rows = ws_ptr<float>(ws, lay.background_partial_base);
     for (int b = 0; b < B; ++b)
@@ -533,7 +552,7 @@ int vetrast_backward(vetrast_ctx* ctx, const vetrast_backward_args* g, void* str
             bp.N                = N;
             bp.K                = p.debug_max_list_length;
             bp.use_environment_map              = p.use_environment_map;
-            bp.need_point_gradient              = (p.need_point_gradient && g->grad_points) ? 1 : 0;
+            bp.need_point_gradient              = want_image_gradient ? 1 : 0;
             bp.quirk_background_confidence_leak = p.quirk_background_confidence_leak;
             for (int l = 0; l < VETRAST_MAX_LAYERS; ++l)
             {
@@ -567,7 +586,8 @@ int vetrast_backward(vetrast_ctx* ctx, const vetrast_backward_args* g, void* str
             gp.grad_points         = g->grad_points;
             gp.grad_point_count    = g->grad_point_count;
             gp.K                   = p.debug_max_list_length;
-            gp.need_point_gradient = (p.need_point_gradient && g->grad_points) ? 1 : 0;
+            gp.need_point_gradient = want_image_gradient ? 1 : 0;
+            gp.camera_partial      = want_camera ? camera_rows : nullptr;
             gp.accumulate          = (add_to_rows || b > 0) ? 1 : 0;
             const dim3 grid(grid_for(N)), blk(kBlock);
             switch (C)
@@ -577,6 +597,13 @@ int vetrast_backward(vetrast_ctx* ctx, const vetrast_backward_args* g, void* str
                 case 3: hipLaunchKernelGGL(gather_point_gradients_kernel<3>, grid, blk, 0, stream, gp); break;
                 default: hipLaunchKernelGGL(gather_point_gradients_kernel<4>, grid, blk, 0, stream, gp); break;
             }
+        }
+        if (want_camera)
+        {
+            ScopeTimer tm(ctx, stream, VETRAST_SCOPE_BACKWARD_GATHER);
+            hipLaunchKernelGGL(reduce_camera_kernel, dim3(1), dim3(kBlock), 0, stream, camera_rows, grid_for(N),
+                               a->views[b].image_index, a->views[b].camera_index, p.K_gradient_factor, g->grad_pose,
+                               g->grad_pose_count, g->grad_intrinsics, g->grad_intrinsics_count);
         }
         {
             // after the per-point kernel: it overwrites confidence row 0, the leak term is added on top
@@ -592,6 +619,14 @@ int vetrast_backward(vetrast_ctx* ctx, const vetrast_backward_args* g, void* str
         ScopeTimer tm(ctx, stream, VETRAST_SCOPE_BACKWARD_POST);
         hipLaunchKernelGGL(normalize_point_gradient_kernel, dim3(grid_for(N)), dim3(kBlock), 0, stream,
                            g->grad_points, g->grad_point_count, N, p.point_gradient_normalization);
+    }
+    if (want_camera && p.camera_gradient_normalization)
+    {
+        ScopeTimer tm(ctx, stream, VETRAST_SCOPE_BACKWARD_POST);
+        const int n = std::max(a->num_poses, a->num_cameras);
+        hipLaunchKernelGGL(normalize_camera_gradients_kernel, dim3(grid_for(n)), dim3(kBlock), 0, stream, g->grad_pose,
+                           g->grad_pose_count, a->num_poses, g->grad_intrinsics, g->grad_intrinsics_count,
+                           a->num_cameras);
     }
     VET_HIP(ctx, hipGetLastError());
     return VETRAST_OK;

@@ -31,6 +31,8 @@ def make_params(scene: Scene, **overrides) -> abi.Params:
     p.check_normal = 0
     p.quirk_background_confidence_leak = 0
     p.point_gradient_normalization = 0
+    p.K_gradient_factor = 0.5
+    p.camera_gradient_normalization = 0
     for k, v in {**scene.params, **overrides}.items():
         if not hasattr(p, k):
             raise AttributeError(f"vetrast_params has no field {k}")
@@ -177,7 +179,8 @@ class Rasterizer:
         abi.check(self.lib.vetrast_forward(self.ctx, C.byref(args), self._stream()), "forward")
         return ForwardResult(out, masks, workspace, lay, args, (views, dev, params))
 
-    def backward(self, fwd: ForwardResult, grad_out: List[torch.Tensor], want_points=True, **param_overrides):
+    def backward(self, fwd: ForwardResult, grad_out: List[torch.Tensor], want_points=True, want_cameras=False,
+                 **param_overrides):
         dev = fwd.keep[1]
         scene = dev.scene
         N, Cn = scene.num_points, scene.num_channels
@@ -201,6 +204,16 @@ class Rasterizer:
             res["point_count"] = torch.empty((N,), dtype=torch.float32, device=dev.device)
             g.grad_points = res["points"].data_ptr()
             g.grad_point_count = res["point_count"].data_ptr()
+        if want_cameras:
+            F, ncam = int(scene.poses_se3.shape[0]), int(scene.intrinsics.shape[0])
+            res["pose"] = torch.empty((F, 6), dtype=torch.float64, device=dev.device)
+            res["pose_count"] = torch.empty((F,), dtype=torch.float32, device=dev.device)
+            res["intrinsics"] = torch.empty((ncam, 13), dtype=torch.float32, device=dev.device)
+            res["intrinsics_count"] = torch.empty((ncam,), dtype=torch.float32, device=dev.device)
+            g.grad_pose = res["pose"].data_ptr()
+            g.grad_pose_count = res["pose_count"].data_ptr()
+            g.grad_intrinsics = res["intrinsics"].data_ptr()
+            g.grad_intrinsics_count = res["intrinsics_count"].data_ptr()
         abi.check(self.lib.vetrast_backward(self.ctx, C.byref(g), self._stream()), "backward")
         res["_args"] = g
         return res

@@ -36,6 +36,8 @@ vetrast_params to_abi_params(const RenderParams& p, int num_layers)
     q.check_normal                     = p.check_normal ? 1 : 0;
     q.quirk_background_confidence_leak = p.quirk_background_confidence_leak ? 1 : 0;
     q.point_gradient_normalization     = p.point_gradient_normalization;
+    q.K_gradient_factor                = p.K_gradient_factor;
+    q.camera_gradient_normalization    = p.camera_gradient_normalization ? 1 : 0;
     return q;
 }
 
@@ -143,8 +145,9 @@ torch::autograd::variable_list PointRender::forward(torch::autograd::AutogradCon
     vetrast_workspace_layout lay;
     check_status(vetrast_workspace_layout_for(a.num_points, B, L, info->images[0].w, info->images[0].h, &lay), "layout");
 
-    const bool need_backward = ctx != nullptr && (texture.requires_grad() || background_color.requires_grad() ||
-                                                  points.requires_grad() || confidence.requires_grad());
+    const bool need_backward =
+        ctx != nullptr && (texture.requires_grad() || background_color.requires_grad() || points.requires_grad() ||
+                           confidence.requires_grad() || pose_tangents.requires_grad() || intrinsics.requires_grad());
     auto u8 = torch::TensorOptions().device(points.device()).dtype(torch::kUInt8);
     torch::Tensor workspace;
     if (need_backward)
@@ -189,6 +192,9 @@ torch::autograd::variable_list PointRender::forward(torch::autograd::AutogradCon
         ctx->saved_data["has_dropout"] = dropout.defined();
         ctx->saved_data["has_index"]   = t_index.defined();
         ctx->saved_data["points_need_grad"] = points.requires_grad();
+        ctx->saved_data["pose_need_grad"]   = pose_tangents.requires_grad();
+        ctx->saved_data["intr_need_grad"]   = intrinsics.requires_grad();
+        ctx->saved_data["num_poses"]        = (int64_t)poses_se3.size(0);
     }
     // masks are not differentiable (the reference detaches them in RenderModule.cpp:74-102)
     if (ctx) ctx->mark_non_differentiable(mask);
@@ -245,12 +251,27 @@ torch::autograd::variable_list PointRender::backward(torch::autograd::AutogradCo
         g.grad_points      = g_points.data_ptr<float>();
         g.grad_point_count = g_point_count.data_ptr<float>();
     }
+    torch::Tensor g_pose, g_pose_count, g_intrinsics, g_intrinsics_count;
+    if (ctx->saved_data["pose_need_grad"].toBool())  // PointRenderer.cu:287-293
+    {
+        const int64_t F      = ctx->saved_data["num_poses"].toInt();
+        g_pose               = torch::empty({F, 6}, points.options().dtype(torch::kFloat64));
+        g_pose_count         = torch::empty({F}, points.options());
+        g.grad_pose          = g_pose.data_ptr<double>();
+        g.grad_pose_count    = g_pose_count.data_ptr<float>();
+    }
+    if (ctx->saved_data["intr_need_grad"].toBool())  // PointRenderer.cu:295-300
+    {
+        g_intrinsics            = torch::empty_like(intrinsics);
+        g_intrinsics_count      = torch::empty({intrinsics.size(0)}, intrinsics.options());
+        g.grad_intrinsics       = g_intrinsics.data_ptr<float>();
+        g.grad_intrinsics_count = g_intrinsics_count.data_ptr<float>();
+    }
     check_status(vetrast_backward(info->cache->ctx, &g, current_stream()), "backward");
 
     // order: texture, background, points, pose_tangent, intrinsics, confidence, dynamic (PointRenderer.cu:1319-1322),
-    // plus one empty gradient for the IValue (RenderInfo.cpp:64). Pose and intrinsics gradients are not computed.
-    return {g_texture, g_background, g_points, torch::Tensor(), torch::Tensor(), g_confidence, torch::Tensor(),
-            torch::Tensor()};
+    // plus one empty gradient for the IValue (RenderInfo.cpp:64). Undefined where the input does not require grad.
+    return {g_texture, g_background, g_points, g_pose, g_intrinsics, g_confidence, torch::Tensor(), torch::Tensor()};
 }
 
 }  // namespace vet_amd
@@ -321,6 +342,8 @@ std::vector<torch::Tensor> blend_point_cloud(torch::Tensor texture, torch::Tenso
         else if (k == "quirk_background_confidence_leak") p.quirk_background_confidence_leak = as_d() != 0;
         else if (k == "point_gradient_normalization") p.point_gradient_normalization = (int)as_d();
         else if (k == "render_mode") p.render_mode = (int)as_d();
+        else if (k == "K_gradient_factor") p.K_gradient_factor = (float)as_d();
+        else if (k == "camera_gradient_normalization") p.camera_gradient_normalization = as_d() != 0;
         else TORCH_CHECK(false, "unknown RenderParams field ", k);
     }
     // the scene bundle only has to live for the duration of apply(): everything backward needs is saved in the graph

@@ -25,6 +25,7 @@ struct RenderParams
     bool check_normal                  = false;
     float dropout                      = 0.25f;
     float drop_out_radius_threshold    = 0.6f;
+    float K_gradient_factor            = 0.5f;
     bool drop_out_points_by_radius     = true;
     int num_texture_channels           = -1;
     bool output_background_mask        = false;
@@ -39,6 +40,7 @@ struct RenderParams
     // Switches for two accidents of the reference implementation; the defaults reproduce it literally.
     bool quirk_background_confidence_leak = true;   // src/lib/rendering/RenderBackward.cu:1157
     int point_gradient_normalization      = 2;      // src/lib/rendering/PointRenderer.cu:1278-1279
+    bool camera_gradient_normalization    = true;   // src/lib/rendering/PointRenderer.cu:1253-1308
 };
 
 // The tensors BlendPointCloud reads through info->scene (src/lib/rendering/RenderInfo.cpp:25-29 and
