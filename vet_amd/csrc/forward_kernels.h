@@ -86,12 +86,15 @@ __global__ void prepare_views_kernel(PrepareViewsArgs args, int first_view, int 
 // Planar descriptors [C,N] + confidence [N] -> one 32-byte record per texture index, so that a fragment costs a single
 // aligned gather instead of C+1 gathers from planes megabytes apart (the reference's BlendMulti reads
 // d_texture.in_texture(ci, idx) per channel, src/lib/rendering/RenderForward.cu:1338-1342).
+// The same launch also zeroes the per-pixel counters of all views (n4 uint4 elements), which saves a launch per call.
 template <int C>
 __global__ void __launch_bounds__(kBlock) pack_descriptors_kernel(const float* __restrict__ texture,
                                                                    const float* __restrict__ confidence,
-                                                                   float4* __restrict__ packed, int N)
+                                                                   float4* __restrict__ packed, int N,
+                                                                   uint4* __restrict__ counters4, size_t n4)
 {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    for (size_t k = (size_t)i; k < n4; k += (size_t)gridDim.x * blockDim.x) counters4[k] = make_uint4(0u, 0u, 0u, 0u);
     if (i >= N) return;
     float t[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll

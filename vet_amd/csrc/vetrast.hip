@@ -359,9 +359,11 @@ int vetrast_forward(vetrast_ctx* ctx, const vetrast_forward_args* a, void* strea
     {
         ScopeTimer tm(ctx, stream, VETRAST_SCOPE_PREPARE);
         // per-pixel counters of all views (contiguous) start at zero; InitializeData, PointRenderer.cu:402-470
-        const size_t n4 = Ppad * B / 4;
-        hipLaunchKernelGGL(fill_u128_kernel, dim3(std::min(grid_for(n4), 4096)), dim3(kBlock), 0, stream,
-                           ws_ptr<uint4>(ws, lay.offsets_base), n4, 0u);
+        const size_t n4  = Ppad * B / 4;
+        uint4* counters4 = ws_ptr<uint4>(ws, lay.offsets_base);
+        if (N == 0)
+            hipLaunchKernelGGL(fill_u128_kernel, dim3(std::min(grid_for(n4), 4096)), dim3(kBlock), 0, stream, counters4,
+                               n4, 0u);
         for (int first = 0; first < B; first += 16)
         {
             PrepareViewsArgs pv;
@@ -385,10 +387,10 @@ int vetrast_forward(vetrast_ctx* ctx, const vetrast_forward_args* a, void* strea
             const dim3 g(grid_for(N)), blk(kBlock);
             switch (C)
             {
-                case 1: hipLaunchKernelGGL(pack_descriptors_kernel<1>, g, blk, 0, stream, a->texture, a->confidence, packed, N); break;
-                case 2: hipLaunchKernelGGL(pack_descriptors_kernel<2>, g, blk, 0, stream, a->texture, a->confidence, packed, N); break;
-                case 3: hipLaunchKernelGGL(pack_descriptors_kernel<3>, g, blk, 0, stream, a->texture, a->confidence, packed, N); break;
-                default: hipLaunchKernelGGL(pack_descriptors_kernel<4>, g, blk, 0, stream, a->texture, a->confidence, packed, N); break;
+                case 1: hipLaunchKernelGGL(pack_descriptors_kernel<1>, g, blk, 0, stream, a->texture, a->confidence, packed, N, counters4, n4); break;
+                case 2: hipLaunchKernelGGL(pack_descriptors_kernel<2>, g, blk, 0, stream, a->texture, a->confidence, packed, N, counters4, n4); break;
+                case 3: hipLaunchKernelGGL(pack_descriptors_kernel<3>, g, blk, 0, stream, a->texture, a->confidence, packed, N, counters4, n4); break;
+                default: hipLaunchKernelGGL(pack_descriptors_kernel<4>, g, blk, 0, stream, a->texture, a->confidence, packed, N, counters4, n4); break;
             }
         }
     }
