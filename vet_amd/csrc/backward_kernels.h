@@ -76,7 +76,10 @@ __global__ void __launch_bounds__(kBlock) blend_backward_kernel(BackwardPass a)
     __shared__ uint32_t s_base[kWaves][kWave];
     __shared__ float s_carry[kWaves][kWave];
     __shared__ float4 s_g[kWaves][kWave];
-    __shared__ float4 s_nb[kWaves][kWave][8];  // I(x-1), I(x+1), I(y-1), I(y+1), G(x-1), G(x+1), G(y-1), G(y+1)
+    // position heuristic of a pixel as coefficients: d image x = (t . ax + bx) / C, d image y = (t . ay + by) / C
+    __shared__ float4 s_ax[kWaves][kWave];
+    __shared__ float4 s_ay[kWaves][kWave];
+    __shared__ float2 s_bxy[kWaves][kWave];
     __shared__ uint8_t s_point[kWaves][kWave];
     __shared__ uint8_t s_item[kWaves][kWaveItems];
     __shared__ float red[kWaves][C + 1];
@@ -125,28 +128,28 @@ __global__ void __launch_bounds__(kBlock) blend_backward_kernel(BackwardPass a)
         s_point[wave][lane] = do_point ? 1 : 0;
         if (do_point)
         {
+            // The reference evaluates, per fragment with descriptor t and per channel,
+            //   1/2 * ( -(t - I(x-1)) * G(x-1) + (t - I(x+1)) * G(x+1) )        (RenderBackward.cu:1364-1371)
+            // and the same in y. That is linear in t: t * 1/2 (G(x+1) - G(x-1)) + 1/2 (I(x-1) G(x-1) - I(x+1) G(x+1)),
+            // so the neighbour samples are folded once per pixel into C slopes and one offset per axis.
             const float* I = a.out[l];
-            float nb[8][4];
-#pragma unroll
-            for (int k = 0; k < 8; ++k)
-#pragma unroll
-                for (int ci = 0; ci < 4; ++ci) nb[k][ci] = 0.f;
+            float ax[4] = {0.f, 0.f, 0.f, 0.f}, ay[4] = {0.f, 0.f, 0.f, 0.f};
+            float bx = 0.f, by = 0.f;
 #pragma unroll
             for (int ci = 0; ci < C; ++ci)
             {
                 const float* Ic = I + ci * plane + local;
                 const float* Gc = G + ci * plane + local;
-                nb[0][ci] = Ic[-1];
-                nb[1][ci] = Ic[1];
-                nb[2][ci] = Ic[-lw];
-                nb[3][ci] = Ic[lw];
-                nb[4][ci] = Gc[-1];
-                nb[5][ci] = Gc[1];
-                nb[6][ci] = Gc[-lw];
-                nb[7][ci] = Gc[lw];
+                const float Ix0 = Ic[-1], Ix1 = Ic[1], Iy0 = Ic[-lw], Iy1 = Ic[lw];
+                const float Gx0 = Gc[-1], Gx1 = Gc[1], Gy0 = Gc[-lw], Gy1 = Gc[lw];
+                ax[ci] = 0.5f * (Gx1 - Gx0);
+                ay[ci] = 0.5f * (Gy1 - Gy0);
+                bx += 0.5f * (Ix0 * Gx0 - Ix1 * Gx1);
+                by += 0.5f * (Iy0 * Gy0 - Iy1 * Gy1);
             }
-#pragma unroll
-            for (int k = 0; k < 8; ++k) s_nb[wave][lane][k] = make_float4(nb[k][0], nb[k][1], nb[k][2], nb[k][3]);
+            s_ax[wave][lane]  = make_float4(ax[0], ax[1], ax[2], ax[3]);
+            s_ay[wave][lane]  = make_float4(ay[0], ay[1], ay[2], ay[3]);
+            s_bxy[wave][lane] = make_float2(bx, by);
         }
     }
 
@@ -228,23 +231,15 @@ __global__ void __launch_bounds__(kBlock) blend_backward_kernel(BackwardPass a)
                 float gp0 = 0.f, gp1 = 0.f;
                 if (s_point[wave][p])
                 {
-                    float nb[8][4];
-#pragma unroll
-                    for (int q8 = 0; q8 < 8; ++q8)
-                    {
-                        const float4 w4 = s_nb[wave][p][q8];
-                        nb[q8][0] = w4.x, nb[q8][1] = w4.y, nb[q8][2] = w4.z, nb[q8][3] = w4.w;
-                    }
-                    float dR_dpx = 0.f, dR_dpy = 0.f;
+                    const float4 ax4 = s_ax[wave][p], ay4 = s_ay[wave][p];
+                    const float2 b2  = s_bxy[wave][p];
+                    const float ax[4] = {ax4.x, ax4.y, ax4.z, ax4.w}, ay[4] = {ay4.x, ay4.y, ay4.z, ay4.w};
+                    float dR_dpx = b2.x, dR_dpy = b2.y;
 #pragma unroll
                     for (int ci = 0; ci < C; ++ci)
                     {
-                        const float d_x0 = -(t[ci] - nb[0][ci]) * nb[4][ci];
-                        const float d_x1 = (t[ci] - nb[1][ci]) * nb[5][ci];
-                        const float d_y0 = -(t[ci] - nb[2][ci]) * nb[6][ci];
-                        const float d_y1 = (t[ci] - nb[3][ci]) * nb[7][ci];
-                        dR_dpx += 0.5f * (d_x0 + d_x1);
-                        dR_dpy += 0.5f * (d_y0 + d_y1);
+                        dR_dpx += t[ci] * ax[ci];
+                        dR_dpy += t[ci] * ay[ci];
                     }
                     gp0 = dR_dpx / (float)C;  // image-space gradient of this fragment at the layer's resolution;
                     gp1 = dR_dpy / (float)C;  // the per-point kernel pushes it through the projection Jacobian
