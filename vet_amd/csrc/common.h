@@ -109,20 +109,20 @@ __device__ __forceinline__ int layer_of_pixel(const LayerTable& ly, uint32_t q)
 
 // Workgroup -> pixel mapping of the per-pixel kernels (blend, backward). A workgroup owns a 16x16 pixel tile (a wave
 // 16x4 of it), because the fragments of neighbouring pixels come from the same few 256-point blocks of the cloud and
-// their descriptor / position records then share cache lines. Workgroups are dealt round-robin to the 8 XCDs, each with
-// its own L2, so XCD k = b % 8 is given the k-th eighth of the tiles of EVERY layer (the coarse layers carry as many
-// fragments as the fine ones in far fewer tiles, so each XCD needs its share of each), coarsest layer first: every XCD
-// walks contiguous runs of tiles and finds in its L2 the lines the tile before (and the tile row above) brought in.
+// their descriptor records then share cache lines. The same point shows up once per layer, in the tiles that cover the
+// same part of the screen, so the tiles are grouped into screen regions: a region is one tile of the coarsest layer plus
+// the 4, 16, 64 ... tiles of the finer layers over the same area, and is walked coarsest layer first. Workgroups are
+// dealt round-robin to the 8 XCDs (each with its own L2), so workgroup b belongs to XCD b % 8 and takes slot b / 8 of
+// that XCD's run of regions (region r goes to XCD r % 8): what one layer's tiles pulled into the XCD's L2 is still there
+// when the next layer's tiles of the region ask for the same points.
 constexpr int kTile = 16;
 constexpr int kXcds = 8;
 struct TileMap
 {
     int L;
-    uint32_t tiles[VETRAST_MAX_LAYERS];    // tiles of layer l
-    uint32_t tiles_x[VETRAST_MAX_LAYERS];  // tiles per tile row of layer l
-    uint32_t chunk[VETRAST_MAX_LAYERS];    // tiles of layer l per XCD = ceil(tiles / 8)
-    uint32_t start[VETRAST_MAX_LAYERS];    // first per-XCD slot of layer l (slots run from the coarsest layer down)
-    uint32_t slots_per_xcd;                // sum of chunk[]
+    uint32_t regions_x, regions;     // region grid (regions per row, total)
+    uint32_t tiles_per_region;       // (4^L - 1) / 3
+    uint32_t regions_per_xcd;        // ceil(regions / 8)
 };
 
 struct TilePixel
@@ -139,19 +139,26 @@ __device__ __forceinline__ TilePixel tile_pixel(const TileMap& tm, const LayerTa
     r.active = false;
     r.l = r.x = r.y = 0;
     r.q = r.local = 0;
-    const uint32_t b    = blockIdx.x;
-    const uint32_t xcd  = b % kXcds;
-    const uint32_t slot = b / kXcds;
-    int l               = 0;
-#pragma unroll
-    for (int k = 1; k < VETRAST_MAX_LAYERS; ++k)
-        if (k < tm.L && slot < tm.start[k - 1]) l = k;  // start[] decreases with l: start[L-1] = 0
-    const uint32_t t = xcd * tm.chunk[l] + (slot - tm.start[l]);
-    if (slot >= tm.slots_per_xcd || t >= tm.tiles[l]) return r;
-    const uint32_t ty = t / tm.tiles_x[l], tx = t - ty * tm.tiles_x[l];
-    r.l               = l;
-    r.x               = (int)(tx * kTile + (threadIdx.x & (kTile - 1)));
-    r.y               = (int)(ty * kTile + (threadIdx.x / kTile));
+    const uint32_t b      = blockIdx.x;
+    const uint32_t xcd    = b % kXcds;
+    const uint32_t slot   = b / kXcds;
+    const uint32_t region = (slot / tm.tiles_per_region) * kXcds + xcd;
+    uint32_t t            = slot % tm.tiles_per_region;  // tile inside the region, coarsest layer first
+    if (region >= tm.regions) return r;
+    // layer L-1 has 1 tile per region, L-2 has 4, L-3 has 16, ...
+    int l          = tm.L - 1;
+    uint32_t side  = 1;  // tiles per region side in layer l
+    while (t >= side * side)
+    {
+        t -= side * side;
+        side <<= 1;
+        --l;
+    }
+    const uint32_t ry = region / tm.regions_x, rx = region - ry * tm.regions_x;
+    const uint32_t ty = ry * side + t / side, tx = rx * side + (t & (side - 1));
+    r.l = l;
+    r.x = (int)(tx * kTile + (threadIdx.x & (kTile - 1)));
+    r.y = (int)(ty * kTile + (threadIdx.x / kTile));
     if (r.x >= ly.w[l] || r.y >= ly.h[l]) return r;
     r.local  = (uint32_t)r.y * (uint32_t)ly.w[l] + (uint32_t)r.x;
     r.q      = ly.base[l] + r.local;

@@ -195,20 +195,22 @@ TileMap make_tile_map(const LayerTable& ly)
     TileMap m;
     std::memset(&m, 0, sizeof(m));
     m.L = ly.L;
-    for (int l = 0; l < ly.L; ++l)
-    {
-        m.tiles_x[l] = (uint32_t)(ly.w[l] + kTile - 1) / kTile;
-        m.tiles[l]   = m.tiles_x[l] * ((uint32_t)(ly.h[l] + kTile - 1) / kTile);
-        m.chunk[l]   = (m.tiles[l] + kXcds - 1) / kXcds;
-    }
-    uint32_t slot = 0;
-    for (int l = ly.L - 1; l >= 0; --l)
-    {
-        m.start[l] = slot;
-        slot += m.chunk[l];
-    }
-    m.slots_per_xcd = slot;
+    // a region is one 16x16 tile of the coarsest layer; over the finer layers it covers (16 << k)^2 pixels. Layer sizes
+    // come from integer halving, so the finest layer can be a few pixels larger than 2^(L-1) times the coarsest one:
+    // size the region grid from the finest layer.
+    const uint32_t span = (uint32_t)kTile << (ly.L - 1);
+    m.regions_x         = ((uint32_t)ly.w[0] + span - 1) / span;
+    m.regions           = m.regions_x * (((uint32_t)ly.h[0] + span - 1) / span);
+    uint32_t tiles      = 0;
+    for (int k = 0; k < ly.L; ++k) tiles += 1u << (2 * k);
+    m.tiles_per_region = tiles;
+    m.regions_per_xcd  = (m.regions + kXcds - 1) / kXcds;
     return m;
+}
+
+uint32_t tile_grid(const TileMap& m)
+{
+    return m.regions_per_xcd * m.tiles_per_region * kXcds;
 }
 
 ViewPass make_view_pass(const vetrast_forward_args* a, const vetrast_workspace_layout& lay, const LayerTable& ly, int b)
@@ -322,7 +324,7 @@ int vetrast_workspace_layout_for(int32_t N, int32_t B, int32_t L, int32_t w, int
     lay->partial_base       = at;
     at += align_up(cap * 8 * sizeof(float), kAlign);
     lay->background_partial_base = at;
-    at += align_up((size_t)make_tile_map(t).slots_per_xcd * kXcds * kBackgroundRow * sizeof(float), kAlign);
+    at += align_up((size_t)tile_grid(make_tile_map(t)) * kBackgroundRow * sizeof(float), kAlign);
     lay->camera_partial_base = at;
     at += align_up(((size_t)N + kBlock - 1) / kBlock * kCameraRow * sizeof(double), kAlign);
     lay->total_bytes = align_up(at, kAlign);
@@ -456,7 +458,7 @@ int vetrast_forward(vetrast_ctx* ctx, const vetrast_forward_args* a, void* strea
                 bp.out[l]          = a->out[l] + (size_t)b * C * plane;
                 if (p.output_background_mask) bp.out_mask[l] = a->out_mask[l] + (size_t)b * plane;
             }
-            const dim3 g(tiles.slots_per_xcd * kXcds), blk(kBlock);
+            const dim3 g(tile_grid(tiles)), blk(kBlock);
             switch (C)
             {
                 case 1: hipLaunchKernelGGL(blend_kernel<1>, g, blk, 0, stream, bp); break;
@@ -565,7 +567,7 @@ int vetrast_backward(vetrast_ctx* ctx, const vetrast_backward_args* g, void* str
                 bp.grad_out[l]     = g->grad_out[l] + (size_t)b * C * plane;
                 bp.out[l]          = a->out[l] + (size_t)b * C * plane;
             }
-            const dim3 grid(tiles.slots_per_xcd * kXcds), blk(kBlock);
+            const dim3 grid(tile_grid(tiles)), blk(kBlock);
             switch (C)
             {
                 case 1: hipLaunchKernelGGL(blend_backward_kernel<1>, grid, blk, 0, stream, bp); break;
@@ -611,7 +613,7 @@ int vetrast_backward(vetrast_ctx* ctx, const vetrast_backward_args* g, void* str
             // after the per-point kernel: it overwrites confidence row 0, the leak term is added on top
             ScopeTimer tm(ctx, stream, VETRAST_SCOPE_BACKWARD_GATHER);
             hipLaunchKernelGGL(reduce_background_kernel, dim3(1), dim3(kBlock), 0, stream, background_rows,
-                               (int)(tiles.slots_per_xcd * kXcds), C, g->grad_background, g->grad_confidence,
+                               (int)(tile_grid(tiles)), C, g->grad_background, g->grad_confidence,
                                (p.quirk_background_confidence_leak && !p.use_environment_map && N > 0) ? 1 : 0,
                                b > 0 ? 1 : 0);
         }
