@@ -55,7 +55,12 @@ def measured_traffic():
     res = {}
     if not os.path.exists(TRAFFIC_FILE):
         return res
+    in_table = False
     for line in open(TRAFFIC_FILE):
+        if line.startswith("## "):
+            in_table = line.startswith("## Per scope")
+        if not in_table:
+            continue
         m = re.match(r"^\|\s*([A-Z_]+)\s*\|\s*([0-9.]+)\s*\|\s*([0-9.]+)\s*\|", line)
         if m:
             res[m.group(1)] = (float(m.group(2)) + float(m.group(3))) * 1024.0
