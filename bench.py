@@ -32,10 +32,10 @@ def algorithmic_bytes(N, P, F, Fk, Cn):
     N points, P pixels over all layers, F fragments, Fk fragments kept after the top-K cut.
     """
     fwd = {
-        "COUNT": 16 * N + 4 * P,                      # positions read, counts written
-        "SCAN": 8 * P,                                # counts read, offsets written
+        # the model's terms, booked on the kernels that do the corresponding work here
+        "COUNT": 16 * N,                              # positions read
         "FILL": 16 * N + 8 * F,                       # positions read again, fragment records written
-        "SORT": 16 * F,                               # records read and written
+        "BUILD": 4 * P + 8 * P + 16 * F,              # per-pixel counts, counts -> offsets, records read and written sorted
         "BLEND": 8 * Fk + (4 * Cn + 4) * Fk + 4 * P + 4 * Cn * P + 4 * P,  # lists, descriptor+confidence, offsets, out, weight
     }
     # The per-pixel kernel reads upstream grads and forward outputs (8CP), lists (8Fk), descriptor+confidence (4(C+1)Fk)
@@ -88,7 +88,8 @@ def run_scene(scene, backward, steps, warmup, profile=True):
     K = params.debug_max_list_length
     F = int(off[-1])
     Fk = int(np.minimum(counts, K).sum()) if K > 0 else F
-    F_layers = [int(off[int(lay.layer_pixel_base[l + 1])] - off[int(lay.layer_pixel_base[l])]) for l in range(L)]
+    bases = fwd.layer_bases()
+    F_layers = [int(off[bases[l + 1]] - off[bases[l]]) for l in range(L)]
 
     bargs = None
     if backward:
@@ -187,7 +188,7 @@ def main():
                       "frac": round(nbytes / 1e6 / t / HBM_PEAK_GBS, 4) if t > 0 else None}
         if k in traffic:
             kernels[k]["hbm_traffic_MB"] = round(traffic[k] / 1e6, 1)
-    for k in ("PREPARE", "BACKWARD_PREPARE", "BACKWARD_POST"):
+    for k in ("PREPARE", "SCAN", "BACKWARD_PREPARE", "BACKWARD_POST"):
         if r["per_step_ms"].get(k, 0.0) > 0:
             kernels[k] = {"ms": round(r["per_step_ms"][k], 5), "alg_MB": 0.0, "GBps": None, "frac": None}
     dominant = max(alg.keys(), key=lambda k: r["per_step_ms"].get(k, 0.0))

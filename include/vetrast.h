@@ -92,10 +92,10 @@ typedef struct vetrast_ctx vetrast_ctx;
 typedef enum vetrast_scope
 {
     VETRAST_SCOPE_PREPARE = 0,      /* "Build Cache": zero-fill, view preparation, descriptor interleave */
-    VETRAST_SCOPE_COUNT,            /* "CountingPass" */
-    VETRAST_SCOPE_SCAN,             /* "CreateAndAllocateBuffers" (prefix scan; no allocation here) */
-    VETRAST_SCOPE_FILL,             /* "CollectionPass" */
-    VETRAST_SCOPE_SORT,             /* "SortingPass" */
+    VETRAST_SCOPE_COUNT,            /* "CountingPass": fragments per bin (a 16x16 pixel tile or a piece of one) */
+    VETRAST_SCOPE_SCAN,             /* "CreateAndAllocateBuffers" (prefix scan over the bins; no allocation here) */
+    VETRAST_SCOPE_FILL,             /* "CollectionPass", first half: fragment records grouped by bin */
+    VETRAST_SCOPE_BUILD,            /* "CollectionPass" second half + "SortingPass": sorted per-pixel lists of every bin */
     VETRAST_SCOPE_BLEND,            /* "BlendingPass" */
     VETRAST_SCOPE_BACKWARD_PREPARE, /* "Prepare Backward": zero-fill of gradient buffers */
     VETRAST_SCOPE_BACKWARD_BLEND,   /* "BlendBackwards", per-pixel part */
@@ -105,12 +105,17 @@ typedef enum vetrast_scope
 } vetrast_scope;
 
 /* Byte offsets of the arrays inside the forward workspace, so that a caller (or a test) can read the
- * per-pixel fragment lists. Pixels of all layers are numbered consecutively: q = layer_pixel_base[l] + y*w_l + x. */
+ * per-pixel fragment lists. Pixels are numbered tile by tile: every layer is cut into 16x16 pixel tiles (the last
+ * column / row of tiles may hang over the image; those pixels exist in the numbering and have empty lists), and
+ *   q = 256 * (layer_tile_base[l] + (y / 16) * layer_tiles_x[l] + x / 16) + 16 * (y % 16) + x % 16. */
 typedef struct vetrast_workspace_layout
 {
     int32_t layer_w[VETRAST_MAX_LAYERS];
     int32_t layer_h[VETRAST_MAX_LAYERS];
-    int64_t layer_pixel_base[VETRAST_MAX_LAYERS + 1]; /* [L] = total pixel count P of one view */
+    int32_t layer_tiles_x[VETRAST_MAX_LAYERS];        /* tiles per row of the layer = ceil(w_l / 16) */
+    int32_t reserved0;
+    int64_t layer_tile_base[VETRAST_MAX_LAYERS + 1];  /* first tile of the layer; [L] = number of tiles T */
+    int64_t layer_pixel_base[VETRAST_MAX_LAYERS + 1]; /* 256 * layer_tile_base; [L] = pixel numbers P of one view */
     int64_t fragment_capacity;                        /* N * L, the per-view upper bound on fragments */
     size_t total_bytes;
     /* per-view arrays: offset of view b = base + b * stride */
@@ -122,9 +127,12 @@ typedef struct vetrast_workspace_layout
     size_t cut_flags_base, cut_flags_stride; /* uint8 [P]: 1 where the top-K cut dropped fragments of the pixel */
     /* shared by all views */
     size_t packed_base;    /* float [N][8]: descriptor (4, zero padded), confidence, 3 pad */
-    size_t slots_base;     /* uint32 [L][N]: per (layer, point) arrival rank inside its pixel, 0xFFFFFFFF = no fragment */
+    size_t slots_base;     /* uint32 [L][N]: per (layer, point) arrival rank inside its tile (scratch between two passes) */
     size_t views_base;     /* prepared per-view camera constants */
     size_t scan_partials_base;
+    int64_t num_bins;      /* bins of one view: runs of 256 / 64 / 16 / 4 consecutive pixel numbers, chosen per layer from N */
+    size_t bin_counts_base, bin_counts_stride; /* per view, uint32 [num_bins+1 padded]: fragments per bin, then their exclusive scan */
+    size_t binned_base;    /* uint32 [N*L][4]: fragment records grouped by bin (key low, key high, pixel in bin, 0); scratch */
     size_t flags_base;     /* uint32 [4] device status flags */
     size_t forward_only_bytes; /* a forward call with save_for_backward = 0 needs only this much */
     size_t partial_base;   /* float [L][N][8]: backward scratch, gradient record of the fragment of point i in layer l */

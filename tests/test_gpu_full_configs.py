@@ -102,7 +102,7 @@ def test_config5_depth_complexity_full_size(rasterizer, oracle):
     params, dev, res, ref = _forward_parity(scene, rasterizer, oracle, need_point_gradient=1)
     off = res.offsets(0)
     counts = np.diff(off)
-    P3 = int(res.layout.layer_pixel_base[3])
+    P3 = res.layer_bases()[3]
     assert counts[P3:].mean() > 100, "the coarsest layer must average more than 100 fragments per pixel"
     _backward_parity(scene, res, ref, rasterizer, oracle)
 

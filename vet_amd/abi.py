@@ -20,7 +20,7 @@ CAMERA_OCAM = 1
 CAMERA_SPHERICAL = 2
 
 SCOPE_NAMES = [
-    "PREPARE", "COUNT", "SCAN", "FILL", "SORT", "BLEND", "BACKWARD_PREPARE", "BACKWARD_BLEND", "BACKWARD_GATHER", "BACKWARD_POST",
+    "PREPARE", "COUNT", "SCAN", "FILL", "BUILD", "BLEND", "BACKWARD_PREPARE", "BACKWARD_BLEND", "BACKWARD_GATHER", "BACKWARD_POST",
 ]
 SCOPE_COUNT = len(SCOPE_NAMES)
 
@@ -59,6 +59,9 @@ class WorkspaceLayout(C.Structure):
     _fields_ = [
         ("layer_w", C.c_int32 * MAX_LAYERS),
         ("layer_h", C.c_int32 * MAX_LAYERS),
+        ("layer_tiles_x", C.c_int32 * MAX_LAYERS),
+        ("reserved0", C.c_int32),
+        ("layer_tile_base", C.c_int64 * (MAX_LAYERS + 1)),
         ("layer_pixel_base", C.c_int64 * (MAX_LAYERS + 1)),
         ("fragment_capacity", C.c_int64),
         ("total_bytes", C.c_size_t),
@@ -71,6 +74,9 @@ class WorkspaceLayout(C.Structure):
         ("slots_base", C.c_size_t),
         ("views_base", C.c_size_t),
         ("scan_partials_base", C.c_size_t),
+        ("num_bins", C.c_int64),
+        ("bin_counts_base", C.c_size_t), ("bin_counts_stride", C.c_size_t),
+        ("binned_base", C.c_size_t),
         ("flags_base", C.c_size_t),
         ("forward_only_bytes", C.c_size_t),
         ("partial_base", C.c_size_t),

@@ -223,6 +223,7 @@ __global__ void __launch_bounds__(kBlock) blend_backward_kernel(BackwardPass a)
             float S        = (lane + 1 < kWave && pn == p) ? vn : 0.f;  // deeper fragments of this round
             if (valid) S += s_carry[wave][p];                            // and of the rounds / windows before
             if (valid && (lane == 0 || pp != p)) s_carry[wave][p] += v;  // one lane per pixel moves the carry on
+            float4 rec_lo = make_float4(0.f, 0.f, 0.f, 0.f), rec_hi = rec_lo;
             if (ti >= 0)
             {
                 const float g[4]  = {g4.x, g4.y, g4.z, g4.w};
@@ -247,8 +248,23 @@ __global__ void __launch_bounds__(kBlock) blend_backward_kernel(BackwardPass a)
                 float gt[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int ci = 0; ci < C; ++ci) gt[ci] = Tc * g[ci];
-                partial_l[2 * (size_t)id]     = make_float4(gt[0], gt[1], gt[2], gt[3]);
-                partial_l[2 * (size_t)id + 1] = make_float4(gconf, gp0, gp1, 0.f);
+                rec_lo = make_float4(gt[0], gt[1], gt[2], gt[3]);
+                rec_hi = make_float4(gconf, gp0, gp1, 0.f);
+            }
+            {
+                // Record stores, two lanes per record: first the even lane's record (even lane its low half, odd lane
+                // the high half), then the odd lane's, so that each instruction issues one 32-byte request per record.
+                const int odd        = lane & 1;
+                const int own        = ti >= 0 ? id : -1;
+                const int other      = pair_other(own);
+                const float4 o_lo    = pair_other(rec_lo);
+                const float4 o_hi    = pair_other(rec_hi);
+                const int id_first   = odd ? other : own;
+                const int id_second  = odd ? own : other;
+                const float4 v_first = odd ? o_hi : rec_lo;
+                const float4 v_second = odd ? rec_hi : o_lo;
+                if (id_first >= 0) partial_l[2 * (size_t)id_first + odd] = v_first;
+                if (id_second >= 0) partial_l[2 * (size_t)id_second + odd] = v_second;
             }
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
             __builtin_amdgcn_wave_barrier();
@@ -340,7 +356,7 @@ struct GatherPass
     ViewPass vp;
     const uint32_t* offsets;
     const uint64_t* fragments;
-    const uint8_t* list_is_cut;  // per pixel, written by the sort
+    const uint8_t* list_is_cut;  // per pixel, written by the build pass
     const float4* partial;
     float* grad_texture;      // [C,N]
     float* grad_confidence;   // [N]
@@ -388,7 +404,8 @@ __global__ void __launch_bounds__(kBlock) gather_point_gradients_kernel(GatherPa
             const float fx = rintf(ipx), fy = rintf(ipy);
             if (!(fx >= 0.f && fx < (float)ly.w[l] && fy >= 0.f && fy < (float)ly.h[l])) continue;
             const int x = (int)fx, y = (int)fy;
-            const uint32_t q   = ly.base[l] + (uint32_t)y * (uint32_t)ly.w[l] + (uint32_t)x;
+            const uint32_t q   = (ly.tile_base[l] + (uint32_t)(y / kTile) * (uint32_t)ly.tiles_x[l] + (uint32_t)(x / kTile)) * kTilePixels +
+                               (uint32_t)(y % kTile) * kTile + (uint32_t)(x % kTile);
             if (a.K > 0 && a.list_is_cut[q] && key > a.fragments[a.offsets[q] + a.K - 1]) continue;  // cut away
             const float4 r0 = a.partial[2 * ((size_t)l * a.vp.N + i)];
             const float4 r1 = a.partial[2 * ((size_t)l * a.vp.N + i) + 1];

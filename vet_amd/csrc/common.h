@@ -32,13 +32,27 @@ struct DeviceView
 };
 static_assert(sizeof(DeviceView) == 32 * 4, "DeviceView is 32 floats");
 
-// Pixels of all layers of one view are numbered consecutively: q = base[l] + y * w[l] + x.
+// Pixels are numbered tile by tile: every layer is cut into 16x16 pixel tiles (the last column and row of tiles may
+// hang over the image), tiles are numbered row-major inside a layer and layer after layer, and pixel (x, y) of layer l is
+//   q = 256 * (tile_base[l] + (y / 16) * tiles_x[l] + x / 16) + 16 * (y % 16) + x % 16.
+// The 256 pixels of a tile are consecutive, so a tile's fragment lists form one contiguous stretch of the fragment
+// buffer and a workgroup that owns a tile reads and writes its per-pixel arrays fully coalesced. Pixels of overhanging
+// tiles that lie outside the image exist in the numbering and always have empty lists.
+constexpr int kTile       = 16;
+constexpr int kTilePixels = kTile * kTile;
 struct LayerTable
 {
     int L;
     int w[VETRAST_MAX_LAYERS];
     int h[VETRAST_MAX_LAYERS];
-    uint32_t base[VETRAST_MAX_LAYERS + 1];
+    int tiles_x[VETRAST_MAX_LAYERS];
+    int tiles_y[VETRAST_MAX_LAYERS];
+    uint32_t tile_base[VETRAST_MAX_LAYERS + 1];  // first tile of the layer; [L] = number of tiles
+    uint32_t base[VETRAST_MAX_LAYERS + 1];       // first pixel number of the layer = 256 * tile_base
+    // Bins of the list-building passes: runs of 2^bin_shift consecutive pixel numbers (256 = a tile, 64 = a 16x4 strip
+    // of it, 16 = one row of it, 4), chosen per layer so that a bin is expected to hold about a thousand fragments.
+    int bin_shift[VETRAST_MAX_LAYERS];
+    uint32_t bin_base[VETRAST_MAX_LAYERS + 1];  // first bin of the layer; [L] = number of bins
 };
 
 // Launch descriptor shared by the forward kernels of one view.
@@ -89,13 +103,35 @@ __device__ __forceinline__ bool project_point(const DeviceView& c, const float4 
     return true;
 }
 
-// Pixel of layer l for a projected point, or -1. The caller halves ipx/ipy/radius between layers
-// (src/lib/rendering/RenderForward.cu:856,888-891); rintf is round-half-even like __float2int_rn.
-__device__ __forceinline__ int64_t layer_pixel(const LayerTable& ly, int l, float ipx, float ipy)
+// Tile and pixel-in-tile of layer l for a projected point; false if it falls outside the layer. The caller halves
+// ipx/ipy/radius between layers (src/lib/rendering/RenderForward.cu:856,888-891); rintf is round-half-even like
+// __float2int_rn.
+__device__ __forceinline__ bool layer_tile_pixel(const LayerTable& ly, int l, float ipx, float ipy, uint32_t& tile,
+                                                 uint32_t& in_tile)
 {
     const float fx = rintf(ipx), fy = rintf(ipy);
-    if (!(fx >= 0.f && fx < (float)ly.w[l] && fy >= 0.f && fy < (float)ly.h[l])) return -1;
-    return (int64_t)ly.base[l] + (int64_t)(int)fy * ly.w[l] + (int)fx;
+    if (!(fx >= 0.f && fx < (float)ly.w[l] && fy >= 0.f && fy < (float)ly.h[l])) return false;
+    const uint32_t x = (uint32_t)(int)fx, y = (uint32_t)(int)fy;
+    tile    = ly.tile_base[l] + (y / kTile) * (uint32_t)ly.tiles_x[l] + x / kTile;
+    in_tile = (y % kTile) * kTile + x % kTile;
+    return true;
+}
+
+// Bin and pixel-in-bin of a pixel given as (tile, pixel in tile) of layer l.
+__device__ __forceinline__ void bin_of_pixel(const LayerTable& ly, int l, uint32_t tile, uint32_t in_tile, uint32_t& bin,
+                                             uint32_t& in_bin)
+{
+    const uint32_t in_layer = (tile - ly.tile_base[l]) * kTilePixels + in_tile;
+    bin    = ly.bin_base[l] + (in_layer >> ly.bin_shift[l]);
+    in_bin = in_layer & ((1u << ly.bin_shift[l]) - 1u);
+}
+
+// Pixel number of layer l for a projected point, or -1.
+__device__ __forceinline__ int64_t layer_pixel(const LayerTable& ly, int l, float ipx, float ipy)
+{
+    uint32_t tile, in_tile;
+    if (!layer_tile_pixel(ly, l, ipx, ipy, tile, in_tile)) return -1;
+    return (int64_t)tile * kTilePixels + in_tile;
 }
 
 __device__ __forceinline__ int layer_of_pixel(const LayerTable& ly, uint32_t q)
@@ -107,15 +143,24 @@ __device__ __forceinline__ int layer_of_pixel(const LayerTable& ly, uint32_t q)
     return l;
 }
 
-// Workgroup -> pixel mapping of the per-pixel kernels (blend, backward). A workgroup owns a 16x16 pixel tile (a wave
-// 16x4 of it), because the fragments of neighbouring pixels come from the same few 256-point blocks of the cloud and
-// their descriptor records then share cache lines. The same point shows up once per layer, in the tiles that cover the
-// same part of the screen, so the tiles are grouped into screen regions: a region is one tile of the coarsest layer plus
-// the 4, 16, 64 ... tiles of the finer layers over the same area, and is walked coarsest layer first. Workgroups are
-// dealt round-robin to the 8 XCDs (each with its own L2), so workgroup b belongs to XCD b % 8 and takes slot b / 8 of
-// that XCD's run of regions (region r goes to XCD r % 8): what one layer's tiles pulled into the XCD's L2 is still there
+// Value the other lane of a pair (lane ^ 1) holds: a DPP register move (quad_perm [1,0,3,2]). Every lane of the wave
+// must be active. Used to let two neighbouring lanes fetch or store the two 16-byte halves of ONE 32-byte record with
+// one instruction: the memory pipeline then sees one 32-byte request per record instead of two 16-byte ones.
+__device__ __forceinline__ int pair_other(int v) { return __builtin_amdgcn_update_dpp(0, v, 0xB1, 0xF, 0xF, false); }
+__device__ __forceinline__ float pair_other(float v) { return __int_as_float(pair_other(__float_as_int(v))); }
+__device__ __forceinline__ float4 pair_other(float4 v)
+{
+    return make_float4(pair_other(v.x), pair_other(v.y), pair_other(v.z), pair_other(v.w));
+}
+
+// Workgroup -> tile mapping of the per-pixel kernels (blend, backward): a workgroup owns a tile, a wave 16x4 pixels of
+// it, because the fragments of neighbouring pixels come from the same few 256-point blocks of the cloud and their
+// descriptor records then share cache lines. The same point shows up once per layer, in the tiles that cover the same
+// part of the screen, so the tiles are grouped into screen regions: a region is one tile of the coarsest layer plus the
+// 4, 16, 64 ... tiles of the finer layers over the same area, and is walked coarsest layer first. Workgroups are dealt
+// round-robin to the 8 XCDs (each with its own L2), so workgroup b belongs to XCD b % 8 and takes slot b / 8 of that
+// XCD's run of regions (region r goes to XCD r % 8): what one layer's tiles pulled into the XCD's L2 is still there
 // when the next layer's tiles of the region ask for the same points.
-constexpr int kTile = 16;
 constexpr int kXcds = 8;
 struct TileMap
 {
@@ -127,10 +172,10 @@ struct TileMap
 
 struct TilePixel
 {
-    bool active;
+    bool active;     // the pixel lies inside the layer
     int l, x, y;
     uint32_t q;      // pixel number over all layers
-    uint32_t local;  // y * w + x inside the layer
+    uint32_t local;  // y * w + x inside the layer: index into the image planes
 };
 
 __device__ __forceinline__ TilePixel tile_pixel(const TileMap& tm, const LayerTable& ly)
@@ -157,11 +202,12 @@ __device__ __forceinline__ TilePixel tile_pixel(const TileMap& tm, const LayerTa
     const uint32_t ry = region / tm.regions_x, rx = region - ry * tm.regions_x;
     const uint32_t ty = ry * side + t / side, tx = rx * side + (t & (side - 1));
     r.l = l;
+    if (tx >= (uint32_t)ly.tiles_x[l] || ty >= (uint32_t)ly.tiles_y[l]) return r;
     r.x = (int)(tx * kTile + (threadIdx.x & (kTile - 1)));
     r.y = (int)(ty * kTile + (threadIdx.x / kTile));
+    r.q = (ly.tile_base[l] + ty * (uint32_t)ly.tiles_x[l] + tx) * kTilePixels + threadIdx.x;
     if (r.x >= ly.w[l] || r.y >= ly.h[l]) return r;
     r.local  = (uint32_t)r.y * (uint32_t)ly.w[l] + (uint32_t)r.x;
-    r.q      = ly.base[l] + r.local;
     r.active = true;
     return r;
 }

@@ -114,35 +114,64 @@ __device__ __forceinline__ bool point_is_skipped(const ViewPass& a, int i)
     return false;
 }
 
-// Project every point and count it in the pixel it rounds to, in every layer. The returning atomic hands each
-// (point, layer) its arrival rank inside the pixel, which the fill pass turns into a buffer position without a second
-// atomic. Counterpart of CountingPrepassMulti<L,false> (src/lib/rendering/RenderForward.cu:806-905).
-//
-// Global atomics are the scarce resource here (MI355X retires about 26 G of them per second whatever their scope,
-// return mode or address spread), and VET hands over clouds in Morton order with 256-point blocks
-// (src/lib/data/SceneData.cpp:105-106), so the 256 points of a workgroup fall into few pixels of the coarse layers.
-// The workgroup therefore first counts its (pixel, layer) hits in an LDS hash table (LDS atomics), then issues ONE
-// global atomic per distinct pixel for the whole group, and every point's rank is group base + rank inside the group.
-constexpr int kCountTableBits = 11;  // 2048 entries for at most 256 points x 5 layers: load factor <= 0.63
-constexpr int kCountTable     = 1 << kCountTableBits;
-constexpr uint32_t kEmptyKey  = 0xFFFFFFFFu;
+// ---- binning ---------------------------------------------------------------------------------------------------------
+// The reference counts every (point, layer) hit with one global atomic on its pixel, fills the lists with a second one
+// (CountingPrepassMulti / CollectMulti, src/lib/rendering/RenderForward.cu:806-905,1011-1096) and then sorts every
+// list. MI355X retires about 26 G global atomics per second whatever their scope, return mode or address spread, and at
+// the fine layers nearly every fragment has a pixel of its own, so per-pixel atomics alone would cost more than the
+// rest of the forward pass. The lists are therefore built in two levels:
+//   1. bin_count_kernel: fragments per BIN, a run of 256 / 64 / 16 / 4 consecutive pixel numbers (a 16x16 tile or a
+//      piece of one; the denser the layer, the smaller its bins). VET hands over clouds in Morton order with 256-point
+//      blocks (src/lib/data/SceneData.cpp:105-106), so the 64 points of a wave fall into a handful of bins per layer:
+//      the wave groups its hits by bin with ballots and issues one returning atomic per distinct bin, which also gives
+//      every hit its arrival rank inside the bin.
+//   2. exclusive scan over the bin counts.
+//   3. bin_fill_kernel: second projection; the fragment record goes to bin start + rank: a bin's records are contiguous.
+//   4. bin_build_kernel: one workgroup per bin counts the pixels, scans them, scatters the keys and sorts the lists, all
+//      in LDS. Pixels are numbered tile by tile, so the scan of the bin counts IS the start of every bin's lists and no
+//      scan over the pixels is needed.
 
-__global__ void __launch_bounds__(kBlock) count_kernel(ViewPass a, uint32_t* __restrict__ counts,
-                                                        uint32_t* __restrict__ slots)
+// Per-lane grouping of equal bin numbers inside a wave: leader = lowest lane with the same bin, rank = number of
+// lower lanes with the same bin, count = size of the group. Pure ballots, no memory traffic.
+struct WaveGroup
 {
-    __shared__ uint32_t t_key[kCountTable];
-    __shared__ uint32_t t_val[kCountTable];  // hits of the group in the pixel, then the group's base rank
-    for (int e = threadIdx.x; e < kCountTable; e += kBlock)
-    {
-        t_key[e] = kEmptyKey;
-        t_val[e] = 0u;
-    }
-    __syncthreads();
+    int leader;
+    uint32_t rank, count;
+};
 
-    const int i = blockIdx.x * blockDim.x + threadIdx.x;
-    uint32_t entry[VETRAST_MAX_LAYERS], rank[VETRAST_MAX_LAYERS];
+__device__ __forceinline__ WaveGroup group_by_bin(bool has, uint32_t bin, int lane)
+{
+    WaveGroup g;
+    g.leader = lane;
+    g.rank = g.count = 0;
+    const uint64_t lanes_below = (1ull << lane) - 1ull;
+    uint64_t todo = __ballot(has);
+    while (todo != 0ull)
+    {
+        const int first        = __ffsll((unsigned long long)todo) - 1;
+        const uint32_t b_first = (uint32_t)__shfl((int)bin, first, kWave);
+        const bool mine        = has && bin == b_first;
+        const uint64_t same    = __ballot(mine);
+        if (mine)
+        {
+            g.leader = first;
+            g.rank   = (uint32_t)__popcll(same & lanes_below);
+            g.count  = (uint32_t)__popcll(same);
+        }
+        todo &= ~same;
+    }
+    return g;
+}
+
+__global__ void __launch_bounds__(kBlock) bin_count_kernel(ViewPass a, uint32_t* __restrict__ bin_counts,
+                                                            uint32_t* __restrict__ slots)
+{
+    const int i    = blockIdx.x * blockDim.x + threadIdx.x;
+    const int lane = threadIdx.x & (kWave - 1);
+    bool has[VETRAST_MAX_LAYERS];
+    uint32_t bin[VETRAST_MAX_LAYERS];
 #pragma unroll
-    for (int l = 0; l < VETRAST_MAX_LAYERS; ++l) entry[l] = kEmptyKey;
+    for (int l = 0; l < VETRAST_MAX_LAYERS; ++l) has[l] = false, bin[l] = 0;
     Projected p;
     if (i < a.N && !point_is_skipped(a, i) && project_point(*a.view, a.position[i], p))
     {
@@ -152,37 +181,37 @@ __global__ void __launch_bounds__(kBlock) count_kernel(ViewPass a, uint32_t* __r
         {
             if (l >= a.ly.L) break;
             if (a.drop_by_radius && radius < a.radius_threshold) break;
-            const int64_t q64 = layer_pixel(a.ly, l, ipx, ipy);
-            if (q64 < 0) continue;
-            const uint32_t q = (uint32_t)q64;
-            uint32_t h       = (q * 2654435761u) >> (32 - kCountTableBits);
-            while (true)  // linear probing; the table can never fill up
-            {
-                const uint32_t old = atomicCAS(&t_key[h], kEmptyKey, q);
-                if (old == kEmptyKey || old == q) break;
-                h = (h + 1) & (kCountTable - 1);
-            }
-            entry[l] = h;
-            rank[l]  = atomicAdd(&t_val[h], 1u);
+            uint32_t tile, in_tile, in_bin;
+            has[l] = layer_tile_pixel(a.ly, l, ipx, ipy, tile, in_tile);
+            if (has[l]) bin_of_pixel(a.ly, l, tile, in_tile, bin[l], in_bin);
         }
     }
-    __syncthreads();
-    for (int e = threadIdx.x; e < kCountTable; e += kBlock)
-    {
-        const uint32_t q = t_key[e];
-        if (q != kEmptyKey) t_val[e] = atomicAdd(&counts[q], t_val[e]);
-    }
-    __syncthreads();
+    // group first, then all atomics of the wave at once (they are independent), then one wait
+    WaveGroup g[VETRAST_MAX_LAYERS];
+    uint32_t base[VETRAST_MAX_LAYERS];
 #pragma unroll
     for (int l = 0; l < VETRAST_MAX_LAYERS; ++l)
-        if (entry[l] != kEmptyKey) slots[(size_t)l * a.N + i] = t_val[entry[l]] + rank[l];
+    {
+        base[l] = 0;
+        if (l < a.ly.L) g[l] = group_by_bin(has[l], bin[l], lane);
+    }
+#pragma unroll
+    for (int l = 0; l < VETRAST_MAX_LAYERS; ++l)
+        if (l < a.ly.L && has[l] && g[l].leader == lane) base[l] = atomicAdd(&bin_counts[bin[l]], g[l].count);
+#pragma unroll
+    for (int l = 0; l < VETRAST_MAX_LAYERS; ++l)
+    {
+        if (l >= a.ly.L) break;
+        const uint32_t group_base = (uint32_t)__shfl((int)base[l], g[l].leader, kWave);
+        if (has[l]) slots[(size_t)l * a.N + i] = group_base + g[l].rank;
+    }
 }
 
-// ---- exclusive scan of the per-pixel counts, in place, in two launches -------------------------------------------
+// ---- exclusive scan of the per-tile counts, in place, in two launches --------------------------------------------
 // Launch 1: one partial sum per 4096 counts. Launch 2: every workgroup adds up the partials in front of it (a few
 // hundred values, cache resident), then scans its own 4096 counts. No workgroup waits for another one.
 // Counterpart of thrust::exclusive_scan + the two .item<int>() read-backs (src/lib/rendering/PointRenderer.cu:799-813);
-// the total lands at counts[P] because the array is zero padded behind P.
+// the total lands at counts[T] because the array is zero padded behind the T tile counts.
 __device__ __forceinline__ uint32_t wave_inclusive_scan(uint32_t v, int lane)
 {
 #pragma unroll
@@ -263,27 +292,71 @@ __global__ void __launch_bounds__(kBlock) scan_apply_kernel(uint4* __restrict__ 
     }
 }
 
-// Second projection of every point; writes its 64-bit record (depth bits, point id) at scan[pixel] + rank.
-// Counterpart of CollectMulti<L,false> (src/lib/rendering/RenderForward.cu:1011-1096), which draws the rank from a
-// second atomic counter image and stores depth and id in two separate rows.
-__global__ void __launch_bounds__(kBlock) fill_kernel(ViewPass a, const uint32_t* __restrict__ offsets,
-                                                       const uint32_t* __restrict__ slots,
-                                                       uint64_t* __restrict__ fragments, uint32_t capacity)
+// The same scan in one launch by one workgroup of 1024 threads, for up to 16 K counts (a 1080p frame has some ten
+// thousand bins): thread t owns the 16 consecutive counts [16 t, 16 t + 16). The array is zero padded to a multiple of
+// 4096 counts, so whole uint4 loads never leave it.
+constexpr int kScanSmallBlock = 1024;
+constexpr int kScanSmallMax   = kScanSmallBlock * kScanPerThread;
+
+__global__ void __launch_bounds__(kScanSmallBlock) scan_small_kernel(uint4* __restrict__ counts4, uint32_t n)
+{
+    __shared__ uint32_t wave_tot[kScanSmallBlock / kWave];
+    const bool mine_any = (uint32_t)threadIdx.x * kScanPerThread < n;
+    uint4* mine         = counts4 + threadIdx.x * (kScanPerThread / 4);
+    uint4 v[kScanPerThread / 4];
+    uint32_t sum = 0;
+#pragma unroll
+    for (int k = 0; k < kScanPerThread / 4; ++k)
+    {
+        v[k] = mine_any ? mine[k] : make_uint4(0u, 0u, 0u, 0u);
+        sum += (v[k].x + v[k].y) + (v[k].z + v[k].w);
+    }
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    const uint32_t incl = wave_inclusive_scan(sum, lane);
+    if (lane == kWave - 1) wave_tot[wave] = incl;
+    __syncthreads();
+    uint32_t run = incl - sum;
+    for (int k = 0; k < wave; ++k) run += wave_tot[k];
+    if (!mine_any) return;
+#pragma unroll
+    for (int k = 0; k < kScanPerThread / 4; ++k)
+    {
+        uint4 o;
+        o.x = run;
+        run += v[k].x;
+        o.y = run;
+        run += v[k].y;
+        o.z = run;
+        run += v[k].z;
+        o.w = run;
+        run += v[k].w;
+        mine[k] = o;
+    }
+}
+
+// Second projection of every point; its record (64-bit key = depth bits << 32 | point id, pixel inside the bin) goes
+// to the bin's start + the rank the count pass drew. Counterpart of CollectMulti<L,false>
+// (src/lib/rendering/RenderForward.cu:1011-1096), which draws the rank from a second atomic counter image and stores
+// depth and id in two separate rows.
+__global__ void __launch_bounds__(kBlock) bin_fill_kernel(ViewPass a, const uint32_t* __restrict__ bin_offsets,
+                                                           const uint32_t* __restrict__ slots,
+                                                           uint4* __restrict__ binned, uint32_t capacity)
 {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= a.N) return;
     if (point_is_skipped(a, i)) return;
     Projected p;
     if (!project_point(*a.view, a.position[i], p)) return;
-    const uint64_t key = ((uint64_t)__float_as_uint(p.z) << 32) | (uint32_t)i;
+    const uint32_t depth_bits = __float_as_uint(p.z);
     float ipx = p.ipx, ipy = p.ipy, radius = p.radius;
     for (int l = 0; l < a.ly.L; ++l, radius *= 0.5f, ipx *= 0.5f, ipy *= 0.5f)
     {
         if (a.drop_by_radius && radius < a.radius_threshold) break;
-        const int64_t q = layer_pixel(a.ly, l, ipx, ipy);
-        if (q < 0) continue;
-        const uint32_t pos = offsets[q] + slots[(size_t)l * a.N + i];
-        if (pos < capacity) fragments[pos] = key;  // always true when count and fill agree; guards the store
+        uint32_t tile, in_tile, bin, in_bin;
+        if (!layer_tile_pixel(a.ly, l, ipx, ipy, tile, in_tile)) continue;
+        bin_of_pixel(a.ly, l, tile, in_tile, bin, in_bin);
+        const uint32_t pos = bin_offsets[bin] + slots[(size_t)l * a.N + i];
+        if (pos < capacity) binned[pos] = make_uint4((uint32_t)i, depth_bits, in_bin, 0u);  // guard: never false
     }
 }
 

@@ -1,7 +1,7 @@
 // Per-pixel sort of the fragment lists by the 64-bit key (depth bits << 32 | point id), ascending, with the top-K cut.
 //
-// A wave owns 64 consecutive pixels; because the scan runs over the same pixel order their lists are one contiguous
-// stretch of the fragment buffer. Lists are grouped by padded power-of-two length m = 2,4,...,64 and 64/m lists are
+// A wave owns up to 64 consecutive pixels of a bin, whose lists are one contiguous stretch of the fragment buffer (or of
+// the bin's copy in LDS). Lists are grouped by padded power-of-two length m = 2,4,...,64 and 64/m lists are
 // sorted at a time by one bitonic network held in registers (one key per lane, partner exchange by lane shuffles).
 // Lists longer than 64 keep the K smallest keys with a streaming wave-wide selection, or are sorted in place in
 // global memory when no cut applies.
@@ -102,7 +102,7 @@ __device__ __forceinline__ uint64_t bitonic_merge64(uint64_t key, int lane)
 
 // Sort `count` lists of class LOG (2^(LOG-1) < n <= 2^LOG) found in the wave; src_lane[r] is the lane that owns the r-th.
 template <int LOG>
-__device__ __forceinline__ void sort_class(uint64_t* __restrict__ fragments, const uint8_t* src_lane, int count,
+__device__ __forceinline__ void sort_class(uint64_t* fragments, const uint8_t* src_lane, int count,
                                            uint32_t off, uint32_t n, int lane, int K)
 {
     constexpr int m        = 1 << LOG;
@@ -126,7 +126,7 @@ __device__ __forceinline__ void sort_class(uint64_t* __restrict__ fragments, con
 // K smallest keys (K <= 64) of a list longer than 64, sorted, written to its first K places. The wave keeps the 64
 // smallest keys seen so far in sorted order; a chunk of 64 further keys is looked at only if one of them beats the
 // current K-th smallest.
-__device__ __forceinline__ void select_smallest(uint64_t* __restrict__ list, uint32_t n, int lane, int K)
+__device__ __forceinline__ void select_smallest(uint64_t* list, uint32_t n, int lane, int K)
 {
     uint64_t best = list[lane];  // n > 64
     best          = bitonic_sort_groups<6>(best, lane);
@@ -188,43 +188,11 @@ __device__ __forceinline__ void sort_in_memory(uint64_t* list, uint32_t n, int l
     }
 }
 
-// How waves are dealt to pixels: layer l is served by waves [first_wave[l], first_wave[l+1]), each owning
-// pixels_per_wave[l] consecutive pixels (a power of two <= 64). Coarse layers carry the same number of fragments in far
-// fewer pixels, so they get fewer pixels per wave; otherwise a handful of waves would sort most of the frame alone.
-struct SortWaveMap
+// Sorts the lists of one wave: lane i holds the start `off` (an index into `fragments`) and the length `n` of its list
+// (n = 0 for lanes without a list). `fragments` may point to global memory or to LDS.
+__device__ __forceinline__ void sort_wave_lists(uint64_t* fragments, uint8_t* src_lane, uint32_t off, uint32_t n,
+                                                int lane, int K)
 {
-    int L;
-    uint32_t first_wave[VETRAST_MAX_LAYERS + 1];
-    uint32_t pixels_per_wave[VETRAST_MAX_LAYERS];
-    uint32_t pixel_base[VETRAST_MAX_LAYERS + 1];
-};
-
-__global__ void __launch_bounds__(kBlock) sort_lists_kernel(const uint32_t* __restrict__ offsets,
-                                                             uint64_t* __restrict__ fragments,
-                                                             uint8_t* __restrict__ list_is_cut, SortWaveMap map, int K)
-{
-    __shared__ uint8_t src_lane_all[kBlock / kWave][kWave];
-    const int lane    = threadIdx.x & (kWave - 1);
-    const int wave    = threadIdx.x / kWave;
-    uint8_t* src_lane = src_lane_all[wave];
-    const uint32_t gw = blockIdx.x * (kBlock / kWave) + wave;  // global wave number
-    int l             = 0;
-#pragma unroll
-    for (int k = 1; k < VETRAST_MAX_LAYERS; ++k)
-        if (k < map.L && gw >= map.first_wave[k]) l = k;
-    uint32_t off = 0, n = 0;
-    if (gw < map.first_wave[map.L] && (uint32_t)lane < map.pixels_per_wave[l])
-    {
-        const uint32_t q = map.pixel_base[l] + (gw - map.first_wave[l]) * map.pixels_per_wave[l] + lane;
-        if (q < map.pixel_base[l + 1])
-        {
-            off = offsets[q];
-            n   = offsets[q + 1] - off;
-            // one byte per pixel: does the top-K cut drop fragments here? The backward per-point kernel only has to look
-            // up the K-th key of a pixel where this is set (a few percent of the pixels at the fine layers).
-            list_is_cut[q] = (K > 0 && n > (uint32_t)K) ? 1 : 0;
-        }
-    }
     // class = ceil(log2(n)) for 2 <= n <= 64, 0 for n <= 1 (nothing to do), 7 for n > 64
     int cls = 0;
     if (n > 64)

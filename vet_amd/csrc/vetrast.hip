@@ -11,6 +11,7 @@
 #include "common.h"
 #include "forward_kernels.h"
 #include "sort_kernels.h"
+#include "build_kernels.h"
 #include "backward_kernels.h"
 
 using namespace vetrast;
@@ -91,22 +92,39 @@ inline int grid_for(size_t n, int block = kBlock)
     return (int)((n + block - 1) / block);
 }
 
-LayerTable make_layer_table(int w, int h, int L)
+// N only steers the bin sizes: N / pixels bounds the mean list length of a layer from above without any device read.
+LayerTable make_layer_table(int w, int h, int L, int64_t N)
 {
     LayerTable t;
     std::memset(&t, 0, sizeof(t));
-    t.L          = L;
-    uint32_t run = 0;
+    t.L           = L;
+    uint32_t tile = 0, bin = 0;
     for (int l = 0; l < L; ++l)
     {
-        t.w[l]    = w;
-        t.h[l]    = h;
-        t.base[l] = run;
-        run += (uint32_t)w * (uint32_t)h;
+        t.w[l]         = w;
+        t.h[l]         = h;
+        t.tiles_x[l]   = (w + kTile - 1) / kTile;
+        t.tiles_y[l]   = (h + kTile - 1) / kTile;
+        t.tile_base[l] = tile;
+        t.base[l]      = tile * kTilePixels;
+        const uint32_t tiles = (uint32_t)t.tiles_x[l] * (uint32_t)t.tiles_y[l];
+        tile += tiles;
+        // largest bin of 256, 64, 16 or 4 pixels expected to hold at most 1024 fragments
+        const double mean_len = (double)N / ((double)w * (double)h);
+        int shift             = 8;
+        while (shift > 2 && mean_len * (double)(1 << shift) > 1024.0) shift -= 2;
+        t.bin_shift[l] = shift;
+        t.bin_base[l]  = bin;
+        bin += tiles << (8 - shift);
         w /= 2;
         h /= 2;
     }
-    for (int l = L; l <= VETRAST_MAX_LAYERS; ++l) t.base[l] = run;
+    for (int l = L; l <= VETRAST_MAX_LAYERS; ++l)
+    {
+        t.tile_base[l] = tile;
+        t.base[l]      = tile * kTilePixels;
+        t.bin_base[l]  = bin;
+    }
     return t;
 }
 
@@ -118,7 +136,8 @@ int check_dims(int64_t N, int B, int L, int w, int h)
     if (N * L >= (int64_t)0xFFFFFFF0ll) return VETRAST_ERR_INVALID_ARG;
     int64_t P = 0;
     int lw = w, lh = h;
-    for (int l = 0; l < L; ++l, lw /= 2, lh /= 2) P += (int64_t)lw * lh;
+    for (int l = 0; l < L; ++l, lw /= 2, lh /= 2)
+        P += (int64_t)((lw + kTile - 1) / kTile) * ((lh + kTile - 1) / kTile) * kTilePixels;
     if (P + kScanPerBlock >= (int64_t)0x7FFFFFFFll) return VETRAST_ERR_INVALID_ARG;
     return VETRAST_OK;
 }
@@ -161,33 +180,6 @@ template <class T>
 inline T* ws_ptr(void* ws, size_t off)
 {
     return reinterpret_cast<T*>(static_cast<char*>(ws) + off);
-}
-
-// Pixels per wave in the sort: about 128 fragments per wave if every point were visible in the layer (N / pixels is an
-// upper bound of the mean list length that needs no device read-back), between 4 and 64, a power of two.
-SortWaveMap make_sort_wave_map(const LayerTable& ly, int N)
-{
-    SortWaveMap m;
-    std::memset(&m, 0, sizeof(m));
-    m.L           = ly.L;
-    uint32_t wave = 0;
-    for (int l = 0; l < ly.L; ++l)
-    {
-        const uint32_t pixels = (uint32_t)ly.w[l] * (uint32_t)ly.h[l];
-        const double mean_len = (double)N / (double)pixels;
-        uint32_t ppw          = 64;
-        while (ppw > 4 && mean_len * ppw > 128.0) ppw >>= 1;
-        m.first_wave[l]      = wave;
-        m.pixels_per_wave[l] = ppw;
-        m.pixel_base[l]      = ly.base[l];
-        wave += (pixels + ppw - 1) / ppw;
-    }
-    for (int l = ly.L; l <= VETRAST_MAX_LAYERS; ++l)
-    {
-        m.first_wave[l] = wave;
-        m.pixel_base[l] = ly.base[ly.L];
-    }
-    return m;
 }
 
 TileMap make_tile_map(const LayerTable& ly)
@@ -282,25 +274,37 @@ int vetrast_workspace_layout_for(int32_t N, int32_t B, int32_t L, int32_t w, int
     int st = check_dims(N, B, L, w, h);
     if (st != VETRAST_OK) return st;
     std::memset(lay, 0, sizeof(*lay));
-    LayerTable t = make_layer_table(w, h, L);
+    LayerTable t = make_layer_table(w, h, L, N);
     for (int l = 0; l < L; ++l)
     {
         lay->layer_w[l] = t.w[l];
         lay->layer_h[l] = t.h[l];
     }
-    for (int l = 0; l <= VETRAST_MAX_LAYERS; ++l) lay->layer_pixel_base[l] = t.base[l < L ? l : L];
+    for (int l = 0; l < L; ++l) lay->layer_tiles_x[l] = t.tiles_x[l];
+    for (int l = 0; l <= VETRAST_MAX_LAYERS; ++l)
+    {
+        lay->layer_tile_base[l]  = t.tile_base[l < L ? l : L];
+        lay->layer_pixel_base[l] = t.base[l < L ? l : L];
+    }
     const size_t P         = t.base[L];
-    const size_t Ppad      = align_up(P + 1, kScanPerBlock);
+    const size_t bins      = t.bin_base[L];
+    const size_t Tpad      = align_up(bins + 1, kScanPerBlock);
+    lay->num_bins          = (int64_t)bins;
     const size_t cap       = (size_t)N * L;
     lay->fragment_capacity = (int64_t)cap;
     size_t at              = 0;
     lay->flags_base        = at;
     at += kAlign;
-    lay->offsets_base   = at;
-    lay->offsets_stride = Ppad * sizeof(uint32_t);
-    at += lay->offsets_stride * B;
+    lay->bin_counts_base   = at;
+    lay->bin_counts_stride = Tpad * sizeof(uint32_t);
+    at += lay->bin_counts_stride * B;
     lay->scan_partials_base = at;
-    at += align_up((Ppad / kScanPerBlock) * sizeof(uint32_t), kAlign);
+    at += align_up((Tpad / kScanPerBlock) * sizeof(uint32_t), kAlign);
+    lay->offsets_base   = at;
+    lay->offsets_stride = align_up((P + 1) * sizeof(uint32_t), kAlign);
+    at += lay->offsets_stride * B;
+    lay->binned_base = at;
+    at += align_up(cap * sizeof(uint4), kAlign);
     lay->views_base = at;
     at += align_up((size_t)B * sizeof(DeviceView), kAlign);
     lay->packed_base = at;
@@ -347,10 +351,11 @@ int vetrast_forward(vetrast_ctx* ctx, const vetrast_forward_args* a, void* strea
     hipStream_t stream      = (hipStream_t)stream_;
     const vetrast_params& p = a->params;
     const int N = a->num_points, B = a->num_views, L = p.num_layers, C = p.num_texture_channels;
-    const LayerTable ly = make_layer_table(a->views[0].w, a->views[0].h, L);
+    const LayerTable ly = make_layer_table(a->views[0].w, a->views[0].h, L, N);
     const TileMap tiles = make_tile_map(ly);
     const uint32_t P    = ly.base[L];
-    const size_t Ppad   = lay.offsets_stride / sizeof(uint32_t);
+    const uint32_t bins = ly.bin_base[L];
+    const size_t Tpad   = lay.bin_counts_stride / sizeof(uint32_t);
     void* ws            = a->workspace;
     uint32_t* flags     = ws_ptr<uint32_t>(ws, lay.flags_base);
     float4* packed      = ws_ptr<float4>(ws, lay.packed_base);
@@ -360,9 +365,9 @@ int vetrast_forward(vetrast_ctx* ctx, const vetrast_forward_args* a, void* strea
 
     {
         ScopeTimer tm(ctx, stream, VETRAST_SCOPE_PREPARE);
-        // per-pixel counters of all views (contiguous) start at zero; InitializeData, PointRenderer.cu:402-470
-        const size_t n4  = Ppad * B / 4;
-        uint4* counters4 = ws_ptr<uint4>(ws, lay.offsets_base);
+        // per-bin counters of all views (contiguous) start at zero; InitializeData, PointRenderer.cu:402-470
+        const size_t n4  = Tpad * B / 4;
+        uint4* counters4 = ws_ptr<uint4>(ws, lay.bin_counts_base);
         if (N == 0)
             hipLaunchKernelGGL(fill_u128_kernel, dim3(std::min(grid_for(n4), 4096)), dim3(kBlock), 0, stream, counters4,
                                n4, 0u);
@@ -404,33 +409,46 @@ int vetrast_forward(vetrast_ctx* ctx, const vetrast_forward_args* a, void* strea
         uint64_t* fragments = ws_ptr<uint64_t>(ws, lay.fragments_base + lay.fragments_stride * b);
         float* trans        = ws_ptr<float>(ws, lay.transmittance_base + lay.transmittance_stride * b);
         float* weight       = ws_ptr<float>(ws, lay.weight_base + lay.weight_stride * b);
+        uint32_t* bin_counts     = ws_ptr<uint32_t>(ws, lay.bin_counts_base + lay.bin_counts_stride * b);
+        uint4* binned            = ws_ptr<uint4>(ws, lay.binned_base);
+        uint8_t* list_is_cut     = ws_ptr<uint8_t>(ws, lay.cut_flags_base + lay.cut_flags_stride * b);
         if (N > 0)
         {
             ScopeTimer tm(ctx, stream, VETRAST_SCOPE_COUNT);
-            hipLaunchKernelGGL(count_kernel, dim3(grid_for(N)), dim3(kBlock), 0, stream, vp, offsets, slots);
+            hipLaunchKernelGGL(bin_count_kernel, dim3(grid_for(N)), dim3(kBlock), 0, stream, vp, bin_counts, slots);
         }
         {
             ScopeTimer tm(ctx, stream, VETRAST_SCOPE_SCAN);
-            const int blocks = (int)(Ppad / kScanPerBlock);
-            hipLaunchKernelGGL(scan_partials_kernel, dim3(blocks), dim3(kBlock), 0, stream,
-                               reinterpret_cast<const uint4*>(offsets), partials);
-            hipLaunchKernelGGL(scan_apply_kernel, dim3(blocks), dim3(kBlock), 0, stream,
-                               reinterpret_cast<uint4*>(offsets), partials);
+            if (bins + 1 <= (uint32_t)kScanSmallMax)
+                hipLaunchKernelGGL(scan_small_kernel, dim3(1), dim3(kScanSmallBlock), 0, stream,
+                                   reinterpret_cast<uint4*>(bin_counts), bins + 1);
+            else
+            {
+                const int blocks = (int)(Tpad / kScanPerBlock);
+                hipLaunchKernelGGL(scan_partials_kernel, dim3(blocks), dim3(kBlock), 0, stream,
+                                   reinterpret_cast<const uint4*>(bin_counts), partials);
+                hipLaunchKernelGGL(scan_apply_kernel, dim3(blocks), dim3(kBlock), 0, stream,
+                                   reinterpret_cast<uint4*>(bin_counts), partials);
+            }
         }
         if (N > 0)
         {
             ScopeTimer tm(ctx, stream, VETRAST_SCOPE_FILL);
-            hipLaunchKernelGGL(fill_kernel, dim3(grid_for(N)), dim3(kBlock), 0, stream, vp, offsets, slots, fragments,
+            hipLaunchKernelGGL(bin_fill_kernel, dim3(grid_for(N)), dim3(kBlock), 0, stream, vp, bin_counts, slots, binned,
                                (uint32_t)lay.fragment_capacity);
         }
-        if (N > 0)
         {
-            ScopeTimer tm(ctx, stream, VETRAST_SCOPE_SORT);
-            const SortWaveMap map = make_sort_wave_map(ly, N);
-            hipLaunchKernelGGL(sort_lists_kernel, dim3((map.first_wave[L] + kBlock / kWave - 1) / (kBlock / kWave)),
-                               dim3(kBlock), 0, stream, offsets, fragments,
-                               ws_ptr<uint8_t>(ws, lay.cut_flags_base + lay.cut_flags_stride * b), map,
-                               p.debug_max_list_length);
+            ScopeTimer tm(ctx, stream, VETRAST_SCOPE_BUILD);
+            BuildPass bp;
+            bp.bin_offsets   = bin_counts;
+            bp.binned        = binned;
+            bp.offsets       = offsets;
+            bp.fragments     = fragments;
+            bp.list_is_cut   = list_is_cut;
+            bp.ly            = ly;
+            bp.num_bins      = bins;
+            bp.K             = p.debug_max_list_length;
+            hipLaunchKernelGGL(bin_build_kernel, dim3(bins), dim3(kBlock), 0, stream, bp);
         }
         {
             ScopeTimer tm(ctx, stream, VETRAST_SCOPE_BLEND);
@@ -490,7 +508,7 @@ int vetrast_backward(vetrast_ctx* ctx, const vetrast_backward_args* g, void* str
         if (!g->grad_out[l]) return VETRAST_ERR_INVALID_ARG;
     hipStream_t stream = (hipStream_t)stream_;
     const int N = a->num_points, B = a->num_views, L = p.num_layers, C = p.num_texture_channels;
-    const LayerTable ly = make_layer_table(a->views[0].w, a->views[0].h, L);
+    const LayerTable ly = make_layer_table(a->views[0].w, a->views[0].h, L, N);
     const TileMap tiles = make_tile_map(ly);
     const uint32_t P    = ly.base[L];
     void* ws            = a->workspace;
@@ -702,7 +720,7 @@ const char* vetrast_scope_name(int32_t scope)
         case VETRAST_SCOPE_COUNT: return "CountingPass";
         case VETRAST_SCOPE_SCAN: return "CreateAndAllocateBuffers";
         case VETRAST_SCOPE_FILL: return "CollectionPass";
-        case VETRAST_SCOPE_SORT: return "SortingPass";
+        case VETRAST_SCOPE_BUILD: return "CollectionPass (per-pixel lists) + SortingPass";
         case VETRAST_SCOPE_BLEND: return "BlendingPass";
         case VETRAST_SCOPE_BACKWARD_PREPARE: return "Prepare Backward";
         case VETRAST_SCOPE_BACKWARD_BLEND: return "BlendBackwards";

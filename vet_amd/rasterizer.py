@@ -77,29 +77,74 @@ class ForwardResult:
         raw = self.workspace[base + stride * b: base + stride * b + nbytes]
         return raw.view(dtype)
 
-    def total_pixels(self):
-        return int(self.layout.layer_pixel_base[self.args.params.num_layers])
+    # The workspace numbers pixels tile by tile (16x16 tiles, see include/vetrast.h). The accessors below hand the lists
+    # back in image order instead: layer after layer, row-major inside a layer, which is the order a reader expects and
+    # the order the CPU check uses.
+    def num_layers(self):
+        return int(self.args.params.num_layers)
 
-    def offsets(self, b=0):
-        """int64 numpy copy of the exclusive scan [P+1] of view b."""
-        P = self.total_pixels()
-        t = self._view_array(self.layout.offsets_base, self.layout.offsets_stride, b, torch.int32, P + 1)
+    def layer_bases(self):
+        """Image-order pixel number of the first pixel of every layer, plus the total."""
+        lay, run, bases = self.layout, 0, []
+        for l in range(self.num_layers()):
+            bases.append(run)
+            run += int(lay.layer_w[l]) * int(lay.layer_h[l])
+        return bases + [run]
+
+    def total_pixels(self):
+        return self.layer_bases()[-1]
+
+    def device_pixels(self):
+        return int(self.layout.layer_pixel_base[self.num_layers()])
+
+    def pixel_map(self):
+        """int64 [total_pixels]: workspace pixel number of every image-order pixel."""
+        if getattr(self, "_pixel_map", None) is None:
+            lay, parts = self.layout, []
+            for l in range(self.num_layers()):
+                w, h = int(lay.layer_w[l]), int(lay.layer_h[l])
+                y, x = np.meshgrid(np.arange(h, dtype=np.int64), np.arange(w, dtype=np.int64), indexing="ij")
+                tile = int(lay.layer_tile_base[l]) + (y // 16) * int(lay.layer_tiles_x[l]) + x // 16
+                parts.append((tile * 256 + (y % 16) * 16 + x % 16).reshape(-1))
+            self._pixel_map = np.concatenate(parts)
+        return self._pixel_map
+
+    def device_offsets(self, b=0):
+        """int64 numpy copy of the list starts [device_pixels + 1] of view b, in workspace pixel order."""
+        t = self._view_array(self.layout.offsets_base, self.layout.offsets_stride, b, torch.int32,
+                             self.device_pixels() + 1)
         return t.cpu().numpy().astype(np.int64) & 0xFFFFFFFF
 
+    def _gather_index(self, b):
+        """(image-order exclusive scan [P+1], workspace position of every fragment in image order)."""
+        dev = self.device_offsets(b)
+        m = self.pixel_map()
+        counts = dev[m + 1] - dev[m]
+        off = np.concatenate([[0], np.cumsum(counts)]).astype(np.int64)
+        src = np.repeat(dev[m] - off[:-1], counts) + np.arange(off[-1], dtype=np.int64)
+        return off, src
+
+    def offsets(self, b=0):
+        """int64 exclusive scan [P+1] of the per-pixel fragment counts of view b, image order."""
+        return self._gather_index(b)[0]
+
     def fragments(self, b=0):
-        """uint64 numpy copy of the fragment buffer of view b, cut to the number of fragments."""
-        total = int(self.offsets(b)[-1])
-        t = self._view_array(self.layout.fragments_base, self.layout.fragments_stride, b, torch.int64, total)
-        return t.cpu().numpy().view(np.uint64)
+        """uint64 fragment keys of view b, the lists concatenated in image order."""
+        _, src = self._gather_index(b)
+        t = self._view_array(self.layout.fragments_base, self.layout.fragments_stride, b, torch.int64,
+                             int(self.layout.fragment_capacity))
+        return t.cpu().numpy().view(np.uint64)[src]
 
     def transmittance(self, b=0):
-        total = int(self.offsets(b)[-1])
-        return self._view_array(self.layout.transmittance_base, self.layout.transmittance_stride, b, torch.float32,
-                                total).cpu().numpy()
+        _, src = self._gather_index(b)
+        t = self._view_array(self.layout.transmittance_base, self.layout.transmittance_stride, b, torch.float32,
+                             int(self.layout.fragment_capacity))
+        return t.cpu().numpy()[src]
 
     def weight(self, b=0):
-        return self._view_array(self.layout.weight_base, self.layout.weight_stride, b, torch.float32,
-                                self.total_pixels()).cpu().numpy()
+        t = self._view_array(self.layout.weight_base, self.layout.weight_stride, b, torch.float32,
+                             self.device_pixels())
+        return t.cpu().numpy()[self.pixel_map()]
 
 
 class DeviceScene:
