@@ -35,8 +35,9 @@ def algorithmic_bytes(N, P, F, Fk, Cn):
         # the model's terms, booked on the kernels that do the corresponding work here
         "COUNT": 16 * N,                              # positions read
         "FILL": 16 * N + 8 * F,                       # positions read again, fragment records written
-        "BUILD": 4 * P + 8 * P + 16 * F,              # per-pixel counts, counts -> offsets, records read and written sorted
-        "BLEND": 8 * Fk + (4 * Cn + 4) * Fk + 4 * P + 4 * Cn * P + 4 * P,  # lists, descriptor+confidence, offsets, out, weight
+        # per-pixel counts, counts -> offsets, records read and written sorted; then the blend: lists, descriptor +
+        # confidence, offsets, out, weight
+        "BUILD": 4 * P + 8 * P + 16 * F + 8 * Fk + (4 * Cn + 4) * Fk + 4 * P + 4 * Cn * P + 4 * P,
     }
     # The per-pixel kernel reads upstream grads and forward outputs (8CP), lists (8Fk), descriptor+confidence (4(C+1)Fk)
     # and writes one half of the gradient read-modify-write (4(C+1+4)Fk); the per-point kernel reads positions (16Fk in the

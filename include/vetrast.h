@@ -95,8 +95,7 @@ typedef enum vetrast_scope
     VETRAST_SCOPE_COUNT,            /* "CountingPass": fragments per bin (a 16x16 pixel tile or a piece of one) */
     VETRAST_SCOPE_SCAN,             /* "CreateAndAllocateBuffers" (prefix scan over the bins; no allocation here) */
     VETRAST_SCOPE_FILL,             /* "CollectionPass", first half: fragment records grouped by bin */
-    VETRAST_SCOPE_BUILD,            /* "CollectionPass" second half + "SortingPass": sorted per-pixel lists of every bin */
-    VETRAST_SCOPE_BLEND,            /* "BlendingPass" */
+    VETRAST_SCOPE_BUILD,            /* "CollectionPass" second half + "SortingPass" + "BlendingPass": one pass per bin */
     VETRAST_SCOPE_BACKWARD_PREPARE, /* "Prepare Backward": zero-fill of gradient buffers */
     VETRAST_SCOPE_BACKWARD_BLEND,   /* "BlendBackwards", per-pixel part */
     VETRAST_SCOPE_BACKWARD_GATHER,  /* "BlendBackwards", per-point sum of the stored fragment gradients */

@@ -12,8 +12,16 @@ namespace vetrast
 // holds for bins of up to kBuildCap records, which is what the bin sizes are chosen for. Bigger bins (far more points
 // in one place than the layer's average) stream their records twice from global memory instead and sort their lists in
 // place in the fragment buffer.
+//
+// A bin that was sorted in LDS is blended right there as well (BlendMulti, src/lib/rendering/RenderForward.cu:1303-1357):
+// all 256 threads gather the descriptor records of a stretch of kept fragments into an LDS stage (one independent
+// gather per lane), then the thread that owns a pixel walks its fragments of that stretch front to back in exactly the
+// reference's order: out += (T*c)*t, T = (1-c)*T. The transmittance in front of every fragment is parked in the high
+// half of its key in LDS (the depth bits have gone out to the fragment buffer by then) and written out coalesced.
+// Bins that did not fit are flagged and blended by blend_kernel.
 constexpr int kBuildPerThread = 8;
 constexpr int kBuildCap       = kBlock * kBuildPerThread;  // 2048 records = 16 KB of keys in LDS
+constexpr int kStage          = 256;                       // descriptor records staged per round (8 KB)
 
 struct BuildPass
 {
@@ -21,12 +29,24 @@ struct BuildPass
     const uint4* binned;
     uint32_t* offsets;    // [P + 1] per pixel: start of its list; [P] = fragments of the view
     uint64_t* fragments;
-    uint8_t* list_is_cut;    // [P]
+    uint8_t* list_is_cut;   // [P]
+    // blending
+    const int32_t* index;
+    const float4* packed;
+    const float* background;
+    float* transmittance;  // per fragment, null unless the backward pass will run
+    float* weight;         // per pixel
+    float* out[VETRAST_MAX_LAYERS];       // already offset to this view
+    float* out_mask[VETRAST_MAX_LAYERS];  // already offset to this view, or null
     LayerTable ly;
     uint32_t num_bins;
+    int N;
     int K;
+    int use_environment_map;
+    float mask_value;
 };
 
+template <int C>
 __global__ void __launch_bounds__(kBlock) bin_build_kernel(BuildPass a)
 {
     __shared__ uint32_t s_cnt[kTilePixels];
@@ -34,6 +54,8 @@ __global__ void __launch_bounds__(kBlock) bin_build_kernel(BuildPass a)
     __shared__ uint32_t s_wave_tot[kBlock / kWave];
     __shared__ uint8_t s_src_lane[kBlock / kWave][kWave];
     __shared__ uint64_t s_keys[kBuildCap];
+    __shared__ uint8_t s_pix[kBuildCap];       // pixel (inside the bin) of every list place
+    __shared__ float4 s_stage[kStage][2];      // descriptor, confidence of the staged fragments
     const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
     const uint32_t bin = a.num_bins - 1u - blockIdx.x;  // coarse layers first
     int l              = 0;
@@ -43,8 +65,9 @@ __global__ void __launch_bounds__(kBlock) bin_build_kernel(BuildPass a)
     const int shift       = a.ly.bin_shift[l];
     const uint32_t pixels = 1u << shift;  // pixels of this bin
     const uint32_t q0     = a.ly.base[l] + ((bin - a.ly.bin_base[l]) << shift);
-    const uint32_t begin  = a.bin_offsets[bin];
-    const uint32_t n      = a.bin_offsets[bin + 1] - begin;
+    // the same for every lane: tell the compiler, so that loops over the bin's records become scalar branches
+    const uint32_t begin  = (uint32_t)__builtin_amdgcn_readfirstlane((int)a.bin_offsets[bin]);
+    const uint32_t n      = (uint32_t)__builtin_amdgcn_readfirstlane((int)a.bin_offsets[bin + 1]) - begin;
     const uint4* recs     = a.binned + begin;
     const bool in_lds     = n <= (uint32_t)kBuildCap;
     s_cnt[tid] = 0u;
@@ -58,9 +81,14 @@ __global__ void __launch_bounds__(kBlock) bin_build_kernel(BuildPass a)
 #pragma unroll
         for (int k = 0; k < kBuildPerThread; ++k)
         {
+            where[k] = 0xFFFFFFFFu;
+            key[k]   = 0ull;
+        }
+#pragma unroll
+        for (int k = 0; k < kBuildPerThread; ++k)
+        {
+            if ((uint32_t)(k * kBlock) >= n) break;  // uniform: most bins hold a few hundred records
             const uint32_t r = (uint32_t)(k * kBlock + tid);
-            where[k]         = 0xFFFFFFFFu;
-            key[k]           = 0ull;
             if (r < n)
             {
                 const uint4 rec     = recs[r];
@@ -117,15 +145,79 @@ __global__ void __launch_bounds__(kBlock) bin_build_kernel(BuildPass a)
         list_off          = s_prefix[px];
         list_len          = s_cnt[px];
     }
+    const uint32_t keep = a.K > 0 ? min(c, (uint32_t)a.K) : c;  // kept fragments of the pixel this thread owns
+    float T = 1.f;
+    float color[C];
+#pragma unroll
+    for (int ci = 0; ci < C; ++ci) color[ci] = 0.f;
     if (in_lds)
     {
 #pragma unroll
         for (int k = 0; k < kBuildPerThread; ++k)
-            if (where[k] != 0xFFFFFFFFu) s_keys[s_prefix[where[k] & 0xFF] + (where[k] >> 8)] = key[k];
+            if ((uint32_t)(k * kBlock) < n && where[k] != 0xFFFFFFFFu)
+            {
+                const uint32_t place = s_prefix[where[k] & 0xFF] + (where[k] >> 8);
+                s_keys[place]        = key[k];
+                s_pix[place]         = (uint8_t)(where[k] & 0xFF);
+            }
         __syncthreads();
         sort_wave_lists(s_keys, s_src_lane[wave], list_off, list_len, lane, a.K);
         __syncthreads();
         for (uint32_t r = tid; r < n; r += kBlock) a.fragments[begin + r] = s_keys[r];
+        __syncthreads();  // the depth halves have been read; they now hold the transmittances
+
+        // ---- blend
+        float* s_T = reinterpret_cast<float*>(s_keys);  // s_T[2 r + 1]: transmittance in front of the fragment at r
+        const uint32_t* s_id = reinterpret_cast<const uint32_t*>(s_keys);  // s_id[2 r]: its point id
+        for (uint32_t base = 0; base < n; base += kStage)
+        {
+#pragma unroll
+            for (int k = 0; k < (kStage + kBlock - 1) / kBlock; ++k)
+            {
+                const uint32_t r = base + k * kBlock + tid;
+                if (k * kBlock + tid >= kStage || r >= n) continue;
+                const uint32_t px  = s_pix[r];
+                const uint32_t len = a.K > 0 ? min(s_cnt[px], (uint32_t)a.K) : s_cnt[px];
+                if (r - s_prefix[px] >= len) continue;  // cut away
+                const int id = (int)s_id[2 * r];
+                // an id or texture index out of range cannot come from a list the fill pass wrote; such a fragment
+                // blends as fully transparent (the reference asserts on the texture index, RenderForward.cu:1335-1336)
+                int ti = -1;
+                if ((uint32_t)id < (uint32_t)a.N) ti = a.index ? a.index[id] : id;
+                float4 t4 = make_float4(0.f, 0.f, 0.f, 0.f), c4 = t4;
+                if ((uint32_t)ti < (uint32_t)a.N)
+                {
+                    t4 = a.packed[2 * (size_t)ti];
+                    c4 = a.packed[2 * (size_t)ti + 1];
+                }
+                s_stage[r - base][0] = t4;
+                s_stage[r - base][1] = c4;
+            }
+            __syncthreads();
+            if ((uint32_t)tid < pixels)
+            {
+                const uint32_t lo = max(start, base), hi = min(start + keep, base + (uint32_t)kStage);
+                for (uint32_t r = lo; r < hi; ++r)
+                {
+                    const float4 t4 = s_stage[r - base][0];
+                    const float cf  = s_stage[r - base][1].x;
+                    s_T[2 * r + 1]  = T;
+                    const float t[4] = {t4.x, t4.y, t4.z, t4.w};
+                    const float Tc   = T * cf;
+#pragma unroll
+                    for (int ci = 0; ci < C; ++ci) color[ci] = Tc * t[ci] + color[ci];
+                    T = (1.f - cf) * T;
+                }
+            }
+            __syncthreads();
+        }
+        if (a.transmittance)
+            for (uint32_t r = tid; r < n; r += kBlock)
+            {
+                const uint32_t px  = s_pix[r];
+                const uint32_t len = a.K > 0 ? min(s_cnt[px], (uint32_t)a.K) : s_cnt[px];
+                if (r - s_prefix[px] < len) a.transmittance[begin + r] = s_T[2 * r + 1];
+            }
     }
     else
     {
@@ -155,6 +247,34 @@ __global__ void __launch_bounds__(kBlock) bin_build_kernel(BuildPass a)
         __threadfence_block();  // the keys other waves stored are read below
         __syncthreads();
         sort_wave_lists(a.fragments + begin, s_src_lane[wave], list_off, list_len, lane, a.K);
+        __threadfence_block();
+        __syncthreads();
+        if ((uint32_t)tid < pixels)
+            blend_list_from_memory<C>(a.fragments + begin + start, keep, a.index, a.packed, a.N,
+                                      a.transmittance ? a.transmittance + begin + start : nullptr, T, color);
+    }
+
+    if ((uint32_t)tid < pixels)
+    {
+        // pixel number -> image coordinates
+        const uint32_t q        = q0 + tid;
+        const uint32_t in_layer = q - a.ly.base[l];
+        const uint32_t tile     = in_layer / kTilePixels;
+        const uint32_t ty = tile / (uint32_t)a.ly.tiles_x[l], tx = tile - ty * (uint32_t)a.ly.tiles_x[l];
+        const int x = (int)(tx * kTile + (q & (kTile - 1))), y = (int)(ty * kTile + ((q / kTile) & (kTile - 1)));
+        if (x < a.ly.w[l] && y < a.ly.h[l])
+        {
+            const size_t plane   = (size_t)a.ly.w[l] * a.ly.h[l];
+            const uint32_t local = (uint32_t)y * (uint32_t)a.ly.w[l] + (uint32_t)x;
+#pragma unroll
+            for (int ci = 0; ci < C; ++ci)
+            {
+                if (!a.use_environment_map) color[ci] = (T * 1.f) * a.background[ci] + color[ci];
+                a.out[l][ci * plane + local] = color[ci];
+            }
+            a.weight[q] = T;
+            if (a.out_mask[l]) a.out_mask[l][local] = (T == 0.f) ? a.mask_value : 1.f;
+        }
     }
 }
 

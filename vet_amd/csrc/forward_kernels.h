@@ -144,18 +144,19 @@ __device__ __forceinline__ WaveGroup group_by_bin(bool has, uint32_t bin, int la
     WaveGroup g;
     g.leader = lane;
     g.rank = g.count = 0;
-    const uint64_t lanes_below = (1ull << lane) - 1ull;
     uint64_t todo = __ballot(has);
-    while (todo != 0ull)
+    while (todo != 0ull)  // one turn per distinct bin; everything but the compare and the selects is scalar
     {
         const int first        = __ffsll((unsigned long long)todo) - 1;
-        const uint32_t b_first = (uint32_t)__shfl((int)bin, first, kWave);
+        const uint32_t b_first = (uint32_t)__builtin_amdgcn_readlane((int)bin, first);
         const bool mine        = has && bin == b_first;
         const uint64_t same    = __ballot(mine);
+        // number of set bits of `same` below this lane
+        const uint32_t below = __builtin_amdgcn_mbcnt_hi((uint32_t)(same >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)same, 0u));
         if (mine)
         {
             g.leader = first;
-            g.rank   = (uint32_t)__popcll(same & lanes_below);
+            g.rank   = below;
             g.count  = (uint32_t)__popcll(same);
         }
         todo &= ~same;
@@ -360,47 +361,15 @@ __global__ void __launch_bounds__(kBlock) bin_fill_kernel(ViewPass a, const uint
     }
 }
 
-struct BlendPass
-{
-    const uint32_t* offsets;
-    const uint64_t* fragments;
-    const int32_t* index;
-    const float4* packed;
-    const float* background;
-    float* transmittance;  // per fragment, null unless the backward pass will run
-    float* weight;         // per pixel
-    float* out[VETRAST_MAX_LAYERS];       // already offset to this view
-    float* out_mask[VETRAST_MAX_LAYERS];  // already offset to this view, or null
-    LayerTable ly;
-    TileMap tiles;
-    uint32_t P;
-    int N;
-    int K;
-    int use_environment_map;
-    float mask_value;
-};
-
-// One thread per pixel walks the sorted list front to back: out += (T*c)*t, T = (1-c)*T, in exactly this order, then
-// the background behind the last fragment. Counterpart of BlendMulti (src/lib/rendering/RenderForward.cu:1303-1357)
-// and CreateMask (src/lib/rendering/PointRenderer.cu:216-235). Pixels of all layers are served by one launch; the
-// reference also uses 16x16 workgroups (RenderForward.cu:1385), one launch per layer.
+// Front-to-back blend of one pixel's sorted list read from memory: out += (T*c)*t, T = (1-c)*T, in exactly this order
+// (BlendMulti, src/lib/rendering/RenderForward.cu:1303-1357). The list is walked in chunks of kBlendChunk fragments: all
+// keys of a chunk are loaded first, then all descriptor records, and only then the (strictly sequential) arithmetic
+// runs, so a thread keeps several gathers in flight instead of one dependent load chain per fragment.
 template <int C>
-__global__ void __launch_bounds__(kBlock) blend_kernel(BlendPass a)
+__device__ __forceinline__ void blend_list_from_memory(const uint64_t* list, uint32_t n, const int32_t* index,
+                                                       const float4* packed, int N, float* transmittance, float& T,
+                                                       float (&color)[C])
 {
-    const TilePixel px = tile_pixel(a.tiles, a.ly);
-    if (!px.active) return;
-    const uint32_t q   = px.q;
-    const uint32_t off = a.offsets[q];
-    uint32_t n         = a.offsets[q + 1] - off;
-    if (a.K > 0) n = min(n, (uint32_t)a.K);
-    float T = 1.f;
-    float color[C];
-#pragma unroll
-    for (int ci = 0; ci < C; ++ci) color[ci] = 0.f;
-    const uint64_t* list = a.fragments + off;
-    // The list is walked in chunks of kBlendChunk fragments: all keys of a chunk are loaded first, then all descriptor
-    // records, and only then the (strictly sequential) blend arithmetic runs, so a thread keeps several gathers in
-    // flight instead of one dependent load chain per fragment.
     for (uint32_t base = 0; base < n; base += kBlendChunk)
     {
         int ti[kBlendChunk];
@@ -415,8 +384,8 @@ __global__ void __launch_bounds__(kBlock) blend_kernel(BlendPass a)
                 const int id = (int)(uint32_t)list[base + u];
                 // an id or texture index out of range cannot come from a list the fill pass wrote; such a fragment is
                 // skipped instead of gathered (the reference asserts on the texture index, RenderForward.cu:1335-1336)
-                if ((uint32_t)id < (uint32_t)a.N) ti[u] = a.index ? a.index[id] : id;
-                if ((uint32_t)ti[u] >= (uint32_t)a.N) ti[u] = -1;
+                if ((uint32_t)id < (uint32_t)N) ti[u] = index ? index[id] : id;
+                if ((uint32_t)ti[u] >= (uint32_t)N) ti[u] = -1;
             }
         }
 #pragma unroll
@@ -424,8 +393,8 @@ __global__ void __launch_bounds__(kBlock) blend_kernel(BlendPass a)
         {
             if (ti[u] >= 0)
             {
-                t4[u] = a.packed[2 * (size_t)ti[u]];
-                c[u]  = a.packed[2 * (size_t)ti[u] + 1].x;
+                t4[u] = packed[2 * (size_t)ti[u]];
+                c[u]  = packed[2 * (size_t)ti[u] + 1].x;
             }
         }
 #pragma unroll
@@ -433,7 +402,7 @@ __global__ void __launch_bounds__(kBlock) blend_kernel(BlendPass a)
         {
             if (ti[u] >= 0)
             {
-                if (a.transmittance) a.transmittance[off + base + u] = T;
+                if (transmittance) transmittance[base + u] = T;
                 const float t[4] = {t4[u].x, t4[u].y, t4[u].z, t4[u].w};
                 const float Tc   = T * c[u];
 #pragma unroll
@@ -442,17 +411,6 @@ __global__ void __launch_bounds__(kBlock) blend_kernel(BlendPass a)
             }
         }
     }
-    const int l          = px.l;
-    const size_t plane   = (size_t)a.ly.w[l] * a.ly.h[l];
-    const uint32_t local = px.local;
-#pragma unroll
-    for (int ci = 0; ci < C; ++ci)
-    {
-        if (!a.use_environment_map) color[ci] = (T * 1.f) * a.background[ci] + color[ci];
-        a.out[l][ci * plane + local] = color[ci];
-    }
-    a.weight[q] = T;
-    if (a.out_mask[l]) a.out_mask[l][local] = (T == 0.f) ? a.mask_value : 1.f;
 }
 
 }  // namespace vetrast

@@ -352,8 +352,6 @@ int vetrast_forward(vetrast_ctx* ctx, const vetrast_forward_args* a, void* strea
     const vetrast_params& p = a->params;
     const int N = a->num_points, B = a->num_views, L = p.num_layers, C = p.num_texture_channels;
     const LayerTable ly = make_layer_table(a->views[0].w, a->views[0].h, L, N);
-    const TileMap tiles = make_tile_map(ly);
-    const uint32_t P    = ly.base[L];
     const uint32_t bins = ly.bin_base[L];
     const size_t Tpad   = lay.bin_counts_stride / sizeof(uint32_t);
     void* ws            = a->workspace;
@@ -437,52 +435,44 @@ int vetrast_forward(vetrast_ctx* ctx, const vetrast_forward_args* a, void* strea
             hipLaunchKernelGGL(bin_fill_kernel, dim3(grid_for(N)), dim3(kBlock), 0, stream, vp, bin_counts, slots, binned,
                                (uint32_t)lay.fragment_capacity);
         }
+        float* out[VETRAST_MAX_LAYERS];
+        float* out_mask[VETRAST_MAX_LAYERS];
+        for (int l = 0; l < VETRAST_MAX_LAYERS; ++l)
+        {
+            out[l]      = nullptr;
+            out_mask[l] = nullptr;
+            if (l >= L) continue;
+            const size_t plane = (size_t)ly.w[l] * ly.h[l];
+            out[l]             = a->out[l] + (size_t)b * C * plane;
+            if (p.output_background_mask) out_mask[l] = a->out_mask[l] + (size_t)b * plane;
+        }
         {
             ScopeTimer tm(ctx, stream, VETRAST_SCOPE_BUILD);
             BuildPass bp;
-            bp.bin_offsets   = bin_counts;
-            bp.binned        = binned;
-            bp.offsets       = offsets;
-            bp.fragments     = fragments;
-            bp.list_is_cut   = list_is_cut;
-            bp.ly            = ly;
-            bp.num_bins      = bins;
-            bp.K             = p.debug_max_list_length;
-            hipLaunchKernelGGL(bin_build_kernel, dim3(bins), dim3(kBlock), 0, stream, bp);
-        }
-        {
-            ScopeTimer tm(ctx, stream, VETRAST_SCOPE_BLEND);
-            BlendPass bp;
+            bp.bin_offsets         = bin_counts;
+            bp.binned              = binned;
             bp.offsets             = offsets;
             bp.fragments           = fragments;
+            bp.list_is_cut         = list_is_cut;
             bp.index               = a->index;
             bp.packed              = packed;
             bp.background          = a->background;
             bp.transmittance       = a->save_for_backward ? trans : nullptr;
             bp.weight              = weight;
             bp.ly                  = ly;
-            bp.tiles               = tiles;
-            bp.P                   = P;
+            bp.num_bins            = bins;
             bp.N                   = N;
             bp.K                   = p.debug_max_list_length;
             bp.use_environment_map = p.use_environment_map;
             bp.mask_value          = p.output_background_mask_value;
-            for (int l = 0; l < VETRAST_MAX_LAYERS; ++l)
-            {
-                bp.out[l]      = nullptr;
-                bp.out_mask[l] = nullptr;
-                if (l >= L) continue;
-                const size_t plane = (size_t)ly.w[l] * ly.h[l];
-                bp.out[l]          = a->out[l] + (size_t)b * C * plane;
-                if (p.output_background_mask) bp.out_mask[l] = a->out_mask[l] + (size_t)b * plane;
-            }
-            const dim3 g(tile_grid(tiles)), blk(kBlock);
+            for (int l = 0; l < VETRAST_MAX_LAYERS; ++l) bp.out[l] = out[l], bp.out_mask[l] = out_mask[l];
+            const dim3 g(bins), blk(kBlock);
             switch (C)
             {
-                case 1: hipLaunchKernelGGL(blend_kernel<1>, g, blk, 0, stream, bp); break;
-                case 2: hipLaunchKernelGGL(blend_kernel<2>, g, blk, 0, stream, bp); break;
-                case 3: hipLaunchKernelGGL(blend_kernel<3>, g, blk, 0, stream, bp); break;
-                default: hipLaunchKernelGGL(blend_kernel<4>, g, blk, 0, stream, bp); break;
+                case 1: hipLaunchKernelGGL(bin_build_kernel<1>, g, blk, 0, stream, bp); break;
+                case 2: hipLaunchKernelGGL(bin_build_kernel<2>, g, blk, 0, stream, bp); break;
+                case 3: hipLaunchKernelGGL(bin_build_kernel<3>, g, blk, 0, stream, bp); break;
+                default: hipLaunchKernelGGL(bin_build_kernel<4>, g, blk, 0, stream, bp); break;
             }
         }
     }
@@ -720,8 +710,7 @@ const char* vetrast_scope_name(int32_t scope)
         case VETRAST_SCOPE_COUNT: return "CountingPass";
         case VETRAST_SCOPE_SCAN: return "CreateAndAllocateBuffers";
         case VETRAST_SCOPE_FILL: return "CollectionPass";
-        case VETRAST_SCOPE_BUILD: return "CollectionPass (per-pixel lists) + SortingPass";
-        case VETRAST_SCOPE_BLEND: return "BlendingPass";
+        case VETRAST_SCOPE_BUILD: return "CollectionPass (per-pixel lists) + SortingPass + BlendingPass";
         case VETRAST_SCOPE_BACKWARD_PREPARE: return "Prepare Backward";
         case VETRAST_SCOPE_BACKWARD_BLEND: return "BlendBackwards";
         case VETRAST_SCOPE_BACKWARD_GATHER: return "BlendBackwards (per-point sum)";
