@@ -189,7 +189,7 @@ def main():
                       "frac": round(nbytes / 1e6 / t / HBM_PEAK_GBS, 4) if t > 0 else None}
         if k in traffic:
             kernels[k]["hbm_traffic_MB"] = round(traffic[k] / 1e6, 1)
-    for k in ("PREPARE", "SCAN", "BACKWARD_PREPARE", "BACKWARD_POST"):
+    for k in ("PREPARE", "PACK", "SCAN", "BACKWARD_PREPARE", "BACKWARD_POST"):
         if r["per_step_ms"].get(k, 0.0) > 0:
             kernels[k] = {"ms": round(r["per_step_ms"][k], 5), "alg_MB": 0.0, "GBps": None, "frac": None}
     dominant = max(alg.keys(), key=lambda k: r["per_step_ms"].get(k, 0.0))

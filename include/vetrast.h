@@ -91,7 +91,9 @@ typedef struct vetrast_ctx vetrast_ctx;
  * (src/lib/rendering/PointRenderer.cu:249,770,791,843,872,886,1222,1252). */
 typedef enum vetrast_scope
 {
-    VETRAST_SCOPE_PREPARE = 0,      /* "Build Cache": zero-fill, view preparation, descriptor interleave */
+    VETRAST_SCOPE_PREPARE = 0,      /* "Build Cache": zero-fill, view preparation */
+    VETRAST_SCOPE_PACK,             /* "Build Cache": descriptor interleave; runs on a stream of the context's own beside
+                                       COUNT..FILL, so its time is not part of the sum of the others */
     VETRAST_SCOPE_COUNT,            /* "CountingPass": fragments per bin (a 16x16 pixel tile or a piece of one) */
     VETRAST_SCOPE_SCAN,             /* "CreateAndAllocateBuffers" (prefix scan over the bins; no allocation here) */
     VETRAST_SCOPE_FILL,             /* "CollectionPass", first half: fragment records grouped by bin */

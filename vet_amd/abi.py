@@ -20,7 +20,7 @@ CAMERA_OCAM = 1
 CAMERA_SPHERICAL = 2
 
 SCOPE_NAMES = [
-    "PREPARE", "COUNT", "SCAN", "FILL", "BUILD", "BACKWARD_PREPARE", "BACKWARD_BLEND", "BACKWARD_GATHER", "BACKWARD_POST",
+    "PREPARE", "PACK", "COUNT", "SCAN", "FILL", "BUILD", "BACKWARD_PREPARE", "BACKWARD_BLEND", "BACKWARD_GATHER", "BACKWARD_POST",
 ]
 SCOPE_COUNT = len(SCOPE_NAMES)
 

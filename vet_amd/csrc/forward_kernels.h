@@ -34,10 +34,21 @@ struct PrepareViewsArgs
 // One thread per view: pose (unit quaternion + translation, double) -> 3x4 float matrix, intrinsics row -> K.
 // The reference casts the SE3d to float in every thread (src/lib/rendering/RenderConstants.h:78); here the rotation
 // matrix is formed once, in double, and rounded once. Non-zero distortion coefficients raise flag bit 0.
-__global__ void prepare_views_kernel(PrepareViewsArgs args, int first_view, int num_views,
-                                     const double* __restrict__ poses_se3, const float* __restrict__ intrinsics,
-                                     DeviceView* __restrict__ views, uint32_t* __restrict__ flags)
+// Workgroups beyond the first zero the per-bin counters of all views (n4 uint4 elements).
+__global__ void __launch_bounds__(kBlock) prepare_views_kernel(PrepareViewsArgs args, int first_view, int num_views,
+                                                                const double* __restrict__ poses_se3,
+                                                                const float* __restrict__ intrinsics,
+                                                                DeviceView* __restrict__ views,
+                                                                uint32_t* __restrict__ flags,
+                                                                uint4* __restrict__ counters4, size_t n4)
 {
+    if (blockIdx.x > 0)
+    {
+        const size_t stride = (size_t)(gridDim.x - 1) * blockDim.x;
+        for (size_t i = (size_t)(blockIdx.x - 1) * blockDim.x + threadIdx.x; i < n4; i += stride)
+            counters4[i] = make_uint4(0u, 0u, 0u, 0u);
+        return;
+    }
     const int k = threadIdx.x;
     if (first_view == 0)
     {
@@ -86,15 +97,12 @@ __global__ void prepare_views_kernel(PrepareViewsArgs args, int first_view, int 
 // Planar descriptors [C,N] + confidence [N] -> one 32-byte record per texture index, so that a fragment costs a single
 // aligned gather instead of C+1 gathers from planes megabytes apart (the reference's BlendMulti reads
 // d_texture.in_texture(ci, idx) per channel, src/lib/rendering/RenderForward.cu:1338-1342).
-// The same launch also zeroes the per-pixel counters of all views (n4 uint4 elements), which saves a launch per call.
 template <int C>
 __global__ void __launch_bounds__(kBlock) pack_descriptors_kernel(const float* __restrict__ texture,
                                                                    const float* __restrict__ confidence,
-                                                                   float4* __restrict__ packed, int N,
-                                                                   uint4* __restrict__ counters4, size_t n4)
+                                                                   float4* __restrict__ packed, int N)
 {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
-    for (size_t k = (size_t)i; k < n4; k += (size_t)gridDim.x * blockDim.x) counters4[k] = make_uint4(0u, 0u, 0u, 0u);
     if (i >= N) return;
     float t[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll

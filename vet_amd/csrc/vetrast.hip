@@ -26,6 +26,10 @@ struct vetrast_ctx
         int scope;
         hipEvent_t start, stop;
     };
+    // The descriptor interleave only feeds the last forward kernel, so it runs beside the binning kernels on a stream
+    // of the context's own, forked from and joined back into the caller's stream with events.
+    hipStream_t side  = nullptr;
+    hipEvent_t forked = nullptr, joined = nullptr;
     std::vector<Span> spans;             // recorded since the last reset
     std::vector<hipEvent_t> free_events;  // recycled events
     float acc_ms[VETRAST_SCOPE_COUNT_]      = {};
@@ -233,9 +237,12 @@ int vetrast_create(vetrast_ctx** out_ctx)
     vetrast_ctx* ctx = new (std::nothrow) vetrast_ctx();
     if (!ctx) return VETRAST_ERR_INVALID_ARG;
     hipError_t e = hipGetDevice(&ctx->device);
+    if (e == hipSuccess) e = hipStreamCreateWithFlags(&ctx->side, hipStreamNonBlocking);
+    if (e == hipSuccess) e = hipEventCreateWithFlags(&ctx->forked, hipEventDisableTiming);
+    if (e == hipSuccess) e = hipEventCreateWithFlags(&ctx->joined, hipEventDisableTiming);
     if (e != hipSuccess)
     {
-        delete ctx;
+        vetrast_destroy(ctx);
         return VETRAST_ERR_HIP;
     }
     *out_ctx = ctx;
@@ -251,6 +258,9 @@ void vetrast_destroy(vetrast_ctx* ctx)
         (void)hipEventDestroy(s.stop);
     }
     for (auto e : ctx->free_events) (void)hipEventDestroy(e);
+    if (ctx->forked) (void)hipEventDestroy(ctx->forked);
+    if (ctx->joined) (void)hipEventDestroy(ctx->joined);
+    if (ctx->side) (void)hipStreamDestroy(ctx->side);
     delete ctx;
 }
 
@@ -361,14 +371,30 @@ int vetrast_forward(vetrast_ctx* ctx, const vetrast_forward_args* a, void* strea
     uint32_t* partials  = ws_ptr<uint32_t>(ws, lay.scan_partials_base);
     DeviceView* views   = ws_ptr<DeviceView>(ws, lay.views_base);
 
+    if (N > 0)
+    {
+        // descriptor interleave on the side stream; joined again in front of the build pass of the first view
+        VET_HIP(ctx, hipEventRecord(ctx->forked, stream));
+        VET_HIP(ctx, hipStreamWaitEvent(ctx->side, ctx->forked, 0));
+        {
+            ScopeTimer tm(ctx, ctx->side, VETRAST_SCOPE_PACK);
+            const dim3 g(grid_for(N)), blk(kBlock);
+            switch (C)
+            {
+                case 1: hipLaunchKernelGGL(pack_descriptors_kernel<1>, g, blk, 0, ctx->side, a->texture, a->confidence, packed, N); break;
+                case 2: hipLaunchKernelGGL(pack_descriptors_kernel<2>, g, blk, 0, ctx->side, a->texture, a->confidence, packed, N); break;
+                case 3: hipLaunchKernelGGL(pack_descriptors_kernel<3>, g, blk, 0, ctx->side, a->texture, a->confidence, packed, N); break;
+                default: hipLaunchKernelGGL(pack_descriptors_kernel<4>, g, blk, 0, ctx->side, a->texture, a->confidence, packed, N); break;
+            }
+        }
+        VET_HIP(ctx, hipEventRecord(ctx->joined, ctx->side));
+    }
     {
         ScopeTimer tm(ctx, stream, VETRAST_SCOPE_PREPARE);
         // per-bin counters of all views (contiguous) start at zero; InitializeData, PointRenderer.cu:402-470
         const size_t n4  = Tpad * B / 4;
         uint4* counters4 = ws_ptr<uint4>(ws, lay.bin_counts_base);
-        if (N == 0)
-            hipLaunchKernelGGL(fill_u128_kernel, dim3(std::min(grid_for(n4), 4096)), dim3(kBlock), 0, stream, counters4,
-                               n4, 0u);
+        const int zero_blocks = std::min(grid_for(n4), 1024);
         for (int first = 0; first < B; first += 16)
         {
             PrepareViewsArgs pv;
@@ -384,19 +410,8 @@ int vetrast_forward(vetrast_ctx* ctx, const vetrast_forward_args* a, void* strea
                 for (int j = 0; j < 5; ++j) s.crop[j] = v.crop_transform[j];
                 for (int j = 0; j < 4; ++j) s.rot[j] = v.crop_rotation[j];
             }
-            hipLaunchKernelGGL(prepare_views_kernel, dim3(1), dim3(kWave), 0, stream, pv, first, cnt, a->poses_se3,
-                               a->intrinsics, views, flags);
-        }
-        if (N > 0)
-        {
-            const dim3 g(grid_for(N)), blk(kBlock);
-            switch (C)
-            {
-                case 1: hipLaunchKernelGGL(pack_descriptors_kernel<1>, g, blk, 0, stream, a->texture, a->confidence, packed, N, counters4, n4); break;
-                case 2: hipLaunchKernelGGL(pack_descriptors_kernel<2>, g, blk, 0, stream, a->texture, a->confidence, packed, N, counters4, n4); break;
-                case 3: hipLaunchKernelGGL(pack_descriptors_kernel<3>, g, blk, 0, stream, a->texture, a->confidence, packed, N, counters4, n4); break;
-                default: hipLaunchKernelGGL(pack_descriptors_kernel<4>, g, blk, 0, stream, a->texture, a->confidence, packed, N, counters4, n4); break;
-            }
+            hipLaunchKernelGGL(prepare_views_kernel, dim3(1 + (first == 0 ? zero_blocks : 0)), dim3(kBlock), 0, stream, pv,
+                               first, cnt, a->poses_se3, a->intrinsics, views, flags, counters4, n4);
         }
     }
 
@@ -446,6 +461,7 @@ int vetrast_forward(vetrast_ctx* ctx, const vetrast_forward_args* a, void* strea
             out[l]             = a->out[l] + (size_t)b * C * plane;
             if (p.output_background_mask) out_mask[l] = a->out_mask[l] + (size_t)b * plane;
         }
+        if (b == 0 && N > 0) VET_HIP(ctx, hipStreamWaitEvent(stream, ctx->joined, 0));
         {
             ScopeTimer tm(ctx, stream, VETRAST_SCOPE_BUILD);
             BuildPass bp;
@@ -707,6 +723,7 @@ const char* vetrast_scope_name(int32_t scope)
     switch (scope)
     {
         case VETRAST_SCOPE_PREPARE: return "Build Cache";
+        case VETRAST_SCOPE_PACK: return "Build Cache (descriptor interleave, beside the binning passes)";
         case VETRAST_SCOPE_COUNT: return "CountingPass";
         case VETRAST_SCOPE_SCAN: return "CreateAndAllocateBuffers";
         case VETRAST_SCOPE_FILL: return "CollectionPass";
