@@ -294,26 +294,27 @@ __global__ void __launch_bounds__(kBlock) blend_backward_kernel(BackwardPass a)
 // Sums the per-workgroup background rows of one view (one workgroup, fixed order, so the result is reproducible) and
 // adds the background pseudo-fragment's alpha gradient to confidence row 0 when that switch of the reference's
 // behaviour is on (src/lib/rendering/RenderBackward.cu:1130-1131,1157).
-__global__ void __launch_bounds__(kBlock) reduce_background_kernel(const float* __restrict__ rows, int num_rows, int C,
-                                                                    float* __restrict__ grad_background,
-                                                                    float* __restrict__ grad_confidence, int add_leak,
-                                                                    int accumulate)
+constexpr int kReduceBlock = 1024;  // one workgroup of 16 waves: the rows are summed in one launch, in a fixed order
+__global__ void __launch_bounds__(kReduceBlock) reduce_background_kernel(const float* __restrict__ rows, int num_rows,
+                                                                          int C, float* __restrict__ grad_background,
+                                                                          float* __restrict__ grad_confidence,
+                                                                          int add_leak, int accumulate)
 {
-    __shared__ float red[kBlock / kWave][kBackgroundRow];
+    __shared__ float red[kReduceBlock / kWave][kBackgroundRow];
     float acc[kBackgroundRow];
 #pragma unroll
     for (int k = 0; k < kBackgroundRow; ++k) acc[k] = 0.f;
     // eight independent row loads per thread and trip: one workgroup has to pull in ~10^4 rows and would otherwise sit
     // on one memory round trip per row
-    constexpr int kUnroll = 8;
-    for (int r0 = threadIdx.x; r0 < num_rows; r0 += kBlock * kUnroll)
+    constexpr int kUnroll = 4;
+    for (int r0 = threadIdx.x; r0 < num_rows; r0 += kReduceBlock * kUnroll)
     {
         float4 a0[kUnroll];
         float a1[kUnroll];
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u)
         {
-            const int r = r0 + u * kBlock;
+            const int r = r0 + u * kReduceBlock;
             a0[u]       = make_float4(0.f, 0.f, 0.f, 0.f);
             a1[u]       = 0.f;
             if (r < num_rows)
@@ -342,8 +343,9 @@ __global__ void __launch_bounds__(kBlock) reduce_background_kernel(const float* 
     __syncthreads();
     if (threadIdx.x <= C)
     {
-        const int k   = threadIdx.x;
-        const float s = (red[0][k] + red[1][k]) + (red[2][k] + red[3][k]);
+        const int k = threadIdx.x;
+        float s     = 0.f;
+        for (int w = 0; w < kReduceBlock / kWave; ++w) s += red[w][k];
         if (k < C)
             grad_background[k] = accumulate ? grad_background[k] + s : s;
         else if (add_leak)

@@ -636,7 +636,7 @@ int vetrast_backward(vetrast_ctx* ctx, const vetrast_backward_args* g, void* str
         {
             // after the per-point kernel: it overwrites confidence row 0, the leak term is added on top
             ScopeTimer tm(ctx, stream, VETRAST_SCOPE_BACKWARD_GATHER);
-            hipLaunchKernelGGL(reduce_background_kernel, dim3(1), dim3(kBlock), 0, stream, background_rows,
+            hipLaunchKernelGGL(reduce_background_kernel, dim3(1), dim3(kReduceBlock), 0, stream, background_rows,
                                (int)(tile_grid(tiles)), C, g->grad_background, g->grad_confidence,
                                (p.quirk_background_confidence_leak && !p.use_environment_map && N > 0) ? 1 : 0,
                                b > 0 ? 1 : 0);
