@@ -294,27 +294,31 @@ __global__ void __launch_bounds__(kBlock) blend_backward_kernel(BackwardPass a)
 // Sums the per-workgroup background rows of one view (one workgroup, fixed order, so the result is reproducible) and
 // adds the background pseudo-fragment's alpha gradient to confidence row 0 when that switch of the reference's
 // behaviour is on (src/lib/rendering/RenderBackward.cu:1130-1131,1157).
-constexpr int kReduceBlock = 1024;  // one workgroup of 16 waves: the rows are summed in one launch, in a fixed order
-__global__ void __launch_bounds__(kReduceBlock) reduce_background_kernel(const float* __restrict__ rows, int num_rows,
-                                                                          int C, float* __restrict__ grad_background,
-                                                                          float* __restrict__ grad_confidence,
-                                                                          int add_leak, int accumulate)
+// Sum of the per-workgroup background rows of one view by one workgroup of BLOCK threads, in a fixed order, so the
+// result is reproducible. Also adds the background pseudo-fragment's alpha gradient to confidence row 0 when that switch
+// of the reference's behaviour is on (src/lib/rendering/RenderBackward.cu:1130-1131,1157); with `leak_atomic` that
+// add is an atomic (rows are being added to by other workgroups), otherwise the caller guarantees row 0 has its value.
+template <int BLOCK>
+__device__ __forceinline__ void sum_background_rows(const float* __restrict__ rows, int num_rows, int C,
+                                                    float* __restrict__ grad_background,
+                                                    float* __restrict__ grad_confidence, int add_leak, int accumulate,
+                                                    int leak_atomic)
 {
-    __shared__ float red[kReduceBlock / kWave][kBackgroundRow];
+    __shared__ float red[BLOCK / kWave][kBackgroundRow];
     float acc[kBackgroundRow];
 #pragma unroll
     for (int k = 0; k < kBackgroundRow; ++k) acc[k] = 0.f;
-    // eight independent row loads per thread and trip: one workgroup has to pull in ~10^4 rows and would otherwise sit
-    // on one memory round trip per row
+    // several independent row loads per thread and trip: one workgroup has to pull in ~10^4 rows and would otherwise
+    // sit on one memory round trip per row
     constexpr int kUnroll = 4;
-    for (int r0 = threadIdx.x; r0 < num_rows; r0 += kReduceBlock * kUnroll)
+    for (int r0 = threadIdx.x; r0 < num_rows; r0 += BLOCK * kUnroll)
     {
         float4 a0[kUnroll];
         float a1[kUnroll];
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u)
         {
-            const int r = r0 + u * kReduceBlock;
+            const int r = r0 + u * BLOCK;
             a0[u]       = make_float4(0.f, 0.f, 0.f, 0.f);
             a1[u]       = 0.f;
             if (r < num_rows)
@@ -345,12 +349,27 @@ __global__ void __launch_bounds__(kReduceBlock) reduce_background_kernel(const f
     {
         const int k = threadIdx.x;
         float s     = 0.f;
-        for (int w = 0; w < kReduceBlock / kWave; ++w) s += red[w][k];
+        for (int w = 0; w < BLOCK / kWave; ++w) s += red[w][k];
         if (k < C)
             grad_background[k] = accumulate ? grad_background[k] + s : s;
         else if (add_leak)
-            grad_confidence[0] += s;
+        {
+            if (leak_atomic)
+                atomicAdd(&grad_confidence[0], s);
+            else
+                grad_confidence[0] += s;
+        }
     }
+}
+
+// Stand-alone form for a cloud without points (the per-point kernel, which otherwise does this sum, is not launched).
+constexpr int kReduceBlock = 1024;
+__global__ void __launch_bounds__(kReduceBlock) reduce_background_kernel(const float* __restrict__ rows, int num_rows,
+                                                                          int C, float* __restrict__ grad_background,
+                                                                          float* __restrict__ grad_confidence,
+                                                                          int add_leak, int accumulate)
+{
+    sum_background_rows<kReduceBlock>(rows, num_rows, C, grad_background, grad_confidence, add_leak, accumulate, 0);
 }
 
 struct GatherPass
@@ -368,6 +387,12 @@ struct GatherPass
     int K;
     int need_point_gradient;
     int accumulate;  // 0: overwrite the gradient rows (first view), 1: add to them (further views)
+    // background gradient: workgroup 0 also sums the rows the per-pixel kernel left (hidden behind the other workgroups)
+    const float* background_rows;
+    int num_background_rows;
+    float* grad_background;
+    int add_leak;
+    int background_accumulate;
 };
 
 constexpr int kCameraRow = 12;  // doubles per workgroup row: 6 pose tangent, fx, fy, cx, cy, fragment count, pad
@@ -473,9 +498,11 @@ __global__ void __launch_bounds__(kBlock) gather_point_gradients_kernel(GatherPa
             a.camera_partial[(size_t)blockIdx.x * kCameraRow + threadIdx.x] =
                 (cam_red[0][threadIdx.x] + cam_red[1][threadIdx.x]) + (cam_red[2][threadIdx.x] + cam_red[3][threadIdx.x]);
     }
-    if (!alive) return;
     const int N = a.vp.N;
-    if (a.vp.index)
+    if (!alive)
+    {
+    }
+    else if (a.vp.index)
     {
         const int ti = a.vp.index[i];
         if ((uint32_t)ti < (uint32_t)N)
@@ -498,7 +525,7 @@ __global__ void __launch_bounds__(kBlock) gather_point_gradients_kernel(GatherPa
         for (int ci = 0; ci < C; ++ci) a.grad_texture[(size_t)ci * N + i] = gt[ci];
         a.grad_confidence[i] = gc;
     }
-    if (a.grad_points)
+    if (alive && a.grad_points)
     {
         float4* gp = reinterpret_cast<float4*>(a.grad_points) + i;
         if (a.accumulate)
@@ -512,6 +539,14 @@ __global__ void __launch_bounds__(kBlock) gather_point_gradients_kernel(GatherPa
             *gp                   = make_float4(gx, gy, gz, 0.f);
             a.grad_point_count[i] = cnt;
         }
+    }
+    if (blockIdx.x == 0)
+    {
+        // Without an index indirection confidence row 0 has just been written by thread 0 of this workgroup, which is
+        // also the thread that adds the leak term; with one, rows are added to with atomics by every workgroup.
+        __syncthreads();
+        sum_background_rows<kBlock>(a.background_rows, a.num_background_rows, C, a.grad_background, a.grad_confidence,
+                                    a.add_leak, a.background_accumulate, a.vp.index != nullptr);
     }
 }
 

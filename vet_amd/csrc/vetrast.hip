@@ -617,6 +617,11 @@ int vetrast_backward(vetrast_ctx* ctx, const vetrast_backward_args* g, void* str
             gp.need_point_gradient = want_image_gradient ? 1 : 0;
             gp.camera_partial      = want_camera ? camera_rows : nullptr;
             gp.accumulate          = (add_to_rows || b > 0) ? 1 : 0;
+            gp.background_rows       = background_rows;
+            gp.num_background_rows   = (int)tile_grid(tiles);
+            gp.grad_background       = g->grad_background;
+            gp.add_leak              = (p.quirk_background_confidence_leak && !p.use_environment_map) ? 1 : 0;
+            gp.background_accumulate = b > 0 ? 1 : 0;
             const dim3 grid(grid_for(N)), blk(kBlock);
             switch (C)
             {
@@ -633,13 +638,12 @@ int vetrast_backward(vetrast_ctx* ctx, const vetrast_backward_args* g, void* str
                                a->views[b].image_index, a->views[b].camera_index, p.K_gradient_factor, g->grad_pose,
                                g->grad_pose_count, g->grad_intrinsics, g->grad_intrinsics_count);
         }
+        if (N == 0)
         {
-            // after the per-point kernel: it overwrites confidence row 0, the leak term is added on top
             ScopeTimer tm(ctx, stream, VETRAST_SCOPE_BACKWARD_GATHER);
             hipLaunchKernelGGL(reduce_background_kernel, dim3(1), dim3(kReduceBlock), 0, stream, background_rows,
                                (int)(tile_grid(tiles)), C, g->grad_background, g->grad_confidence,
-                               (p.quirk_background_confidence_leak && !p.use_environment_map && N > 0) ? 1 : 0,
-                               b > 0 ? 1 : 0);
+                               0, b > 0 ? 1 : 0);
         }
     }
     if (g->grad_points && p.point_gradient_normalization != 0 && N > 0)
