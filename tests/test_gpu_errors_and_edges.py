@@ -164,3 +164,16 @@ def test_forward_backward_can_be_captured_in_a_hip_graph(rasterizer, oracle):
         again = rasterizer.forward(dev, params)
         torch.cuda.synchronize()
         assert torch.equal(again.out[0], want_out[0])
+
+
+@pytest.mark.parametrize("K", [16, 0])
+def test_cluster_far_denser_than_the_layer_average(K, rasterizer, oracle):
+    """All points inside a 3x3 pixel patch of a 96x64 image: the bins that hold them are thousands of times fuller than
+    the host-side estimate they were sized for, so they take the path that streams a bin from memory, sorts lists of
+    thousands of keys in place and blends one thread per pixel."""
+    scene = synthetic.tiny_scene(num_points=30_000, w=96, h=64, num_layers=3, K=K, seed=61)
+    scene.position[:, 0] *= 0.02
+    scene.position[:, 1] *= 0.02
+    res, ref, _ = _parity(scene, rasterizer, oracle, backward=(K > 0), need_point_gradient=1)
+    counts = np.diff(res.offsets(0))
+    assert counts.max() > 2500 and (counts > 0).sum() < 40
