@@ -83,7 +83,15 @@ typedef struct vetrast_params
     int32_t camera_gradient_normalization;    /* 0: leave sums and counts; 1: divide each pose / intrinsics row by its
                                                  count as src/lib/rendering/PointRenderer.cu:1253-1308 does (the count
                                                  grows by 1/1024 per fragment, so this is 1024 x the mean) */
+    int32_t render_mode;                      /* RenderParams::render_mode, src/lib/data/Settings.h: 0 or 1 = FULL_BLEND
+                                                 (a point lands in the pixel it rounds to), 3 = BILINEAR_BLEND (a point
+                                                 lands in the 2x2 pixels around it, alpha = bilinear weight x confidence,
+                                                 blending stops once the transmittance falls below 0.001). Other values
+                                                 are refused. */
 } vetrast_params;
+
+#define VETRAST_RENDER_FULL_BLEND 1
+#define VETRAST_RENDER_BILINEAR_BLEND 3
 
 typedef struct vetrast_ctx vetrast_ctx;
 

@@ -31,7 +31,7 @@ def load():
         lib = C.CDLL(LIB_PATH)
         lib.vetref_forward.restype = C.c_int
         lib.vetref_forward.argtypes = [C.POINTER(abi.ForwardArgs), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
-                                       C.c_int]
+                                       C.c_void_p, C.c_int]
         lib.vetref_backward.restype = C.c_int
         lib.vetref_backward.argtypes = [C.POINTER(abi.BackwardArgs), C.c_void_p, C.c_void_p, C.c_int]
         lib.vetref_prepare_view.restype = C.c_int
@@ -55,7 +55,7 @@ class OracleForward:
         B, Cn, N, L = len(scene.views), scene.num_channels, scene.num_points, scene.num_layers
         self.sizes = scene.layer_sizes()
         self.P = sum(w * h for w, h in self.sizes)
-        self.cap = N * L
+        self.cap = N * L * (4 if params.render_mode == abi.RENDER_BILINEAR_BLEND else 1)
         self.out = [np.zeros((B, Cn, h, w), np.float32) for (w, h) in self.sizes]
         self.out_mask = [np.zeros((B, 1, h, w), np.float32) if params.output_background_mask else None
                          for (w, h) in self.sizes]
@@ -63,6 +63,7 @@ class OracleForward:
         self.fragments = np.zeros((B, max(self.cap, 1)), np.uint64)
         self.transmittance = np.zeros((B, max(self.cap, 1)), np.float32)
         self.weight = np.zeros((B, self.P), np.float32)
+        self.kept = np.zeros((B, self.P), np.uint32)  # fragments of every pixel that took part in the blend
         self.inputs = {k: (None if getattr(scene, k) is None else np.ascontiguousarray(getattr(scene, k)))
                        for k in ("position", "index", "texture", "confidence", "background", "dropout", "poses_se3",
                                  "intrinsics")}
@@ -74,7 +75,8 @@ class OracleForward:
             a.out_mask[l] = _addr(self.out_mask[l])
         self.args = a
         self.status = load().vetref_forward(C.byref(a), _addr(self.offsets), _addr(self.fragments),
-                                            _addr(self.transmittance), _addr(self.weight), num_threads)
+                                            _addr(self.transmittance), _addr(self.weight), _addr(self.kept),
+                                            num_threads)
 
     def layer_base(self, l):
         return sum(w * h for w, h in self.sizes[:l])

@@ -1,6 +1,6 @@
 // CPU oracle of the blending point rasterizer — TEST INFRASTRUCTURE ONLY (see vetrast_oracle.h).
 //
-// Scalar restatement of the reference's FULL_BLEND path. Every function names the reference lines it follows
+// Scalar restatement of the reference's FULL_BLEND and BILINEAR_BLEND paths. Every function names the reference lines it follows
 // (paths relative to the reference's src/lib/). Build with -ffp-contract=off: the canonical arithmetic has no
 // fused multiply-add, every operation is rounded on its own, in the order written here.
 #include "vetrast_oracle.h"
@@ -142,6 +142,62 @@ inline void for_each_layer_pixel(const Projected& pr, const Layers& ly, const ve
     }
 }
 
+// BILINEAR_BLEND: visits the up to four pixels around a point, layer by layer, with the corner number
+// y_j * 2 + x_i. The loops of CountingPrepassMulti<L,true> / CollectMulti<L,true>:
+// rendering/RenderForward.cu:863-885 and :1097-1134. __float2int_rd = floor.
+template <class F>
+inline void for_each_layer_corner(const Projected& pr, const Layers& ly, const vetrast_params& prm, F&& fn)
+{
+    float ipx = pr.ipx, ipy = pr.ipy, radius = pr.radius;
+    for (int l = 0; l < ly.L; ++l, radius *= 0.5f, ipx *= 0.5f, ipy *= 0.5f)
+    {
+        if (prm.drop_out_points_by_radius && radius < prm.drop_out_radius_threshold) break;
+        const float fx = std::floor(ipx), fy = std::floor(ipy);
+        for (int y_j = 0; y_j <= 1; ++y_j)
+            for (int x_i = 0; x_i <= 1; ++x_i)
+            {
+                const float px = fx + (float)x_i, py = fy + (float)y_j;
+                if (!(px >= 0.f && px < (float)ly.w[l] && py >= 0.f && py < (float)ly.h[l])) continue;
+                fn(l, (int)px, (int)py, y_j * 2 + x_i);
+            }
+    }
+}
+
+// Image position of a projected point at layer l: l exact halvings (RenderForward.cu:856).
+inline void layer_position(const Projected& pr, int l, float& ipx, float& ipy)
+{
+    ipx = pr.ipx;
+    ipy = pr.ipy;
+    for (int k = 0; k < l; ++k) ipx *= 0.5f, ipy *= 0.5f;
+}
+
+// compute_blending_fac, rendering/PointBlending.h:12-44: the four bilinear weights of a position and, optionally, their
+// derivatives J[corner][0..1] with respect to (x, y).
+inline void blending_fac(float u, float v, float fac[4], float J[4][2])
+{
+    const float sx = u - std::floor(u), sy = v - std::floor(v);
+    fac[0] = (1 - sx) * (1 - sy);
+    fac[1] = sx * (1 - sy);
+    fac[2] = (1 - sx) * sy;
+    fac[3] = sx * sy;
+    if (J)
+    {
+        J[0][0] = sy - 1;
+        J[0][1] = sx - 1;
+        J[1][0] = 1 - sy;
+        J[1][1] = -sx;
+        J[2][0] = -sy;
+        J[2][1] = 1 - sx;
+        J[3][0] = sy;
+        J[3][1] = sx;
+    }
+}
+
+inline bool is_bilinear(const vetrast_params& p)
+{
+    return p.render_mode == VETRAST_RENDER_BILINEAR_BLEND;
+}
+
 struct Scene
 {
     const vetrast_forward_args* a;
@@ -161,6 +217,8 @@ int validate(const vetrast_forward_args* a)
     if (p.num_layers < 1 || p.num_layers > VETRAST_MAX_LAYERS) return VETRAST_ERR_INVALID_ARG;
     if (p.num_texture_channels < 1 || p.num_texture_channels > VETRAST_MAX_CHANNELS) return VETRAST_ERR_INVALID_ARG;
     if (p.check_normal) return VETRAST_ERR_UNSUPPORTED;
+    if (p.render_mode != 0 && p.render_mode != VETRAST_RENDER_FULL_BLEND && !is_bilinear(p)) return VETRAST_ERR_UNSUPPORTED;
+    if (is_bilinear(p) && a->num_points > (1 << 30)) return VETRAST_ERR_INVALID_ARG;  // id and corner share 32 key bits
     for (int b = 0; b < a->num_views; ++b)
     {
         const vetrast_view& v = a->views[b];
@@ -179,7 +237,7 @@ Scene make_scene(const vetrast_forward_args* a)
     s.a   = a;
     s.ly  = make_layers(a->views[0].w, a->views[0].h, a->params.num_layers);
     s.P   = s.ly.base[s.ly.L];
-    s.cap = (int64_t)a->num_points * a->params.num_layers;
+    s.cap = (int64_t)a->num_points * a->params.num_layers * (is_bilinear(a->params) ? 4 : 1);
     for (int b = 0; b < a->num_views; ++b)
     {
         const vetrast_view& v = a->views[b];
@@ -216,6 +274,200 @@ inline void atomic_add(float* p, float v, bool parallel)
     }
     else
         *p += v;
+}
+
+struct PointGrad
+{
+    float gp[3];
+    double gpose[6];
+    float gk[5];
+};
+
+// ProjectPointPinholeBackward, rendering/PointRendererHelper.h:317-372, for zero distortion (J_p_dis = I), with the
+// crop transform scaled by 0.5^layer (all five coefficients, rendering/RenderBackward.cu:1381-1385 and :3100-3106):
+// image-space gradient (gxp, gyp) of layer l -> gradients of the point, the pose tangent and fx, fy, cx, cy, s.
+// J_point = R, J_p_div = [1/z 0 -x/z^2; 0 1/z -y/z^2].
+inline PointGrad project_point_backward(const Prepared& cam, const vetrast_view& v, int l, const float* p4, float gxp,
+                                        float gyp)
+{
+    PointGrad o;
+    for (int k = 0; k < 3; ++k) o.gp[k] = 0.f;
+    for (int k = 0; k < 6; ++k) o.gpose[k] = 0.0;
+    for (int k = 0; k < 5; ++k) o.gk[k] = 0.f;
+    const float scale = powf(0.5f, float(l));
+    const float cfx = v.crop_transform[0] * scale, cfy = v.crop_transform[1] * scale, cs = v.crop_transform[4] * scale;
+    const float px = p4[0], py = p4[1], pz = p4[2];
+    const float vx = ((cam.r[0] * px + cam.r[1] * py) + cam.r[2] * pz) + cam.t[0];
+    const float vy = ((cam.r[3] * px + cam.r[4] * py) + cam.r[5] * pz) + cam.t[1];
+    const float vz = ((cam.r[6] * px + cam.r[7] * py) + cam.r[8] * pz) + cam.t[2];
+    if (vz > 0.f)
+    {
+        const float ar = v.crop_rotation[0] * gxp + v.crop_rotation[2] * gyp;  // J_rot^T grad
+        const float br = v.crop_rotation[1] * gxp + v.crop_rotation[3] * gyp;
+        const float a2 = cfx * ar;  // J_p_K2^T
+        const float b2 = cs * ar + cfy * br;
+        const float d0 = cam.fx * a2;  // J_p_K1^T
+        const float d1 = cam.s * a2 + cam.fy * b2;
+        const float iz = 1.f / vz;
+        const float e0 = iz * d0, e1 = iz * d1;
+        const float e2 = (-vx * iz * iz) * d0 + (-vy * iz * iz) * d1;
+        o.gp[0]        = (cam.r[0] * e0 + cam.r[3] * e1) + cam.r[6] * e2;  // R^T
+        o.gp[1]        = (cam.r[1] * e0 + cam.r[4] * e1) + cam.r[7] * e2;
+        o.gp[2]        = (cam.r[2] * e0 + cam.r[5] * e1) + cam.r[8] * e2;
+        // J_pose^T e with J_pose = [I | -[view_p]x]: the tangent (translation, rotation) acts on the left,
+        // pose <- exp(tangent) * pose (ApplyTangent, rendering/PointRenderer.cu:1325-1341)
+        o.gpose[0] = e0;
+        o.gpose[1] = e1;
+        o.gpose[2] = e2;
+        o.gpose[3] = vy * e2 - vz * e1;  // view_p x e
+        o.gpose[4] = vz * e0 - vx * e2;
+        o.gpose[5] = vx * e1 - vy * e0;
+        // J_k_K1^T grad_p_k2: image = (fx*nx + s*ny + cx, fy*ny + cy), columns fx, fy, cx, cy, s
+        const float nx = vx / vz, ny = vy / vz;
+        o.gk[0] = nx * a2;
+        o.gk[1] = ny * b2;
+        o.gk[2] = a2;
+        o.gk[3] = b2;
+        o.gk[4] = ny * a2;
+    }
+    return o;
+}
+
+// The per-fragment scatter of rendering/RenderBackward.cu:1401-1459 (FULL_BLEND) and :3117-3175 (BILINEAR_BLEND); the
+// two differ in what they add to the pose count per fragment (1/1024 there, 1 here).
+inline void scatter_point_grad(const vetrast_backward_args* g, const vetrast_view& v, int point_id, const PointGrad& pg,
+                               float pose_count_step, float k_factor, bool par)
+{
+    if (g->grad_points)
+    {
+        for (int k = 0; k < 3; ++k) atomic_add(&g->grad_points[4 * (size_t)point_id + k], pg.gp[k], par);
+        atomic_add(&g->grad_point_count[point_id], 1.f, par);
+    }
+    if (g->grad_pose)
+    {
+        for (int k = 0; k < 6; ++k)
+        {
+            double* dst = &g->grad_pose[6 * (size_t)v.image_index + k];
+            if (par)
+            {
+#pragma omp atomic
+                *dst += pg.gpose[k];
+            }
+            else
+                *dst += pg.gpose[k];
+        }
+        atomic_add(&g->grad_pose_count[v.image_index], pose_count_step, par);
+    }
+    if (g->grad_intrinsics)  // g_k(4) *= 0 removes the skew
+    {
+        float gk[5] = {pg.gk[0], pg.gk[1], pg.gk[2], pg.gk[3], pg.gk[4]};
+        gk[4] *= 0;
+        for (int k = 0; k < 5; ++k)
+            atomic_add(&g->grad_intrinsics[13 * (size_t)v.camera_index + k], k_factor * gk[k], par);
+        // the eight distortion columns need saiga's distortion Jacobian: left at zero
+        atomic_add(&g->grad_intrinsics_count[v.camera_index], 1.f / 1024.f, par);
+    }
+}
+
+// One pixel of BlendBackwardsBilinear<C>, rendering/RenderBackward.cu:2893-3232, followed literally including the
+// O(n^2) inner loop. sum_back is the per-fragment gradient_sum_backwards row (indexed by list position).
+void bilinear_pixel_backward(const vetrast_backward_args* g, const Scene& s, int b, int l, int gx, int gy,
+                             uint32_t offset, int size_of_chunk, const uint64_t* frag, const float* G, float* sum_back,
+                             bool need_point_gradients, bool par)
+{
+    const vetrast_forward_args* a = &g->fwd;
+    const vetrast_params& pr      = a->params;
+    const Prepared& cam           = s.cams[b];
+    const vetrast_view& v         = a->views[b];
+    const int N = a->num_points, C = pr.num_texture_channels;
+    const int lw = s.ly.w[l], lh = s.ly.h[l];
+    const size_t plane = (size_t)lw * lh;
+    auto get_point_id      = [&](uint32_t pos) { return (int)((uint32_t)frag[pos] >> 2); };
+    auto sample_texture_id = [&](uint32_t pos) {
+        const int id = get_point_id(pos);
+        return a->index ? a->index[id] : id;
+    };
+    // per_point_data of the fragment: (uv, corner); uv is the projection of the point at this layer again
+    auto get_uv = [&](uint32_t pos, float& u, float& w2) {
+        Projected pp;
+        project(cam, v, a->position + 4 * (size_t)get_point_id(pos), pp);
+        layer_position(pp, l, u, w2);
+    };
+    auto get_subpixel_weight = [&](uint32_t pos) {
+        float u, w2, fac[4];
+        get_uv(pos, u, w2);
+        blending_fac(u, w2, fac, nullptr);
+        return fac[(uint32_t)frag[pos] & 3u];
+    };
+    {
+        float alpha_dest    = 1.f;
+        const int list_size = pr.use_environment_map ? size_of_chunk : size_of_chunk + 1;
+        for (int i = 0; i < list_size; ++i)
+        {
+            const bool is_foreground       = i != size_of_chunk;
+            const uint32_t full_buffer_pos = offset + (uint32_t)i;
+            int texture_index              = 0;
+            if (is_foreground) texture_index = sample_texture_id(full_buffer_pos);
+            float alpha_val = 1.f;
+            if (is_foreground) alpha_val = get_subpixel_weight(full_buffer_pos) * a->confidence[texture_index];
+            float colors[VETRAST_MAX_CHANNELS], grad_in[VETRAST_MAX_CHANNELS];
+            for (int ci = 0; ci < C; ++ci)
+                colors[ci] = is_foreground ? a->texture[(size_t)ci * N + texture_index] : a->background[ci];
+            float g_alpha = 0;
+            for (int ci = 0; ci < C; ++ci)
+            {
+                grad_in[ci]   = G[ci * plane + (size_t)gy * lw + gx];
+                float g_col   = alpha_dest * alpha_val * grad_in[ci];
+                float* target = is_foreground ? &g->grad_texture[(size_t)ci * N + texture_index] : &g->grad_background[ci];
+                atomic_add(target, g_col, par);
+                g_alpha += colors[ci] * grad_in[ci];
+            }
+            g_alpha *= alpha_dest;
+            if (is_foreground) sum_back[full_buffer_pos] += g_alpha;  // :2987 (guarded here, unlike FULL_BLEND)
+            for (int j = 0; j < i; ++j)
+            {
+                const uint32_t pos_iter    = offset + (uint32_t)j;
+                const int texture_iter     = sample_texture_id(pos_iter);
+                const float alpha_val_iter = get_subpixel_weight(pos_iter) * a->confidence[texture_iter];
+                float g_iter               = 0;
+                for (int ci = 0; ci < C; ++ci)
+                {
+                    const float epsilon = 1e-9;
+                    float g_alpha_iter  = (grad_in[ci] * colors[ci] * alpha_dest * alpha_val / (1 - alpha_val_iter + epsilon));
+                    g_iter -= g_alpha_iter;
+                }
+                sum_back[pos_iter] += g_iter;
+            }
+            alpha_dest = compute_new_alphadest(alpha_dest, alpha_val);
+            if (alpha_dest < 0.001)  // :3014-3019: later fragments took no part in the forward blend either
+            {
+                if (is_foreground) size_of_chunk = i + 1;
+                break;
+            }
+        }
+    }
+    // confidence and position gradients, only for pixels more than 2 away from the border (:3044)
+    const int edge = std::min(std::min(gx, gy), std::min(lw - 1 - gx, lh - 1 - gy));
+    if (!(edge > 2)) return;
+    for (int i = 0; i < size_of_chunk; ++i)
+    {
+        const uint32_t full_buffer_pos = offset + (uint32_t)i;
+        const int texture_index        = sample_texture_id(full_buffer_pos);
+        float u, w2, fac[4], J[4][2];
+        get_uv(full_buffer_pos, u, w2);
+        const int blend_index  = (int)((uint32_t)frag[full_buffer_pos] & 3u);
+        const float grad_alpha = sum_back[full_buffer_pos];
+        blending_fac(u, w2, fac, J);
+        atomic_add(&g->grad_confidence[texture_index], fac[blend_index] * grad_alpha, par);  // dA/dc = blend factor
+        if (!need_point_gradients) continue;
+        const float grad_blend_single = a->confidence[texture_index] * grad_alpha;  // dA/db = confidence
+        // dR_dp = J_uv_b^T * grad_blending, grad_blending zero but for this corner (:3083-3088)
+        const float gxp    = J[blend_index][0] * grad_blend_single;
+        const float gyp    = J[blend_index][1] * grad_blend_single;
+        const int point_id = get_point_id(full_buffer_pos);
+        const PointGrad pg = project_point_backward(cam, v, l, a->position + 4 * (size_t)point_id, gxp, gyp);
+        scatter_point_grad(g, v, point_id, pg, 1.f, pr.K_gradient_factor, par);  // pose count +1 here (:3146)
+    }
 }
 
 }  // namespace
@@ -261,7 +513,7 @@ extern "C" int vetref_project_point(const float* m, const vetrast_view* view, co
 // Forward pass. Host sequence of BlendPointCloudForward, rendering/PointRenderer.cu:768-899:
 // counting pass, exclusive scan, collection pass, per-pixel sort, blend.
 extern "C" int vetref_forward(const vetrast_forward_args* a, uint32_t* offsets, uint64_t* fragments,
-                              float* transmittance, float* weight, int num_threads)
+                              float* transmittance, float* weight, uint32_t* kept, int num_threads)
 {
     int st = validate(a);
     if (st != VETRAST_OK) return st;
@@ -274,6 +526,7 @@ extern "C" int vetref_forward(const vetrast_forward_args* a, uint32_t* offsets, 
     const int K              = a->params.debug_max_list_length;
     const vetrast_params& pr = a->params;
     const bool par           = num_threads > 1;
+    const bool bilinear      = is_bilinear(pr);
 #ifdef _OPENMP
     omp_set_num_threads(num_threads > 0 ? num_threads : 1);
 #endif
@@ -285,6 +538,7 @@ extern "C" int vetref_forward(const vetrast_forward_args* a, uint32_t* offsets, 
         uint32_t* off         = offsets + (size_t)b * (s.P + 1);
         uint64_t* frag        = fragments + (size_t)b * s.cap;
         float* wgt            = weight + (size_t)b * s.P;
+        uint32_t* kept_b      = kept ? kept + (size_t)b * s.P : nullptr;
         std::vector<uint32_t> count((size_t)s.P, 0u), cursor((size_t)s.P, 0u);
 
         // CountingPrepassMulti<L,false>, rendering/RenderForward.cu:806-905 (the depth atomicMin image is not
@@ -295,13 +549,17 @@ extern "C" int vetref_forward(const vetrast_forward_args* a, uint32_t* offsets, 
             if (point_skipped(a, b, i)) continue;
             Projected p;
             if (!project(cam, v, a->position + 4 * (size_t)i, p)) continue;
-            for_each_layer_pixel(p, s.ly, pr, [&](int l, int x, int y) {
+            auto hit = [&](int l, int x, int y) {
                 uint32_t* c = &count[(size_t)(s.ly.base[l] + (int64_t)y * s.ly.w[l] + x)];
                 if (par)
                     __atomic_fetch_add(c, 1u, __ATOMIC_RELAXED);
                 else
                     ++*c;
-            });
+            };
+            if (bilinear)
+                for_each_layer_corner(p, s.ly, pr, [&](int l, int x, int y, int) { hit(l, x, y); });
+            else
+                for_each_layer_pixel(p, s.ly, pr, hit);
         }
 
         // thrust::exclusive_scan per layer, rendering/PointRenderer.cu:799-813. The layers are concatenated here,
@@ -322,16 +580,23 @@ extern "C" int vetref_forward(const vetrast_forward_args* a, uint32_t* offsets, 
             if (point_skipped(a, b, i)) continue;
             Projected p;
             if (!project(cam, v, a->position + 4 * (size_t)i, p)) continue;
-            const uint64_t key = ((uint64_t)float_bits(p.z) << 32) | (uint32_t)i;
-            for_each_layer_pixel(p, s.ly, pr, [&](int l, int x, int y) {
+            // Record: depth bits above the point id. In BILINEAR_BLEND the reference keeps (id, ip, corner) in a side
+            // table addressed through the record (RenderForward.cu:1112-1128); here the corner rides in the two low
+            // key bits next to the id, and ip is the (deterministic) projection of that point again.
+            auto put = [&](int l, int x, int y, uint32_t low) {
                 const size_t q = (size_t)(s.ly.base[l] + (int64_t)y * s.ly.w[l] + x);
                 uint32_t slot;
                 if (par)
                     slot = __atomic_fetch_add(&cursor[q], 1u, __ATOMIC_RELAXED);
                 else
                     slot = cursor[q]++;
-                frag[off[q] + slot] = key;
-            });
+                frag[off[q] + slot] = ((uint64_t)float_bits(p.z) << 32) | low;
+            };
+            if (bilinear)
+                for_each_layer_corner(p, s.ly, pr,
+                                      [&](int l, int x, int y, int corner) { put(l, x, y, ((uint32_t)i << 2) | (uint32_t)corner); });
+            else
+                for_each_layer_pixel(p, s.ly, pr, [&](int l, int x, int y) { put(l, x, y, (uint32_t)i); });
         }
 
         // SortMulti, rendering/RenderForward.cu:1277-1300 and rendering/AlphaListSort.cu:23-32: ascending depth per
@@ -354,11 +619,24 @@ extern "C" int vetref_forward(const vetrast_forward_args* a, uint32_t* offsets, 
                     float alpha_dest = 1.f;
                     float color_out[VETRAST_MAX_CHANNELS];
                     for (int ci = 0; ci < C; ++ci) color_out[ci] = 0.f;
+                    int blended = 0;  // fragments that took part
                     for (int i = 0; i < size_of_chunk; ++i)
                     {
-                        const int point_id      = (int)(uint32_t)frag[o + i];
+                        const uint32_t low      = (uint32_t)frag[o + i];
+                        const int point_id      = bilinear ? (int)(low >> 2) : (int)low;
                         const int texture_index = a->index ? a->index[point_id] : point_id;
-                        const float conf        = a->confidence[texture_index];
+                        float conf              = a->confidence[texture_index];
+                        if (bilinear)
+                        {
+                            // BlendMultiBilinear, rendering/RenderForward.cu:1539-1644: alpha = bilinear weight of
+                            // this pixel's corner x confidence
+                            Projected pp;
+                            project(cam, v, a->position + 4 * (size_t)point_id, pp);
+                            float u, w2, fac[4];
+                            layer_position(pp, l, u, w2);
+                            blending_fac(u, w2, fac, nullptr);
+                            conf = fac[low & 3u] * conf;
+                        }
                         if (transmittance) transmittance[(size_t)b * s.cap + o + i] = alpha_dest;
                         for (int ci = 0; ci < C; ++ci)
                         {
@@ -366,10 +644,13 @@ extern "C" int vetref_forward(const vetrast_forward_args* a, uint32_t* offsets, 
                             color_out[ci]     = compute_blend(alpha_dest, conf, color, color_out[ci]);
                         }
                         alpha_dest = compute_new_alphadest(alpha_dest, conf);
+                        ++blended;
+                        if (bilinear && alpha_dest < 0.001) break;  // RenderForward.cu:1626 (compared as double)
                     }
+                    if (kept_b) kept_b[q] = (uint32_t)blended;
                     for (int ci = 0; ci < C; ++ci)
                     {
-                        if (!pr.use_environment_map)
+                        if (!pr.use_environment_map && (!bilinear || alpha_dest >= 0.001))  // :1633-1636
                             color_out[ci] = compute_blend(alpha_dest, 1.f, a->background[ci], color_out[ci]);
                         out[((size_t)ci * lh + y) * lw + x] = color_out[ci];
                     }
@@ -426,12 +707,16 @@ extern "C" int vetref_backward(const vetrast_backward_args* g, const uint32_t* o
     }
     const bool need_point_gradients = pr.need_point_gradient && (g->grad_points || g->grad_pose || g->grad_intrinsics);
 
+    const bool bilinear = is_bilinear(pr);
+    // gradient_sum_backwards: one zeroed float per fragment, rendering/PointRenderer.cu:1186-1200
+    std::vector<float> sum_back(bilinear ? (size_t)s.cap : 0, 0.f);
     for (int b = 0; b < a->num_views; ++b)
     {
         const Prepared& cam   = s.cams[b];
         const vetrast_view& v = a->views[b];
         const uint32_t* off   = offsets + (size_t)b * (s.P + 1);
         const uint64_t* frag  = fragments + (size_t)b * s.cap;
+        std::fill(sum_back.begin(), sum_back.end(), 0.f);
         for (int l = 0; l < s.ly.L; ++l)
         {
             const int lw = s.ly.w[l], lh = s.ly.h[l];
@@ -446,6 +731,12 @@ extern "C" int vetref_backward(const vetrast_backward_args* g, const uint32_t* o
                     const uint32_t offset      = off[q];
                     int size_of_chunk          = (int)(off[q + 1] - offset);
                     if (K > 0) size_of_chunk   = std::min(K, size_of_chunk);  // RenderBackward.cu:1098-1100
+                    if (bilinear)
+                    {
+                        bilinear_pixel_backward(g, s, b, l, gx, gy, offset, size_of_chunk, frag, G, sum_back.data() + 0,
+                                                need_point_gradients, par);
+                        continue;
+                    }
                     auto sample_point_id       = [&](int pos) { return (int)(uint32_t)frag[pos]; };
                     auto sample_texture_index  = [&](int pos) {
                         const int id = sample_point_id(pos);
@@ -526,80 +817,9 @@ extern "C" int vetref_backward(const vetrast_backward_args* g, const uint32_t* o
                             dR_dpy += 0.5f * (dI_dp_at_py0 + dI_dp_at_py1);
                         }
                         const float gxp = dR_dpx / float(C), gyp = dR_dpy / float(C);  // :1374
-                        // crop_transform.scale(0.5^layer): all five coefficients, RenderBackward.cu:1381-1385
-                        const float scale = powf(0.5f, float(l));
-                        const float cfx = v.crop_transform[0] * scale, cfy = v.crop_transform[1] * scale,
-                                    cs = v.crop_transform[4] * scale;
-                        // ProjectPointPinholeBackward, rendering/PointRendererHelper.h:317-372 (zero distortion:
-                        // J_p_dis = I); J_point = R, J_p_div = [1/z 0 -x/z^2; 0 1/z -y/z^2].
-                        const float* p4 = a->position + 4 * (size_t)point_id;
-                        const float px = p4[0], py = p4[1], pz = p4[2];
-                        const float vx = ((cam.r[0] * px + cam.r[1] * py) + cam.r[2] * pz) + cam.t[0];
-                        const float vy = ((cam.r[3] * px + cam.r[4] * py) + cam.r[5] * pz) + cam.t[1];
-                        const float vz = ((cam.r[6] * px + cam.r[7] * py) + cam.r[8] * pz) + cam.t[2];
-                        float gp[3] = {0.f, 0.f, 0.f};
-                        double gpose[6] = {0, 0, 0, 0, 0, 0};
-                        float gk[5]     = {0.f, 0.f, 0.f, 0.f, 0.f};
-                        if (vz > 0.f)
-                        {
-                            const float ar = v.crop_rotation[0] * gxp + v.crop_rotation[2] * gyp;  // J_rot^T grad
-                            const float br = v.crop_rotation[1] * gxp + v.crop_rotation[3] * gyp;
-                            const float a2 = cfx * ar;            // J_p_K2^T
-                            const float b2 = cs * ar + cfy * br;
-                            const float d0 = cam.fx * a2;         // J_p_K1^T
-                            const float d1 = cam.s * a2 + cam.fy * b2;
-                            const float iz = 1.f / vz;
-                            const float e0 = iz * d0, e1 = iz * d1;
-                            const float e2 = (-vx * iz * iz) * d0 + (-vy * iz * iz) * d1;
-                            gp[0]          = (cam.r[0] * e0 + cam.r[3] * e1) + cam.r[6] * e2;  // R^T
-                            gp[1]          = (cam.r[1] * e0 + cam.r[4] * e1) + cam.r[7] * e2;
-                            gp[2]          = (cam.r[2] * e0 + cam.r[5] * e1) + cam.r[8] * e2;
-                            // J_pose^T e with J_pose = [I | -[view_p]x]: the tangent (translation, rotation) acts on
-                            // the left, pose <- exp(tangent) * pose (ApplyTangent, rendering/PointRenderer.cu:1325-1341)
-                            gpose[0] = e0;
-                            gpose[1] = e1;
-                            gpose[2] = e2;
-                            gpose[3] = vy * e2 - vz * e1;  // view_p x e
-                            gpose[4] = vz * e0 - vx * e2;
-                            gpose[5] = vx * e1 - vy * e0;
-                            // J_k_K1^T grad_p_k2: image = (fx*nx + s*ny + cx, fy*ny + cy), columns fx, fy, cx, cy, s
-                            const float nx = vx / vz, ny = vy / vz;
-                            gk[0] = nx * a2;
-                            gk[1] = ny * b2;
-                            gk[2] = a2;
-                            gk[3] = b2;
-                            gk[4] = ny * a2;
-                        }
-                        if (g->grad_points)
-                        {
-                            for (int k = 0; k < 3; ++k)
-                                atomic_add(&g->grad_points[4 * (size_t)point_id + k], gp[k], par);
-                            atomic_add(&g->grad_point_count[point_id], 1.f, par);  // RenderBackward.cu:1407
-                        }
-                        if (g->grad_pose)  // RenderBackward.cu:1418-1426
-                        {
-                            for (int k = 0; k < 6; ++k)
-                            {
-                                double* dst = &g->grad_pose[6 * (size_t)v.image_index + k];
-                                if (par)
-                                {
-#pragma omp atomic
-                                    *dst += gpose[k];
-                                }
-                                else
-                                    *dst += gpose[k];
-                            }
-                            atomic_add(&g->grad_pose_count[v.image_index], 1.f / 1024.f, par);
-                        }
-                        if (g->grad_intrinsics)  // RenderBackward.cu:1428-1459; g_k(4) *= 0 removes the skew
-                        {
-                            gk[4] *= 0;
-                            for (int k = 0; k < 5; ++k)
-                                atomic_add(&g->grad_intrinsics[13 * (size_t)v.camera_index + k],
-                                           pr.K_gradient_factor * gk[k], par);
-                            // the eight distortion columns need saiga's distortion Jacobian: left at zero
-                            atomic_add(&g->grad_intrinsics_count[v.camera_index], 1.f / 1024.f, par);
-                        }
+                        const PointGrad pg =
+                            project_point_backward(cam, v, l, a->position + 4 * (size_t)point_id, gxp, gyp);
+                        scatter_point_grad(g, v, point_id, pg, 1.f / 1024.f, pr.K_gradient_factor, par);
                     }
                 }
         }

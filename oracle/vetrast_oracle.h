@@ -1,7 +1,8 @@
 /*
  * CPU oracle of the blending point rasterizer — TEST INFRASTRUCTURE ONLY.
  *
- * A plain scalar restatement of the reference's FULL_BLEND path (lfranke/VET, src/lib/rendering). It exists to
+ * A plain scalar restatement of the reference's FULL_BLEND path and of its BILINEAR_BLEND path (params.render_mode = 3)
+ * (lfranke/VET, src/lib/rendering). It exists to
  * check the GPU library and to be timed as the CPU baseline; nothing that ships may call it. Only tests/,
  * __graft_entry__.smoke() and bench.py's cpu_baseline leg load this library.
  *
@@ -9,7 +10,8 @@
  * the workspace ignored; saved state goes to explicit caller-allocated arrays instead:
  *   offsets       uint32 [B][P+1]   exclusive scan of per-pixel counts, pixels of all layers concatenated
  *   fragments     uint64 [B][N*L]   (depth_bits << 32) | point_id; every pixel list fully sorted ascending
- *   transmittance float  [B][N*L]   transmittance in front of fragment i for i < min(count, K)
+ *                                   (BILINEAR_BLEND: [B][4*N*L], low word = point_id << 2 | corner, corner = 2*dy + dx)
+ *   transmittance float  [B][N*L]   transmittance in front of fragment i for every fragment that took part in the blend
  *   weight        float  [B][P]     final transmittance per pixel
  *
  * Parity status of the pieces (what pins each is in tests/test_oracle_*.py):
@@ -23,6 +25,10 @@
  *   value gradients   pinned by double-precision central differences of an independent numpy blend
  *   position gradient literal restatement; the heuristic is checked on hand-computed cases, the projection Jacobian
  *                     by finite differences; saiga's operator order inside the Jacobians is PARITY UNPINNED
+ *   bilinear mode     splat weights pinned by closed forms (weights of a point sum to 1 over its 2x2 pixels, a point on
+ *                     a pixel centre lands in one pixel), the blend and its early exit by an independent numpy blend,
+ *                     value and position gradients by double-precision central differences of that blend (the
+ *                     position gradient is analytic in this mode, so finite differences do pin it)
  *   distortion != 0, check_normal, OCam, spherical: not implemented (rejected), PARITY UNPINNED
  */
 #ifndef VETRAST_ORACLE_H
@@ -41,8 +47,10 @@ int vetref_prepare_view(const double* pose8, const float* intrinsics13, float* o
 /* Project one point for one prepared view; returns 0 if rejected (z == 0). ip_z_r = {ip.x, ip.y, z, radius_px}. */
 int vetref_project_point(const float* prepared17, const vetrast_view* view, const float* position4, float* ip_z_r);
 
+/* kept (optional): uint32 [B][P], the number of fragments of every pixel that took part in the blend: min(count, K), and
+ * in BILINEAR_BLEND also cut where the transmittance fell below 0.001. */
 int vetref_forward(const vetrast_forward_args* args, uint32_t* offsets, uint64_t* fragments, float* transmittance,
-                   float* weight, int num_threads);
+                   float* weight, uint32_t* kept, int num_threads);
 
 int vetref_backward(const vetrast_backward_args* args, const uint32_t* offsets, const uint64_t* fragments,
                     int num_threads);

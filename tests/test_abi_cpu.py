@@ -30,7 +30,7 @@ def test_library_exports_every_declared_symbol():
 def test_struct_sizes_are_the_c_ones():
     # sizes the C compiler gives the structs of include/vetrast.h (LP64)
     assert C.sizeof(abi.View) == 5 * 4 + 9 * 4
-    assert C.sizeof(abi.Params) == 16 * 4
+    assert C.sizeof(abi.Params) == 17 * 4
     assert C.sizeof(abi.ForwardArgs) % 8 == 0
     assert abi.BackwardArgs.grad_out.offset == C.sizeof(abi.ForwardArgs)
 

@@ -19,6 +19,9 @@ CAMERA_PINHOLE_DISTORTION = 0
 CAMERA_OCAM = 1
 CAMERA_SPHERICAL = 2
 
+RENDER_FULL_BLEND = 1
+RENDER_BILINEAR_BLEND = 3
+
 SCOPE_NAMES = [
     "PREPARE", "PACK", "COUNT", "SCAN", "FILL", "BUILD", "BACKWARD_PREPARE", "BACKWARD_BLEND", "BACKWARD_GATHER", "BACKWARD_POST",
 ]
@@ -52,6 +55,7 @@ class Params(C.Structure):
         ("point_gradient_normalization", C.c_int32),
         ("K_gradient_factor", C.c_float),
         ("camera_gradient_normalization", C.c_int32),
+        ("render_mode", C.c_int32),
     ]
 
 

@@ -33,6 +33,7 @@ def make_params(scene: Scene, **overrides) -> abi.Params:
     p.point_gradient_normalization = 0
     p.K_gradient_factor = 0.5
     p.camera_gradient_normalization = 0
+    p.render_mode = abi.RENDER_FULL_BLEND
     for k, v in {**scene.params, **overrides}.items():
         if not hasattr(p, k):
             raise AttributeError(f"vetrast_params has no field {k}")
