@@ -125,7 +125,9 @@ typedef struct vetrast_workspace_layout
     int32_t reserved0;
     int64_t layer_tile_base[VETRAST_MAX_LAYERS + 1];  /* first tile of the layer; [L] = number of tiles T */
     int64_t layer_pixel_base[VETRAST_MAX_LAYERS + 1]; /* 256 * layer_tile_base; [L] = pixel numbers P of one view */
-    int64_t fragment_capacity;                        /* N * L, the per-view upper bound on fragments */
+    int64_t fragment_capacity;                        /* N * L * hits_per_layer, the per-view upper bound on fragments */
+    int32_t hits_per_layer;                           /* 1 (FULL_BLEND) or 4 (BILINEAR_BLEND): fragments of a point per layer */
+    int32_t reserved1;
     size_t total_bytes;
     /* per-view arrays: offset of view b = base + b * stride */
     size_t offsets_base, offsets_stride;     /* uint32 [P+1]: exclusive scan of per-pixel counts; [P] = fragments of the view */
@@ -133,7 +135,8 @@ typedef struct vetrast_workspace_layout
                                                 first min(count, K) entries of a pixel's list are sorted and meaningful */
     size_t transmittance_base, transmittance_stride; /* float [N*L]: transmittance in front of each kept fragment */
     size_t weight_base, weight_stride;       /* float [P]: final transmittance per pixel (the reference's `weight` image) */
-    size_t cut_flags_base, cut_flags_stride; /* uint8 [P]: 1 where the top-K cut dropped fragments of the pixel */
+    size_t kept_base, kept_stride;           /* uint32 [P]: fragments of the pixel's list that took part in the blend */
+    size_t cut_flags_base, cut_flags_stride; /* uint8 [P]: 1 where some fragments of the pixel's list did not (top-K cut, saturation) */
     /* shared by all views */
     size_t packed_base;    /* float [N][8]: descriptor (4, zero padded), confidence, 3 pad */
     size_t slots_base;     /* uint32 [L][N]: per (layer, point) arrival rank inside its tile (scratch between two passes) */
@@ -210,6 +213,10 @@ int vetrast_layer_sizes(int32_t w, int32_t h, int32_t num_layers, int32_t* layer
  * here the buffer has the upper bound N*L entries per view instead, so no read-back is needed. */
 int vetrast_workspace_layout_for(int32_t num_points, int32_t num_views, int32_t num_layers, int32_t w, int32_t h,
                                  vetrast_workspace_layout* layout);
+/* The same for a given render mode (BILINEAR_BLEND needs room for four fragments per point and layer);
+ * vetrast_workspace_layout_for and vetrast_forward_workspace_bytes are the FULL_BLEND case. */
+int vetrast_workspace_layout_for_mode(int32_t num_points, int32_t num_views, int32_t num_layers, int32_t w, int32_t h,
+                                      int32_t render_mode, vetrast_workspace_layout* layout);
 size_t vetrast_forward_workspace_bytes(int32_t num_points, int32_t num_views, int32_t num_layers, int32_t w, int32_t h);
 
 /* Forward: project, count, scan, fill, per-pixel sort by (depth bits, point id), top-K cut, front-to-back blend.

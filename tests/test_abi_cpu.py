@@ -65,6 +65,7 @@ def test_workspace_layout_is_aligned_and_disjoint():
         ("tile_counts", lay.bin_counts_base, lay.bin_counts_stride * B),
         ("binned", lay.binned_base, N * L * 16),
         ("cut_flags", lay.cut_flags_base, lay.cut_flags_stride * B),
+        ("kept", lay.kept_base, lay.kept_stride * B),
         ("fragments", lay.fragments_base, lay.fragments_stride * B),
         ("transmittance", lay.transmittance_base, lay.transmittance_stride * B),
         ("weight", lay.weight_base, lay.weight_stride * B),
@@ -93,6 +94,11 @@ def test_workspace_layout_is_aligned_and_disjoint():
     assert lib.vetrast_workspace_layout_for(N, B, 5, 8, 8, C.byref(lay)) == abi.ERR_INVALID_ARG  # coarsest layer empty
     assert lib.vetrast_workspace_layout_for(2_000_000_000, B, 4, w, h, C.byref(lay)) == abi.ERR_INVALID_ARG
     assert lib.vetrast_forward_workspace_bytes(N, 0, L, w, h) == 0
+    # BILINEAR_BLEND: four fragments per point and layer
+    full = lay.total_bytes
+    assert lib.vetrast_workspace_layout_for_mode(N, B, L, w, h, abi.RENDER_BILINEAR_BLEND, C.byref(lay)) == 0
+    assert lay.hits_per_layer == 4 and lay.fragment_capacity == 4 * N * L and lay.total_bytes > 3 * full
+    assert lib.vetrast_workspace_layout_for_mode(N, B, L, w, h, 2, C.byref(lay)) == abi.ERR_UNSUPPORTED
 
 
 def test_status_and_scope_names():

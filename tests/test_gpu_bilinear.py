@@ -1,0 +1,86 @@
+"""GPU parity of BILINEAR_BLEND (render_mode 3): the HIP path through the C ABI against the CPU oracle.
+
+Bars as for the other mode: per-pixel counts and the blended part of every fragment list bit-exact, stored
+transmittances, weights and blended features bit-exact (same operation order), gradients within 1e-4 relative.
+"""
+import numpy as np
+import pytest
+import torch
+
+from tests.helpers import max_rel_err
+from vet_amd import abi, synthetic
+from vet_amd.rasterizer import DeviceScene, make_params
+
+pytestmark = pytest.mark.gpu
+MODE = dict(render_mode=abi.RENDER_BILINEAR_BLEND)
+
+
+def _opaque(scene, factor=1.6):
+    scene.confidence[:] = np.clip(scene.confidence * factor, 0, 0.98)  # so that the 0.001 cut triggers
+    return scene
+
+
+def _scenes():
+    yield "tiny_K4", synthetic.tiny_scene(), {}
+    yield "tiny_dense_K16", _opaque(synthetic.tiny_scene(num_points=6000, K=16, seed=71)), {}
+    yield "tiny_dense_nocut_3ch", _opaque(synthetic.tiny_scene(num_points=5000, K=-1, channels=3, seed=72)), {}
+    yield "tiny_long_lists", _opaque(synthetic.tiny_scene(num_points=40000, K=0, seed=73), 1.0), {}
+    yield "tiny_2views_envmap", synthetic.tiny_scene(num_points=3000, K=8, num_views=2, seed=74), {"use_environment_map": 1}
+    yield "tiny_radius_dropout", synthetic.tiny_scene(num_points=3000, K=8, seed=75), {"drop_out_points_by_radius": 1}
+    yield "odd_size_5_layers", synthetic.tiny_scene(num_points=9000, w=83, h=61, num_layers=5, K=6, seed=76), {}
+    yield "config1", synthetic.config1(), {}
+    yield "config2_200k", synthetic.config2(num_points=200_000), {}
+
+
+SCENES = list(_scenes())
+
+
+def _blended_mask(off, kept):
+    """True for the fragments of every list that took part in the blend (the first kept[q] of each)."""
+    counts = np.diff(off)
+    rank = np.arange(off[-1], dtype=np.int64) - np.repeat(off[:-1], counts)
+    return rank < np.repeat(kept, counts)
+
+
+def _check_forward(scene, overrides, rasterizer, oracle):
+    params = make_params(scene, **{**overrides, **MODE})
+    ref = oracle.forward(scene, params)
+    dev = DeviceScene(scene)
+    res = rasterizer.forward(dev, params, save_for_backward=True)
+    torch.cuda.synchronize()
+    assert rasterizer.check_device_flags(res) == 0
+    saturated = 0
+    for b in range(len(scene.views)):
+        off = res.offsets(b)
+        np.testing.assert_array_equal(off, ref.offsets[b].astype(np.int64), err_msg="per-pixel counts differ")
+        total = int(off[-1])
+        kept = res.kept(b)
+        np.testing.assert_array_equal(kept, ref.kept[b].astype(np.int64), err_msg="blended fragment counts differ")
+        K = params.debug_max_list_length
+        saturated += int((kept < (np.minimum(np.diff(off), K) if K > 0 else np.diff(off))).sum())
+        m = _blended_mask(off, kept)
+        np.testing.assert_array_equal(res.fragments(b)[m], ref.fragments[b, :total][m], err_msg="fragment lists differ")
+        np.testing.assert_array_equal(res.transmittance(b)[m], ref.transmittance[b, :total][m])
+        np.testing.assert_array_equal(res.weight(b), ref.weight[b])
+    for l in range(scene.num_layers):
+        np.testing.assert_array_equal(res.out[l].cpu().numpy(), ref.out[l])
+    return ref, dev, res, saturated
+
+
+@pytest.mark.parametrize("name,scene,overrides", SCENES, ids=[s[0] for s in SCENES])
+def test_forward_matches_oracle(name, scene, overrides, rasterizer, oracle):
+    _, _, _, saturated = _check_forward(scene, overrides, rasterizer, oracle)
+    if "nocut" in name or "long" in name:
+        assert saturated > 50, "the scene must exercise the early exit"
+
+
+def test_mode_3_needs_the_bigger_workspace(rasterizer):
+    scene = synthetic.tiny_scene(num_points=500)
+    dev = DeviceScene(scene)
+    small = torch.empty(rasterizer.layout(scene).total_bytes, dtype=torch.uint8, device="cuda")
+    with pytest.raises(abi.VetrastError) as e:
+        rasterizer.forward(dev, make_params(scene, **MODE), workspace=small)
+    assert e.value.status == abi.ERR_WORKSPACE_SMALL
+    with pytest.raises(abi.VetrastError) as e:
+        rasterizer.forward(dev, make_params(scene, render_mode=2))
+    assert e.value.status == abi.ERR_UNSUPPORTED

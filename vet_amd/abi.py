@@ -68,11 +68,14 @@ class WorkspaceLayout(C.Structure):
         ("layer_tile_base", C.c_int64 * (MAX_LAYERS + 1)),
         ("layer_pixel_base", C.c_int64 * (MAX_LAYERS + 1)),
         ("fragment_capacity", C.c_int64),
+        ("hits_per_layer", C.c_int32),
+        ("reserved1", C.c_int32),
         ("total_bytes", C.c_size_t),
         ("offsets_base", C.c_size_t), ("offsets_stride", C.c_size_t),
         ("fragments_base", C.c_size_t), ("fragments_stride", C.c_size_t),
         ("transmittance_base", C.c_size_t), ("transmittance_stride", C.c_size_t),
         ("weight_base", C.c_size_t), ("weight_stride", C.c_size_t),
+        ("kept_base", C.c_size_t), ("kept_stride", C.c_size_t),
         ("cut_flags_base", C.c_size_t), ("cut_flags_stride", C.c_size_t),
         ("packed_base", C.c_size_t),
         ("slots_base", C.c_size_t),
@@ -133,6 +136,8 @@ SYMBOLS = {
     "vetrast_layer_sizes": (C.c_int, [C.c_int32, C.c_int32, C.c_int32, C.POINTER(C.c_int32), C.POINTER(C.c_int32)]),
     "vetrast_workspace_layout_for": (C.c_int, [C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_int32,
                                                C.POINTER(WorkspaceLayout)]),
+    "vetrast_workspace_layout_for_mode": (C.c_int, [C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_int32,
+                                                    C.POINTER(WorkspaceLayout)]),
     "vetrast_forward_workspace_bytes": (C.c_size_t, [C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_int32]),
     "vetrast_forward": (C.c_int, [C.c_void_p, C.POINTER(ForwardArgs), C.c_void_p]),
     "vetrast_backward": (C.c_int, [C.c_void_p, C.POINTER(BackwardArgs), C.c_void_p]),

@@ -30,7 +30,10 @@ struct BuildPass
     uint32_t* offsets;    // [P + 1] per pixel: start of its list; [P] = fragments of the view
     uint64_t* fragments;
     uint8_t* list_is_cut;   // [P]
+    uint32_t* kept;         // [P] fragments of the pixel that took part in the blend
     // blending
+    const float4* position;   // BILINEAR_BLEND only: the alpha of a fragment depends on where its point projects to
+    const DeviceView* view;
     const int32_t* index;
     const float4* packed;
     const float* background;
@@ -46,7 +49,33 @@ struct BuildPass
     float mask_value;
 };
 
-template <int C>
+// Alpha of a fragment: the point's confidence, in BILINEAR_BLEND times the bilinear weight of the pixel's corner at the
+// point's position in this layer (BlendMultiBilinear, src/lib/rendering/RenderForward.cu:1586-1613). The position is
+// the same projection the binning passes computed, so the weight is reproduced bit for bit.
+template <bool BILINEAR>
+__device__ __forceinline__ float fragment_alpha(const BuildPass& a, int l, uint32_t low, float confidence)
+{
+    if constexpr (!BILINEAR)
+        return confidence;
+    else
+    {
+        Projected p;
+        if (!project_point(*a.view, a.position[low >> 2], p)) return 0.f;  // cannot happen for a listed fragment
+        float u = p.ipx, v = p.ipy;
+        for (int k = 0; k < l; ++k) u *= 0.5f, v *= 0.5f;
+        return bilinear_weight(u, v, (int)(low & 3u)) * confidence;
+    }
+}
+
+// BILINEAR_BLEND stops a pixel once its transmittance is below 0.001 (compared in double as in the reference,
+// src/lib/rendering/RenderForward.cu:1626) and then leaves the background out as well (:1633).
+template <bool BILINEAR>
+__device__ __forceinline__ bool blend_is_saturated(float T)
+{
+    return BILINEAR && (double)T < 0.001;
+}
+
+template <int C, bool BILINEAR>
 __global__ void __launch_bounds__(kBlock) bin_build_kernel(BuildPass a)
 {
     __shared__ uint32_t s_cnt[kTilePixels];
@@ -54,6 +83,7 @@ __global__ void __launch_bounds__(kBlock) bin_build_kernel(BuildPass a)
     __shared__ uint32_t s_wave_tot[kBlock / kWave];
     __shared__ uint8_t s_src_lane[kBlock / kWave][kWave];
     __shared__ uint64_t s_keys[kBuildCap];
+    __shared__ uint32_t s_used[kTilePixels];   // fragments of the pixel that took part in the blend
     __shared__ uint8_t s_pix[kBuildCap];       // pixel (inside the bin) of every list place
     __shared__ float4 s_stage[kStage][2];      // descriptor, confidence of the staged fragments
     const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
@@ -130,9 +160,6 @@ __global__ void __launch_bounds__(kBlock) bin_build_kernel(BuildPass a)
         const uint32_t q = q0 + tid;
         a.offsets[q]     = begin + start;
         if (bin == a.num_bins - 1u && (uint32_t)tid == pixels - 1u) a.offsets[q + 1] = begin + n;
-        // one byte per pixel: does the top-K cut drop fragments here? The backward per-point kernel only has to look up
-        // the K-th key of a pixel where this is set.
-        a.list_is_cut[q] = (a.K > 0 && c > (uint32_t)a.K) ? 1 : 0;
     }
     __syncthreads();
 
@@ -145,7 +172,9 @@ __global__ void __launch_bounds__(kBlock) bin_build_kernel(BuildPass a)
         list_off          = s_prefix[px];
         list_len          = s_cnt[px];
     }
-    const uint32_t keep = a.K > 0 ? min(c, (uint32_t)a.K) : c;  // kept fragments of the pixel this thread owns
+    const uint32_t keep = a.K > 0 ? min(c, (uint32_t)a.K) : c;  // fragments of this thread's pixel left by the top-K cut
+    uint32_t used       = 0;                                    // ... that took part in the blend
+    bool saturated      = false;
     float T = 1.f;
     float color[C];
 #pragma unroll
@@ -179,7 +208,8 @@ __global__ void __launch_bounds__(kBlock) bin_build_kernel(BuildPass a)
                 const uint32_t px  = s_pix[r];
                 const uint32_t len = a.K > 0 ? min(s_cnt[px], (uint32_t)a.K) : s_cnt[px];
                 if (r - s_prefix[px] >= len) continue;  // cut away
-                const int id = (int)s_id[2 * r];
+                const uint32_t low = s_id[2 * r];
+                const int id       = BILINEAR ? (int)(low >> 2) : (int)low;
                 // an id or texture index out of range cannot come from a list the fill pass wrote; such a fragment
                 // blends as fully transparent (the reference asserts on the texture index, RenderForward.cu:1335-1336)
                 int ti = -1;
@@ -187,8 +217,9 @@ __global__ void __launch_bounds__(kBlock) bin_build_kernel(BuildPass a)
                 float4 t4 = make_float4(0.f, 0.f, 0.f, 0.f), c4 = t4;
                 if ((uint32_t)ti < (uint32_t)a.N)
                 {
-                    t4 = a.packed[2 * (size_t)ti];
-                    c4 = a.packed[2 * (size_t)ti + 1];
+                    t4   = a.packed[2 * (size_t)ti];
+                    c4   = a.packed[2 * (size_t)ti + 1];
+                    c4.x = fragment_alpha<BILINEAR>(a, l, low, c4.x);
                 }
                 s_stage[r - base][0] = t4;
                 s_stage[r - base][1] = c4;
@@ -197,7 +228,7 @@ __global__ void __launch_bounds__(kBlock) bin_build_kernel(BuildPass a)
             if ((uint32_t)tid < pixels)
             {
                 const uint32_t lo = max(start, base), hi = min(start + keep, base + (uint32_t)kStage);
-                for (uint32_t r = lo; r < hi; ++r)
+                for (uint32_t r = lo; r < hi && !saturated; ++r)
                 {
                     const float4 t4 = s_stage[r - base][0];
                     const float cf  = s_stage[r - base][1].x;
@@ -207,16 +238,19 @@ __global__ void __launch_bounds__(kBlock) bin_build_kernel(BuildPass a)
 #pragma unroll
                     for (int ci = 0; ci < C; ++ci) color[ci] = Tc * t[ci] + color[ci];
                     T = (1.f - cf) * T;
+                    ++used;
+                    saturated = blend_is_saturated<BILINEAR>(T);
                 }
             }
             __syncthreads();
         }
+        s_used[tid] = used;
+        __syncthreads();
         if (a.transmittance)
             for (uint32_t r = tid; r < n; r += kBlock)
             {
-                const uint32_t px  = s_pix[r];
-                const uint32_t len = a.K > 0 ? min(s_cnt[px], (uint32_t)a.K) : s_cnt[px];
-                if (r - s_prefix[px] < len) a.transmittance[begin + r] = s_T[2 * r + 1];
+                const uint32_t px = s_pix[r];
+                if (r - s_prefix[px] < s_used[px]) a.transmittance[begin + r] = s_T[2 * r + 1];
             }
     }
     else
@@ -250,14 +284,50 @@ __global__ void __launch_bounds__(kBlock) bin_build_kernel(BuildPass a)
         __threadfence_block();
         __syncthreads();
         if ((uint32_t)tid < pixels)
-            blend_list_from_memory<C>(a.fragments + begin + start, keep, a.index, a.packed, a.N,
-                                      a.transmittance ? a.transmittance + begin + start : nullptr, T, color);
+        {
+            if constexpr (!BILINEAR)
+            {
+                blend_list_from_memory<C>(a.fragments + begin + start, keep, a.index, a.packed, a.N,
+                                          a.transmittance ? a.transmittance + begin + start : nullptr, T, color);
+                used = keep;
+            }
+            else
+            {
+                const uint64_t* list = a.fragments + begin + start;
+                for (uint32_t j = 0; j < keep && !saturated; ++j)
+                {
+                    const uint32_t low = (uint32_t)list[j];
+                    const int id       = (int)(low >> 2);
+                    int ti             = -1;
+                    if ((uint32_t)id < (uint32_t)a.N) ti = a.index ? a.index[id] : id;
+                    float4 t4 = make_float4(0.f, 0.f, 0.f, 0.f);
+                    float cf  = 0.f;
+                    if ((uint32_t)ti < (uint32_t)a.N)
+                    {
+                        t4 = a.packed[2 * (size_t)ti];
+                        cf = fragment_alpha<BILINEAR>(a, l, low, a.packed[2 * (size_t)ti + 1].x);
+                    }
+                    if (a.transmittance) a.transmittance[begin + start + j] = T;
+                    const float t[4] = {t4.x, t4.y, t4.z, t4.w};
+                    const float Tc   = T * cf;
+#pragma unroll
+                    for (int ci = 0; ci < C; ++ci) color[ci] = Tc * t[ci] + color[ci];
+                    T = (1.f - cf) * T;
+                    ++used;
+                    saturated = blend_is_saturated<BILINEAR>(T);
+                }
+            }
+        }
     }
 
     if ((uint32_t)tid < pixels)
     {
         // pixel number -> image coordinates
-        const uint32_t q        = q0 + tid;
+        const uint32_t q = q0 + tid;
+        // How many fragments of the list took part, and one byte that says whether any did not (top-K cut, saturation):
+        // the backward per-point kernel only has to look at the last blended key of a pixel where this is set.
+        a.kept[q]        = used;
+        a.list_is_cut[q] = used < c ? 1 : 0;
         const uint32_t in_layer = q - a.ly.base[l];
         const uint32_t tile     = in_layer / kTilePixels;
         const uint32_t ty = tile / (uint32_t)a.ly.tiles_x[l], tx = tile - ty * (uint32_t)a.ly.tiles_x[l];
@@ -269,7 +339,7 @@ __global__ void __launch_bounds__(kBlock) bin_build_kernel(BuildPass a)
 #pragma unroll
             for (int ci = 0; ci < C; ++ci)
             {
-                if (!a.use_environment_map) color[ci] = (T * 1.f) * a.background[ci] + color[ci];
+                if (!a.use_environment_map && !saturated) color[ci] = (T * 1.f) * a.background[ci] + color[ci];
                 a.out[l][ci * plane + local] = color[ci];
             }
             a.weight[q] = T;

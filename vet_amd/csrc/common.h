@@ -103,18 +103,55 @@ __device__ __forceinline__ bool project_point(const DeviceView& c, const float4 
     return true;
 }
 
-// Tile and pixel-in-tile of layer l for a projected point; false if it falls outside the layer. The caller halves
-// ipx/ipy/radius between layers (src/lib/rendering/RenderForward.cu:856,888-891); rintf is round-half-even like
-// __float2int_rn.
-__device__ __forceinline__ bool layer_tile_pixel(const LayerTable& ly, int l, float ipx, float ipy, uint32_t& tile,
-                                                 uint32_t& in_tile)
+// Tile and pixel-in-tile of the pixel with (integral) float coordinates (fx, fy) of layer l; false outside the layer.
+__device__ __forceinline__ bool tile_of_pixel(const LayerTable& ly, int l, float fx, float fy, uint32_t& tile,
+                                              uint32_t& in_tile)
 {
-    const float fx = rintf(ipx), fy = rintf(ipy);
     if (!(fx >= 0.f && fx < (float)ly.w[l] && fy >= 0.f && fy < (float)ly.h[l])) return false;
     const uint32_t x = (uint32_t)(int)fx, y = (uint32_t)(int)fy;
     tile    = ly.tile_base[l] + (y / kTile) * (uint32_t)ly.tiles_x[l] + x / kTile;
     in_tile = (y % kTile) * kTile + x % kTile;
     return true;
+}
+
+// Pixel a projected point lands in at layer l, as hit number h of HITS. The caller halves ipx/ipy/radius between
+// layers (src/lib/rendering/RenderForward.cu:856,888-891).
+//   HITS = 1 (FULL_BLEND): the pixel the position rounds to; rintf is round-half-even like __float2int_rn.
+//   HITS = 4 (BILINEAR_BLEND): the 2x2 pixels around the position, floor + (h & 1, h >> 1); h is the corner number
+//   y_j * 2 + x_i of src/lib/rendering/RenderForward.cu:865-885,1097-1134.
+template <int HITS>
+__device__ __forceinline__ bool layer_hit(const LayerTable& ly, int l, float ipx, float ipy, int h, uint32_t& tile,
+                                          uint32_t& in_tile)
+{
+    if constexpr (HITS == 1)
+        return tile_of_pixel(ly, l, rintf(ipx), rintf(ipy), tile, in_tile);
+    else
+        return tile_of_pixel(ly, l, floorf(ipx) + (float)(h & 1), floorf(ipy) + (float)(h >> 1), tile, in_tile);
+}
+
+__device__ __forceinline__ bool layer_tile_pixel(const LayerTable& ly, int l, float ipx, float ipy, uint32_t& tile,
+                                                 uint32_t& in_tile)
+{
+    return layer_hit<1>(ly, l, ipx, ipy, 0, tile, in_tile);
+}
+
+// compute_blending_fac (src/lib/rendering/PointBlending.h:12-44): bilinear weight of corner `corner` of a position, and
+// optionally its derivative with respect to the position.
+__device__ __forceinline__ float bilinear_weight(float u, float v, int corner, float* d_du = nullptr,
+                                                 float* d_dv = nullptr)
+{
+    const float sx = u - floorf(u), sy = v - floorf(v);
+    const float wx = (corner & 1) ? sx : 1.f - sx;
+    const float wy = (corner & 2) ? sy : 1.f - sy;
+    if (d_du)
+    {
+        // J(0) = (sy - 1, sx - 1), J(1) = (1 - sy, -sx), J(2) = (-sy, 1 - sx), J(3) = (sy, sx)
+        const float jx[4] = {sy - 1.f, 1.f - sy, -sy, sy};
+        const float jy[4] = {sx - 1.f, -sx, 1.f - sx, sx};
+        *d_du = jx[corner];
+        *d_dv = jy[corner];
+    }
+    return wx * wy;
 }
 
 // Bin and pixel-in-bin of a pixel given as (tile, pixel in tile) of layer l.

@@ -172,15 +172,19 @@ __device__ __forceinline__ WaveGroup group_by_bin(bool has, uint32_t bin, int la
     return g;
 }
 
+// HITS = 1: a point lands in the pixel it rounds to (FULL_BLEND); HITS = 4: in the 2x2 pixels around it (BILINEAR_BLEND),
+// each of which is a fragment of its own with its own bin. slots is [L][HITS][N].
+template <int HITS>
 __global__ void __launch_bounds__(kBlock) bin_count_kernel(ViewPass a, uint32_t* __restrict__ bin_counts,
                                                             uint32_t* __restrict__ slots)
 {
     const int i    = blockIdx.x * blockDim.x + threadIdx.x;
     const int lane = threadIdx.x & (kWave - 1);
-    bool has[VETRAST_MAX_LAYERS];
-    uint32_t bin[VETRAST_MAX_LAYERS];
+    constexpr int kHits = VETRAST_MAX_LAYERS * HITS;
+    bool has[kHits];
+    uint32_t bin[kHits];
 #pragma unroll
-    for (int l = 0; l < VETRAST_MAX_LAYERS; ++l) has[l] = false, bin[l] = 0;
+    for (int k = 0; k < kHits; ++k) has[k] = false, bin[k] = 0;
     Projected p;
     if (i < a.N && !point_is_skipped(a, i) && project_point(*a.view, a.position[i], p))
     {
@@ -190,29 +194,33 @@ __global__ void __launch_bounds__(kBlock) bin_count_kernel(ViewPass a, uint32_t*
         {
             if (l >= a.ly.L) break;
             if (a.drop_by_radius && radius < a.radius_threshold) break;
-            uint32_t tile, in_tile, in_bin;
-            has[l] = layer_tile_pixel(a.ly, l, ipx, ipy, tile, in_tile);
-            if (has[l]) bin_of_pixel(a.ly, l, tile, in_tile, bin[l], in_bin);
+#pragma unroll
+            for (int h = 0; h < HITS; ++h)
+            {
+                uint32_t tile, in_tile, in_bin;
+                has[l * HITS + h] = layer_hit<HITS>(a.ly, l, ipx, ipy, h, tile, in_tile);
+                if (has[l * HITS + h]) bin_of_pixel(a.ly, l, tile, in_tile, bin[l * HITS + h], in_bin);
+            }
         }
     }
-    // group first, then all atomics of the wave at once (they are independent), then one wait
-    WaveGroup g[VETRAST_MAX_LAYERS];
-    uint32_t base[VETRAST_MAX_LAYERS];
+    // group, and issue the group's atomic right away: the atomics of a wave are independent and their results are only
+    // looked at after the last one has been issued, so the wave waits once
+    uint32_t base[kHits], who[kHits];  // who = leader lane | rank in the group << 8
 #pragma unroll
-    for (int l = 0; l < VETRAST_MAX_LAYERS; ++l)
+    for (int k = 0; k < kHits; ++k)
     {
-        base[l] = 0;
-        if (l < a.ly.L) g[l] = group_by_bin(has[l], bin[l], lane);
+        base[k] = 0, who[k] = 0;
+        if (k / HITS >= a.ly.L) continue;
+        const WaveGroup g = group_by_bin(has[k], bin[k], lane);
+        who[k]            = (uint32_t)g.leader | (g.rank << 8);
+        if (has[k] && g.leader == lane) base[k] = atomicAdd(&bin_counts[bin[k]], g.count);
     }
 #pragma unroll
-    for (int l = 0; l < VETRAST_MAX_LAYERS; ++l)
-        if (l < a.ly.L && has[l] && g[l].leader == lane) base[l] = atomicAdd(&bin_counts[bin[l]], g[l].count);
-#pragma unroll
-    for (int l = 0; l < VETRAST_MAX_LAYERS; ++l)
+    for (int k = 0; k < kHits; ++k)
     {
-        if (l >= a.ly.L) break;
-        const uint32_t group_base = (uint32_t)__shfl((int)base[l], g[l].leader, kWave);
-        if (has[l]) slots[(size_t)l * a.N + i] = group_base + g[l].rank;
+        if (k / HITS >= a.ly.L) continue;
+        const uint32_t group_base = (uint32_t)__shfl((int)base[k], (int)(who[k] & 0xFF), kWave);
+        if (has[k]) slots[(size_t)k * a.N + i] = group_base + (who[k] >> 8);
     }
 }
 
@@ -347,6 +355,8 @@ __global__ void __launch_bounds__(kScanSmallBlock) scan_small_kernel(uint4* __re
 // to the bin's start + the rank the count pass drew. Counterpart of CollectMulti<L,false>
 // (src/lib/rendering/RenderForward.cu:1011-1096), which draws the rank from a second atomic counter image and stores
 // depth and id in two separate rows.
+// In BILINEAR_BLEND (HITS = 4) the low key word is point id << 2 | corner.
+template <int HITS>
 __global__ void __launch_bounds__(kBlock) bin_fill_kernel(ViewPass a, const uint32_t* __restrict__ bin_offsets,
                                                            const uint32_t* __restrict__ slots,
                                                            uint4* __restrict__ binned, uint32_t capacity)
@@ -361,11 +371,16 @@ __global__ void __launch_bounds__(kBlock) bin_fill_kernel(ViewPass a, const uint
     for (int l = 0; l < a.ly.L; ++l, radius *= 0.5f, ipx *= 0.5f, ipy *= 0.5f)
     {
         if (a.drop_by_radius && radius < a.radius_threshold) break;
-        uint32_t tile, in_tile, bin, in_bin;
-        if (!layer_tile_pixel(a.ly, l, ipx, ipy, tile, in_tile)) continue;
-        bin_of_pixel(a.ly, l, tile, in_tile, bin, in_bin);
-        const uint32_t pos = bin_offsets[bin] + slots[(size_t)l * a.N + i];
-        if (pos < capacity) binned[pos] = make_uint4((uint32_t)i, depth_bits, in_bin, 0u);  // guard: never false
+#pragma unroll
+        for (int h = 0; h < HITS; ++h)
+        {
+            uint32_t tile, in_tile, bin, in_bin;
+            if (!layer_hit<HITS>(a.ly, l, ipx, ipy, h, tile, in_tile)) continue;
+            bin_of_pixel(a.ly, l, tile, in_tile, bin, in_bin);
+            const uint32_t pos = bin_offsets[bin] + slots[(size_t)(l * HITS + h) * a.N + i];
+            const uint32_t low = HITS == 1 ? (uint32_t)i : (((uint32_t)i << 2) | (uint32_t)h);
+            if (pos < capacity) binned[pos] = make_uint4(low, depth_bits, in_bin, 0u);  // guard: never false
+        }
     }
 }
 

@@ -132,12 +132,26 @@ LayerTable make_layer_table(int w, int h, int L, int64_t N)
     return t;
 }
 
-int check_dims(int64_t N, int B, int L, int w, int h)
+// Fragments a point can leave in one layer: 1 (the pixel it rounds to) or the 2x2 pixels around it.
+inline int hits_of_mode(int render_mode)
+{
+    return render_mode == VETRAST_RENDER_BILINEAR_BLEND ? 4 : 1;
+}
+
+inline int check_mode(int render_mode)
+{
+    return (render_mode == 0 || render_mode == VETRAST_RENDER_FULL_BLEND || render_mode == VETRAST_RENDER_BILINEAR_BLEND)
+               ? VETRAST_OK
+               : VETRAST_ERR_UNSUPPORTED;
+}
+
+int check_dims(int64_t N, int B, int L, int w, int h, int hits)
 {
     if (N < 0 || B < 1 || L < 1 || L > VETRAST_MAX_LAYERS || w < 1 || h < 1) return VETRAST_ERR_INVALID_ARG;
     if ((w >> (L - 1)) < 1 || (h >> (L - 1)) < 1) return VETRAST_ERR_INVALID_ARG;  // coarsest layer must not be empty
-    // fragment positions and pixel numbers are 32-bit
-    if (N * L >= (int64_t)0xFFFFFFF0ll) return VETRAST_ERR_INVALID_ARG;
+    // fragment positions and pixel numbers are 32-bit; with 4 hits the point id shares a key word with the corner
+    if (N * L * hits >= (int64_t)0xFFFFFFF0ll) return VETRAST_ERR_INVALID_ARG;
+    if (hits > 1 && N > (int64_t)(1 << 30)) return VETRAST_ERR_INVALID_ARG;
     int64_t P = 0;
     int lw = w, lh = h;
     for (int l = 0; l < L; ++l, lw /= 2, lh /= 2)
@@ -156,8 +170,10 @@ int validate_forward(const vetrast_forward_args* a, vetrast_workspace_layout* la
     if (a->num_views < 1 || a->num_poses < 1 || a->num_cameras < 1) return VETRAST_ERR_INVALID_ARG;
     if (p.num_texture_channels < 1 || p.num_texture_channels > VETRAST_MAX_CHANNELS) return VETRAST_ERR_INVALID_ARG;
     if (p.check_normal) return VETRAST_ERR_UNSUPPORTED;
+    int st = check_mode(p.render_mode);
+    if (st != VETRAST_OK) return st;
     const int w = a->views[0].w, h = a->views[0].h;
-    int st = check_dims(a->num_points, a->num_views, p.num_layers, w, h);
+    st          = check_dims(a->num_points, a->num_views, p.num_layers, w, h, hits_of_mode(p.render_mode));
     if (st != VETRAST_OK) return st;
     for (int b = 0; b < a->num_views; ++b)
     {
@@ -173,7 +189,7 @@ int validate_forward(const vetrast_forward_args* a, vetrast_workspace_layout* la
         if (p.output_background_mask && !a->out_mask[l]) return VETRAST_ERR_INVALID_ARG;
     }
     if (((uintptr_t)a->workspace % kAlign) != 0 || ((uintptr_t)a->position % 16) != 0) return VETRAST_ERR_INVALID_ARG;
-    st = vetrast_workspace_layout_for(a->num_points, a->num_views, p.num_layers, w, h, lay);
+    st = vetrast_workspace_layout_for_mode(a->num_points, a->num_views, p.num_layers, w, h, p.render_mode, lay);
     if (st != VETRAST_OK) return st;
     const size_t need = a->save_for_backward ? lay->total_bytes : lay->forward_only_bytes;
     if (a->workspace_bytes < need) return VETRAST_ERR_WORKSPACE_SMALL;
@@ -280,11 +296,20 @@ int vetrast_layer_sizes(int32_t w, int32_t h, int32_t num_layers, int32_t* layer
 
 int vetrast_workspace_layout_for(int32_t N, int32_t B, int32_t L, int32_t w, int32_t h, vetrast_workspace_layout* lay)
 {
+    return vetrast_workspace_layout_for_mode(N, B, L, w, h, VETRAST_RENDER_FULL_BLEND, lay);
+}
+
+int vetrast_workspace_layout_for_mode(int32_t N, int32_t B, int32_t L, int32_t w, int32_t h, int32_t render_mode,
+                                      vetrast_workspace_layout* lay)
+{
     if (!lay) return VETRAST_ERR_INVALID_ARG;
-    int st = check_dims(N, B, L, w, h);
+    int st = check_mode(render_mode);
+    if (st != VETRAST_OK) return st;
+    const int hits = hits_of_mode(render_mode);
+    st             = check_dims(N, B, L, w, h, hits);
     if (st != VETRAST_OK) return st;
     std::memset(lay, 0, sizeof(*lay));
-    LayerTable t = make_layer_table(w, h, L, N);
+    LayerTable t = make_layer_table(w, h, L, (int64_t)N * hits);
     for (int l = 0; l < L; ++l)
     {
         lay->layer_w[l] = t.w[l];
@@ -300,8 +325,9 @@ int vetrast_workspace_layout_for(int32_t N, int32_t B, int32_t L, int32_t w, int
     const size_t bins      = t.bin_base[L];
     const size_t Tpad      = align_up(bins + 1, kScanPerBlock);
     lay->num_bins          = (int64_t)bins;
-    const size_t cap       = (size_t)N * L;
+    const size_t cap       = (size_t)N * L * hits;
     lay->fragment_capacity = (int64_t)cap;
+    lay->hits_per_layer    = hits;
     size_t at              = 0;
     lay->flags_base        = at;
     at += kAlign;
@@ -324,6 +350,9 @@ int vetrast_workspace_layout_for(int32_t N, int32_t B, int32_t L, int32_t w, int
     lay->weight_base   = at;
     lay->weight_stride = align_up(P * sizeof(float), kAlign);
     at += lay->weight_stride * B;
+    lay->kept_base   = at;
+    lay->kept_stride = align_up(P * sizeof(uint32_t), kAlign);
+    at += lay->kept_stride * B;
     lay->cut_flags_base   = at;
     lay->cut_flags_stride = align_up(P, kAlign);
     at += lay->cut_flags_stride * B;
@@ -361,7 +390,8 @@ int vetrast_forward(vetrast_ctx* ctx, const vetrast_forward_args* a, void* strea
     hipStream_t stream      = (hipStream_t)stream_;
     const vetrast_params& p = a->params;
     const int N = a->num_points, B = a->num_views, L = p.num_layers, C = p.num_texture_channels;
-    const LayerTable ly = make_layer_table(a->views[0].w, a->views[0].h, L, N);
+    const int hits      = hits_of_mode(p.render_mode);
+    const LayerTable ly = make_layer_table(a->views[0].w, a->views[0].h, L, (int64_t)N * hits);
     const uint32_t bins = ly.bin_base[L];
     const size_t Tpad   = lay.bin_counts_stride / sizeof(uint32_t);
     void* ws            = a->workspace;
@@ -428,7 +458,10 @@ int vetrast_forward(vetrast_ctx* ctx, const vetrast_forward_args* a, void* strea
         if (N > 0)
         {
             ScopeTimer tm(ctx, stream, VETRAST_SCOPE_COUNT);
-            hipLaunchKernelGGL(bin_count_kernel, dim3(grid_for(N)), dim3(kBlock), 0, stream, vp, bin_counts, slots);
+            if (hits == 1)
+                hipLaunchKernelGGL(bin_count_kernel<1>, dim3(grid_for(N)), dim3(kBlock), 0, stream, vp, bin_counts, slots);
+            else
+                hipLaunchKernelGGL(bin_count_kernel<4>, dim3(grid_for(N)), dim3(kBlock), 0, stream, vp, bin_counts, slots);
         }
         {
             ScopeTimer tm(ctx, stream, VETRAST_SCOPE_SCAN);
@@ -447,8 +480,12 @@ int vetrast_forward(vetrast_ctx* ctx, const vetrast_forward_args* a, void* strea
         if (N > 0)
         {
             ScopeTimer tm(ctx, stream, VETRAST_SCOPE_FILL);
-            hipLaunchKernelGGL(bin_fill_kernel, dim3(grid_for(N)), dim3(kBlock), 0, stream, vp, bin_counts, slots, binned,
-                               (uint32_t)lay.fragment_capacity);
+            if (hits == 1)
+                hipLaunchKernelGGL(bin_fill_kernel<1>, dim3(grid_for(N)), dim3(kBlock), 0, stream, vp, bin_counts, slots,
+                                   binned, (uint32_t)lay.fragment_capacity);
+            else
+                hipLaunchKernelGGL(bin_fill_kernel<4>, dim3(grid_for(N)), dim3(kBlock), 0, stream, vp, bin_counts, slots,
+                                   binned, (uint32_t)lay.fragment_capacity);
         }
         float* out[VETRAST_MAX_LAYERS];
         float* out_mask[VETRAST_MAX_LAYERS];
@@ -470,6 +507,9 @@ int vetrast_forward(vetrast_ctx* ctx, const vetrast_forward_args* a, void* strea
             bp.offsets             = offsets;
             bp.fragments           = fragments;
             bp.list_is_cut         = list_is_cut;
+            bp.kept                = ws_ptr<uint32_t>(ws, lay.kept_base + lay.kept_stride * b);
+            bp.position            = vp.position;
+            bp.view                = vp.view;
             bp.index               = a->index;
             bp.packed              = packed;
             bp.background          = a->background;
@@ -483,13 +523,22 @@ int vetrast_forward(vetrast_ctx* ctx, const vetrast_forward_args* a, void* strea
             bp.mask_value          = p.output_background_mask_value;
             for (int l = 0; l < VETRAST_MAX_LAYERS; ++l) bp.out[l] = out[l], bp.out_mask[l] = out_mask[l];
             const dim3 g(bins), blk(kBlock);
-            switch (C)
-            {
-                case 1: hipLaunchKernelGGL(bin_build_kernel<1>, g, blk, 0, stream, bp); break;
-                case 2: hipLaunchKernelGGL(bin_build_kernel<2>, g, blk, 0, stream, bp); break;
-                case 3: hipLaunchKernelGGL(bin_build_kernel<3>, g, blk, 0, stream, bp); break;
-                default: hipLaunchKernelGGL(bin_build_kernel<4>, g, blk, 0, stream, bp); break;
-            }
+            if (hits == 1)
+                switch (C)
+                {
+                    case 1: hipLaunchKernelGGL((bin_build_kernel<1, false>), g, blk, 0, stream, bp); break;
+                    case 2: hipLaunchKernelGGL((bin_build_kernel<2, false>), g, blk, 0, stream, bp); break;
+                    case 3: hipLaunchKernelGGL((bin_build_kernel<3, false>), g, blk, 0, stream, bp); break;
+                    default: hipLaunchKernelGGL((bin_build_kernel<4, false>), g, blk, 0, stream, bp); break;
+                }
+            else
+                switch (C)
+                {
+                    case 1: hipLaunchKernelGGL((bin_build_kernel<1, true>), g, blk, 0, stream, bp); break;
+                    case 2: hipLaunchKernelGGL((bin_build_kernel<2, true>), g, blk, 0, stream, bp); break;
+                    case 3: hipLaunchKernelGGL((bin_build_kernel<3, true>), g, blk, 0, stream, bp); break;
+                    default: hipLaunchKernelGGL((bin_build_kernel<4, true>), g, blk, 0, stream, bp); break;
+                }
         }
     }
     VET_HIP(ctx, hipGetLastError());
@@ -504,6 +553,7 @@ int vetrast_backward(vetrast_ctx* ctx, const vetrast_backward_args* g, void* str
     int st = validate_forward(a, &lay);
     if (st != VETRAST_OK) return st;
     if (!a->save_for_backward) return VETRAST_ERR_INVALID_ARG;
+    if (hits_of_mode(a->params.render_mode) != 1) return VETRAST_ERR_UNSUPPORTED;
     if (!g->grad_texture || !g->grad_confidence || !g->grad_background) return VETRAST_ERR_INVALID_ARG;
     if (g->grad_points && !g->grad_point_count) return VETRAST_ERR_INVALID_ARG;
     if (g->grad_points && ((uintptr_t)g->grad_points % 16) != 0) return VETRAST_ERR_INVALID_ARG;

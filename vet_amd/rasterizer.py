@@ -142,6 +142,11 @@ class ForwardResult:
                              int(self.layout.fragment_capacity))
         return t.cpu().numpy()[src]
 
+    def kept(self, b=0):
+        """int64 [total_pixels]: fragments of every pixel's list that took part in the blend, image order."""
+        t = self._view_array(self.layout.kept_base, self.layout.kept_stride, b, torch.int32, self.device_pixels())
+        return t.cpu().numpy().astype(np.int64)[self.pixel_map()]
+
     def weight(self, b=0):
         t = self._view_array(self.layout.weight_base, self.layout.weight_stride, b, torch.float32,
                              self.device_pixels())
@@ -192,18 +197,18 @@ class Rasterizer:
     def _stream():
         return C.c_void_p(torch.cuda.current_stream().cuda_stream)
 
-    def layout(self, scene: Scene) -> abi.WorkspaceLayout:
+    def layout(self, scene: Scene, render_mode=abi.RENDER_FULL_BLEND) -> abi.WorkspaceLayout:
         lay = abi.WorkspaceLayout()
         v = scene.views[0]
-        abi.check(self.lib.vetrast_workspace_layout_for(scene.num_points, len(scene.views), scene.num_layers, v.w, v.h,
-                                                        C.byref(lay)), "workspace_layout_for")
+        abi.check(self.lib.vetrast_workspace_layout_for_mode(scene.num_points, len(scene.views), scene.num_layers, v.w,
+                                                             v.h, render_mode, C.byref(lay)), "workspace_layout_for_mode")
         return lay
 
     def forward(self, dev: DeviceScene, params: abi.Params = None, save_for_backward=True, workspace=None,
                 out=None) -> ForwardResult:
         scene = dev.scene
         params = params or make_params(scene)
-        lay = self.layout(scene)
+        lay = self.layout(scene, params.render_mode)
         if workspace is None:
             workspace = torch.empty(lay.total_bytes, dtype=torch.uint8, device=dev.device)
         B, Cn = len(scene.views), scene.num_channels
