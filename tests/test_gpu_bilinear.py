@@ -84,3 +84,57 @@ def test_mode_3_needs_the_bigger_workspace(rasterizer):
     with pytest.raises(abi.VetrastError) as e:
         rasterizer.forward(dev, make_params(scene, render_mode=2))
     assert e.value.status == abi.ERR_UNSUPPORTED
+
+
+GRAD_TOL = 1e-4
+
+
+@pytest.mark.parametrize("name,scene,overrides", SCENES, ids=[s[0] for s in SCENES])
+def test_backward_matches_oracle(name, scene, overrides, rasterizer, oracle):
+    if name == "tiny_long_lists":
+        pytest.skip("the oracle's literal O(n^2) loop over lists of hundreds of fragments takes minutes")
+    print(f"[case] bilinear backward {name} N={scene.num_points}", flush=True)
+    ref, dev, res, _ = _check_forward(scene, dict(overrides, need_point_gradient=1), rasterizer, oracle)
+    grad_out = scene.grad_out()
+    ref_g = oracle.backward(ref, grad_out)
+    got_g = rasterizer.backward(res, [torch.from_numpy(g).cuda() for g in grad_out])
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(got_g["point_count"].cpu().numpy(), ref_g["point_count"])
+    for key in ("texture", "confidence", "background", "points"):
+        err = max_rel_err(got_g[key].cpu().numpy(), ref_g[key])
+        print(f"  {key}: max rel err {err:.3e}", flush=True)
+        assert err <= GRAD_TOL, key
+
+
+def test_backward_with_index_views_and_cameras(rasterizer, oracle):
+    """Texture index indirection, two views, pose and intrinsics gradients (the pose count grows by 1 per fragment in
+    this mode, the intrinsics count by 1/1024)."""
+    scene = synthetic.tiny_scene(num_points=4000, K=8, seed=77, num_views=2)
+    rng = np.random.default_rng(6)
+    scene.index = rng.integers(0, 900, size=scene.num_points).astype(np.int32)
+    ref, dev, res, _ = _check_forward(scene, {"need_point_gradient": 1}, rasterizer, oracle)
+    grad_out = scene.grad_out()
+    ref_g = oracle.backward(ref, grad_out, want_cameras=True)
+    got_g = rasterizer.backward(res, [torch.from_numpy(g).cuda() for g in grad_out], want_cameras=True)
+    torch.cuda.synchronize()
+    got = {k: v.cpu().numpy() for k, v in got_g.items() if k != "_args"}
+    np.testing.assert_array_equal(got["point_count"], ref_g["point_count"])
+    for key in ("texture", "confidence", "background", "points", "pose", "intrinsics"):
+        assert max_rel_err(got[key], ref_g[key]) <= GRAD_TOL, key
+    np.testing.assert_allclose(got["pose_count"], ref_g["pose_count"], rtol=1e-6)
+    np.testing.assert_allclose(got["intrinsics_count"], ref_g["intrinsics_count"], rtol=1e-4)
+    assert got["pose_count"][0] > 100
+
+
+def test_backward_is_reproducible_and_linear(rasterizer):
+    scene = synthetic.config2(num_points=100_000, w=480, h=270)
+    dev = DeviceScene(scene)
+    res = rasterizer.forward(dev, make_params(scene, need_point_gradient=1, **MODE))
+    go = [torch.from_numpy(g).cuda() for g in scene.grad_out()]
+    a = {k: v.clone() for k, v in rasterizer.backward(res, go).items() if k != "_args"}
+    b = {k: v.clone() for k, v in rasterizer.backward(res, go).items() if k != "_args"}
+    c = {k: v.clone() for k, v in rasterizer.backward(res, [2.0 * g for g in go]).items() if k != "_args"}
+    for k in a:
+        assert torch.equal(a[k], b[k]), k
+        if k != "point_count":
+            assert torch.equal(c[k], 2.0 * a[k]), k

@@ -14,15 +14,18 @@ namespace vetrast
 struct BackwardPass
 {
     const uint32_t* offsets;
+    const uint32_t* kept;        // per pixel: fragments of its list that took part in the forward blend
     const uint64_t* fragments;
-    const float* transmittance;  // per kept fragment, saved by the forward blend
-    const float* weight;         // per pixel: transmittance behind the last kept fragment
+    const float* transmittance;  // per blended fragment, saved by the forward blend
+    const float* weight;         // per pixel: transmittance behind the last blended fragment
+    const float4* position;      // BILINEAR_BLEND: a fragment's alpha and its derivative depend on the point's projection
+    const DeviceView* view;
     const int32_t* index;
     const float4* packed;
     const float* background;
     const float* grad_out[VETRAST_MAX_LAYERS];  // already offset to this view
     const float* out[VETRAST_MAX_LAYERS];       // forward result, already offset to this view
-    float4* partial;          // [L][N] records of 2 float4: (d tex0..3), (d conf, d image x, d image y, 0)
+    float4* partial;          // [L][hits][N] records of 2 float4: (d tex0..3), (d conf, d image x, d image y, 0)
     float* background_partial;  // [workgroups][8]: per-workgroup sums of d background[0..C) and of the leak term
     LayerTable ly;
     TileMap tiles;
@@ -68,7 +71,13 @@ __device__ __forceinline__ bool interior_pixel(int x, int y, int w, int h)
 constexpr int kWindow     = 16;                 // fragments per pixel in one window
 constexpr int kWaveItems  = kWave * kWindow;    // item table of a wave
 
-template <int C>
+//
+// BILINEAR_BLEND (BlendBackwardsBilinear<C>, src/lib/rendering/RenderBackward.cu:2893-3232) has the same structure with
+// alpha_j = bilinear weight_j * confidence_j in place of c_j: d alpha_j = T_j * (t_j . g) - S_j / (1 - alpha_j + 1e-9),
+// the background only counts if the forward blend reached it (transmittance still >= 0.001), and, at pixels more than
+// 2 away from the border only, d conf_j = weight_j * d alpha_j and the position gradient is the analytic
+// d weight_j / d position * confidence_j * d alpha_j. A record goes to partial[layer][corner][point].
+template <int C, bool BILINEAR>
 __global__ void __launch_bounds__(kBlock) blend_backward_kernel(BackwardPass a)
 {
     constexpr int kWaves = kBlock / kWave;
@@ -103,13 +112,14 @@ __global__ void __launch_bounds__(kBlock) blend_backward_kernel(BackwardPass a)
 #pragma unroll
         for (int ci = 0; ci < C; ++ci) g[ci] = G[ci * plane + local];
         off = a.offsets[px.q];
-        n   = a.offsets[px.q + 1] - off;
-        if (a.K > 0) n = min(n, (uint32_t)a.K);
+        n   = a.kept[px.q];
 
         float S = 0.f;
-        if (!a.use_environment_map)
+        const float Tn = a.use_environment_map ? 0.f : a.weight[px.q];
+        // BILINEAR_BLEND leaves the background out once the transmittance is below 0.001 (RenderBackward.cu:3014-3019:
+        // the loop stops before the background element)
+        if (!a.use_environment_map && !(BILINEAR && (double)Tn < 0.001))
         {
-            const float Tn = a.weight[px.q];
             float dot      = 0.f;
 #pragma unroll
             for (int ci = 0; ci < C; ++ci)
@@ -119,14 +129,15 @@ __global__ void __launch_bounds__(kBlock) blend_backward_kernel(BackwardPass a)
                 dot += bgc * g[ci];
                 S += ((g[ci] * bgc) * Tn) * 1.f;
             }
-            if (a.quirk_background_confidence_leak) leak = dot * Tn;
+            if (!BILINEAR && a.quirk_background_confidence_leak) leak = dot * Tn;
         }
-        const bool do_point = a.need_point_gradient && n > 0 && interior_pixel(px.x, px.y, lw, lh);
+        const bool inner    = interior_pixel(px.x, px.y, lw, lh);
+        const bool do_point = a.need_point_gradient && n > 0 && inner;
         s_off[wave][lane]   = off;
         s_carry[wave][lane] = S;
         s_g[wave][lane]     = make_float4(g[0], g[1], g[2], g[3]);
-        s_point[wave][lane] = do_point ? 1 : 0;
-        if (do_point)
+        s_point[wave][lane] = (do_point ? 1 : 0) | (inner ? 2 : 0);
+        if (do_point && !BILINEAR)
         {
             // The reference evaluates, per fragment with descriptor t and per channel,
             //   1/2 * ( -(t - I(x-1)) * G(x-1) + (t - I(x+1)) * G(x+1) )        (RenderBackward.cu:1364-1371)
@@ -157,7 +168,7 @@ __global__ void __launch_bounds__(kBlock) blend_backward_kernel(BackwardPass a)
     uint32_t max_n = n;
 #pragma unroll
     for (int d = kWave / 2; d >= 1; d >>= 1) max_n = max(max_n, (uint32_t)__shfl_xor((int)max_n, d, kWave));
-    float4* partial_l = a.partial + 2 * (size_t)l * a.N;
+    float4* partial_l = a.partial + 2 * (size_t)l * (BILINEAR ? 4 : 1) * a.N;
     for (int jw = max_n == 0 ? -1 : (int)((max_n - 1) / kWindow) * kWindow; jw >= 0; jw -= kWindow)
     {
         const uint32_t nw = (n > (uint32_t)jw) ? min(n - (uint32_t)jw, (uint32_t)kWindow) : 0u;
@@ -184,21 +195,40 @@ __global__ void __launch_bounds__(kBlock) blend_backward_kernel(BackwardPass a)
             float x = 0.f, T = 0.f, c = 0.f, dot = 0.f;
             float t[4] = {0.f, 0.f, 0.f, 0.f};
             float4 g4  = make_float4(0.f, 0.f, 0.f, 0.f);
-            int id = -1, ti = -1;
+            int id = -1, ti = -1, corner = 0;
+            float4 wp = make_float4(0.f, 0.f, 0.f, 0.f);
             if (valid)
             {
                 const uint32_t pos = s_off[wave][p] + (uint32_t)jw + (k - s_base[wave][p]);
-                id                 = (int)(uint32_t)a.fragments[pos];
+                const uint32_t low = (uint32_t)a.fragments[pos];
+                id                 = BILINEAR ? (int)(low >> 2) : (int)low;
+                corner             = BILINEAR ? (int)(low & 3u) : 0;
                 T                  = a.transmittance[pos];
                 // guards the gathers; never false for a workspace the forward pass wrote
                 if ((uint32_t)id < (uint32_t)a.N) ti = a.index ? a.index[id] : id;
                 if ((uint32_t)ti >= (uint32_t)a.N) ti = -1;
                 g4 = s_g[wave][p];
             }
+            float conf = 0.f, fac = 1.f, fac_du = 0.f, fac_dv = 0.f;
             if (ti >= 0)
             {
                 const float4 t4 = a.packed[2 * (size_t)ti];
-                c               = a.packed[2 * (size_t)ti + 1].x;
+                conf            = a.packed[2 * (size_t)ti + 1].x;
+                c               = conf;
+                if constexpr (BILINEAR)
+                {
+                    // alpha = bilinear weight of this pixel's corner at the point's position in this layer x confidence
+                    wp = a.position[id];
+                    Projected pr;
+                    fac = 0.f;
+                    if (project_point(*a.view, wp, pr))
+                    {
+                        float u = pr.ipx, v = pr.ipy;
+                        for (int h = 0; h < l; ++h) u *= 0.5f, v *= 0.5f;
+                        fac = bilinear_weight(u, v, corner, &fac_du, &fac_dv);
+                    }
+                    c = fac * conf;
+                }
                 t[0] = t4.x, t[1] = t4.y, t[2] = t4.z, t[3] = t4.w;
                 const float g[4] = {g4.x, g4.y, g4.z, g4.w};
 #pragma unroll
@@ -227,10 +257,24 @@ __global__ void __launch_bounds__(kBlock) blend_backward_kernel(BackwardPass a)
             if (ti >= 0)
             {
                 const float g[4]  = {g4.x, g4.y, g4.z, g4.w};
-                const float Tc    = T * c;
-                const float gconf = dot * T - S / ((1.f - c) + 1e-9f);
+                const float Tc     = T * c;
+                const float galpha = dot * T - S / ((1.f - c) + 1e-9f);
+                float gconf        = galpha;
                 float gp0 = 0.f, gp1 = 0.f;
-                if (s_point[wave][p])
+                if constexpr (BILINEAR)
+                {
+                    // confidence and position gradients only at pixels more than 2 away from the border
+                    // (RenderBackward.cu:3044); dA/dc = weight, dA/dweight = confidence (:3075-3088)
+                    const int flags = s_point[wave][p];
+                    gconf           = (flags & 2) ? fac * galpha : 0.f;
+                    if (flags & 1)
+                    {
+                        const float single = conf * galpha;
+                        gp0                = fac_du * single;
+                        gp1                = fac_dv * single;
+                    }
+                }
+                else if (s_point[wave][p] & 1)
                 {
                     const float4 ax4 = s_ax[wave][p], ay4 = s_ay[wave][p];
                     const float2 b2  = s_bxy[wave][p];
@@ -255,7 +299,7 @@ __global__ void __launch_bounds__(kBlock) blend_backward_kernel(BackwardPass a)
                 // Record stores, two lanes per record: first the even lane's record (even lane its low half, odd lane
                 // the high half), then the odd lane's, so that each instruction issues one 32-byte request per record.
                 const int odd        = lane & 1;
-                const int own        = ti >= 0 ? id : -1;
+                const int own        = ti >= 0 ? (BILINEAR ? corner * a.N + id : id) : -1;
                 const int other      = pair_other(own);
                 const float4 o_lo    = pair_other(rec_lo);
                 const float4 o_hi    = pair_other(rec_hi);
@@ -263,6 +307,7 @@ __global__ void __launch_bounds__(kBlock) blend_backward_kernel(BackwardPass a)
                 const int id_second  = odd ? own : other;
                 const float4 v_first = odd ? o_hi : rec_lo;
                 const float4 v_second = odd ? rec_hi : o_lo;
+                // own/other are record numbers: the point id, in BILINEAR_BLEND behind the corner's block of N records
                 if (id_first >= 0) partial_l[2 * (size_t)id_first + odd] = v_first;
                 if (id_second >= 0) partial_l[2 * (size_t)id_second + odd] = v_second;
             }
@@ -378,6 +423,7 @@ struct GatherPass
     const uint32_t* offsets;
     const uint64_t* fragments;
     const uint8_t* list_is_cut;  // per pixel, written by the build pass
+    const uint32_t* kept;        // per pixel: fragments of its list that took part in the blend
     const float4* partial;
     float* grad_texture;      // [C,N]
     float* grad_confidence;   // [N]
@@ -401,7 +447,9 @@ constexpr int kCameraRow = 12;  // doubles per workgroup row: 6 pose tangent, fx
 // whether its fragment survived the top-K cut (its key is not larger than the K-th key of that pixel's sorted list), and
 // sum the stored records. With a texture index indirection several points may share a descriptor row; only then the
 // descriptor and confidence sums are added with atomics (onto rows the host zero-filled).
-template <int C>
+// HITS = 4 (BILINEAR_BLEND): a point has up to four fragments per layer, one per corner of its 2x2 pixels, with records
+// at partial[layer][corner][point].
+template <int C, int HITS>
 __global__ void __launch_bounds__(kBlock) gather_point_gradients_kernel(GatherPass a)
 {
     const int i      = blockIdx.x * blockDim.x + threadIdx.x;
@@ -422,20 +470,32 @@ __global__ void __launch_bounds__(kBlock) gather_point_gradients_kernel(GatherPa
         const float vx = ((cam.r[0] * wp.x + cam.r[1] * wp.y) + cam.r[2] * wp.z) + cam.t[0];
         const float vy = ((cam.r[3] * wp.x + cam.r[4] * wp.y) + cam.r[5] * wp.z) + cam.t[1];
         const float vz = ((cam.r[6] * wp.x + cam.r[7] * wp.y) + cam.r[8] * wp.z) + cam.t[2];
-        const uint64_t key = ((uint64_t)__float_as_uint(p.z) << 32) | (uint32_t)i;
+        const uint64_t depth_key = (uint64_t)__float_as_uint(p.z) << 32;
         float ipx = p.ipx, ipy = p.ipy, radius = p.radius;
         const LayerTable& ly = a.vp.ly;
         for (int l = 0; l < ly.L; ++l, radius *= 0.5f, ipx *= 0.5f, ipy *= 0.5f)
         {
             if (a.vp.drop_by_radius && radius < a.vp.radius_threshold) break;
-            const float fx = rintf(ipx), fy = rintf(ipy);
+#pragma unroll
+          for (int h = 0; h < HITS; ++h)
+          {
+            const float fx = HITS == 1 ? rintf(ipx) : floorf(ipx) + (float)(h & 1);
+            const float fy = HITS == 1 ? rintf(ipy) : floorf(ipy) + (float)(h >> 1);
             if (!(fx >= 0.f && fx < (float)ly.w[l] && fy >= 0.f && fy < (float)ly.h[l])) continue;
             const int x = (int)fx, y = (int)fy;
             const uint32_t q   = (ly.tile_base[l] + (uint32_t)(y / kTile) * (uint32_t)ly.tiles_x[l] + (uint32_t)(x / kTile)) * kTilePixels +
                                (uint32_t)(y % kTile) * kTile + (uint32_t)(x % kTile);
-            if (a.K > 0 && a.list_is_cut[q] && key > a.fragments[a.offsets[q] + a.K - 1]) continue;  // cut away
-            const float4 r0 = a.partial[2 * ((size_t)l * a.vp.N + i)];
-            const float4 r1 = a.partial[2 * ((size_t)l * a.vp.N + i) + 1];
+            // Did the fragment take part in the blend? Only where the pixel's list was not blended to its end (top-K
+            // cut, saturation) the last blended key has to be looked up.
+            if (a.list_is_cut[q])
+            {
+                const uint32_t nk  = a.kept[q];
+                const uint64_t key = depth_key | (HITS == 1 ? (uint32_t)i : (((uint32_t)i << 2) | (uint32_t)h));
+                if (nk == 0 || key > a.fragments[a.offsets[q] + nk - 1]) continue;
+            }
+            const size_t rec = (size_t)(l * HITS + h) * a.vp.N + i;
+            const float4 r0  = a.partial[2 * rec];
+            const float4 r1  = a.partial[2 * rec + 1];
             const float r[4] = {r0.x, r0.y, r0.z, r0.w};
 #pragma unroll
             for (int ci = 0; ci < C; ++ci) gt[ci] += r[ci];
@@ -478,6 +538,7 @@ __global__ void __launch_bounds__(kBlock) gather_point_gradients_kernel(GatherPa
                     cam_sum[9] += b2;
                 }
             }
+          }
         }
     }
     if (a.camera_partial)
@@ -551,14 +612,15 @@ __global__ void __launch_bounds__(kBlock) gather_point_gradients_kernel(GatherPa
 }
 
 // Adds the per-workgroup camera rows of one view to the pose row image_index (double) and the intrinsics row
-// camera_index (fx, fy, cx, cy times K_gradient_factor; skew and distortion columns stay zero), and the fragment count
-// / 1024 to both count arrays, as src/lib/rendering/RenderBackward.cu:1418-1459 does per fragment with atomics.
+// camera_index (fx, fy, cx, cy times K_gradient_factor; skew and distortion columns stay zero), and the scaled fragment
+// count to both count arrays, as src/lib/rendering/RenderBackward.cu:1418-1459 does per fragment with atomics.
 __global__ void __launch_bounds__(kBlock) reduce_camera_kernel(const double* __restrict__ rows, int num_rows,
                                                                 int image_index, int camera_index, float k_factor,
                                                                 double* __restrict__ grad_pose,
                                                                 float* __restrict__ grad_pose_count,
                                                                 float* __restrict__ grad_intrinsics,
-                                                                float* __restrict__ grad_intrinsics_count)
+                                                                float* __restrict__ grad_intrinsics_count,
+                                                                float pose_count_step)
 {
     __shared__ double red[kBlock / kWave][kCameraRow];
     double acc[11];
@@ -595,9 +657,10 @@ __global__ void __launch_bounds__(kBlock) reduce_camera_kernel(const double* __r
         }
         else
         {
-            const float c = (float)(s / 1024.0);
-            if (grad_pose) grad_pose_count[image_index] += c;
-            if (grad_intrinsics) grad_intrinsics_count[camera_index] += c;
+            // per fragment the reference adds 1/1024 to both counts in FULL_BLEND, but 1 to the pose count in
+            // BILINEAR_BLEND (src/lib/rendering/RenderBackward.cu:1425,1458 and :3146,3174)
+            if (grad_pose) grad_pose_count[image_index] += (float)(s * (double)pose_count_step);
+            if (grad_intrinsics) grad_intrinsics_count[camera_index] += (float)(s / 1024.0);
         }
     }
 }

@@ -553,7 +553,6 @@ int vetrast_backward(vetrast_ctx* ctx, const vetrast_backward_args* g, void* str
     int st = validate_forward(a, &lay);
     if (st != VETRAST_OK) return st;
     if (!a->save_for_backward) return VETRAST_ERR_INVALID_ARG;
-    if (hits_of_mode(a->params.render_mode) != 1) return VETRAST_ERR_UNSUPPORTED;
     if (!g->grad_texture || !g->grad_confidence || !g->grad_background) return VETRAST_ERR_INVALID_ARG;
     if (g->grad_points && !g->grad_point_count) return VETRAST_ERR_INVALID_ARG;
     if (g->grad_points && ((uintptr_t)g->grad_points % 16) != 0) return VETRAST_ERR_INVALID_ARG;
@@ -564,7 +563,8 @@ int vetrast_backward(vetrast_ctx* ctx, const vetrast_backward_args* g, void* str
         if (!g->grad_out[l]) return VETRAST_ERR_INVALID_ARG;
     hipStream_t stream = (hipStream_t)stream_;
     const int N = a->num_points, B = a->num_views, L = p.num_layers, C = p.num_texture_channels;
-    const LayerTable ly = make_layer_table(a->views[0].w, a->views[0].h, L, N);
+    const int hits      = hits_of_mode(p.render_mode);
+    const LayerTable ly = make_layer_table(a->views[0].w, a->views[0].h, L, (int64_t)N * hits);
     const TileMap tiles = make_tile_map(ly);
     const uint32_t P    = ly.base[L];
     void* ws            = a->workspace;
@@ -616,6 +616,9 @@ int vetrast_backward(vetrast_ctx* ctx, const vetrast_backward_args* g, void* str
             ScopeTimer tm(ctx, stream, VETRAST_SCOPE_BACKWARD_BLEND);
             BackwardPass bp;
             bp.offsets          = offsets;
+            bp.kept             = ws_ptr<uint32_t>(ws, lay.kept_base + lay.kept_stride * b);
+            bp.position         = reinterpret_cast<const float4*>(a->position);
+            bp.view             = ws_ptr<DeviceView>(ws, lay.views_base) + b;
             bp.fragments        = fragments;
             bp.transmittance    = ws_ptr<float>(ws, lay.transmittance_base + lay.transmittance_stride * b);
             bp.weight           = ws_ptr<float>(ws, lay.weight_base + lay.weight_stride * b);
@@ -642,13 +645,22 @@ int vetrast_backward(vetrast_ctx* ctx, const vetrast_backward_args* g, void* str
                 bp.out[l]          = a->out[l] + (size_t)b * C * plane;
             }
             const dim3 grid(tile_grid(tiles)), blk(kBlock);
-            switch (C)
-            {
-                case 1: hipLaunchKernelGGL(blend_backward_kernel<1>, grid, blk, 0, stream, bp); break;
-                case 2: hipLaunchKernelGGL(blend_backward_kernel<2>, grid, blk, 0, stream, bp); break;
-                case 3: hipLaunchKernelGGL(blend_backward_kernel<3>, grid, blk, 0, stream, bp); break;
-                default: hipLaunchKernelGGL(blend_backward_kernel<4>, grid, blk, 0, stream, bp); break;
-            }
+            if (hits == 1)
+                switch (C)
+                {
+                    case 1: hipLaunchKernelGGL((blend_backward_kernel<1, false>), grid, blk, 0, stream, bp); break;
+                    case 2: hipLaunchKernelGGL((blend_backward_kernel<2, false>), grid, blk, 0, stream, bp); break;
+                    case 3: hipLaunchKernelGGL((blend_backward_kernel<3, false>), grid, blk, 0, stream, bp); break;
+                    default: hipLaunchKernelGGL((blend_backward_kernel<4, false>), grid, blk, 0, stream, bp); break;
+                }
+            else
+                switch (C)
+                {
+                    case 1: hipLaunchKernelGGL((blend_backward_kernel<1, true>), grid, blk, 0, stream, bp); break;
+                    case 2: hipLaunchKernelGGL((blend_backward_kernel<2, true>), grid, blk, 0, stream, bp); break;
+                    case 3: hipLaunchKernelGGL((blend_backward_kernel<3, true>), grid, blk, 0, stream, bp); break;
+                    default: hipLaunchKernelGGL((blend_backward_kernel<4, true>), grid, blk, 0, stream, bp); break;
+                }
         }
         if (N > 0)
         {
@@ -658,6 +670,7 @@ int vetrast_backward(vetrast_ctx* ctx, const vetrast_backward_args* g, void* str
             gp.offsets             = offsets;
             gp.fragments           = fragments;
             gp.list_is_cut         = ws_ptr<uint8_t>(ws, lay.cut_flags_base + lay.cut_flags_stride * b);
+            gp.kept                = ws_ptr<uint32_t>(ws, lay.kept_base + lay.kept_stride * b);
             gp.partial             = partial;
             gp.grad_texture        = g->grad_texture;
             gp.grad_confidence     = g->grad_confidence;
@@ -670,23 +683,33 @@ int vetrast_backward(vetrast_ctx* ctx, const vetrast_backward_args* g, void* str
             gp.background_rows       = background_rows;
             gp.num_background_rows   = (int)tile_grid(tiles);
             gp.grad_background       = g->grad_background;
-            gp.add_leak              = (p.quirk_background_confidence_leak && !p.use_environment_map) ? 1 : 0;
+            gp.add_leak              = (p.quirk_background_confidence_leak && !p.use_environment_map && hits == 1) ? 1 : 0;
             gp.background_accumulate = b > 0 ? 1 : 0;
             const dim3 grid(grid_for(N)), blk(kBlock);
-            switch (C)
-            {
-                case 1: hipLaunchKernelGGL(gather_point_gradients_kernel<1>, grid, blk, 0, stream, gp); break;
-                case 2: hipLaunchKernelGGL(gather_point_gradients_kernel<2>, grid, blk, 0, stream, gp); break;
-                case 3: hipLaunchKernelGGL(gather_point_gradients_kernel<3>, grid, blk, 0, stream, gp); break;
-                default: hipLaunchKernelGGL(gather_point_gradients_kernel<4>, grid, blk, 0, stream, gp); break;
-            }
+            if (hits == 1)
+                switch (C)
+                {
+                    case 1: hipLaunchKernelGGL((gather_point_gradients_kernel<1, 1>), grid, blk, 0, stream, gp); break;
+                    case 2: hipLaunchKernelGGL((gather_point_gradients_kernel<2, 1>), grid, blk, 0, stream, gp); break;
+                    case 3: hipLaunchKernelGGL((gather_point_gradients_kernel<3, 1>), grid, blk, 0, stream, gp); break;
+                    default: hipLaunchKernelGGL((gather_point_gradients_kernel<4, 1>), grid, blk, 0, stream, gp); break;
+                }
+            else
+                switch (C)
+                {
+                    case 1: hipLaunchKernelGGL((gather_point_gradients_kernel<1, 4>), grid, blk, 0, stream, gp); break;
+                    case 2: hipLaunchKernelGGL((gather_point_gradients_kernel<2, 4>), grid, blk, 0, stream, gp); break;
+                    case 3: hipLaunchKernelGGL((gather_point_gradients_kernel<3, 4>), grid, blk, 0, stream, gp); break;
+                    default: hipLaunchKernelGGL((gather_point_gradients_kernel<4, 4>), grid, blk, 0, stream, gp); break;
+                }
         }
         if (want_camera)
         {
             ScopeTimer tm(ctx, stream, VETRAST_SCOPE_BACKWARD_GATHER);
             hipLaunchKernelGGL(reduce_camera_kernel, dim3(1), dim3(kBlock), 0, stream, camera_rows, grid_for(N),
                                a->views[b].image_index, a->views[b].camera_index, p.K_gradient_factor, g->grad_pose,
-                               g->grad_pose_count, g->grad_intrinsics, g->grad_intrinsics_count);
+                               g->grad_pose_count, g->grad_intrinsics, g->grad_intrinsics_count,
+                               hits == 1 ? 1.f / 1024.f : 1.f);
         }
         if (N == 0)
         {
