@@ -138,3 +138,40 @@ def test_backward_is_reproducible_and_linear(rasterizer):
         assert torch.equal(a[k], b[k]), k
         if k != "point_count":
             assert torch.equal(c[k], 2.0 * a[k]), k
+
+
+def test_config3_full_size(rasterizer, oracle):
+    """BASELINE config 3 (2 M points, 1080p, 4 layers, K = 16) in BILINEAR_BLEND: 15 M fragments."""
+    print("[case] bilinear config 3, 2M points, 1080p, forward+backward", flush=True)
+    scene = synthetic.config3()
+    params = make_params(scene, need_point_gradient=1, **MODE)
+    dev = DeviceScene(scene)
+    res = rasterizer.forward(dev, params, save_for_backward=True)
+    torch.cuda.synchronize()
+    ref = oracle.forward(scene, params, num_threads=16)
+    off = res.offsets(0)
+    np.testing.assert_array_equal(off, ref.offsets[0].astype(np.int64))
+    assert off[-1] > 3.9 * 3_800_000  # four fragments per visible (point, layer) but for the image border
+    kept = res.kept(0)
+    np.testing.assert_array_equal(kept, ref.kept[0].astype(np.int64))
+    m = _blended_mask(off, kept)
+    np.testing.assert_array_equal(res.fragments(0)[m], ref.fragments[0, :int(off[-1])][m])
+    np.testing.assert_array_equal(res.weight(0), ref.weight[0])
+    for l in range(scene.num_layers):
+        np.testing.assert_array_equal(res.out[l].cpu().numpy(), ref.out[l])
+    grad_out = scene.grad_out()
+    got = rasterizer.backward(res, [torch.from_numpy(g).cuda() for g in grad_out])
+    torch.cuda.synchronize()
+    want = oracle.backward(ref, grad_out, num_threads=16)
+    np.testing.assert_array_equal(got["point_count"].cpu().numpy(), want["point_count"])
+    for key in ("texture", "confidence", "points"):
+        err = max_rel_err(got[key].cpu().numpy(), want[key])
+        print(f"  {key}: max rel err {err:.3e}", flush=True)
+        assert err <= GRAD_TOL, key
+    # background: against the float64 sum over the pixels whose blend reached the background (T >= 0.001)
+    bg64 = np.zeros(scene.num_channels)
+    for l, (w, h) in enumerate(scene.layer_sizes()):
+        T = ref.weight[0, ref.layer_base(l):ref.layer_base(l) + w * h].astype(np.float64).reshape(h, w)
+        T = np.where(T >= 0.001, T, 0.0)
+        bg64 += (grad_out[l][0].astype(np.float64) * T[None]).sum(axis=(1, 2))
+    assert max_rel_err(got["background"].cpu().numpy(), bg64) <= 1e-4

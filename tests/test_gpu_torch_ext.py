@@ -19,14 +19,15 @@ def _views(scene):
             for v in scene.views]
 
 
+@pytest.mark.parametrize("render_mode", [1, 3], ids=["full_blend", "bilinear_blend"])
 @pytest.mark.parametrize("literal", [True, False], ids=["reference_literal", "clean"])
-def test_autograd_matches_oracle(literal, oracle):
+def test_autograd_matches_oracle(literal, render_mode, oracle):
     from vet_amd import torch_ops
 
     scene = synthetic.tiny_scene(num_points=5000, K=8, seed=31, num_views=2)
     quirks = dict(quirk_background_confidence_leak=1 if literal else 0,
                   point_gradient_normalization=2 if literal else 0,
-                  camera_gradient_normalization=1 if literal else 0)
+                  camera_gradient_normalization=1 if literal else 0, render_mode=render_mode)
     params = make_params(scene, need_point_gradient=1, **quirks)
     ref = oracle.forward(scene, params)
     grad_out = scene.grad_out()

@@ -2,6 +2,8 @@
 // calling the C ABI of include/vetrast.h. See point_render.h for the reference lines each piece mirrors.
 #include "point_render.h"
 
+#include <cstring>
+
 #include <c10/hip/HIPStream.h>
 #include <torch/extension.h>
 
@@ -22,6 +24,8 @@ void* current_stream()
 vetrast_params to_abi_params(const RenderParams& p, int num_layers)
 {
     vetrast_params q;
+    std::memset(&q, 0, sizeof(q));
+    q.render_mode                      = p.render_mode;
     q.num_texture_channels             = p.num_texture_channels;
     q.num_layers                       = num_layers;
     q.debug_max_list_length            = p.debug_max_list_length;
@@ -66,7 +70,9 @@ vetrast_forward_args make_forward_args(NeuralRenderInfo* info, const torch::Tens
     TORCH_CHECK(poses_se3.defined() && poses_se3.is_cuda() && poses_se3.scalar_type() == torch::kFloat64 &&
                     poses_se3.is_contiguous() && poses_se3.dim() == 2 && poses_se3.size(1) == 8,
                 "poses_se3 must be a contiguous [F,8] float64 tensor on the GPU");
-    TORCH_CHECK(info->params.render_mode == 1, "only render_mode 1 (FULL_BLEND) is implemented");
+    TORCH_CHECK(info->params.render_mode == VETRAST_RENDER_FULL_BLEND ||
+                    info->params.render_mode == VETRAST_RENDER_BILINEAR_BLEND,
+                "only render_mode 1 (FULL_BLEND) and 3 (BILINEAR_BLEND) are implemented");
     TORCH_CHECK(!info->params.add_depth_to_network, "add_depth_to_network is not part of the blending path");
     TORCH_CHECK(!info->images.empty(), "no views");
 
@@ -143,7 +149,9 @@ torch::autograd::variable_list PointRender::forward(torch::autograd::AutogradCon
     vetrast_forward_args a =
         make_forward_args(info, texture, background_color, points, intrinsics, confidence, dropout, poses_se3, t_index);
     vetrast_workspace_layout lay;
-    check_status(vetrast_workspace_layout_for(a.num_points, B, L, info->images[0].w, info->images[0].h, &lay), "layout");
+    check_status(vetrast_workspace_layout_for_mode(a.num_points, B, L, info->images[0].w, info->images[0].h,
+                                                   a.params.render_mode, &lay),
+                 "layout");
 
     const bool need_backward =
         ctx != nullptr && (texture.requires_grad() || background_color.requires_grad() || points.requires_grad() ||
