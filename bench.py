@@ -68,17 +68,17 @@ def measured_traffic():
     return res
 
 
-def run_scene(scene, backward, steps, warmup, profile=True):
+def run_scene(scene, backward, steps, warmup, profile=True, render_mode=1):
     import torch
 
     from vet_amd import abi
     from vet_amd.rasterizer import DeviceScene, Rasterizer, make_params
 
-    params = make_params(scene, need_point_gradient=1 if backward else 0)
+    params = make_params(scene, need_point_gradient=1 if backward else 0, render_mode=render_mode)
     N, Cn, L = scene.num_points, scene.num_channels, scene.num_layers
     rast = Rasterizer()
     dev = DeviceScene(scene)
-    lay = rast.layout(scene)
+    lay = rast.layout(scene, render_mode)
     workspace = torch.empty(lay.total_bytes, dtype=torch.uint8, device="cuda")
     out = [torch.empty((len(scene.views), Cn, h, w), dtype=torch.float32, device="cuda") for (w, h) in scene.layer_sizes()]
     fwd = rast.forward(dev, params, save_for_backward=backward, workspace=workspace, out=out)
@@ -88,7 +88,7 @@ def run_scene(scene, backward, steps, warmup, profile=True):
     counts = np.diff(off)
     K = params.debug_max_list_length
     F = int(off[-1])
-    Fk = int(np.minimum(counts, K).sum()) if K > 0 else F
+    Fk = int(fwd.kept(0).sum())  # fragments that took part in the blend (top-K cut, in mode 3 also saturation)
     bases = fwd.layer_bases()
     F_layers = [int(off[bases[l + 1]] - off[bases[l]]) for l in range(L)]
 
@@ -149,6 +149,8 @@ def main():
     ap.add_argument("--config", type=int, default=3, choices=[2, 3, 5])
     ap.add_argument("--points", type=int, default=None, help="override the point count (debug runs)")
     ap.add_argument("--point-order", default="vet_preprocess", choices=["vet_preprocess", "generated"])
+    ap.add_argument("--render-mode", type=int, default=1, choices=[1, 3],
+                    help="1 = FULL_BLEND (the headline workload), 3 = BILINEAR_BLEND (four fragments per point and layer)")
     ap.add_argument("--no-second-order", action="store_true", help="skip timing the other point order")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-threads", type=int, default=0, help="0 = min(16, available cores)")
@@ -172,7 +174,7 @@ def main():
     make = {2: synthetic.config2, 3: synthetic.config3, 5: synthetic.config5}[args.config]
     backward = args.config != 2
     scene = make(**kw)
-    r = run_scene(scene, backward, args.steps, args.warmup)
+    r = run_scene(scene, backward, args.steps, args.warmup, render_mode=args.render_mode)
     N, P, F, Fk, Cn, L, K = r["N"], r["P"], r["F"], r["Fk"], r["Cn"], r["L"], r["K"]
     ms_step, ms_fwd = r["ms_step"], r["ms_fwd"]
 
@@ -180,7 +182,8 @@ def main():
     alg = dict(fwd_b)
     if backward:
         alg.update(bwd_b)
-    traffic = measured_traffic() if (args.config == 3 and args.points is None and args.point_order == "vet_preprocess") else {}
+    traffic = measured_traffic() if (args.config == 3 and args.points is None and args.point_order == "vet_preprocess"
+                                     and args.render_mode == 1) else {}
     kernels = {}
     for k, nbytes in alg.items():
         t = r["per_step_ms"].get(k, 0.0)
@@ -213,8 +216,9 @@ def main():
         "config": {
             "workload": f"BASELINE config {args.config} ({scene.name}): N={N} points, {scene.views[0].w}x{scene.views[0].h}, "
                         f"L={L} layers, K={K}, C={Cn}, B=1 view, " + ("forward+backward" if backward else "forward")
-                        + f", point order {args.point_order}",
-            "point_order": args.point_order,
+                        + f", point order {args.point_order}"
+                        + (", render_mode 3 (BILINEAR_BLEND)" if args.render_mode == 3 else ", render_mode 1 (FULL_BLEND)"),
+            "point_order": args.point_order, "render_mode": args.render_mode,
             "fragments_per_layer": r["F_layers"], "fragments": F, "fragments_kept": Fk, "pixels": P,
         },
         "forward_ms": round(ms_fwd, 5),
@@ -240,7 +244,8 @@ def main():
         # VET hands the rasterizer Morton-ordered clouds with shuffled 256-point blocks; the generator's raw order
         # (random inside each primitive) is timed as well so that the effect of that order is visible.
         other = "generated" if args.point_order == "vet_preprocess" else "vet_preprocess"
-        r2 = run_scene(make(**dict(kw, point_order=other)), backward, max(10, args.steps // 2), 5, profile=False)
+        r2 = run_scene(make(**dict(kw, point_order=other)), backward, max(10, args.steps // 2), 5, profile=False,
+                       render_mode=args.render_mode)
         result["other_point_order"] = {"point_order": other, "ms_per_step": round(r2["ms_step"], 5),
                                        "forward_ms": round(r2["ms_fwd"], 5)}
 

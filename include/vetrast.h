@@ -135,7 +135,8 @@ typedef struct vetrast_workspace_layout
                                                 first min(count, K) entries of a pixel's list are sorted and meaningful */
     size_t transmittance_base, transmittance_stride; /* float [N*L]: transmittance in front of each kept fragment */
     size_t weight_base, weight_stride;       /* float [P]: final transmittance per pixel (the reference's `weight` image) */
-    size_t kept_base, kept_stride;           /* uint32 [P]: fragments of the pixel's list that took part in the blend */
+    size_t kept_base, kept_stride;           /* uint32 [P], BILINEAR_BLEND only: fragments of the pixel's list that took part in
+                                                the blend (FULL_BLEND: min(count, K), not stored) */
     size_t cut_flags_base, cut_flags_stride; /* uint8 [P]: 1 where some fragments of the pixel's list did not (top-K cut, saturation) */
     /* shared by all views */
     size_t packed_base;    /* float [N][8]: descriptor (4, zero padded), confidence, 3 pad */

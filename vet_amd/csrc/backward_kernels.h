@@ -14,7 +14,7 @@ namespace vetrast
 struct BackwardPass
 {
     const uint32_t* offsets;
-    const uint32_t* kept;        // per pixel: fragments of its list that took part in the forward blend
+    const uint32_t* kept;        // per pixel, BILINEAR_BLEND: fragments of its list that took part in the forward blend
     const uint64_t* fragments;
     const float* transmittance;  // per blended fragment, saved by the forward blend
     const float* weight;         // per pixel: transmittance behind the last blended fragment
@@ -112,7 +112,13 @@ __global__ void __launch_bounds__(kBlock) blend_backward_kernel(BackwardPass a)
 #pragma unroll
         for (int ci = 0; ci < C; ++ci) g[ci] = G[ci * plane + local];
         off = a.offsets[px.q];
-        n   = a.kept[px.q];
+        if constexpr (BILINEAR)
+            n = a.kept[px.q];
+        else
+        {
+            n = a.offsets[px.q + 1] - off;
+            if (a.K > 0) n = min(n, (uint32_t)a.K);
+        }
 
         float S = 0.f;
         const float Tn = a.use_environment_map ? 0.f : a.weight[px.q];
@@ -423,7 +429,7 @@ struct GatherPass
     const uint32_t* offsets;
     const uint64_t* fragments;
     const uint8_t* list_is_cut;  // per pixel, written by the build pass
-    const uint32_t* kept;        // per pixel: fragments of its list that took part in the blend
+    const uint32_t* kept;        // per pixel, BILINEAR_BLEND: fragments of its list that took part in the blend
     const float4* partial;
     float* grad_texture;      // [C,N]
     float* grad_confidence;   // [N]
@@ -489,7 +495,7 @@ __global__ void __launch_bounds__(kBlock) gather_point_gradients_kernel(GatherPa
             // cut, saturation) the last blended key has to be looked up.
             if (a.list_is_cut[q])
             {
-                const uint32_t nk  = a.kept[q];
+                const uint32_t nk  = HITS == 1 ? (uint32_t)a.K : a.kept[q];  // FULL_BLEND: cut means count > K > 0
                 const uint64_t key = depth_key | (HITS == 1 ? (uint32_t)i : (((uint32_t)i << 2) | (uint32_t)h));
                 if (nk == 0 || key > a.fragments[a.offsets[q] + nk - 1]) continue;
             }

@@ -326,7 +326,8 @@ __global__ void __launch_bounds__(kBlock) bin_build_kernel(BuildPass a)
         const uint32_t q = q0 + tid;
         // How many fragments of the list took part, and one byte that says whether any did not (top-K cut, saturation):
         // the backward per-point kernel only has to look at the last blended key of a pixel where this is set.
-        a.kept[q]        = used;
+        // (FULL_BLEND blends min(count, K) fragments, which the readers work out themselves: the array is not written.)
+        if constexpr (BILINEAR) a.kept[q] = used;
         a.list_is_cut[q] = used < c ? 1 : 0;
         const uint32_t in_layer = q - a.ly.base[l];
         const uint32_t tile     = in_layer / kTilePixels;

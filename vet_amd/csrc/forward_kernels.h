@@ -181,46 +181,39 @@ __global__ void __launch_bounds__(kBlock) bin_count_kernel(ViewPass a, uint32_t*
     const int i    = blockIdx.x * blockDim.x + threadIdx.x;
     const int lane = threadIdx.x & (kWave - 1);
     constexpr int kHits = VETRAST_MAX_LAYERS * HITS;
-    bool has[kHits];
-    uint32_t bin[kHits];
-#pragma unroll
-    for (int k = 0; k < kHits; ++k) has[k] = false, bin[k] = 0;
     Projected p;
-    if (i < a.N && !point_is_skipped(a, i) && project_point(*a.view, a.position[i], p))
-    {
-        float ipx = p.ipx, ipy = p.ipy, radius = p.radius;
+    const bool visible = i < a.N && !point_is_skipped(a, i) && project_point(*a.view, a.position[i], p);
+    float ipx = visible ? p.ipx : 0.f, ipy = visible ? p.ipy : 0.f, radius = visible ? p.radius : 0.f;
+    bool dropped = !visible;  // from the layer on at which the splat radius falls under the threshold
+    // Hit by hit: group the wave's hits by bin and issue the group's atomic right away. The atomics of a wave are
+    // independent and their results are only looked at after the last one has been issued, so the wave waits once.
+    // Only two registers per hit stay alive: the atomic's result and who = leader lane | rank << 8 | has << 31.
+    uint32_t base[kHits], who[kHits];
 #pragma unroll
-        for (int l = 0; l < VETRAST_MAX_LAYERS; ++l, radius *= 0.5f, ipx *= 0.5f, ipy *= 0.5f)
+    for (int l = 0; l < VETRAST_MAX_LAYERS; ++l, radius *= 0.5f, ipx *= 0.5f, ipy *= 0.5f)
+    {
+#pragma unroll
+        for (int h = 0; h < HITS; ++h) base[l * HITS + h] = 0, who[l * HITS + h] = 0;
+        if (l >= a.ly.L) continue;
+        if (a.drop_by_radius && radius < a.radius_threshold) dropped = true;
+#pragma unroll
+        for (int h = 0; h < HITS; ++h)
         {
-            if (l >= a.ly.L) break;
-            if (a.drop_by_radius && radius < a.radius_threshold) break;
-#pragma unroll
-            for (int h = 0; h < HITS; ++h)
-            {
-                uint32_t tile, in_tile, in_bin;
-                has[l * HITS + h] = layer_hit<HITS>(a.ly, l, ipx, ipy, h, tile, in_tile);
-                if (has[l * HITS + h]) bin_of_pixel(a.ly, l, tile, in_tile, bin[l * HITS + h], in_bin);
-            }
+            const int k = l * HITS + h;
+            uint32_t tile = 0, in_tile = 0, bin = 0, in_bin;
+            const bool has = !dropped && layer_hit<HITS>(a.ly, l, ipx, ipy, h, tile, in_tile);
+            if (has) bin_of_pixel(a.ly, l, tile, in_tile, bin, in_bin);
+            const WaveGroup g = group_by_bin(has, bin, lane);
+            who[k]            = (uint32_t)g.leader | (g.rank << 8) | (has ? 0x80000000u : 0u);
+            if (has && g.leader == lane) base[k] = atomicAdd(&bin_counts[bin], g.count);
         }
-    }
-    // group, and issue the group's atomic right away: the atomics of a wave are independent and their results are only
-    // looked at after the last one has been issued, so the wave waits once
-    uint32_t base[kHits], who[kHits];  // who = leader lane | rank in the group << 8
-#pragma unroll
-    for (int k = 0; k < kHits; ++k)
-    {
-        base[k] = 0, who[k] = 0;
-        if (k / HITS >= a.ly.L) continue;
-        const WaveGroup g = group_by_bin(has[k], bin[k], lane);
-        who[k]            = (uint32_t)g.leader | (g.rank << 8);
-        if (has[k] && g.leader == lane) base[k] = atomicAdd(&bin_counts[bin[k]], g.count);
     }
 #pragma unroll
     for (int k = 0; k < kHits; ++k)
     {
         if (k / HITS >= a.ly.L) continue;
         const uint32_t group_base = (uint32_t)__shfl((int)base[k], (int)(who[k] & 0xFF), kWave);
-        if (has[k]) slots[(size_t)k * a.N + i] = group_base + (who[k] >> 8);
+        if (who[k] & 0x80000000u) slots[(size_t)k * a.N + i] = group_base + ((who[k] >> 8) & 0x7FFFu);
     }
 }
 

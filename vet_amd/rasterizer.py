@@ -144,6 +144,9 @@ class ForwardResult:
 
     def kept(self, b=0):
         """int64 [total_pixels]: fragments of every pixel's list that took part in the blend, image order."""
+        if int(self.args.params.render_mode) != abi.RENDER_BILINEAR_BLEND:  # not stored: min(count, K)
+            counts, K = np.diff(self.offsets(b)), int(self.args.params.debug_max_list_length)
+            return np.minimum(counts, K) if K > 0 else counts
         t = self._view_array(self.layout.kept_base, self.layout.kept_stride, b, torch.int32, self.device_pixels())
         return t.cpu().numpy().astype(np.int64)[self.pixel_map()]
 
