@@ -88,6 +88,13 @@ typedef struct vetrast_params
                                                  lands in the 2x2 pixels around it, alpha = bilinear weight x confidence,
                                                  blending stops once the transmittance falls below 0.001). Other values
                                                  are refused. */
+    /* The steps VET runs on the optimised tensors right before the rasterizer, fused into it
+     * (NeuralPointTextureImpl::PrepareConfidence / PrepareTexture, src/lib/models/NeuralTexture.h:38-55; called from
+     * src/lib/models/Pipeline.cpp:113-124). With them on, `confidence`, `texture` and `background` are the RAW tensors
+     * and the gradients vetrast_backward returns are those of the raw tensors. */
+    int32_t confidence_activation;            /* 0: confidence is used as given; 1: sigmoid(confidence_scale * confidence) */
+    float confidence_scale;                   /* 10 + sigmoid_narrowing_factor * epoch in VET */
+    int32_t texture_abs;                      /* 1: |texture| and |background| (PipelineParams::non_subzero_texture) */
 } vetrast_params;
 
 #define VETRAST_RENDER_FULL_BLEND 1
@@ -146,7 +153,7 @@ typedef struct vetrast_workspace_layout
     int64_t num_bins;      /* bins of one view: runs of 256 / 64 / 16 / 4 consecutive pixel numbers, chosen per layer from N */
     size_t bin_counts_base, bin_counts_stride; /* per view, uint32 [num_bins+1 padded]: fragments per bin, then their exclusive scan */
     size_t binned_base;    /* uint32 [N*L][4]: fragment records grouped by bin (key low, key high, pixel in bin, 0); scratch */
-    size_t flags_base;     /* uint32 [4] device status flags */
+    size_t flags_base;     /* uint32 [4] device status flags, then at +64 bytes float [4]: the background as it is blended */
     size_t forward_only_bytes; /* a forward call with save_for_backward = 0 needs only this much */
     size_t partial_base;   /* float [L][N][8]: backward scratch, gradient record of the fragment of point i in layer l */
     size_t background_partial_base; /* float [workgroups][8]: backward scratch, per-workgroup background-gradient sums */
@@ -233,6 +240,26 @@ int vetrast_backward(vetrast_ctx* ctx, const vetrast_backward_args* args, void* 
  * distortion model is not available, so such input is flagged instead of guessed). */
 int vetrast_query_device_flags(vetrast_ctx* ctx, const void* workspace, const vetrast_workspace_layout* layout,
                                void* stream);
+
+/* One Adam step on a flat float tensor, the update MyAdam::step applies to texture_raw, confidence_raw and
+ * background_color_raw after every batch (src/lib/models/my_adam.cpp:25-104 = torch's Adam without amsgrad; options as
+ * in src/lib/data/NeuralScene.cpp:238-281): one kernel instead of the ~10 elementwise launches of the tensor-op form.
+ *   g = grad + weight_decay * param;  m = beta1 * m + (1 - beta1) * g;  v = beta2 * v + (1 - beta2) * g * g;
+ *   param -= lr / (1 - beta1^step) * m / (sqrt(v) / sqrt(1 - beta2^step) + eps)
+ * `step` is the state's step count after the increment (1 on the first call). With zero_grad the gradient is cleared
+ * in the same pass (texture_optimizer->zero_grad(), src/lib/data/NeuralScene.cpp:1247-1248). */
+typedef struct vetrast_adam_args
+{
+    float* param;      /* device [n] */
+    float* grad;       /* device [n] */
+    float* exp_avg;    /* device [n], zero before the first step */
+    float* exp_avg_sq; /* device [n], zero before the first step */
+    int64_t n;
+    int64_t step;
+    double lr, beta1, beta2, eps, weight_decay; /* doubles as in torch's AdamOptions: 1 - beta2 must not be formed in float */
+    int32_t zero_grad;
+} vetrast_adam_args;
+int vetrast_adam_step(vetrast_ctx* ctx, const vetrast_adam_args* args, void* stream);
 
 /* Per-kernel timing, the counterpart of NeuralRenderInfo::timer_system (src/lib/rendering/PointRenderer.h:32).
  * With profiling enabled every launch is bracketed by HIP events on the call's stream; vetrast_scope_times

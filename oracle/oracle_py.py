@@ -38,6 +38,10 @@ def load():
         lib.vetref_prepare_view.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p]
         lib.vetref_project_point.restype = C.c_int
         lib.vetref_project_point.argtypes = [C.c_void_p, C.POINTER(abi.View), C.c_void_p, C.c_void_p]
+        lib.vetref_sigmoid.restype = C.c_int
+        lib.vetref_sigmoid.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_float]
+        lib.vetref_adam_step.restype = C.c_int
+        lib.vetref_adam_step.argtypes = [C.POINTER(abi.AdamArgs)]
         _lib = lib
     return _lib
 
@@ -148,3 +152,25 @@ def project_point(prepared17, view: abi.View, position4):
     p = np.ascontiguousarray(position4, np.float32)
     ok = load().vetref_project_point(_addr(m), C.byref(view), _addr(p), _addr(out))
     return bool(ok), out
+
+
+def sigmoid(x, scale):
+    """sigmoid(scale * x) in the canonical float32 arithmetic of the fused confidence activation."""
+    x = np.ascontiguousarray(x, np.float32)
+    y = np.empty_like(x)
+    load().vetref_sigmoid(_addr(x), _addr(y), x.size, scale)
+    return y
+
+
+def adam_step(param, grad, exp_avg, exp_avg_sq, step, lr, beta1=0.9, beta2=0.999, eps=1e-8, weight_decay=0.0,
+              zero_grad=False):
+    """One Adam step in place on float32 numpy arrays."""
+    a = abi.AdamArgs()
+    for name, arr in (("param", param), ("grad", grad), ("exp_avg", exp_avg), ("exp_avg_sq", exp_avg_sq)):
+        assert arr.dtype == np.float32 and arr.flags.c_contiguous
+        setattr(a, name, _addr(arr))
+    a.n, a.step = param.size, step
+    a.lr, a.beta1, a.beta2, a.eps, a.weight_decay, a.zero_grad = lr, beta1, beta2, eps, weight_decay, int(zero_grad)
+    st = load().vetref_adam_step(C.byref(a))
+    if st != 0:
+        raise abi.VetrastError(st, "oracle adam_step")

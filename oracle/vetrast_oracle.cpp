@@ -193,6 +193,77 @@ inline void blending_fac(float u, float v, float fac[4], float J[4][2])
     }
 }
 
+// exp and the logistic function from +, *, rint and one division only (library exp routines differ in the last bits
+// between platforms): Cody-Waite reduction x = k ln2 + r, a degree-7 Taylor polynomial of e^r, scaling by 2^k through
+// the exponent bits. Canonical arithmetic of the fused confidence activation.
+inline float exp_canon(float x)
+{
+    x             = std::fmin(std::fmax(x, -87.f), 88.f);
+    const float k = std::rint(x * 1.44269504088896341f);
+    float r       = x - k * 0.693145751953125f;
+    r             = r - k * 1.42860682030941723e-06f;
+    float p       = 1.f / 5040.f;
+    p             = p * r + 1.f / 720.f;
+    p             = p * r + 1.f / 120.f;
+    p             = p * r + 1.f / 24.f;
+    p             = p * r + 1.f / 6.f;
+    p             = p * r + 0.5f;
+    p             = p * r + 1.f;
+    p             = p * r + 1.f;
+    const uint32_t bits = (uint32_t)((int)k + 127) << 23;
+    float scale;
+    std::memcpy(&scale, &bits, 4);
+    return p * scale;
+}
+
+inline float sigmoid_canon(float x)
+{
+    return 1.f / (1.f + exp_canon(-x));
+}
+
+// The tensors as the rasterizer blends them: NeuralPointTextureImpl::PrepareConfidence / PrepareTexture,
+// models/NeuralTexture.h:38-55 (sigmoid((10 + narrowing) * confidence_raw); abs or clone of texture_raw and
+// background_color_raw), when those steps are switched on in the params.
+struct PreparedInputs
+{
+    std::vector<float> texture, confidence, background;
+    vetrast_forward_args args;  // a copy that points to the prepared tensors, with the switches off
+};
+
+inline bool needs_preparation(const vetrast_params& p)
+{
+    return p.confidence_activation != 0 || p.texture_abs != 0;
+}
+
+inline void prepare_inputs(const vetrast_forward_args* a, PreparedInputs& o)
+{
+    const vetrast_params& p = a->params;
+    const size_t N = (size_t)a->num_points, C = (size_t)p.num_texture_channels;
+    o.args = *a;
+    if (p.confidence_activation)
+    {
+        o.confidence.resize(N);
+        for (size_t i = 0; i < N; ++i) o.confidence[i] = sigmoid_canon(p.confidence_scale * a->confidence[i]);
+        o.args.confidence = o.confidence.data();
+    }
+    if (p.texture_abs)
+    {
+        o.texture.resize(C * N);
+        for (size_t i = 0; i < C * N; ++i) o.texture[i] = std::fabs(a->texture[i]);
+        o.background.resize(C);
+        for (size_t i = 0; i < C; ++i) o.background[i] = std::fabs(a->background[i]);
+        o.args.texture    = o.texture.data();
+        o.args.background = o.background.data();
+    }
+    o.args.params.confidence_activation = 0;
+    o.args.params.texture_abs           = 0;
+}
+
+inline float sign_of(float x)
+{
+    return x > 0.f ? 1.f : (x < 0.f ? -1.f : 0.f);  // torch's abs backward: grad * sign(x)
+}
+
 inline bool is_bilinear(const vetrast_params& p)
 {
     return p.render_mode == VETRAST_RENDER_BILINEAR_BLEND;
@@ -517,6 +588,12 @@ extern "C" int vetref_forward(const vetrast_forward_args* a, uint32_t* offsets, 
 {
     int st = validate(a);
     if (st != VETRAST_OK) return st;
+    if (needs_preparation(a->params))
+    {
+        PreparedInputs prep;
+        prepare_inputs(a, prep);
+        return vetref_forward(&prep.args, offsets, fragments, transmittance, weight, kept, num_threads);
+    }
     if (!offsets || !fragments || !weight) return VETRAST_ERR_INVALID_ARG;
     for (int l = 0; l < a->params.num_layers; ++l)
         if (!a->out[l]) return VETRAST_ERR_INVALID_ARG;
@@ -674,6 +751,31 @@ extern "C" int vetref_backward(const vetrast_backward_args* g, const uint32_t* o
     int st                        = validate(a);
     if (st != VETRAST_OK) return st;
     if (!g->grad_texture || !g->grad_confidence || !g->grad_background) return VETRAST_ERR_INVALID_ARG;
+    if (needs_preparation(a->params))
+    {
+        // gradients of the prepared tensors first, then the chain rule of the preparation steps (what autograd does
+        // with torch::sigmoid and torch::abs in the reference)
+        PreparedInputs prep;
+        prepare_inputs(a, prep);
+        vetrast_backward_args g2 = *g;
+        g2.fwd                   = prep.args;
+        st                       = vetref_backward(&g2, offsets, fragments, num_threads);
+        if (st != VETRAST_OK) return st;
+        const vetrast_params& p = a->params;
+        const size_t N = (size_t)a->num_points, C = (size_t)p.num_texture_channels;
+        if (p.confidence_activation)
+            for (size_t i = 0; i < N; ++i)
+            {
+                const float sgm = prep.confidence[i];
+                g->grad_confidence[i] = g->grad_confidence[i] * ((p.confidence_scale * sgm) * (1.f - sgm));
+            }
+        if (p.texture_abs)
+        {
+            for (size_t i = 0; i < C * N; ++i) g->grad_texture[i] = g->grad_texture[i] * sign_of(a->texture[i]);
+            for (size_t i = 0; i < C; ++i) g->grad_background[i] = g->grad_background[i] * sign_of(a->background[i]);
+        }
+        return VETRAST_OK;
+    }
     if (g->grad_points && !g->grad_point_count) return VETRAST_ERR_INVALID_ARG;
     if (g->grad_pose && !g->grad_pose_count) return VETRAST_ERR_INVALID_ARG;
     if (g->grad_intrinsics && !g->grad_intrinsics_count) return VETRAST_ERR_INVALID_ARG;
@@ -863,6 +965,39 @@ extern "C" int vetref_backward(const vetrast_backward_args* g, const uint32_t* o
             if (c > 0)
                 for (int k = 0; k < 3; ++k) g->grad_points[3 * (size_t)i + k] /= c;
         }
+    }
+    return VETRAST_OK;
+}
+
+// torch::sigmoid(scale * x) in the canonical arithmetic (exposed so that tests can pin it against a float64 logistic).
+extern "C" int vetref_sigmoid(const float* x, float* y, int64_t n, float scale)
+{
+    for (int64_t i = 0; i < n; ++i) y[i] = sigmoid_canon(scale * x[i]);
+    return VETRAST_OK;
+}
+
+// One Adam step: MyAdam::step, models/my_adam.cpp:66-101 (torch's Adam without amsgrad), every operation rounded on its
+// own in the order of the tensor ops there; bias corrections in double as at :72-73.
+extern "C" int vetref_adam_step(const vetrast_adam_args* a)
+{
+    if (!a || a->n < 0 || a->step < 1) return VETRAST_ERR_INVALID_ARG;
+    const double bc1 = 1.0 - std::pow(a->beta1, (double)a->step);
+    const double bc2 = 1.0 - std::pow(a->beta2, (double)a->step);
+    const float sqrt_bc2 = (float)std::sqrt(bc2), step_size = (float)(a->lr / bc1);
+    const float omb1 = (float)(1.0 - a->beta1), omb2 = (float)(1.0 - a->beta2);
+    const float beta1 = (float)a->beta1, beta2 = (float)a->beta2, eps = (float)a->eps, wd = (float)a->weight_decay;
+    for (int64_t i = 0; i < a->n; ++i)
+    {
+        const float p = a->param[i];
+        float gr      = a->grad[i];
+        if (wd != 0.f) gr = gr + wd * p;
+        const float m     = a->exp_avg[i] * beta1 + omb1 * gr;
+        const float v     = a->exp_avg_sq[i] * beta2 + (omb2 * gr) * gr;
+        const float denom = std::sqrt(v) / sqrt_bc2 + eps;
+        a->exp_avg[i]     = m;
+        a->exp_avg_sq[i]  = v;
+        a->param[i]       = p + (-step_size) * (m / denom);
+        if (a->zero_grad) a->grad[i] = 0.f;
     }
     return VETRAST_OK;
 }

@@ -29,6 +29,10 @@
  *                     a pixel centre lands in one pixel), the blend and its early exit by an independent numpy blend,
  *                     value and position gradients by double-precision central differences of that blend (the
  *                     position gradient is analytic in this mode, so finite differences do pin it)
+ *   fused preparation confidence = sigmoid(scale * raw) pinned against a float64 logistic (<= 4e-7 relative: the exact bits of
+ *                     torch::sigmoid are PARITY UNPINNED), |texture| / |background| and the chain rule of both by
+ *                     comparing with the unfused path fed the prepared tensors and torch autograd
+ *   Adam step         pinned against torch.optim.Adam on the CPU over several steps with and without weight decay
  *   distortion != 0, check_normal, OCam, spherical: not implemented (rejected), PARITY UNPINNED
  */
 #ifndef VETRAST_ORACLE_H
@@ -54,6 +58,12 @@ int vetref_forward(const vetrast_forward_args* args, uint32_t* offsets, uint64_t
 
 int vetref_backward(const vetrast_backward_args* args, const uint32_t* offsets, const uint64_t* fragments,
                     int num_threads);
+
+/* sigmoid(scale * x) in the canonical arithmetic of the fused confidence activation (params.confidence_activation). */
+int vetref_sigmoid(const float* x, float* y, int64_t n, float scale);
+
+/* One Adam step on host arrays (MyAdam::step). */
+int vetref_adam_step(const vetrast_adam_args* args);
 
 #ifdef __cplusplus
 }

@@ -56,6 +56,9 @@ class Params(C.Structure):
         ("K_gradient_factor", C.c_float),
         ("camera_gradient_normalization", C.c_int32),
         ("render_mode", C.c_int32),
+        ("confidence_activation", C.c_int32),
+        ("confidence_scale", C.c_float),
+        ("texture_abs", C.c_int32),
     ]
 
 
@@ -89,6 +92,16 @@ class WorkspaceLayout(C.Structure):
         ("partial_base", C.c_size_t),
         ("background_partial_base", C.c_size_t),
         ("camera_partial_base", C.c_size_t),
+    ]
+
+
+class AdamArgs(C.Structure):
+    _fields_ = [
+        ("param", C.c_void_p), ("grad", C.c_void_p), ("exp_avg", C.c_void_p), ("exp_avg_sq", C.c_void_p),
+        ("n", C.c_int64), ("step", C.c_int64),
+        ("lr", C.c_double), ("beta1", C.c_double), ("beta2", C.c_double), ("eps", C.c_double),
+        ("weight_decay", C.c_double),
+        ("zero_grad", C.c_int32),
     ]
 
 
@@ -141,6 +154,7 @@ SYMBOLS = {
     "vetrast_forward_workspace_bytes": (C.c_size_t, [C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_int32]),
     "vetrast_forward": (C.c_int, [C.c_void_p, C.POINTER(ForwardArgs), C.c_void_p]),
     "vetrast_backward": (C.c_int, [C.c_void_p, C.POINTER(BackwardArgs), C.c_void_p]),
+    "vetrast_adam_step": (C.c_int, [C.c_void_p, C.POINTER(AdamArgs), C.c_void_p]),
     "vetrast_query_device_flags": (C.c_int, [C.c_void_p, C.c_void_p, C.POINTER(WorkspaceLayout), C.c_void_p]),
     "vetrast_set_profiling": (C.c_int, [C.c_void_p, C.c_int32]),
     "vetrast_reset_scope_times": (C.c_int, [C.c_void_p]),

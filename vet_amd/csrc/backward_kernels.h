@@ -353,7 +353,8 @@ template <int BLOCK>
 __device__ __forceinline__ void sum_background_rows(const float* __restrict__ rows, int num_rows, int C,
                                                     float* __restrict__ grad_background,
                                                     float* __restrict__ grad_confidence, int add_leak, int accumulate,
-                                                    int leak_atomic)
+                                                    int leak_atomic, const float* abs_of = nullptr,
+                                                    float leak_factor = 1.f)
 {
     __shared__ float red[BLOCK / kWave][kBackgroundRow];
     float acc[kBackgroundRow];
@@ -402,9 +403,13 @@ __device__ __forceinline__ void sum_background_rows(const float* __restrict__ ro
         float s     = 0.f;
         for (int w = 0; w < BLOCK / kWave; ++w) s += red[w][k];
         if (k < C)
+        {
+            if (abs_of) s = s * (abs_of[k] > 0.f ? 1.f : (abs_of[k] < 0.f ? -1.f : 0.f));  // background = |raw|
             grad_background[k] = accumulate ? grad_background[k] + s : s;
+        }
         else if (add_leak)
         {
+            s = s * leak_factor;  // chain rule of a fused confidence activation for row 0
             if (leak_atomic)
                 atomicAdd(&grad_confidence[0], s);
             else
@@ -418,9 +423,11 @@ constexpr int kReduceBlock = 1024;
 __global__ void __launch_bounds__(kReduceBlock) reduce_background_kernel(const float* __restrict__ rows, int num_rows,
                                                                           int C, float* __restrict__ grad_background,
                                                                           float* __restrict__ grad_confidence,
-                                                                          int add_leak, int accumulate)
+                                                                          int add_leak, int accumulate,
+                                                                          const float* __restrict__ abs_of)
 {
-    sum_background_rows<kReduceBlock>(rows, num_rows, C, grad_background, grad_confidence, add_leak, accumulate, 0);
+    sum_background_rows<kReduceBlock>(rows, num_rows, C, grad_background, grad_confidence, add_leak, accumulate, 0,
+                                      abs_of);
 }
 
 struct GatherPass
@@ -445,7 +452,20 @@ struct GatherPass
     float* grad_background;
     int add_leak;
     int background_accumulate;
+    // chain rule of the fused preparation steps (confidence = sigmoid(scale * raw), texture = |raw|, background = |raw|):
+    // the gradients written are those of the raw tensors
+    const float4* packed;      // prepared confidence of a row: packed[2 * row + 1].x
+    const float* texture_raw;  // [C,N]
+    const float* background_raw;
+    int confidence_activation;
+    float confidence_scale;
+    int texture_abs;
 };
+
+__device__ __forceinline__ float sign_of(float x)
+{
+    return x > 0.f ? 1.f : (x < 0.f ? -1.f : 0.f);  // torch's abs backward: grad * sign(x)
+}
 
 constexpr int kCameraRow = 12;  // doubles per workgroup row: 6 pose tangent, fx, fy, cx, cy, fragment count, pad
 
@@ -566,6 +586,23 @@ __global__ void __launch_bounds__(kBlock) gather_point_gradients_kernel(GatherPa
                 (cam_red[0][threadIdx.x] + cam_red[1][threadIdx.x]) + (cam_red[2][threadIdx.x] + cam_red[3][threadIdx.x]);
     }
     const int N = a.vp.N;
+    if (alive && (a.confidence_activation || a.texture_abs))
+    {
+        const int row = a.vp.index ? a.vp.index[i] : i;
+        if ((uint32_t)row < (uint32_t)N)
+        {
+            if (a.confidence_activation)
+            {
+                const float s = a.packed[2 * (size_t)row + 1].x;  // d sigmoid(k x) / dx = k s (1 - s)
+                gc            = gc * ((a.confidence_scale * s) * (1.f - s));
+            }
+            if (a.texture_abs)
+            {
+#pragma unroll
+                for (int ci = 0; ci < C; ++ci) gt[ci] = gt[ci] * sign_of(a.texture_raw[(size_t)ci * N + row]);
+            }
+        }
+    }
     if (!alive)
     {
     }
@@ -612,8 +649,15 @@ __global__ void __launch_bounds__(kBlock) gather_point_gradients_kernel(GatherPa
         // Without an index indirection confidence row 0 has just been written by thread 0 of this workgroup, which is
         // also the thread that adds the leak term; with one, rows are added to with atomics by every workgroup.
         __syncthreads();
+        float leak_factor = 1.f;
+        if (a.confidence_activation && a.add_leak)
+        {
+            const float s0 = a.packed[1].x;
+            leak_factor    = (a.confidence_scale * s0) * (1.f - s0);
+        }
         sum_background_rows<kBlock>(a.background_rows, a.num_background_rows, C, a.grad_background, a.grad_confidence,
-                                    a.add_leak, a.background_accumulate, a.vp.index != nullptr);
+                                    a.add_leak, a.background_accumulate, a.vp.index != nullptr,
+                                    a.texture_abs ? a.background_raw : nullptr, leak_factor);
     }
 }
 

@@ -15,6 +15,7 @@ constexpr int kScanPerThread  = 16;
 constexpr int kScanPerBlock   = kBlock * kScanPerThread;  // 4096 counts per workgroup
 constexpr int kBlendChunk     = 4;            // fragments a blend / backward thread prefetches at a time
 constexpr int kBackgroundRow  = 8;            // floats per workgroup row of background-gradient partial sums
+constexpr int kPreparedBackgroundOffset = 16;  // float index inside the flags block: the background as it is blended
 constexpr int kPackedFloats   = 8;            // interleaved record: 4 descriptor floats, confidence, 3 pad
 
 // Camera constants of one view, written by prepare_views_kernel and read (uniformly) by every other kernel.
@@ -69,6 +70,8 @@ struct ViewPass
     float radius_threshold;
     int viewer_only;
     float stability_cutoff;
+    int confidence_activation;  // 1: `confidence` holds raw values, the confidence is sigmoid(confidence_scale * raw)
+    float confidence_scale;
 };
 
 struct Projected
@@ -178,6 +181,40 @@ __device__ __forceinline__ int layer_of_pixel(const LayerTable& ly, uint32_t q)
     for (int k = 1; k < VETRAST_MAX_LAYERS; ++k)
         if (k < ly.L && q >= ly.base[k]) l = k;
     return l;
+}
+
+// exp and the logistic function from +, *, rint and one division only, so that the CPU check of the same formulas
+// agrees bit for bit (library exp routines differ in the last bits between platforms). Cody-Waite reduction
+// x = k ln2 + r, |r| <= ln2 / 2, a degree-7 Taylor polynomial of e^r (relative error about 1e-7), scaling by 2^k through
+// the exponent bits.
+__host__ __device__ __forceinline__ float exp_canon(float x)
+{
+    x             = fminf(fmaxf(x, -87.f), 88.f);
+    const float k = rintf(x * 1.44269504088896341f);
+    float r       = x - k * 0.693145751953125f;
+    r             = r - k * 1.42860682030941723e-06f;
+    float p       = 1.f / 5040.f;
+    p             = p * r + 1.f / 720.f;
+    p             = p * r + 1.f / 120.f;
+    p             = p * r + 1.f / 24.f;
+    p             = p * r + 1.f / 6.f;
+    p             = p * r + 0.5f;
+    p             = p * r + 1.f;
+    p             = p * r + 1.f;
+    const int e   = (int)k + 127;  // 40 .. 254
+    union
+    {
+        uint32_t u;
+        float f;
+    } scale;
+    scale.u = (uint32_t)e << 23;
+    return p * scale.f;
+}
+
+// torch::sigmoid(scale * x) of NeuralPointTextureImpl::PrepareConfidence (src/lib/models/NeuralTexture.h:38-41).
+__host__ __device__ __forceinline__ float sigmoid_canon(float x)
+{
+    return 1.f / (1.f + exp_canon(-x));
 }
 
 // Value the other lane of a pair (lane ^ 1) holds: a DPP register move (quad_perm [1,0,3,2]). Every lane of the wave

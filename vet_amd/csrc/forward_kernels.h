@@ -19,6 +19,31 @@ __global__ void __launch_bounds__(kBlock) fill_u128_kernel(uint4* __restrict__ d
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += stride) dst[i] = v;
 }
 
+// One Adam step on n floats (MyAdam::step, src/lib/models/my_adam.cpp:66-101, i.e. torch's Adam without amsgrad), every
+// operation rounded on its own in the order of the tensor ops there. inv_sqrt_bc2 = 1 / sqrt(1 - beta2^step) and
+// step_size = lr / (1 - beta1^step) come from the host in double, rounded once.
+__global__ void __launch_bounds__(kBlock) adam_step_kernel(float* __restrict__ param, float* __restrict__ grad,
+                                                            float* __restrict__ exp_avg, float* __restrict__ exp_avg_sq,
+                                                            size_t n, float beta1, float beta2, float one_minus_beta1,
+                                                            float one_minus_beta2, float sqrt_bc2, float step_size,
+                                                            float eps, float weight_decay, int zero_grad)
+{
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride)
+    {
+        const float p = param[i];
+        float g       = grad[i];
+        if (weight_decay != 0.f) g = g + weight_decay * p;            // grad.add(p, weight_decay)
+        const float m = exp_avg[i] * beta1 + one_minus_beta1 * g;      // mul_(beta1).add_(grad, 1 - beta1)
+        const float v = exp_avg_sq[i] * beta2 + (one_minus_beta2 * g) * g;  // mul_(beta2).addcmul_(grad, grad, 1 - beta2)
+        const float denom = sqrtf(v) / sqrt_bc2 + eps;                 // (sqrt() / sqrt(bias_correction2)).add_(eps)
+        exp_avg[i]    = m;
+        exp_avg_sq[i] = v;
+        param[i]      = p + (-step_size) * (m / denom);                // addcdiv_(exp_avg, denom, -step_size)
+        if (zero_grad) grad[i] = 0.f;
+    }
+}
+
 struct ViewSource
 {
     int image_index, camera_index, w, h;
@@ -40,7 +65,9 @@ __global__ void __launch_bounds__(kBlock) prepare_views_kernel(PrepareViewsArgs 
                                                                 const float* __restrict__ intrinsics,
                                                                 DeviceView* __restrict__ views,
                                                                 uint32_t* __restrict__ flags,
-                                                                uint4* __restrict__ counters4, size_t n4)
+                                                                uint4* __restrict__ counters4, size_t n4,
+                                                                const float* __restrict__ background, int channels,
+                                                                int texture_abs)
 {
     if (blockIdx.x > 0)
     {
@@ -54,6 +81,12 @@ __global__ void __launch_bounds__(kBlock) prepare_views_kernel(PrepareViewsArgs 
     {
         // the device flag word starts every call at zero
         if (k < 4) flags[k] = 0u;
+        // the background as it is blended: PrepareTexture, src/lib/models/NeuralTexture.h:43-55
+        if (k < VETRAST_MAX_CHANNELS)
+        {
+            const float bg = k < channels ? background[k] : 0.f;
+            reinterpret_cast<float*>(flags)[kPreparedBackgroundOffset + k] = texture_abs ? fabsf(bg) : bg;
+        }
         __syncthreads();
     }
     if (k >= num_views) return;
@@ -97,18 +130,29 @@ __global__ void __launch_bounds__(kBlock) prepare_views_kernel(PrepareViewsArgs 
 // Planar descriptors [C,N] + confidence [N] -> one 32-byte record per texture index, so that a fragment costs a single
 // aligned gather instead of C+1 gathers from planes megabytes apart (the reference's BlendMulti reads
 // d_texture.in_texture(ci, idx) per channel, src/lib/rendering/RenderForward.cu:1338-1342).
+// The launch also applies the steps VET runs on the raw tensors right before rendering, when they are switched on:
+// confidence = sigmoid(scale * raw) and texture = |raw| (NeuralPointTextureImpl::PrepareConfidence / PrepareTexture,
+// src/lib/models/NeuralTexture.h:38-55).
 template <int C>
 __global__ void __launch_bounds__(kBlock) pack_descriptors_kernel(const float* __restrict__ texture,
                                                                    const float* __restrict__ confidence,
-                                                                   float4* __restrict__ packed, int N)
+                                                                   float4* __restrict__ packed, int N,
+                                                                   int confidence_activation, float confidence_scale,
+                                                                   int texture_abs)
 {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= N) return;
     float t[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int ci = 0; ci < C; ++ci) t[ci] = texture[(size_t)ci * N + i];
+    for (int ci = 0; ci < C; ++ci)
+    {
+        t[ci] = texture[(size_t)ci * N + i];
+        if (texture_abs) t[ci] = fabsf(t[ci]);
+    }
+    float c = confidence[i];
+    if (confidence_activation) c = sigmoid_canon(confidence_scale * c);
     packed[2 * (size_t)i]     = make_float4(t[0], t[1], t[2], t[3]);
-    packed[2 * (size_t)i + 1] = make_float4(confidence[i], 0.f, 0.f, 0.f);
+    packed[2 * (size_t)i + 1] = make_float4(c, 0.f, 0.f, 0.f);
 }
 
 __device__ __forceinline__ bool point_is_skipped(const ViewPass& a, int i)
@@ -117,7 +161,9 @@ __device__ __forceinline__ bool point_is_skipped(const ViewPass& a, int i)
     if (a.viewer_only)
     {
         const int ti = a.index ? a.index[i] : i;
-        if (a.confidence[ti] < a.stability_cutoff) return true;
+        float c      = a.confidence[ti];
+        if (a.confidence_activation) c = sigmoid_canon(a.confidence_scale * c);
+        if (c < a.stability_cutoff) return true;
     }
     return false;
 }

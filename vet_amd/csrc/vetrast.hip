@@ -4,6 +4,7 @@
 // device->host reads, per-frame allocations and __constant__ uploads.
 #include <hip/hip_runtime.h>
 
+#include <cmath>
 #include <cstring>
 #include <new>
 #include <vector>
@@ -239,6 +240,8 @@ ViewPass make_view_pass(const vetrast_forward_args* a, const vetrast_workspace_l
     vp.radius_threshold = a->params.drop_out_radius_threshold;
     vp.viewer_only      = a->params.viewer_only;
     vp.stability_cutoff = a->params.stability_cutoff_value;
+    vp.confidence_activation = a->params.confidence_activation;
+    vp.confidence_scale      = a->params.confidence_scale;
     return vp;
 }
 
@@ -411,10 +414,10 @@ int vetrast_forward(vetrast_ctx* ctx, const vetrast_forward_args* a, void* strea
             const dim3 g(grid_for(N)), blk(kBlock);
             switch (C)
             {
-                case 1: hipLaunchKernelGGL(pack_descriptors_kernel<1>, g, blk, 0, ctx->side, a->texture, a->confidence, packed, N); break;
-                case 2: hipLaunchKernelGGL(pack_descriptors_kernel<2>, g, blk, 0, ctx->side, a->texture, a->confidence, packed, N); break;
-                case 3: hipLaunchKernelGGL(pack_descriptors_kernel<3>, g, blk, 0, ctx->side, a->texture, a->confidence, packed, N); break;
-                default: hipLaunchKernelGGL(pack_descriptors_kernel<4>, g, blk, 0, ctx->side, a->texture, a->confidence, packed, N); break;
+                case 1: hipLaunchKernelGGL(pack_descriptors_kernel<1>, g, blk, 0, ctx->side, a->texture, a->confidence, packed, N, p.confidence_activation, p.confidence_scale, p.texture_abs); break;
+                case 2: hipLaunchKernelGGL(pack_descriptors_kernel<2>, g, blk, 0, ctx->side, a->texture, a->confidence, packed, N, p.confidence_activation, p.confidence_scale, p.texture_abs); break;
+                case 3: hipLaunchKernelGGL(pack_descriptors_kernel<3>, g, blk, 0, ctx->side, a->texture, a->confidence, packed, N, p.confidence_activation, p.confidence_scale, p.texture_abs); break;
+                default: hipLaunchKernelGGL(pack_descriptors_kernel<4>, g, blk, 0, ctx->side, a->texture, a->confidence, packed, N, p.confidence_activation, p.confidence_scale, p.texture_abs); break;
             }
         }
         VET_HIP(ctx, hipEventRecord(ctx->joined, ctx->side));
@@ -441,7 +444,8 @@ int vetrast_forward(vetrast_ctx* ctx, const vetrast_forward_args* a, void* strea
                 for (int j = 0; j < 4; ++j) s.rot[j] = v.crop_rotation[j];
             }
             hipLaunchKernelGGL(prepare_views_kernel, dim3(1 + (first == 0 ? zero_blocks : 0)), dim3(kBlock), 0, stream, pv,
-                               first, cnt, a->poses_se3, a->intrinsics, views, flags, counters4, n4);
+                               first, cnt, a->poses_se3, a->intrinsics, views, flags, counters4, n4, a->background, C,
+                               p.texture_abs);
         }
     }
 
@@ -512,7 +516,7 @@ int vetrast_forward(vetrast_ctx* ctx, const vetrast_forward_args* a, void* strea
             bp.view                = vp.view;
             bp.index               = a->index;
             bp.packed              = packed;
-            bp.background          = a->background;
+            bp.background          = reinterpret_cast<const float*>(flags) + kPreparedBackgroundOffset;
             bp.transmittance       = a->save_for_backward ? trans : nullptr;
             bp.weight              = weight;
             bp.ly                  = ly;
@@ -624,7 +628,7 @@ int vetrast_backward(vetrast_ctx* ctx, const vetrast_backward_args* g, void* str
             bp.weight           = ws_ptr<float>(ws, lay.weight_base + lay.weight_stride * b);
             bp.index            = a->index;
             bp.packed           = ws_ptr<float4>(ws, lay.packed_base);
-            bp.background       = a->background;
+            bp.background       = ws_ptr<const float>(ws, lay.flags_base) + kPreparedBackgroundOffset;
             bp.partial          = partial;
             bp.background_partial = background_rows;
             bp.ly               = ly;
@@ -685,6 +689,12 @@ int vetrast_backward(vetrast_ctx* ctx, const vetrast_backward_args* g, void* str
             gp.grad_background       = g->grad_background;
             gp.add_leak              = (p.quirk_background_confidence_leak && !p.use_environment_map && hits == 1) ? 1 : 0;
             gp.background_accumulate = b > 0 ? 1 : 0;
+            gp.packed                = ws_ptr<float4>(ws, lay.packed_base);
+            gp.texture_raw           = a->texture;
+            gp.background_raw        = a->background;
+            gp.confidence_activation = p.confidence_activation;
+            gp.confidence_scale      = p.confidence_scale;
+            gp.texture_abs           = p.texture_abs;
             const dim3 grid(grid_for(N)), blk(kBlock);
             if (hits == 1)
                 switch (C)
@@ -716,7 +726,7 @@ int vetrast_backward(vetrast_ctx* ctx, const vetrast_backward_args* g, void* str
             ScopeTimer tm(ctx, stream, VETRAST_SCOPE_BACKWARD_GATHER);
             hipLaunchKernelGGL(reduce_background_kernel, dim3(1), dim3(kReduceBlock), 0, stream, background_rows,
                                (int)(tile_grid(tiles)), C, g->grad_background, g->grad_confidence,
-                               0, b > 0 ? 1 : 0);
+                               0, b > 0 ? 1 : 0, p.texture_abs ? a->background : nullptr);
         }
     }
     if (g->grad_points && p.point_gradient_normalization != 0 && N > 0)
@@ -733,6 +743,28 @@ int vetrast_backward(vetrast_ctx* ctx, const vetrast_backward_args* g, void* str
                            g->grad_pose_count, a->num_poses, g->grad_intrinsics, g->grad_intrinsics_count,
                            a->num_cameras);
     }
+    VET_HIP(ctx, hipGetLastError());
+    return VETRAST_OK;
+}
+
+int vetrast_adam_step(vetrast_ctx* ctx, const vetrast_adam_args* a, void* stream_)
+{
+    if (!ctx || !a) return VETRAST_ERR_INVALID_ARG;
+    if (a->n < 0 || a->step < 1) return VETRAST_ERR_INVALID_ARG;
+    if (a->n == 0) return VETRAST_OK;
+    if (!a->param || !a->grad || !a->exp_avg || !a->exp_avg_sq) return VETRAST_ERR_INVALID_ARG;
+    // bias corrections in double as in src/lib/models/my_adam.cpp:72-73,97-100, handed to the kernel rounded once
+    const double bc1 = 1.0 - std::pow(a->beta1, (double)a->step);
+    const double bc2 = 1.0 - std::pow(a->beta2, (double)a->step);
+    if (!(bc1 > 0.0) || !(bc2 > 0.0)) return VETRAST_ERR_INVALID_ARG;
+    const float sqrt_bc2  = (float)std::sqrt(bc2);
+    const float step_size = (float)(a->lr / bc1);
+    hipStream_t stream    = (hipStream_t)stream_;
+    const int blocks      = (int)std::min<int64_t>((a->n + kBlock - 1) / kBlock, 16384);
+    hipLaunchKernelGGL(adam_step_kernel, dim3(blocks), dim3(kBlock), 0, stream, a->param, a->grad, a->exp_avg,
+                       a->exp_avg_sq, (size_t)a->n, (float)a->beta1, (float)a->beta2, (float)(1.0 - a->beta1),
+                       (float)(1.0 - a->beta2), sqrt_bc2, step_size, (float)a->eps, (float)a->weight_decay,
+                       a->zero_grad);
     VET_HIP(ctx, hipGetLastError());
     return VETRAST_OK;
 }

@@ -34,6 +34,9 @@ def make_params(scene: Scene, **overrides) -> abi.Params:
     p.K_gradient_factor = 0.5
     p.camera_gradient_normalization = 0
     p.render_mode = abi.RENDER_FULL_BLEND
+    p.confidence_activation = 0
+    p.confidence_scale = 10.0
+    p.texture_abs = 0
     for k, v in {**scene.params, **overrides}.items():
         if not hasattr(p, k):
             raise AttributeError(f"vetrast_params has no field {k}")
@@ -271,6 +274,17 @@ class Rasterizer:
         abi.check(self.lib.vetrast_backward(self.ctx, C.byref(g), self._stream()), "backward")
         res["_args"] = g
         return res
+
+    def adam_step(self, param, grad, exp_avg, exp_avg_sq, step, lr, beta1=0.9, beta2=0.999, eps=1e-8,
+                  weight_decay=0.0, zero_grad=False):
+        """One fused Adam step in place on contiguous float32 CUDA tensors (vetrast_adam_step)."""
+        a = abi.AdamArgs()
+        for name, t in (("param", param), ("grad", grad), ("exp_avg", exp_avg), ("exp_avg_sq", exp_avg_sq)):
+            assert t.is_cuda and t.dtype == torch.float32 and t.is_contiguous() and t.numel() == param.numel()
+            setattr(a, name, t.data_ptr())
+        a.n, a.step = param.numel(), step
+        a.lr, a.beta1, a.beta2, a.eps, a.weight_decay, a.zero_grad = lr, beta1, beta2, eps, weight_decay, int(zero_grad)
+        abi.check(self.lib.vetrast_adam_step(self.ctx, C.byref(a), self._stream()), "adam_step")
 
     def check_device_flags(self, fwd: ForwardResult):
         return self.lib.vetrast_query_device_flags(self.ctx, C.c_void_p(fwd.workspace.data_ptr()),
