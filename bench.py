@@ -141,6 +141,55 @@ def run_scene(scene, backward, steps, warmup, profile=True, render_mode=1):
     return res
 
 
+def time_fused_steps(scene, render_mode, steps):
+    """The steps VET runs either side of the rasterizer, fused into the library: the frame with the confidence sigmoid
+    and |texture| folded in (raw tensors in, raw gradients out), and the one-kernel Adam step over texture, confidence
+    and background (vetrast_adam_step). Reported beside the headline number, not part of it."""
+    import torch
+
+    from vet_amd import abi
+    from vet_amd.rasterizer import DeviceScene, Rasterizer, make_params
+
+    rast = Rasterizer()
+    dev = DeviceScene(scene)
+    params = make_params(scene, need_point_gradient=1, render_mode=render_mode, confidence_activation=1,
+                         confidence_scale=10.0, texture_abs=1)
+    fwd = rast.forward(dev, params, save_for_backward=True)
+    grad_out = [torch.from_numpy(g).cuda() for g in scene.grad_out()]
+    bargs = rast.backward(fwd, grad_out)["_args"]
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    def timed(fn, n):
+        for _ in range(3):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(n):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) * 1e3 / n
+
+    def frame():
+        abi.check(rast.lib.vetrast_forward(rast.ctx, C.byref(fwd.args), stream), "forward")
+        abi.check(rast.lib.vetrast_backward(rast.ctx, C.byref(bargs), stream), "backward")
+
+    ms_frame = timed(frame, steps)
+    n = (scene.num_channels + 1) * scene.num_points + scene.num_channels
+    p, g, m, v = (torch.zeros(n, dtype=torch.float32, device="cuda") for _ in range(4))
+    g.normal_()
+    state = {"step": 0}
+
+    def adam():
+        state["step"] += 1
+        rast.adam_step(p, g, m, v, state["step"], 1e-3)
+
+    ms_adam = timed(adam, steps)
+    adam_bytes = 28.0 * n  # param, grad, two moments read; param and moments written
+    return {"frame_with_fused_sigmoid_abs_ms": round(ms_frame, 5), "adam_step_ms": round(ms_adam, 5),
+            "adam_elements": n, "adam_GBps": round(adam_bytes / 1e6 / ms_adam, 1),
+            "adam_frac_of_hbm_peak": round(adam_bytes / 1e6 / ms_adam / HBM_PEAK_GBS, 4)}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -248,6 +297,9 @@ def main():
                        render_mode=args.render_mode)
         result["other_point_order"] = {"point_order": other, "ms_per_step": round(r2["ms_step"], 5),
                                        "forward_ms": round(r2["ms_fwd"], 5)}
+
+    if backward and not args.no_second_order:
+        result["fused_steps"] = time_fused_steps(scene, args.render_mode, max(10, args.steps // 2))
 
     if not args.no_cpu_baseline:
         from oracle import oracle_py

@@ -80,3 +80,51 @@ def test_no_grad_call_and_masks(oracle):
     for l in range(L):
         np.testing.assert_array_equal(outs[l].cpu().numpy(), ref.out[l])
         np.testing.assert_array_equal(outs[L + l].cpu().numpy(), ref.out_mask[l])
+
+
+def test_training_step_on_raw_tensors_with_fused_steps(oracle):
+    """What one VET iteration does around the rasterizer, on the raw tensors: sigmoid on confidence_raw and abs on
+    texture_raw fused into the render call, autograd back to the raw tensors, then MyAdam.step + zero_grad. Compared
+    with the unfused formulation in torch (sigmoid/abs as tensor ops, torch.optim.Adam)."""
+    from vet_amd import torch_ops
+
+    scene = synthetic.tiny_scene(num_points=4000, K=8, seed=33)
+    rng = np.random.default_rng(2)
+    conf_raw = (0.2 * rng.standard_normal(scene.num_points)).astype(np.float32).reshape(1, -1)
+    tex_raw = rng.standard_normal(scene.texture.shape).astype(np.float32)
+    bg_raw = np.array([0.2, -0.5, 0.7, -0.3], np.float32)
+    grad_out = [torch.from_numpy(g).cuda() for g in scene.grad_out()]
+    cu = lambda a, rg=False: torch.from_numpy(np.ascontiguousarray(a)).cuda().requires_grad_(rg)
+    common = dict(use_environment_map=0, need_point_gradient=0, drop_out_points_by_radius=0,
+                  debug_max_list_length=scene.max_list_length, quirk_background_confidence_leak=0,
+                  point_gradient_normalization=0)
+
+    def render(texture, background, confidence, **extra):
+        points = cu(scene.position)
+        tangents = torch.zeros((scene.poses_se3.shape[0], 6), dtype=torch.float64, device="cuda")
+        outs = torch_ops.blend_point_cloud(texture, background, points, tangents, cu(scene.intrinsics), confidence,
+                                           cu(scene.poses_se3), None, _views(scene), scene.num_layers, train=False,
+                                           **common, **extra)
+        return sum((o * g).sum() for o, g in zip(outs, grad_out))
+
+    # fused: raw tensors in, raw gradients out, fused Adam
+    f = [cu(tex_raw, True), cu(bg_raw, True), cu(conf_raw, True)]
+    opt_f = torch_ops.MyAdam([([f[0]], 0.01), ([f[1]], 0.004), ([f[2]], 0.002)])
+    # unfused: the same with tensor ops
+    u = [cu(tex_raw, True), cu(bg_raw, True), cu(conf_raw, True)]
+    opt_u = torch.optim.Adam([{"params": [u[0]], "lr": 0.01}, {"params": [u[1]], "lr": 0.004},
+                              {"params": [u[2]], "lr": 0.002}])
+    for it in range(3):
+        loss_f = render(f[0], f[1], f[2], fused_confidence_scale=10.0, fused_texture_abs=1)
+        loss_f.backward()
+        loss_u = render(torch.abs(u[0]), torch.abs(u[1]), torch.sigmoid(10.0 * u[2]))
+        loss_u.backward()
+        assert abs(loss_f.item() - loss_u.item()) <= 1e-4 * max(1.0, abs(loss_u.item()))
+        for a, b in zip(f, u):
+            assert max_rel_err(a.grad.cpu().numpy(), b.grad.cpu().numpy()) <= 1e-4
+        opt_f.step(zero_grad=True)
+        opt_u.step()
+        opt_u.zero_grad()
+        for a, b in zip(f, u):
+            assert not a.grad.any()
+            assert max_rel_err(a.detach().cpu().numpy(), b.detach().cpu().numpy()) <= 1e-4, it

@@ -42,6 +42,9 @@ vetrast_params to_abi_params(const RenderParams& p, int num_layers)
     q.point_gradient_normalization     = p.point_gradient_normalization;
     q.K_gradient_factor                = p.K_gradient_factor;
     q.camera_gradient_normalization    = p.camera_gradient_normalization ? 1 : 0;
+    q.confidence_activation            = p.fused_confidence_scale > 0.f ? 1 : 0;
+    q.confidence_scale                 = p.fused_confidence_scale;
+    q.texture_abs                      = p.fused_texture_abs ? 1 : 0;
     return q;
 }
 
@@ -352,6 +355,8 @@ std::vector<torch::Tensor> blend_point_cloud(torch::Tensor texture, torch::Tenso
         else if (k == "render_mode") p.render_mode = (int)as_d();
         else if (k == "K_gradient_factor") p.K_gradient_factor = (float)as_d();
         else if (k == "camera_gradient_normalization") p.camera_gradient_normalization = as_d() != 0;
+        else if (k == "fused_confidence_scale") p.fused_confidence_scale = (float)as_d();
+        else if (k == "fused_texture_abs") p.fused_texture_abs = as_d() != 0;
         else TORCH_CHECK(false, "unknown RenderParams field ", k);
     }
     // the scene bundle only has to live for the duration of apply(): everything backward needs is saved in the graph
@@ -359,8 +364,75 @@ std::vector<torch::Tensor> blend_point_cloud(torch::Tensor texture, torch::Tenso
 }
 }  // namespace
 
+namespace vet_amd
+{
+MyAdam::MyAdam(std::vector<Group> groups, double beta1, double beta2, double eps, double weight_decay)
+    : groups_(std::move(groups)), beta1_(beta1), beta2_(beta2), eps_(eps), weight_decay_(weight_decay),
+      cache_(std::make_unique<PointRendererCache>())
+{
+    state_.resize(groups_.size());
+    for (size_t g = 0; g < groups_.size(); ++g) state_[g].resize(groups_[g].params.size());
+}
+
+void MyAdam::step(bool zero_grad)
+{
+    torch::NoGradGuard no_grad;
+    for (size_t g = 0; g < groups_.size(); ++g)
+        for (size_t k = 0; k < groups_[g].params.size(); ++k)
+        {
+            torch::Tensor& p = groups_[g].params[k];
+            if (!p.grad().defined()) continue;  // my_adam.cpp:38-41
+            torch::Tensor grad = p.grad();
+            TORCH_CHECK(p.is_cuda() && p.scalar_type() == torch::kFloat32 && p.is_contiguous() && grad.is_contiguous() &&
+                            grad.scalar_type() == torch::kFloat32,
+                        "MyAdam: parameters and gradients must be contiguous float32 tensors on the GPU");
+            State& st = state_[g][k];
+            if (!st.exp_avg.defined() || st.exp_avg.numel() != p.numel())  // state initialisation, my_adam.cpp:48-62
+            {
+                st.exp_avg    = torch::zeros_like(p);
+                st.exp_avg_sq = torch::zeros_like(p);
+                st.step       = 0;
+            }
+            st.step += 1;
+            vetrast_adam_args a;
+            std::memset(&a, 0, sizeof(a));
+            a.param        = p.data_ptr<float>();
+            a.grad         = grad.data_ptr<float>();
+            a.exp_avg      = st.exp_avg.data_ptr<float>();
+            a.exp_avg_sq   = st.exp_avg_sq.data_ptr<float>();
+            a.n            = p.numel();
+            a.step         = st.step;
+            a.lr           = groups_[g].lr;
+            a.beta1        = beta1_;
+            a.beta2        = beta2_;
+            a.eps          = eps_;
+            a.weight_decay = weight_decay_;
+            a.zero_grad    = zero_grad ? 1 : 0;
+            check_status(vetrast_adam_step(cache_->ctx, &a, c10::hip::getCurrentHIPStream().stream()), "adam_step");
+        }
+}
+
+void MyAdam::zero_grad()
+{
+    for (auto& g : groups_)
+        for (auto& p : g.params)
+            if (p.grad().defined()) p.mutable_grad().zero_();
+}
+}  // namespace vet_amd
+
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
 {
+    pybind11::class_<vet_amd::MyAdam>(m, "MyAdam")
+        .def(pybind11::init([](std::vector<std::pair<std::vector<torch::Tensor>, double>> groups, double beta1,
+                               double beta2, double eps, double weight_decay) {
+                 std::vector<vet_amd::MyAdam::Group> gs;
+                 for (auto& g : groups) gs.push_back({g.first, g.second});
+                 return std::make_unique<vet_amd::MyAdam>(std::move(gs), beta1, beta2, eps, weight_decay);
+             }),
+             pybind11::arg("groups"), pybind11::arg("beta1") = 0.9, pybind11::arg("beta2") = 0.999,
+             pybind11::arg("eps") = 1e-8, pybind11::arg("weight_decay") = 0.0)
+        .def("step", &vet_amd::MyAdam::step, pybind11::arg("zero_grad") = false)
+        .def("zero_grad", &vet_amd::MyAdam::zero_grad);
     m.def("blend_point_cloud", &blend_point_cloud,
           "BlendPointCloud(NeuralRenderInfo*) of the reference, with the scene passed as tensors");
 }

@@ -41,6 +41,11 @@ struct RenderParams
     bool quirk_background_confidence_leak = true;   // src/lib/rendering/RenderBackward.cu:1157
     int point_gradient_normalization      = 2;      // src/lib/rendering/PointRenderer.cu:1278-1279
     bool camera_gradient_normalization    = true;   // src/lib/rendering/PointRenderer.cu:1253-1308
+    // The two steps Pipeline.cpp:113-124 runs on the optimised tensors right before rendering, fused into the rasterizer
+    // when switched on; `texture`, `background_color` and `confidence` passed to BlendPointCloud are then the RAW tensors
+    // (texture_raw, background_color_raw, confidence_raw) and autograd returns the gradients of those.
+    float fused_confidence_scale = 0.f;  // > 0: confidence = sigmoid(scale * raw), scale = 10 + narrowing * epoch
+    bool fused_texture_abs       = false;  // texture = |raw|, background = |raw| (non_subzero_texture)
 };
 
 // The tensors BlendPointCloud reads through info->scene (src/lib/rendering/RenderInfo.cpp:25-29 and
@@ -93,6 +98,36 @@ struct PointRender : public torch::autograd::Function<PointRender>
                                                   torch::IValue info);
     static torch::autograd::variable_list backward(torch::autograd::AutogradContext* ctx,
                                                    torch::autograd::variable_list grad_output);
+};
+
+// Adam over groups of flat float tensors with one kernel per tensor and step: the update of torch::optim::MyAdam
+// (src/lib/models/my_adam.cpp:25-104) as the reference sets it up for texture_raw, background_color_raw and confidence_raw,
+// one group and learning rate each (src/lib/data/NeuralScene.cpp:238-281), stepped and cleared once per batch (:1247-1248).
+class MyAdam
+{
+   public:
+    struct Group
+    {
+        std::vector<torch::Tensor> params;
+        double lr = 1e-3;
+    };
+    explicit MyAdam(std::vector<Group> groups, double beta1 = 0.9, double beta2 = 0.999, double eps = 1e-8,
+                    double weight_decay = 0.0);
+    // One step on every parameter that has a gradient; with zero_grad the gradients are cleared in the same pass
+    // (texture_optimizer->step(); texture_optimizer->zero_grad();).
+    void step(bool zero_grad = false);
+    void zero_grad();
+
+   private:
+    struct State
+    {
+        torch::Tensor exp_avg, exp_avg_sq;
+        int64_t step = 0;
+    };
+    std::vector<Group> groups_;
+    std::vector<std::vector<State>> state_;
+    double beta1_, beta2_, eps_, weight_decay_;
+    std::unique_ptr<PointRendererCache> cache_;
 };
 
 // Render the scene into a batch of images; every image is a pyramid of layers: L tensors [B,C,h_l,w_l], then L masks

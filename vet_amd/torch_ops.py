@@ -31,3 +31,9 @@ def blend_point_cloud(texture, background_color, points, pose_tangents, intrinsi
     return load().blend_point_cloud(texture, background_color, points, pose_tangents, intrinsics, confidence, poses_se3,
                                     t_index, [list(map(float, v)) for v in views], int(num_layers), bool(train),
                                     {k: float(v) for k, v in params.items()})
+
+
+def MyAdam(groups, beta1=0.9, beta2=0.999, eps=1e-8, weight_decay=0.0):
+    """The reference's texture optimiser (torch::optim::MyAdam, src/lib/models/my_adam.cpp) with one fused kernel per
+    tensor and step. groups: list of (list of float32 CUDA parameter tensors, learning rate)."""
+    return load().MyAdam([(list(ts), float(lr)) for ts, lr in groups], beta1, beta2, eps, weight_decay)
