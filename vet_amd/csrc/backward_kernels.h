@@ -29,7 +29,6 @@ struct BackwardPass
     float* background_partial;  // [workgroups][8]: per-workgroup sums of d background[0..C) and of the leak term
     LayerTable ly;
     TileMap tiles;
-    uint32_t P;
     int N;
     int K;
     int use_environment_map;

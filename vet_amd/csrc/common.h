@@ -9,7 +9,6 @@ namespace vetrast
 {
 constexpr int kBlock          = 256;          // threads per workgroup = 4 wave64
 constexpr int kWave           = 64;
-constexpr uint32_t kNoSlot    = 0xFFFFFFFFu;
 constexpr uint64_t kInfKey    = ~0ull;        // sorts behind every real (depth bits, point id) key
 constexpr int kScanPerThread  = 16;
 constexpr int kScanPerBlock   = kBlock * kScanPerThread;  // 4096 counts per workgroup
@@ -132,12 +131,6 @@ __device__ __forceinline__ bool layer_hit(const LayerTable& ly, int l, float ipx
         return tile_of_pixel(ly, l, floorf(ipx) + (float)(h & 1), floorf(ipy) + (float)(h >> 1), tile, in_tile);
 }
 
-__device__ __forceinline__ bool layer_tile_pixel(const LayerTable& ly, int l, float ipx, float ipy, uint32_t& tile,
-                                                 uint32_t& in_tile)
-{
-    return layer_hit<1>(ly, l, ipx, ipy, 0, tile, in_tile);
-}
-
 // compute_blending_fac (src/lib/rendering/PointBlending.h:12-44): bilinear weight of corner `corner` of a position, and
 // optionally its derivative with respect to the position.
 __device__ __forceinline__ float bilinear_weight(float u, float v, int corner, float* d_du = nullptr,
@@ -164,23 +157,6 @@ __device__ __forceinline__ void bin_of_pixel(const LayerTable& ly, int l, uint32
     const uint32_t in_layer = (tile - ly.tile_base[l]) * kTilePixels + in_tile;
     bin    = ly.bin_base[l] + (in_layer >> ly.bin_shift[l]);
     in_bin = in_layer & ((1u << ly.bin_shift[l]) - 1u);
-}
-
-// Pixel number of layer l for a projected point, or -1.
-__device__ __forceinline__ int64_t layer_pixel(const LayerTable& ly, int l, float ipx, float ipy)
-{
-    uint32_t tile, in_tile;
-    if (!layer_tile_pixel(ly, l, ipx, ipy, tile, in_tile)) return -1;
-    return (int64_t)tile * kTilePixels + in_tile;
-}
-
-__device__ __forceinline__ int layer_of_pixel(const LayerTable& ly, uint32_t q)
-{
-    int l = 0;
-#pragma unroll
-    for (int k = 1; k < VETRAST_MAX_LAYERS; ++k)
-        if (k < ly.L && q >= ly.base[k]) l = k;
-    return l;
 }
 
 // exp and the logistic function from +, *, rint and one division only, so that the CPU check of the same formulas

@@ -1,4 +1,5 @@
-// Forward kernels: zero fill, view preparation, descriptor interleave, project+count, scan, fill, blend.
+// Forward kernels: zero fill, view preparation, descriptor interleave (+ fused preparation steps), Adam step, per-bin
+// count, scan, fill. The per-bin build / sort / blend pass is in build_kernels.h.
 #pragma once
 #include "common.h"
 
@@ -9,14 +10,6 @@ __global__ void __launch_bounds__(kBlock) fill_u32_kernel(uint32_t* __restrict__
 {
     const size_t stride = (size_t)gridDim.x * blockDim.x;
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) dst[i] = value;
-}
-
-// 16-byte wide variant for the big buffers; n4 counts uint4 elements.
-__global__ void __launch_bounds__(kBlock) fill_u128_kernel(uint4* __restrict__ dst, size_t n4, uint32_t value)
-{
-    const size_t stride = (size_t)gridDim.x * blockDim.x;
-    const uint4 v       = make_uint4(value, value, value, value);
-    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += stride) dst[i] = v;
 }
 
 // One Adam step on n floats (MyAdam::step, src/lib/models/my_adam.cpp:66-101, i.e. torch's Adam without amsgrad), every

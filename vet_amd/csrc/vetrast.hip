@@ -570,7 +570,6 @@ int vetrast_backward(vetrast_ctx* ctx, const vetrast_backward_args* g, void* str
     const int hits      = hits_of_mode(p.render_mode);
     const LayerTable ly = make_layer_table(a->views[0].w, a->views[0].h, L, (int64_t)N * hits);
     const TileMap tiles = make_tile_map(ly);
-    const uint32_t P    = ly.base[L];
     void* ws            = a->workspace;
 
     // The per-point kernel overwrites every gradient row in the first view, so the zeros_like fills of
@@ -633,7 +632,6 @@ int vetrast_backward(vetrast_ctx* ctx, const vetrast_backward_args* g, void* str
             bp.background_partial = background_rows;
             bp.ly               = ly;
             bp.tiles            = tiles;
-            bp.P                = P;
             bp.N                = N;
             bp.K                = p.debug_max_list_length;
             bp.use_environment_map              = p.use_environment_map;
