@@ -190,6 +190,51 @@ def time_fused_steps(scene, render_mode, steps):
             "adam_frac_of_hbm_peak": round(adam_bytes / 1e6 / ms_adam / HBM_PEAK_GBS, 4)}
 
 
+def time_lift_error(scene, steps, cpu_threads):
+    """Error lifting (vetrast_lift_error; the reference's FillSceneGridWithLoss), the step that runs once per view in the
+    epoch before VET adds points: the scene's grid at 0.25 m under the scene's own camera and a synthetic 3-channel
+    error image. Reported beside the headline number, not part of it; the CPU oracle is timed on the same call."""
+    import torch
+
+    from vet_amd import synthetic
+    from vet_amd.rasterizer import Rasterizer
+
+    rast = Rasterizer()
+    cell_size = 0.25
+    mn, ln = synthetic.cell_grid(scene.position[:, :3], cell_size)
+    view = scene.views[0]
+    img = synthetic.error_image(5, 3, view.h, view.w)
+    to_dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
+    d_mn, d_ln, d_img, d_pose, d_intr = (to_dev(a) for a in (mn, ln, img, scene.poses_se3, scene.intrinsics))
+    val = torch.zeros(len(mn), dtype=torch.float32, device="cuda")
+    cnt = torch.zeros(len(mn), dtype=torch.int32, device="cuda")
+    ws = rast.lift_error(d_mn, d_ln, val, cnt, view, d_pose, d_intr, d_img)
+    torch.cuda.synchronize()
+    pixels = int(cnt.sum().item())
+    queued = int(ws[128:132].view(torch.int32).item())
+    for _ in range(3):
+        rast.lift_error(d_mn, d_ln, val, cnt, view, d_pose, d_intr, d_img, workspace=ws)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        rast.lift_error(d_mn, d_ln, val, cnt, view, d_pose, d_intr, d_img, workspace=ws)
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / steps
+    out = {"cells": int(len(mn)), "cell_size_m": cell_size, "cells_on_shared_path": queued, "pixels_added": pixels,
+           "ms_per_call": round(ms, 5), "pixels_added_per_s": round(pixels / ms * 1e3, 0)}
+    if cpu_threads:
+        from oracle import oracle_py
+
+        v = np.zeros(len(mn), np.float32)
+        c = np.zeros(len(mn), np.int32)
+        t0 = time.perf_counter()
+        oracle_py.lift_error(mn, ln, v, c, view, scene.poses_se3, scene.intrinsics, img, num_threads=cpu_threads)
+        out["cpu_oracle_ms"] = round((time.perf_counter() - t0) * 1e3, 1)
+        out["cpu_oracle_threads"] = cpu_threads
+        out["counts_equal_cpu_oracle"] = bool(np.array_equal(c, cnt.cpu().numpy() // (steps + 4)))
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -300,6 +345,10 @@ def main():
 
     if backward and not args.no_second_order:
         result["fused_steps"] = time_fused_steps(scene, args.render_mode, max(10, args.steps // 2))
+
+    if not args.no_second_order:
+        lift_threads = 0 if args.no_cpu_baseline else (args.cpu_threads or min(16, len(os.sched_getaffinity(0))))
+        result["lift_error"] = time_lift_error(scene, max(10, args.steps // 2), lift_threads)
 
     if not args.no_cpu_baseline:
         from oracle import oracle_py

@@ -117,6 +117,7 @@ typedef enum vetrast_scope
     VETRAST_SCOPE_BACKWARD_BLEND,   /* "BlendBackwards", per-pixel part */
     VETRAST_SCOPE_BACKWARD_GATHER,  /* "BlendBackwards", per-point sum of the stored fragment gradients */
     VETRAST_SCOPE_BACKWARD_POST,    /* "Post Process Gradient" */
+    VETRAST_SCOPE_LIFT_ERROR,       /* vetrast_lift_error (the reference times FillSceneGridWithLoss in no scope) */
     VETRAST_SCOPE_COUNT_
 } vetrast_scope;
 
@@ -260,6 +261,47 @@ typedef struct vetrast_adam_args
     int32_t zero_grad;
 } vetrast_adam_args;
 int vetrast_adam_step(vetrast_ctx* ctx, const vetrast_adam_args* args, void* stream);
+
+/* Error lifting: adds the per-pixel error of one rendered view to every cell of the scene grid whose projection covers
+ * the pixel. Replaces PointRendererCache::FillSceneGridWithLoss and its kernel FillSceneGridWithLossRasterize
+ * (src/lib/rendering/RenderForward.cu:605-632,639-791; called once per view of a batch in the epoch before points are
+ * added, src/apps/train.cpp:1069-1078; cell tensors: src/lib/rendering/NeuralPointCloudCuda.h:100-106,166-191,
+ * built by UpdateCellStructureForPointOptim, src/lib/rendering/NeuralPointCloudCuda.cpp:95-147).
+ *
+ * For every cell: the 8 corners bb_min + bb_length * {000,100,010,001,110,101,011,111} are projected like points
+ * (pinhole, zero distortion, crop transform and rotation of `view`); a cell with a corner at or behind the camera
+ * plane is skipped; the pixel box of the 8 projections is cut to the image minus a border of `border_pixels`
+ * (VETRAST_LIFT_BORDER_PIXELS in the reference); every integer pixel of the box that lies in one of the 12 projected
+ * face triangles adds sum_c |loss_image[c][y][x]| to cell_value and 1 to cell_access_count.
+ *
+ * The reference adds the float terms with atomics in arrival order; here the terms of a cell are summed in double and
+ * added to cell_value with one rounding, which makes the call reproducible. cell_value and cell_access_count are
+ * accumulated into, not cleared (ResetCellValues / NormalizeBBCellValue stay with the caller,
+ * src/lib/rendering/NeuralPointCloudCuda.h:42-52). */
+#define VETRAST_LIFT_BORDER_PIXELS 32
+/* Byte offset inside the workspace of a uint32 that is 1 after the call if the camera row holds non-zero distortion
+ * coefficients (they are ignored, as in vetrast_forward), else 0. */
+#define VETRAST_LIFT_FLAGS_OFFSET 192
+typedef struct vetrast_lift_args
+{
+    int64_t num_cells;
+    const float* cell_bb_min;    /* device [num_cells,3] (t_cell_bb_min) */
+    const float* cell_bb_length; /* device [num_cells,3] (t_cell_bb_length) */
+    float* cell_value;           /* device [num_cells] (t_cell_value, [num_cells,1]); accumulated into */
+    int32_t* cell_access_count;  /* device [num_cells] (t_cell_access_count); accumulated into */
+    int32_t num_poses;           /* rows of poses_se3 */
+    int32_t num_cameras;
+    const double* poses_se3;     /* device [num_poses,8], as in vetrast_forward_args */
+    const float* intrinsics;     /* device [num_cameras,13], as in vetrast_forward_args */
+    vetrast_view view;           /* the view the error image belongs to (images[batch]); w / 2, h / 2 is the crop rotation centre */
+    const float* loss_image;     /* device [channels,height,width], e.g. |target - output| of that view */
+    int32_t channels, height, width;
+    int32_t border_pixels;       /* >= 0; the reference's constant is VETRAST_LIFT_BORDER_PIXELS */
+    void* workspace;             /* device, 256-byte aligned, vetrast_lift_workspace_bytes(num_cells) bytes */
+    size_t workspace_bytes;
+} vetrast_lift_args;
+size_t vetrast_lift_workspace_bytes(int64_t num_cells);
+int vetrast_lift_error(vetrast_ctx* ctx, const vetrast_lift_args* args, void* stream);
 
 /* Per-kernel timing, the counterpart of NeuralRenderInfo::timer_system (src/lib/rendering/PointRenderer.h:32).
  * With profiling enabled every launch is bracketed by HIP events on the call's stream; vetrast_scope_times

@@ -10,7 +10,7 @@ import subprocess
 import numpy as np
 
 from vet_amd import abi
-from vet_amd.rasterizer import fill_forward_args, make_params, make_views
+from vet_amd.rasterizer import fill_forward_args, fill_lift_args, make_params, make_views
 from vet_amd.synthetic import Scene
 
 HERE = os.path.dirname(os.path.abspath(__file__))
@@ -42,6 +42,8 @@ def load():
         lib.vetref_sigmoid.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_float]
         lib.vetref_adam_step.restype = C.c_int
         lib.vetref_adam_step.argtypes = [C.POINTER(abi.AdamArgs)]
+        lib.vetref_lift_error.restype = C.c_int
+        lib.vetref_lift_error.argtypes = [C.POINTER(abi.LiftArgs), C.c_int]
         _lib = lib
     return _lib
 
@@ -174,3 +176,21 @@ def adam_step(param, grad, exp_avg, exp_avg_sq, step, lr, beta1=0.9, beta2=0.999
     st = load().vetref_adam_step(C.byref(a))
     if st != 0:
         raise abi.VetrastError(st, "oracle adam_step")
+
+
+def lift_error(cell_bb_min, cell_bb_length, cell_value, cell_access_count, view, poses_se3, intrinsics, loss_image,
+               border_pixels=abi.LIFT_BORDER_PIXELS, num_threads=1):
+    """Error lifting on numpy arrays, in place on cell_value (float32 [n]) and cell_access_count (int32 [n])."""
+    a = abi.LiftArgs()
+    for name, arr, dt in (("cell_bb_min", cell_bb_min, np.float32), ("cell_bb_length", cell_bb_length, np.float32),
+                          ("cell_value", cell_value, np.float32), ("cell_access_count", cell_access_count, np.int32),
+                          ("poses_se3", poses_se3, np.float64), ("intrinsics", intrinsics, np.float32),
+                          ("loss_image", loss_image, np.float32)):
+        assert arr.dtype == dt and arr.flags.c_contiguous, name
+        setattr(a, name, _addr(arr))
+    a.num_cells = cell_value.size
+    assert cell_bb_min.shape == (a.num_cells, 3) and cell_bb_length.shape == (a.num_cells, 3)
+    fill_lift_args(a, view, poses_se3, intrinsics, loss_image, border_pixels)
+    st = load().vetref_lift_error(C.byref(a), num_threads)
+    if st != 0:
+        raise abi.VetrastError(st, "oracle lift_error")

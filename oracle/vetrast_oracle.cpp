@@ -1001,3 +1001,96 @@ extern "C" int vetref_adam_step(const vetrast_adam_args* a)
     }
     return VETRAST_OK;
 }
+
+// sign() and PointInTriangle(), rendering/RenderForward.cu:605-625.
+static inline float lift_sign(const float* p1, const float* p2, const float* p3)
+{
+    return (p1[0] - p3[0]) * (p2[1] - p3[1]) - (p2[0] - p3[0]) * (p1[1] - p3[1]);
+}
+
+static inline bool lift_point_in_triangle(const float* pt, const float* v1, const float* v2, const float* v3)
+{
+    const float d1 = lift_sign(pt, v1, v2), d2 = lift_sign(pt, v2, v3), d3 = lift_sign(pt, v3, v1);
+    const bool has_neg = (d1 < 0) || (d2 < 0) || (d3 < 0);
+    const bool has_pos = (d1 > 0) || (d2 > 0) || (d3 > 0);
+    return !(has_neg && has_pos);
+}
+
+// Error lifting: FillSceneGridWithLossRasterize, rendering/RenderForward.cu:639-761, one cell after the other and the
+// pixels of a cell in the order of the reference's xy_c counter. The reference leaves a cell when min_depths is set,
+// which a lane may read before the lanes that project have written it (no __syncwarp, :704-705); the oracle takes the
+// evident intent: a cell with any corner at z <= 0 is skipped. The float terms of a cell are summed in double and added
+// to cell_value with one rounding (the reference's atomicAdd order is unspecified).
+extern "C" int vetref_lift_error(const vetrast_lift_args* a, int num_threads)
+{
+    if (!a || a->num_cells < 0 || a->channels < 1 || a->height < 1 || a->width < 1) return VETRAST_ERR_INVALID_ARG;
+    const vetrast_view& v = a->view;
+    if (v.image_index < 0 || v.image_index >= a->num_poses || v.camera_index < 0 || v.camera_index >= a->num_cameras)
+        return VETRAST_ERR_INVALID_ARG;
+    const Prepared cam = prepare(a->poses_se3 + 8 * (size_t)v.image_index, a->intrinsics + 13 * (size_t)v.camera_index);
+    const int border   = a->border_pixels;
+    const int W = a->width, H = a->height;
+    static const int tris[12][3]    = {{0, 1, 4}, {0, 4, 2}, {1, 5, 7}, {1, 7, 4}, {5, 3, 6}, {5, 6, 7},
+                                       {3, 0, 6}, {0, 6, 2}, {3, 0, 5}, {0, 5, 1}, {2, 4, 6}, {4, 6, 7}};
+    static const float bb_facs[8][3] = {{0, 0, 0}, {1, 0, 0}, {0, 1, 0}, {0, 0, 1}, {1, 1, 0}, {1, 0, 1}, {0, 1, 1}, {1, 1, 1}};
+    omp_set_num_threads(num_threads > 0 ? num_threads : 1);
+#pragma omp parallel for schedule(dynamic, 16) if (num_threads > 1)
+    for (int64_t cell = 0; cell < a->num_cells; ++cell)
+    {
+        float proj[8][2];
+        bool behind = false;
+        for (int i = 0; i < 8; ++i)
+        {
+            float p4[4];
+            for (int k = 0; k < 3; ++k) p4[k] = a->cell_bb_min[3 * cell + k] + a->cell_bb_length[3 * cell + k] * bb_facs[i][k];
+            p4[3] = 0.f;
+            Projected o;
+            if (!project(cam, v, p4, o))  // z <= 0 (:694)
+            {
+                behind = true;
+                break;
+            }
+            proj[i][0] = o.ipx;
+            proj[i][1] = o.ipy;
+        }
+        if (behind) continue;
+        float max_x = -10000000.f, max_y = -10000000.f, min_x = 10000000.f, min_y = 10000000.f;
+        for (int i = 0; i < 8; ++i)
+        {
+            max_x = std::fmax(proj[i][0], max_x);
+            max_y = std::fmax(proj[i][1], max_y);
+            min_x = std::fmin(proj[i][0], min_x);
+            min_y = std::fmin(proj[i][1], min_y);
+        }
+        if (max_x < border || min_x >= W - border || max_y < border || min_y >= H - border) continue;
+        min_x = std::fmax(min_x, (float)border);
+        min_y = std::fmax(min_y, (float)border);
+        max_x = std::fmin(max_x, (float)(W - border));
+        max_y = std::fmin(max_y, (float)(H - border));
+        const int y_size = int(max_y - min_y);
+        const int x_size = int(max_x - min_x);
+        double sum = 0.0;
+        int count  = 0;
+        for (int xy_c = 0; xy_c < y_size * x_size; ++xy_c)
+        {
+            const int x_c     = (int)((float)(xy_c % x_size) + min_x);
+            const int y_c     = (int)((float)(xy_c / x_size) + min_y);
+            const float pt[2] = {(float)x_c, (float)y_c};
+            bool is_in        = false;
+            for (int t = 0; t < 12; ++t)
+                if (lift_point_in_triangle(pt, proj[tris[t][0]], proj[tris[t][1]], proj[tris[t][2]])) is_in = true;
+            if (!is_in) continue;
+            if (x_c < 0 || x_c >= W || y_c < 0 || y_c >= H) continue;  // cannot happen with border >= 0
+            float grad = 0.f;
+            for (int i = 0; i < a->channels; ++i) grad += std::fabs(a->loss_image[((size_t)i * H + y_c) * W + x_c]);
+            sum += (double)grad;
+            count += 1;
+        }
+        if (count > 0)
+        {
+            a->cell_value[cell]        = (float)((double)a->cell_value[cell] + sum);
+            a->cell_access_count[cell] = a->cell_access_count[cell] + count;
+        }
+    }
+    return VETRAST_OK;
+}

@@ -33,6 +33,13 @@
  *                     torch::sigmoid are PARITY UNPINNED), |texture| / |background| and the chain rule of both by
  *                     comparing with the unfused path fed the prepared tensors and torch autograd
  *   Adam step         pinned against torch.optim.Adam on the CPU over several steps with and without weight decay
+ *   error lifting     literal restatement; pinned by an independent numpy rasterization (the union of the 12 projected
+ *                     face triangles is the convex hull of the 8 projected corners, tested with half-plane checks of a
+ *                     hull built by scipy, away from the hull's boundary), by closed forms (an axis-aligned cell seen
+ *                     head-on covers a known pixel rectangle, a constant error image gives value = channels * count)
+ *                     and by the skip rules (corner behind the camera, box outside the border). The reference kernel
+ *                     is compiled with nvcc's default fused multiply-add; which side of a triangle edge a pixel
+ *                     exactly on it falls under that contraction is PARITY UNPINNED
  *   distortion != 0, check_normal, OCam, spherical: not implemented (rejected), PARITY UNPINNED
  */
 #ifndef VETRAST_ORACLE_H
@@ -64,6 +71,9 @@ int vetref_sigmoid(const float* x, float* y, int64_t n, float scale);
 
 /* One Adam step on host arrays (MyAdam::step). */
 int vetref_adam_step(const vetrast_adam_args* args);
+
+/* Error lifting on host arrays (FillSceneGridWithLossRasterize); the workspace is ignored. */
+int vetref_lift_error(const vetrast_lift_args* args, int num_threads);
 
 #ifdef __cplusplus
 }

@@ -21,7 +21,7 @@ def declared_functions():
 def test_library_exports_every_declared_symbol():
     lib = abi.load_library()
     names = declared_functions()
-    assert len(names) >= 16
+    assert len(names) >= 18
     assert sorted(abi.SYMBOLS) == names, "vet_amd/abi.py and include/vetrast.h disagree"
     for n in names:
         assert getattr(lib, n) is not None
@@ -31,6 +31,8 @@ def test_struct_sizes_are_the_c_ones():
     # sizes the C compiler gives the structs of include/vetrast.h (LP64)
     assert C.sizeof(abi.View) == 5 * 4 + 9 * 4
     assert C.sizeof(abi.Params) == 20 * 4
+    assert C.sizeof(abi.LiftArgs) == 8 + 4 * 8 + 2 * 4 + 2 * 8 + C.sizeof(abi.View) + 8 + 4 * 4 + 2 * 8 == 160
+    assert abi.LiftArgs.loss_image.offset % 8 == 0
     assert C.sizeof(abi.ForwardArgs) % 8 == 0
     assert abi.BackwardArgs.grad_out.offset == C.sizeof(abi.ForwardArgs)
 

@@ -24,6 +24,7 @@ RENDER_BILINEAR_BLEND = 3
 
 SCOPE_NAMES = [
     "PREPARE", "PACK", "COUNT", "SCAN", "FILL", "BUILD", "BACKWARD_PREPARE", "BACKWARD_BLEND", "BACKWARD_GATHER", "BACKWARD_POST",
+    "LIFT_ERROR",
 ]
 SCOPE_COUNT = len(SCOPE_NAMES)
 
@@ -105,6 +106,26 @@ class AdamArgs(C.Structure):
     ]
 
 
+LIFT_BORDER_PIXELS = 32
+LIFT_FLAGS_OFFSET = 192
+
+
+class LiftArgs(C.Structure):
+    _fields_ = [
+        ("num_cells", C.c_int64),
+        ("cell_bb_min", C.c_void_p), ("cell_bb_length", C.c_void_p),
+        ("cell_value", C.c_void_p), ("cell_access_count", C.c_void_p),
+        ("num_poses", C.c_int32), ("num_cameras", C.c_int32),
+        ("poses_se3", C.c_void_p), ("intrinsics", C.c_void_p),
+        ("view", View),
+        ("loss_image", C.c_void_p),
+        ("channels", C.c_int32), ("height", C.c_int32), ("width", C.c_int32),
+        ("border_pixels", C.c_int32),
+        ("workspace", C.c_void_p),
+        ("workspace_bytes", C.c_size_t),
+    ]
+
+
 class ForwardArgs(C.Structure):
     _fields_ = [
         ("num_points", C.c_int32), ("num_views", C.c_int32), ("num_poses", C.c_int32), ("num_cameras", C.c_int32),
@@ -155,6 +176,8 @@ SYMBOLS = {
     "vetrast_forward": (C.c_int, [C.c_void_p, C.POINTER(ForwardArgs), C.c_void_p]),
     "vetrast_backward": (C.c_int, [C.c_void_p, C.POINTER(BackwardArgs), C.c_void_p]),
     "vetrast_adam_step": (C.c_int, [C.c_void_p, C.POINTER(AdamArgs), C.c_void_p]),
+    "vetrast_lift_workspace_bytes": (C.c_size_t, [C.c_int64]),
+    "vetrast_lift_error": (C.c_int, [C.c_void_p, C.POINTER(LiftArgs), C.c_void_p]),
     "vetrast_query_device_flags": (C.c_int, [C.c_void_p, C.c_void_p, C.POINTER(WorkspaceLayout), C.c_void_p]),
     "vetrast_set_profiling": (C.c_int, [C.c_void_p, C.c_int32]),
     "vetrast_reset_scope_times": (C.c_int, [C.c_void_p]),

@@ -49,9 +49,48 @@ struct PrepareViewsArgs
     ViewSource src[16];
 };
 
-// One thread per view: pose (unit quaternion + translation, double) -> 3x4 float matrix, intrinsics row -> K.
+// Camera constants of one view: pose (unit quaternion + translation, double) -> 3x4 float matrix, intrinsics row -> K.
 // The reference casts the SE3d to float in every thread (src/lib/rendering/RenderConstants.h:78); here the rotation
-// matrix is formed once, in double, and rounded once. Non-zero distortion coefficients raise flag bit 0.
+// matrix is formed once, in double, and rounded once. `distorted` reports non-zero distortion coefficients.
+__device__ __forceinline__ DeviceView make_device_view(const ViewSource& s, const double* __restrict__ poses_se3,
+                                                       const float* __restrict__ intrinsics, bool& distorted)
+{
+    const double* q = poses_se3 + 8 * (size_t)s.image_index;
+    const float* in = intrinsics + 13 * (size_t)s.camera_index;
+    DeviceView v;
+    const double x = q[0], y = q[1], z = q[2], w = q[3];
+    const double tx = 2.0 * x, ty = 2.0 * y, tz = 2.0 * z;
+    const double twx = tx * w, twy = ty * w, twz = tz * w;
+    const double txx = tx * x, txy = ty * x, txz = tz * x;
+    const double tyy = ty * y, tyz = tz * y, tzz = tz * z;
+    v.r[0] = (float)(1.0 - (tyy + tzz));
+    v.r[1] = (float)(txy - twz);
+    v.r[2] = (float)(txz + twy);
+    v.r[3] = (float)(txy + twz);
+    v.r[4] = (float)(1.0 - (txx + tzz));
+    v.r[5] = (float)(tyz - twx);
+    v.r[6] = (float)(txz - twy);
+    v.r[7] = (float)(tyz + twx);
+    v.r[8] = (float)(1.0 - (txx + tyy));
+    v.t[0] = (float)q[4];
+    v.t[1] = (float)q[5];
+    v.t[2] = (float)q[6];
+    v.fx   = in[0];
+    v.fy   = in[1];
+    v.cx   = in[2];
+    v.cy   = in[3];
+    v.s    = in[4];
+    distorted = false;
+    for (int j = 5; j < 13; ++j) distorted |= (in[j] != 0.f);
+    for (int j = 0; j < 5; ++j) v.crop[j] = s.crop[j];
+    for (int j = 0; j < 4; ++j) v.rot[j] = s.rot[j];
+    v.ccx = (float)(s.w / 2);
+    v.ccy = (float)(s.h / 2);
+    for (int j = 0; j < 4; ++j) v.pad[j] = 0.f;
+    return v;
+}
+
+// One thread per view fills its camera constants; non-zero distortion coefficients raise flag bit 0.
 // Workgroups beyond the first zero the per-bin counters of all views (n4 uint4 elements).
 __global__ void __launch_bounds__(kBlock) prepare_views_kernel(PrepareViewsArgs args, int first_view, int num_views,
                                                                 const double* __restrict__ poses_se3,
@@ -83,40 +122,9 @@ __global__ void __launch_bounds__(kBlock) prepare_views_kernel(PrepareViewsArgs 
         __syncthreads();
     }
     if (k >= num_views) return;
-    const ViewSource& s = args.src[k];
-    const double* q     = poses_se3 + 8 * (size_t)s.image_index;
-    const float* in     = intrinsics + 13 * (size_t)s.camera_index;
-    DeviceView v;
-    const double x = q[0], y = q[1], z = q[2], w = q[3];
-    const double tx = 2.0 * x, ty = 2.0 * y, tz = 2.0 * z;
-    const double twx = tx * w, twy = ty * w, twz = tz * w;
-    const double txx = tx * x, txy = ty * x, txz = tz * x;
-    const double tyy = ty * y, tyz = tz * y, tzz = tz * z;
-    v.r[0] = (float)(1.0 - (tyy + tzz));
-    v.r[1] = (float)(txy - twz);
-    v.r[2] = (float)(txz + twy);
-    v.r[3] = (float)(txy + twz);
-    v.r[4] = (float)(1.0 - (txx + tzz));
-    v.r[5] = (float)(tyz - twx);
-    v.r[6] = (float)(txz - twy);
-    v.r[7] = (float)(tyz + twx);
-    v.r[8] = (float)(1.0 - (txx + tyy));
-    v.t[0] = (float)q[4];
-    v.t[1] = (float)q[5];
-    v.t[2] = (float)q[6];
-    v.fx   = in[0];
-    v.fy   = in[1];
-    v.cx   = in[2];
-    v.cy   = in[3];
-    v.s    = in[4];
     bool distorted = false;
-    for (int j = 5; j < 13; ++j) distorted |= (in[j] != 0.f);
+    const DeviceView v = make_device_view(args.src[k], poses_se3, intrinsics, distorted);
     if (distorted) atomicOr(flags, 1u);
-    for (int j = 0; j < 5; ++j) v.crop[j] = s.crop[j];
-    for (int j = 0; j < 4; ++j) v.rot[j] = s.rot[j];
-    v.ccx = (float)(s.w / 2);
-    v.ccy = (float)(s.h / 2);
-    for (int j = 0; j < 4; ++j) v.pad[j] = 0.f;
     views[first_view + k] = v;
 }
 

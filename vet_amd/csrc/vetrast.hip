@@ -14,6 +14,7 @@
 #include "sort_kernels.h"
 #include "build_kernels.h"
 #include "backward_kernels.h"
+#include "lift_kernels.h"
 
 using namespace vetrast;
 
@@ -767,6 +768,78 @@ int vetrast_adam_step(vetrast_ctx* ctx, const vetrast_adam_args* a, void* stream
     return VETRAST_OK;
 }
 
+size_t vetrast_lift_workspace_bytes(int64_t num_cells)
+{
+    if (num_cells < 0) return 0;
+    // header (camera constants, queue length, flag word), queue entries, one double per queue slot, chunk prefix sums
+    return kLiftHeader + align_up((size_t)num_cells * sizeof(uint2), kAlign) +
+           align_up((size_t)num_cells * sizeof(double), kAlign) +
+           align_up(((size_t)num_cells + 1) * sizeof(unsigned long long), kAlign);
+}
+
+int vetrast_lift_error(vetrast_ctx* ctx, const vetrast_lift_args* a, void* stream_)
+{
+    if (!ctx || !a) return VETRAST_ERR_INVALID_ARG;
+    if (a->num_cells < 0 || a->num_cells > (int64_t)1 << 30) return VETRAST_ERR_INVALID_ARG;
+    if (a->channels < 1 || a->height < 1 || a->width < 1 || a->border_pixels < 0) return VETRAST_ERR_INVALID_ARG;
+    // pixel numbers inside a cell's box go through float arithmetic that is exact below 2^24
+    if ((int64_t)a->height * a->width >= (int64_t)1 << 24) return VETRAST_ERR_INVALID_ARG;
+    const vetrast_view& v = a->view;
+    if (v.camera_model_type != VETRAST_CAMERA_PINHOLE_DISTORTION) return VETRAST_ERR_UNSUPPORTED;
+    if (v.image_index < 0 || v.image_index >= a->num_poses) return VETRAST_ERR_INVALID_ARG;
+    if (v.camera_index < 0 || v.camera_index >= a->num_cameras) return VETRAST_ERR_INVALID_ARG;
+    if (a->num_cells == 0) return VETRAST_OK;
+    if (!a->cell_bb_min || !a->cell_bb_length || !a->cell_value || !a->cell_access_count || !a->poses_se3 ||
+        !a->intrinsics || !a->loss_image || !a->workspace)
+        return VETRAST_ERR_INVALID_ARG;
+    if (reinterpret_cast<uintptr_t>(a->workspace) % kAlign) return VETRAST_ERR_INVALID_ARG;
+    if (a->workspace_bytes < vetrast_lift_workspace_bytes(a->num_cells)) return VETRAST_ERR_WORKSPACE_SMALL;
+
+    hipStream_t stream = (hipStream_t)stream_;
+    char* ws           = static_cast<char*>(a->workspace);
+    LiftPass lp;
+    lp.bb_min       = a->cell_bb_min;
+    lp.bb_length    = a->cell_bb_length;
+    lp.value        = a->cell_value;
+    lp.access_count = a->cell_access_count;
+    lp.loss         = a->loss_image;
+    lp.num_cells    = a->num_cells;
+    lp.channels     = a->channels;
+    lp.height       = a->height;
+    lp.width        = a->width;
+    lp.border       = a->border_pixels;
+    lp.view         = reinterpret_cast<const DeviceView*>(ws);
+    lp.queue_length = reinterpret_cast<uint32_t*>(ws + sizeof(DeviceView));
+    lp.queue        = reinterpret_cast<uint2*>(ws + kLiftHeader);
+    lp.sums = reinterpret_cast<double*>(ws + kLiftHeader + align_up((size_t)a->num_cells * sizeof(uint2), kAlign));
+    lp.starts = reinterpret_cast<unsigned long long*>(reinterpret_cast<char*>(lp.sums) +
+                                                      align_up((size_t)a->num_cells * sizeof(double), kAlign));
+    uint32_t* flags = reinterpret_cast<uint32_t*>(ws + VETRAST_LIFT_FLAGS_OFFSET);
+
+    ViewSource src;
+    src.image_index  = v.image_index;
+    src.camera_index = v.camera_index;
+    src.w            = v.w;
+    src.h            = v.h;
+    for (int j = 0; j < 5; ++j) src.crop[j] = v.crop_transform[j];
+    for (int j = 0; j < 4; ++j) src.rot[j] = v.crop_rotation[j];
+
+    ScopeTimer tm(ctx, stream, VETRAST_SCOPE_LIFT_ERROR);
+    hipLaunchKernelGGL(lift_prepare_kernel, dim3(1), dim3(kWave), 0, stream, src, a->poses_se3, a->intrinsics,
+                       reinterpret_cast<DeviceView*>(ws), lp.queue_length, flags);
+    const int waves_per_block = kBlock / kWave;
+    hipLaunchKernelGGL(lift_cells_kernel, dim3((unsigned)((a->num_cells + waves_per_block - 1) / waves_per_block)),
+                       dim3(kBlock), 0, stream, lp);
+    // The queue length stays on the device, so the shared pass is launched at a fixed width and splits the chunks
+    // it finds evenly.
+    hipLaunchKernelGGL(lift_scan_kernel, dim3(1), dim3(kLiftScanBlock), 0, stream, lp);
+    hipLaunchKernelGGL(lift_queued_kernel, dim3(2048), dim3(kBlock), 0, stream, lp);
+    hipLaunchKernelGGL(lift_finish_kernel, dim3((unsigned)std::min<int64_t>(grid_for((size_t)a->num_cells), 256)),
+                       dim3(kBlock), 0, stream, lp);
+    VET_HIP(ctx, hipGetLastError());
+    return VETRAST_OK;
+}
+
 int vetrast_query_device_flags(vetrast_ctx* ctx, const void* workspace, const vetrast_workspace_layout* layout,
                                void* stream)
 {
@@ -839,6 +912,7 @@ const char* vetrast_scope_name(int32_t scope)
         case VETRAST_SCOPE_BACKWARD_BLEND: return "BlendBackwards";
         case VETRAST_SCOPE_BACKWARD_GATHER: return "BlendBackwards (per-point sum)";
         case VETRAST_SCOPE_BACKWARD_POST: return "Post Process Gradient";
+        case VETRAST_SCOPE_LIFT_ERROR: return "FillSceneGridWithLoss";
         default: return "?";
     }
 }

@@ -67,6 +67,18 @@ def fill_forward_args(args: abi.ForwardArgs, scene: Scene, params: abi.Params, v
     args.params = params
 
 
+def fill_lift_args(a, view, poses_se3, intrinsics, loss_image, border_pixels):
+    """Scalar part of vetrast_lift_args shared by host and device callers; `view` is a synthetic.View."""
+    a.num_poses, a.num_cameras = int(poses_se3.shape[0]), int(intrinsics.shape[0])
+    a.view.w, a.view.h = view.w, view.h
+    a.view.image_index, a.view.camera_index = view.image_index, view.camera_index
+    a.view.camera_model_type = view.camera_model_type
+    a.view.crop_transform = (C.c_float * 5)(*view.crop_transform)
+    a.view.crop_rotation = (C.c_float * 4)(*view.crop_rotation)
+    a.channels, a.height, a.width = (int(d) for d in loss_image.shape)
+    a.border_pixels = border_pixels
+
+
 @dataclass
 class ForwardResult:
     out: List[torch.Tensor]
@@ -285,6 +297,35 @@ class Rasterizer:
         a.n, a.step = param.numel(), step
         a.lr, a.beta1, a.beta2, a.eps, a.weight_decay, a.zero_grad = lr, beta1, beta2, eps, weight_decay, int(zero_grad)
         abi.check(self.lib.vetrast_adam_step(self.ctx, C.byref(a), self._stream()), "adam_step")
+
+    def lift_error(self, cell_bb_min, cell_bb_length, cell_value, cell_access_count, view, poses_se3, intrinsics,
+                   loss_image, border_pixels=abi.LIFT_BORDER_PIXELS, workspace=None):
+        """Adds the error image of one view to the grid cells its pixels fall in, in place on cell_value (float32 [n]
+        or [n,1]) and cell_access_count (int32) (vetrast_lift_error; the reference's FillSceneGridWithLoss). All
+        arguments but `view` (a synthetic.View) are contiguous CUDA tensors. Returns the workspace, whose flag word
+        `lift_flags` reads."""
+        a = abi.LiftArgs()
+        for name, t, dt in (("cell_bb_min", cell_bb_min, torch.float32), ("cell_bb_length", cell_bb_length, torch.float32),
+                            ("cell_value", cell_value, torch.float32), ("cell_access_count", cell_access_count, torch.int32),
+                            ("poses_se3", poses_se3, torch.float64), ("intrinsics", intrinsics, torch.float32),
+                            ("loss_image", loss_image, torch.float32)):
+            assert t.is_cuda and t.dtype == dt and t.is_contiguous(), name
+            setattr(a, name, t.data_ptr())
+        a.num_cells = cell_value.numel()
+        assert cell_bb_min.numel() == 3 * a.num_cells and cell_bb_length.numel() == 3 * a.num_cells
+        assert cell_access_count.numel() == a.num_cells and loss_image.dim() == 3
+        fill_lift_args(a, view, poses_se3, intrinsics, loss_image, border_pixels)
+        need = int(self.lib.vetrast_lift_workspace_bytes(a.num_cells))
+        if workspace is None:
+            workspace = torch.empty(max(need, 256), dtype=torch.uint8, device=loss_image.device)
+        a.workspace, a.workspace_bytes = workspace.data_ptr(), workspace.numel()
+        abi.check(self.lib.vetrast_lift_error(self.ctx, C.byref(a), self._stream()), "lift_error")
+        return workspace
+
+    @staticmethod
+    def lift_flags(workspace):
+        """Blocking: the flag word of a lift_error workspace (1: the camera row had non-zero distortion)."""
+        return int(workspace[abi.LIFT_FLAGS_OFFSET:abi.LIFT_FLAGS_OFFSET + 4].view(torch.int32).item())
 
     def check_device_flags(self, fwd: ForwardResult):
         return self.lib.vetrast_query_device_flags(self.ctx, C.c_void_p(fwd.workspace.data_ptr()),

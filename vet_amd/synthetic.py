@@ -317,3 +317,32 @@ def tiny_scene(num_points=300, w=24, h=16, num_layers=3, K=4, seed=7, channels=4
     views = [ViewSpec(w, h, image_index=b) for b in range(num_views)]
     return Scene("tiny", pos, tex, conf, bg, poses, _intrinsics(0.45 * w, 0.45 * w, w / 2.0, h / 2.0, 0.0), views,
                  num_layers=num_layers, max_list_length=K, seed=seed)
+
+
+def cell_grid(xyz, cell_size):
+    """Uniform grid of cells over the bounding box of the points, built the way VET does for point adding
+    (UpdateCellStructureForPointOptim, src/lib/rendering/NeuralPointCloudCuda.cpp:95-147): the box grows by 0.01 on
+    every side, ceil(extent / cell_size) slices per axis, cells numbered x fastest, then y, then z.
+    Returns (bb_min [n,3] f32, bb_length [n,3] f32)."""
+    lo = xyz.min(axis=0).astype(np.float32) - np.float32(0.01)
+    hi = xyz.max(axis=0).astype(np.float32) + np.float32(0.01)
+    size = np.float32(cell_size)
+    slices = np.ceil((hi - lo) / size).astype(np.int64)
+    zz, yy, xx = np.meshgrid(np.arange(slices[2]), np.arange(slices[1]), np.arange(slices[0]), indexing="ij")
+    steps = np.stack([xx.ravel(), yy.ravel(), zz.ravel()], axis=1).astype(np.float32)
+    bb_min = (lo[None, :] + steps * size).astype(np.float32)
+    bb_length = np.full_like(bb_min, size)
+    return np.ascontiguousarray(bb_min), np.ascontiguousarray(bb_length)
+
+
+def error_image(seed, channels, h, w):
+    """A per-pixel error image [channels,h,w] of either sign (the lifting takes absolute values): smooth blobs plus
+    noise, like |target - output| of a half-trained scene with the sign kept."""
+    st = Stream(seed, "error_image")
+    y, x = np.mgrid[0:h, 0:w].astype(np.float32)
+    img = np.empty((channels, h, w), dtype=np.float32)
+    for c in range(channels):
+        fx, fy, ph = st.uniform(3)
+        blob = np.sin(x * np.float32(0.01 + 0.03 * fx) + np.float32(6.0 * ph)) * np.cos(y * np.float32(0.01 + 0.03 * fy))
+        img[c] = (0.2 * blob + 0.05 * st.normal(h * w).reshape(h, w)).astype(np.float32)
+    return np.ascontiguousarray(img)
