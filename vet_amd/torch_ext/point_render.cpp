@@ -119,6 +119,49 @@ PointRendererCache::~PointRendererCache()
     vetrast_destroy(ctx);
 }
 
+void PointRendererCache::FillSceneGridWithLoss(int batch, const CellTensors& cells,
+                                               const std::vector<ReducedImageInfo>& images, torch::Tensor poses_se3,
+                                               torch::Tensor intrinsics, torch::Tensor loss_img)
+{
+    TORCH_CHECK(batch >= 0 && batch < (int)images.size(), "FillSceneGridWithLoss: batch index out of range");
+    auto is_dev = [](const torch::Tensor& t, torch::ScalarType ty) {
+        return t.defined() && t.is_cuda() && t.scalar_type() == ty && t.is_contiguous();
+    };
+    TORCH_CHECK(is_dev(cells.t_cell_bb_min, torch::kFloat32) && is_dev(cells.t_cell_bb_length, torch::kFloat32) &&
+                    is_dev(cells.t_cell_value, torch::kFloat32) && is_dev(cells.t_cell_access_count, torch::kInt32),
+                "FillSceneGridWithLoss: cell tensors must be contiguous CUDA tensors (float32, float32, float32, int32)");
+    TORCH_CHECK(is_dev(poses_se3, torch::kFloat64) && is_dev(intrinsics, torch::kFloat32) && is_dev(loss_img, torch::kFloat32),
+                "FillSceneGridWithLoss: poses_se3 (float64), intrinsics and loss_img (float32) must be contiguous CUDA tensors");
+    TORCH_CHECK(loss_img.dim() == 3, "FillSceneGridWithLoss: loss_img is [C,h,w]");
+    const int64_t n = cells.t_cell_value.numel();
+    TORCH_CHECK(cells.t_cell_bb_min.numel() == 3 * n && cells.t_cell_bb_length.numel() == 3 * n &&
+                    cells.t_cell_access_count.numel() == n,
+                "FillSceneGridWithLoss: cell tensors disagree in size");
+    vetrast_lift_args a;
+    std::memset(&a, 0, sizeof(a));
+    a.num_cells         = n;
+    a.cell_bb_min       = cells.t_cell_bb_min.data_ptr<float>();
+    a.cell_bb_length    = cells.t_cell_bb_length.data_ptr<float>();
+    a.cell_value        = cells.t_cell_value.data_ptr<float>();
+    a.cell_access_count = cells.t_cell_access_count.data_ptr<int32_t>();
+    a.num_poses         = (int32_t)poses_se3.size(0);
+    a.num_cameras       = (int32_t)intrinsics.size(0);
+    a.poses_se3         = poses_se3.data_ptr<double>();
+    a.intrinsics        = intrinsics.data_ptr<float>();
+    a.view              = images[batch];
+    a.loss_image        = loss_img.data_ptr<float>();
+    a.channels          = (int32_t)loss_img.size(0);
+    a.height            = (int32_t)loss_img.size(1);
+    a.width             = (int32_t)loss_img.size(2);
+    a.border_pixels     = VETRAST_LIFT_BORDER_PIXELS;
+    const int64_t need  = (int64_t)vetrast_lift_workspace_bytes(n);
+    if (!lift_workspace.defined() || lift_workspace.numel() < need || lift_workspace.device() != loss_img.device())
+        lift_workspace = torch::empty({std::max<int64_t>(need, 256)}, torch::dtype(torch::kUInt8).device(loss_img.device()));
+    a.workspace       = lift_workspace.data_ptr();
+    a.workspace_bytes = (size_t)lift_workspace.numel();
+    check_status(vetrast_lift_error(ctx, &a, c10::hip::getCurrentHIPStream().stream()), "lift_error");
+}
+
 std::vector<torch::Tensor> BlendPointCloud(NeuralRenderInfo* info)
 {
     TORCH_CHECK(info && info->scene && info->cache, "BlendPointCloud: scene and cache must be set");
@@ -433,6 +476,30 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
              pybind11::arg("eps") = 1e-8, pybind11::arg("weight_decay") = 0.0)
         .def("step", &vet_amd::MyAdam::step, pybind11::arg("zero_grad") = false)
         .def("zero_grad", &vet_amd::MyAdam::zero_grad);
+    m.def(
+        "fill_scene_grid_with_loss",
+        [](int batch, torch::Tensor bb_min, torch::Tensor bb_length, torch::Tensor value, torch::Tensor access_count,
+           std::vector<std::vector<double>> views, torch::Tensor poses_se3, torch::Tensor intrinsics,
+           torch::Tensor loss_img) {
+            if (!g_cache) g_cache = std::make_shared<vet_amd::PointRendererCache>();
+            std::vector<vet_amd::ReducedImageInfo> images;
+            for (auto& v : views)
+            {
+                TORCH_CHECK(v.size() == 14, "a view is w,h,image_index,camera_index,camera_model_type,crop[5],rot[4]");
+                vet_amd::ReducedImageInfo r;
+                r.w                 = (int)v[0];
+                r.h                 = (int)v[1];
+                r.image_index       = (int)v[2];
+                r.camera_index      = (int)v[3];
+                r.camera_model_type = (int)v[4];
+                for (int j = 0; j < 5; ++j) r.crop_transform[j] = (float)v[5 + j];
+                for (int j = 0; j < 4; ++j) r.crop_rotation[j] = (float)v[10 + j];
+                images.push_back(r);
+            }
+            g_cache->FillSceneGridWithLoss(batch, {bb_min, bb_length, value, access_count}, images, poses_se3,
+                                           intrinsics, loss_img);
+        },
+        "PointRendererCache::FillSceneGridWithLoss of the reference, with the cell tensors passed one by one");
     m.def("blend_point_cloud", &blend_point_cloud,
           "BlendPointCloud(NeuralRenderInfo*) of the reference, with the scene passed as tensors");
 }

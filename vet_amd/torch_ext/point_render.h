@@ -63,6 +63,15 @@ struct SceneTensors
     torch::Tensor t_index;                    // scene->point_cloud_cuda->t_index           [N,1] i32, may be undefined
 };
 
+// The cell tensors of the point cloud (src/lib/rendering/NeuralPointCloudCuda.h:100-106).
+struct CellTensors
+{
+    torch::Tensor t_cell_bb_min;        // [n,3] f32
+    torch::Tensor t_cell_bb_length;     // [n,3] f32
+    torch::Tensor t_cell_value;         // [n,1] f32
+    torch::Tensor t_cell_access_count;  // [n,1] i32
+};
+
 // Owns the vetrast context and the workspace that is re-used between no-grad calls
 // (counterpart of PointRendererCache, src/lib/rendering/PointRenderer.h:112-248).
 class PointRendererCache
@@ -74,6 +83,15 @@ class PointRendererCache
     PointRendererCache& operator=(const PointRendererCache&) = delete;
     vetrast_ctx* ctx = nullptr;
     torch::Tensor eval_workspace;
+
+    // Adds the error image of view `batch` to the cells its pixels fall in
+    // (PointRendererCache::FillSceneGridWithLoss(int batch, NeuralPointCloudCuda point_cloud, std::vector<ReducedImageInfo>
+    // images, torch::Tensor loss_img), src/lib/rendering/PointRenderer.h:175, src/lib/rendering/RenderForward.cu:763-791).
+    // The point cloud object is replaced by its four cell tensors and the pose / intrinsics tables the reference reads
+    // from device constants are passed along. cells.value and cells.access_count are updated in place.
+    void FillSceneGridWithLoss(int batch, const CellTensors& cells, const std::vector<ReducedImageInfo>& images,
+                               torch::Tensor poses_se3, torch::Tensor intrinsics, torch::Tensor loss_img);
+    torch::Tensor lift_workspace;
 };
 
 class NeuralRenderInfo : public torch::CustomClassHolder

@@ -37,3 +37,11 @@ def MyAdam(groups, beta1=0.9, beta2=0.999, eps=1e-8, weight_decay=0.0):
     """The reference's texture optimiser (torch::optim::MyAdam, src/lib/models/my_adam.cpp) with one fused kernel per
     tensor and step. groups: list of (list of float32 CUDA parameter tensors, learning rate)."""
     return load().MyAdam([(list(ts), float(lr)) for ts, lr in groups], beta1, beta2, eps, weight_decay)
+
+
+def fill_scene_grid_with_loss(batch, cell_bb_min, cell_bb_length, cell_value, cell_access_count, views, poses_se3,
+                              intrinsics, loss_img):
+    """PointRendererCache::FillSceneGridWithLoss of the reference (src/lib/rendering/RenderForward.cu:763-791): adds
+    the error image [C,h,w] of view `batch` to cell_value / cell_access_count in place. views as in blend_point_cloud."""
+    load().fill_scene_grid_with_loss(int(batch), cell_bb_min, cell_bb_length, cell_value, cell_access_count,
+                                     [list(map(float, v)) for v in views], poses_se3, intrinsics, loss_img)
