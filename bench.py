@@ -247,6 +247,8 @@ def main():
                     help="1 = FULL_BLEND (the headline workload), 3 = BILINEAR_BLEND (four fragments per point and layer)")
     ap.add_argument("--no-second-order", action="store_true", help="skip timing the other point order")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--lift-only", action="store_true",
+                    help="time only the error lifting on the configuration's scene and print its object")
     ap.add_argument("--cpu-threads", type=int, default=0, help="0 = min(16, available cores)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -268,6 +270,10 @@ def main():
     make = {2: synthetic.config2, 3: synthetic.config3, 5: synthetic.config5}[args.config]
     backward = args.config != 2
     scene = make(**kw)
+    if args.lift_only:
+        threads = 0 if args.no_cpu_baseline else (args.cpu_threads or min(16, len(os.sched_getaffinity(0))))
+        print(json.dumps({"lift_error": time_lift_error(scene, args.steps, threads)}))
+        return
     r = run_scene(scene, backward, args.steps, args.warmup, render_mode=args.render_mode)
     N, P, F, Fk, Cn, L, K = r["N"], r["P"], r["F"], r["Fk"], r["Cn"], r["L"], r["K"]
     ms_step, ms_fwd = r["ms_step"], r["ms_fwd"]
