@@ -86,8 +86,10 @@ typedef struct vetrast_params
     int32_t render_mode;                      /* RenderParams::render_mode, src/lib/data/Settings.h: 0 or 1 = FULL_BLEND
                                                  (a point lands in the pixel it rounds to), 3 = BILINEAR_BLEND (a point
                                                  lands in the 2x2 pixels around it, alpha = bilinear weight x confidence,
-                                                 blending stops once the transmittance falls below 0.001). Other values
-                                                 are refused. */
+                                                 blending stops once the transmittance falls below 0.001), 2 =
+                                                 FUZZY_BLEND (FULL_BLEND lists; the nearest fragments of a pixel that
+                                                 lie within depth_accept_blend of the first one are averaged before
+                                                 they are blended). Other values are refused. */
     /* The steps VET runs on the optimised tensors right before the rasterizer, fused into it
      * (NeuralPointTextureImpl::PrepareConfidence / PrepareTexture, src/lib/models/NeuralTexture.h:38-55; called from
      * src/lib/models/Pipeline.cpp:113-124). With them on, `confidence`, `texture` and `background` are the RAW tensors
@@ -95,9 +97,12 @@ typedef struct vetrast_params
     int32_t confidence_activation;            /* 0: confidence is used as given; 1: sigmoid(confidence_scale * confidence) */
     float confidence_scale;                   /* 10 + sigmoid_narrowing_factor * epoch in VET */
     int32_t texture_abs;                      /* 1: |texture| and |background| (PipelineParams::non_subzero_texture) */
+    float depth_accept_blend;                 /* FUZZY_BLEND: depth range of a bucket, RenderParams::depth_accept_blend
+                                                 (src/lib/data/Settings.h:42, default 0.01) */
 } vetrast_params;
 
 #define VETRAST_RENDER_FULL_BLEND 1
+#define VETRAST_RENDER_FUZZY_BLEND 2
 #define VETRAST_RENDER_BILINEAR_BLEND 3
 
 typedef struct vetrast_ctx vetrast_ctx;

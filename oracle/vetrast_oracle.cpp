@@ -264,6 +264,11 @@ inline float sign_of(float x)
     return x > 0.f ? 1.f : (x < 0.f ? -1.f : 0.f);  // torch's abs backward: grad * sign(x)
 }
 
+inline bool is_fuzzy(const vetrast_params& p)
+{
+    return p.render_mode == VETRAST_RENDER_FUZZY_BLEND;
+}
+
 inline bool is_bilinear(const vetrast_params& p)
 {
     return p.render_mode == VETRAST_RENDER_BILINEAR_BLEND;
@@ -288,7 +293,8 @@ int validate(const vetrast_forward_args* a)
     if (p.num_layers < 1 || p.num_layers > VETRAST_MAX_LAYERS) return VETRAST_ERR_INVALID_ARG;
     if (p.num_texture_channels < 1 || p.num_texture_channels > VETRAST_MAX_CHANNELS) return VETRAST_ERR_INVALID_ARG;
     if (p.check_normal) return VETRAST_ERR_UNSUPPORTED;
-    if (p.render_mode != 0 && p.render_mode != VETRAST_RENDER_FULL_BLEND && !is_bilinear(p)) return VETRAST_ERR_UNSUPPORTED;
+    if (p.render_mode != 0 && p.render_mode != VETRAST_RENDER_FULL_BLEND && !is_bilinear(p) && !is_fuzzy(p))
+        return VETRAST_ERR_UNSUPPORTED;
     if (is_bilinear(p) && a->num_points > (1 << 30)) return VETRAST_ERR_INVALID_ARG;  // id and corner share 32 key bits
     for (int b = 0; b < a->num_views; ++b)
     {
@@ -541,6 +547,106 @@ void bilinear_pixel_backward(const vetrast_backward_args* g, const Scene& s, int
     }
 }
 
+// Value gradients of one pixel in FUZZY_BLEND: the first half of BlendBackwardsFuzzy<C>,
+// rendering/RenderBackward.cu:570-727, literally. Unlike the forward kernel this one starts every new bucket at the
+// depth of its first fragment (:712), so buckets form all along the list, the background (depth MAX_DEPTH_CONST = 1e5)
+// closes the last one and is a bucket of its own. A bucket's gradient is shared out evenly among its elements; every
+// element in front of a bucket receives the bucket's whole transmittance term divided by (1 - mean confidence of the
+// element's own bucket) (:654-672, the mean confidences are the values the kernel parks in gradient_sum_backwards).
+// The position part of that kernel (:729-1080) computes the same heuristic as BlendBackwards2, so the caller shares it.
+void fuzzy_pixel_value_gradients(const vetrast_backward_args* g, int N, int C, const float* G, size_t plane,
+                                 size_t pixel, uint32_t offset, int size_of_chunk, const uint64_t* frag, bool par)
+{
+    const vetrast_forward_args* a = &g->fwd;
+    const vetrast_params& pr      = a->params;
+    const float MAX_DEPTH_CONST   = 100000.f;  // rendering/RenderConstants.h:30
+    auto texture_index_at         = [&](int pos) {
+        const int id = (int)(uint32_t)frag[pos];
+        return a->index ? a->index[id] : id;
+    };
+    auto depth_at = [&](int pos) {
+        const uint32_t bits = (uint32_t)(frag[pos] >> 32);
+        float d;
+        std::memcpy(&d, &bits, 4);
+        return d;
+    };
+    std::vector<float> saved_confidence((size_t)size_of_chunk + 1, 0.f);  // gradient_sum_backwards row C of this pixel
+    float accumulation_last_min_d = 0.f;
+    float accumulation_desc[VETRAST_MAX_CHANNELS];
+    float accumulation_conf_val = 0.f;
+    int accumulation_num_elems  = 0;
+    int accum_start_index       = 0;
+    float alpha_dest            = 1.f;
+    for (int ci = 0; ci < C; ++ci) accumulation_desc[ci] = 0.f;
+
+    auto accumulateCollectedBackwards = [&]() {
+        const float inv_weight     = 1.f / float(accumulation_num_elems);
+        const float confidence_val = accumulation_conf_val * inv_weight;
+        float colors[VETRAST_MAX_CHANNELS], grad_in[VETRAST_MAX_CHANNELS], g_colors[VETRAST_MAX_CHANNELS];
+        float g_alpha = 0;
+        for (int ci = 0; ci < C; ++ci)
+        {
+            colors[ci]   = accumulation_desc[ci] * inv_weight;
+            grad_in[ci]  = G[ci * plane + pixel];
+            g_colors[ci] = alpha_dest * confidence_val * grad_in[ci];
+            g_alpha += colors[ci] * grad_in[ci];
+        }
+        g_alpha *= alpha_dest;
+        for (int t = accum_start_index; t < accum_start_index + accumulation_num_elems; ++t)
+        {
+            const bool is_foreground = t != size_of_chunk;
+            const int texture_index  = is_foreground ? texture_index_at((int)offset + t) : 0;
+            for (int ci = 0; ci < C; ++ci)
+            {
+                float* target = is_foreground ? &g->grad_texture[(size_t)ci * N + texture_index] : &g->grad_background[ci];
+                atomic_add(target, g_colors[ci] * inv_weight, par);
+            }
+            if (is_foreground)
+            {
+                atomic_add(&g->grad_confidence[texture_index], g_alpha * inv_weight, par);
+                saved_confidence[(size_t)t] = confidence_val;
+            }
+        }
+        for (int j = 0; j < accum_start_index; ++j)
+        {
+            const int texture_index_iter    = texture_index_at((int)offset + j);
+            const float confidence_val_iter = saved_confidence[(size_t)j];
+            float g_iter                    = 0;
+            for (int ci = 0; ci < C; ++ci)
+            {
+                const float epsilon = 1e-9;
+                float g_alpha_iter =
+                    (grad_in[ci] * colors[ci] * alpha_dest * confidence_val / (1 - confidence_val_iter + epsilon));
+                g_iter -= g_alpha_iter;
+            }
+            atomic_add(&g->grad_confidence[texture_index_iter], g_iter, par);
+        }
+        alpha_dest = compute_new_alphadest(alpha_dest, confidence_val);
+    };
+
+    const int list_size = pr.use_environment_map ? size_of_chunk : size_of_chunk + 1;
+    for (int i = 0; i < list_size; ++i)
+    {
+        const bool is_foreground = i != size_of_chunk;
+        const float d            = is_foreground ? depth_at((int)offset + i) : MAX_DEPTH_CONST;
+        if (!(d - accumulation_last_min_d < pr.depth_accept_blend))
+        {
+            if (i != 0) accumulateCollectedBackwards();
+            accumulation_conf_val  = 0.f;
+            accumulation_num_elems = 0;
+            for (int ci = 0; ci < C; ++ci) accumulation_desc[ci] = 0.f;
+            accumulation_last_min_d = d;
+            accum_start_index       = i;
+        }
+        const int texture_index = is_foreground ? texture_index_at((int)offset + i) : 0;
+        accumulation_conf_val += is_foreground ? a->confidence[texture_index] : 1.f;
+        for (int ci = 0; ci < C; ++ci)
+            accumulation_desc[ci] += is_foreground ? a->texture[(size_t)ci * N + texture_index] : a->background[ci];
+        ++accumulation_num_elems;
+    }
+    if (accumulation_num_elems > 0) accumulateCollectedBackwards();
+}
+
 }  // namespace
 
 extern "C" int vetref_prepare_view(const double* pose8, const float* intrinsics13, float* out17)
@@ -604,6 +710,7 @@ extern "C" int vetref_forward(const vetrast_forward_args* a, uint32_t* offsets, 
     const vetrast_params& pr = a->params;
     const bool par           = num_threads > 1;
     const bool bilinear      = is_bilinear(pr);
+    const bool fuzzy         = is_fuzzy(pr);
 #ifdef _OPENMP
     omp_set_num_threads(num_threads > 0 ? num_threads : 1);
 #endif
@@ -697,7 +804,55 @@ extern "C" int vetref_forward(const vetrast_forward_args* a, uint32_t* offsets, 
                     float color_out[VETRAST_MAX_CHANNELS];
                     for (int ci = 0; ci < C; ++ci) color_out[ci] = 0.f;
                     int blended = 0;  // fragments that took part
-                    for (int i = 0; i < size_of_chunk; ++i)
+                    if (fuzzy)
+                    {
+                        // BlendMultiFuzzy, rendering/RenderForward.cu:1393-1503: fragments are collected while their
+                        // depth stays within depth_accept_blend of the first one of the bucket, the bucket is blended
+                        // as one fragment with the mean confidence and the mean descriptor. After the first bucket
+                        // the reference resets its reference depth to -100000 (:1468), not to the next depth, so
+                        // every later fragment closes the bucket before it: only the nearest bucket averages.
+                        float accumulation_last_min_d = 0.f;
+                        float accumulation_desc[VETRAST_MAX_CHANNELS];
+                        float accumulation_conf_val = 0.f;
+                        int accumulation_num_elems  = 0;
+                        for (int ci = 0; ci < C; ++ci) accumulation_desc[ci] = 0.f;
+                        auto accumulateCollected = [&]() {
+                            const float confidence_val = accumulation_conf_val / float(accumulation_num_elems);
+                            for (int ci = 0; ci < C; ++ci)
+                            {
+                                const float color = accumulation_desc[ci] / float(accumulation_num_elems);
+                                color_out[ci]     = compute_blend(alpha_dest, confidence_val, color, color_out[ci]);
+                            }
+                            alpha_dest = compute_new_alphadest(alpha_dest, confidence_val);
+                        };
+                        for (int i = 0; i < size_of_chunk; ++i)
+                        {
+                            const int point_id      = (int)(uint32_t)frag[o + i];
+                            const int texture_index = a->index ? a->index[point_id] : point_id;
+                            const uint32_t dbits    = (uint32_t)(frag[o + i] >> 32);
+                            float d;
+                            std::memcpy(&d, &dbits, 4);
+                            if (accumulation_last_min_d == 0.f) accumulation_last_min_d = d;
+                            if (!(d - accumulation_last_min_d < pr.depth_accept_blend))
+                            {
+                                accumulateCollected();
+                                accumulation_last_min_d = -100000.f;
+                                accumulation_conf_val   = 0.f;
+                                accumulation_num_elems  = 0;
+                                for (int ci = 0; ci < C; ++ci) accumulation_desc[ci] = 0.f;
+                            }
+                            // saved for inspection only (the fuzzy backward pass recomputes its own chain): the
+                            // transmittance in front of the bucket the fragment joins
+                            if (transmittance) transmittance[(size_t)b * s.cap + o + i] = alpha_dest;
+                            accumulation_conf_val += a->confidence[texture_index];
+                            for (int ci = 0; ci < C; ++ci)
+                                accumulation_desc[ci] += a->texture[(size_t)ci * N + texture_index];
+                            ++accumulation_num_elems;
+                            ++blended;
+                        }
+                        if (accumulation_num_elems > 0) accumulateCollected();
+                    }
+                    for (int i = 0; i < size_of_chunk && !fuzzy; ++i)
                     {
                         const uint32_t low      = (uint32_t)frag[o + i];
                         const int point_id      = bilinear ? (int)(low >> 2) : (int)low;
@@ -810,6 +965,7 @@ extern "C" int vetref_backward(const vetrast_backward_args* g, const uint32_t* o
     const bool need_point_gradients = pr.need_point_gradient && (g->grad_points || g->grad_pose || g->grad_intrinsics);
 
     const bool bilinear = is_bilinear(pr);
+    const bool fuzzy    = is_fuzzy(pr);
     // gradient_sum_backwards: one zeroed float per fragment, rendering/PointRenderer.cu:1186-1200
     std::vector<float> sum_back(bilinear ? (size_t)s.cap : 0, 0.f);
     for (int b = 0; b < a->num_views; ++b)
@@ -844,7 +1000,10 @@ extern "C" int vetref_backward(const vetrast_backward_args* g, const uint32_t* o
                         const int id = sample_point_id(pos);
                         return a->index ? a->index[id] : id;
                     };
+                    if (fuzzy)
+                        fuzzy_pixel_value_gradients(g, N, C, G, plane, (size_t)gy * lw + gx, offset, size_of_chunk, frag, par);
                     // ---- value gradients, RenderBackward.cu:1118-1181
+                    if (!fuzzy)
                     {
                         float alpha_dest = 1.f;
                         const int list_size = pr.use_environment_map ? size_of_chunk : size_of_chunk + 1;

@@ -30,7 +30,7 @@ def test_library_exports_every_declared_symbol():
 def test_struct_sizes_are_the_c_ones():
     # sizes the C compiler gives the structs of include/vetrast.h (LP64)
     assert C.sizeof(abi.View) == 5 * 4 + 9 * 4
-    assert C.sizeof(abi.Params) == 20 * 4
+    assert C.sizeof(abi.Params) == 21 * 4
     assert C.sizeof(abi.LiftArgs) == 8 + 4 * 8 + 2 * 4 + 2 * 8 + C.sizeof(abi.View) + 8 + 4 * 4 + 2 * 8 == 160
     assert abi.LiftArgs.loss_image.offset % 8 == 0
     assert C.sizeof(abi.ForwardArgs) % 8 == 0
@@ -100,7 +100,10 @@ def test_workspace_layout_is_aligned_and_disjoint():
     full = lay.total_bytes
     assert lib.vetrast_workspace_layout_for_mode(N, B, L, w, h, abi.RENDER_BILINEAR_BLEND, C.byref(lay)) == 0
     assert lay.hits_per_layer == 4 and lay.fragment_capacity == 4 * N * L and lay.total_bytes > 3 * full
-    assert lib.vetrast_workspace_layout_for_mode(N, B, L, w, h, 2, C.byref(lay)) == abi.ERR_UNSUPPORTED
+    # FUZZY_BLEND uses the FULL_BLEND lists; other mode numbers are refused
+    assert lib.vetrast_workspace_layout_for_mode(N, B, L, w, h, abi.RENDER_FUZZY_BLEND, C.byref(lay)) == 0
+    assert lay.hits_per_layer == 1 and lay.total_bytes == full
+    assert lib.vetrast_workspace_layout_for_mode(N, B, L, w, h, 4, C.byref(lay)) == abi.ERR_UNSUPPORTED
 
 
 def test_status_and_scope_names():

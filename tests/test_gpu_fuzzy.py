@@ -1,0 +1,134 @@
+"""GPU parity of FUZZY_BLEND (render_mode 2): the HIP path through the C ABI against the CPU oracle.
+
+Bars as for the other modes: lists, stored transmittances, weights and blended features bit-exact (same operation
+order), gradients within 1e-4 relative.
+"""
+import numpy as np
+import pytest
+import torch
+
+from tests.helpers import kept_mask, max_rel_err
+from vet_amd import abi, synthetic
+from vet_amd.rasterizer import DeviceScene, make_params
+
+pytestmark = pytest.mark.gpu
+MODE = dict(render_mode=abi.RENDER_FUZZY_BLEND)
+
+
+def _levels(scene, step=0.25, seed=5):
+    """Moves the points onto depth levels with a jitter below the default depth range, so that buckets form everywhere."""
+    rng = np.random.default_rng(seed)
+    level = np.round(scene.position[:, 2] / step)
+    scene.position[:, 2] = (level * step + rng.uniform(0.0, 0.008, len(level))).astype(np.float32)
+    return scene
+
+
+def _scenes():
+    yield "tiny_K4", synthetic.tiny_scene(), {}
+    yield "tiny_levels_K8", _levels(synthetic.tiny_scene(num_points=6000, K=8, seed=81)), {}
+    yield "tiny_levels_nocut_3ch", _levels(synthetic.tiny_scene(num_points=5000, K=-1, channels=3, seed=82)), {}
+    yield "tiny_long_lists_levels", _levels(synthetic.tiny_scene(num_points=40000, K=0, seed=83)), {}
+    yield "tiny_long_lists_K16", _levels(synthetic.tiny_scene(num_points=40000, K=16, seed=84)), {}
+    yield "tiny_2views_envmap", _levels(synthetic.tiny_scene(num_points=3000, K=8, num_views=2, seed=85)), \
+        {"use_environment_map": 1}
+    yield "wide_depth_range", synthetic.tiny_scene(num_points=5000, K=12, seed=86), {"depth_accept_blend": 0.3}
+    yield "odd_size_5_layers", _levels(synthetic.tiny_scene(num_points=9000, w=83, h=61, num_layers=5, K=6, seed=87)), {}
+    yield "config1", synthetic.config1(), {"depth_accept_blend": 0.05}
+    yield "config2_200k", synthetic.config2(num_points=200_000), {"depth_accept_blend": 0.05}
+
+
+SCENES = list(_scenes())
+
+
+def _check_forward(scene, overrides, rasterizer, oracle):
+    params = make_params(scene, **{**MODE, **overrides})
+    ref = oracle.forward(scene, params)
+    dev = DeviceScene(scene)
+    res = rasterizer.forward(dev, params, save_for_backward=True)
+    torch.cuda.synchronize()
+    assert rasterizer.check_device_flags(res) == 0
+    K = params.debug_max_list_length
+    for b in range(len(scene.views)):
+        off = res.offsets(b)
+        np.testing.assert_array_equal(off, ref.offsets[b].astype(np.int64))
+        total = int(off[-1])
+        keep = kept_mask(off, K)
+        np.testing.assert_array_equal(res.fragments(b)[keep], ref.fragments[b, :total][keep])
+        np.testing.assert_array_equal(res.transmittance(b)[keep], ref.transmittance[b, :total][keep])
+        np.testing.assert_array_equal(res.weight(b), ref.weight[b])
+    for l in range(scene.num_layers):
+        np.testing.assert_array_equal(res.out[l].cpu().numpy(), ref.out[l])
+    return params, ref, dev, res
+
+
+@pytest.mark.parametrize("name,scene,overrides", SCENES, ids=[s[0] for s in SCENES])
+def test_forward_matches_oracle(name, scene, overrides, rasterizer, oracle):
+    print(f"[case] fuzzy forward {name} N={scene.num_points}", flush=True)
+    _check_forward(scene, overrides, rasterizer, oracle)
+
+
+@pytest.mark.parametrize("name,scene,overrides", SCENES, ids=[s[0] for s in SCENES])
+def test_backward_matches_oracle(name, scene, overrides, rasterizer, oracle):
+    print(f"[case] fuzzy backward {name} N={scene.num_points}", flush=True)
+    overrides = dict(overrides, need_point_gradient=1)
+    params, ref, dev, res = _check_forward(scene, overrides, rasterizer, oracle)
+    grad_out = scene.grad_out()
+    want = oracle.backward(ref, grad_out)
+    got = rasterizer.backward(res, [torch.from_numpy(g).cuda() for g in grad_out])
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(got["point_count"].cpu().numpy(), want["point_count"])
+    for key in ("texture", "confidence", "background", "points"):
+        err = max_rel_err(got[key].cpu().numpy(), want[key])
+        print(f"  {key}: max rel err {err:.3e}", flush=True)
+        assert err <= 1e-4, key
+
+
+def test_fuzzy_differs_from_full_blend_on_levels(rasterizer):
+    """The mode is not FULL_BLEND under another name: where several fragments share the nearest level the image
+    changes; with a vanishing depth range it is FULL_BLEND bit for bit."""
+    scene = _levels(synthetic.tiny_scene(num_points=6000, K=8, seed=88))
+    dev = DeviceScene(scene)
+    full = [o.clone() for o in rasterizer.forward(dev, make_params(scene)).out]
+    fuzzy = [o.clone() for o in rasterizer.forward(dev, make_params(scene, **MODE)).out]
+    same = [o.clone() for o in rasterizer.forward(dev, make_params(scene, depth_accept_blend=1e-12, **MODE)).out]
+    torch.cuda.synchronize()
+    assert max(float((a - b).abs().max()) for a, b in zip(full, fuzzy)) > 1e-3
+    for a, b in zip(full, same):
+        assert torch.equal(a, b)
+
+
+def test_leak_switch_has_no_effect_and_index_indirection(rasterizer, oracle):
+    """The background never adds to confidence row 0 in this mode (guarded in the reference), whatever the switch
+    says; several points sharing a descriptor row add up."""
+    scene = _levels(synthetic.tiny_scene(num_points=4000, K=8, seed=89))
+    rng = np.random.default_rng(1)
+    scene.index = rng.integers(0, 500, size=scene.num_points).astype(np.int32)
+    params, ref, dev, res = _check_forward(scene, {"quirk_background_confidence_leak": 1}, rasterizer, oracle)
+    grad_out = scene.grad_out()
+    want = oracle.backward(ref, grad_out, want_points=False)
+    got = rasterizer.backward(res, [torch.from_numpy(g).cuda() for g in grad_out], want_points=False)
+    torch.cuda.synchronize()
+    for key in ("texture", "confidence", "background"):
+        assert max_rel_err(got[key].cpu().numpy(), want[key]) <= 1e-4, key
+    params0 = make_params(scene, **MODE)
+    ref0 = oracle.forward(scene, params0)
+    want0 = oracle.backward(ref0, grad_out, want_points=False)
+    np.testing.assert_array_equal(want0["confidence"], want["confidence"])
+
+
+def test_config3_full_size(rasterizer, oracle):
+    print("[case] fuzzy config 3, 2M points, 1080p, forward+backward", flush=True)
+    scene = synthetic.config3()
+    over = {"need_point_gradient": 1, "depth_accept_blend": 0.05}
+    params, ref, dev, res = _check_forward(scene, over, rasterizer, oracle)
+    grad_out = scene.grad_out()
+    want = oracle.backward(ref, grad_out, num_threads=16)
+    got = rasterizer.backward(res, [torch.from_numpy(g).cuda() for g in grad_out])
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(got["point_count"].cpu().numpy(), want["point_count"])
+    for key in ("texture", "confidence", "points"):
+        err = max_rel_err(got[key].cpu().numpy(), want[key])
+        print(f"  {key}: max rel err {err:.3e}", flush=True)
+        assert err <= 1e-4, key
+    # the background gradient is one float32 sum over 2.75 M pixels on either side: compare loosely, as for FULL_BLEND
+    assert max_rel_err(got["background"].cpu().numpy(), want["background"]) <= 2e-3

@@ -20,6 +20,7 @@ CAMERA_OCAM = 1
 CAMERA_SPHERICAL = 2
 
 RENDER_FULL_BLEND = 1
+RENDER_FUZZY_BLEND = 2
 RENDER_BILINEAR_BLEND = 3
 
 SCOPE_NAMES = [
@@ -60,6 +61,7 @@ class Params(C.Structure):
         ("confidence_activation", C.c_int32),
         ("confidence_scale", C.c_float),
         ("texture_abs", C.c_int32),
+        ("depth_accept_blend", C.c_float),
     ]
 
 

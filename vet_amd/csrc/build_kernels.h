@@ -47,6 +47,7 @@ struct BuildPass
     int K;
     int use_environment_map;
     float mask_value;
+    float depth_accept;  // FUZZY_BLEND: depth range of a bucket
 };
 
 // Alpha of a fragment: the point's confidence, in BILINEAR_BLEND times the bilinear weight of the pixel's corner at the
@@ -75,9 +76,57 @@ __device__ __forceinline__ bool blend_is_saturated(float T)
     return BILINEAR && (double)T < 0.001;
 }
 
-template <int C, bool BILINEAR>
+// FUZZY_BLEND (BlendMultiFuzzy, src/lib/rendering/RenderForward.cu:1393-1503): fragments are collected while their depth
+// stays within depth_accept of the bucket's first one; a bucket is blended as ONE fragment with the mean confidence and
+// the mean descriptor of its elements. After the first bucket the reference sets its reference depth to -100000 (:1468)
+// instead of the next fragment's depth, so every later fragment closes the bucket in front of it: only the nearest
+// bucket ever holds more than one fragment, and a one-element bucket blends exactly like FULL_BLEND (x / 1.0f == x).
+template <int C>
+struct FuzzyBucket
+{
+    float last_min = 0.f, conf = 0.f;
+    float t[C];
+    int m = 0;
+    __device__ __forceinline__ FuzzyBucket()
+    {
+#pragma unroll
+        for (int ci = 0; ci < C; ++ci) t[ci] = 0.f;
+    }
+    // blends the collected elements into (T, color)
+    __device__ __forceinline__ void flush(float& T, float (&color)[C])
+    {
+        const float cf = conf / (float)m;
+        const float Tc = T * cf;
+#pragma unroll
+        for (int ci = 0; ci < C; ++ci) color[ci] = Tc * (t[ci] / (float)m) + color[ci];
+        T = (1.f - cf) * T;
+    }
+    // fragment at depth d with confidence cf and descriptor td joins; closes the bucket in front of it first if d is
+    // out of its range
+    __device__ __forceinline__ void add(float d, float cf, const float (&td)[4], float depth_accept, float& T,
+                                        float (&color)[C])
+    {
+        if (last_min == 0.f) last_min = d;
+        if (!(d - last_min < depth_accept))
+        {
+            flush(T, color);
+            last_min = -100000.f;
+            conf     = 0.f;
+            m        = 0;
+#pragma unroll
+            for (int ci = 0; ci < C; ++ci) t[ci] = 0.f;
+        }
+        conf += cf;
+#pragma unroll
+        for (int ci = 0; ci < C; ++ci) t[ci] += td[ci];
+        ++m;
+    }
+};
+
+template <int C, bool BILINEAR, bool FUZZY = false>
 __global__ void __launch_bounds__(kBlock) bin_build_kernel(BuildPass a)
 {
+    static_assert(!(BILINEAR && FUZZY), "one blend rule at a time");
     __shared__ uint32_t s_cnt[kTilePixels];
     __shared__ uint32_t s_prefix[kTilePixels];
     __shared__ uint32_t s_wave_tot[kBlock / kWave];
@@ -179,6 +228,7 @@ __global__ void __launch_bounds__(kBlock) bin_build_kernel(BuildPass a)
     float color[C];
 #pragma unroll
     for (int ci = 0; ci < C; ++ci) color[ci] = 0.f;
+    FuzzyBucket<C> fuzzy;  // FUZZY_BLEND only
     if (in_lds)
     {
 #pragma unroll
@@ -232,8 +282,18 @@ __global__ void __launch_bounds__(kBlock) bin_build_kernel(BuildPass a)
                 {
                     const float4 t4 = s_stage[r - base][0];
                     const float cf  = s_stage[r - base][1].x;
-                    s_T[2 * r + 1]  = T;
                     const float t[4] = {t4.x, t4.y, t4.z, t4.w};
+                    if constexpr (FUZZY)
+                    {
+                        // the depth half of the key is read before the transmittance takes its place; what is stored
+                        // is the transmittance in front of the bucket the fragment joins
+                        const float d = s_T[2 * r + 1];
+                        fuzzy.add(d, cf, t, a.depth_accept, T, color);
+                        s_T[2 * r + 1] = T;
+                        ++used;
+                        continue;
+                    }
+                    s_T[2 * r + 1]  = T;
                     const float Tc   = T * cf;
 #pragma unroll
                     for (int ci = 0; ci < C; ++ci) color[ci] = Tc * t[ci] + color[ci];
@@ -244,6 +304,8 @@ __global__ void __launch_bounds__(kBlock) bin_build_kernel(BuildPass a)
             }
             __syncthreads();
         }
+        if constexpr (FUZZY)
+            if (fuzzy.m > 0) fuzzy.flush(T, color);
         s_used[tid] = used;
         __syncthreads();
         if (a.transmittance)
@@ -285,7 +347,30 @@ __global__ void __launch_bounds__(kBlock) bin_build_kernel(BuildPass a)
         __syncthreads();
         if ((uint32_t)tid < pixels)
         {
-            if constexpr (!BILINEAR)
+            if constexpr (FUZZY)
+            {
+                const uint64_t* list = a.fragments + begin + start;
+                for (uint32_t j = 0; j < keep; ++j)
+                {
+                    const uint64_t k = list[j];
+                    const int id     = (int)(uint32_t)k;
+                    int ti           = -1;
+                    if ((uint32_t)id < (uint32_t)a.N) ti = a.index ? a.index[id] : id;
+                    float4 t4 = make_float4(0.f, 0.f, 0.f, 0.f);
+                    float cf  = 0.f;
+                    if ((uint32_t)ti < (uint32_t)a.N)
+                    {
+                        t4 = a.packed[2 * (size_t)ti];
+                        cf = a.packed[2 * (size_t)ti + 1].x;
+                    }
+                    const float t[4] = {t4.x, t4.y, t4.z, t4.w};
+                    fuzzy.add(__uint_as_float((uint32_t)(k >> 32)), cf, t, a.depth_accept, T, color);
+                    if (a.transmittance) a.transmittance[begin + start + j] = T;
+                }
+                if (fuzzy.m > 0) fuzzy.flush(T, color);
+                used = keep;
+            }
+            else if constexpr (!BILINEAR)
             {
                 blend_list_from_memory<C>(a.fragments + begin + start, keep, a.index, a.packed, a.N,
                                           a.transmittance ? a.transmittance + begin + start : nullptr, T, color);

@@ -142,7 +142,8 @@ inline int hits_of_mode(int render_mode)
 
 inline int check_mode(int render_mode)
 {
-    return (render_mode == 0 || render_mode == VETRAST_RENDER_FULL_BLEND || render_mode == VETRAST_RENDER_BILINEAR_BLEND)
+    return (render_mode == 0 || render_mode == VETRAST_RENDER_FULL_BLEND || render_mode == VETRAST_RENDER_FUZZY_BLEND ||
+            render_mode == VETRAST_RENDER_BILINEAR_BLEND)
                ? VETRAST_OK
                : VETRAST_ERR_UNSUPPORTED;
 }
@@ -526,9 +527,18 @@ int vetrast_forward(vetrast_ctx* ctx, const vetrast_forward_args* a, void* strea
             bp.K                   = p.debug_max_list_length;
             bp.use_environment_map = p.use_environment_map;
             bp.mask_value          = p.output_background_mask_value;
+            bp.depth_accept        = p.depth_accept_blend;
             for (int l = 0; l < VETRAST_MAX_LAYERS; ++l) bp.out[l] = out[l], bp.out_mask[l] = out_mask[l];
             const dim3 g(bins), blk(kBlock);
-            if (hits == 1)
+            if (p.render_mode == VETRAST_RENDER_FUZZY_BLEND)
+                switch (C)
+                {
+                    case 1: hipLaunchKernelGGL((bin_build_kernel<1, false, true>), g, blk, 0, stream, bp); break;
+                    case 2: hipLaunchKernelGGL((bin_build_kernel<2, false, true>), g, blk, 0, stream, bp); break;
+                    case 3: hipLaunchKernelGGL((bin_build_kernel<3, false, true>), g, blk, 0, stream, bp); break;
+                    default: hipLaunchKernelGGL((bin_build_kernel<4, false, true>), g, blk, 0, stream, bp); break;
+                }
+            else if (hits == 1)
                 switch (C)
                 {
                     case 1: hipLaunchKernelGGL((bin_build_kernel<1, false>), g, blk, 0, stream, bp); break;
@@ -648,7 +658,15 @@ int vetrast_backward(vetrast_ctx* ctx, const vetrast_backward_args* g, void* str
                 bp.out[l]          = a->out[l] + (size_t)b * C * plane;
             }
             const dim3 grid(tile_grid(tiles)), blk(kBlock);
-            if (hits == 1)
+            if (p.render_mode == VETRAST_RENDER_FUZZY_BLEND)
+                switch (C)
+                {
+                    case 1: hipLaunchKernelGGL(blend_backward_fuzzy_kernel<1>, grid, blk, 0, stream, bp, p.depth_accept_blend); break;
+                    case 2: hipLaunchKernelGGL(blend_backward_fuzzy_kernel<2>, grid, blk, 0, stream, bp, p.depth_accept_blend); break;
+                    case 3: hipLaunchKernelGGL(blend_backward_fuzzy_kernel<3>, grid, blk, 0, stream, bp, p.depth_accept_blend); break;
+                    default: hipLaunchKernelGGL(blend_backward_fuzzy_kernel<4>, grid, blk, 0, stream, bp, p.depth_accept_blend); break;
+                }
+            else if (hits == 1)
                 switch (C)
                 {
                     case 1: hipLaunchKernelGGL((blend_backward_kernel<1, false>), grid, blk, 0, stream, bp); break;
@@ -686,7 +704,10 @@ int vetrast_backward(vetrast_ctx* ctx, const vetrast_backward_args* g, void* str
             gp.background_rows       = background_rows;
             gp.num_background_rows   = (int)tile_grid(tiles);
             gp.grad_background       = g->grad_background;
-            gp.add_leak              = (p.quirk_background_confidence_leak && !p.use_environment_map && hits == 1) ? 1 : 0;
+            gp.add_leak = (p.quirk_background_confidence_leak && !p.use_environment_map && hits == 1 &&
+                           p.render_mode != VETRAST_RENDER_FUZZY_BLEND)
+                              ? 1
+                              : 0;
             gp.background_accumulate = b > 0 ? 1 : 0;
             gp.packed                = ws_ptr<float4>(ws, lay.packed_base);
             gp.texture_raw           = a->texture;

@@ -37,6 +37,7 @@ def make_params(scene: Scene, **overrides) -> abi.Params:
     p.confidence_activation = 0
     p.confidence_scale = 10.0
     p.texture_abs = 0
+    p.depth_accept_blend = 0.01
     for k, v in {**scene.params, **overrides}.items():
         if not hasattr(p, k):
             raise AttributeError(f"vetrast_params has no field {k}")
