@@ -243,7 +243,7 @@ def main():
     ap.add_argument("--config", type=int, default=3, choices=[2, 3, 5])
     ap.add_argument("--points", type=int, default=None, help="override the point count (debug runs)")
     ap.add_argument("--point-order", default="vet_preprocess", choices=["vet_preprocess", "generated"])
-    ap.add_argument("--render-mode", type=int, default=1, choices=[1, 3],
+    ap.add_argument("--render-mode", type=int, default=1, choices=[1, 2, 3],
                     help="1 = FULL_BLEND (the headline workload), 3 = BILINEAR_BLEND (four fragments per point and layer)")
     ap.add_argument("--no-second-order", action="store_true", help="skip timing the other point order")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -317,7 +317,8 @@ def main():
             "workload": f"BASELINE config {args.config} ({scene.name}): N={N} points, {scene.views[0].w}x{scene.views[0].h}, "
                         f"L={L} layers, K={K}, C={Cn}, B=1 view, " + ("forward+backward" if backward else "forward")
                         + f", point order {args.point_order}"
-                        + (", render_mode 3 (BILINEAR_BLEND)" if args.render_mode == 3 else ", render_mode 1 (FULL_BLEND)"),
+                        + {1: ", render_mode 1 (FULL_BLEND)", 2: ", render_mode 2 (FUZZY_BLEND, depth_accept_blend 0.01)",
+                           3: ", render_mode 3 (BILINEAR_BLEND)"}[args.render_mode],
             "point_order": args.point_order, "render_mode": args.render_mode,
             "fragments_per_layer": r["F_layers"], "fragments": F, "fragments_kept": Fk, "pixels": P,
         },

@@ -98,7 +98,7 @@ typedef struct vetrast_params
     float confidence_scale;                   /* 10 + sigmoid_narrowing_factor * epoch in VET */
     int32_t texture_abs;                      /* 1: |texture| and |background| (PipelineParams::non_subzero_texture) */
     float depth_accept_blend;                 /* FUZZY_BLEND: depth range of a bucket, RenderParams::depth_accept_blend
-                                                 (src/lib/data/Settings.h:42, default 0.01) */
+                                                 (src/lib/data/Settings.h:42, default 0.01); must lie in (0, 1e4) */
 } vetrast_params;
 
 #define VETRAST_RENDER_FULL_BLEND 1

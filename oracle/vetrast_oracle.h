@@ -1,8 +1,8 @@
 /*
  * CPU oracle of the blending point rasterizer — TEST INFRASTRUCTURE ONLY.
  *
- * A plain scalar restatement of the reference's FULL_BLEND path and of its BILINEAR_BLEND path (params.render_mode = 3)
- * (lfranke/VET, src/lib/rendering). It exists to
+ * A plain scalar restatement of the reference's FULL_BLEND path, of its BILINEAR_BLEND path (params.render_mode = 3)
+ * and of its FUZZY_BLEND path (params.render_mode = 2) (lfranke/VET, src/lib/rendering). It exists to
  * check the GPU library and to be timed as the CPU baseline; nothing that ships may call it. Only tests/,
  * __graft_entry__.smoke() and bench.py's cpu_baseline leg load this library.
  *
@@ -29,6 +29,10 @@
  *                     a pixel centre lands in one pixel), the blend and its early exit by an independent numpy blend,
  *                     value and position gradients by double-precision central differences of that blend (the
  *                     position gradient is analytic in this mode, so finite differences do pin it)
+ *   fuzzy mode        (render_mode 2) pinned by: a vanishing depth range is FULL_BLEND; on scenes whose buckets are fixed
+ *                     by construction (points on depth levels) an independent float64 model gives the forward image
+ *                     (nearest level averaged only), the descriptor/background gradients (central differences) and the
+ *                     confidence gradient (own bucket's term + bucket size x later buckets' terms)
  *   fused preparation confidence = sigmoid(scale * raw) pinned against a float64 logistic (<= 4e-7 relative: the exact bits of
  *                     torch::sigmoid are PARITY UNPINNED), |texture| / |background| and the chain rule of both by
  *                     comparing with the unfused path fed the prepared tensors and torch autograd

@@ -82,7 +82,7 @@ def test_mode_3_needs_the_bigger_workspace(rasterizer):
         rasterizer.forward(dev, make_params(scene, **MODE), workspace=small)
     assert e.value.status == abi.ERR_WORKSPACE_SMALL
     with pytest.raises(abi.VetrastError) as e:
-        rasterizer.forward(dev, make_params(scene, render_mode=2))
+        rasterizer.forward(dev, make_params(scene, render_mode=4))
     assert e.value.status == abi.ERR_UNSUPPORTED
 
 

@@ -132,3 +132,13 @@ def test_config3_full_size(rasterizer, oracle):
         assert err <= 1e-4, key
     # the background gradient is one float32 sum over 2.75 M pixels on either side: compare loosely, as for FULL_BLEND
     assert max_rel_err(got["background"].cpu().numpy(), want["background"]) <= 2e-3
+
+
+def test_depth_range_is_checked(rasterizer):
+    scene = synthetic.tiny_scene(num_points=500)
+    dev = DeviceScene(scene)
+    for bad in (0.0, -1.0, 1e5, float("nan")):
+        with pytest.raises(abi.VetrastError) as e:
+            rasterizer.forward(dev, make_params(scene, depth_accept_blend=bad, **MODE))
+        assert e.value.status == abi.ERR_INVALID_ARG
+    rasterizer.forward(dev, make_params(scene, depth_accept_blend=0.0))  # ignored by the other modes

@@ -19,7 +19,7 @@ def _views(scene):
             for v in scene.views]
 
 
-@pytest.mark.parametrize("render_mode", [1, 3], ids=["full_blend", "bilinear_blend"])
+@pytest.mark.parametrize("render_mode", [1, 2, 3], ids=["full_blend", "fuzzy_blend", "bilinear_blend"])
 @pytest.mark.parametrize("literal", [True, False], ids=["reference_literal", "clean"])
 def test_autograd_matches_oracle(literal, render_mode, oracle):
     from vet_amd import torch_ops

@@ -80,11 +80,14 @@ __device__ __forceinline__ bool blend_is_saturated(float T)
 // stays within depth_accept of the bucket's first one; a bucket is blended as ONE fragment with the mean confidence and
 // the mean descriptor of its elements. After the first bucket the reference sets its reference depth to -100000 (:1468)
 // instead of the next fragment's depth, so every later fragment closes the bucket in front of it: only the nearest
-// bucket ever holds more than one fragment, and a one-element bucket blends exactly like FULL_BLEND (x / 1.0f == x).
+// bucket ever holds more than one fragment, and a one-element bucket blends exactly like a FULL_BLEND fragment
+// (x / 1.0f == x). So the state below only lives until the nearest bucket is closed; from then on the ordinary blend
+// step runs. (That needs depth + 100000 >= depth_accept, which the host checks: depth_accept < 10000.)
 template <int C>
 struct FuzzyBucket
 {
-    float last_min = 0.f, conf = 0.f;
+    bool open = true;  // the nearest bucket is still collecting
+    float first_depth = 0.f, conf = 0.f;
     float t[C];
     int m = 0;
     __device__ __forceinline__ FuzzyBucket()
@@ -92,34 +95,33 @@ struct FuzzyBucket
 #pragma unroll
         for (int ci = 0; ci < C; ++ci) t[ci] = 0.f;
     }
-    // blends the collected elements into (T, color)
+    // blends the collected elements into (T, color) as one fragment
     __device__ __forceinline__ void flush(float& T, float (&color)[C])
     {
-        const float cf = conf / (float)m;
+        const float fm = (float)m;
+        const float cf = conf / fm;
         const float Tc = T * cf;
 #pragma unroll
-        for (int ci = 0; ci < C; ++ci) color[ci] = Tc * (t[ci] / (float)m) + color[ci];
-        T = (1.f - cf) * T;
+        for (int ci = 0; ci < C; ++ci) color[ci] = Tc * (t[ci] / fm) + color[ci];
+        T    = (1.f - cf) * T;
+        open = false;
     }
-    // fragment at depth d with confidence cf and descriptor td joins; closes the bucket in front of it first if d is
-    // out of its range
-    __device__ __forceinline__ void add(float d, float cf, const float (&td)[4], float depth_accept, float& T,
-                                        float (&color)[C])
+    // Fragment at depth d: true if it joined the nearest bucket; false if it lies behind it, in which case the bucket
+    // has been blended and the caller blends the fragment by itself.
+    __device__ __forceinline__ bool take(float d, float cf, const float (&td)[4], float depth_accept, float& T,
+                                         float (&color)[C])
     {
-        if (last_min == 0.f) last_min = d;
-        if (!(d - last_min < depth_accept))
+        if (m == 0) first_depth = d;
+        if (!(d - first_depth < depth_accept))
         {
             flush(T, color);
-            last_min = -100000.f;
-            conf     = 0.f;
-            m        = 0;
-#pragma unroll
-            for (int ci = 0; ci < C; ++ci) t[ci] = 0.f;
+            return false;
         }
         conf += cf;
 #pragma unroll
         for (int ci = 0; ci < C; ++ci) t[ci] += td[ci];
         ++m;
+        return true;
     }
 };
 
@@ -271,6 +273,8 @@ __global__ void __launch_bounds__(kBlock) bin_build_kernel(BuildPass a)
                     c4   = a.packed[2 * (size_t)ti + 1];
                     c4.x = fragment_alpha<BILINEAR>(a, l, low, c4.x);
                 }
+                // FUZZY_BLEND buckets by depth: it rides along in the stage (the key's depth half is still intact here)
+                if constexpr (FUZZY) c4.y = __uint_as_float(s_id[2 * r + 1]);
                 s_stage[r - base][0] = t4;
                 s_stage[r - base][1] = c4;
             }
@@ -281,17 +285,18 @@ __global__ void __launch_bounds__(kBlock) bin_build_kernel(BuildPass a)
                 for (uint32_t r = lo; r < hi && !saturated; ++r)
                 {
                     const float4 t4 = s_stage[r - base][0];
-                    const float cf  = s_stage[r - base][1].x;
+                    const float2 cd = *reinterpret_cast<const float2*>(&s_stage[r - base][1]);  // confidence, depth
+                    const float cf  = cd.x;
                     const float t[4] = {t4.x, t4.y, t4.z, t4.w};
                     if constexpr (FUZZY)
                     {
-                        // the depth half of the key is read before the transmittance takes its place; what is stored
-                        // is the transmittance in front of the bucket the fragment joins
-                        const float d = s_T[2 * r + 1];
-                        fuzzy.add(d, cf, t, a.depth_accept, T, color);
-                        s_T[2 * r + 1] = T;
-                        ++used;
-                        continue;
+                        // what is stored is the transmittance in front of the bucket the fragment joins
+                        if (fuzzy.open && fuzzy.take(cd.y, cf, t, a.depth_accept, T, color))
+                        {
+                            s_T[2 * r + 1] = T;
+                            ++used;
+                            continue;
+                        }
                     }
                     s_T[2 * r + 1]  = T;
                     const float Tc   = T * cf;
@@ -305,7 +310,7 @@ __global__ void __launch_bounds__(kBlock) bin_build_kernel(BuildPass a)
             __syncthreads();
         }
         if constexpr (FUZZY)
-            if (fuzzy.m > 0) fuzzy.flush(T, color);
+            if (fuzzy.open && fuzzy.m > 0) fuzzy.flush(T, color);
         s_used[tid] = used;
         __syncthreads();
         if (a.transmittance)
@@ -364,10 +369,16 @@ __global__ void __launch_bounds__(kBlock) bin_build_kernel(BuildPass a)
                         cf = a.packed[2 * (size_t)ti + 1].x;
                     }
                     const float t[4] = {t4.x, t4.y, t4.z, t4.w};
-                    fuzzy.add(__uint_as_float((uint32_t)(k >> 32)), cf, t, a.depth_accept, T, color);
+                    const bool joined =
+                        fuzzy.open && fuzzy.take(__uint_as_float((uint32_t)(k >> 32)), cf, t, a.depth_accept, T, color);
                     if (a.transmittance) a.transmittance[begin + start + j] = T;
+                    if (joined) continue;
+                    const float Tc = T * cf;
+#pragma unroll
+                    for (int ci = 0; ci < C; ++ci) color[ci] = Tc * t[ci] + color[ci];
+                    T = (1.f - cf) * T;
                 }
-                if (fuzzy.m > 0) fuzzy.flush(T, color);
+                if (fuzzy.open && fuzzy.m > 0) fuzzy.flush(T, color);
                 used = keep;
             }
             else if constexpr (!BILINEAR)

@@ -175,6 +175,9 @@ int validate_forward(const vetrast_forward_args* a, vetrast_workspace_layout* la
     if (p.check_normal) return VETRAST_ERR_UNSUPPORTED;
     int st = check_mode(p.render_mode);
     if (st != VETRAST_OK) return st;
+    // FUZZY_BLEND: a range <= 0 divides 0 by 0 in the reference's first bucket; the kernels rely on range < 1e4
+    if (p.render_mode == VETRAST_RENDER_FUZZY_BLEND && !(p.depth_accept_blend > 0.f && p.depth_accept_blend < 1e4f))
+        return VETRAST_ERR_INVALID_ARG;
     const int w = a->views[0].w, h = a->views[0].h;
     st          = check_dims(a->num_points, a->num_views, p.num_layers, w, h, hits_of_mode(p.render_mode));
     if (st != VETRAST_OK) return st;

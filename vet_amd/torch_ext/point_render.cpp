@@ -26,6 +26,7 @@ vetrast_params to_abi_params(const RenderParams& p, int num_layers)
     vetrast_params q;
     std::memset(&q, 0, sizeof(q));
     q.render_mode                      = p.render_mode;
+    q.depth_accept_blend               = p.depth_accept_blend;
     q.num_texture_channels             = p.num_texture_channels;
     q.num_layers                       = num_layers;
     q.debug_max_list_length            = p.debug_max_list_length;
@@ -74,8 +75,9 @@ vetrast_forward_args make_forward_args(NeuralRenderInfo* info, const torch::Tens
                     poses_se3.is_contiguous() && poses_se3.dim() == 2 && poses_se3.size(1) == 8,
                 "poses_se3 must be a contiguous [F,8] float64 tensor on the GPU");
     TORCH_CHECK(info->params.render_mode == VETRAST_RENDER_FULL_BLEND ||
+                    info->params.render_mode == VETRAST_RENDER_FUZZY_BLEND ||
                     info->params.render_mode == VETRAST_RENDER_BILINEAR_BLEND,
-                "only render_mode 1 (FULL_BLEND) and 3 (BILINEAR_BLEND) are implemented");
+                "only render_mode 1 (FULL_BLEND), 2 (FUZZY_BLEND) and 3 (BILINEAR_BLEND) are implemented");
     TORCH_CHECK(!info->params.add_depth_to_network, "add_depth_to_network is not part of the blending path");
     TORCH_CHECK(!info->images.empty(), "no views");
 
@@ -396,6 +398,7 @@ std::vector<torch::Tensor> blend_point_cloud(torch::Tensor texture, torch::Tenso
         else if (k == "quirk_background_confidence_leak") p.quirk_background_confidence_leak = as_d() != 0;
         else if (k == "point_gradient_normalization") p.point_gradient_normalization = (int)as_d();
         else if (k == "render_mode") p.render_mode = (int)as_d();
+        else if (k == "depth_accept_blend") p.depth_accept_blend = (float)as_d();
         else if (k == "K_gradient_factor") p.K_gradient_factor = (float)as_d();
         else if (k == "camera_gradient_normalization") p.camera_gradient_normalization = as_d() != 0;
         else if (k == "fused_confidence_scale") p.fused_confidence_scale = (float)as_d();

@@ -34,7 +34,8 @@ struct RenderParams
     float stability_cutoff_value       = 10000.f;
     bool need_point_gradient           = true;
     bool use_environment_map           = true;
-    int render_mode                    = 1;  // 1 = FULL_BLEND, 3 = BILINEAR_BLEND; modes 0 and 2 are not implemented
+    int render_mode                    = 1;  // 1 = FULL_BLEND, 2 = FUZZY_BLEND, 3 = BILINEAR_BLEND; mode 0 is not implemented
+    float depth_accept_blend           = 0.01f;  // FUZZY_BLEND: depth range of a bucket
     bool viewer_only                   = false;
     int debug_max_list_length          = -1;
     // Switches for two accidents of the reference implementation; the defaults reproduce it literally.
