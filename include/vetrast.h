@@ -83,13 +83,14 @@ typedef struct vetrast_params
     int32_t camera_gradient_normalization;    /* 0: leave sums and counts; 1: divide each pose / intrinsics row by its
                                                  count as src/lib/rendering/PointRenderer.cu:1253-1308 does (the count
                                                  grows by 1/1024 per fragment, so this is 1024 x the mean) */
-    int32_t render_mode;                      /* RenderParams::render_mode, src/lib/data/Settings.h: 0 or 1 = FULL_BLEND
+    int32_t render_mode;                      /* RenderParams::render_mode, src/lib/data/Settings.h: 1 = FULL_BLEND
                                                  (a point lands in the pixel it rounds to), 3 = BILINEAR_BLEND (a point
                                                  lands in the 2x2 pixels around it, alpha = bilinear weight x confidence,
                                                  blending stops once the transmittance falls below 0.001), 2 =
                                                  FUZZY_BLEND (FULL_BLEND lists; the nearest fragments of a pixel that
                                                  lie within depth_accept_blend of the first one are averaged before
-                                                 they are blended). Other values are refused. */
+                                                 they are blended). Other values (0 = FUZZY_DT, the
+                                                 depth-test mode, included) are refused. */
     /* The steps VET runs on the optimised tensors right before the rasterizer, fused into it
      * (NeuralPointTextureImpl::PrepareConfidence / PrepareTexture, src/lib/models/NeuralTexture.h:38-55; called from
      * src/lib/models/Pipeline.cpp:113-124). With them on, `confidence`, `texture` and `background` are the RAW tensors

@@ -293,7 +293,7 @@ int validate(const vetrast_forward_args* a)
     if (p.num_layers < 1 || p.num_layers > VETRAST_MAX_LAYERS) return VETRAST_ERR_INVALID_ARG;
     if (p.num_texture_channels < 1 || p.num_texture_channels > VETRAST_MAX_CHANNELS) return VETRAST_ERR_INVALID_ARG;
     if (p.check_normal) return VETRAST_ERR_UNSUPPORTED;
-    if (p.render_mode != 0 && p.render_mode != VETRAST_RENDER_FULL_BLEND && !is_bilinear(p) && !is_fuzzy(p))
+    if (p.render_mode != VETRAST_RENDER_FULL_BLEND && !is_bilinear(p) && !is_fuzzy(p))
         return VETRAST_ERR_UNSUPPORTED;
     if (is_bilinear(p) && a->num_points > (1 << 30)) return VETRAST_ERR_INVALID_ARG;  // id and corner share 32 key bits
     for (int b = 0; b < a->num_views; ++b)

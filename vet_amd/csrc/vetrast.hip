@@ -142,7 +142,7 @@ inline int hits_of_mode(int render_mode)
 
 inline int check_mode(int render_mode)
 {
-    return (render_mode == 0 || render_mode == VETRAST_RENDER_FULL_BLEND || render_mode == VETRAST_RENDER_FUZZY_BLEND ||
+    return (render_mode == VETRAST_RENDER_FULL_BLEND || render_mode == VETRAST_RENDER_FUZZY_BLEND ||
             render_mode == VETRAST_RENDER_BILINEAR_BLEND)
                ? VETRAST_OK
                : VETRAST_ERR_UNSUPPORTED;
