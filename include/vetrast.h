@@ -196,7 +196,7 @@ typedef struct vetrast_forward_args
 /* Arguments of the backward pass. Replaces BlendPointCloudBackward's inputs and its seven returned tensors
  * (src/lib/rendering/PointRenderer.cu:1111-1323). The workspace and `out` must be those of the matching forward call
  * (made with save_for_backward = 1) and unchanged since; this is the saved state of
- * src/lib/rendering/PointRenderer.cu:1027-1059. */
+ * src/lib/rendering/PointRenderer.cu:1027-1059. fwd.out_mask is not used and may be left NULL. */
 typedef struct vetrast_backward_args
 {
     vetrast_forward_args fwd;                      /* same values as passed to vetrast_forward */

@@ -155,3 +155,50 @@ def test_fill_scene_grid_with_loss_through_the_shim(oracle):
     np.testing.assert_allclose(value.cpu().numpy().ravel(), want_v, rtol=1e-6)
     normalised = value / torch.where(count != 0, count, torch.ones_like(count))   # NormalizeBBCellValue
     np.testing.assert_allclose(normalised.cpu().numpy().ravel(), want_v / np.maximum(want_c, 1), rtol=1e-6)
+
+
+def test_render_module_glue_super_sampling_and_mask_channel(oracle):
+    """PointRenderModuleImpl::forward (src/lib/rendering/RenderModule.cpp:45-245) around the rasterizer: with
+    super_sampling the views are rendered at twice the size (crop transform scaled by 2) and 2x2 blocks averaged; the
+    masks come back detached and, with cat_masks_to_color, as an extra image channel. Checked against the oracle
+    rendering the doubled views, pooled by hand, and against autograd through the pooling."""
+    from vet_amd import torch_ops
+    from vet_amd.synthetic import ViewSpec
+
+    scene = synthetic.tiny_scene(num_points=3000, K=8, seed=33, w=32, h=24, num_layers=3)
+    big = synthetic.tiny_scene(num_points=3000, K=8, seed=33, w=32, h=24, num_layers=3)
+    big.views = [ViewSpec(64, 48, crop_transform=(2.0, 2.0, 0.0, 0.0, 0.0))]
+    params = make_params(big, output_background_mask=1, output_background_mask_value=0.25, need_point_gradient=0)
+    ref = oracle.forward(big, params)
+    pool = lambda a: a.reshape(a.shape[0], a.shape[1], a.shape[2] // 2, 2, a.shape[3] // 2, 2).mean(axis=(3, 5))
+
+    cu = lambda a, rg=False: torch.from_numpy(np.ascontiguousarray(a)).cuda().requires_grad_(rg)
+    texture, confidence = cu(scene.texture, True), cu(scene.confidence.reshape(1, -1), True)
+    views = _views(scene)
+    outs = torch_ops.blend_point_cloud(texture, cu(scene.background), cu(scene.position),
+                                       torch.zeros((1, 6), dtype=torch.float64, device="cuda"), cu(scene.intrinsics),
+                                       confidence, cu(scene.poses_se3), None, views, scene.num_layers, train=True,
+                                       use_environment_map=0, drop_out_points_by_radius=0, need_point_gradient=0,
+                                       debug_max_list_length=scene.max_list_length, output_background_mask=1,
+                                       output_background_mask_value=0.25, quirk_background_confidence_leak=0,
+                                       super_sampling=1, cat_masks_to_color=1)
+    L = scene.num_layers
+    assert len(outs) == 2 * L
+    for l, (w, h) in enumerate(scene.layer_sizes()):
+        img, mask = outs[l], outs[L + l]
+        assert tuple(img.shape) == (1, scene.num_channels + 1, h, w) and tuple(mask.shape) == (1, 1, h, w)
+        assert not mask.requires_grad
+        np.testing.assert_allclose(img[:, :-1].detach().cpu().numpy(), pool(ref.out[l]), rtol=1e-6, atol=1e-7)
+        np.testing.assert_allclose(mask.cpu().numpy(), pool(ref.out_mask[l]), rtol=1e-6)
+        np.testing.assert_array_equal(img[:, -1:].detach().cpu().numpy(), mask.cpu().numpy())
+    # gradients flow through the pooling into the rasterizer: upstream gradient g on the pooled image is g / 4 on
+    # each of the four pixels it averages
+    grad_small = [np.random.default_rng(5 + l).normal(size=(1, scene.num_channels, h, w)).astype(np.float32)
+                  for l, (w, h) in enumerate(scene.layer_sizes())]
+    loss = sum((outs[l][:, :-1] * cu(grad_small[l])).sum() for l in range(L))
+    loss.backward()
+    grad_big = [np.repeat(np.repeat(g, 2, axis=2), 2, axis=3) * np.float32(0.25) for g in grad_small]
+    want = oracle.backward(ref, grad_big, want_points=False)
+    assert max_rel_err(texture.grad.cpu().numpy(), want["texture"]) <= 1e-4
+    assert max_rel_err(confidence.grad.cpu().numpy().ravel(), want["confidence"]) <= 1e-4
+    assert views == _views(scene), "the views are restored after the call"

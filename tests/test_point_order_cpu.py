@@ -1,0 +1,60 @@
+"""The point order VET's preprocessing produces (Morton order, then shuffled 256-point blocks) as the shim computes it:
+against an independent bit-by-bit interleave, against the numpy generator of the benchmark scenes, and its block
+structure. Runs on the CPU (the function is host code)."""
+import numpy as np
+import torch
+
+from vet_amd import synthetic, torch_ops
+
+
+def _morton_by_hand(xyz):
+    """63-bit Morton code with plain Python integers: bit k of axis a goes to bit 3k + a."""
+    lo, hi = xyz.min(axis=0), xyz.max(axis=0)
+    cells = np.floor((xyz - lo) / np.maximum(hi - lo, 1e-30) * ((1 << 21) - 1)).astype(np.int64)
+    codes = []
+    for c in cells:
+        code = 0
+        for a in range(3):
+            for k in range(21):
+                code |= ((int(c[a]) >> k) & 1) << (3 * k + a)
+        codes.append(code)
+    return codes
+
+
+def test_single_block_is_the_morton_order():
+    rng = np.random.default_rng(0)
+    xyz = rng.uniform(-3, 5, size=(2000, 3))
+    order = torch_ops.morton_block_shuffle_order(torch.from_numpy(xyz), block=4096, seed=7).numpy()
+    assert sorted(order.tolist()) == list(range(2000))
+    codes = _morton_by_hand(xyz)
+    sorted_codes = [codes[i] for i in order]
+    assert all(a <= b for a, b in zip(sorted_codes, sorted_codes[1:]))
+    # the generator of the benchmark scenes computes the same order (one block: nothing to shuffle)
+    np.testing.assert_array_equal(order, synthetic.vet_preprocess_order(xyz, seed=3, block=4096))
+    # float32 [N,4] input (the rasterizer's position tensor) works as well
+    pos4 = torch.zeros((2000, 4), dtype=torch.float32)
+    pos4[:, :3] = torch.from_numpy(xyz).float()
+    order4 = torch_ops.morton_block_shuffle_order(pos4, block=4096).numpy()
+    codes4 = _morton_by_hand(pos4[:, :3].double().numpy())
+    assert all(codes4[a] <= codes4[b] for a, b in zip(order4, order4[1:]))
+
+
+def test_blocks_are_shuffled_whole():
+    rng = np.random.default_rng(1)
+    xyz = rng.normal(size=(10_000, 3))
+    morton = torch_ops.morton_block_shuffle_order(torch.from_numpy(xyz), block=1 << 20).numpy()
+    a = torch_ops.morton_block_shuffle_order(torch.from_numpy(xyz), block=256, seed=1).numpy()
+    b = torch_ops.morton_block_shuffle_order(torch.from_numpy(xyz), block=256, seed=2).numpy()
+    assert sorted(a.tolist()) == list(range(10_000)) and sorted(b.tolist()) == list(range(10_000))
+    assert not np.array_equal(a, b) and not np.array_equal(a, morton)
+    np.testing.assert_array_equal(a, torch_ops.morton_block_shuffle_order(torch.from_numpy(xyz), block=256, seed=1).numpy())
+    # every run of the result that came from one block is a stretch of the Morton order
+    where = np.empty(10_000, np.int64)
+    where[morton] = np.arange(10_000)
+    pos = where[a]
+    blocks = pos // 256
+    starts = np.flatnonzero(np.diff(blocks) != 0) + 1
+    for seg in np.split(pos, starts):
+        assert np.all(np.diff(seg) == 1) and seg[0] % 256 == 0
+    assert len(starts) + 1 == (10_000 + 255) // 256
+    assert torch_ops.morton_block_shuffle_order(torch.zeros((0, 3))).numel() == 0

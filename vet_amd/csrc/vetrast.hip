@@ -163,7 +163,8 @@ int check_dims(int64_t N, int B, int L, int w, int h, int hits)
     return VETRAST_OK;
 }
 
-int validate_forward(const vetrast_forward_args* a, vetrast_workspace_layout* lay)
+// `for_backward`: the masks are not read or written by the backward pass, so their pointers may be missing there.
+int validate_forward(const vetrast_forward_args* a, vetrast_workspace_layout* lay, bool for_backward = false)
 {
     if (!a) return VETRAST_ERR_INVALID_ARG;
     const vetrast_params& p = a->params;
@@ -192,7 +193,7 @@ int validate_forward(const vetrast_forward_args* a, vetrast_workspace_layout* la
     for (int l = 0; l < p.num_layers; ++l)
     {
         if (!a->out[l]) return VETRAST_ERR_INVALID_ARG;
-        if (p.output_background_mask && !a->out_mask[l]) return VETRAST_ERR_INVALID_ARG;
+        if (p.output_background_mask && !for_backward && !a->out_mask[l]) return VETRAST_ERR_INVALID_ARG;
     }
     if (((uintptr_t)a->workspace % kAlign) != 0 || ((uintptr_t)a->position % 16) != 0) return VETRAST_ERR_INVALID_ARG;
     st = vetrast_workspace_layout_for_mode(a->num_points, a->num_views, p.num_layers, w, h, p.render_mode, lay);
@@ -568,7 +569,7 @@ int vetrast_backward(vetrast_ctx* ctx, const vetrast_backward_args* g, void* str
     if (!ctx || !g) return VETRAST_ERR_INVALID_ARG;
     const vetrast_forward_args* a = &g->fwd;
     vetrast_workspace_layout lay;
-    int st = validate_forward(a, &lay);
+    int st = validate_forward(a, &lay, /*for_backward=*/true);
     if (st != VETRAST_OK) return st;
     if (!a->save_for_backward) return VETRAST_ERR_INVALID_ARG;
     if (!g->grad_texture || !g->grad_confidence || !g->grad_background) return VETRAST_ERR_INVALID_ARG;

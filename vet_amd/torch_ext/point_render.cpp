@@ -2,7 +2,10 @@
 // calling the C ABI of include/vetrast.h. See point_render.h for the reference lines each piece mirrors.
 #include "point_render.h"
 
+#include <algorithm>
+#include <cmath>
 #include <cstring>
+#include <random>
 
 #include <c10/hip/HIPStream.h>
 #include <torch/extension.h>
@@ -337,6 +340,121 @@ TORCH_LIBRARY(vet_amd, m)
     m.class_<vet_amd::NeuralRenderInfo>("NeuralRenderInfo").def(torch::init());
 }
 
+namespace vet_amd
+{
+std::pair<std::vector<torch::Tensor>, std::vector<torch::Tensor>> PointRenderModule::forward(NeuralRenderInfo* nri)
+{
+    TORCH_CHECK(nri, "PointRenderModule::forward: null NeuralRenderInfo");
+    TORCH_CHECK(!nri->params.add_depth_to_network, "add_depth_to_network is not available");
+    nri->cache = cache.get();
+    // IntrinsicsPinhole::scale multiplies all five entries (fx, fy, cx, cy, s)
+    auto rescale = [&](float f) {
+        for (auto& i : nri->images)
+        {
+            i.w = f > 1.f ? i.w * 2 : i.w / 2;
+            i.h = f > 1.f ? i.h * 2 : i.h / 2;
+            for (int k = 0; k < 5; ++k) i.crop_transform[k] *= f;
+        }
+    };
+    if (super_sampling) rescale(2.f);
+    std::vector<torch::Tensor> combined;
+    try
+    {
+        combined = BlendPointCloud(nri);
+    }
+    catch (...)
+    {
+        if (super_sampling) rescale(0.5f);
+        throw;
+    }
+    const int L = nri->num_layers;
+    std::vector<torch::Tensor> images(combined.begin(), combined.begin() + L);
+    std::vector<torch::Tensor> masks;
+    if (nri->params.output_background_mask)
+    {
+        TORCH_CHECK((int)combined.size() == 2 * L, "BlendPointCloud returned ", combined.size(), " tensors, expected ", 2 * L);
+        masks.assign(combined.begin() + L, combined.end());
+        for (auto& m : masks) m = m.detach();
+    }
+    if (super_sampling)
+    {
+        for (auto& img : images) img = torch::avg_pool2d(img, {2, 2});
+        for (auto& m : masks) m = torch::avg_pool2d(m, {2, 2});
+        rescale(0.5f);
+    }
+    if (cat_masks_to_color)
+    {
+        TORCH_CHECK(!masks.empty(), "cat_masks_to_color needs output_background_mask");
+        for (int i = 0; i < L; ++i) images[i] = torch::cat({images[i], masks[i]}, 1);
+    }
+    TORCH_CHECK(images.front().size(2) == nri->images.front().h && images.front().size(3) == nri->images.front().w,
+                "PointRenderModule: output size does not match the view");
+    return {images, masks};
+}
+
+namespace
+{
+inline uint64_t spread_bits21(uint64_t v)
+{
+    v &= 0x1FFFFFull;
+    v = (v | (v << 32)) & 0x1F00000000FFFFull;
+    v = (v | (v << 16)) & 0x1F0000FF0000FFull;
+    v = (v | (v << 8)) & 0x100F00F00F00F00Full;
+    v = (v | (v << 4)) & 0x10C30C30C30C30C3ull;
+    v = (v | (v << 2)) & 0x1249249249249249ull;
+    return v;
+}
+}  // namespace
+
+torch::Tensor MortonBlockShuffleOrder(torch::Tensor positions, int64_t block, uint64_t seed)
+{
+    TORCH_CHECK(positions.dim() == 2 && positions.size(1) >= 3 && !positions.is_cuda() && block >= 1,
+                "MortonBlockShuffleOrder: positions is a [N,3] or [N,4] CPU tensor, block >= 1");
+    const torch::Tensor p = positions.slice(1, 0, 3).to(torch::kFloat64).contiguous();
+    const int64_t n       = p.size(0);
+    torch::Tensor out     = torch::empty({n}, torch::kInt64);
+    if (n == 0) return out;
+    const double* x = p.data_ptr<double>();
+    double lo[3], hi[3];
+    for (int k = 0; k < 3; ++k) lo[k] = hi[k] = x[k];
+    for (int64_t i = 0; i < n; ++i)
+        for (int k = 0; k < 3; ++k)
+        {
+            lo[k] = std::min(lo[k], x[3 * i + k]);
+            hi[k] = std::max(hi[k], x[3 * i + k]);
+        }
+    std::vector<std::pair<uint64_t, int64_t>> keyed((size_t)n);
+    for (int64_t i = 0; i < n; ++i)
+    {
+        uint64_t code = 0;
+        for (int k = 0; k < 3; ++k)
+        {
+            const double ext = std::max(hi[k] - lo[k], 1e-30);
+            const uint64_t c = (uint64_t)std::floor((x[3 * i + k] - lo[k]) / ext * (double)((1 << 21) - 1));
+            code |= spread_bits21(c) << k;
+        }
+        keyed[(size_t)i] = {code, i};
+    }
+    std::stable_sort(keyed.begin(), keyed.end(),
+                     [](const std::pair<uint64_t, int64_t>& a, const std::pair<uint64_t, int64_t>& b) { return a.first < b.first; });
+    const int64_t blocks = (n + block - 1) / block;
+    std::vector<int64_t> block_order((size_t)blocks);
+    for (int64_t b = 0; b < blocks; ++b) block_order[(size_t)b] = b;
+    std::mt19937_64 gen(seed);
+    for (int64_t b = blocks - 1; b > 0; --b)  // Fisher-Yates
+    {
+        const int64_t j = (int64_t)(gen() % (uint64_t)(b + 1));
+        std::swap(block_order[(size_t)b], block_order[(size_t)j]);
+    }
+    int64_t* o = out.data_ptr<int64_t>();
+    int64_t w  = 0;
+    for (int64_t b = 0; b < blocks; ++b)
+        for (int64_t k = block_order[(size_t)b] * block; k < std::min(n, (block_order[(size_t)b] + 1) * block); ++k)
+            o[w++] = keyed[(size_t)k].second;
+    return out;
+}
+}  // namespace vet_amd
+
 // ---- Python binding used by the tests: builds a NeuralRenderInfo from plain arguments and calls BlendPointCloud ----
 namespace
 {
@@ -381,6 +499,7 @@ std::vector<torch::Tensor> blend_point_cloud(torch::Tensor texture, torch::Tenso
     }
     RenderParams& p = nri.params;
     p.dropout       = 0.f;
+    bool super_sampling = false, cat_masks_to_color = false;
     for (auto item : params)
     {
         const std::string k = pybind11::cast<std::string>(item.first);
@@ -403,7 +522,21 @@ std::vector<torch::Tensor> blend_point_cloud(torch::Tensor texture, torch::Tenso
         else if (k == "camera_gradient_normalization") p.camera_gradient_normalization = as_d() != 0;
         else if (k == "fused_confidence_scale") p.fused_confidence_scale = (float)as_d();
         else if (k == "fused_texture_abs") p.fused_texture_abs = as_d() != 0;
+        else if (k == "super_sampling") super_sampling = as_d() != 0;
+        else if (k == "cat_masks_to_color") cat_masks_to_color = as_d() != 0;
         else TORCH_CHECK(false, "unknown RenderParams field ", k);
+    }
+    if (super_sampling || cat_masks_to_color)
+    {
+        // through the caller glue of the reference (PointRenderModuleImpl::forward): images, then masks
+        PointRenderModule module;
+        module.cache              = g_cache;
+        module.super_sampling     = super_sampling;
+        module.cat_masks_to_color = cat_masks_to_color;
+        auto result               = module.forward(&nri);
+        std::vector<torch::Tensor> out = result.first;
+        out.insert(out.end(), result.second.begin(), result.second.end());
+        return out;
     }
     // the scene bundle only has to live for the duration of apply(): everything backward needs is saved in the graph
     return BlendPointCloud(&nri);
@@ -503,6 +636,9 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
                                            intrinsics, loss_img);
         },
         "PointRendererCache::FillSceneGridWithLoss of the reference, with the cell tensors passed one by one");
+    m.def("morton_block_shuffle_order", &vet_amd::MortonBlockShuffleOrder, pybind11::arg("positions"),
+          pybind11::arg("block") = 256, pybind11::arg("seed") = 0,
+          "ReorderMorton64 + RandomBlockShuffle(block) of the reference's scene preprocessing, as a permutation");
     m.def("blend_point_cloud", &blend_point_cloud,
           "BlendPointCloud(NeuralRenderInfo*) of the reference, with the scene passed as tensors");
 }

@@ -153,4 +153,29 @@ class MyAdam
 // [B,1,h_l,w_l] if output_background_mask.
 std::vector<torch::Tensor> BlendPointCloud(NeuralRenderInfo* info);
 
+// The caller of BlendPointCloud in VET: PointRenderModuleImpl::forward(NeuralRenderInfo*)
+// (src/lib/rendering/RenderModule.cpp:45-245). It owns the cache, renders at twice the resolution and averages 2x2
+// blocks when super_sampling is on (:60-68,102-127), splits the flat output list into images and (detached) masks
+// (:74-100) and appends the masks to the images as an extra channel when cat_masks_to_color is on (:204-210).
+// The environment-map branch (:129-202) and add_depth_to_network need modules outside the rasterizer and are refused.
+class PointRenderModule
+{
+   public:
+    bool super_sampling     = false;  // RenderParams::super_sampling, src/lib/data/Settings.h:38
+    bool cat_masks_to_color = false;  // PipelineParams::cat_masks_to_color, src/lib/data/Settings.h:295
+    PointRenderModule() : cache(std::make_shared<PointRendererCache>()) {}
+    // {images, masks}: L images [B,C(+1),h_l,w_l]; L masks [B,1,h_l,w_l] if output_background_mask, else none
+    std::pair<std::vector<torch::Tensor>, std::vector<torch::Tensor>> forward(NeuralRenderInfo* nri);
+    std::shared_ptr<PointRendererCache> cache;
+};
+
+// The order VET's scene preprocessing gives a point cloud before the rasterizer ever sees it
+// (point_cloud.ReorderMorton64(); point_cloud.RandomBlockShuffle(256); src/lib/data/SceneData.cpp:105-106): points sorted
+// by the 63-bit Morton code of their position inside the cloud's bounding box (21 bits per axis), then whole blocks of
+// `block` consecutive points shuffled. It is what gives the binning passes their locality (neighbouring threads hit
+// neighbouring pixels) while no pixel's fragments arrive from one workgroup only. positions: [N,3] or [N,4] float CPU
+// tensor; returns the permutation [N] int64 (new index -> old index). The Morton part is deterministic; the block
+// shuffle uses std::mt19937_64(seed) (saiga's generator is not part of the reference tree).
+torch::Tensor MortonBlockShuffleOrder(torch::Tensor positions, int64_t block = 256, uint64_t seed = 0);
+
 }  // namespace vet_amd

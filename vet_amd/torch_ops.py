@@ -45,3 +45,9 @@ def fill_scene_grid_with_loss(batch, cell_bb_min, cell_bb_length, cell_value, ce
     the error image [C,h,w] of view `batch` to cell_value / cell_access_count in place. views as in blend_point_cloud."""
     load().fill_scene_grid_with_loss(int(batch), cell_bb_min, cell_bb_length, cell_value, cell_access_count,
                                      [list(map(float, v)) for v in views], poses_se3, intrinsics, loss_img)
+
+
+def morton_block_shuffle_order(positions, block=256, seed=0):
+    """The point order of the reference's scene preprocessing (ReorderMorton64 + RandomBlockShuffle(256),
+    src/lib/data/SceneData.cpp:105-106) as a permutation [N] int64 of a [N,3] or [N,4] CPU tensor of positions."""
+    return load().morton_block_shuffle_order(positions, int(block), int(seed))
