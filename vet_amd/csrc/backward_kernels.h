@@ -243,7 +243,7 @@ __global__ void __launch_bounds__(kBlock) blend_backward_kernel(BackwardPass a)
                     x += ((g[ci] * t[ci]) * T) * c;
                 }
             }
-            // suffix sum over the fragments of the same pixel that sit in higher lanes of this round
+            // suffix sum over the fragments of the same pixel that sit in higher lanes of this step
             float v = x;
 #pragma unroll
             for (int d = 1; d < kWave; d <<= 1)
@@ -255,8 +255,8 @@ __global__ void __launch_bounds__(kBlock) blend_backward_kernel(BackwardPass a)
             const float vn = __shfl_down(v, 1, kWave);
             const int pn   = __shfl_down(p, 1, kWave);
             const int pp   = __shfl_up(p, 1, kWave);
-            float S        = (lane + 1 < kWave && pn == p) ? vn : 0.f;  // deeper fragments of this round
-            if (valid) S += s_carry[wave][p];                            // and of the rounds / windows before
+            float S        = (lane + 1 < kWave && pn == p) ? vn : 0.f;  // deeper fragments of this step
+            if (valid) S += s_carry[wave][p];                            // and of the steps / windows before
             if (valid && (lane == 0 || pp != p)) s_carry[wave][p] += v;  // one lane per pixel moves the carry on
             float4 rec_lo = make_float4(0.f, 0.f, 0.f, 0.f), rec_hi = rec_lo;
             if (ti >= 0)
