@@ -177,3 +177,22 @@ def test_cluster_far_denser_than_the_layer_average(K, rasterizer, oracle):
     res, ref, _ = _parity(scene, rasterizer, oracle, backward=(K > 0), need_point_gradient=1)
     counts = np.diff(res.offsets(0))
     assert counts.max() > 2500 and (counts > 0).sum() < 40
+
+
+def test_more_views_than_one_preparation_launch_holds(rasterizer, oracle):
+    """18 views: the view constants are prepared 16 per launch, the second launch must not reset what the first wrote."""
+    print("[case] 18 views", flush=True)
+    scene = synthetic.tiny_scene(num_points=1500, K=6, seed=53, num_views=18)
+    params = make_params(scene, need_point_gradient=1)
+    ref = oracle.forward(scene, params)
+    dev = DeviceScene(scene)
+    res = rasterizer.forward(dev, params, save_for_backward=True)
+    torch.cuda.synchronize()
+    for l in range(scene.num_layers):
+        np.testing.assert_array_equal(res.out[l].cpu().numpy(), ref.out[l])
+    grad_out = scene.grad_out()
+    want = oracle.backward(ref, grad_out, want_cameras=True)
+    got = rasterizer.backward(res, [torch.from_numpy(g).cuda() for g in grad_out], want_cameras=True)
+    torch.cuda.synchronize()
+    for key in ("texture", "confidence", "background", "points", "pose"):
+        assert max_rel_err(got[key].cpu().numpy(), want[key]) <= 1e-4, key
