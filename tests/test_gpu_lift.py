@@ -145,3 +145,36 @@ def test_argument_checks(rasterizer):
     rasterizer.lift_error(*args, border_pixels=32)
     torch.cuda.synchronize()
     assert int(cnt.sum()) == 0
+
+
+def test_lift_replays_from_a_hip_graph(rasterizer, oracle):
+    """vetrast_lift_error only launches kernels (no memsets, allocations or host reads): captured in a graph and
+    replayed, each replay adds the same counts and sums again; eager work (an optimiser step) runs between replays."""
+    import ctypes as C
+
+    mn, ln, view, poses, intr, img = _rotated_view_case(7)
+    n = len(mn)
+    want_v, want_c = np.zeros(n, np.float32), np.zeros(n, np.int32)
+    oracle.lift_error(mn, ln, want_v, want_c, view, poses, intr, img, border_pixels=8)
+    dev = [torch.from_numpy(np.ascontiguousarray(a)).cuda() for a in (mn, ln, poses, intr, img)]
+    val = torch.zeros(n, device="cuda")
+    cnt = torch.zeros(n, dtype=torch.int32, device="cuda")
+    ws = rasterizer.lift_error(dev[0], dev[1], val, cnt, view, dev[2], dev[3], dev[4], border_pixels=8)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(cnt.cpu().numpy(), want_c)
+    p = torch.linspace(-1, 1, 5000, device="cuda")
+    g = torch.cos(torch.arange(5000, device="cuda", dtype=torch.float32))
+    m, v = torch.zeros_like(p), torch.zeros_like(p)
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            rasterizer.lift_error(dev[0], dev[1], val, cnt, view, dev[2], dev[3], dev[4], border_pixels=8, workspace=ws)
+    for replay in range(3):
+        graph.replay()
+        torch.cuda.synchronize()
+        np.testing.assert_array_equal(cnt.cpu().numpy(), (replay + 2) * want_c)
+        np.testing.assert_allclose(val.cpu().numpy(), (replay + 2) * want_v.astype(np.float64), rtol=2e-6)
+        rasterizer.adam_step(p, g, m, v, replay + 1, 1e-2)  # eager work between the replays
+        torch.cuda.synchronize()
+    assert torch.isfinite(p).all()
