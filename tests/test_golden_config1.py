@@ -109,3 +109,39 @@ def test_gpu_reproduces_the_bilinear_golden_vector(rasterizer, scene, golden_bil
     g = rasterizer.backward(res, [torch.from_numpy(t).cuda() for t in scene.grad_out()])
     torch.cuda.synchronize()
     _check_bilinear_gradients({k: v.cpu().numpy() for k, v in g.items() if k != "_args"}, golden_bilinear)
+
+
+# ---- the same scene in FUZZY_BLEND (render_mode 2, depth range 0.5) ---------------------------------------------------
+FUZZY_FIXTURE = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "config1_fuzzy_oracle.npz")
+FUZZY = dict(render_mode=2, depth_accept_blend=0.5, need_point_gradient=1)
+
+
+@pytest.fixture(scope="module")
+def golden_fuzzy():
+    return np.load(FUZZY_FIXTURE, allow_pickle=False)
+
+
+def test_oracle_reproduces_the_fuzzy_golden_vector(oracle, scene, golden_fuzzy):
+    f = oracle.forward(scene, **FUZZY)
+    np.testing.assert_array_equal(f.out[0][0][:, 96:160:4, :], golden_fuzzy["out_rows"])
+    assert sha(f.out[0][0]) == str(golden_fuzzy["out_sha256"])
+    assert sha(f.fragments[0, :int(f.offsets[0, -1])]) == str(golden_fuzzy["fragments_sha256"])
+    assert sha(f.weight[0]) == str(golden_fuzzy["weight_sha256"])
+    _check_bilinear_gradients(oracle.backward(f, scene.grad_out()), golden_fuzzy)
+
+
+@pytest.mark.gpu
+def test_gpu_reproduces_the_fuzzy_golden_vector(rasterizer, scene, golden_fuzzy):
+    import torch
+
+    from vet_amd.rasterizer import DeviceScene, make_params
+
+    res = rasterizer.forward(DeviceScene(scene), make_params(scene, **FUZZY))
+    torch.cuda.synchronize()
+    out = res.out[0].cpu().numpy()[0]
+    np.testing.assert_array_equal(out[:, 96:160:4, :], golden_fuzzy["out_rows"])
+    assert sha(out) == str(golden_fuzzy["out_sha256"])
+    assert sha(res.weight(0)) == str(golden_fuzzy["weight_sha256"])
+    g = rasterizer.backward(res, [torch.from_numpy(t).cuda() for t in scene.grad_out()])
+    torch.cuda.synchronize()
+    _check_bilinear_gradients({k: v.cpu().numpy() for k, v in g.items() if k != "_args"}, golden_fuzzy)
