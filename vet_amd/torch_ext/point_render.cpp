@@ -5,6 +5,7 @@
 #include <algorithm>
 #include <cmath>
 #include <cstring>
+#include <fstream>
 #include <random>
 
 #include <c10/hip/HIPStream.h>
@@ -394,6 +395,107 @@ std::pair<std::vector<torch::Tensor>, std::vector<torch::Tensor>> PointRenderMod
 
 namespace
 {
+bool file_exists(const std::string& path)
+{
+    std::ifstream f(path, std::ios::binary);
+    return f.good();
+}
+
+// One entry of a module archive; false if the archive has no entry of that name.
+bool read_entry(torch::serialize::InputArchive& ar, const char* name, torch::Tensor& t, bool is_buffer)
+{
+    return ar.try_read(name, t, is_buffer);
+}
+}  // namespace
+
+SceneTensors LoadSceneCheckpoint(const std::string& prefix, torch::Device device)
+{
+    SceneTensors st;
+    auto open = [&](const char* file, torch::serialize::InputArchive& ar) {
+        const std::string path = prefix + file;
+        if (!file_exists(path)) return false;
+        ar.load_from(path, device);
+        return true;
+    };
+    {
+        torch::serialize::InputArchive ar;
+        if (open("points.pth", ar))
+        {
+            TORCH_CHECK(read_entry(ar, "t_position", st.t_position, false), "points.pth has no t_position");
+            read_entry(ar, "t_index", st.t_index, true);
+            TORCH_CHECK(st.t_position.scalar_type() == torch::kFloat32 && st.t_position.dim() == 2 && st.t_position.size(1) == 4,
+                        "t_position must be [N,4] float32");
+            TORCH_CHECK(!st.t_index.defined() ||
+                            (st.t_index.scalar_type() == torch::kInt32 && st.t_index.size(0) == st.t_position.size(0)),
+                        "t_index must be [N,1] int32");  // NeuralScene.cpp:357-360
+        }
+    }
+    {
+        torch::serialize::InputArchive ar;
+        if (open("texture.pth", ar))
+        {
+            TORCH_CHECK(read_entry(ar, "texture", st.texture, false), "texture.pth has no texture");
+            TORCH_CHECK(read_entry(ar, "background_color", st.background_color, false), "texture.pth has no background_color");
+            TORCH_CHECK(read_entry(ar, "confidence_value_of_point", st.confidence_value_of_point, false),
+                        "texture.pth has no confidence_value_of_point");
+        }
+    }
+    {
+        torch::serialize::InputArchive ar;
+        if (open("poses.pth", ar))
+        {
+            TORCH_CHECK(read_entry(ar, "tangent_poses", st.tangent_poses, false), "poses.pth has no tangent_poses");
+            TORCH_CHECK(read_entry(ar, "poses_se3", st.poses_se3, true), "poses.pth has no poses_se3");
+            TORCH_CHECK(st.poses_se3.scalar_type() == torch::kFloat64 && st.tangent_poses.scalar_type() == torch::kFloat64,
+                        "poses are float64");  // NeuralScene.cpp:385-386
+        }
+    }
+    {
+        torch::serialize::InputArchive ar;
+        if (open("intrinsics.pth", ar))
+            TORCH_CHECK(read_entry(ar, "intrinsics", st.intrinsics, false), "intrinsics.pth has no intrinsics");
+    }
+    return st;
+}
+
+void SaveSceneCheckpoint(const std::string& prefix, const SceneTensors& st)
+{
+    auto cpu = [](const torch::Tensor& t) { return t.detach().to(torch::kCPU).contiguous(); };
+    if (st.t_position.defined())
+    {
+        torch::serialize::OutputArchive ar;
+        ar.write("t_position", cpu(st.t_position), false);
+        if (st.t_index.defined()) ar.write("t_index", cpu(st.t_index), true);
+        ar.save_to(prefix + "points.pth");
+    }
+    if (st.texture.defined())
+    {
+        TORCH_CHECK(st.background_color.defined() && st.confidence_value_of_point.defined(),
+                    "SaveSceneCheckpoint: texture, background_color and confidence_value_of_point go together");
+        torch::serialize::OutputArchive ar;
+        ar.write("texture", cpu(st.texture), false);
+        ar.write("background_color", cpu(st.background_color), false);
+        ar.write("confidence_value_of_point", cpu(st.confidence_value_of_point), false);
+        ar.save_to(prefix + "texture.pth");
+    }
+    if (st.poses_se3.defined())
+    {
+        TORCH_CHECK(st.tangent_poses.defined(), "SaveSceneCheckpoint: poses_se3 and tangent_poses go together");
+        torch::serialize::OutputArchive ar;
+        ar.write("tangent_poses", cpu(st.tangent_poses), false);
+        ar.write("poses_se3", cpu(st.poses_se3), true);
+        ar.save_to(prefix + "poses.pth");
+    }
+    if (st.intrinsics.defined())
+    {
+        torch::serialize::OutputArchive ar;
+        ar.write("intrinsics", cpu(st.intrinsics), false);
+        ar.save_to(prefix + "intrinsics.pth");
+    }
+}
+
+namespace
+{
 inline uint64_t spread_bits21(uint64_t v)
 {
     v &= 0x1FFFFFull;
@@ -636,6 +738,46 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
                                            intrinsics, loss_img);
         },
         "PointRendererCache::FillSceneGridWithLoss of the reference, with the cell tensors passed one by one");
+    m.def(
+        "save_scene_checkpoint",
+        [](const std::string& prefix, pybind11::dict tensors) {
+            vet_amd::SceneTensors st;
+            for (auto item : tensors)
+            {
+                const std::string k = pybind11::cast<std::string>(item.first);
+                torch::Tensor t     = pybind11::cast<torch::Tensor>(item.second);
+                if (k == "texture") st.texture = t;
+                else if (k == "background_color") st.background_color = t;
+                else if (k == "confidence_value_of_point") st.confidence_value_of_point = t;
+                else if (k == "t_position") st.t_position = t;
+                else if (k == "t_index") st.t_index = t;
+                else if (k == "tangent_poses") st.tangent_poses = t;
+                else if (k == "poses_se3") st.poses_se3 = t;
+                else if (k == "intrinsics") st.intrinsics = t;
+                else TORCH_CHECK(false, "unknown scene tensor ", k);
+            }
+            vet_amd::SaveSceneCheckpoint(prefix, st);
+        },
+        "NeuralScene::SaveCheckpoint of the reference for the tensors the rasterizer reads");
+    m.def(
+        "load_scene_checkpoint",
+        [](const std::string& prefix) {
+            const vet_amd::SceneTensors st = vet_amd::LoadSceneCheckpoint(prefix, torch::kCPU);
+            pybind11::dict d;
+            auto put = [&](const char* k, const torch::Tensor& t) {
+                if (t.defined()) d[k] = t;
+            };
+            put("texture", st.texture);
+            put("background_color", st.background_color);
+            put("confidence_value_of_point", st.confidence_value_of_point);
+            put("t_position", st.t_position);
+            put("t_index", st.t_index);
+            put("tangent_poses", st.tangent_poses);
+            put("poses_se3", st.poses_se3);
+            put("intrinsics", st.intrinsics);
+            return d;
+        },
+        "NeuralScene::LoadCheckpoint of the reference for the tensors the rasterizer reads");
     m.def("morton_block_shuffle_order", &vet_amd::MortonBlockShuffleOrder, pybind11::arg("positions"),
           pybind11::arg("block") = 256, pybind11::arg("seed") = 0,
           "ReorderMorton64 + RandomBlockShuffle(block) of the reference's scene preprocessing, as a permutation");

@@ -10,6 +10,7 @@
 #include <torch/torch.h>
 
 #include <memory>
+#include <string>
 #include <vector>
 
 #include "../../include/vetrast.h"
@@ -168,6 +169,21 @@ class PointRenderModule
     std::pair<std::vector<torch::Tensor>, std::vector<torch::Tensor>> forward(NeuralRenderInfo* nri);
     std::shared_ptr<PointRendererCache> cache;
 };
+
+// VET's scene checkpoints (NeuralScene::SaveCheckpoint / LoadCheckpoint, src/lib/data/NeuralScene.cpp:343-437) are four
+// libtorch module archives, <prefix>points.pth, texture.pth, poses.pth and intrinsics.pth, whose entries carry the names
+// the modules registered their tensors under:
+//   points.pth      parameter "t_position" [N,4] f32, buffer "t_index" [N,1] i32   (src/lib/rendering/NeuralPointCloudCuda.cpp:71-72)
+//   texture.pth     parameters "texture" [C,N], "background_color" [C], "confidence_value_of_point" [1,N]: the RAW tensors
+//                   (before abs / sigmoid)                                          (src/lib/models/NeuralTexture.cpp:45-47)
+//   poses.pth       parameter "tangent_poses" [F,6] f64, buffer "poses_se3" [F,8] f64 (src/lib/data/NeuralStructure.cpp:29-30)
+//   intrinsics.pth  parameter "intrinsics" [Ncam,13] f32                             (src/lib/data/NeuralStructure.cpp:96)
+// These two functions read and write exactly those entries into / from the tensor bundle the rasterizer takes, so a
+// scene trained by VET renders here and the other way round. Entries of the reference's modules that the rasterizer
+// does not read (normals, original colours, cell tensors, the environment map) are neither written nor required; a
+// missing file leaves the corresponding tensors undefined.
+SceneTensors LoadSceneCheckpoint(const std::string& prefix, torch::Device device = torch::kCPU);
+void SaveSceneCheckpoint(const std::string& prefix, const SceneTensors& scene);
 
 // The order VET's scene preprocessing gives a point cloud before the rasterizer ever sees it
 // (point_cloud.ReorderMorton64(); point_cloud.RandomBlockShuffle(256); src/lib/data/SceneData.cpp:105-106): points sorted

@@ -51,3 +51,16 @@ def morton_block_shuffle_order(positions, block=256, seed=0):
     """The point order of the reference's scene preprocessing (ReorderMorton64 + RandomBlockShuffle(256),
     src/lib/data/SceneData.cpp:105-106) as a permutation [N] int64 of a [N,3] or [N,4] CPU tensor of positions."""
     return load().morton_block_shuffle_order(positions, int(block), int(seed))
+
+
+def save_scene_checkpoint(prefix, **tensors):
+    """Writes VET's scene checkpoint files (<prefix>points.pth, texture.pth, poses.pth, intrinsics.pth; the reference's
+    NeuralScene::SaveCheckpoint, src/lib/data/NeuralScene.cpp:407-431) for the given tensors: t_position, t_index,
+    texture, background_color, confidence_value_of_point (the raw tensors), tangent_poses, poses_se3, intrinsics."""
+    load().save_scene_checkpoint(str(prefix), dict(tensors))
+
+
+def load_scene_checkpoint(prefix):
+    """Reads the same files back (NeuralScene::LoadCheckpoint, src/lib/data/NeuralScene.cpp:343-405) as a dict of CPU
+    tensors; files that do not exist leave their tensors out."""
+    return dict(load().load_scene_checkpoint(str(prefix)))
