@@ -703,7 +703,9 @@ __global__ void __launch_bounds__(kBlock) gather_point_gradients_kernel(GatherPa
                                (uint32_t)(y % kTile) * kTile + (uint32_t)(x % kTile);
             // Did the fragment take part in the blend? Only where the pixel's list was not blended to its end (top-K
             // cut, saturation) the last blended key has to be looked up.
-            if (a.list_is_cut[q])
+            // (FULL_BLEND without a cut never sets the flag; the K > 0 test keeps a corrupted flag byte from turning
+            // K <= 0 into an index.)
+            if (a.list_is_cut[q] && (HITS != 1 || a.K > 0))
             {
                 const uint32_t nk  = HITS == 1 ? (uint32_t)a.K : a.kept[q];  // FULL_BLEND: cut means count > K > 0
                 const uint64_t key = depth_key | (HITS == 1 ? (uint32_t)i : (((uint32_t)i << 2) | (uint32_t)h));
