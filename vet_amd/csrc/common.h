@@ -212,12 +212,17 @@ __device__ __forceinline__ float4 pair_other(float4 v)
 // XCD's run of regions (region r goes to XCD r % 8): what one layer's tiles pulled into the XCD's L2 is still there
 // when the next layer's tiles of the region ask for the same points.
 constexpr int kXcds = 8;
+// A layer whose pixels hold long lists is split: a workgroup then owns one 16x4 strip of a tile and each of its waves
+// one row of 16 pixels (lanes 16..63 carry no pixel, only fragments), so that such a layer (few pixels, many fragments)
+// is spread over four times as many waves, each with a quarter of the rounds to run one after the other.
 struct TileMap
 {
     int L;
     uint32_t regions_x, regions;     // region grid (regions per row, total)
     uint32_t tiles_per_region;       // (4^L - 1) / 3
     uint32_t regions_per_xcd;        // ceil(regions / 8)
+    uint32_t split[VETRAST_MAX_LAYERS];  // workgroups per tile of the layer: 1, or 4 (one per 16x4 strip)
+    uint32_t groups_per_region;      // sum over the layers of (tiles of the layer in a region) x split
 };
 
 struct TilePixel
@@ -237,25 +242,34 @@ __device__ __forceinline__ TilePixel tile_pixel(const TileMap& tm, const LayerTa
     const uint32_t b      = blockIdx.x;
     const uint32_t xcd    = b % kXcds;
     const uint32_t slot   = b / kXcds;
-    const uint32_t region = (slot / tm.tiles_per_region) * kXcds + xcd;
-    uint32_t t            = slot % tm.tiles_per_region;  // tile inside the region, coarsest layer first
+    const uint32_t region = (slot / tm.groups_per_region) * kXcds + xcd;
+    uint32_t t            = slot % tm.groups_per_region;  // workgroup inside the region, coarsest layer first
     if (region >= tm.regions) return r;
-    // layer L-1 has 1 tile per region, L-2 has 4, L-3 has 16, ...
+    // layer L-1 has 1 tile per region, L-2 has 4, L-3 has 16, ...; split[l] workgroups per tile
     int l          = tm.L - 1;
     uint32_t side  = 1;  // tiles per region side in layer l
-    while (t >= side * side)
+    while (t >= side * side * tm.split[l])
     {
-        t -= side * side;
+        t -= side * side * tm.split[l];
         side <<= 1;
         --l;
     }
+    const uint32_t strip = t % tm.split[l];  // 16x4 strip of the tile, if the layer is split
+    t /= tm.split[l];
     const uint32_t ry = region / tm.regions_x, rx = region - ry * tm.regions_x;
     const uint32_t ty = ry * side + t / side, tx = rx * side + (t & (side - 1));
     r.l = l;
     if (tx >= (uint32_t)ly.tiles_x[l] || ty >= (uint32_t)ly.tiles_y[l]) return r;
-    r.x = (int)(tx * kTile + (threadIdx.x & (kTile - 1)));
-    r.y = (int)(ty * kTile + (threadIdx.x / kTile));
-    r.q = (ly.tile_base[l] + ty * (uint32_t)ly.tiles_x[l] + tx) * kTilePixels + threadIdx.x;
+    uint32_t in_tile = threadIdx.x;  // 16 * (row of the tile) + column
+    if (tm.split[l] != 1)
+    {
+        const uint32_t lane = threadIdx.x & (kWave - 1);
+        if (lane >= (uint32_t)kTile) return r;  // this lane carries no pixel
+        in_tile = (strip * 4 + threadIdx.x / kWave) * kTile + lane;
+    }
+    r.x = (int)(tx * kTile + (in_tile & (kTile - 1)));
+    r.y = (int)(ty * kTile + (in_tile / kTile));
+    r.q = (ly.tile_base[l] + ty * (uint32_t)ly.tiles_x[l] + tx) * kTilePixels + in_tile;
     if (r.x >= ly.w[l] || r.y >= ly.h[l]) return r;
     r.local  = (uint32_t)r.y * (uint32_t)ly.w[l] + (uint32_t)r.x;
     r.active = true;

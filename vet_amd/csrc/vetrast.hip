@@ -41,6 +41,7 @@ struct vetrast_ctx
 namespace
 {
 constexpr size_t kAlign = 256;
+constexpr double kSplitListLength = 8.0;  // layers that blend at least this many fragments per pixel are split
 inline size_t align_up(size_t v, size_t a)
 {
     return (v + a - 1) / a * a;
@@ -209,11 +210,15 @@ inline T* ws_ptr(void* ws, size_t off)
     return reinterpret_cast<T*>(static_cast<char*>(ws) + off);
 }
 
-TileMap make_tile_map(const LayerTable& ly)
+// `list_bound[l]`: an upper bound of the mean number of fragments a pixel of layer l blends (null: no layer is split;
+// `split_all`: every layer is, which is what buffers are sized for).
+TileMap make_tile_map(const LayerTable& ly, const double* list_bound = nullptr, bool split_all = false)
 {
     TileMap m;
     std::memset(&m, 0, sizeof(m));
     m.L = ly.L;
+    for (int l = 0; l < VETRAST_MAX_LAYERS; ++l)
+        m.split[l] = (split_all || (list_bound && l < ly.L && list_bound[l] >= kSplitListLength)) ? 4u : 1u;
     // a region is one 16x16 tile of the coarsest layer; over the finer layers it covers (16 << k)^2 pixels. Layer sizes
     // come from integer halving, so the finest layer can be a few pixels larger than 2^(L-1) times the coarsest one:
     // size the region grid from the finest layer.
@@ -224,12 +229,14 @@ TileMap make_tile_map(const LayerTable& ly)
     for (int k = 0; k < ly.L; ++k) tiles += 1u << (2 * k);
     m.tiles_per_region = tiles;
     m.regions_per_xcd  = (m.regions + kXcds - 1) / kXcds;
+    m.groups_per_region = 0;
+    for (int l = 0; l < ly.L; ++l) m.groups_per_region += (1u << (2 * (ly.L - 1 - l))) * m.split[l];
     return m;
 }
 
 uint32_t tile_grid(const TileMap& m)
 {
-    return m.regions_per_xcd * m.tiles_per_region * kXcds;
+    return m.regions_per_xcd * m.groups_per_region * kXcds;
 }
 
 ViewPass make_view_pass(const vetrast_forward_args* a, const vetrast_workspace_layout& lay, const LayerTable& ly, int b)
@@ -376,7 +383,7 @@ int vetrast_workspace_layout_for_mode(int32_t N, int32_t B, int32_t L, int32_t w
     lay->partial_base       = at;
     at += align_up(cap * 8 * sizeof(float), kAlign);
     lay->background_partial_base = at;
-    at += align_up((size_t)tile_grid(make_tile_map(t)) * kBackgroundRow * sizeof(float), kAlign);
+    at += align_up((size_t)tile_grid(make_tile_map(t, nullptr, true)) * kBackgroundRow * sizeof(float), kAlign);
     lay->camera_partial_base = at;
     at += align_up(((size_t)N + kBlock - 1) / kBlock * kCameraRow * sizeof(double), kAlign);
     lay->total_bytes = align_up(at, kAlign);
@@ -584,7 +591,16 @@ int vetrast_backward(vetrast_ctx* ctx, const vetrast_backward_args* g, void* str
     const int N = a->num_points, B = a->num_views, L = p.num_layers, C = p.num_texture_channels;
     const int hits      = hits_of_mode(p.render_mode);
     const LayerTable ly = make_layer_table(a->views[0].w, a->views[0].h, L, (int64_t)N * hits);
-    const TileMap tiles = make_tile_map(ly);
+    // fragments a pixel of layer l blends, bounded from above without a device read: all points land in the layer, the
+    // top-K cut
+    double list_bound[VETRAST_MAX_LAYERS] = {};
+    for (int l = 0; l < L; ++l)
+    {
+        list_bound[l] = (double)N * hits / ((double)ly.w[l] * ly.h[l]);
+        if (p.debug_max_list_length > 0) list_bound[l] = std::min(list_bound[l], (double)p.debug_max_list_length);
+    }
+    // (the FUZZY_BLEND kernel walks a pixel's list in one thread and wants every lane to carry a pixel)
+    const TileMap tiles = make_tile_map(ly, p.render_mode == VETRAST_RENDER_FUZZY_BLEND ? nullptr : list_bound);
     void* ws            = a->workspace;
 
     // The per-point kernel overwrites every gradient row in the first view, so the zeros_like fills of
