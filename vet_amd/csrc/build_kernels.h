@@ -130,6 +130,56 @@ struct FuzzyBucket
     }
 };
 
+// Sorts list[0, n), n <= kBuildCap, by the whole workgroup through the LDS room `room` (kBuildCap keys). Copy in (padded
+// with +infinity to a power of two), every wave sorts 64-key chunks in registers, then the chunks are merged pairwise,
+// level by level, in the all-ascending form of the bitonic network: a mirror step and the halving steps over 64 or more
+// places run on LDS with a barrier each, the last six halving steps of every level again in registers. A list of 512
+// keys takes 13 barriers instead of the 45 of the plain network. Every thread of the workgroup must call.
+__device__ __forceinline__ void block_sort_in_lds(uint64_t* list, uint32_t n, uint64_t* room, int tid)
+{
+    const int lane = tid & (kWave - 1), wave = tid / kWave;
+    uint32_t m = kWave;
+    while (m < n) m <<= 1;  // <= kBuildCap
+    for (uint32_t k = tid; k < m; k += kBlock) room[k] = k < n ? list[k] : kInfKey;
+    __syncthreads();
+    const uint32_t chunks = m / kWave;
+    for (uint32_t c = wave; c < chunks; c += kBlock / kWave)
+        room[c * kWave + lane] = bitonic_sort_groups<6>(room[c * kWave + lane], lane);
+    __syncthreads();
+    auto order = [&](uint32_t i, uint32_t j) {  // i < j: the smaller key to place i
+        const uint64_t x = room[i], y = room[j];
+        if (y < x)
+        {
+            room[i] = y;
+            room[j] = x;
+        }
+    };
+    for (uint32_t k = 2 * kWave; k <= m; k <<= 1)
+    {
+        const uint32_t hk = k >> 1;
+        for (uint32_t p = tid; p < (m >> 1); p += kBlock)  // mirror step inside every block of k places
+        {
+            const uint32_t blk = p / hk, r = p % hk;
+            order(blk * k + r, blk * k + (k - 1 - r));
+        }
+        __syncthreads();
+        for (uint32_t jj = k >> 2; jj >= (uint32_t)kWave; jj >>= 1)
+        {
+            for (uint32_t p = tid; p < (m >> 1); p += kBlock)
+            {
+                const uint32_t i = (p / jj) * 2 * jj + (p % jj);
+                order(i, i + jj);
+            }
+            __syncthreads();
+        }
+        for (uint32_t c = wave; c < chunks; c += kBlock / kWave)
+            room[c * kWave + lane] = bitonic_merge64(room[c * kWave + lane], lane);
+        __syncthreads();
+    }
+    for (uint32_t k = tid; k < n; k += kBlock) list[k] = room[k];
+    __syncthreads();
+}
+
 template <int C, bool BILINEAR, bool FUZZY = false>
 __global__ void __launch_bounds__(kBlock) bin_build_kernel(BuildPass a)
 {
@@ -138,6 +188,7 @@ __global__ void __launch_bounds__(kBlock) bin_build_kernel(BuildPass a)
     __shared__ uint32_t s_prefix[kTilePixels];
     __shared__ uint32_t s_wave_tot[kBlock / kWave];
     __shared__ uint8_t s_src_lane[kBlock / kWave][kWave];
+    __shared__ uint64_t s_block_sorted[kBlock / kWave];  // pixels whose lists the whole workgroup sorts, a mask per wave
     __shared__ uint64_t s_keys[kBuildCap];
     __shared__ uint32_t s_used[kTilePixels];   // fragments of the pixel that took part in the blend
     __shared__ uint8_t s_pix[kBuildCap];       // pixel (inside the bin) of every list place
@@ -352,10 +403,98 @@ __global__ void __launch_bounds__(kBlock) bin_build_kernel(BuildPass a)
         }
         __threadfence_block();  // the keys other waves stored are read below
         __syncthreads();
-        sort_wave_lists(a.fragments + begin, s_src_lane[wave], list_off, list_len, lane, a.K);
+        // Lists that have to be sorted in full and are too long for a wave's registers are sorted by the whole
+        // workgroup through the key array in LDS, which is not in use on this path, one list after the other (in global
+        // memory every step of the network costs a memory round trip, and such a list needs dozens of steps).
+        const bool full_sort = !(a.K > 0 && a.K <= kWave);
+        sort_wave_lists(a.fragments + begin, s_src_lane[wave], list_off, list_len, lane, a.K,
+                        /*skip_longer=*/(uint32_t)kBuildCap);
         __threadfence_block();
         __syncthreads();
-        if ((uint32_t)tid < pixels)
+        if (full_sort)
+        {
+            const bool mine = (uint32_t)tid < pixels && c > kRegisterSortKeys && c <= (uint32_t)kBuildCap;  // pixel tid
+            const uint64_t wave_mask = __ballot(mine);
+            if (lane == 0) s_block_sorted[wave] = wave_mask;
+            __syncthreads();
+            for (int w = 0; w < kBlock / kWave; ++w)  // the same trips for every thread
+            {
+                uint64_t todo = s_block_sorted[w];
+                while (todo != 0ull)
+                {
+                    const uint32_t px = w * kWave + (__ffsll((unsigned long long)todo) - 1);
+                    todo &= todo - 1ull;
+                    block_sort_in_lds(a.fragments + begin + s_prefix[px], s_cnt[px], s_keys, tid);
+                }
+            }
+        }
+        __threadfence_block();
+        __syncthreads();
+        if (a.K <= 0 && n > 16u * pixels)
+        {
+            // Without a cut the lists of a streamed bin of few pixels run to hundreds of fragments. One thread walking such a list
+            // with a memory round trip every few fragments would hold the whole workgroup up, so the bin is blended
+            // like one in LDS: all threads gather the descriptor records of a stretch of list places into the stage,
+            // then the pixel's thread walks its fragments of that stretch. Keys come from the fragment buffer and the
+            // transmittances go straight to memory.
+            const uint64_t* list_mem = a.fragments + begin;
+            for (uint32_t base = 0; base < n; base += kStage)
+            {
+#pragma unroll
+                for (int k = 0; k < (kStage + kBlock - 1) / kBlock; ++k)
+                {
+                    const uint32_t r = base + k * kBlock + tid;
+                    if (k * kBlock + tid >= kStage || r >= n) continue;
+                    const uint64_t k64 = list_mem[r];
+                    const uint32_t low = (uint32_t)k64;
+                    const int id       = BILINEAR ? (int)(low >> 2) : (int)low;
+                    int ti             = -1;
+                    if ((uint32_t)id < (uint32_t)a.N) ti = a.index ? a.index[id] : id;
+                    float4 t4 = make_float4(0.f, 0.f, 0.f, 0.f), c4 = t4;
+                    if ((uint32_t)ti < (uint32_t)a.N)
+                    {
+                        t4   = a.packed[2 * (size_t)ti];
+                        c4   = a.packed[2 * (size_t)ti + 1];
+                        c4.x = fragment_alpha<BILINEAR>(a, l, low, c4.x);
+                    }
+                    if constexpr (FUZZY) c4.y = __uint_as_float((uint32_t)(k64 >> 32));
+                    s_stage[r - base][0] = t4;
+                    s_stage[r - base][1] = c4;
+                }
+                __syncthreads();
+                if ((uint32_t)tid < pixels)
+                {
+                    const uint32_t lo = max(start, base), hi = min(start + keep, base + (uint32_t)kStage);
+                    for (uint32_t r = lo; r < hi && !saturated; ++r)
+                    {
+                        const float4 t4 = s_stage[r - base][0];
+                        const float2 cd = *reinterpret_cast<const float2*>(&s_stage[r - base][1]);  // confidence, depth
+                        const float cf  = cd.x;
+                        const float t[4] = {t4.x, t4.y, t4.z, t4.w};
+                        if constexpr (FUZZY)
+                        {
+                            if (fuzzy.open && fuzzy.take(cd.y, cf, t, a.depth_accept, T, color))
+                            {
+                                if (a.transmittance) a.transmittance[begin + r] = T;
+                                ++used;
+                                continue;
+                            }
+                        }
+                        if (a.transmittance) a.transmittance[begin + r] = T;
+                        const float Tc = T * cf;
+#pragma unroll
+                        for (int ci = 0; ci < C; ++ci) color[ci] = Tc * t[ci] + color[ci];
+                        T = (1.f - cf) * T;
+                        ++used;
+                        saturated = blend_is_saturated<BILINEAR>(T);
+                    }
+                }
+                __syncthreads();
+            }
+            if constexpr (FUZZY)
+                if (fuzzy.open && fuzzy.m > 0) fuzzy.flush(T, color);
+        }
+        else if ((uint32_t)tid < pixels)
         {
             if constexpr (FUZZY)
             {

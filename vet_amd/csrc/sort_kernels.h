@@ -188,10 +188,69 @@ __device__ __forceinline__ void sort_in_memory(uint64_t* list, uint32_t n, int l
     }
 }
 
+// Sorts a list of 64 < n <= 64 * CH keys by one wave with the keys in registers, CH keys per lane (chunk q holds places
+// 64 q .. 64 q + 63; places beyond n act as +infinity). Every chunk is sorted by the 64-lane network, then chunks are
+// merged pairwise, level by level, in the all-ascending form of the bitonic network: the mirror step and the halving
+// steps over 64 or more places pair whole chunks register against register (the mirror step with the partner chunk
+// reversed across the wave), the last six halving steps of a level run inside every chunk. One load and one store per key.
+template <int CH>
+__device__ __forceinline__ void sort_in_registers(uint64_t* list, uint32_t n, int lane)
+{
+    uint64_t c[CH];
+#pragma unroll
+    for (int q = 0; q < CH; ++q)
+    {
+        const uint32_t idx = q * kWave + lane;
+        c[q]               = idx < n ? list[idx] : kInfKey;
+    }
+#pragma unroll
+    for (int q = 0; q < CH; ++q) c[q] = bitonic_sort_groups<6>(c[q], lane);
+    auto reversed = [&](uint64_t v) {
+        const uint32_t lo = lane_xor<63>((uint32_t)v, lane), hi = lane_xor<63>((uint32_t)(v >> 32), lane);
+        return ((uint64_t)hi << 32) | lo;
+    };
+#pragma unroll
+    for (int w = 2; w <= CH; w <<= 1)  // w chunks per block of this level
+    {
+#pragma unroll
+        for (int q = 0; q < CH; ++q)
+            if ((q % w) < w / 2)
+            {
+                const int p        = q - (q % w) + (w - 1 - (q % w));
+                const uint64_t r   = reversed(c[p]);
+                const uint64_t mn  = r < c[q] ? r : c[q], mx = r < c[q] ? c[q] : r;
+                c[q]               = mn;
+                c[p]               = reversed(mx);
+            }
+#pragma unroll
+        for (int d = w / 4; d >= 1; d >>= 1)
+#pragma unroll
+            for (int q = 0; q < CH; ++q)
+                if ((q & d) == 0)
+                {
+                    const uint64_t x = c[q], y = c[q + d];
+                    c[q]             = y < x ? y : x;
+                    c[q + d]         = y < x ? x : y;
+                }
+#pragma unroll
+        for (int q = 0; q < CH; ++q) c[q] = bitonic_merge64(c[q], lane);
+    }
+#pragma unroll
+    for (int q = 0; q < CH; ++q)
+    {
+        const uint32_t idx = q * kWave + lane;
+        if (idx < n) list[idx] = c[q];
+    }
+}
+
+constexpr uint32_t kRegisterSortKeys = 256;  // longest list sort_wave_lists sorts in registers
+
 // Sorts the lists of one wave: lane i holds the start `off` (an index into `fragments`) and the length `n` of its list
-// (n = 0 for lanes without a list). `fragments` may point to global memory or to LDS.
+// (n = 0 for lanes without a list). `fragments` may point to global memory or to LDS. Lists that have to be sorted in
+// full and hold more than kRegisterSortKeys and up to `skip_longer` keys are left alone: the caller sorts them by other
+// means.
 __device__ __forceinline__ void sort_wave_lists(uint64_t* fragments, uint8_t* src_lane, uint32_t off, uint32_t n,
-                                                int lane, int K)
+                                                int lane, int K, uint32_t skip_longer = 0)
 {
     // class = ceil(log2(n)) for 2 <= n <= 64, 0 for n <= 1 (nothing to do), 7 for n > 64
     int cls = 0;
@@ -234,6 +293,12 @@ __device__ __forceinline__ void sort_wave_lists(uint64_t* fragments, uint8_t* sr
         const uint32_t nn = __shfl(n, src, kWave);
         if (K > 0 && K <= kWave)
             select_smallest(fragments + o, nn, lane, K);
+        else if (nn <= 2 * kWave)
+            sort_in_registers<2>(fragments + o, nn, lane);
+        else if (nn <= kRegisterSortKeys)
+            sort_in_registers<4>(fragments + o, nn, lane);
+        else if (nn <= skip_longer)
+            continue;  // the caller sorts lists of this length with the whole workgroup
         else
             sort_in_memory(fragments + o, nn, lane);
     }
