@@ -196,3 +196,43 @@ def test_more_views_than_one_preparation_launch_holds(rasterizer, oracle):
     torch.cuda.synchronize()
     for key in ("texture", "confidence", "background", "points", "pose"):
         assert max_rel_err(got[key].cpu().numpy(), want[key]) <= 1e-4, key
+
+
+_LENGTHS_IN_ONE_SMALL_BIN = [1, 2, 63, 64, 65, 127, 128, 129]   # 579 keys: the bin is built in LDS
+_LENGTHS_IN_ONE_FULL_BIN = [200, 255, 256, 257]                  # 968 keys, still in LDS, one list beyond a wave's registers
+_LENGTHS_APART = [300, 511, 512, 513, 700, 1023, 1024, 1025, 1500, 4097]  # each makes its bin stream from memory
+
+
+@pytest.mark.parametrize("K", [0, 100, 16])
+@pytest.mark.parametrize("mode", [abi.RENDER_FULL_BLEND, abi.RENDER_FUZZY_BLEND])
+def test_list_lengths_around_every_sorting_limit(K, mode, rasterizer, oracle):
+    """Pixels that receive exactly 63, 64, 65, ..., 1025, 4097 points: one length either side of every limit between
+    the sorting methods (one wave's network, two or four keys per lane in registers, the workgroup's sort in LDS, the
+    in-place sort in memory), in bins built in LDS and in bins streamed from memory. A quarter of the points share their
+    depth with another point of the same pixel, so the order inside ties is checked as well."""
+    print(f"[case] list lengths around the sorting limits K={K} mode={mode}", flush=True)
+    w, h = 64, 32
+    where = [((2 + i, 1), n) for i, n in enumerate(_LENGTHS_IN_ONE_SMALL_BIN)]
+    where += [((34 + i, 17), n) for i, n in enumerate(_LENGTHS_IN_ONE_FULL_BIN)]
+    where += [((4 + 6 * (i % 5) + 32 * (i // 5 % 2), 9 + 16 * (i // 5 % 2)), n) for i, n in enumerate(_LENGTHS_APART)]
+    total = sum(n for _, n in where)
+    scene = synthetic.tiny_scene(num_points=total, w=w, h=h, num_layers=1, K=K, seed=97)
+    rng = np.random.default_rng(97)
+    fx, cx, cy = 0.45 * w, w / 2.0, h / 2.0
+    first = 0
+    for (px, py), n in where:
+        z = rng.uniform(-0.4, 1.4, size=n)
+        z[n // 4 * 3:] = z[: n - n // 4 * 3]           # depth ties inside the list
+        z = z.astype(np.float32).astype(np.float64)
+        scene.position[first:first + n, 0] = ((px - cx) * (z + 2.0) / fx).astype(np.float32)
+        scene.position[first:first + n, 1] = ((py - cy) * (z + 2.0) / fx).astype(np.float32)
+        scene.position[first:first + n, 2] = z.astype(np.float32)
+        first += n
+    order = rng.permutation(total)                     # list places do not follow the point order
+    scene.position = np.ascontiguousarray(scene.position[order])
+    res, ref, _ = _parity(scene, rasterizer, oracle, backward=(K > 0), need_point_gradient=1, render_mode=mode,
+                          depth_accept_blend=0.05)
+    counts = np.diff(res.offsets(0)).reshape(h, w)
+    for (px, py), n in where:
+        assert counts[py, px] == n, (px, py, n, counts[py, px])
+    assert counts.sum() == total
