@@ -191,6 +191,11 @@ typedef struct vetrast_forward_args
     float* out_mask[VETRAST_MAX_LAYERS]; /* device, layer l: [B,1,h_l,w_l]; only with output_background_mask */
     void* workspace;                     /* device, 256-byte aligned */
     size_t workspace_bytes;
+    /* Optional, layer l: device [B,1,h_l,w_l], the transmittance left behind the last blended fragment of every pixel
+     * (1 where no point landed): the `weight` tensor of the reference's layer cache
+     * (src/lib/rendering/RenderForward.cu:1355-1356), which PointRenderModuleImpl::forward hands to the environment map
+     * (src/lib/rendering/RenderModule.cpp:132-196). NULL = not wanted. */
+    float* out_weight[VETRAST_MAX_LAYERS];
 } vetrast_forward_args;
 
 /* Arguments of the backward pass. Replaces BlendPointCloudBackward's inputs and its seven returned tensors

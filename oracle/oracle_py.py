@@ -29,6 +29,10 @@ def load():
         if not os.path.exists(LIB_PATH):
             raise OSError(f"{LIB_PATH} is missing: run `make -C oracle`")
         lib = C.CDLL(LIB_PATH)
+        sizes = (C.c_uint64 * 4)()
+        mirrors = [C.sizeof(t) for t in (abi.ForwardArgs, abi.BackwardArgs, abi.AdamArgs, abi.LiftArgs)]
+        if not hasattr(lib, "vetref_struct_sizes") or lib.vetref_struct_sizes(sizes) != 0 or list(sizes) != mirrors:
+            raise OSError(f"{LIB_PATH} was built from another version of include/vetrast.h: run `make -C oracle`")
         lib.vetref_forward.restype = C.c_int
         lib.vetref_forward.argtypes = [C.POINTER(abi.ForwardArgs), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
                                        C.c_void_p, C.c_int]

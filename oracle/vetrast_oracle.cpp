@@ -1129,6 +1129,15 @@ extern "C" int vetref_backward(const vetrast_backward_args* g, const uint32_t* o
 }
 
 // torch::sigmoid(scale * x) in the canonical arithmetic (exposed so that tests can pin it against a float64 logistic).
+extern "C" int vetref_struct_sizes(uint64_t sizes[4])
+{
+    sizes[0] = sizeof(vetrast_forward_args);
+    sizes[1] = sizeof(vetrast_backward_args);
+    sizes[2] = sizeof(vetrast_adam_args);
+    sizes[3] = sizeof(vetrast_lift_args);
+    return 0;
+}
+
 extern "C" int vetref_sigmoid(const float* x, float* y, int64_t n, float scale)
 {
     for (int64_t i = 0; i < n; ++i) y[i] = sigmoid_canon(scale * x[i]);

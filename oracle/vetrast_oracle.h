@@ -79,6 +79,10 @@ int vetref_adam_step(const vetrast_adam_args* args);
 /* Error lifting on host arrays (FillSceneGridWithLossRasterize); the workspace is ignored. */
 int vetref_lift_error(const vetrast_lift_args* args, int num_threads);
 
+/* Sizes of the argument structs this library was compiled with (forward, backward, adam, lift arguments): lets a
+ * caller that mirrors them notice a library built from an older header instead of reading past a struct. */
+int vetref_struct_sizes(uint64_t sizes[4]);
+
 #ifdef __cplusplus
 }
 #endif

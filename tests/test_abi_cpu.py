@@ -37,6 +37,37 @@ def test_struct_sizes_are_the_c_ones():
     assert abi.BackwardArgs.grad_out.offset == C.sizeof(abi.ForwardArgs)
 
 
+def test_every_struct_field_sits_where_the_c_compiler_puts_it(tmp_path):
+    """Compiles include/vetrast.h with gcc and compares size and every field offset of every struct with the ctypes
+    mirror in vet_amd/abi.py (field names are the same on both sides)."""
+    import subprocess
+
+    pairs = [("vetrast_view", abi.View), ("vetrast_params", abi.Params), ("vetrast_workspace_layout", abi.WorkspaceLayout),
+             ("vetrast_forward_args", abi.ForwardArgs), ("vetrast_backward_args", abi.BackwardArgs),
+             ("vetrast_adam_args", abi.AdamArgs), ("vetrast_lift_args", abi.LiftArgs)]
+    lines = ['#include <stdio.h>', '#include <stddef.h>', '#include "vetrast.h"', 'int main(void) {']
+    for cname, mirror in pairs:
+        lines.append(f'printf("{cname} size %zu\\n", sizeof({cname}));')
+        for field, _ in mirror._fields_:
+            lines.append(f'printf("{cname} {field} %zu\\n", offsetof({cname}, {field}));')
+    lines += ['return 0; }']
+    src = tmp_path / "layout.c"
+    src.write_text("\n".join(lines))
+    exe = tmp_path / "layout"
+    subprocess.run(["gcc", "-std=c99", "-I", os.path.join(ROOT, "include"), str(src), "-o", str(exe)], check=True)
+    got = {}
+    for line in subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.splitlines():
+        cname, field, value = line.split()
+        got[(cname, field)] = int(value)
+    for cname, mirror in pairs:
+        assert got[(cname, "size")] == C.sizeof(mirror), cname
+        for field, _ in mirror._fields_:
+            assert got[(cname, field)] == getattr(mirror, field).offset, (cname, field)
+        # the sizes agree and the last mirrored field ends inside the struct: no member of the C struct is missing
+        last, last_type = mirror._fields_[-1]
+        assert getattr(mirror, last).offset + C.sizeof(last_type) <= C.sizeof(mirror)
+
+
 def test_layer_sizes_halve_with_integer_division():
     lib = abi.load_library()
     w = (C.c_int32 * 5)()

@@ -9,7 +9,7 @@ import pytest
 import torch
 
 from tests.helpers import kept_mask, max_rel_err
-from vet_amd import synthetic
+from vet_amd import abi, synthetic
 from vet_amd.rasterizer import DeviceScene, make_params
 
 pytestmark = pytest.mark.gpu
@@ -172,3 +172,21 @@ def test_camera_gradients_without_point_gradient_buffer(rasterizer, oracle):
     torch.cuda.synchronize()
     assert max_rel_err(got["pose"].cpu().numpy(), want["pose"]) <= GRAD_TOL
     assert max_rel_err(got["intrinsics"].cpu().numpy(), want["intrinsics"]) <= GRAD_TOL
+
+
+@pytest.mark.parametrize("mode", [abi.RENDER_FULL_BLEND, abi.RENDER_FUZZY_BLEND, abi.RENDER_BILINEAR_BLEND])
+def test_per_pixel_weight_output(mode, rasterizer, oracle):
+    """The optional out_weight tensors: the transmittance behind the last blended fragment of every pixel in image order
+    (the `weight` tensor of the reference's layer cache), 1 where no point landed, for every view and layer."""
+    print(f"[case] per-pixel weight output mode={mode}", flush=True)
+    scene = synthetic.tiny_scene(num_points=2500, K=6, seed=71, w=37, h=21, num_layers=3, num_views=2)
+    scene.confidence[::4] = 1.0
+    params = make_params(scene, render_mode=mode, depth_accept_blend=0.05)
+    ref = oracle.forward(scene, params)
+    res = rasterizer.forward(DeviceScene(scene), params, want_weight=True)
+    torch.cuda.synchronize()
+    assert res.out_weight is not None and len(res.out_weight) == scene.num_layers
+    for b in range(len(scene.views)):
+        got = np.concatenate([w[b].cpu().numpy().ravel() for w in res.out_weight])
+        np.testing.assert_array_equal(got, ref.weight[b])
+        assert (got == 1.0).any() and (got < 1.0).any()

@@ -146,6 +146,7 @@ class ForwardArgs(C.Structure):
         ("out_mask", C.c_void_p * MAX_LAYERS),
         ("workspace", C.c_void_p),
         ("workspace_bytes", C.c_size_t),
+        ("out_weight", C.c_void_p * MAX_LAYERS),
     ]
 
 

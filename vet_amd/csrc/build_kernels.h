@@ -46,6 +46,7 @@ struct BuildPass
     float* weight;         // per pixel
     float* out[VETRAST_MAX_LAYERS];       // already offset to this view
     float* out_mask[VETRAST_MAX_LAYERS];  // already offset to this view, or null
+    float* out_weight[VETRAST_MAX_LAYERS];  // the same
     LayerTable ly;
     uint32_t num_bins;
     int N;
@@ -585,6 +586,7 @@ __global__ void __launch_bounds__(kBlock) bin_build_kernel(BuildPass a)
             }
             a.weight[q] = T;
             if (a.out_mask[l]) a.out_mask[l][local] = (T == 0.f) ? a.mask_value : 1.f;
+            if (a.out_weight[l]) a.out_weight[l][local] = T;
         }
     }
 }

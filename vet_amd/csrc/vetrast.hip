@@ -506,14 +506,17 @@ int vetrast_forward(vetrast_ctx* ctx, const vetrast_forward_args* a, void* strea
         }
         float* out[VETRAST_MAX_LAYERS];
         float* out_mask[VETRAST_MAX_LAYERS];
+        float* out_weight[VETRAST_MAX_LAYERS];
         for (int l = 0; l < VETRAST_MAX_LAYERS; ++l)
         {
-            out[l]      = nullptr;
-            out_mask[l] = nullptr;
+            out[l]        = nullptr;
+            out_mask[l]   = nullptr;
+            out_weight[l] = nullptr;
             if (l >= L) continue;
             const size_t plane = (size_t)ly.w[l] * ly.h[l];
             out[l]             = a->out[l] + (size_t)b * C * plane;
             if (p.output_background_mask) out_mask[l] = a->out_mask[l] + (size_t)b * plane;
+            if (a->out_weight[l]) out_weight[l] = a->out_weight[l] + (size_t)b * plane;
         }
         if (b == 0 && N > 0) VET_HIP(ctx, hipStreamWaitEvent(stream, ctx->joined, 0));
         {
@@ -539,7 +542,8 @@ int vetrast_forward(vetrast_ctx* ctx, const vetrast_forward_args* a, void* strea
             bp.use_environment_map = p.use_environment_map;
             bp.mask_value          = p.output_background_mask_value;
             bp.depth_accept        = p.depth_accept_blend;
-            for (int l = 0; l < VETRAST_MAX_LAYERS; ++l) bp.out[l] = out[l], bp.out_mask[l] = out_mask[l];
+            for (int l = 0; l < VETRAST_MAX_LAYERS; ++l)
+                bp.out[l] = out[l], bp.out_mask[l] = out_mask[l], bp.out_weight[l] = out_weight[l];
             const dim3 g(bins), blk(kBlock);
             if (p.render_mode == VETRAST_RENDER_FUZZY_BLEND)
                 switch (C)

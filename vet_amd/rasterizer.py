@@ -88,6 +88,7 @@ class ForwardResult:
     layout: abi.WorkspaceLayout
     args: abi.ForwardArgs
     keep: tuple  # objects that must outlive `args`
+    out_weight: Optional[List[torch.Tensor]] = None  # [B,1,h,w] per layer, only with want_weight
 
     def _view_array(self, base, stride, b, dtype, count):
         nbytes = count * torch.empty((), dtype=dtype).element_size()
@@ -224,7 +225,7 @@ class Rasterizer:
         return lay
 
     def forward(self, dev: DeviceScene, params: abi.Params = None, save_for_backward=True, workspace=None,
-                out=None) -> ForwardResult:
+                out=None, want_weight=False) -> ForwardResult:
         scene = dev.scene
         params = params or make_params(scene)
         lay = self.layout(scene, params.render_mode)
@@ -244,10 +245,15 @@ class Rasterizer:
         for l in range(len(sizes)):
             args.out[l] = out[l].data_ptr()
             args.out_mask[l] = masks[l].data_ptr() if masks[l] is not None else None
+        weights = None
+        if want_weight:
+            weights = [torch.empty((B, 1, h, w), dtype=torch.float32, device=dev.device) for (w, h) in sizes]
+            for l in range(len(sizes)):
+                args.out_weight[l] = weights[l].data_ptr()
         args.workspace = workspace.data_ptr()
         args.workspace_bytes = workspace.numel()
         abi.check(self.lib.vetrast_forward(self.ctx, C.byref(args), self._stream()), "forward")
-        return ForwardResult(out, masks, workspace, lay, args, (views, dev, params))
+        return ForwardResult(out, masks, workspace, lay, args, (views, dev, params), weights)
 
     def backward(self, fwd: ForwardResult, grad_out: List[torch.Tensor], want_points=True, want_cameras=False,
                  **param_overrides):

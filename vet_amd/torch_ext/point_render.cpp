@@ -235,6 +235,15 @@ torch::autograd::variable_list PointRender::forward(torch::autograd::AutogradCon
             a.out_mask[l] = mask[l].data_ptr<float>();
         }
     }
+    if (info->cache->keep_layer_weights)
+    {
+        info->cache->layer_weights.resize(L);
+        for (int l = 0; l < L; ++l)
+        {
+            info->cache->layer_weights[l] = torch::empty({B, 1, lay.layer_h[l], lay.layer_w[l]}, f32);
+            a.out_weight[l]               = info->cache->layer_weights[l].data_ptr<float>();
+        }
+    }
     a.workspace         = workspace.data_ptr();
     a.workspace_bytes   = (size_t)workspace.numel();
     a.save_for_backward = need_backward ? 1 : 0;
@@ -348,6 +357,10 @@ std::pair<std::vector<torch::Tensor>, std::vector<torch::Tensor>> PointRenderMod
     TORCH_CHECK(nri, "PointRenderModule::forward: null NeuralRenderInfo");
     TORCH_CHECK(!nri->params.add_depth_to_network, "add_depth_to_network is not available");
     nri->cache = cache.get();
+    const bool with_environment = environment_map && enable_environment_map;
+    TORCH_CHECK(!with_environment || nri->params.output_background_mask,
+                "the environment map needs output_background_mask");  // RenderModule.cpp:155
+    cache->keep_layer_weights = with_environment;
     // IntrinsicsPinhole::scale multiplies all five entries (fx, fy, cx, cy, s)
     auto rescale = [&](float f) {
         for (auto& i : nri->images)
@@ -382,6 +395,34 @@ std::pair<std::vector<torch::Tensor>, std::vector<torch::Tensor>> PointRenderMod
         for (auto& img : images) img = torch::avg_pool2d(img, {2, 2});
         for (auto& m : masks) m = torch::avg_pool2d(m, {2, 2});
         rescale(0.5f);
+    }
+    if (with_environment)
+    {
+        // RenderModule.cpp:129-202 (the FUZZY_DT masking of :143-151 belongs to the depth-test mode, which is refused)
+        const int64_t B = images.front().size(0);
+        std::vector<std::vector<torch::Tensor>> layers(L);
+        for (int i = 0; i < L; ++i)
+            for (int64_t b = 0; b < B; ++b) layers[i].push_back(cache->layer_weights[i].slice(0, b, b + 1).clone());
+        std::vector<torch::Tensor> env_maps = environment_map(layers, nri);
+        TORCH_CHECK((int)env_maps.size() == L, "the environment map returned ", env_maps.size(), " layers, expected ", L);
+        for (int i = 0; i < L; ++i)
+        {
+            if (cat_env_to_color)
+            {
+                images[i] = torch::cat({images[i], env_maps[i]}, 1);
+                continue;
+            }
+            torch::Tensor masking = torch::ones_like(env_maps[i]);
+            if (no_envmap_at_points)
+            {
+                std::vector<torch::Tensor> per_view;
+                for (int64_t b = 0; b < B; ++b)
+                    per_view.push_back(torch::where(layers[i][b] > 0.001, torch::zeros_like(layers[i][b]),
+                                                    torch::ones_like(layers[i][b])));
+                masking = torch::cat(per_view, 0).repeat({1, env_maps[i].size(1), 1, 1});  // num_texture_channels
+            }
+            images[i] = images[i] + masking * env_maps[i];
+        }
     }
     if (cat_masks_to_color)
     {
@@ -566,7 +607,7 @@ std::vector<torch::Tensor> blend_point_cloud(torch::Tensor texture, torch::Tenso
                                              torch::Tensor pose_tangents, torch::Tensor intrinsics,
                                              torch::Tensor confidence, torch::Tensor poses_se3, torch::Tensor t_index,
                                              std::vector<std::vector<double>> views, int num_layers, bool train,
-                                             pybind11::dict params)
+                                             pybind11::dict params, pybind11::object environment)
 {
     using namespace vet_amd;
     if (!g_cache) g_cache = std::make_shared<PointRendererCache>();
@@ -601,7 +642,7 @@ std::vector<torch::Tensor> blend_point_cloud(torch::Tensor texture, torch::Tenso
     }
     RenderParams& p = nri.params;
     p.dropout       = 0.f;
-    bool super_sampling = false, cat_masks_to_color = false;
+    bool super_sampling = false, cat_masks_to_color = false, cat_env_to_color = false, no_envmap_at_points = true;
     for (auto item : params)
     {
         const std::string k = pybind11::cast<std::string>(item.first);
@@ -626,15 +667,23 @@ std::vector<torch::Tensor> blend_point_cloud(torch::Tensor texture, torch::Tenso
         else if (k == "fused_texture_abs") p.fused_texture_abs = as_d() != 0;
         else if (k == "super_sampling") super_sampling = as_d() != 0;
         else if (k == "cat_masks_to_color") cat_masks_to_color = as_d() != 0;
+        else if (k == "cat_env_to_color") cat_env_to_color = as_d() != 0;
+        else if (k == "no_envmap_at_points") no_envmap_at_points = as_d() != 0;
         else TORCH_CHECK(false, "unknown RenderParams field ", k);
     }
-    if (super_sampling || cat_masks_to_color)
+    if (super_sampling || cat_masks_to_color || !environment.is_none())
     {
         // through the caller glue of the reference (PointRenderModuleImpl::forward): images, then masks
         PointRenderModule module;
         module.cache              = g_cache;
         module.super_sampling     = super_sampling;
         module.cat_masks_to_color = cat_masks_to_color;
+        module.cat_env_to_color    = cat_env_to_color;
+        module.no_envmap_at_points = no_envmap_at_points;
+        if (!environment.is_none())
+            module.environment_map = [environment](const std::vector<std::vector<torch::Tensor>>& layers, NeuralRenderInfo*) {
+                return pybind11::cast<std::vector<torch::Tensor>>(environment(layers));
+            };
         auto result               = module.forward(&nri);
         std::vector<torch::Tensor> out = result.first;
         out.insert(out.end(), result.second.begin(), result.second.end());
@@ -781,6 +830,11 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
     m.def("morton_block_shuffle_order", &vet_amd::MortonBlockShuffleOrder, pybind11::arg("positions"),
           pybind11::arg("block") = 256, pybind11::arg("seed") = 0,
           "ReorderMorton64 + RandomBlockShuffle(block) of the reference's scene preprocessing, as a permutation");
-    m.def("blend_point_cloud", &blend_point_cloud,
-          "BlendPointCloud(NeuralRenderInfo*) of the reference, with the scene passed as tensors");
+    m.def("blend_point_cloud", &blend_point_cloud, pybind11::arg("texture"), pybind11::arg("background_color"),
+          pybind11::arg("points"), pybind11::arg("pose_tangents"), pybind11::arg("intrinsics"), pybind11::arg("confidence"),
+          pybind11::arg("poses_se3"), pybind11::arg("t_index"), pybind11::arg("views"), pybind11::arg("num_layers"),
+          pybind11::arg("train"), pybind11::arg("params"), pybind11::arg("environment") = pybind11::none(),
+          "BlendPointCloud(NeuralRenderInfo*) of the reference, with the scene passed as tensors; `environment`, a "
+          "callable (layers[l][b] weight tensors) -> L tensors, routes the call through the render module's "
+          "environment-map branch");
 }

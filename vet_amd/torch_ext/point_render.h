@@ -9,6 +9,7 @@
 #pragma once
 #include <torch/torch.h>
 
+#include <functional>
 #include <memory>
 #include <string>
 #include <vector>
@@ -85,6 +86,11 @@ class PointRendererCache
     PointRendererCache& operator=(const PointRendererCache&) = delete;
     vetrast_ctx* ctx = nullptr;
     torch::Tensor eval_workspace;
+    // layers_cuda[l].weight of the reference's cache (src/lib/rendering/PointRenderer.h:131, written at
+    // src/lib/rendering/RenderForward.cu:1355-1356): per layer [B,1,h_l,w_l], the transmittance left behind the last
+    // blended fragment of every pixel. Only kept up to date by BlendPointCloud while keep_layer_weights is set.
+    bool keep_layer_weights = false;
+    std::vector<torch::Tensor> layer_weights;
 
     // Adds the error image of view `batch` to the cells its pixels fall in
     // (PointRendererCache::FillSceneGridWithLoss(int batch, NeuralPointCloudCuda point_cloud, std::vector<ReducedImageInfo>
@@ -158,12 +164,22 @@ std::vector<torch::Tensor> BlendPointCloud(NeuralRenderInfo* info);
 // (src/lib/rendering/RenderModule.cpp:45-245). It owns the cache, renders at twice the resolution and averages 2x2
 // blocks when super_sampling is on (:60-68,102-127), splits the flat output list into images and (detached) masks
 // (:74-100) and appends the masks to the images as an extra channel when cat_masks_to_color is on (:204-210).
-// The environment-map branch (:129-202) and add_depth_to_network need modules outside the rasterizer and are refused.
+// The environment-map branch (:129-202) is there too, with the map itself (a module outside the rasterizer) behind a
+// callback: it receives layers[l][b] = a clone of the [1,1,h_l,w_l] slice of the cache's weight tensor, as
+// EnvironmentMap::Sample2 does, and returns L tensors [B,C_env,h_l,w_l] that are appended as channels (cat_env_to_color)
+// or added to the images, masked to the pixels whose weight is at most 0.001 when no_envmap_at_points is on (:180-196,
+// literally: the reference zeroes the map where the weight EXCEEDS 0.001). add_depth_to_network is refused.
 class PointRenderModule
 {
    public:
+    using EnvironmentSampler =
+        std::function<std::vector<torch::Tensor>(const std::vector<std::vector<torch::Tensor>>& layers, NeuralRenderInfo* nri)>;
     bool super_sampling     = false;  // RenderParams::super_sampling, src/lib/data/Settings.h:38
     bool cat_masks_to_color = false;  // PipelineParams::cat_masks_to_color, src/lib/data/Settings.h:295
+    EnvironmentSampler environment_map;   // nri->scene->environment_map->Sample2(...), bound by the caller; empty = no map
+    bool enable_environment_map = true;   // PipelineParams::enable_environment_map (only looked at with a sampler set)
+    bool cat_env_to_color       = false;  // PipelineParams::cat_env_to_color
+    bool no_envmap_at_points    = true;   // RenderParams::no_envmap_at_points, src/lib/data/Settings.h:73
     PointRenderModule() : cache(std::make_shared<PointRendererCache>()) {}
     // {images, masks}: L images [B,C(+1),h_l,w_l]; L masks [B,1,h_l,w_l] if output_background_mask, else none
     std::pair<std::vector<torch::Tensor>, std::vector<torch::Tensor>> forward(NeuralRenderInfo* nri);

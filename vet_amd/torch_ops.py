@@ -20,17 +20,21 @@ def load():
 
 
 def blend_point_cloud(texture, background_color, points, pose_tangents, intrinsics, confidence, poses_se3, t_index,
-                      views, num_layers, train=False, **params):
+                      views, num_layers, train=False, environment=None, **params):
     """BlendPointCloud of the reference (src/lib/rendering/PointRenderer.h:53) on tensors; differentiable.
 
     views: list of (w, h, image_index, camera_index, camera_model, crop fx,fy,cx,cy,s, rot r00,r01,r10,r11).
     Returns L tensors [B,C,h_l,w_l], then L masks if output_background_mask.
+    environment: a callable standing in for the environment map of PointRenderModuleImpl::forward
+    (src/lib/rendering/RenderModule.cpp:129-202): it gets layers[l][b] = the [1,1,h_l,w_l] per-pixel transmittance left
+    behind the points and returns L tensors [B,C_env,h_l,w_l]; they are added to the images (masked with
+    no_envmap_at_points, the default) or appended as channels (cat_env_to_color). Needs output_background_mask.
     """
     if t_index is None:
         t_index = torch.empty(0, dtype=torch.int32, device=points.device)
     return load().blend_point_cloud(texture, background_color, points, pose_tangents, intrinsics, confidence, poses_se3,
                                     t_index, [list(map(float, v)) for v in views], int(num_layers), bool(train),
-                                    {k: float(v) for k, v in params.items()})
+                                    {k: float(v) for k, v in params.items()}, environment)
 
 
 def MyAdam(groups, beta1=0.9, beta2=0.999, eps=1e-8, weight_decay=0.0):
