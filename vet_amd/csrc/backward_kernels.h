@@ -174,9 +174,22 @@ __global__ void __launch_bounds__(kBlock) blend_backward_kernel(BackwardPass a)
 #pragma unroll
     for (int d = kWave / 2; d >= 1; d >>= 1) max_n = max(max_n, (uint32_t)__shfl_xor((int)max_n, d, kWave));
     float4* partial_l = a.partial + 2 * (size_t)l * (BILINEAR ? 4 : 1) * a.N;
-    for (int jw = max_n == 0 ? -1 : (int)((max_n - 1) / kWindow) * kWindow; jw >= 0; jw -= kWindow)
+    // Windows run from the deepest list places to the nearest. Where only a few pixels of the wave still have fragments
+    // that deep (uncut lists of hundreds of fragments at a handful of pixels), a window of 16 places would fill a
+    // quarter of the lanes or less and every window costs a dependent chain of memory round trips, so the window is
+    // widened to 64 places (at most 16 pixels reach into it) or 256 places (at most 4): the item table never holds
+    // more than kWaveItems entries.
+    for (uint32_t top = (max_n + kWindow - 1) / kWindow * kWindow; top > 0;)
     {
-        const uint32_t nw = (n > (uint32_t)jw) ? min(n - (uint32_t)jw, (uint32_t)kWindow) : 0u;
+        uint32_t width = kWindow;
+        if (top >= 4u * kWindow && __popcll(__ballot(n + 4u * kWindow > top)) <= kWave / 4)
+        {
+            width = 4u * kWindow;
+            if (top >= 16u * kWindow && __popcll(__ballot(n + 16u * kWindow > top)) <= kWave / 16) width = 16u * kWindow;
+        }
+        top -= width;
+        const uint32_t jw = top;
+        const uint32_t nw = (n > jw) ? min(n - jw, width) : 0u;
         uint32_t incl     = nw;
 #pragma unroll
         for (int d = 1; d < kWave; d <<= 1)
@@ -204,7 +217,7 @@ __global__ void __launch_bounds__(kBlock) blend_backward_kernel(BackwardPass a)
             float4 wp = make_float4(0.f, 0.f, 0.f, 0.f);
             if (valid)
             {
-                const uint32_t pos = s_off[wave][p] + (uint32_t)jw + (k - s_base[wave][p]);
+                const uint32_t pos = s_off[wave][p] + jw + (k - s_base[wave][p]);
                 const uint32_t low = (uint32_t)a.fragments[pos];
                 id                 = BILINEAR ? (int)(low >> 2) : (int)low;
                 corner             = BILINEAR ? (int)(low & 3u) : 0;
