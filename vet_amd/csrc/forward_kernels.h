@@ -219,6 +219,45 @@ __device__ __forceinline__ WaveGroup group_by_bin(bool has, uint32_t bin, int la
     return g;
 }
 
+// The same with 1..4 hits per lane for the bin. The group's slots are laid out place by place: first the first hit of
+// every lane of the group in lane order, then the second hits, and so on, so that the fill pass, which stores one hit
+// per lane and instruction, writes runs of consecutive records. ranks holds the slot (inside the group) of the lane's
+// hit at place o in bits 8 o .. 8 o + 7 (a group has at most 256 hits), total the size of the group.
+struct WeightedGroup
+{
+    int leader;
+    uint32_t ranks, total;
+};
+
+__device__ __forceinline__ WeightedGroup group_by_bin_weighted(bool has, uint32_t bin, uint32_t weight, int lane)
+{
+    WeightedGroup g;
+    g.leader = lane;
+    g.ranks = g.total = 0;
+    uint64_t todo     = __ballot(has);
+    while (todo != 0ull)
+    {
+        const int first        = __ffsll((unsigned long long)todo) - 1;
+        const uint32_t b_first = (uint32_t)__builtin_amdgcn_readlane((int)bin, first);
+        const bool mine        = has && bin == b_first;
+        const uint64_t m0 = __ballot(mine), m1 = __ballot(mine && weight > 1u), m2 = __ballot(mine && weight > 2u),
+                       m3 = __ballot(mine && weight > 3u);
+        const uint32_t c0 = (uint32_t)__popcll(m0), c1 = (uint32_t)__popcll(m1), c2 = (uint32_t)__popcll(m2),
+                       c3 = (uint32_t)__popcll(m3);
+        auto below = [](uint64_t m) {
+            return __builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)m, 0u));
+        };
+        if (mine)
+        {
+            g.leader = first;
+            g.ranks  = below(m0) | ((c0 + below(m1)) << 8) | ((c0 + c1 + below(m2)) << 16) | ((c0 + c1 + c2 + below(m3)) << 24);
+            g.total  = c0 + c1 + c2 + c3;
+        }
+        todo &= ~m0;
+    }
+    return g;
+}
+
 // HITS = 1: a point lands in the pixel it rounds to (FULL_BLEND); HITS = 4: in the 2x2 pixels around it (BILINEAR_BLEND),
 // each of which is a fragment of its own with its own bin. slots is [L][HITS][N].
 template <int HITS>
@@ -232,35 +271,110 @@ __global__ void __launch_bounds__(kBlock) bin_count_kernel(ViewPass a, uint32_t*
     const bool visible = i < a.N && !point_is_skipped(a, i) && project_point(*a.view, a.position[i], p);
     float ipx = visible ? p.ipx : 0.f, ipy = visible ? p.ipy : 0.f, radius = visible ? p.radius : 0.f;
     bool dropped = !visible;  // from the layer on at which the splat radius falls under the threshold
-    // Hit by hit: group the wave's hits by bin and issue the group's atomic right away. The atomics of a wave are
-    // independent and their results are only looked at after the last one has been issued, so the wave waits once.
-    // Only two registers per hit stay alive: the atomic's result and who = leader lane | rank << 8 | has << 31.
-    uint32_t base[kHits], who[kHits];
-#pragma unroll
-    for (int l = 0; l < VETRAST_MAX_LAYERS; ++l, radius *= 0.5f, ipx *= 0.5f, ipy *= 0.5f)
+    if constexpr (HITS == 1)
     {
+        // Hit by hit: group the wave's hits by bin and issue the group's atomic right away. The atomics of a wave are
+        // independent and their results are only looked at after the last one has been issued, so the wave waits once.
+        // Only two registers per hit stay alive: the atomic's result and who = leader lane | rank << 8 | has << 31.
+        uint32_t base[kHits], who[kHits];
 #pragma unroll
-        for (int h = 0; h < HITS; ++h) base[l * HITS + h] = 0, who[l * HITS + h] = 0;
-        if (l >= a.ly.L) continue;
-        if (a.drop_by_radius && radius < a.radius_threshold) dropped = true;
-#pragma unroll
-        for (int h = 0; h < HITS; ++h)
+        for (int l = 0; l < VETRAST_MAX_LAYERS; ++l, radius *= 0.5f, ipx *= 0.5f, ipy *= 0.5f)
         {
-            const int k = l * HITS + h;
+            base[l] = 0, who[l] = 0;
+            if (l >= a.ly.L) continue;
+            if (a.drop_by_radius && radius < a.radius_threshold) dropped = true;
             uint32_t tile = 0, in_tile = 0, bin = 0, in_bin;
-            const bool has = !dropped && layer_hit<HITS>(a.ly, l, ipx, ipy, h, tile, in_tile);
+            const bool has = !dropped && layer_hit<HITS>(a.ly, l, ipx, ipy, 0, tile, in_tile);
             if (has) bin_of_pixel(a.ly, l, tile, in_tile, bin, in_bin);
             const WaveGroup g = group_by_bin(has, bin, lane);
-            who[k]            = (uint32_t)g.leader | (g.rank << 8) | (has ? 0x80000000u : 0u);
-            if (has && g.leader == lane) base[k] = atomicAdd(&bin_counts[bin], g.count);
+            who[l]            = (uint32_t)g.leader | (g.rank << 8) | (has ? 0x80000000u : 0u);
+            if (has && g.leader == lane) base[l] = atomicAdd(&bin_counts[bin], g.count);
+        }
+#pragma unroll
+        for (int k = 0; k < kHits; ++k)
+        {
+            if (k >= a.ly.L) continue;
+            const uint32_t group_base = (uint32_t)__shfl((int)base[k], (int)(who[k] & 0xFF), kWave);
+            if (who[k] & 0x80000000u) slots[(size_t)k * a.N + i] = group_base + ((who[k] >> 8) & 0x7FFFu);
         }
     }
-#pragma unroll
-    for (int k = 0; k < kHits; ++k)
+    else
     {
-        if (k / HITS >= a.ly.L) continue;
-        const uint32_t group_base = (uint32_t)__shfl((int)base[k], (int)(who[k] & 0xFF), kWave);
-        if (who[k] & 0x80000000u) slots[(size_t)k * a.N + i] = group_base + ((who[k] >> 8) & 0x7FFFu);
+        // The four pixels of a point mostly lie in one bin or two. Per layer the hits of a lane are therefore taken
+        // bin by bin: in every turn a lane brings all its remaining hits that share the bin of its first remaining
+        // hit, as one entry of that weight, so a layer takes as many grouping turns as the lane with the most
+        // distinct bins has (1 or 2 as a rule, never more than 4) instead of 4, and one atomic per bin and turn.
+        // The results of a layer's atomics are looked at after those of the next layer have been issued.
+        // Kept per layer and turn: the atomic's result, the leader lane and the packed ranks; per layer, 5 bits per
+        // hit: valid | turn << 1 | place among the lane's hits of that turn << 3.
+        constexpr int kTurns = HITS;
+        uint32_t base[VETRAST_MAX_LAYERS][kTurns], leader[VETRAST_MAX_LAYERS][kTurns], ranks[VETRAST_MAX_LAYERS][kTurns],
+            code[VETRAST_MAX_LAYERS];
+        auto store_slots = [&](int l) {
+            uint32_t start[kTurns];  // first slot of the group this lane's hits of every turn belong to
+#pragma unroll
+            for (int t = 0; t < kTurns; ++t) start[t] = (uint32_t)__shfl((int)base[l][t], (int)leader[l][t], kWave);
+#pragma unroll
+            for (int h = 0; h < HITS; ++h)
+            {
+                const uint32_t c = code[l] >> (5 * h);
+                if (!(c & 1u)) continue;
+                const uint32_t t = (c >> 1) & 3u, place = (c >> 3) & 3u;
+                const uint32_t s = t == 0 ? start[0] : t == 1 ? start[1] : t == 2 ? start[2] : start[3];
+                const uint32_t r = t == 0 ? ranks[l][0] : t == 1 ? ranks[l][1] : t == 2 ? ranks[l][2] : ranks[l][3];
+                slots[(size_t)(l * HITS + h) * a.N + i] = s + ((r >> (8u * place)) & 0xFFu);
+            }
+        };
+#pragma unroll
+        for (int l = 0; l < VETRAST_MAX_LAYERS; ++l, radius *= 0.5f, ipx *= 0.5f, ipy *= 0.5f)
+        {
+            code[l] = 0;
+#pragma unroll
+            for (int t = 0; t < kTurns; ++t) base[l][t] = 0, leader[l][t] = 0, ranks[l][t] = 0;
+            if (l < a.ly.L)
+            {
+                if (a.drop_by_radius && radius < a.radius_threshold) dropped = true;
+                uint32_t bin[HITS];
+                uint32_t left = 0;  // hits not yet counted, one bit each
+#pragma unroll
+                for (int h = 0; h < HITS; ++h)
+                {
+                    uint32_t tile = 0, in_tile = 0, in_bin;
+                    bin[h]         = 0;
+                    const bool has = !dropped && layer_hit<HITS>(a.ly, l, ipx, ipy, h, tile, in_tile);
+                    if (has)
+                    {
+                        bin_of_pixel(a.ly, l, tile, in_tile, bin[h], in_bin);
+                        left |= 1u << h;
+                    }
+                }
+#pragma unroll
+                for (int t = 0; t < kTurns; ++t)
+                {
+                    if (__ballot(left != 0u) == 0ull) break;  // the same for the whole wave
+                    uint32_t key = 0;
+#pragma unroll
+                    for (int h = HITS - 1; h >= 0; --h)
+                        if (left & (1u << h)) key = bin[h];  // bin of the first remaining hit
+                    uint32_t weight = 0;
+#pragma unroll
+                    for (int h = 0; h < HITS; ++h)
+                        if ((left & (1u << h)) && bin[h] == key)
+                        {
+                            code[l] |= (1u | ((uint32_t)t << 1) | (weight << 3)) << (5 * h);
+                            ++weight;
+                            left &= ~(1u << h);
+                        }
+                    const bool has        = weight != 0u;
+                    const WeightedGroup g = group_by_bin_weighted(has, key, weight, lane);
+                    leader[l][t]          = (uint32_t)g.leader;
+                    ranks[l][t]           = g.ranks;
+                    if (has && g.leader == lane) base[l][t] = atomicAdd(&bin_counts[key], g.total);
+                }
+            }
+            if (l >= 1 && l - 1 < a.ly.L) store_slots(l - 1);
+        }
+        if (VETRAST_MAX_LAYERS - 1 < a.ly.L) store_slots(VETRAST_MAX_LAYERS - 1);
     }
 }
 
