@@ -165,6 +165,9 @@ typedef struct vetrast_workspace_layout
     size_t partial_base;   /* float [L][N][8]: backward scratch, gradient record of the fragment of point i in layer l */
     size_t background_partial_base; /* float [workgroups][8]: backward scratch, per-workgroup background-gradient sums */
     size_t camera_partial_base;     /* double [ceil(N/256)][12]: backward scratch, per-workgroup pose / intrinsics sums */
+    size_t projected_base, projected_stride; /* per view, float [N][2], BILINEAR_BLEND only (stride 0 otherwise): image
+                                                position of every visible point at layer 0, from which the blend and its
+                                                backward pass form the bilinear weights */
 } vetrast_workspace_layout;
 
 /* Arguments of the forward pass. Replaces the inputs PointRender::forward receives

@@ -18,8 +18,8 @@ struct BackwardPass
     const uint64_t* fragments;
     const float* transmittance;  // per blended fragment, saved by the forward blend
     const float* weight;         // per pixel: transmittance behind the last blended fragment
-    const float4* position;      // BILINEAR_BLEND: a fragment's alpha and its derivative depend on the point's projection
-    const DeviceView* view;
+    const float2* projected;     // BILINEAR_BLEND: [N] where a point projects to at layer 0 (a fragment's alpha and its
+                                 // derivative depend on it); written by the forward pass
     const int32_t* index;
     const float4* packed;
     const float* background;
@@ -214,7 +214,6 @@ __global__ void __launch_bounds__(kBlock) blend_backward_kernel(BackwardPass a)
             float t[4] = {0.f, 0.f, 0.f, 0.f};
             float4 g4  = make_float4(0.f, 0.f, 0.f, 0.f);
             int id = -1, ti = -1, corner = 0;
-            float4 wp = make_float4(0.f, 0.f, 0.f, 0.f);
             if (valid)
             {
                 const uint32_t pos = s_off[wave][p] + jw + (k - s_base[wave][p]);
@@ -235,16 +234,12 @@ __global__ void __launch_bounds__(kBlock) blend_backward_kernel(BackwardPass a)
                 c               = conf;
                 if constexpr (BILINEAR)
                 {
-                    // alpha = bilinear weight of this pixel's corner at the point's position in this layer x confidence
-                    wp = a.position[id];
-                    Projected pr;
-                    fac = 0.f;
-                    if (project_point(*a.view, wp, pr))
-                    {
-                        float u = pr.ipx, v = pr.ipy;
-                        for (int h = 0; h < l; ++h) u *= 0.5f, v *= 0.5f;
-                        fac = bilinear_weight(u, v, corner, &fac_du, &fac_dv);
-                    }
+                    // alpha = bilinear weight of this pixel's corner at the point's position in this layer x confidence;
+                    // the position is the one the fill pass stored for the forward blend
+                    const float2 ip = a.projected[id];
+                    float u = ip.x, v = ip.y;
+                    for (int h = 0; h < l; ++h) u *= 0.5f, v *= 0.5f;
+                    fac = bilinear_weight(u, v, corner, &fac_du, &fac_dv);
                     c = fac * conf;
                 }
                 t[0] = t4.x, t[1] = t4.y, t[2] = t4.z, t[3] = t4.w;

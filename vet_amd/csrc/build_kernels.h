@@ -37,8 +37,8 @@ struct BuildPass
     uint8_t* list_is_cut;   // [P]
     uint32_t* kept;         // [P] fragments of the pixel that took part in the blend
     // blending
-    const float4* position;   // BILINEAR_BLEND only: the alpha of a fragment depends on where its point projects to
-    const DeviceView* view;
+    const float2* projected;  // BILINEAR_BLEND only: [N] where a point projects to at layer 0 (the alpha of a fragment
+                              // depends on it)
     const int32_t* index;
     const float4* packed;
     const float* background;
@@ -58,7 +58,7 @@ struct BuildPass
 
 // Alpha of a fragment: the point's confidence, in BILINEAR_BLEND times the bilinear weight of the pixel's corner at the
 // point's position in this layer (BlendMultiBilinear, src/lib/rendering/RenderForward.cu:1586-1613). The position is
-// the same projection the binning passes computed, so the weight is reproduced bit for bit.
+// the projection the fill pass stored, so the weight is reproduced bit for bit.
 template <bool BILINEAR>
 __device__ __forceinline__ float fragment_alpha(const BuildPass& a, int l, uint32_t low, float confidence)
 {
@@ -66,9 +66,8 @@ __device__ __forceinline__ float fragment_alpha(const BuildPass& a, int l, uint3
         return confidence;
     else
     {
-        Projected p;
-        if (!project_point(*a.view, a.position[low >> 2], p)) return 0.f;  // cannot happen for a listed fragment
-        float u = p.ipx, v = p.ipy;
+        const float2 ip = a.projected[low >> 2];  // written by the fill pass for every point that has fragments
+        float u = ip.x, v = ip.y;
         for (int k = 0; k < l; ++k) u *= 0.5f, v *= 0.5f;
         return bilinear_weight(u, v, (int)(low & 3u)) * confidence;
     }

@@ -71,6 +71,7 @@ struct ViewPass
     float stability_cutoff;
     int confidence_activation;  // 1: `confidence` holds raw values, the confidence is sigmoid(confidence_scale * raw)
     float confidence_scale;
+    float2* projected;  // BILINEAR_BLEND: [N] image position of every visible point at layer 0, written by the fill pass
 };
 
 struct Projected

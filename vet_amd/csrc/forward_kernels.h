@@ -522,6 +522,9 @@ __global__ void __launch_bounds__(kBlock) bin_fill_kernel(ViewPass a, const uint
     if (!project_point(*a.view, a.position[i], p)) return;
     const uint32_t depth_bits = __float_as_uint(p.z);
     float ipx = p.ipx, ipy = p.ipy, radius = p.radius;
+    // The blend and its backward pass form a fragment's bilinear weight from the point's image position; they read it
+    // from here (8 bytes) instead of projecting the point again for every one of its fragments.
+    if constexpr (HITS == 4) a.projected[i] = make_float2(ipx, ipy);
     for (int l = 0; l < a.ly.L; ++l, radius *= 0.5f, ipx *= 0.5f, ipy *= 0.5f)
     {
         if (a.drop_by_radius && radius < a.radius_threshold) break;

@@ -255,6 +255,7 @@ ViewPass make_view_pass(const vetrast_forward_args* a, const vetrast_workspace_l
     vp.stability_cutoff = a->params.stability_cutoff_value;
     vp.confidence_activation = a->params.confidence_activation;
     vp.confidence_scale      = a->params.confidence_scale;
+    vp.projected = lay.projected_stride ? ws_ptr<float2>(a->workspace, lay.projected_base + lay.projected_stride * b) : nullptr;
     return vp;
 }
 
@@ -378,6 +379,9 @@ int vetrast_workspace_layout_for_mode(int32_t N, int32_t B, int32_t L, int32_t w
     lay->transmittance_base   = at;
     lay->transmittance_stride = align_up(cap * sizeof(float), kAlign);
     at += lay->transmittance_stride * B;
+    lay->projected_base   = at;
+    lay->projected_stride = hits == 4 ? align_up((size_t)N * sizeof(float2), kAlign) : 0;
+    at += lay->projected_stride * B;
     lay->forward_only_bytes = align_up(at, kAlign);
     at                      = lay->forward_only_bytes;
     lay->partial_base       = at;
@@ -528,8 +532,7 @@ int vetrast_forward(vetrast_ctx* ctx, const vetrast_forward_args* a, void* strea
             bp.fragments           = fragments;
             bp.list_is_cut         = list_is_cut;
             bp.kept                = ws_ptr<uint32_t>(ws, lay.kept_base + lay.kept_stride * b);
-            bp.position            = vp.position;
-            bp.view                = vp.view;
+            bp.projected           = vp.projected;
             bp.index               = a->index;
             bp.packed              = packed;
             bp.background          = reinterpret_cast<const float*>(flags) + kPreparedBackgroundOffset;
@@ -655,8 +658,7 @@ int vetrast_backward(vetrast_ctx* ctx, const vetrast_backward_args* g, void* str
             BackwardPass bp;
             bp.offsets          = offsets;
             bp.kept             = ws_ptr<uint32_t>(ws, lay.kept_base + lay.kept_stride * b);
-            bp.position         = reinterpret_cast<const float4*>(a->position);
-            bp.view             = ws_ptr<DeviceView>(ws, lay.views_base) + b;
+            bp.projected        = lay.projected_stride ? ws_ptr<float2>(ws, lay.projected_base + lay.projected_stride * b) : nullptr;
             bp.fragments        = fragments;
             bp.transmittance    = ws_ptr<float>(ws, lay.transmittance_base + lay.transmittance_stride * b);
             bp.weight           = ws_ptr<float>(ws, lay.weight_base + lay.weight_stride * b);
