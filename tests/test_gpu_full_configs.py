@@ -89,6 +89,20 @@ def test_config3_generated_point_order(rasterizer, oracle):
     _backward_parity(scene, res, ref, rasterizer, oracle)
 
 
+@pytest.mark.parametrize("drop_by_radius", [0, 1])
+def test_config3_without_the_cut_as_vet_ships_it(drop_by_radius, rasterizer, oracle):
+    """debug_max_list_length = -1 (configs/config.ini:123): no top-K cut, so the coarse layers blend lists of hundreds to
+    thousands of fragments, sorted in full; with and without the radius drop-out VET trains with."""
+    print(f"[case] config 3 without a cut, drop_out_points_by_radius={drop_by_radius}, forward+backward", flush=True)
+    scene = synthetic.config3(K=-1)
+    _, dev, res, ref = _forward_parity(scene, rasterizer, oracle, need_point_gradient=1,
+                                       drop_out_points_by_radius=drop_by_radius)
+    counts = np.diff(res.offsets(0))
+    print(f"  longest list {counts.max()}, lists beyond 64 / 256 / 1024 keys: {(counts > 64).sum()} / "
+          f"{(counts > 256).sum()} / {(counts > 1024).sum()}", flush=True)
+    _backward_parity(scene, res, ref, rasterizer, oracle)
+
+
 def test_config4_batch_of_views_full_size(rasterizer, oracle):
     print("[case] config 4, 5.5M points incl. 3 environment spheres, 4 views", flush=True)
     scene = synthetic.config4()
