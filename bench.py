@@ -33,8 +33,10 @@ def algorithmic_bytes(N, P, F, Fk, Cn):
     """
     fwd = {
         # the model's terms, booked on the kernels that do the corresponding work here
-        "COUNT": 16 * N,                              # positions read
-        "FILL": 16 * N + 8 * F,                       # positions read again, fragment records written
+        # one pass over the points projects them, counts the bins and writes the fragment records (the model reads the
+        # positions twice, as the reference's two passes do; both reads are booked here)
+        "COUNT": 32 * N + 8 * F,
+        "FILL": 0,                                    # files the few records that overflow a bin's own room
         # per-pixel counts, counts -> offsets, records read and written sorted; then the blend: lists, descriptor +
         # confidence, offsets, out, weight
         "BUILD": 4 * P + 8 * P + 16 * F + 8 * Fk + (4 * Cn + 4) * Fk + 4 * P + 4 * Cn * P + 4 * P,

@@ -115,9 +115,11 @@ typedef enum vetrast_scope
     VETRAST_SCOPE_PREPARE = 0,      /* "Build Cache": zero-fill, view preparation */
     VETRAST_SCOPE_PACK,             /* "Build Cache": descriptor interleave; runs on a stream of the context's own beside
                                        COUNT..FILL, so its time is not part of the sum of the others */
-    VETRAST_SCOPE_COUNT,            /* "CountingPass": fragments per bin (a 16x16 pixel tile or a piece of one) */
+    VETRAST_SCOPE_COUNT,            /* "CountingPass": fragments per bin (a 16x16 pixel tile or a piece of one) and, in
+                                       the same pass over the points, the fragment records written to their bins */
     VETRAST_SCOPE_SCAN,             /* "CreateAndAllocateBuffers" (prefix scan over the bins; no allocation here) */
-    VETRAST_SCOPE_FILL,             /* "CollectionPass", first half: fragment records grouped by bin */
+    VETRAST_SCOPE_FILL,             /* "CollectionPass", first half: the records that did not fit their bin's own room
+                                       are filed behind the scan (an almost empty kernel as a rule) */
     VETRAST_SCOPE_BUILD,            /* "CollectionPass" second half + "SortingPass" + "BlendingPass": one pass per bin */
     VETRAST_SCOPE_BACKWARD_PREPARE, /* "Prepare Backward": zero-fill of gradient buffers */
     VETRAST_SCOPE_BACKWARD_BLEND,   /* "BlendBackwards", per-pixel part */
@@ -154,17 +156,24 @@ typedef struct vetrast_workspace_layout
     size_t cut_flags_base, cut_flags_stride; /* uint8 [P]: 1 where some fragments of the pixel's list did not (top-K cut, saturation) */
     /* shared by all views */
     size_t packed_base;    /* float [N][8]: descriptor (4, zero padded), confidence, 3 pad */
-    size_t slots_base;     /* uint32 [L][N]: per (layer, point) arrival rank inside its tile (scratch between two passes) */
+    size_t slots_base;     /* uint32 [N*L*hits]: rank inside its bin of every record in the overflow log (scratch) */
     size_t views_base;     /* prepared per-view camera constants */
     size_t scan_partials_base;
     int64_t num_bins;      /* bins of one view: runs of 256 / 64 / 16 / 4 consecutive pixel numbers, chosen per layer from N */
     size_t bin_counts_base, bin_counts_stride; /* per view, uint32 [num_bins+1 padded]: fragments per bin, then their exclusive scan */
-    size_t binned_base;    /* uint32 [N*L][4]: fragment records grouped by bin (key low, key high, pixel in bin, 0); scratch */
+    size_t binned_base;    /* uint32 [N*L*hits][4]: compact array of fragment records (key low, key high, pixel in bin, 0),
+                              only used for the records beyond a bin's own room; scratch */
     size_t flags_base;     /* uint32 [4] device status flags, then at +64 bytes float [4]: the background as it is blended */
     size_t forward_only_bytes; /* a forward call with save_for_backward = 0 needs only this much */
     size_t partial_base;   /* float [L][N][8]: backward scratch, gradient record of the fragment of point i in layer l */
     size_t background_partial_base; /* float [workgroups][8]: backward scratch, per-workgroup background-gradient sums */
     size_t camera_partial_base;     /* double [ceil(N/256)][12]: backward scratch, per-workgroup pose / intrinsics sums */
+    /* scratch shared by all views: the scatter pass writes the records of bin b to primary[b][rank] while rank < 2048;
+     * records beyond that go to a log (record + bin, rank in the slots array) and are filed into the compact array
+     * after the scan. log_cursor: uint32 per view, entries in the log. */
+    size_t primary_base;   /* uint32 [num_bins][2048][4] */
+    size_t log_base;       /* uint32 [N*L*hits][4] */
+    size_t log_cursor_base;
     size_t projected_base, projected_stride; /* per view, float [N][2], BILINEAR_BLEND only (stride 0 otherwise): image
                                                 position of every visible point at layer 0, from which the blend and its
                                                 backward pass form the bilinear weights */

@@ -235,7 +235,7 @@ __global__ void __launch_bounds__(kBlock) blend_backward_kernel(BackwardPass a)
                 if constexpr (BILINEAR)
                 {
                     // alpha = bilinear weight of this pixel's corner at the point's position in this layer x confidence;
-                    // the position is the one the fill pass stored for the forward blend
+                    // the position is the one the scatter pass stored for the forward blend
                     const float2 ip = a.projected[id];
                     float u = ip.x, v = ip.y;
                     for (int h = 0; h < l; ++h) u *= 0.5f, v *= 0.5f;
@@ -667,7 +667,7 @@ __device__ __forceinline__ float sign_of(float x)
 
 constexpr int kCameraRow = 12;  // doubles per workgroup row: 6 pose tangent, fx, fy, cx, cy, fragment count, pad
 
-// One thread per point: find the pixel the point fell into in every layer (the same projection as the count pass), decide
+// One thread per point: find the pixel the point fell into in every layer (the same projection as the scatter pass), decide
 // whether its fragment survived the top-K cut (its key is not larger than the K-th key of that pixel's sorted list), and
 // sum the stored records. With a texture index indirection several points may share a descriptor row; only then the
 // descriptor and confidence sums are added with atomics (onto rows the host zero-filled).

@@ -26,12 +26,14 @@ namespace vetrast
 // on the 10 M point cloud.
 constexpr int kBuildPerThread = 4;
 constexpr int kBuildCap       = kBlock * kBuildPerThread;  // 1024 records = 8 KB of keys in LDS
+static_assert(kPrimaryCap >= kBuildCap, "a bin built in LDS must find all its records in its own room");
 constexpr int kStage          = 256;                       // descriptor records staged per round (8 KB)
 
 struct BuildPass
 {
     const uint32_t* bin_offsets;  // [bins + 1] exclusive scan of the bin counts
-    const uint4* binned;
+    const uint4* primary;         // [bins][kPrimaryCap] fragment records, the first kPrimaryCap of every bin
+    const uint4* binned;          // compact array: record r >= kPrimaryCap of a bin sits at bin_offsets[bin] + r
     uint32_t* offsets;    // [P + 1] per pixel: start of its list; [P] = fragments of the view
     uint64_t* fragments;
     uint8_t* list_is_cut;   // [P]
@@ -58,7 +60,7 @@ struct BuildPass
 
 // Alpha of a fragment: the point's confidence, in BILINEAR_BLEND times the bilinear weight of the pixel's corner at the
 // point's position in this layer (BlendMultiBilinear, src/lib/rendering/RenderForward.cu:1586-1613). The position is
-// the projection the fill pass stored, so the weight is reproduced bit for bit.
+// the projection the scatter pass stored, so the weight is reproduced bit for bit.
 template <bool BILINEAR>
 __device__ __forceinline__ float fragment_alpha(const BuildPass& a, int l, uint32_t low, float confidence)
 {
@@ -66,7 +68,7 @@ __device__ __forceinline__ float fragment_alpha(const BuildPass& a, int l, uint3
         return confidence;
     else
     {
-        const float2 ip = a.projected[low >> 2];  // written by the fill pass for every point that has fragments
+        const float2 ip = a.projected[low >> 2];  // written by the scatter pass for every point that has fragments
         float u = ip.x, v = ip.y;
         for (int k = 0; k < l; ++k) u *= 0.5f, v *= 0.5f;
         return bilinear_weight(u, v, (int)(low & 3u)) * confidence;
@@ -205,7 +207,9 @@ __global__ void __launch_bounds__(kBlock) bin_build_kernel(BuildPass a)
     // the same for every lane: tell the compiler, so that loops over the bin's records become scalar branches
     const uint32_t begin  = (uint32_t)__builtin_amdgcn_readfirstlane((int)a.bin_offsets[bin]);
     const uint32_t n      = (uint32_t)__builtin_amdgcn_readfirstlane((int)a.bin_offsets[bin + 1]) - begin;
-    const uint4* recs     = a.binned + begin;
+    // record r of the bin: its own room first, what did not fit there in the compact array
+    const uint4* recs = a.primary + (size_t)bin * kPrimaryCap;
+    const uint4* more = a.binned + begin;
     const bool in_lds     = n <= (uint32_t)kBuildCap;
     s_cnt[tid] = 0u;
     __syncthreads();
@@ -245,7 +249,7 @@ __global__ void __launch_bounds__(kBlock) bin_build_kernel(BuildPass a)
             for (int k = 0; k < 4; ++k)
             {
                 const uint32_t r = r0 + k * kBlock + tid;
-                px[k]            = r < n ? (recs[r].z & (pixels - 1u)) : 0xFFFFFFFFu;
+                px[k]            = r < n ? ((r < (uint32_t)kPrimaryCap ? recs[r] : more[r]).z & (pixels - 1u)) : 0xFFFFFFFFu;
             }
 #pragma unroll
             for (int k = 0; k < 4; ++k)
@@ -318,7 +322,7 @@ __global__ void __launch_bounds__(kBlock) bin_build_kernel(BuildPass a)
                 if (r - s_prefix[px] >= len) continue;  // cut away
                 const uint32_t low = s_id[2 * r];
                 const int id       = BILINEAR ? (int)(low >> 2) : (int)low;
-                // an id or texture index out of range cannot come from a list the fill pass wrote; such a fragment
+                // an id or texture index out of range cannot come from a list the scatter pass wrote; such a fragment
                 // blends as fully transparent (the reference asserts on the texture index, RenderForward.cu:1335-1336)
                 int ti = -1;
                 if ((uint32_t)id < (uint32_t)a.N) ti = a.index ? a.index[id] : id;
@@ -390,7 +394,7 @@ __global__ void __launch_bounds__(kBlock) bin_build_kernel(BuildPass a)
             for (int k = 0; k < 4; ++k)
             {
                 const uint32_t r = r0 + k * kBlock + tid;
-                rec[k]           = r < n ? recs[r] : make_uint4(0u, 0u, 0xFFFFFFFFu, 0u);
+                rec[k]           = r < n ? (r < (uint32_t)kPrimaryCap ? recs[r] : more[r]) : make_uint4(0u, 0u, 0xFFFFFFFFu, 0u);
             }
 #pragma unroll
             for (int k = 0; k < 4; ++k)

@@ -16,6 +16,7 @@ constexpr int kBlendChunk     = 4;            // fragments a blend / backward th
 constexpr int kBackgroundRow  = 8;            // floats per workgroup row of background-gradient partial sums
 constexpr int kPreparedBackgroundOffset = 16;  // float index inside the flags block: the background as it is blended
 constexpr int kPackedFloats   = 8;            // interleaved record: 4 descriptor floats, confidence, 3 pad
+constexpr int kPrimaryCap     = 2048;         // fragment records every bin has room for (bins are sized for <= 1024 expected)
 
 // Camera constants of one view, written by prepare_views_kernel and read (uniformly) by every other kernel.
 // Counterpart of what the reference pulls per thread out of d_render_params.Pose()/PinholeIntrinsics() and the
@@ -71,7 +72,7 @@ struct ViewPass
     float stability_cutoff;
     int confidence_activation;  // 1: `confidence` holds raw values, the confidence is sigmoid(confidence_scale * raw)
     float confidence_scale;
-    float2* projected;  // BILINEAR_BLEND: [N] image position of every visible point at layer 0, written by the fill pass
+    float2* projected;  // BILINEAR_BLEND: [N] image position of every visible point at layer 0, written by the scatter pass
 };
 
 struct Projected

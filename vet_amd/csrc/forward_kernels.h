@@ -175,14 +175,14 @@ __device__ __forceinline__ bool point_is_skipped(const ViewPass& a, int i)
 // list. MI355X retires about 26 G global atomics per second whatever their scope, return mode or address spread, and at
 // the fine layers nearly every fragment has a pixel of its own, so per-pixel atomics alone would cost more than the
 // rest of the forward pass. The lists are therefore built in two levels:
-//   1. bin_count_kernel: fragments per BIN, a run of 256 / 64 / 16 / 4 consecutive pixel numbers (a 16x16 tile or a
-//      piece of one; the denser the layer, the smaller its bins). VET hands over clouds in Morton order with 256-point
-//      blocks (src/lib/data/SceneData.cpp:105-106), so the 64 points of a wave fall into a handful of bins per layer:
-//      the wave groups its hits by bin with ballots and issues one returning atomic per distinct bin, which also gives
-//      every hit its arrival rank inside the bin.
-//   2. exclusive scan over the bin counts.
-//   3. bin_fill_kernel: second projection; the fragment record goes to bin start + rank: a bin's records are contiguous.
-//   4. bin_build_kernel: one workgroup per bin counts the pixels, scans them, scatters the keys and sorts the lists, all
+//   1. bin_scatter_kernel: one pass over the points. A BIN is a run of 256 / 64 / 16 / 4 consecutive pixel numbers (a
+//      16x16 tile or a piece of one; the denser the layer, the smaller its bins). VET hands over clouds in Morton order
+//      with 256-point blocks (src/lib/data/SceneData.cpp:105-106), so the 64 points of a wave fall into a handful of
+//      bins per layer: the wave groups its hits by bin with ballots and issues one returning atomic per distinct bin,
+//      which counts the bin and gives every hit its arrival rank inside it; the fragment record goes straight to
+//      place `rank` of the room the bin owns (no second projection pass).
+//   2. exclusive scan over the bin counts (overflow_move_kernel then files the few records that did not fit a bin's room).
+//   3. bin_build_kernel: one workgroup per bin counts the pixels, scans them, scatters the keys and sorts the lists, all
 //      in LDS. Pixels are numbered tile by tile, so the scan of the bin counts IS the start of every bin's lists and no
 //      scan over the pixels is needed.
 
@@ -220,8 +220,8 @@ __device__ __forceinline__ WaveGroup group_by_bin(bool has, uint32_t bin, int la
 }
 
 // The same with 1..4 hits per lane for the bin. The group's slots are laid out place by place: first the first hit of
-// every lane of the group in lane order, then the second hits, and so on, so that the fill pass, which stores one hit
-// per lane and instruction, writes runs of consecutive records. ranks holds the slot (inside the group) of the lane's
+// every lane of the group in lane order, then the second hits, and so on, so that the record stores, one hit per
+// lane and instruction, write runs of consecutive records. ranks holds the slot (inside the group) of the lane's
 // hit at place o in bits 8 o .. 8 o + 7 (a group has at most 256 hits), total the size of the group.
 struct WeightedGroup
 {
@@ -258,59 +258,108 @@ __device__ __forceinline__ WeightedGroup group_by_bin_weighted(bool has, uint32_
     return g;
 }
 
-// HITS = 1: a point lands in the pixel it rounds to (FULL_BLEND); HITS = 4: in the 2x2 pixels around it (BILINEAR_BLEND),
-// each of which is a fragment of its own with its own bin. slots is [L][HITS][N].
+// Where the scatter pass puts a fragment record (64-bit key = depth bits << 32 | point id, pixel inside the bin).
+// Every bin owns room for kPrimaryCap records; a record whose rank inside its bin is beyond that is appended to a log
+// (with its bin and rank), from where overflow_move_kernel brings it to the bin's place in the compact array once the
+// scan of the bin counts is known. Bins are sized for an expected 1024 records at most, so the log stays empty or
+// short unless the cloud is far denser somewhere than on average.
+struct ScatterTargets
+{
+    uint4* primary;        // [bins][kPrimaryCap] records
+    uint4* log;            // [log_capacity]: key low, key high, pixel in bin, bin
+    uint32_t* log_rank;    // [log_capacity]: rank of the logged record inside its bin
+    uint32_t* log_cursor;  // entries in the log (this view)
+    uint32_t log_capacity;
+};
+
+// One record to its bin; `valid` lanes carry one. Called by the whole wave (uniform control flow).
+__device__ __forceinline__ void store_record(const ScatterTargets& t, bool valid, uint32_t bin, uint32_t rank,
+                                             uint32_t low, uint32_t depth_bits, uint32_t in_bin, int lane)
+{
+    const bool over = valid && rank >= (uint32_t)kPrimaryCap;
+    if (valid && !over) t.primary[(size_t)bin * kPrimaryCap + rank] = make_uint4(low, depth_bits, in_bin, 0u);
+    const uint64_t m = __ballot(over);
+    if (m != 0ull)  // rare
+    {
+        const int leader = __ffsll((unsigned long long)m) - 1;
+        uint32_t first   = 0;
+        if (lane == leader) first = atomicAdd(t.log_cursor, (uint32_t)__popcll(m));
+        first = (uint32_t)__shfl((int)first, leader, kWave);
+        const uint32_t pos =
+            first + __builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)m, 0u));
+        if (over && pos < t.log_capacity)  // guard: the log has room for every hit of the view
+        {
+            t.log[pos]      = make_uint4(low, depth_bits, in_bin, bin);
+            t.log_rank[pos] = rank;
+        }
+    }
+}
+
+// The one pass over the points: projection, the bin of every hit, the hit's rank inside its bin (which also counts
+// the bin) and the fragment record written to the bin's room. Counterpart of CountingPrepassMulti and CollectMulti
+// (src/lib/rendering/RenderForward.cu:806-905,1011-1096), which project every point twice and draw count and rank
+// from two atomic counter images.
+// HITS = 1: a point lands in the pixel it rounds to (FULL_BLEND); HITS = 4: in the 2x2 pixels around it
+// (BILINEAR_BLEND), each of which is a fragment of its own with its own bin; the low key word is then
+// point id << 2 | corner.
 template <int HITS>
-__global__ void __launch_bounds__(kBlock) bin_count_kernel(ViewPass a, uint32_t* __restrict__ bin_counts,
-                                                            uint32_t* __restrict__ slots)
+__global__ void __launch_bounds__(kBlock) bin_scatter_kernel(ViewPass a, uint32_t* __restrict__ bin_counts,
+                                                              ScatterTargets out)
 {
     const int i    = blockIdx.x * blockDim.x + threadIdx.x;
     const int lane = threadIdx.x & (kWave - 1);
-    constexpr int kHits = VETRAST_MAX_LAYERS * HITS;
     Projected p;
+    p.ipx = p.ipy = p.z = p.radius = 0.f;
     const bool visible = i < a.N && !point_is_skipped(a, i) && project_point(*a.view, a.position[i], p);
     float ipx = visible ? p.ipx : 0.f, ipy = visible ? p.ipy : 0.f, radius = visible ? p.radius : 0.f;
+    const uint32_t depth_bits = __float_as_uint(p.z);
     bool dropped = !visible;  // from the layer on at which the splat radius falls under the threshold
     if constexpr (HITS == 1)
     {
-        // Hit by hit: group the wave's hits by bin and issue the group's atomic right away. The atomics of a wave are
-        // independent and their results are only looked at after the last one has been issued, so the wave waits once.
-        // Only two registers per hit stay alive: the atomic's result and who = leader lane | rank << 8 | has << 31.
-        uint32_t base[kHits], who[kHits];
+        // Layer by layer: group the wave's hits by bin and issue the group's atomic right away. The atomics of a wave
+        // are independent and their results are only looked at after the last one has been issued, so the wave waits
+        // once. Kept per layer: the atomic's result, the bin, and
+        // who = leader lane | rank << 8 | pixel in bin << 16 | has << 31.
+        uint32_t base[VETRAST_MAX_LAYERS], who[VETRAST_MAX_LAYERS], bins[VETRAST_MAX_LAYERS];
 #pragma unroll
         for (int l = 0; l < VETRAST_MAX_LAYERS; ++l, radius *= 0.5f, ipx *= 0.5f, ipy *= 0.5f)
         {
-            base[l] = 0, who[l] = 0;
+            base[l] = 0, who[l] = 0, bins[l] = 0;
             if (l >= a.ly.L) continue;
             if (a.drop_by_radius && radius < a.radius_threshold) dropped = true;
-            uint32_t tile = 0, in_tile = 0, bin = 0, in_bin;
+            uint32_t tile = 0, in_tile = 0, bin = 0, in_bin = 0;
             const bool has = !dropped && layer_hit<HITS>(a.ly, l, ipx, ipy, 0, tile, in_tile);
             if (has) bin_of_pixel(a.ly, l, tile, in_tile, bin, in_bin);
             const WaveGroup g = group_by_bin(has, bin, lane);
-            who[l]            = (uint32_t)g.leader | (g.rank << 8) | (has ? 0x80000000u : 0u);
+            who[l]            = (uint32_t)g.leader | (g.rank << 8) | (in_bin << 16) | (has ? 0x80000000u : 0u);
+            bins[l]           = bin;
             if (has && g.leader == lane) base[l] = atomicAdd(&bin_counts[bin], g.count);
         }
 #pragma unroll
-        for (int k = 0; k < kHits; ++k)
+        for (int l = 0; l < VETRAST_MAX_LAYERS; ++l)
         {
-            if (k >= a.ly.L) continue;
-            const uint32_t group_base = (uint32_t)__shfl((int)base[k], (int)(who[k] & 0xFF), kWave);
-            if (who[k] & 0x80000000u) slots[(size_t)k * a.N + i] = group_base + ((who[k] >> 8) & 0x7FFFu);
+            if (l >= a.ly.L) continue;
+            const uint32_t group_base = (uint32_t)__shfl((int)base[l], (int)(who[l] & 0xFF), kWave);
+            store_record(out, (who[l] & 0x80000000u) != 0u, bins[l], group_base + ((who[l] >> 8) & 0xFFu), (uint32_t)i,
+                         depth_bits, (who[l] >> 16) & 0xFFu, lane);
         }
     }
     else
     {
+        // The blend and its backward pass form a fragment's bilinear weight from the point's image position; they
+        // read it from here (8 bytes) instead of projecting the point again for every one of its fragments.
+        if (visible) a.projected[i] = make_float2(p.ipx, p.ipy);
         // The four pixels of a point mostly lie in one bin or two. Per layer the hits of a lane are therefore taken
         // bin by bin: in every turn a lane brings all its remaining hits that share the bin of its first remaining
         // hit, as one entry of that weight, so a layer takes as many grouping turns as the lane with the most
         // distinct bins has (1 or 2 as a rule, never more than 4) instead of 4, and one atomic per bin and turn.
         // The results of a layer's atomics are looked at after those of the next layer have been issued.
-        // Kept per layer and turn: the atomic's result, the leader lane and the packed ranks; per layer, 5 bits per
-        // hit: valid | turn << 1 | place among the lane's hits of that turn << 3.
+        // Kept per layer and turn: the atomic's result, the leader lane, the packed ranks and the bin; per layer,
+        // 5 bits per hit: valid | turn << 1 | place among the lane's hits of that turn << 3, and the four pixels in bin.
         constexpr int kTurns = HITS;
         uint32_t base[VETRAST_MAX_LAYERS][kTurns], leader[VETRAST_MAX_LAYERS][kTurns], ranks[VETRAST_MAX_LAYERS][kTurns],
-            code[VETRAST_MAX_LAYERS];
-        auto store_slots = [&](int l) {
+            bins[VETRAST_MAX_LAYERS][kTurns], code[VETRAST_MAX_LAYERS], in_bins[VETRAST_MAX_LAYERS];
+        auto store_layer = [&](int l) {
             uint32_t start[kTurns];  // first slot of the group this lane's hits of every turn belong to
 #pragma unroll
             for (int t = 0; t < kTurns; ++t) start[t] = (uint32_t)__shfl((int)base[l][t], (int)leader[l][t], kWave);
@@ -318,19 +367,20 @@ __global__ void __launch_bounds__(kBlock) bin_count_kernel(ViewPass a, uint32_t*
             for (int h = 0; h < HITS; ++h)
             {
                 const uint32_t c = code[l] >> (5 * h);
-                if (!(c & 1u)) continue;
                 const uint32_t t = (c >> 1) & 3u, place = (c >> 3) & 3u;
                 const uint32_t s = t == 0 ? start[0] : t == 1 ? start[1] : t == 2 ? start[2] : start[3];
                 const uint32_t r = t == 0 ? ranks[l][0] : t == 1 ? ranks[l][1] : t == 2 ? ranks[l][2] : ranks[l][3];
-                slots[(size_t)(l * HITS + h) * a.N + i] = s + ((r >> (8u * place)) & 0xFFu);
+                const uint32_t b = t == 0 ? bins[l][0] : t == 1 ? bins[l][1] : t == 2 ? bins[l][2] : bins[l][3];
+                store_record(out, (c & 1u) != 0u, b, s + ((r >> (8u * place)) & 0xFFu), ((uint32_t)i << 2) | (uint32_t)h,
+                             depth_bits, (in_bins[l] >> (8 * h)) & 0xFFu, lane);
             }
         };
 #pragma unroll
         for (int l = 0; l < VETRAST_MAX_LAYERS; ++l, radius *= 0.5f, ipx *= 0.5f, ipy *= 0.5f)
         {
-            code[l] = 0;
+            code[l] = 0, in_bins[l] = 0;
 #pragma unroll
-            for (int t = 0; t < kTurns; ++t) base[l][t] = 0, leader[l][t] = 0, ranks[l][t] = 0;
+            for (int t = 0; t < kTurns; ++t) base[l][t] = 0, leader[l][t] = 0, ranks[l][t] = 0, bins[l][t] = 0;
             if (l < a.ly.L)
             {
                 if (a.drop_by_radius && radius < a.radius_threshold) dropped = true;
@@ -339,13 +389,14 @@ __global__ void __launch_bounds__(kBlock) bin_count_kernel(ViewPass a, uint32_t*
 #pragma unroll
                 for (int h = 0; h < HITS; ++h)
                 {
-                    uint32_t tile = 0, in_tile = 0, in_bin;
+                    uint32_t tile = 0, in_tile = 0, in_bin = 0;
                     bin[h]         = 0;
                     const bool has = !dropped && layer_hit<HITS>(a.ly, l, ipx, ipy, h, tile, in_tile);
                     if (has)
                     {
                         bin_of_pixel(a.ly, l, tile, in_tile, bin[h], in_bin);
                         left |= 1u << h;
+                        in_bins[l] |= in_bin << (8 * h);
                     }
                 }
 #pragma unroll
@@ -369,12 +420,27 @@ __global__ void __launch_bounds__(kBlock) bin_count_kernel(ViewPass a, uint32_t*
                     const WeightedGroup g = group_by_bin_weighted(has, key, weight, lane);
                     leader[l][t]          = (uint32_t)g.leader;
                     ranks[l][t]           = g.ranks;
+                    bins[l][t]            = key;
                     if (has && g.leader == lane) base[l][t] = atomicAdd(&bin_counts[key], g.total);
                 }
             }
-            if (l >= 1 && l - 1 < a.ly.L) store_slots(l - 1);
+            if (l >= 1 && l - 1 < a.ly.L) store_layer(l - 1);
         }
-        if (VETRAST_MAX_LAYERS - 1 < a.ly.L) store_slots(VETRAST_MAX_LAYERS - 1);
+        if (VETRAST_MAX_LAYERS - 1 < a.ly.L) store_layer(VETRAST_MAX_LAYERS - 1);
+    }
+}
+
+// Brings the logged records (rank beyond the bin's own room) to the bin's place in the compact array:
+// binned[bin_offsets[bin] + rank]. Runs after the scan of the bin counts; the log is empty as a rule.
+__global__ void __launch_bounds__(kBlock) overflow_move_kernel(ScatterTargets in, const uint32_t* __restrict__ bin_offsets,
+                                                                uint4* __restrict__ binned, uint32_t capacity)
+{
+    const uint32_t entries = min(*in.log_cursor, in.log_capacity);
+    for (uint32_t e = blockIdx.x * blockDim.x + threadIdx.x; e < entries; e += gridDim.x * blockDim.x)
+    {
+        const uint4 rec    = in.log[e];
+        const uint32_t pos = bin_offsets[rec.w] + in.log_rank[e];
+        if (pos < capacity) binned[pos] = make_uint4(rec.x, rec.y, rec.z, 0u);  // guard: never false
     }
 }
 
@@ -505,42 +571,6 @@ __global__ void __launch_bounds__(kScanSmallBlock) scan_small_kernel(uint4* __re
     }
 }
 
-// Second projection of every point; its record (64-bit key = depth bits << 32 | point id, pixel inside the bin) goes
-// to the bin's start + the rank the count pass drew. Counterpart of CollectMulti<L,false>
-// (src/lib/rendering/RenderForward.cu:1011-1096), which draws the rank from a second atomic counter image and stores
-// depth and id in two separate rows.
-// In BILINEAR_BLEND (HITS = 4) the low key word is point id << 2 | corner.
-template <int HITS>
-__global__ void __launch_bounds__(kBlock) bin_fill_kernel(ViewPass a, const uint32_t* __restrict__ bin_offsets,
-                                                           const uint32_t* __restrict__ slots,
-                                                           uint4* __restrict__ binned, uint32_t capacity)
-{
-    const int i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (i >= a.N) return;
-    if (point_is_skipped(a, i)) return;
-    Projected p;
-    if (!project_point(*a.view, a.position[i], p)) return;
-    const uint32_t depth_bits = __float_as_uint(p.z);
-    float ipx = p.ipx, ipy = p.ipy, radius = p.radius;
-    // The blend and its backward pass form a fragment's bilinear weight from the point's image position; they read it
-    // from here (8 bytes) instead of projecting the point again for every one of its fragments.
-    if constexpr (HITS == 4) a.projected[i] = make_float2(ipx, ipy);
-    for (int l = 0; l < a.ly.L; ++l, radius *= 0.5f, ipx *= 0.5f, ipy *= 0.5f)
-    {
-        if (a.drop_by_radius && radius < a.radius_threshold) break;
-#pragma unroll
-        for (int h = 0; h < HITS; ++h)
-        {
-            uint32_t tile, in_tile, bin, in_bin;
-            if (!layer_hit<HITS>(a.ly, l, ipx, ipy, h, tile, in_tile)) continue;
-            bin_of_pixel(a.ly, l, tile, in_tile, bin, in_bin);
-            const uint32_t pos = bin_offsets[bin] + slots[(size_t)(l * HITS + h) * a.N + i];
-            const uint32_t low = HITS == 1 ? (uint32_t)i : (((uint32_t)i << 2) | (uint32_t)h);
-            if (pos < capacity) binned[pos] = make_uint4(low, depth_bits, in_bin, 0u);  // guard: never false
-        }
-    }
-}
-
 // Front-to-back blend of one pixel's sorted list read from memory: out += (T*c)*t, T = (1-c)*T, in exactly this order
 // (BlendMulti, src/lib/rendering/RenderForward.cu:1303-1357). The list is walked in chunks of kBlendChunk fragments: all
 // keys of a chunk are loaded first, then all descriptor records, and only then the (strictly sequential) arithmetic
@@ -562,7 +592,7 @@ __device__ __forceinline__ void blend_list_from_memory(const uint64_t* list, uin
             if (base + u < n)
             {
                 const int id = (int)(uint32_t)list[base + u];
-                // an id or texture index out of range cannot come from a list the fill pass wrote; such a fragment is
+                // an id or texture index out of range cannot come from a list the scatter pass wrote; such a fragment is
                 // skipped instead of gathered (the reference asserts on the texture index, RenderForward.cu:1335-1336)
                 if ((uint32_t)id < (uint32_t)N) ti[u] = index ? index[id] : id;
                 if ((uint32_t)ti[u] >= (uint32_t)N) ti[u] = -1;

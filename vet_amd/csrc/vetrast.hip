@@ -351,6 +351,8 @@ int vetrast_workspace_layout_for_mode(int32_t N, int32_t B, int32_t L, int32_t w
     lay->bin_counts_base   = at;
     lay->bin_counts_stride = Tpad * sizeof(uint32_t);
     at += lay->bin_counts_stride * B;
+    lay->log_cursor_base = at;  // right behind the bin counters: one zero-fill covers both
+    at += align_up((size_t)B * sizeof(uint32_t), kAlign);
     lay->scan_partials_base = at;
     at += align_up((Tpad / kScanPerBlock) * sizeof(uint32_t), kAlign);
     lay->offsets_base   = at;
@@ -358,6 +360,10 @@ int vetrast_workspace_layout_for_mode(int32_t N, int32_t B, int32_t L, int32_t w
     at += lay->offsets_stride * B;
     lay->binned_base = at;
     at += align_up(cap * sizeof(uint4), kAlign);
+    lay->log_base = at;
+    at += align_up(cap * sizeof(uint4), kAlign);
+    lay->primary_base = at;
+    at += align_up(bins * (size_t)kPrimaryCap * sizeof(uint4), kAlign);
     lay->views_base = at;
     at += align_up((size_t)B * sizeof(DeviceView), kAlign);
     lay->packed_base = at;
@@ -442,7 +448,7 @@ int vetrast_forward(vetrast_ctx* ctx, const vetrast_forward_args* a, void* strea
     {
         ScopeTimer tm(ctx, stream, VETRAST_SCOPE_PREPARE);
         // per-bin counters of all views (contiguous) start at zero; InitializeData, PointRenderer.cu:402-470
-        const size_t n4  = Tpad * B / 4;
+        const size_t n4  = (Tpad * B * sizeof(uint32_t) + align_up((size_t)B * sizeof(uint32_t), kAlign)) / sizeof(uint4);
         uint4* counters4 = ws_ptr<uint4>(ws, lay.bin_counts_base);
         const int zero_blocks = std::min(grid_for(n4), 1024);
         for (int first = 0; first < B; first += 16)
@@ -475,14 +481,20 @@ int vetrast_forward(vetrast_ctx* ctx, const vetrast_forward_args* a, void* strea
         float* weight       = ws_ptr<float>(ws, lay.weight_base + lay.weight_stride * b);
         uint32_t* bin_counts     = ws_ptr<uint32_t>(ws, lay.bin_counts_base + lay.bin_counts_stride * b);
         uint4* binned            = ws_ptr<uint4>(ws, lay.binned_base);
+        ScatterTargets targets;
+        targets.primary      = ws_ptr<uint4>(ws, lay.primary_base);
+        targets.log          = ws_ptr<uint4>(ws, lay.log_base);
+        targets.log_rank     = slots;
+        targets.log_cursor   = ws_ptr<uint32_t>(ws, lay.log_cursor_base) + b;
+        targets.log_capacity = (uint32_t)lay.fragment_capacity;
         uint8_t* list_is_cut     = ws_ptr<uint8_t>(ws, lay.cut_flags_base + lay.cut_flags_stride * b);
         if (N > 0)
         {
             ScopeTimer tm(ctx, stream, VETRAST_SCOPE_COUNT);
             if (hits == 1)
-                hipLaunchKernelGGL(bin_count_kernel<1>, dim3(grid_for(N)), dim3(kBlock), 0, stream, vp, bin_counts, slots);
+                hipLaunchKernelGGL(bin_scatter_kernel<1>, dim3(grid_for(N)), dim3(kBlock), 0, stream, vp, bin_counts, targets);
             else
-                hipLaunchKernelGGL(bin_count_kernel<4>, dim3(grid_for(N)), dim3(kBlock), 0, stream, vp, bin_counts, slots);
+                hipLaunchKernelGGL(bin_scatter_kernel<4>, dim3(grid_for(N)), dim3(kBlock), 0, stream, vp, bin_counts, targets);
         }
         {
             ScopeTimer tm(ctx, stream, VETRAST_SCOPE_SCAN);
@@ -501,12 +513,9 @@ int vetrast_forward(vetrast_ctx* ctx, const vetrast_forward_args* a, void* strea
         if (N > 0)
         {
             ScopeTimer tm(ctx, stream, VETRAST_SCOPE_FILL);
-            if (hits == 1)
-                hipLaunchKernelGGL(bin_fill_kernel<1>, dim3(grid_for(N)), dim3(kBlock), 0, stream, vp, bin_counts, slots,
-                                   binned, (uint32_t)lay.fragment_capacity);
-            else
-                hipLaunchKernelGGL(bin_fill_kernel<4>, dim3(grid_for(N)), dim3(kBlock), 0, stream, vp, bin_counts, slots,
-                                   binned, (uint32_t)lay.fragment_capacity);
+            // the few records beyond their bin's own room, if any
+            hipLaunchKernelGGL(overflow_move_kernel, dim3(256), dim3(kBlock), 0, stream, targets, bin_counts, binned,
+                               (uint32_t)lay.fragment_capacity);
         }
         float* out[VETRAST_MAX_LAYERS];
         float* out_mask[VETRAST_MAX_LAYERS];
@@ -527,6 +536,7 @@ int vetrast_forward(vetrast_ctx* ctx, const vetrast_forward_args* a, void* strea
             ScopeTimer tm(ctx, stream, VETRAST_SCOPE_BUILD);
             BuildPass bp;
             bp.bin_offsets         = bin_counts;
+            bp.primary             = targets.primary;
             bp.binned              = binned;
             bp.offsets             = offsets;
             bp.fragments           = fragments;
