@@ -156,7 +156,7 @@ typedef struct vetrast_workspace_layout
     size_t cut_flags_base, cut_flags_stride; /* uint8 [P]: 1 where some fragments of the pixel's list did not (top-K cut, saturation) */
     /* shared by all views */
     size_t packed_base;    /* float [N][8]: descriptor (4, zero padded), confidence, 3 pad */
-    size_t slots_base;     /* uint32 [N*L*hits]: rank inside its bin of every record in the overflow log (scratch) */
+    size_t slots_base;     /* uint32, shaped like the log: rank inside its bin of every logged record (scratch) */
     size_t views_base;     /* prepared per-view camera constants */
     size_t scan_partials_base;
     int64_t num_bins;      /* bins of one view: runs of 256 / 64 / 16 / 4 consecutive pixel numbers, chosen per layer from N */
@@ -169,10 +169,10 @@ typedef struct vetrast_workspace_layout
     size_t background_partial_base; /* float [workgroups][8]: backward scratch, per-workgroup background-gradient sums */
     size_t camera_partial_base;     /* double [ceil(N/256)][12]: backward scratch, per-workgroup pose / intrinsics sums */
     /* scratch shared by all views: the scatter pass writes the records of bin b to primary[b][rank] while rank < 2048;
-     * records beyond that go to a log (record + bin, rank in the slots array) and are filed into the compact array
-     * after the scan. log_cursor: uint32 per view, entries in the log. */
+     * records beyond that go to a log of 256 segments (record + bin, rank in the slots array) and are filed into the
+     * compact array after the scan. log_cursor: per view, 256 uint32 64 bytes apart, entries in every segment. */
     size_t primary_base;   /* uint32 [num_bins][2048][4] */
-    size_t log_base;       /* uint32 [N*L*hits][4] */
+    size_t log_base;       /* uint32 [256][ceil(ceil(N/256)/256)*256*L*hits][4] */
     size_t log_cursor_base;
     size_t projected_base, projected_stride; /* per view, float [N][2], BILINEAR_BLEND only (stride 0 otherwise): image
                                                 position of every visible point at layer 0, from which the blend and its

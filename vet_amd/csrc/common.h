@@ -17,6 +17,8 @@ constexpr int kBackgroundRow  = 8;            // floats per workgroup row of bac
 constexpr int kPreparedBackgroundOffset = 16;  // float index inside the flags block: the background as it is blended
 constexpr int kPackedFloats   = 8;            // interleaved record: 4 descriptor floats, confidence, 3 pad
 constexpr int kPrimaryCap     = 2048;         // fragment records every bin has room for (bins are sized for <= 1024 expected)
+constexpr int kLogSegments    = 256;          // the overflow log is cut into this many segments with a cursor each
+constexpr int kLogCursorStride = 16;          // uint32 between two cursors (64 bytes: one cursor per cache line)
 
 // Camera constants of one view, written by prepare_views_kernel and read (uniformly) by every other kernel.
 // Counterpart of what the reference pulls per thread out of d_render_params.Pose()/PinholeIntrinsics() and the

@@ -261,15 +261,17 @@ __device__ __forceinline__ WeightedGroup group_by_bin_weighted(bool has, uint32_
 // Where the scatter pass puts a fragment record (64-bit key = depth bits << 32 | point id, pixel inside the bin).
 // Every bin owns room for kPrimaryCap records; a record whose rank inside its bin is beyond that is appended to a log
 // (with its bin and rank), from where overflow_move_kernel brings it to the bin's place in the compact array once the
-// scan of the bin counts is known. Bins are sized for an expected 1024 records at most, so the log stays empty or
+// scan of the bin counts is known. The log is cut into segments, one per residue of the workgroup number, each with a
+// cursor in a cache line of its own: appends to one cursor would queue up behind each other where many bins overflow
+// (a workgroup's segment has room for every hit the workgroups of that residue can produce). Bins are sized for an expected 1024 records at most, so the log stays empty or
 // short unless the cloud is far denser somewhere than on average.
 struct ScatterTargets
 {
     uint4* primary;        // [bins][kPrimaryCap] records
-    uint4* log;            // [log_capacity]: key low, key high, pixel in bin, bin
-    uint32_t* log_rank;    // [log_capacity]: rank of the logged record inside its bin
-    uint32_t* log_cursor;  // entries in the log (this view)
-    uint32_t log_capacity;
+    uint4* log;            // [kLogSegments][segment_capacity]: key low, key high, pixel in bin, bin
+    uint32_t* log_rank;    // the same shape: rank of the logged record inside its bin
+    uint32_t* log_cursor;  // [kLogSegments], kLogCursorStride apart: entries in every segment (this view)
+    uint32_t segment_capacity;
 };
 
 // One record to its bin; `valid` lanes carry one. Called by the whole wave (uniform control flow).
@@ -281,16 +283,18 @@ __device__ __forceinline__ void store_record(const ScatterTargets& t, bool valid
     const uint64_t m = __ballot(over);
     if (m != 0ull)  // rare
     {
-        const int leader = __ffsll((unsigned long long)m) - 1;
-        uint32_t first   = 0;
-        if (lane == leader) first = atomicAdd(t.log_cursor, (uint32_t)__popcll(m));
+        const uint32_t segment = blockIdx.x % (uint32_t)kLogSegments;
+        const int leader       = __ffsll((unsigned long long)m) - 1;
+        uint32_t first         = 0;
+        if (lane == leader) first = atomicAdd(t.log_cursor + segment * kLogCursorStride, (uint32_t)__popcll(m));
         first = (uint32_t)__shfl((int)first, leader, kWave);
-        const uint32_t pos =
+        const uint32_t at =
             first + __builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)m, 0u));
-        if (over && pos < t.log_capacity)  // guard: the log has room for every hit of the view
+        if (over && at < t.segment_capacity)  // guard: a segment has room for every hit of its workgroups
         {
-            t.log[pos]      = make_uint4(low, depth_bits, in_bin, bin);
-            t.log_rank[pos] = rank;
+            const size_t pos = (size_t)segment * t.segment_capacity + at;
+            t.log[pos]       = make_uint4(low, depth_bits, in_bin, bin);
+            t.log_rank[pos]  = rank;
         }
     }
 }
@@ -435,12 +439,16 @@ __global__ void __launch_bounds__(kBlock) bin_scatter_kernel(ViewPass a, uint32_
 __global__ void __launch_bounds__(kBlock) overflow_move_kernel(ScatterTargets in, const uint32_t* __restrict__ bin_offsets,
                                                                 uint4* __restrict__ binned, uint32_t capacity)
 {
-    const uint32_t entries = min(*in.log_cursor, in.log_capacity);
-    for (uint32_t e = blockIdx.x * blockDim.x + threadIdx.x; e < entries; e += gridDim.x * blockDim.x)
+    for (uint32_t segment = blockIdx.x; segment < (uint32_t)kLogSegments; segment += gridDim.x)
     {
-        const uint4 rec    = in.log[e];
-        const uint32_t pos = bin_offsets[rec.w] + in.log_rank[e];
-        if (pos < capacity) binned[pos] = make_uint4(rec.x, rec.y, rec.z, 0u);  // guard: never false
+        const uint32_t entries = min(in.log_cursor[segment * kLogCursorStride], in.segment_capacity);
+        const size_t first     = (size_t)segment * in.segment_capacity;
+        for (uint32_t e = threadIdx.x; e < entries; e += blockDim.x)
+        {
+            const uint4 rec    = in.log[first + e];
+            const uint32_t pos = bin_offsets[rec.w] + in.log_rank[first + e];
+            if (pos < capacity) binned[pos] = make_uint4(rec.x, rec.y, rec.z, 0u);  // guard: never false
+        }
     }
 }
 

@@ -212,6 +212,16 @@ inline T* ws_ptr(void* ws, size_t off)
 
 // `list_bound[l]`: an upper bound of the mean number of fragments a pixel of layer l blends (null: no layer is split;
 // `split_all`: every layer is, which is what buffers are sized for).
+// The overflow log: workgroup w of the scatter pass appends to segment w % kLogSegments, so a segment needs room for
+// every hit of ceil(workgroups / kLogSegments) workgroups.
+uint32_t log_segment_records(int64_t N, int L, int hits)
+{
+    const int64_t groups = (N + kBlock - 1) / kBlock;
+    return (uint32_t)((groups + kLogSegments - 1) / kLogSegments * kBlock * L * hits);
+}
+size_t log_records(int64_t N, int L, int hits) { return (size_t)log_segment_records(N, L, hits) * kLogSegments; }
+size_t log_cursor_bytes(int B) { return (size_t)B * kLogSegments * kLogCursorStride * sizeof(uint32_t); }
+
 TileMap make_tile_map(const LayerTable& ly, const double* list_bound = nullptr, bool split_all = false)
 {
     TileMap m;
@@ -352,7 +362,7 @@ int vetrast_workspace_layout_for_mode(int32_t N, int32_t B, int32_t L, int32_t w
     lay->bin_counts_stride = Tpad * sizeof(uint32_t);
     at += lay->bin_counts_stride * B;
     lay->log_cursor_base = at;  // right behind the bin counters: one zero-fill covers both
-    at += align_up((size_t)B * sizeof(uint32_t), kAlign);
+    at += log_cursor_bytes(B);
     lay->scan_partials_base = at;
     at += align_up((Tpad / kScanPerBlock) * sizeof(uint32_t), kAlign);
     lay->offsets_base   = at;
@@ -361,7 +371,7 @@ int vetrast_workspace_layout_for_mode(int32_t N, int32_t B, int32_t L, int32_t w
     lay->binned_base = at;
     at += align_up(cap * sizeof(uint4), kAlign);
     lay->log_base = at;
-    at += align_up(cap * sizeof(uint4), kAlign);
+    at += align_up(log_records(N, L, hits) * sizeof(uint4), kAlign);
     lay->primary_base = at;
     at += align_up(bins * (size_t)kPrimaryCap * sizeof(uint4), kAlign);
     lay->views_base = at;
@@ -369,7 +379,7 @@ int vetrast_workspace_layout_for_mode(int32_t N, int32_t B, int32_t L, int32_t w
     lay->packed_base = at;
     at += align_up((size_t)N * kPackedFloats * sizeof(float), kAlign);
     lay->slots_base = at;
-    at += align_up(cap * sizeof(uint32_t), kAlign);
+    at += align_up(log_records(N, L, hits) * sizeof(uint32_t), kAlign);
     lay->weight_base   = at;
     lay->weight_stride = align_up(P * sizeof(float), kAlign);
     at += lay->weight_stride * B;
@@ -448,7 +458,7 @@ int vetrast_forward(vetrast_ctx* ctx, const vetrast_forward_args* a, void* strea
     {
         ScopeTimer tm(ctx, stream, VETRAST_SCOPE_PREPARE);
         // per-bin counters of all views (contiguous) start at zero; InitializeData, PointRenderer.cu:402-470
-        const size_t n4  = (Tpad * B * sizeof(uint32_t) + align_up((size_t)B * sizeof(uint32_t), kAlign)) / sizeof(uint4);
+        const size_t n4  = (Tpad * B * sizeof(uint32_t) + log_cursor_bytes(B)) / sizeof(uint4);
         uint4* counters4 = ws_ptr<uint4>(ws, lay.bin_counts_base);
         const int zero_blocks = std::min(grid_for(n4), 1024);
         for (int first = 0; first < B; first += 16)
@@ -485,8 +495,8 @@ int vetrast_forward(vetrast_ctx* ctx, const vetrast_forward_args* a, void* strea
         targets.primary      = ws_ptr<uint4>(ws, lay.primary_base);
         targets.log          = ws_ptr<uint4>(ws, lay.log_base);
         targets.log_rank     = slots;
-        targets.log_cursor   = ws_ptr<uint32_t>(ws, lay.log_cursor_base) + b;
-        targets.log_capacity = (uint32_t)lay.fragment_capacity;
+        targets.log_cursor   = ws_ptr<uint32_t>(ws, lay.log_cursor_base) + (size_t)b * kLogSegments * kLogCursorStride;
+        targets.segment_capacity = log_segment_records(N, L, hits);
         uint8_t* list_is_cut     = ws_ptr<uint8_t>(ws, lay.cut_flags_base + lay.cut_flags_stride * b);
         if (N > 0)
         {
