@@ -192,7 +192,6 @@ __global__ void __launch_bounds__(kBlock) bin_build_kernel(BuildPass a)
     __shared__ uint8_t s_src_lane[kBlock / kWave][kWave];
     __shared__ uint64_t s_block_sorted[kBlock / kWave];  // pixels whose lists the whole workgroup sorts, a mask per wave
     __shared__ uint64_t s_keys[kBuildCap];
-    __shared__ uint32_t s_used[kTilePixels];   // fragments of the pixel that took part in the blend
     __shared__ uint8_t s_pix[kBuildCap];       // pixel (inside the bin) of every list place
     __shared__ float4 s_stage[kStage][2];      // descriptor, confidence of the staged fragments
     const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
@@ -371,13 +370,15 @@ __global__ void __launch_bounds__(kBlock) bin_build_kernel(BuildPass a)
         }
         if constexpr (FUZZY)
             if (fuzzy.open && fuzzy.m > 0) fuzzy.flush(T, color);
-        s_used[tid] = used;
+        // fragments of the pixel that took part in the blend; the pixel counts are not needed any more (the last read
+        // of them is in front of the closing barrier of the loop above), so their array takes the numbers
+        s_cnt[tid] = used;
         __syncthreads();
         if (a.transmittance)
             for (uint32_t r = tid; r < n; r += kBlock)
             {
                 const uint32_t px = s_pix[r];
-                if (r - s_prefix[px] < s_used[px]) a.transmittance[begin + r] = s_T[2 * r + 1];
+                if (r - s_prefix[px] < s_cnt[px]) a.transmittance[begin + r] = s_T[2 * r + 1];
             }
     }
     else
