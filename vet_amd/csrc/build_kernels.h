@@ -22,7 +22,7 @@ namespace vetrast
 //
 // The LDS capacity is a trade: 2048 records (16 KB of keys, 30 KB in all) kept all but 58 of config 3's 14 400 bins in
 // LDS but let only 5 workgroups share a CU, and a workgroup's life is a chain of memory round trips; with 1024 records
-// (20 KB in all, 7 workgroups per CU) 608 bins stream instead and the pass is still 12 % faster there and 20 % faster
+// (19.8 KB in all, 8 workgroups per CU, the most the hardware holds) 608 bins stream instead and the pass is still 12 % faster there and 20 % faster
 // on the 10 M point cloud.
 constexpr int kBuildPerThread = 4;
 constexpr int kBuildCap       = kBlock * kBuildPerThread;  // 1024 records = 8 KB of keys in LDS
