@@ -107,3 +107,78 @@ def test_random_case(seed, rasterizer, oracle):
         assert np.all(np.isfinite(g)), key
         err = max_rel_err(g, w_) if np.abs(w_).max() > 0 else float(np.abs(g).max())
         assert err <= 1e-4, (key, err)
+
+
+def _draw_clustered(seed):
+    """Scenes whose points crowd into a few spots of the image: bins far beyond the room they own (records go through
+    the overflow log), lists of hundreds to thousands of fragments (every sorting method), with a sparse rest."""
+    rng = np.random.default_rng(5000 + seed)
+    w, h = int(rng.integers(40, 200)), int(rng.integers(30, 120))
+    L = int(rng.integers(1, 5))
+    N = int(rng.choice([20_000, 60_000, 150_000]))
+    K = int(rng.choice([-1, 0, 16, 100]))
+    views = int(rng.integers(1, 3))
+    scene = synthetic.tiny_scene(num_points=N, w=w, h=h, num_layers=L, K=K, seed=6000 + seed, channels=4, num_views=views)
+    spots = int(rng.integers(1, 6))
+    crowd = rng.random(N) < rng.uniform(0.5, 0.95)
+    centre = rng.uniform(-0.6, 0.6, size=(spots, 2))
+    which = rng.integers(0, spots, size=N)
+    spread = rng.choice([0.01, 0.05, 0.15, 0.3])
+    scene.position[crowd, 0] = (centre[which[crowd], 0] + rng.normal(size=int(crowd.sum())) * spread).astype(np.float32)
+    scene.position[crowd, 1] = (centre[which[crowd], 1] * 0.6 + rng.normal(size=int(crowd.sum())) * spread).astype(np.float32)
+    if rng.random() < 0.5:  # depth ties
+        scene.position[:, 2] = (np.round(scene.position[:, 2] / 0.05) * 0.05).astype(np.float32)
+    scene.position = np.ascontiguousarray(scene.position[rng.permutation(N)])
+    over = {
+        "render_mode": int(rng.choice([1, 2, 3])),
+        "depth_accept_blend": 0.05,
+        "need_point_gradient": 1,
+        "drop_out_points_by_radius": int(rng.random() < 0.2),
+        "use_environment_map": int(rng.random() < 0.3),
+    }
+    return scene, over
+
+
+@pytest.mark.parametrize("seed", list(range(12)))
+def test_random_clustered_case(seed, rasterizer, oracle):
+    scene, over = _draw_clustered(seed)
+    print(f"[case] clustered sweep seed={seed} N={scene.num_points} {scene.views[0].w}x{scene.views[0].h} "
+          f"L={scene.num_layers} K={scene.max_list_length} views={len(scene.views)} {over}", flush=True)
+    params = make_params(scene, **over)
+    ref = oracle.forward(scene, params, num_threads=8)
+    dev = DeviceScene(scene)
+    res = rasterizer.forward(dev, params, save_for_backward=True)
+    torch.cuda.synchronize()
+    K = params.debug_max_list_length
+    bilinear = over["render_mode"] == abi.RENDER_BILINEAR_BLEND
+    longest = 0
+    for b in range(len(scene.views)):
+        off = res.offsets(b)
+        np.testing.assert_array_equal(off, ref.offsets[b].astype(np.int64), err_msg="per-pixel counts")
+        total = int(off[-1])
+        counts = np.diff(off)
+        longest = max(longest, int(counts.max()))
+        if bilinear:
+            kept = res.kept(b)
+            np.testing.assert_array_equal(kept, ref.kept[b].astype(np.int64), err_msg="blended counts")
+            keep = (np.arange(total) - np.repeat(off[:-1], counts)) < np.repeat(kept, counts)
+        else:
+            keep = kept_mask(off, K)
+        np.testing.assert_array_equal(res.fragments(b)[keep], ref.fragments[b, :total][keep], err_msg="lists")
+        np.testing.assert_array_equal(res.transmittance(b)[keep], ref.transmittance[b, :total][keep], err_msg="T")
+        np.testing.assert_array_equal(res.weight(b), ref.weight[b], err_msg="weight")
+    print(f"  longest list {longest}", flush=True)
+    for l in range(scene.num_layers):
+        np.testing.assert_array_equal(res.out[l].cpu().numpy(), ref.out[l], err_msg=f"layer {l}")
+    tol = 1e-4  # also for uncut lists of tens of thousands of fragments
+    grad_out = scene.grad_out()
+    want = oracle.backward(ref, grad_out, num_threads=8)
+    got = rasterizer.backward(res, [torch.from_numpy(g).cuda() for g in grad_out])
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(got["point_count"].cpu().numpy(), want["point_count"])
+    for key in ("texture", "confidence", "points"):
+        g, w_ = got[key].cpu().numpy(), want[key]
+        assert np.all(np.isfinite(g)), key
+        err = max_rel_err(g, w_) if np.abs(w_).max() > 0 else float(np.abs(g).max())
+        print(f"  {key}: max rel err {err:.3e}", flush=True)
+        assert err <= tol, (key, err)
