@@ -350,7 +350,7 @@ __global__ void __launch_bounds__(kBlock) blend_backward_kernel(BackwardPass a)
 }
 
 // FUZZY_BLEND, per-pixel part of the backward pass: BlendBackwardsFuzzy<C>, src/lib/rendering/RenderBackward.cu:570-1080.
-// One thread per pixel walks its (cut) list front to back. Fragments are collected into a bucket while their depth
+// One lane per pixel walks its (cut) list front to back. Fragments are collected into a bucket while their depth
 // stays within depth_accept of the bucket's first one (every bucket, unlike the forward kernel, which only averages
 // the nearest one); the background, at depth 1e5, ends up in a bucket of its own. With the bucket's mean confidence c,
 // mean descriptor t, m elements and the transmittance A in front of it:
@@ -359,7 +359,187 @@ __global__ void __launch_bounds__(kBlock) blend_backward_kernel(BackwardPass a)
 // reference hands every element in front of a bucket the bucket's whole term, :654-672). The reference walks all
 // elements in front for every bucket; here the list is walked twice, first for the total of the bucket terms, then
 // with a running prefix, so that S_b = total - prefix. The position part (:729-1080) is the neighbour-difference
-// heuristic of the FULL_BLEND kernel. Records go to partial[layer][point] as there.
+// heuristic of the FULL_BLEND kernel. Records go to partial[layer][point] as there: the position part of an element's
+// record when the element is met in the second pass, the rest when its bucket closes, for which only the keys of the
+// bucket's elements are read again (gathering the descriptor records a third time cost a third of the kernel).
+
+// State of one pixel's walk over its list (one of the two passes at a time).
+template <int C>
+struct FuzzyWalk
+{
+    // the pixel
+    const BackwardPass* a;
+    const uint64_t* list;
+    float4* partial_l;
+    uint32_t n;  // fragments (after the cut)
+    float g[C], ax[C], ay[C], bx, by;
+    bool do_point;
+    float depth_accept;
+    float bg_grad[C];
+    double total, prefix;
+    // the pass
+    int pass;
+    float last_min, acc_conf, A, acc_t[C];
+    uint32_t m, start;
+    int first_id;  // point of the open bucket's first element
+
+    // Descriptor and confidence of list element e from memory; the background is the element behind the last fragment.
+    __device__ __forceinline__ void element(uint32_t e, float (&t)[C], float& conf, float& depth, int& id) const
+    {
+        id = -1;
+        if (e >= n)
+        {
+#pragma unroll
+            for (int ci = 0; ci < C; ++ci) t[ci] = a->background[ci];
+            conf  = 1.f;
+            depth = 100000.f;  // MAX_DEPTH_CONST, src/lib/rendering/RenderConstants.h:30
+            return;
+        }
+        const uint64_t key = list[e];
+        depth              = __uint_as_float((uint32_t)(key >> 32));
+        const int point    = (int)(uint32_t)key;
+        int ti             = -1;
+        if ((uint32_t)point < (uint32_t)a->N) ti = a->index ? a->index[point] : point;
+        float4 t4 = make_float4(0.f, 0.f, 0.f, 0.f);
+        conf      = 0.f;
+        if ((uint32_t)ti < (uint32_t)a->N)
+        {
+            t4   = a->packed[2 * (size_t)ti];
+            conf = a->packed[2 * (size_t)ti + 1].x;
+            id   = point;
+        }
+        const float tt[4] = {t4.x, t4.y, t4.z, t4.w};
+#pragma unroll
+        for (int ci = 0; ci < C; ++ci) t[ci] = tt[ci];
+    }
+
+    __device__ __forceinline__ void begin_pass(int which)
+    {
+        pass     = which;
+        last_min = 0.f, acc_conf = 0.f, A = 1.f;
+#pragma unroll
+        for (int ci = 0; ci < C; ++ci) acc_t[ci] = 0.f;
+        m = 0, start = 0, first_id = -1;
+    }
+
+    // closes the bucket [start, start + m)
+    __device__ __forceinline__ void close_bucket()
+    {
+        const float inv  = 1.f / (float)m;
+        const float conf = acc_conf * inv;
+        float tb[C];
+        float dot = 0.f, x = 0.f;
+#pragma unroll
+        for (int ci = 0; ci < C; ++ci)
+        {
+            tb[ci] = acc_t[ci] * inv;
+            dot += tb[ci] * g[ci];
+            x += ((g[ci] * tb[ci]) * A) * conf;
+        }
+        if (pass == 0)
+            total += (double)x;
+        else
+        {
+            prefix += (double)x;
+            const float S      = (float)(total - prefix);
+            const float galpha = dot * A;
+            const float gconf  = galpha * inv - S / ((1.f - conf) + 1e-9f);
+            float gt[4]        = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int ci = 0; ci < C; ++ci) gt[ci] = ((A * conf) * g[ci]) * inv;
+            // every element of the bucket gets the bucket's descriptor and confidence gradient; the position part of
+            // its record was written when the element was consumed. Only the point ids are needed here: the keys are
+            // read again (neighbouring places, in cache), eight at a time so that the loads overlap, not the
+            // descriptor records.
+            auto give = [&](int id) {
+                partial_l[2 * (size_t)id] = make_float4(gt[0], gt[1], gt[2], gt[3]);
+                reinterpret_cast<float*>(&partial_l[2 * (size_t)id + 1])[0] = gconf;
+            };
+            if (m == 1)
+            {
+                if (start >= n)
+                {
+#pragma unroll
+                    for (int ci = 0; ci < C; ++ci) bg_grad[ci] += gt[ci];
+                }
+                else if (first_id >= 0)
+                    give(first_id);
+            }
+            else
+                for (uint32_t e0 = start; e0 < start + m; e0 += 8)
+                {
+                    int point[8];
+#pragma unroll
+                    for (int u = 0; u < 8; ++u)
+                    {
+                        const uint32_t e = e0 + u;
+                        point[u]         = (e < start + m && e < n) ? (int)(uint32_t)list[e] : -1;
+                    }
+#pragma unroll
+                    for (int u = 0; u < 8; ++u)
+                    {
+                        const uint32_t e = e0 + u;
+                        if (e >= start + m) break;
+                        if (e >= n)
+                        {
+#pragma unroll
+                            for (int ci = 0; ci < C; ++ci) bg_grad[ci] += gt[ci];
+                            continue;
+                        }
+                        int ti = -1;
+                        if ((uint32_t)point[u] < (uint32_t)a->N) ti = a->index ? a->index[point[u]] : point[u];
+                        if ((uint32_t)ti < (uint32_t)a->N) give(point[u]);
+                    }
+                }
+        }
+        A = (1.f - conf) * A;
+    }
+
+    // list element i joins the open bucket or starts the next one
+    __device__ __forceinline__ void consume(uint32_t i, const float (&t)[C], float conf, float d, int id)
+    {
+        if (!(d - last_min < depth_accept))
+        {
+            if (i != 0) close_bucket();
+            acc_conf = 0.f;
+            m        = 0;
+#pragma unroll
+            for (int ci = 0; ci < C; ++ci) acc_t[ci] = 0.f;
+            last_min = d;
+            start    = i;
+            first_id = id;
+        }
+        acc_conf += conf;
+#pragma unroll
+        for (int ci = 0; ci < C; ++ci) acc_t[ci] += t[ci];
+        ++m;
+        if (pass == 1 && id >= 0)
+        {
+            // the position part of the element's record does not depend on its bucket
+            float gp0 = 0.f, gp1 = 0.f;
+            if (do_point)
+            {
+                float dR_dpx = bx, dR_dpy = by;
+#pragma unroll
+                for (int ci = 0; ci < C; ++ci)
+                {
+                    dR_dpx += t[ci] * ax[ci];
+                    dR_dpy += t[ci] * ay[ci];
+                }
+                gp0 = dR_dpx / (float)C;
+                gp1 = dR_dpy / (float)C;
+            }
+            float* rec = reinterpret_cast<float*>(&partial_l[2 * (size_t)id + 1]);
+            rec[1] = gp0, rec[2] = gp1, rec[3] = 0.f;
+        }
+    }
+
+    __device__ __forceinline__ void end_pass()
+    {
+        if (m > 0) close_bucket();
+    }
+};
+
 template <int C>
 __global__ void __launch_bounds__(kBlock) blend_backward_fuzzy_kernel(BackwardPass a, float depth_accept)
 {
@@ -368,9 +548,12 @@ __global__ void __launch_bounds__(kBlock) blend_backward_fuzzy_kernel(BackwardPa
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
     const TilePixel px = tile_pixel(a.tiles, a.ly);
     const int l        = px.l;
-    float bg_grad[C];
+    FuzzyWalk<C> w;
+    w.a = &a, w.list = a.fragments, w.partial_l = a.partial + 2 * (size_t)l * a.N, w.n = 0, w.bx = w.by = 0.f;
+    w.do_point = false, w.depth_accept = depth_accept, w.total = w.prefix = 0.0;
 #pragma unroll
-    for (int ci = 0; ci < C; ++ci) bg_grad[ci] = 0.f;
+    for (int ci = 0; ci < C; ++ci) w.g[ci] = w.ax[ci] = w.ay[ci] = w.bg_grad[ci] = 0.f;
+    bool with_background = false;  // the list ends with the background element
 
     if (px.active)
     {
@@ -378,22 +561,18 @@ __global__ void __launch_bounds__(kBlock) blend_backward_fuzzy_kernel(BackwardPa
         const size_t plane   = (size_t)lw * lh;
         const uint32_t local = px.local;
         const float* G       = a.grad_out[l];
-        float g[C];
 #pragma unroll
-        for (int ci = 0; ci < C; ++ci) g[ci] = G[ci * plane + local];
+        for (int ci = 0; ci < C; ++ci) w.g[ci] = G[ci * plane + local];
         const uint32_t off = a.offsets[px.q];
         uint32_t n         = a.offsets[px.q + 1] - off;
         if (a.K > 0) n = min(n, (uint32_t)a.K);
-        const uint64_t* list = a.fragments + off;
-        float4* partial_l    = a.partial + 2 * (size_t)l * a.N;
-        const uint32_t list_size = a.use_environment_map ? n : n + 1;
+        w.n               = n;
+        w.list            = a.fragments + off;
+        with_background   = !a.use_environment_map;
 
         // position heuristic of this pixel in slope / offset form (see blend_backward_kernel)
-        const bool do_point = a.need_point_gradient && n > 0 && interior_pixel(px.x, px.y, lw, lh);
-        float ax[C], ay[C], bx = 0.f, by = 0.f;
-#pragma unroll
-        for (int ci = 0; ci < C; ++ci) ax[ci] = ay[ci] = 0.f;
-        if (do_point)
+        w.do_point = a.need_point_gradient && n > 0 && interior_pixel(px.x, px.y, lw, lh);
+        if (w.do_point)
         {
             const float* I = a.out[l];
 #pragma unroll
@@ -403,134 +582,38 @@ __global__ void __launch_bounds__(kBlock) blend_backward_fuzzy_kernel(BackwardPa
                 const float* Gc = G + ci * plane + local;
                 const float Ix0 = Ic[-1], Ix1 = Ic[1], Iy0 = Ic[-lw], Iy1 = Ic[lw];
                 const float Gx0 = Gc[-1], Gx1 = Gc[1], Gy0 = Gc[-lw], Gy1 = Gc[lw];
-                ax[ci] = 0.5f * (Gx1 - Gx0);
-                ay[ci] = 0.5f * (Gy1 - Gy0);
-                bx += 0.5f * (Ix0 * Gx0 - Ix1 * Gx1);
-                by += 0.5f * (Iy0 * Gy0 - Iy1 * Gy1);
+                w.ax[ci] = 0.5f * (Gx1 - Gx0);
+                w.ay[ci] = 0.5f * (Gy1 - Gy0);
+                w.bx += 0.5f * (Ix0 * Gx0 - Ix1 * Gx1);
+                w.by += 0.5f * (Iy0 * Gy0 - Iy1 * Gy1);
             }
         }
-
-        // Descriptor and confidence of list element e; the background is the element behind the last fragment.
-        auto element = [&](uint32_t e, float (&t)[C], float& conf, float& depth, int& id) {
-            id = -1;
-            if (e >= n)
-            {
-#pragma unroll
-                for (int ci = 0; ci < C; ++ci) t[ci] = a.background[ci];
-                conf  = 1.f;
-                depth = 100000.f;  // MAX_DEPTH_CONST, src/lib/rendering/RenderConstants.h:30
-                return;
-            }
-            const uint64_t key = list[e];
-            depth              = __uint_as_float((uint32_t)(key >> 32));
-            const int point    = (int)(uint32_t)key;
-            int ti             = -1;
-            if ((uint32_t)point < (uint32_t)a.N) ti = a.index ? a.index[point] : point;
-            float4 t4 = make_float4(0.f, 0.f, 0.f, 0.f);
-            conf      = 0.f;
-            if ((uint32_t)ti < (uint32_t)a.N)
-            {
-                t4   = a.packed[2 * (size_t)ti];
-                conf = a.packed[2 * (size_t)ti + 1].x;
-                id   = point;
-            }
-            const float tt[4] = {t4.x, t4.y, t4.z, t4.w};
-#pragma unroll
-            for (int ci = 0; ci < C; ++ci) t[ci] = tt[ci];
-        };
-
-        double total = 0.0, prefix = 0.0;
+    }
 #pragma unroll 1
-        for (int pass = 0; pass < 2; ++pass)
+    for (int pass = 0; pass < 2; ++pass)
+    {
+        w.begin_pass(pass);
+        for (uint32_t i = 0; i < w.n; ++i)
         {
-            float last_min = 0.f, acc_conf = 0.f, A = 1.f;
-            float acc_t[C];
-#pragma unroll
-            for (int ci = 0; ci < C; ++ci) acc_t[ci] = 0.f;
-            uint32_t m = 0, start = 0;
-            // closes the bucket [start, start + m)
-            auto close_bucket = [&]() {
-                const float inv  = 1.f / (float)m;
-                const float conf = acc_conf * inv;
-                float tb[C];
-                float dot = 0.f, x = 0.f;
-#pragma unroll
-                for (int ci = 0; ci < C; ++ci)
-                {
-                    tb[ci] = acc_t[ci] * inv;
-                    dot += tb[ci] * g[ci];
-                    x += ((g[ci] * tb[ci]) * A) * conf;
-                }
-                if (pass == 0)
-                    total += (double)x;
-                else
-                {
-                    prefix += (double)x;
-                    const float S      = (float)(total - prefix);
-                    const float galpha = dot * A;
-                    const float gconf  = galpha * inv - S / ((1.f - conf) + 1e-9f);
-                    float gt[4]        = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                    for (int ci = 0; ci < C; ++ci) gt[ci] = ((A * conf) * g[ci]) * inv;
-                    for (uint32_t e = start; e < start + m; ++e)
-                    {
-                        if (e >= n)
-                        {
-#pragma unroll
-                            for (int ci = 0; ci < C; ++ci) bg_grad[ci] += gt[ci];
-                            continue;
-                        }
-                        float te[C], ce, de;
-                        int id;
-                        element(e, te, ce, de, id);
-                        if (id < 0) continue;
-                        float gp0 = 0.f, gp1 = 0.f;
-                        if (do_point)
-                        {
-                            float dR_dpx = bx, dR_dpy = by;
-#pragma unroll
-                            for (int ci = 0; ci < C; ++ci)
-                            {
-                                dR_dpx += te[ci] * ax[ci];
-                                dR_dpy += te[ci] * ay[ci];
-                            }
-                            gp0 = dR_dpx / (float)C;
-                            gp1 = dR_dpy / (float)C;
-                        }
-                        partial_l[2 * (size_t)id]     = make_float4(gt[0], gt[1], gt[2], gt[3]);
-                        partial_l[2 * (size_t)id + 1] = make_float4(gconf, gp0, gp1, 0.f);
-                    }
-                }
-                A = (1.f - conf) * A;
-            };
-            for (uint32_t i = 0; i < list_size; ++i)
-            {
-                float t[C], conf, d;
-                int id;
-                element(i, t, conf, d, id);
-                if (!(d - last_min < depth_accept))
-                {
-                    if (i != 0) close_bucket();
-                    acc_conf = 0.f;
-                    m        = 0;
-#pragma unroll
-                    for (int ci = 0; ci < C; ++ci) acc_t[ci] = 0.f;
-                    last_min = d;
-                    start    = i;
-                }
-                acc_conf += conf;
-#pragma unroll
-                for (int ci = 0; ci < C; ++ci) acc_t[ci] += t[ci];
-                ++m;
-            }
-            if (m > 0) close_bucket();
+            float t[C], conf, d;
+            int id;
+            w.element(i, t, conf, d, id);
+            w.consume(i, t, conf, d, id);
         }
+        if (with_background)
+        {
+            float t[C], conf, d;
+            int id;
+            w.element(w.n, t, conf, d, id);  // the background behind the last fragment
+            w.consume(w.n, t, conf, d, id);
+        }
+        w.end_pass();
     }
 
 #pragma unroll
     for (int ci = 0; ci < C; ++ci)
     {
-        const float s = wave_sum(bg_grad[ci]);
+        const float s = wave_sum(w.bg_grad[ci]);
         if (lane == 0) red[wave][ci] = s;
     }
     if (lane == 0) red[wave][C] = 0.f;  // no background-confidence leak in this mode (guarded, RenderBackward.cu:643)
