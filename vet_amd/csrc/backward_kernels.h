@@ -36,10 +36,17 @@ struct BackwardPass
     int quirk_background_confidence_leak;
 };
 
+// Sum over the 64 lanes (xor butterfly, widest step first); every lane gets the total. The four steps inside a row of
+// 16 lanes are DPP moves, only the two widest go through the LDS crossbar.
 __device__ __forceinline__ float wave_sum(float v)
 {
-#pragma unroll
-    for (int d = kWave / 2; d >= 1; d >>= 1) v += __shfl_xor(v, d, kWave);
+    const int lane = threadIdx.x & (kWave - 1);
+    v += __uint_as_float(lane_xor<32>(__float_as_uint(v), lane));
+    v += __uint_as_float(lane_xor<16>(__float_as_uint(v), lane));
+    v += __uint_as_float(lane_xor<8>(__float_as_uint(v), lane));
+    v += __uint_as_float(lane_xor<4>(__float_as_uint(v), lane));
+    v += __uint_as_float(lane_xor<2>(__float_as_uint(v), lane));
+    v += __uint_as_float(lane_xor<1>(__float_as_uint(v), lane));
     return v;
 }
 

@@ -58,6 +58,36 @@ struct LayerTable
     uint32_t bin_base[VETRAST_MAX_LAYERS + 1];  // first bin of the layer; [L] = number of bins
 };
 
+// Value of lane (lane ^ M) for the xor patterns a 64-wide bitonic network needs. Inside a row of 16 lanes the exchange
+// is a DPP move (register to register, a few cycles); only the four patterns that cross rows go through the LDS
+// crossbar (ds_swizzle within 32 lanes, ds_bpermute across the halves).
+template <int CTRL>
+__device__ __forceinline__ uint32_t dpp_move(uint32_t v)
+{
+    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, 0xF, 0xF, false);
+}
+
+template <int M>
+__device__ __forceinline__ uint32_t lane_xor(uint32_t v, int lane)
+{
+    if constexpr (M == 1) return dpp_move<0xB1>(v);         // quad_perm [1,0,3,2]
+    else if constexpr (M == 2) return dpp_move<0x4E>(v);    // quad_perm [2,3,0,1]
+    else if constexpr (M == 3) return dpp_move<0x1B>(v);    // quad_perm [3,2,1,0]
+    else if constexpr (M == 7) return dpp_move<0x141>(v);   // row_half_mirror
+    else if constexpr (M == 15) return dpp_move<0x140>(v);  // row_mirror
+    else if constexpr (M == 8) return dpp_move<0x128>(v);   // row_ror:8
+    else if constexpr (M == 4)
+    {
+        // banks (groups of 4 lanes) 0 and 2 read lane+4 (row_shl:4), banks 1 and 3 read lane-4 (row_shr:4)
+        int t = __builtin_amdgcn_update_dpp((int)v, (int)v, 0x104, 0xF, 0x5, false);
+        t     = __builtin_amdgcn_update_dpp(t, (int)v, 0x114, 0xF, 0xA, false);
+        return (uint32_t)t;
+    }
+    else if constexpr (M == 16) return (uint32_t)__builtin_amdgcn_ds_swizzle((int)v, 0x401F);  // xor 0x10, and 0x1F
+    else if constexpr (M == 31) return (uint32_t)__builtin_amdgcn_ds_swizzle((int)v, 0x7C1F);  // xor 0x1F, and 0x1F
+    else return (uint32_t)__builtin_amdgcn_ds_bpermute((lane ^ M) << 2, (int)v);               // 32, 63
+}
+
 // Launch descriptor shared by the forward kernels of one view.
 struct ViewPass
 {
