@@ -197,13 +197,7 @@ __global__ void __launch_bounds__(kBlock) blend_backward_kernel(BackwardPass a)
         top -= width;
         const uint32_t jw = top;
         const uint32_t nw = (n > jw) ? min(n - jw, width) : 0u;
-        uint32_t incl     = nw;
-#pragma unroll
-        for (int d = 1; d < kWave; d <<= 1)
-        {
-            const uint32_t o = __shfl_up(incl, d, kWave);
-            if (lane >= d) incl += o;
-        }
+        const uint32_t incl = wave_inclusive_scan(nw, lane);
         const uint32_t base  = incl - nw;
         const uint32_t total = __shfl(incl, kWave - 1, kWave);
         s_base[wave][lane]   = base;

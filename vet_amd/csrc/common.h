@@ -88,6 +88,26 @@ __device__ __forceinline__ uint32_t lane_xor(uint32_t v, int lane)
     else return (uint32_t)__builtin_amdgcn_ds_bpermute((lane ^ M) << 2, (int)v);               // 32, 63
 }
 
+// Inclusive prefix sum over the 64 lanes, all of which must be active: four shift-and-add steps inside every row of 16
+// lanes, then the last lane of row 0 (2) is added to row 1 (3) and lane 31 to the upper half; six DPP adds, no LDS
+// permute (lanes a shift leaves without a source add zero).
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ uint32_t dpp_shifted(uint32_t x)
+{
+    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, CTRL, ROW_MASK, 0xF, false);
+}
+
+__device__ __forceinline__ uint32_t wave_inclusive_scan(uint32_t v, int /*lane*/)
+{
+    v += dpp_shifted<0x111, 0xF>(v);  // row_shr:1
+    v += dpp_shifted<0x112, 0xF>(v);  // row_shr:2
+    v += dpp_shifted<0x114, 0xF>(v);  // row_shr:4
+    v += dpp_shifted<0x118, 0xF>(v);  // row_shr:8
+    v += dpp_shifted<0x142, 0xA>(v);  // row_bcast:15 into rows 1 and 3
+    v += dpp_shifted<0x143, 0xC>(v);  // row_bcast:31 into rows 2 and 3
+    return v;
+}
+
 // Launch descriptor shared by the forward kernels of one view.
 struct ViewPass
 {

@@ -457,17 +457,6 @@ __global__ void __launch_bounds__(kBlock) overflow_move_kernel(ScatterTargets in
 // hundred values, cache resident), then scans its own 4096 counts. No workgroup waits for another one.
 // Counterpart of thrust::exclusive_scan + the two .item<int>() read-backs (src/lib/rendering/PointRenderer.cu:799-813);
 // the total lands at counts[T] because the array is zero padded behind the T tile counts.
-__device__ __forceinline__ uint32_t wave_inclusive_scan(uint32_t v, int lane)
-{
-#pragma unroll
-    for (int d = 1; d < kWave; d <<= 1)
-    {
-        const uint32_t o = __shfl_up(v, d, kWave);
-        if (lane >= d) v += o;
-    }
-    return v;
-}
-
 __device__ __forceinline__ uint32_t block_reduce_sum(uint32_t v, uint32_t* lds4)
 {
 #pragma unroll
