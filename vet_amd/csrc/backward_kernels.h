@@ -252,21 +252,25 @@ __global__ void __launch_bounds__(kBlock) blend_backward_kernel(BackwardPass a)
                     x += ((g[ci] * t[ci]) * T) * c;
                 }
             }
-            // suffix sum over the fragments of the same pixel that sit in higher lanes of this step
+            // suffix sum over the fragments of the same pixel that sit in higher lanes of this step. The fragments of a
+            // pixel are neighbouring lanes: `last` is the end of this lane's run, found from the mask of run starts, so
+            // that the scan steps only have to move the sums.
+            const int pp         = __shfl_up(p, 1, kWave);
+            const bool head      = lane == 0 || pp != p;
+            const uint64_t heads = __ballot(head);
+            const uint64_t above = lane == kWave - 1 ? 0ull : heads >> (lane + 1);
+            const int last       = above != 0ull ? lane + __ffsll((unsigned long long)above) - 1 : kWave - 1;
             float v = x;
 #pragma unroll
             for (int d = 1; d < kWave; d <<= 1)
             {
                 const float o = __shfl_down(v, d, kWave);
-                const int po  = __shfl_down(p, d, kWave);
-                if (lane + d < kWave && po == p) v += o;
+                if (lane + d <= last) v += o;
             }
             const float vn = __shfl_down(v, 1, kWave);
-            const int pn   = __shfl_down(p, 1, kWave);
-            const int pp   = __shfl_up(p, 1, kWave);
-            float S        = (lane + 1 < kWave && pn == p) ? vn : 0.f;  // deeper fragments of this step
+            float S        = lane < last ? vn : 0.f;                     // deeper fragments of this step
             if (valid) S += s_carry[wave][p];                            // and of the steps / windows before
-            if (valid && (lane == 0 || pp != p)) s_carry[wave][p] += v;  // one lane per pixel moves the carry on
+            if (valid && head) s_carry[wave][p] += v;                    // one lane per pixel moves the carry on
             float4 rec_lo = make_float4(0.f, 0.f, 0.f, 0.f), rec_hi = rec_lo;
             if (ti >= 0)
             {
