@@ -92,6 +92,9 @@ def test_workspace_layout_is_aligned_and_disjoint():
     assert lay.layer_tile_base[L] == T and lay.layer_pixel_base[L] == P and lay.fragment_capacity == N * L
     assert [lay.layer_tiles_x[l] for l in range(L)] == [120, 60, 30, 15]
     assert [lay.layer_tile_base[l] for l in range(L)] == [0, tiles[0], tiles[0] + tiles[1], sum(tiles[:3])]
+    # the overflow log: 256 segments, each with room for every hit of ceil(workgroups / 256) workgroups of 256 points
+    groups = (N + 255) // 256
+    log_records = 256 * ((groups + 255) // 256 * 256 * L)
     regions = [
         ("flags", lay.flags_base, 16),
         ("offsets", lay.offsets_base, lay.offsets_stride * B),
@@ -103,7 +106,10 @@ def test_workspace_layout_is_aligned_and_disjoint():
         ("transmittance", lay.transmittance_base, lay.transmittance_stride * B),
         ("weight", lay.weight_base, lay.weight_stride * B),
         ("packed", lay.packed_base, N * 32),
-        ("slots", lay.slots_base, N * L * 4),
+        ("slots", lay.slots_base, log_records * 4),
+        ("log", lay.log_base, log_records * 16),
+        ("log_cursor", lay.log_cursor_base, B * 256 * 64),
+        ("primary", lay.primary_base, lay.num_bins * 2048 * 16),
         ("views", lay.views_base, B * 128),
         ("partial", lay.partial_base, N * L * 32),
         ("background_partial", lay.background_partial_base, (P + 255) // 256 * 32),
@@ -120,6 +126,12 @@ def test_workspace_layout_is_aligned_and_disjoint():
     for (n0, b0, s0), (n1, b1, _) in zip(ordered, ordered[1:]):
         assert b0 + s0 <= b1, (n0, n1)
     assert lay.forward_only_bytes <= lay.partial_base < lay.total_bytes
+    # the log cursors sit right behind the bin counters (one zero-fill covers both); BILINEAR_BLEND adds `projected`
+    assert lay.log_cursor_base == lay.bin_counts_base + lay.bin_counts_stride * B
+    assert lay.projected_stride == 0
+    lay3 = abi.WorkspaceLayout()
+    assert lib.vetrast_workspace_layout_for_mode(N, B, L, w, h, abi.RENDER_BILINEAR_BLEND, C.byref(lay3)) == 0
+    assert lay3.projected_stride >= N * 8 and lay3.projected_base + lay3.projected_stride * B <= lay3.forward_only_bytes
     assert lib.vetrast_forward_workspace_bytes(N, B, L, w, h) == lay.total_bytes
     # invalid dimensions
     assert lib.vetrast_workspace_layout_for(N, 0, L, w, h, C.byref(lay)) == abi.ERR_INVALID_ARG
