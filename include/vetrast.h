@@ -174,6 +174,8 @@ typedef struct vetrast_workspace_layout
     size_t primary_base;   /* uint32 [num_bins][2048][4] */
     size_t log_base;       /* uint32 [256][ceil(ceil(N/256)/256)*256*L*hits][4] */
     size_t log_cursor_base;
+    size_t last_key_base, last_key_stride;   /* per view, uint64 [P]: where cut_flags is 1, the key of the last fragment of
+                                                the pixel's list that took part in the blend (0 if none did) */
     size_t projected_base, projected_stride; /* per view, float [N][2], BILINEAR_BLEND only (stride 0 otherwise): image
                                                 position of every visible point at layer 0, from which the blend and its
                                                 backward pass form the bilinear weights */

@@ -96,6 +96,7 @@ class WorkspaceLayout(C.Structure):
         ("background_partial_base", C.c_size_t),
         ("camera_partial_base", C.c_size_t),
         ("primary_base", C.c_size_t), ("log_base", C.c_size_t), ("log_cursor_base", C.c_size_t),
+        ("last_key_base", C.c_size_t), ("last_key_stride", C.c_size_t),
         ("projected_base", C.c_size_t), ("projected_stride", C.c_size_t),
     ]
 

@@ -722,6 +722,7 @@ struct GatherPass
     const uint32_t* offsets;
     const uint64_t* fragments;
     const uint8_t* list_is_cut;  // per pixel, written by the build pass
+    const uint64_t* last_key;    // per pixel with list_is_cut: key of the last fragment that took part in the blend
     const uint32_t* kept;        // per pixel, BILINEAR_BLEND: fragments of its list that took part in the blend
     const float4* partial;
     float* grad_texture;      // [C,N]
@@ -803,9 +804,8 @@ __global__ void __launch_bounds__(kBlock) gather_point_gradients_kernel(GatherPa
             // K <= 0 into an index.)
             if (a.list_is_cut[q] && (HITS != 1 || a.K > 0))
             {
-                const uint32_t nk  = HITS == 1 ? (uint32_t)a.K : a.kept[q];  // FULL_BLEND: cut means count > K > 0
                 const uint64_t key = depth_key | (HITS == 1 ? (uint32_t)i : (((uint32_t)i << 2) | (uint32_t)h));
-                if (nk == 0 || key > a.fragments[a.offsets[q] + nk - 1]) continue;
+                if (key > a.last_key[q]) continue;  // 0 where no fragment was blended: every key is beyond it
             }
             const size_t rec = (size_t)(l * HITS + h) * a.vp.N + i;
             const float4 r0  = a.partial[2 * rec];

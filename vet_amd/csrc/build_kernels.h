@@ -37,6 +37,7 @@ struct BuildPass
     uint32_t* offsets;    // [P + 1] per pixel: start of its list; [P] = fragments of the view
     uint64_t* fragments;
     uint8_t* list_is_cut;   // [P]
+    uint64_t* last_key;     // [P] where list_is_cut: key of the last fragment that took part in the blend (0: none did)
     uint32_t* kept;         // [P] fragments of the pixel that took part in the blend
     // blending
     const float2* projected;  // BILINEAR_BLEND only: [N] where a point projects to at layer 0 (the alpha of a fragment
@@ -574,6 +575,8 @@ __global__ void __launch_bounds__(kBlock) bin_build_kernel(BuildPass a)
         // (FULL_BLEND blends min(count, K) fragments, which the readers work out themselves: the array is not written.)
         if constexpr (BILINEAR) a.kept[q] = used;
         a.list_is_cut[q] = used < c ? 1 : 0;
+        // ... and that key itself (the sorted keys of this bin went out to the fragment buffer before the blend)
+        if (used < c) a.last_key[q] = used ? a.fragments[begin + start + used - 1u] : 0ull;
         const uint32_t in_layer = q - a.ly.base[l];
         const uint32_t tile     = in_layer / kTilePixels;
         const uint32_t ty = tile / (uint32_t)a.ly.tiles_x[l], tx = tile - ty * (uint32_t)a.ly.tiles_x[l];

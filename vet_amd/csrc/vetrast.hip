@@ -395,6 +395,9 @@ int vetrast_workspace_layout_for_mode(int32_t N, int32_t B, int32_t L, int32_t w
     lay->transmittance_base   = at;
     lay->transmittance_stride = align_up(cap * sizeof(float), kAlign);
     at += lay->transmittance_stride * B;
+    lay->last_key_base   = at;
+    lay->last_key_stride = align_up(P * sizeof(uint64_t), kAlign);
+    at += lay->last_key_stride * B;
     lay->projected_base   = at;
     lay->projected_stride = hits == 4 ? align_up((size_t)N * sizeof(float2), kAlign) : 0;
     at += lay->projected_stride * B;
@@ -551,6 +554,7 @@ int vetrast_forward(vetrast_ctx* ctx, const vetrast_forward_args* a, void* strea
             bp.offsets             = offsets;
             bp.fragments           = fragments;
             bp.list_is_cut         = list_is_cut;
+            bp.last_key            = ws_ptr<uint64_t>(ws, lay.last_key_base + lay.last_key_stride * b);
             bp.kept                = ws_ptr<uint32_t>(ws, lay.kept_base + lay.kept_stride * b);
             bp.projected           = vp.projected;
             bp.index               = a->index;
@@ -737,6 +741,7 @@ int vetrast_backward(vetrast_ctx* ctx, const vetrast_backward_args* g, void* str
             gp.offsets             = offsets;
             gp.fragments           = fragments;
             gp.list_is_cut         = ws_ptr<uint8_t>(ws, lay.cut_flags_base + lay.cut_flags_stride * b);
+            gp.last_key            = ws_ptr<uint64_t>(ws, lay.last_key_base + lay.last_key_stride * b);
             gp.kept                = ws_ptr<uint32_t>(ws, lay.kept_base + lay.kept_stride * b);
             gp.partial             = partial;
             gp.grad_texture        = g->grad_texture;
