@@ -236,3 +236,45 @@ def test_list_lengths_around_every_sorting_limit(K, mode, rasterizer, oracle):
     for (px, py), n in where:
         assert counts[py, px] == n, (px, py, n, counts[py, px])
     assert counts.sum() == total
+
+
+def test_two_contexts_on_two_streams_do_not_disturb_each_other(rasterizer, oracle):
+    """There is no process-global state (the reference keeps its parameters in __constant__ symbols,
+    src/lib/rendering/RenderForward.cu:22-27): two contexts with their own workspaces, driven from two streams at the same
+    time, on different scenes and in different modes, give what each gives alone, frame after frame."""
+    from vet_amd.rasterizer import Rasterizer
+
+    print("[case] two contexts on two streams", flush=True)
+    scene_a = synthetic.config2(num_points=150_000, w=640, h=360)
+    scene_b = synthetic.tiny_scene(num_points=60_000, w=320, h=200, num_layers=4, K=-1, seed=77)
+    other = Rasterizer()
+    jobs = []
+    for rast, scene, over in ((rasterizer, scene_a, {}), (other, scene_b, {"render_mode": abi.RENDER_BILINEAR_BLEND})):
+        params = make_params(scene, need_point_gradient=1, **over)
+        dev = DeviceScene(scene)
+        res = rast.forward(dev, params)
+        go = [torch.from_numpy(g).cuda() for g in scene.grad_out()]
+        grads = rast.backward(res, go)
+        torch.cuda.synchronize()
+        want_out = [o.clone() for o in res.out]
+        want_g = {k: v.clone() for k, v in grads.items() if k != "_args"}
+        jobs.append((rast, res, grads, want_out, want_g, torch.cuda.Stream(), go))  # go: the calls hold its pointers
+    for frame in range(4):
+        for rast, res, grads, _, _, stream, _ in jobs:
+            for o in res.out:
+                o.zero_()
+            for k, v in grads.items():
+                if k != "_args":
+                    v.fill_(float("nan"))
+        torch.cuda.synchronize()
+        for _ in range(3):  # several frames in flight on either stream
+            for rast, res, grads, _, _, stream, _ in jobs:
+                s = C.c_void_p(stream.cuda_stream)
+                abi.check(rast.lib.vetrast_forward(rast.ctx, C.byref(res.args), s), "forward")
+                abi.check(rast.lib.vetrast_backward(rast.ctx, C.byref(grads["_args"]), s), "backward")
+        torch.cuda.synchronize()
+        for rast, res, grads, want_out, want_g, _, _ in jobs:
+            for a, b in zip(res.out, want_out):
+                assert torch.equal(a, b), f"frame {frame}"
+            for k, v in want_g.items():
+                assert torch.equal(grads[k], v), (k, frame)

@@ -291,6 +291,9 @@ class Rasterizer:
             g.grad_intrinsics = res["intrinsics"].data_ptr()
             g.grad_intrinsics_count = res["intrinsics_count"].data_ptr()
         abi.check(self.lib.vetrast_backward(self.ctx, C.byref(g), self._stream()), "backward")
+        # the argument block only holds raw pointers: whoever replays it (graph capture, timing loops) needs the
+        # upstream gradients, the forward result and the gradient tensors to stay alive with it
+        g._keepalive = (list(grad_out), fwd, res)
         res["_args"] = g
         return res
 
