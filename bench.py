@@ -6,7 +6,7 @@ on 200 planes/spheres, 1920x1080, 4 layers, K=16, gradients to descriptors, conf
 the workspace are resident in HBM before the timed region starts. Prints ONE JSON line.
 
   python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 2|3|5] [--point-order vet_preprocess|generated]
-                  [--no-cpu-baseline] [--no-second-order]
+                  [--no-cpu-baseline] [--no-second-order | --no-other-order]
 """
 import argparse
 import ctypes as C
@@ -247,7 +247,12 @@ def main():
     ap.add_argument("--point-order", default="vet_preprocess", choices=["vet_preprocess", "generated"])
     ap.add_argument("--render-mode", type=int, default=1, choices=[1, 2, 3],
                     help="1 = FULL_BLEND (the headline workload), 3 = BILINEAR_BLEND (four fragments per point and layer)")
-    ap.add_argument("--no-second-order", action="store_true", help="skip timing the other point order")
+    ap.add_argument("--no-second-order", action="store_true",
+                    help="skip everything beside the headline: the other point order, the fused steps, the error lifting")
+    ap.add_argument("--no-other-order", action="store_true", help="skip timing the other point order only")
+    ap.add_argument("--calibration-kernel", action="store_true",
+                    help="also run the Adam kernel a few times: a streaming kernel that reads 16 and writes 12 bytes per "
+                         "element, against which byte counters of a profiler run are scaled")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--lift-only", action="store_true",
                     help="time only the error lifting on the configuration's scene and print its object")
@@ -343,7 +348,7 @@ def main():
         "kernels": kernels,
     }
 
-    if not args.no_second_order:
+    if not (args.no_second_order or args.no_other_order):
         # VET hands the rasterizer Morton-ordered clouds with shuffled 256-point blocks; the generator's raw order
         # (random inside each primitive) is timed as well so that the effect of that order is visible.
         other = "generated" if args.point_order == "vet_preprocess" else "vet_preprocess"
@@ -354,6 +359,19 @@ def main():
 
     if backward and not args.no_second_order:
         result["fused_steps"] = time_fused_steps(scene, args.render_mode, max(10, args.steps // 2))
+    if args.calibration_kernel:
+        import torch
+
+        from vet_amd.rasterizer import Rasterizer
+
+        n = (scene.num_channels + 1) * scene.num_points + scene.num_channels
+        p_, g_, m_, v_ = (torch.zeros(n, dtype=torch.float32, device="cuda") for _ in range(4))
+        rast_c = Rasterizer()
+        for k in range(3):
+            rast_c.adam_step(p_, g_, m_, v_, k + 1, 1e-3)
+        torch.cuda.synchronize()
+        result["calibration_kernel"] = {"kernel": "adam_step_kernel", "elements": n, "read_bytes": 16 * n,
+                                        "write_bytes": 12 * n}
 
     if not args.no_second_order:
         lift_threads = 0 if args.no_cpu_baseline else (args.cpu_threads or min(16, len(os.sched_getaffinity(0))))

@@ -113,8 +113,8 @@ typedef struct vetrast_ctx vetrast_ctx;
 typedef enum vetrast_scope
 {
     VETRAST_SCOPE_PREPARE = 0,      /* "Build Cache": zero-fill, view preparation */
-    VETRAST_SCOPE_PACK,             /* "Build Cache": descriptor interleave; runs on a stream of the context's own beside
-                                       COUNT..FILL, so its time is not part of the sum of the others */
+    VETRAST_SCOPE_PACK,             /* "Build Cache": descriptor interleave; it rides along with the COUNT kernel of the
+                                       first view, so this scope reports no launches of its own */
     VETRAST_SCOPE_COUNT,            /* "CountingPass": fragments per bin (a 16x16 pixel tile or a piece of one) and, in
                                        the same pass over the points, the fragment records written to their bins */
     VETRAST_SCOPE_SCAN,             /* "CreateAndAllocateBuffers" (prefix scan over the bins; no allocation here) */

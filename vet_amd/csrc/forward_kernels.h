@@ -128,34 +128,6 @@ __global__ void __launch_bounds__(kBlock) prepare_views_kernel(PrepareViewsArgs 
     views[first_view + k] = v;
 }
 
-// Planar descriptors [C,N] + confidence [N] -> one 32-byte record per texture index, so that a fragment costs a single
-// aligned gather instead of C+1 gathers from planes megabytes apart (the reference's BlendMulti reads
-// d_texture.in_texture(ci, idx) per channel, src/lib/rendering/RenderForward.cu:1338-1342).
-// The launch also applies the steps VET runs on the raw tensors right before rendering, when they are switched on:
-// confidence = sigmoid(scale * raw) and texture = |raw| (NeuralPointTextureImpl::PrepareConfidence / PrepareTexture,
-// src/lib/models/NeuralTexture.h:38-55).
-template <int C>
-__global__ void __launch_bounds__(kBlock) pack_descriptors_kernel(const float* __restrict__ texture,
-                                                                   const float* __restrict__ confidence,
-                                                                   float4* __restrict__ packed, int N,
-                                                                   int confidence_activation, float confidence_scale,
-                                                                   int texture_abs)
-{
-    const int i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (i >= N) return;
-    float t[4] = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int ci = 0; ci < C; ++ci)
-    {
-        t[ci] = texture[(size_t)ci * N + i];
-        if (texture_abs) t[ci] = fabsf(t[ci]);
-    }
-    float c = confidence[i];
-    if (confidence_activation) c = sigmoid_canon(confidence_scale * c);
-    packed[2 * (size_t)i]     = make_float4(t[0], t[1], t[2], t[3]);
-    packed[2 * (size_t)i + 1] = make_float4(c, 0.f, 0.f, 0.f);
-}
-
 __device__ __forceinline__ bool point_is_skipped(const ViewPass& a, int i)
 {
     if (a.dropout && a.dropout[i] == 1.f) return true;
@@ -258,6 +230,26 @@ __device__ __forceinline__ WeightedGroup group_by_bin_weighted(bool has, uint32_
     return g;
 }
 
+// Planar descriptors [C,N] + confidence [N] -> one 32-byte record per texture index, so that a fragment costs a single
+// aligned gather instead of C+1 gathers from planes megabytes apart (the reference's BlendMulti reads
+// d_texture.in_texture(ci, idx) per channel, src/lib/rendering/RenderForward.cu:1338-1342).
+// The interleave also applies the steps VET runs on the raw tensors right before rendering, when they are switched on:
+// confidence = sigmoid(scale * raw) and texture = |raw| (NeuralPointTextureImpl::PrepareConfidence / PrepareTexture,
+// src/lib/models/NeuralTexture.h:38-55).
+// It is a side job of the scatter pass of a call's first view (thread i also packs texture row i):
+// the scatter waves spend most of their life waiting for their atomics, so the extra loads and stores ride along
+// (a launch of its own on a second stream took 21 us alone and slowed the scatter pass down by 12 us beside it).
+struct PackJob
+{
+    const float* texture;     // [C,N]
+    const float* confidence;  // [N]
+    float4* packed;           // [N][2], or null: nothing to pack in this launch
+    int N, C;
+    int confidence_activation;
+    float confidence_scale;
+    int texture_abs;
+};
+
 // Where the scatter pass puts a fragment record (64-bit key = depth bits << 32 | point id, pixel inside the bin).
 // Every bin owns room for kPrimaryCap records; a record whose rank inside its bin is beyond that is appended to a log
 // (with its bin and rank), from where overflow_move_kernel brings it to the bin's place in the compact array once the
@@ -308,10 +300,20 @@ __device__ __forceinline__ void store_record(const ScatterTargets& t, bool valid
 // point id << 2 | corner.
 template <int HITS>
 __global__ void __launch_bounds__(kBlock) bin_scatter_kernel(ViewPass a, uint32_t* __restrict__ bin_counts,
-                                                              ScatterTargets out)
+                                                              ScatterTargets out, PackJob pack)
 {
     const int i    = blockIdx.x * blockDim.x + threadIdx.x;
     const int lane = threadIdx.x & (kWave - 1);
+    // side job: texture row i, asked for first and stored last
+    const bool packs = pack.packed != nullptr && i < pack.N;
+    float row[4] = {0.f, 0.f, 0.f, 0.f}, row_confidence = 0.f;
+    if (packs)
+    {
+#pragma unroll
+        for (int ci = 0; ci < VETRAST_MAX_CHANNELS; ++ci)
+            if (ci < pack.C) row[ci] = pack.texture[(size_t)ci * pack.N + i];
+        row_confidence = pack.confidence[i];
+    }
     Projected p;
     p.ipx = p.ipy = p.z = p.radius = 0.f;
     const bool visible = i < a.N && !point_is_skipped(a, i) && project_point(*a.view, a.position[i], p);
@@ -431,6 +433,17 @@ __global__ void __launch_bounds__(kBlock) bin_scatter_kernel(ViewPass a, uint32_
             if (l >= 1 && l - 1 < a.ly.L) store_layer(l - 1);
         }
         if (VETRAST_MAX_LAYERS - 1 < a.ly.L) store_layer(VETRAST_MAX_LAYERS - 1);
+    }
+    if (packs)
+    {
+        if (pack.texture_abs)
+        {
+#pragma unroll
+            for (int ci = 0; ci < VETRAST_MAX_CHANNELS; ++ci) row[ci] = fabsf(row[ci]);
+        }
+        if (pack.confidence_activation) row_confidence = sigmoid_canon(pack.confidence_scale * row_confidence);
+        pack.packed[2 * (size_t)i]     = make_float4(row[0], row[1], row[2], row[3]);
+        pack.packed[2 * (size_t)i + 1] = make_float4(row_confidence, 0.f, 0.f, 0.f);
     }
 }
 

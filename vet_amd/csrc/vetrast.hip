@@ -28,10 +28,6 @@ struct vetrast_ctx
         int scope;
         hipEvent_t start, stop;
     };
-    // The descriptor interleave only feeds the last forward kernel, so it runs beside the binning kernels on a stream
-    // of the context's own, forked from and joined back into the caller's stream with events.
-    hipStream_t side  = nullptr;
-    hipEvent_t forked = nullptr, joined = nullptr;
     std::vector<Span> spans;             // recorded since the last reset
     std::vector<hipEvent_t> free_events;  // recycled events
     float acc_ms[VETRAST_SCOPE_COUNT_]      = {};
@@ -280,9 +276,6 @@ int vetrast_create(vetrast_ctx** out_ctx)
     vetrast_ctx* ctx = new (std::nothrow) vetrast_ctx();
     if (!ctx) return VETRAST_ERR_INVALID_ARG;
     hipError_t e = hipGetDevice(&ctx->device);
-    if (e == hipSuccess) e = hipStreamCreateWithFlags(&ctx->side, hipStreamNonBlocking);
-    if (e == hipSuccess) e = hipEventCreateWithFlags(&ctx->forked, hipEventDisableTiming);
-    if (e == hipSuccess) e = hipEventCreateWithFlags(&ctx->joined, hipEventDisableTiming);
     if (e != hipSuccess)
     {
         vetrast_destroy(ctx);
@@ -301,9 +294,6 @@ void vetrast_destroy(vetrast_ctx* ctx)
         (void)hipEventDestroy(s.stop);
     }
     for (auto e : ctx->free_events) (void)hipEventDestroy(e);
-    if (ctx->forked) (void)hipEventDestroy(ctx->forked);
-    if (ctx->joined) (void)hipEventDestroy(ctx->joined);
-    if (ctx->side) (void)hipStreamDestroy(ctx->side);
     delete ctx;
 }
 
@@ -440,24 +430,6 @@ int vetrast_forward(vetrast_ctx* ctx, const vetrast_forward_args* a, void* strea
     uint32_t* partials  = ws_ptr<uint32_t>(ws, lay.scan_partials_base);
     DeviceView* views   = ws_ptr<DeviceView>(ws, lay.views_base);
 
-    if (N > 0)
-    {
-        // descriptor interleave on the side stream; joined again in front of the build pass of the first view
-        VET_HIP(ctx, hipEventRecord(ctx->forked, stream));
-        VET_HIP(ctx, hipStreamWaitEvent(ctx->side, ctx->forked, 0));
-        {
-            ScopeTimer tm(ctx, ctx->side, VETRAST_SCOPE_PACK);
-            const dim3 g(grid_for(N)), blk(kBlock);
-            switch (C)
-            {
-                case 1: hipLaunchKernelGGL(pack_descriptors_kernel<1>, g, blk, 0, ctx->side, a->texture, a->confidence, packed, N, p.confidence_activation, p.confidence_scale, p.texture_abs); break;
-                case 2: hipLaunchKernelGGL(pack_descriptors_kernel<2>, g, blk, 0, ctx->side, a->texture, a->confidence, packed, N, p.confidence_activation, p.confidence_scale, p.texture_abs); break;
-                case 3: hipLaunchKernelGGL(pack_descriptors_kernel<3>, g, blk, 0, ctx->side, a->texture, a->confidence, packed, N, p.confidence_activation, p.confidence_scale, p.texture_abs); break;
-                default: hipLaunchKernelGGL(pack_descriptors_kernel<4>, g, blk, 0, ctx->side, a->texture, a->confidence, packed, N, p.confidence_activation, p.confidence_scale, p.texture_abs); break;
-            }
-        }
-        VET_HIP(ctx, hipEventRecord(ctx->joined, ctx->side));
-    }
     {
         ScopeTimer tm(ctx, stream, VETRAST_SCOPE_PREPARE);
         // per-bin counters of all views (contiguous) start at zero; InitializeData, PointRenderer.cu:402-470
@@ -500,14 +472,24 @@ int vetrast_forward(vetrast_ctx* ctx, const vetrast_forward_args* a, void* strea
         targets.log_rank     = slots;
         targets.log_cursor   = ws_ptr<uint32_t>(ws, lay.log_cursor_base) + (size_t)b * kLogSegments * kLogCursorStride;
         targets.segment_capacity = log_segment_records(N, L, hits);
+        // the scatter pass of the first view also interleaves the descriptors (PrepareTexture / PrepareConfidence included)
+        PackJob pack;
+        pack.texture               = a->texture;
+        pack.confidence            = a->confidence;
+        pack.packed                = b == 0 ? packed : nullptr;
+        pack.N                     = N;
+        pack.C                     = C;
+        pack.confidence_activation = p.confidence_activation;
+        pack.confidence_scale      = p.confidence_scale;
+        pack.texture_abs           = p.texture_abs;
         uint8_t* list_is_cut     = ws_ptr<uint8_t>(ws, lay.cut_flags_base + lay.cut_flags_stride * b);
         if (N > 0)
         {
             ScopeTimer tm(ctx, stream, VETRAST_SCOPE_COUNT);
             if (hits == 1)
-                hipLaunchKernelGGL(bin_scatter_kernel<1>, dim3(grid_for(N)), dim3(kBlock), 0, stream, vp, bin_counts, targets);
+                hipLaunchKernelGGL(bin_scatter_kernel<1>, dim3(grid_for(N)), dim3(kBlock), 0, stream, vp, bin_counts, targets, pack);
             else
-                hipLaunchKernelGGL(bin_scatter_kernel<4>, dim3(grid_for(N)), dim3(kBlock), 0, stream, vp, bin_counts, targets);
+                hipLaunchKernelGGL(bin_scatter_kernel<4>, dim3(grid_for(N)), dim3(kBlock), 0, stream, vp, bin_counts, targets, pack);
         }
         {
             ScopeTimer tm(ctx, stream, VETRAST_SCOPE_SCAN);
@@ -544,7 +526,6 @@ int vetrast_forward(vetrast_ctx* ctx, const vetrast_forward_args* a, void* strea
             if (p.output_background_mask) out_mask[l] = a->out_mask[l] + (size_t)b * plane;
             if (a->out_weight[l]) out_weight[l] = a->out_weight[l] + (size_t)b * plane;
         }
-        if (b == 0 && N > 0) VET_HIP(ctx, hipStreamWaitEvent(stream, ctx->joined, 0));
         {
             ScopeTimer tm(ctx, stream, VETRAST_SCOPE_BUILD);
             BuildPass bp;
@@ -975,7 +956,7 @@ const char* vetrast_scope_name(int32_t scope)
     switch (scope)
     {
         case VETRAST_SCOPE_PREPARE: return "Build Cache";
-        case VETRAST_SCOPE_PACK: return "Build Cache (descriptor interleave, beside the binning passes)";
+        case VETRAST_SCOPE_PACK: return "Build Cache (descriptor interleave; part of the counting pass, no launch of its own)";
         case VETRAST_SCOPE_COUNT: return "CountingPass";
         case VETRAST_SCOPE_SCAN: return "CreateAndAllocateBuffers";
         case VETRAST_SCOPE_FILL: return "CollectionPass";
