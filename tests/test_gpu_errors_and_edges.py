@@ -278,3 +278,37 @@ def test_two_contexts_on_two_streams_do_not_disturb_each_other(rasterizer, oracl
                 assert torch.equal(a, b), f"frame {frame}"
             for k, v in want_g.items():
                 assert torch.equal(grads[k], v), (k, frame)
+
+
+def test_empty_cloud(rasterizer):
+    """num_points = 0 (the buffers exist, they are just not read): every pixel shows the background, the background
+    gradient is the plain sum of the incoming gradients, nothing else is touched or launched on the points."""
+    print("[case] empty cloud", flush=True)
+    scene = synthetic.tiny_scene(num_points=8, w=40, h=24, num_layers=3, seed=58)
+    dev = DeviceScene(scene)
+    params = make_params(scene, need_point_gradient=1)
+    full = rasterizer.forward(dev, params)  # sizes the workspace and the outputs
+    torch.cuda.synchronize()
+    args = full.args
+    args.num_points = 0
+    for o in full.out:
+        o.fill_(float("nan"))
+    abi.check(rasterizer.lib.vetrast_forward(rasterizer.ctx, C.byref(args), None), "forward, no points")
+    torch.cuda.synchronize()
+    for o in full.out:
+        got = o.cpu().numpy()
+        assert np.all(got == scene.background.reshape(1, -1, 1, 1))
+    g = abi.BackwardArgs()
+    C.memmove(C.byref(g.fwd), C.byref(args), C.sizeof(abi.ForwardArgs))
+    go = [torch.from_numpy(x).cuda() for x in scene.grad_out()]
+    for l, t in enumerate(go):
+        g.grad_out[l] = t.data_ptr()
+    gb = torch.full((scene.num_channels,), float("nan"), device="cuda")
+    gt = torch.zeros((scene.num_channels, 8), device="cuda")
+    gc = torch.zeros((8,), device="cuda")
+    g.grad_texture, g.grad_confidence, g.grad_background = gt.data_ptr(), gc.data_ptr(), gb.data_ptr()
+    abi.check(rasterizer.lib.vetrast_backward(rasterizer.ctx, C.byref(g), None), "backward, no points")
+    torch.cuda.synchronize()
+    exact = sum(x.astype(np.float64).sum(axis=(0, 2, 3)) for x in scene.grad_out())
+    assert max_rel_err(gb.cpu().numpy(), exact) <= 1e-5
+    assert not gt.any() and not gc.any()
