@@ -34,7 +34,8 @@ typedef enum vetrast_status
     VETRAST_ERR_WORKSPACE_SMALL = -2, /* workspace_bytes below vetrast_forward_workspace_bytes() */
     VETRAST_ERR_HIP             = -3, /* a HIP runtime call failed; see vetrast_last_hip_error() */
     VETRAST_ERR_UNSUPPORTED     = -4, /* a reference feature outside the blending path (OCam, normals, ...) */
-    VETRAST_ERR_BAD_INPUT_DATA  = -5  /* device-side check failed (non-zero distortion), from vetrast_query_device_flags */
+    VETRAST_ERR_BAD_INPUT_DATA  = -5, /* device-side check failed (non-zero distortion), from vetrast_query_device_flags */
+    VETRAST_ERR_TOO_LARGE       = -6  /* size beyond the fixed maximum of an entry point that allocates nothing */
 } vetrast_status;
 
 /* Camera model tag of a view. Mirrors enum CameraModel, src/lib/data/SceneData.h:30-35.
@@ -327,6 +328,22 @@ typedef struct vetrast_lift_args
 } vetrast_lift_args;
 size_t vetrast_lift_workspace_bytes(int64_t num_cells);
 int vetrast_lift_error(vetrast_ctx* ctx, const vetrast_lift_args* args, void* stream);
+
+/* vetrast_lift_error for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc). It has no counterpart in the reference. Same arguments, same kernels and
+ * same results as vetrast_lift_error, but `workspace` / `workspace_bytes` are ignored: the scratch is an array inside
+ * the library (about 12.6 MB of device memory per GPU, held until the process ends), whose address on the context's
+ * device vetrast_create looks up once. The call itself allocates and frees nothing, creates no events (it reports no
+ * timing scope) and only launches kernels.
+ *   - num_cells > VETRAST_LIFT_STATIC_MAX_CELLS is refused with VETRAST_ERR_TOO_LARGE.
+ *   - The context's device must be the current device, else VETRAST_ERR_INVALID_ARG.
+ *   - All calls on one GPU share that GPU's array (every call rewrites what it reads, nothing has to be cleared in
+ *     between): calls that overlap on one GPU, on different streams or from different contexts, race. Calls on one
+ *     stream are safe.
+ *   - The distortion flag word of vetrast_lift_error lives in the scratch and cannot be read back here; check the
+ *     intrinsics beforehand. */
+#define VETRAST_LIFT_STATIC_MAX_CELLS (1 << 19)
+int vetrast_lift_error_static(vetrast_ctx* ctx, const vetrast_lift_args* args, void* stream);
 
 /* Per-kernel timing, the counterpart of NeuralRenderInfo::timer_system (src/lib/rendering/PointRenderer.h:32).
  * With profiling enabled every launch is bracketed by HIP events on the call's stream; vetrast_scope_times

@@ -14,6 +14,7 @@ ERR_WORKSPACE_SMALL = -2
 ERR_HIP = -3
 ERR_UNSUPPORTED = -4
 ERR_BAD_INPUT_DATA = -5
+ERR_TOO_LARGE = -6
 
 CAMERA_PINHOLE_DISTORTION = 0
 CAMERA_OCAM = 1
@@ -113,6 +114,7 @@ class AdamArgs(C.Structure):
 
 LIFT_BORDER_PIXELS = 32
 LIFT_FLAGS_OFFSET = 192
+LIFT_STATIC_MAX_CELLS = 1 << 19
 
 
 class LiftArgs(C.Structure):
@@ -184,6 +186,7 @@ SYMBOLS = {
     "vetrast_adam_step": (C.c_int, [C.c_void_p, C.POINTER(AdamArgs), C.c_void_p]),
     "vetrast_lift_workspace_bytes": (C.c_size_t, [C.c_int64]),
     "vetrast_lift_error": (C.c_int, [C.c_void_p, C.POINTER(LiftArgs), C.c_void_p]),
+    "vetrast_lift_error_static": (C.c_int, [C.c_void_p, C.POINTER(LiftArgs), C.c_void_p]),
     "vetrast_query_device_flags": (C.c_int, [C.c_void_p, C.c_void_p, C.POINTER(WorkspaceLayout), C.c_void_p]),
     "vetrast_set_profiling": (C.c_int, [C.c_void_p, C.c_int32]),
     "vetrast_reset_scope_times": (C.c_int, [C.c_void_p]),

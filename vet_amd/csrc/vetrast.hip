@@ -6,6 +6,7 @@
 
 #include <cmath>
 #include <cstring>
+#include <mutex>
 #include <new>
 #include <vector>
 
@@ -32,6 +33,7 @@ struct vetrast_ctx
     std::vector<hipEvent_t> free_events;  // recycled events
     float acc_ms[VETRAST_SCOPE_COUNT_]      = {};
     int32_t acc_launches[VETRAST_SCOPE_COUNT_] = {};
+    char* lift_scratch = nullptr;  // this device's copy of the file-scope scratch array (vetrast_lift_error_static)
 };
 
 namespace
@@ -41,6 +43,15 @@ constexpr double kSplitListLength = 8.0;  // layers that blend at least this man
 inline size_t align_up(size_t v, size_t a)
 {
     return (v + a - 1) / a * a;
+}
+
+// Bytes of error-lifting scratch for num_cells cells: header (camera constants, queue length, flag word), queue
+// entries, one double per queue slot, chunk prefix sums.
+constexpr size_t align_up_c(size_t v, size_t a) { return (v + a - 1) / a * a; }
+constexpr size_t lift_workspace_bytes_for(size_t num_cells)
+{
+    return kLiftHeader + align_up_c(num_cells * sizeof(uint2), kAlign) + align_up_c(num_cells * sizeof(double), kAlign) +
+           align_up_c((num_cells + 1) * sizeof(unsigned long long), kAlign);
 }
 
 #define VET_HIP(ctx, expr)                               \
@@ -265,6 +276,107 @@ ViewPass make_view_pass(const vetrast_forward_args* a, const vetrast_workspace_l
     return vp;
 }
 
+// Scratch of vetrast_lift_error_static: the workspace vetrast_lift_error takes from its caller, as an array of the
+// library's own, sized for VETRAST_LIFT_STATIC_MAX_CELLS cells. Every GPU the library runs on holds a copy of its own
+// until the process ends. In host code this name only stands for the symbol: the device address is looked up once per
+// device (scratch_of_device) and only that pointer is handed to kernels.
+constexpr size_t kLiftStaticBytes = lift_workspace_bytes_for((size_t)VETRAST_LIFT_STATIC_MAX_CELLS);
+static __device__ __align__(256) unsigned char scratch[kLiftStaticBytes];
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+char* g_scratch_ptr[kMaxDevices] = {};
+
+// Address of the scratch array on `device`, which must be the current device. hipSuccess and a non-null pointer on
+// success.
+hipError_t scratch_of_device(int device, char** out)
+{
+    *out = nullptr;
+    if (device < 0 || device >= kMaxDevices) return hipErrorInvalidDevice;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[device])
+    {
+        void* p      = nullptr;
+        hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return e;
+        if (!p || (reinterpret_cast<uintptr_t>(p) % kAlign) != 0) return hipErrorInvalidSymbol;
+        g_scratch_ptr[device] = static_cast<char*>(p);
+    }
+    *out = g_scratch_ptr[device];
+    return hipSuccess;
+}
+
+// Argument checks of the error lifting that do not concern the workspace. VETRAST_OK with *nothing_to_do set for an
+// empty grid.
+int validate_lift(const vetrast_lift_args* a, bool* nothing_to_do)
+{
+    *nothing_to_do = false;
+    if (a->num_cells < 0 || a->num_cells > (int64_t)1 << 30) return VETRAST_ERR_INVALID_ARG;
+    if (a->channels < 1 || a->height < 1 || a->width < 1 || a->border_pixels < 0) return VETRAST_ERR_INVALID_ARG;
+    // pixel numbers inside a cell's box go through float arithmetic that is exact below 2^24
+    if ((int64_t)a->height * a->width >= (int64_t)1 << 24) return VETRAST_ERR_INVALID_ARG;
+    const vetrast_view& v = a->view;
+    if (v.camera_model_type != VETRAST_CAMERA_PINHOLE_DISTORTION) return VETRAST_ERR_UNSUPPORTED;
+    if (v.image_index < 0 || v.image_index >= a->num_poses) return VETRAST_ERR_INVALID_ARG;
+    if (v.camera_index < 0 || v.camera_index >= a->num_cameras) return VETRAST_ERR_INVALID_ARG;
+    if (a->num_cells == 0)
+    {
+        *nothing_to_do = true;
+        return VETRAST_OK;
+    }
+    if (!a->cell_bb_min || !a->cell_bb_length || !a->cell_value || !a->cell_access_count || !a->poses_se3 ||
+        !a->intrinsics || !a->loss_image)
+        return VETRAST_ERR_INVALID_ARG;
+    return VETRAST_OK;
+}
+
+// The five launches of the error lifting with their scratch at `ws` (lift_workspace_bytes_for(num_cells) bytes,
+// 256-byte aligned). Every word of the scratch a kernel reads has been written by an earlier kernel of the same call
+// (the prepare kernel empties the queue, a slot's sum is cleared when the slot is taken), so nothing needs clearing
+// between calls that share one scratch.
+void launch_lift(const vetrast_lift_args* a, char* ws, hipStream_t stream)
+{
+    const vetrast_view& v = a->view;
+    LiftPass lp;
+    lp.bb_min       = a->cell_bb_min;
+    lp.bb_length    = a->cell_bb_length;
+    lp.value        = a->cell_value;
+    lp.access_count = a->cell_access_count;
+    lp.loss         = a->loss_image;
+    lp.num_cells    = a->num_cells;
+    lp.channels     = a->channels;
+    lp.height       = a->height;
+    lp.width        = a->width;
+    lp.border       = a->border_pixels;
+    lp.view         = reinterpret_cast<const DeviceView*>(ws);
+    lp.queue_length = reinterpret_cast<uint32_t*>(ws + sizeof(DeviceView));
+    lp.queue        = reinterpret_cast<uint2*>(ws + kLiftHeader);
+    lp.sums = reinterpret_cast<double*>(ws + kLiftHeader + align_up((size_t)a->num_cells * sizeof(uint2), kAlign));
+    lp.starts = reinterpret_cast<unsigned long long*>(reinterpret_cast<char*>(lp.sums) +
+                                                      align_up((size_t)a->num_cells * sizeof(double), kAlign));
+    uint32_t* flags = reinterpret_cast<uint32_t*>(ws + VETRAST_LIFT_FLAGS_OFFSET);
+
+    ViewSource src;
+    src.image_index  = v.image_index;
+    src.camera_index = v.camera_index;
+    src.w            = v.w;
+    src.h            = v.h;
+    for (int j = 0; j < 5; ++j) src.crop[j] = v.crop_transform[j];
+    for (int j = 0; j < 4; ++j) src.rot[j] = v.crop_rotation[j];
+
+    hipLaunchKernelGGL(lift_prepare_kernel, dim3(1), dim3(kWave), 0, stream, src, a->poses_se3, a->intrinsics,
+                       reinterpret_cast<DeviceView*>(ws), lp.queue_length, flags);
+    const int waves_per_block = kBlock / kWave;
+    hipLaunchKernelGGL(lift_cells_kernel, dim3((unsigned)((a->num_cells + waves_per_block - 1) / waves_per_block)),
+                       dim3(kBlock), 0, stream, lp);
+    // The queue length stays on the device, so the shared pass is launched at a fixed width and splits the chunks
+    // it finds evenly.
+    hipLaunchKernelGGL(lift_scan_kernel, dim3(1), dim3(kLiftScanBlock), 0, stream, lp);
+    hipLaunchKernelGGL(lift_queued_kernel, dim3(2048), dim3(kBlock), 0, stream, lp);
+    hipLaunchKernelGGL(lift_finish_kernel, dim3((unsigned)std::min<int64_t>(grid_for((size_t)a->num_cells), 256)),
+                       dim3(kBlock), 0, stream, lp);
+}
+
 }  // namespace
 
 extern "C" {
@@ -276,6 +388,13 @@ int vetrast_create(vetrast_ctx** out_ctx)
     vetrast_ctx* ctx = new (std::nothrow) vetrast_ctx();
     if (!ctx) return VETRAST_ERR_INVALID_ARG;
     hipError_t e = hipGetDevice(&ctx->device);
+    if (e != hipSuccess)
+    {
+        vetrast_destroy(ctx);
+        return VETRAST_ERR_HIP;
+    }
+    // this device's address of the scratch array of vetrast_lift_error_static, looked up once per device
+    e = scratch_of_device(ctx->device, &ctx->lift_scratch);
     if (e != hipSuccess)
     {
         vetrast_destroy(ctx);
@@ -824,71 +943,37 @@ int vetrast_adam_step(vetrast_ctx* ctx, const vetrast_adam_args* a, void* stream
 size_t vetrast_lift_workspace_bytes(int64_t num_cells)
 {
     if (num_cells < 0) return 0;
-    // header (camera constants, queue length, flag word), queue entries, one double per queue slot, chunk prefix sums
-    return kLiftHeader + align_up((size_t)num_cells * sizeof(uint2), kAlign) +
-           align_up((size_t)num_cells * sizeof(double), kAlign) +
-           align_up(((size_t)num_cells + 1) * sizeof(unsigned long long), kAlign);
+    return lift_workspace_bytes_for((size_t)num_cells);
 }
 
 int vetrast_lift_error(vetrast_ctx* ctx, const vetrast_lift_args* a, void* stream_)
 {
     if (!ctx || !a) return VETRAST_ERR_INVALID_ARG;
-    if (a->num_cells < 0 || a->num_cells > (int64_t)1 << 30) return VETRAST_ERR_INVALID_ARG;
-    if (a->channels < 1 || a->height < 1 || a->width < 1 || a->border_pixels < 0) return VETRAST_ERR_INVALID_ARG;
-    // pixel numbers inside a cell's box go through float arithmetic that is exact below 2^24
-    if ((int64_t)a->height * a->width >= (int64_t)1 << 24) return VETRAST_ERR_INVALID_ARG;
-    const vetrast_view& v = a->view;
-    if (v.camera_model_type != VETRAST_CAMERA_PINHOLE_DISTORTION) return VETRAST_ERR_UNSUPPORTED;
-    if (v.image_index < 0 || v.image_index >= a->num_poses) return VETRAST_ERR_INVALID_ARG;
-    if (v.camera_index < 0 || v.camera_index >= a->num_cameras) return VETRAST_ERR_INVALID_ARG;
-    if (a->num_cells == 0) return VETRAST_OK;
-    if (!a->cell_bb_min || !a->cell_bb_length || !a->cell_value || !a->cell_access_count || !a->poses_se3 ||
-        !a->intrinsics || !a->loss_image || !a->workspace)
-        return VETRAST_ERR_INVALID_ARG;
-    if (reinterpret_cast<uintptr_t>(a->workspace) % kAlign) return VETRAST_ERR_INVALID_ARG;
+    bool nothing_to_do = false;
+    const int st       = validate_lift(a, &nothing_to_do);
+    if (st != VETRAST_OK || nothing_to_do) return st;
+    if (!a->workspace || reinterpret_cast<uintptr_t>(a->workspace) % kAlign) return VETRAST_ERR_INVALID_ARG;
     if (a->workspace_bytes < vetrast_lift_workspace_bytes(a->num_cells)) return VETRAST_ERR_WORKSPACE_SMALL;
-
     hipStream_t stream = (hipStream_t)stream_;
-    char* ws           = static_cast<char*>(a->workspace);
-    LiftPass lp;
-    lp.bb_min       = a->cell_bb_min;
-    lp.bb_length    = a->cell_bb_length;
-    lp.value        = a->cell_value;
-    lp.access_count = a->cell_access_count;
-    lp.loss         = a->loss_image;
-    lp.num_cells    = a->num_cells;
-    lp.channels     = a->channels;
-    lp.height       = a->height;
-    lp.width        = a->width;
-    lp.border       = a->border_pixels;
-    lp.view         = reinterpret_cast<const DeviceView*>(ws);
-    lp.queue_length = reinterpret_cast<uint32_t*>(ws + sizeof(DeviceView));
-    lp.queue        = reinterpret_cast<uint2*>(ws + kLiftHeader);
-    lp.sums = reinterpret_cast<double*>(ws + kLiftHeader + align_up((size_t)a->num_cells * sizeof(uint2), kAlign));
-    lp.starts = reinterpret_cast<unsigned long long*>(reinterpret_cast<char*>(lp.sums) +
-                                                      align_up((size_t)a->num_cells * sizeof(double), kAlign));
-    uint32_t* flags = reinterpret_cast<uint32_t*>(ws + VETRAST_LIFT_FLAGS_OFFSET);
-
-    ViewSource src;
-    src.image_index  = v.image_index;
-    src.camera_index = v.camera_index;
-    src.w            = v.w;
-    src.h            = v.h;
-    for (int j = 0; j < 5; ++j) src.crop[j] = v.crop_transform[j];
-    for (int j = 0; j < 4; ++j) src.rot[j] = v.crop_rotation[j];
-
     ScopeTimer tm(ctx, stream, VETRAST_SCOPE_LIFT_ERROR);
-    hipLaunchKernelGGL(lift_prepare_kernel, dim3(1), dim3(kWave), 0, stream, src, a->poses_se3, a->intrinsics,
-                       reinterpret_cast<DeviceView*>(ws), lp.queue_length, flags);
-    const int waves_per_block = kBlock / kWave;
-    hipLaunchKernelGGL(lift_cells_kernel, dim3((unsigned)((a->num_cells + waves_per_block - 1) / waves_per_block)),
-                       dim3(kBlock), 0, stream, lp);
-    // The queue length stays on the device, so the shared pass is launched at a fixed width and splits the chunks
-    // it finds evenly.
-    hipLaunchKernelGGL(lift_scan_kernel, dim3(1), dim3(kLiftScanBlock), 0, stream, lp);
-    hipLaunchKernelGGL(lift_queued_kernel, dim3(2048), dim3(kBlock), 0, stream, lp);
-    hipLaunchKernelGGL(lift_finish_kernel, dim3((unsigned)std::min<int64_t>(grid_for((size_t)a->num_cells), 256)),
-                       dim3(kBlock), 0, stream, lp);
+    launch_lift(a, static_cast<char*>(a->workspace), stream);
+    VET_HIP(ctx, hipGetLastError());
+    return VETRAST_OK;
+}
+
+int vetrast_lift_error_static(vetrast_ctx* ctx, const vetrast_lift_args* a, void* stream_)
+{
+    if (!ctx || !a) return VETRAST_ERR_INVALID_ARG;
+    bool nothing_to_do = false;
+    const int st       = validate_lift(a, &nothing_to_do);
+    if (st != VETRAST_OK || nothing_to_do) return st;
+    if (a->num_cells > (int64_t)VETRAST_LIFT_STATIC_MAX_CELLS) return VETRAST_ERR_TOO_LARGE;
+    // the scratch pointer belongs to the context's device; kernels launched on another device's stream must not get it
+    int current = -1;
+    VET_HIP(ctx, hipGetDevice(&current));
+    if (current != ctx->device || !ctx->lift_scratch) return VETRAST_ERR_INVALID_ARG;
+    // No timing scope here: a scope takes HIP events and grows a host vector, and this entry point allocates nothing.
+    launch_lift(a, ctx->lift_scratch, (hipStream_t)stream_);
     VET_HIP(ctx, hipGetLastError());
     return VETRAST_OK;
 }
@@ -980,6 +1065,7 @@ const char* vetrast_status_string(int status)
         case VETRAST_ERR_HIP: return "HIP runtime error";
         case VETRAST_ERR_UNSUPPORTED: return "feature outside the implemented blending path";
         case VETRAST_ERR_BAD_INPUT_DATA: return "device-side input check failed (non-zero distortion)";
+        case VETRAST_ERR_TOO_LARGE: return "size beyond the fixed maximum of an allocation-free entry point";
         default: return "unknown status";
     }
 }

@@ -309,11 +309,12 @@ class Rasterizer:
         abi.check(self.lib.vetrast_adam_step(self.ctx, C.byref(a), self._stream()), "adam_step")
 
     def lift_error(self, cell_bb_min, cell_bb_length, cell_value, cell_access_count, view, poses_se3, intrinsics,
-                   loss_image, border_pixels=abi.LIFT_BORDER_PIXELS, workspace=None):
+                   loss_image, border_pixels=abi.LIFT_BORDER_PIXELS, workspace=None, static_scratch=False):
         """Adds the error image of one view to the grid cells its pixels fall in, in place on cell_value (float32 [n]
         or [n,1]) and cell_access_count (int32) (vetrast_lift_error; the reference's FillSceneGridWithLoss). All
         arguments but `view` (a synthetic.View) are contiguous CUDA tensors. Returns the workspace, whose flag word
-        `lift_flags` reads."""
+        `lift_flags` reads. With `static_scratch` the call goes to vetrast_lift_error_static, which takes no workspace
+        (the scratch is an array inside the library) and allocates nothing; None is returned."""
         a = abi.LiftArgs()
         for name, t, dt in (("cell_bb_min", cell_bb_min, torch.float32), ("cell_bb_length", cell_bb_length, torch.float32),
                             ("cell_value", cell_value, torch.float32), ("cell_access_count", cell_access_count, torch.int32),
@@ -325,6 +326,9 @@ class Rasterizer:
         assert cell_bb_min.numel() == 3 * a.num_cells and cell_bb_length.numel() == 3 * a.num_cells
         assert cell_access_count.numel() == a.num_cells and loss_image.dim() == 3
         fill_lift_args(a, view, poses_se3, intrinsics, loss_image, border_pixels)
+        if static_scratch:
+            abi.check(self.lib.vetrast_lift_error_static(self.ctx, C.byref(a), self._stream()), "lift_error_static")
+            return None
         need = int(self.lib.vetrast_lift_workspace_bytes(a.num_cells))
         if workspace is None:
             workspace = torch.empty(max(need, 256), dtype=torch.uint8, device=loss_image.device)
