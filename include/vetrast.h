@@ -163,7 +163,8 @@ typedef struct vetrast_workspace_layout
     int64_t num_bins;      /* bins of one view: runs of 256 / 64 / 16 / 4 consecutive pixel numbers, chosen per layer from N */
     size_t bin_counts_base, bin_counts_stride; /* per view, uint32 [num_bins+1 padded]: fragments per bin, then their exclusive scan */
     size_t binned_base;    /* uint32 [N*L*hits][4]: compact array of fragment records (key low, key high, pixel in bin, 0),
-                              only used for the records beyond a bin's own room; scratch */
+                              only used for the records beyond a bin's own room; scratch. In FULL_BLEND / FUZZY_BLEND with
+                              N <= 2^24 a record is uint32 [2]: (depth bits, point id << 8 | pixel in bin) */
     size_t flags_base;     /* uint32 [4] device status flags, then at +64 bytes float [4]: the background as it is blended */
     size_t forward_only_bytes; /* a forward call with save_for_backward = 0 needs only this much */
     size_t partial_base;   /* float [L][N][8]: backward scratch, gradient record of the fragment of point i in layer l */
@@ -172,7 +173,7 @@ typedef struct vetrast_workspace_layout
     /* scratch shared by all views: the scatter pass writes the records of bin b to primary[b][rank] while rank < 2048;
      * records beyond that go to a log of 256 segments (record + bin, rank in the slots array) and are filed into the
      * compact array after the scan. log_cursor: per view, 256 uint32 64 bytes apart, entries in every segment. */
-    size_t primary_base;   /* uint32 [num_bins][2048][4] */
+    size_t primary_base;   /* uint32 [num_bins][2048][4], or [num_bins][2048][2] with the 8-byte records */
     size_t log_base;       /* uint32 [256][ceil(ceil(N/256)/256)*256*L*hits][4] */
     size_t log_cursor_base;
     size_t last_key_base, last_key_stride;   /* per view, uint64 [P]: where cut_flags is 1, the key of the last fragment of

@@ -99,7 +99,7 @@ def test_workspace_layout_is_aligned_and_disjoint():
         ("flags", lay.flags_base, 16),
         ("offsets", lay.offsets_base, lay.offsets_stride * B),
         ("tile_counts", lay.bin_counts_base, lay.bin_counts_stride * B),
-        ("binned", lay.binned_base, N * L * 16),
+        ("binned", lay.binned_base, N * L * 8),  # 8-byte records: one hit per layer, N <= 2^24
         ("cut_flags", lay.cut_flags_base, lay.cut_flags_stride * B),
         ("kept", lay.kept_base, lay.kept_stride * B),
         ("fragments", lay.fragments_base, lay.fragments_stride * B),
@@ -109,7 +109,7 @@ def test_workspace_layout_is_aligned_and_disjoint():
         ("slots", lay.slots_base, log_records * 4),
         ("log", lay.log_base, log_records * 16),
         ("log_cursor", lay.log_cursor_base, B * 256 * 64),
-        ("primary", lay.primary_base, lay.num_bins * 2048 * 16),
+        ("primary", lay.primary_base, lay.num_bins * 2048 * 8),
         ("views", lay.views_base, B * 128),
         ("partial", lay.partial_base, N * L * 32),
         ("background_partial", lay.background_partial_base, (P + 255) // 256 * 32),

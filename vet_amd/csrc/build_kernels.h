@@ -34,6 +34,7 @@ struct BuildPass
     const uint32_t* bin_offsets;  // [bins + 1] exclusive scan of the bin counts
     const uint4* primary;         // [bins][kPrimaryCap] fragment records, the first kPrimaryCap of every bin
     const uint4* binned;          // compact array: record r >= kPrimaryCap of a bin sits at bin_offsets[bin] + r
+    int compact_records;          // both hold 8-byte records (depth bits, point id << 8 | pixel in bin), see ScatterTargets
     uint32_t* offsets;    // [P + 1] per pixel: start of its list; [P] = fragments of the view
     uint64_t* fragments;
     uint8_t* list_is_cut;   // [P]
@@ -207,9 +208,17 @@ __global__ void __launch_bounds__(kBlock) bin_build_kernel(BuildPass a)
     // the same for every lane: tell the compiler, so that loops over the bin's records become scalar branches
     const uint32_t begin  = (uint32_t)__builtin_amdgcn_readfirstlane((int)a.bin_offsets[bin]);
     const uint32_t n      = (uint32_t)__builtin_amdgcn_readfirstlane((int)a.bin_offsets[bin + 1]) - begin;
-    // record r of the bin: its own room first, what did not fit there in the compact array
-    const uint4* recs = a.primary + (size_t)bin * kPrimaryCap;
-    const uint4* more = a.binned + begin;
+    // record r of the bin: its own room first, what did not fit there in the compact array; as (key low, key high,
+    // pixel in bin, 0) whatever its form in memory
+    auto record = [&](uint32_t r) {
+        const size_t at = r < (uint32_t)kPrimaryCap ? (size_t)bin * kPrimaryCap + r : (size_t)begin + r;
+        if (a.compact_records)
+        {
+            const uint2 v = reinterpret_cast<const uint2*>(r < (uint32_t)kPrimaryCap ? a.primary : a.binned)[at];
+            return make_uint4(v.y >> 8, v.x, v.y & 0xFFu, 0u);
+        }
+        return (r < (uint32_t)kPrimaryCap ? a.primary : a.binned)[at];
+    };
     const bool in_lds     = n <= (uint32_t)kBuildCap;
     s_cnt[tid] = 0u;
     __syncthreads();
@@ -232,7 +241,7 @@ __global__ void __launch_bounds__(kBlock) bin_build_kernel(BuildPass a)
             const uint32_t r = (uint32_t)(k * kBlock + tid);
             if (r < n)
             {
-                const uint4 rec     = recs[r];
+                const uint4 rec     = record(r);
                 const uint32_t px   = rec.z & (pixels - 1u);
                 const uint32_t rank = atomicAdd(&s_cnt[px], 1u);
                 key[k]              = ((uint64_t)rec.y << 32) | rec.x;
@@ -249,7 +258,7 @@ __global__ void __launch_bounds__(kBlock) bin_build_kernel(BuildPass a)
             for (int k = 0; k < 4; ++k)
             {
                 const uint32_t r = r0 + k * kBlock + tid;
-                px[k]            = r < n ? ((r < (uint32_t)kPrimaryCap ? recs[r] : more[r]).z & (pixels - 1u)) : 0xFFFFFFFFu;
+                px[k]            = r < n ? (record(r).z & (pixels - 1u)) : 0xFFFFFFFFu;
             }
 #pragma unroll
             for (int k = 0; k < 4; ++k)
@@ -396,7 +405,7 @@ __global__ void __launch_bounds__(kBlock) bin_build_kernel(BuildPass a)
             for (int k = 0; k < 4; ++k)
             {
                 const uint32_t r = r0 + k * kBlock + tid;
-                rec[k]           = r < n ? (r < (uint32_t)kPrimaryCap ? recs[r] : more[r]) : make_uint4(0u, 0u, 0xFFFFFFFFu, 0u);
+                rec[k]           = r < n ? record(r) : make_uint4(0u, 0u, 0xFFFFFFFFu, 0u);
             }
 #pragma unroll
             for (int k = 0; k < 4; ++k)

@@ -257,9 +257,13 @@ struct PackJob
 // cursor in a cache line of its own: appends to one cursor would queue up behind each other where many bins overflow
 // (a workgroup's segment has room for every hit the workgroups of that residue can produce). Bins are sized for an expected 1024 records at most, so the log stays empty or
 // short unless the cloud is far denser somewhere than on average.
+// A record is 16 bytes (key low, key high, pixel in bin, 0), or, where a point lands in one pixel per layer and point ids
+// fit 24 bits (`compact`), 8 bytes: (key high = depth bits, point id << 8 | pixel in bin). Half the bytes written here
+// and read again by the build pass.
 struct ScatterTargets
 {
-    uint4* primary;        // [bins][kPrimaryCap] records
+    uint4* primary;        // [bins][kPrimaryCap] records (uint2 records when compact)
+    int compact;
     uint4* log;            // [kLogSegments][segment_capacity]: key low, key high, pixel in bin, bin
     uint32_t* log_rank;    // the same shape: rank of the logged record inside its bin
     uint32_t* log_cursor;  // [kLogSegments], kLogCursorStride apart: entries in every segment (this view)
@@ -271,7 +275,13 @@ __device__ __forceinline__ void store_record(const ScatterTargets& t, bool valid
                                              uint32_t low, uint32_t depth_bits, uint32_t in_bin, int lane)
 {
     const bool over = valid && rank >= (uint32_t)kPrimaryCap;
-    if (valid && !over) t.primary[(size_t)bin * kPrimaryCap + rank] = make_uint4(low, depth_bits, in_bin, 0u);
+    if (valid && !over)
+    {
+        if (t.compact)
+            reinterpret_cast<uint2*>(t.primary)[(size_t)bin * kPrimaryCap + rank] = make_uint2(depth_bits, (low << 8) | in_bin);
+        else
+            t.primary[(size_t)bin * kPrimaryCap + rank] = make_uint4(low, depth_bits, in_bin, 0u);
+    }
     const uint64_t m = __ballot(over);
     if (m != 0ull)  // rare
     {
@@ -460,7 +470,11 @@ __global__ void __launch_bounds__(kBlock) overflow_move_kernel(ScatterTargets in
         {
             const uint4 rec    = in.log[first + e];
             const uint32_t pos = bin_offsets[rec.w] + in.log_rank[first + e];
-            if (pos < capacity) binned[pos] = make_uint4(rec.x, rec.y, rec.z, 0u);  // guard: never false
+            if (pos >= capacity) continue;  // guard: never true
+            if (in.compact)
+                reinterpret_cast<uint2*>(binned)[pos] = make_uint2(rec.y, (rec.x << 8) | rec.z);
+            else
+                binned[pos] = make_uint4(rec.x, rec.y, rec.z, 0u);
         }
     }
 }

@@ -148,6 +148,12 @@ inline int hits_of_mode(int render_mode)
     return render_mode == VETRAST_RENDER_BILINEAR_BLEND ? 4 : 1;
 }
 
+// Fragment records of 8 instead of 16 bytes: one hit per point and layer, point ids of 24 bits.
+inline bool compact_records(int64_t N, int hits)
+{
+    return hits == 1 && N <= (int64_t)(1 << 24);
+}
+
 inline int check_mode(int render_mode)
 {
     return (render_mode == VETRAST_RENDER_FULL_BLEND || render_mode == VETRAST_RENDER_FUZZY_BLEND ||
@@ -477,12 +483,13 @@ int vetrast_workspace_layout_for_mode(int32_t N, int32_t B, int32_t L, int32_t w
     lay->offsets_base   = at;
     lay->offsets_stride = align_up((P + 1) * sizeof(uint32_t), kAlign);
     at += lay->offsets_stride * B;
+    const size_t record_bytes = compact_records(N, hits) ? sizeof(uint2) : sizeof(uint4);
     lay->binned_base = at;
-    at += align_up(cap * sizeof(uint4), kAlign);
+    at += align_up(cap * record_bytes, kAlign);
     lay->log_base = at;
     at += align_up(log_records(N, L, hits) * sizeof(uint4), kAlign);
     lay->primary_base = at;
-    at += align_up(bins * (size_t)kPrimaryCap * sizeof(uint4), kAlign);
+    at += align_up(bins * (size_t)kPrimaryCap * record_bytes, kAlign);
     lay->views_base = at;
     at += align_up((size_t)B * sizeof(DeviceView), kAlign);
     lay->packed_base = at;
@@ -587,6 +594,7 @@ int vetrast_forward(vetrast_ctx* ctx, const vetrast_forward_args* a, void* strea
         uint4* binned            = ws_ptr<uint4>(ws, lay.binned_base);
         ScatterTargets targets;
         targets.primary      = ws_ptr<uint4>(ws, lay.primary_base);
+        targets.compact      = compact_records(N, hits) ? 1 : 0;
         targets.log          = ws_ptr<uint4>(ws, lay.log_base);
         targets.log_rank     = slots;
         targets.log_cursor   = ws_ptr<uint32_t>(ws, lay.log_cursor_base) + (size_t)b * kLogSegments * kLogCursorStride;
@@ -651,6 +659,7 @@ int vetrast_forward(vetrast_ctx* ctx, const vetrast_forward_args* a, void* strea
             bp.bin_offsets         = bin_counts;
             bp.primary             = targets.primary;
             bp.binned              = binned;
+            bp.compact_records     = targets.compact;
             bp.offsets             = offsets;
             bp.fragments           = fragments;
             bp.list_is_cut         = list_is_cut;
