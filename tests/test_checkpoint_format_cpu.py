@@ -28,7 +28,9 @@ def test_round_trip_through_the_shim(tmp_path):
     prefix = str(tmp_path / "scene_test_")
     torch_ops.save_scene_checkpoint(prefix, **want)
     got = torch_ops.load_scene_checkpoint(prefix)
-    assert sorted(got) == sorted(want)
+    # t_original_color is always written (the reference's module registers it): zeros when none was given
+    assert sorted(got) == sorted(list(want) + ["t_original_color"])
+    assert got["t_original_color"].shape == (500, 4) and not got["t_original_color"].any()
     for k, v in want.items():
         assert got[k].dtype == v.dtype and torch.equal(got[k], v), k
     # only the files whose tensors were given are written; missing files leave their tensors out
@@ -82,6 +84,71 @@ def test_module_archives_written_by_pytorch_load_through_the_shim(tmp_path):
     torch.jit.script(_Points(want["t_position"], want["t_index"])).save(prefix + "points.pth")
     torch.jit.script(_Texture(want)).save(prefix + "texture.pth")
     got = torch_ops.load_scene_checkpoint(prefix)
-    assert sorted(got) == ["background_color", "confidence_value_of_point", "t_index", "t_position", "texture"]
+    assert sorted(got) == ["background_color", "confidence_value_of_point", "t_index", "t_original_color", "t_position",
+                           "texture"]
     for k in got:
-        assert torch.equal(got[k], want[k]), k
+        if k != "t_original_color":
+            assert torch.equal(got[k], want[k]), k
+
+
+class _StrictPoints(torch.nn.Module):
+    """What torch::load of the reference's NeuralPointCloudCudaImpl demands of points.pth: Module::load reads every name
+    the module registered and throws on a missing one (src/lib/data/NeuralScene.cpp:349). load_state_dict(strict=True)
+    is the same rule on the Python side."""
+
+    def __init__(self, n, with_normal, with_cells, cells=0):
+        super().__init__()
+        self.t_position = torch.nn.Parameter(torch.zeros(n, 4))                      # NeuralPointCloudCuda.cpp:71
+        self.register_buffer("t_index", torch.zeros(n, 1, dtype=torch.int32))         # :72
+        self.register_buffer("t_original_color", torch.zeros(n, 4))                   # :73
+        if with_normal:
+            self.register_buffer("t_normal", torch.zeros(n, 1, dtype=torch.int32))    # :53
+        if with_cells:                                                                # :84-87
+            self.register_buffer("t_cell_bb_min", torch.zeros(cells, 3))
+            self.register_buffer("t_cell_bb_length", torch.zeros(cells, 3))
+            self.register_buffer("t_cell_value", torch.zeros(cells, 1))
+            self.register_buffer("t_cell_access_count", torch.zeros(cells, 1, dtype=torch.int32))
+
+
+def _strict_read(path, module):
+    archive = torch.jit.load(path)
+    state = {k: v for k, v in list(archive.named_parameters()) + list(archive.named_buffers())}
+    module.load_state_dict(state, strict=True)  # raises on a missing or an unexpected name
+    return state
+
+
+def test_points_file_holds_every_tensor_the_reference_module_registers(tmp_path):
+    want = _scene_tensors()
+    # 1. the rasterizer's tensors only, no index: identity index and zero colours are written
+    prefix = str(tmp_path / "scene_c_")
+    torch_ops.save_scene_checkpoint(prefix, t_position=want["t_position"])
+    state = _strict_read(prefix + "points.pth", _StrictPoints(500, False, False))
+    assert torch.equal(state["t_index"], torch.arange(500, dtype=torch.int32).reshape(-1, 1))
+    assert state["t_original_color"].shape == (500, 4) and state["t_original_color"].dtype == torch.float32
+    # 2. a cloud with colours, normals and the cell grid: carried through load and save unchanged
+    rng = np.random.default_rng(3)
+    extra = {
+        "t_original_color": torch.from_numpy(rng.uniform(size=(500, 4)).astype(np.float32)),
+        "t_normal": torch.from_numpy(rng.integers(0, 1 << 30, size=(500, 1)).astype(np.int32)),
+        "t_cell_bb_min": torch.from_numpy(rng.normal(size=(7, 3)).astype(np.float32)),
+        "t_cell_bb_length": torch.from_numpy(rng.uniform(size=(7, 3)).astype(np.float32)),
+        "t_cell_value": torch.from_numpy(rng.uniform(size=(7, 1)).astype(np.float32)),
+        "t_cell_access_count": torch.from_numpy(rng.integers(0, 9, size=(7, 1)).astype(np.int32)),
+    }
+    prefix = str(tmp_path / "scene_d_")
+    torch_ops.save_scene_checkpoint(prefix, t_position=want["t_position"], t_index=want["t_index"], **extra)
+    state = _strict_read(prefix + "points.pth", _StrictPoints(500, True, True, cells=7))
+    loaded = torch_ops.load_scene_checkpoint(prefix)
+    for k, v in extra.items():
+        assert torch.equal(state[k], v) and torch.equal(loaded[k], v), k
+    # ... and once more through the shim: load, save, strict read
+    prefix2 = str(tmp_path / "scene_e_")
+    torch_ops.save_scene_checkpoint(prefix2, **loaded)
+    state2 = _strict_read(prefix2 + "points.pth", _StrictPoints(500, True, True, cells=7))
+    for k in state:
+        assert torch.equal(state2[k], state[k]), k
+    # a module without normals refuses the file that has them, as Module::load would
+    import pytest
+
+    with pytest.raises(RuntimeError):
+        _strict_read(prefix2 + "points.pth", _StrictPoints(500, False, True, cells=7))

@@ -262,3 +262,99 @@ def test_render_module_environment_map_branch(cat_env_to_color, oracle):
     want = oracle.backward(ref, [np.ones_like(o) for o in ref.out], want_points=False)
     assert max_rel_err(texture.grad.cpu().numpy(), want["texture"]) <= 1e-4
     assert max_rel_err(confidence.grad.cpu().numpy().ravel(), want["confidence"]) <= 1e-4
+
+
+def _plain_call(scene, torch_ops, texture=None, confidence=None, intrinsics=None, train=False, **extra):
+    cu = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
+    B = scene.poses_se3.shape[0]
+    return torch_ops.blend_point_cloud(cu(scene.texture) if texture is None else texture, cu(scene.background),
+                                       cu(scene.position), torch.zeros((B, 6), dtype=torch.float64, device="cuda"),
+                                       cu(scene.intrinsics) if intrinsics is None else intrinsics,
+                                       cu(scene.confidence.reshape(1, -1)) if confidence is None else confidence,
+                                       cu(scene.poses_se3), None, _views(scene), scene.num_layers, train=train,
+                                       use_environment_map=0, drop_out_points_by_radius=0, need_point_gradient=0,
+                                       debug_max_list_length=scene.max_list_length, quirk_background_confidence_leak=0,
+                                       **extra)
+
+
+def test_cameras_with_distortion_are_refused_by_the_shim():
+    """Non-zero distortion coefficients (columns 5..12 of the intrinsics) must not render as an undistorted pinhole
+    through the drop-in seam: BlendPointCloud and FillSceneGridWithLoss throw. The check is repeated when the tensor
+    changes in place."""
+    from vet_amd import torch_ops
+
+    scene = synthetic.tiny_scene(num_points=1000, K=8, seed=36)
+    intr = torch.from_numpy(scene.intrinsics.copy()).cuda()
+    outs = _plain_call(scene, torch_ops, intrinsics=intr)  # zero coefficients: fine
+    assert len(outs) == scene.num_layers
+    intr[0, 7] = 1e-3  # k3, changed in place: same storage, new version
+    with pytest.raises(RuntimeError, match="distortion"):
+        _plain_call(scene, torch_ops, intrinsics=intr)
+    mn, ln = synthetic.cell_grid(scene.position[:, :3], 0.5)
+    dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
+    value = torch.zeros((len(mn), 1), device="cuda")
+    count = torch.zeros((len(mn), 1), dtype=torch.int32, device="cuda")
+    with pytest.raises(RuntimeError, match="distortion"):
+        torch_ops.fill_scene_grid_with_loss(0, dev(mn), dev(ln), value, count, _views(scene), dev(scene.poses_se3), intr,
+                                            torch.zeros((3, scene.views[0].h, scene.views[0].w), device="cuda"))
+    assert int(count.sum()) == 0
+    intr[0, 7] = 0.0
+    assert len(_plain_call(scene, torch_ops, intrinsics=intr)) == scene.num_layers
+
+
+def test_add_depth_to_network_appends_a_zero_channel(oracle):
+    """The blend modes never write the depth tensors (src/lib/rendering/PointRenderer.cu:1061-1066 hands out the zero-filled
+    buffers); PointRenderModuleImpl::forward appends them to the images as a channel (RenderModule.cpp:223-232), behind
+    the masks' channel position: images [B,C+1,h,w] with a zero last channel, masks unchanged, gradients as without."""
+    from vet_amd import torch_ops
+
+    scene = synthetic.tiny_scene(num_points=3000, K=8, seed=37, num_views=2)
+    params = make_params(scene, output_background_mask=1, output_background_mask_value=0.5, need_point_gradient=0)
+    ref = oracle.forward(scene, params)
+    cu = lambda a, rg=False: torch.from_numpy(np.ascontiguousarray(a)).cuda().requires_grad_(rg)
+    texture, confidence = cu(scene.texture, True), cu(scene.confidence.reshape(1, -1), True)
+    outs = _plain_call(scene, torch_ops, texture=texture, confidence=confidence, train=True, add_depth_to_network=1,
+                       output_background_mask=1, output_background_mask_value=0.5)
+    L, Cn = scene.num_layers, scene.num_channels
+    assert len(outs) == 2 * L
+    for l in range(L):
+        img = outs[l].detach().cpu().numpy()
+        assert img.shape[1] == Cn + 1
+        np.testing.assert_array_equal(img[:, :Cn], ref.out[l])
+        assert not img[:, Cn:].any()
+        np.testing.assert_array_equal(outs[L + l].cpu().numpy(), ref.out_mask[l])
+    grad_out = scene.grad_out()
+    sum((outs[l][:, :Cn] * cu(grad_out[l])).sum() + outs[l][:, Cn:].sum() for l in range(L)).backward()
+    want = oracle.backward(ref, grad_out, want_points=False)
+    assert max_rel_err(texture.grad.cpu().numpy(), want["texture"]) <= 1e-4
+    assert max_rel_err(confidence.grad.cpu().numpy().ravel(), want["confidence"]) <= 1e-4
+
+
+def test_training_steps_share_one_workspace():
+    """The workspace a training forward saves for its backward pass is taken again by the next step once the graph of
+    the step before is gone; while a graph is alive its workspace is left alone."""
+    from vet_amd import torch_ops
+
+    scene = synthetic.tiny_scene(num_points=2000, K=8, seed=38)
+    cu = lambda a, rg=False: torch.from_numpy(np.ascontiguousarray(a)).cuda().requires_grad_(rg)
+    texture = cu(scene.texture, True)
+    seen = []
+    for it in range(3):
+        outs = _plain_call(scene, torch_ops, texture=texture, train=True)
+        seen.append(torch_ops.train_workspace_info())
+        sum(o.sum() for o in outs).backward()
+        del outs
+    assert seen[0][0] != 0 and seen[0] == seen[1] == seen[2]
+    first_grad = texture.grad.clone()
+    # two graphs alive at once: the second call must not write into the first one's workspace
+    a = _plain_call(scene, torch_ops, texture=texture, train=True)
+    ptr_a = torch_ops.train_workspace_info()[0]
+    b = _plain_call(scene, torch_ops, texture=texture, train=True)
+    ptr_b = torch_ops.train_workspace_info()[0]
+    assert ptr_a != ptr_b
+    texture.grad = None
+    sum(o.sum() for o in a).backward()
+    np.testing.assert_array_equal(texture.grad.cpu().numpy() * 3, first_grad.cpu().numpy())  # same gradient each step
+    texture.grad = None
+    sum(o.sum() for o in b).backward()
+    np.testing.assert_array_equal(texture.grad.cpu().numpy() * 3, first_grad.cpu().numpy())

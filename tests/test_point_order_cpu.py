@@ -58,3 +58,55 @@ def test_blocks_are_shuffled_whole():
         assert np.all(np.diff(seg) == 1) and seg[0] % 256 == 0
     assert len(starts) + 1 == (10_000 + 255) // 256
     assert torch_ops.morton_block_shuffle_order(torch.zeros((0, 3))).numel() == 0
+
+
+def test_blocks_sorted_by_radius():
+    """SceneData::SortBlocksByRadius(256) (src/lib/data/SceneData.cpp:1005-1018): every complete block sorted by radius,
+    the incomplete tail left alone, nothing moves between blocks."""
+    rng = np.random.default_rng(5)
+    radius = rng.uniform(0.001, 0.1, size=1000).astype(np.float32)
+    order = torch_ops.sort_blocks_by_radius_order(torch.from_numpy(radius), block=256).numpy()
+    assert sorted(order.tolist()) == list(range(1000))
+    for b in range(3):  # 1000 // 256 complete blocks
+        seg = order[256 * b:256 * (b + 1)]
+        assert seg.min() >= 256 * b and seg.max() < 256 * (b + 1)
+        assert np.all(np.diff(radius[seg]) >= 0)
+        np.testing.assert_array_equal(seg, 256 * b + np.argsort(radius[256 * b:256 * (b + 1)], kind="stable"))
+    np.testing.assert_array_equal(order[768:], np.arange(768, 1000))
+
+
+def test_scene_preprocess_order_is_the_three_steps_in_a_row():
+    rng = np.random.default_rng(6)
+    pos = np.zeros((5000, 4), np.float32)
+    pos[:, :3] = rng.normal(size=(5000, 3))
+    pos[:, 3] = rng.uniform(0.001, 0.05, size=5000)
+    t = torch.from_numpy(pos)
+    first = torch_ops.morton_block_shuffle_order(t, block=256, seed=9).numpy()
+    second = torch_ops.sort_blocks_by_radius_order(torch.from_numpy(pos[first, 3]), block=256).numpy()
+    got = torch_ops.scene_preprocess_order(t, block=256, seed=9).numpy()
+    np.testing.assert_array_equal(got, first[second])
+    # every block of the result is one block of the shuffled Morton order, radius ascending
+    for b in range(5000 // 256):
+        assert set(got[256 * b:256 * (b + 1)].tolist()) == set(first[256 * b:256 * (b + 1)].tolist())
+        assert np.all(np.diff(pos[got[256 * b:256 * (b + 1)], 3]) >= 0)
+    # the generator of the benchmark scenes sorts its blocks the same way (its block shuffle draws from another
+    # generator, so only the structure can be compared)
+    own = synthetic.vet_preprocess_order(pos[:, :3], seed=9, block=256, radius=pos[:, 3])
+    plain = synthetic.vet_preprocess_order(pos[:, :3], seed=9, block=256)
+    for b in range(5000 // 256):
+        assert set(own[256 * b:256 * (b + 1)].tolist()) == set(plain[256 * b:256 * (b + 1)].tolist())
+        assert np.all(np.diff(pos[own[256 * b:256 * (b + 1)], 3]) >= 0)
+    np.testing.assert_array_equal(own[5000 // 256 * 256:], plain[5000 // 256 * 256:])
+
+
+def test_grown_cloud_order():
+    """A cloud that grew during training (NeuralScene::AddNewPoints appends, src/lib/data/NeuralScene.cpp:1013): the
+    preprocessed part keeps its order, the appended fifth is in arbitrary order."""
+    s = synthetic.config2(num_points=20_000, point_order="grown")
+    ordered = synthetic.config2(num_points=20_000, point_order="vet_preprocess")
+    assert s.num_points == ordered.num_points == 20_000
+    # the same set of points
+    a = np.sort(s.position.view([("", np.float32)] * 4).ravel())
+    b = np.sort(ordered.position.view([("", np.float32)] * 4).ravel())
+    assert np.array_equal(a, b)
+    assert not np.array_equal(s.position, ordered.position)

@@ -177,11 +177,12 @@ def _spread_bits21(v):
     return v
 
 
-def vet_preprocess_order(xyz, seed, block=256):
+def vet_preprocess_order(xyz, seed, block=256, radius=None):
     """The point order VET's scene preprocessing produces before the rasterizer ever sees a cloud:
-    ReorderMorton64() followed by RandomBlockShuffle(256) (src/lib/data/SceneData.cpp:105-106 of the reference).
+    ReorderMorton64() followed by RandomBlockShuffle(256) (src/lib/data/SceneData.cpp:105-106 of the reference) and, with
+    `radius` (the drop-out radius of every point), SortBlocksByRadius(256) (:108,1005-1018).
     Returns the permutation: 63-bit Morton order of the positions in their bounding box, then whole blocks of `block`
-    consecutive points shuffled with the seeded generator."""
+    consecutive points shuffled with the seeded generator, then every complete block sorted by radius."""
     xyz = np.asarray(xyz, dtype=np.float64)
     lo, hi = xyz.min(axis=0), xyz.max(axis=0)
     cell = np.floor((xyz - lo) / np.maximum(hi - lo, 1e-30) * ((1 << 21) - 1)).astype(np.uint64)
@@ -193,7 +194,42 @@ def vet_preprocess_order(xyz, seed, block=256):
     block_perm = np.argsort(keys, kind="stable")
     idx = (block_perm[:, None] * block + np.arange(block)[None, :]).reshape(-1)
     idx = idx[idx < n]
-    return order[idx]
+    order = order[idx]
+    if radius is not None:
+        full = n // block * block
+        r = np.asarray(radius)[order[:full]].reshape(-1, block)
+        inner = np.argsort(r, axis=1, kind="stable") + (np.arange(n // block) * block)[:, None]
+        order = np.concatenate([order[:full][inner.reshape(-1)], order[full:]])
+    return order
+
+
+def ordered_cloud(xyz, radius, seed, point_order):
+    """Positions and radii in one of the orders a rasterizer meets:
+    "vet_preprocess": what VET's loader hands over (Morton order, 256-point blocks shuffled, blocks sorted by radius);
+    "generated": the generator's order (primitive by primitive, random inside);
+    "grown": a cloud that grew during training: four fifths preprocessed, one fifth (a random subset) appended behind
+    them in arbitrary order, as NeuralScene::AddNewPoints leaves it (src/lib/data/NeuralScene.cpp:1013; the reference
+    does not sort again)."""
+    if point_order == "generated":
+        return xyz, radius
+    if point_order == "vet_preprocess":
+        o = vet_preprocess_order(xyz, seed, radius=radius)
+        return xyz[o], radius[o]
+    assert point_order == "grown", point_order
+    n = xyz.shape[0]
+    pick = np.argsort(Stream(seed, "grown").u64(n), kind="stable")
+    old, new = pick[: n - n // 5], pick[n - n // 5:]
+    o = old[vet_preprocess_order(xyz[old], seed, radius=radius[old])]
+    o = np.concatenate([o, new])
+    return xyz[o], radius[o]
+
+
+def point_radii(seed, n, spread):
+    """Drop-out radius per point: 1 cm, or with `spread` > 0 log-normal around it (VET computes it from the distance to
+    the nearest neighbours, src/lib/data/SceneData.cpp:983-1001)."""
+    if spread <= 0:
+        return np.full(n, 0.01, dtype=np.float32)
+    return (0.01 * np.exp(spread * Stream(seed, "radius").normal(n))).astype(np.float32)
 
 
 def _descriptors(seed, N, channels=4, sigma=0.5):
@@ -203,22 +239,19 @@ def _descriptors(seed, N, channels=4, sigma=0.5):
     return tex, conf, bg
 
 
-def config2(num_points=2_000_000, seed=1, w=1920, h=1080, num_layers=4, K=16, point_order="vet_preprocess") -> Scene:
+def config2(num_points=2_000_000, seed=1, w=1920, h=1080, num_layers=4, K=16, point_order="vet_preprocess",
+            radius_spread=0.0) -> Scene:
     """SfM-like scene: points on 200 planes/spheres in a 10 m box, 1080p, fx=1000, 4 layers, K=16.
 
-    point_order: "vet_preprocess" lists the points the way VET's loader hands them to the rasterizer (Morton order,
-    256-point blocks shuffled); "generated" keeps the generator's order (primitive by primitive, random inside)."""
+    point_order: see ordered_cloud. radius_spread: 0 gives every point the drop-out radius 1 cm; > 0 spreads the radii
+    log-normally (for runs with drop_out_points_by_radius)."""
     prims = 200
     per = max(1, num_points // prims)
     N = prims * per
     pos = np.empty((N, 4), dtype=np.float32)
-    xyz = surface_points(seed, prims, per)
-    if point_order == "vet_preprocess":
-        xyz = xyz[vet_preprocess_order(xyz, seed)]
-    else:
-        assert point_order == "generated", point_order
+    xyz, radius = ordered_cloud(surface_points(seed, prims, per), point_radii(seed, N, radius_spread), seed, point_order)
     pos[:, :3] = xyz.astype(np.float32)
-    pos[:, 3] = 0.01
+    pos[:, 3] = radius
     tex, conf, bg = _descriptors(seed, N)
     scale = w / 1920.0
     return Scene("config2_sfm", pos, tex, conf, bg, _identity_pose((0, 0, 4.5)),

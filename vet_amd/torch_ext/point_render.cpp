@@ -82,7 +82,6 @@ vetrast_forward_args make_forward_args(NeuralRenderInfo* info, const torch::Tens
                     info->params.render_mode == VETRAST_RENDER_FUZZY_BLEND ||
                     info->params.render_mode == VETRAST_RENDER_BILINEAR_BLEND,
                 "only render_mode 1 (FULL_BLEND), 2 (FUZZY_BLEND) and 3 (BILINEAR_BLEND) are implemented");
-    TORCH_CHECK(!info->params.add_depth_to_network, "add_depth_to_network is not part of the blending path");
     TORCH_CHECK(!info->images.empty(), "no views");
 
     vetrast_forward_args a;
@@ -125,6 +124,26 @@ PointRendererCache::~PointRendererCache()
     vetrast_destroy(ctx);
 }
 
+void PointRendererCache::CheckIntrinsics(const torch::Tensor& intrinsics)
+{
+    TORCH_CHECK(intrinsics.defined() && intrinsics.dim() == 2 && intrinsics.size(1) == 13,
+                "intrinsics must be [num_cameras,13]");
+    const void* ptr       = intrinsics.data_ptr();
+    const int64_t version = (int64_t)intrinsics._version();
+    if (ptr == checked_intrinsics_ptr_ && version == checked_intrinsics_version_ &&
+        intrinsics.numel() == checked_intrinsics_numel_)
+        return;
+    // blocking: one device -> host read per change of the tensor
+    const bool distorted = intrinsics.detach().slice(1, 5, 13).ne(0).any().item<bool>();
+    TORCH_CHECK(!distorted,
+                "a camera has non-zero distortion coefficients (columns 5..12 of intrinsics): the distortion model of the "
+                "reference lives in saiga and is not implemented; such cameras are refused rather than rendered as "
+                "undistorted pinholes");
+    checked_intrinsics_ptr_     = ptr;
+    checked_intrinsics_version_ = version;
+    checked_intrinsics_numel_   = intrinsics.numel();
+}
+
 void PointRendererCache::FillSceneGridWithLoss(int batch, const CellTensors& cells,
                                                const std::vector<ReducedImageInfo>& images, torch::Tensor poses_se3,
                                                torch::Tensor intrinsics, torch::Tensor loss_img)
@@ -139,6 +158,7 @@ void PointRendererCache::FillSceneGridWithLoss(int batch, const CellTensors& cel
     TORCH_CHECK(is_dev(poses_se3, torch::kFloat64) && is_dev(intrinsics, torch::kFloat32) && is_dev(loss_img, torch::kFloat32),
                 "FillSceneGridWithLoss: poses_se3 (float64), intrinsics and loss_img (float32) must be contiguous CUDA tensors");
     TORCH_CHECK(loss_img.dim() == 3, "FillSceneGridWithLoss: loss_img is [C,h,w]");
+    CheckIntrinsics(intrinsics);
     const int64_t n = cells.t_cell_value.numel();
     TORCH_CHECK(cells.t_cell_bb_min.numel() == 3 * n && cells.t_cell_bb_length.numel() == 3 * n &&
                     cells.t_cell_access_count.numel() == n,
@@ -190,6 +210,7 @@ torch::autograd::variable_list PointRender::forward(torch::autograd::AutogradCon
     const int B = (int)info->images.size(), L = info->num_layers, C = (int)texture.size(0);
     const int64_t N = points.size(0);
     auto f32        = torch::TensorOptions().device(points.device()).dtype(torch::kFloat32);
+    info->cache->CheckIntrinsics(intrinsics);
 
     // dropout mask per view, PointRenderer.cu:461-468 (the mask is 1 where a point is dropped)
     torch::Tensor dropout;
@@ -211,7 +232,14 @@ torch::autograd::variable_list PointRender::forward(torch::autograd::AutogradCon
     auto u8 = torch::TensorOptions().device(points.device()).dtype(torch::kUInt8);
     torch::Tensor workspace;
     if (need_backward)
-        workspace = torch::empty({(int64_t)lay.total_bytes}, u8);  // saved for backward, like the reference's buffers
+    {
+        // Saved for backward, like the reference's buffers. The workspace of the step before is taken again once the
+        // graph that saved it is gone (nothing but the cache holds it): the usual training loop allocates it once.
+        auto& ws = info->cache->train_workspace;
+        if (!ws.defined() || ws.use_count() > 1 || ws.numel() < (int64_t)lay.total_bytes || ws.device() != points.device())
+            ws = torch::empty({(int64_t)lay.total_bytes}, u8);
+        workspace = ws;
+    }
     else
     {
         auto& ws = info->cache->eval_workspace;
@@ -265,8 +293,20 @@ torch::autograd::variable_list PointRender::forward(torch::autograd::AutogradCon
         ctx->saved_data["intr_need_grad"]   = intrinsics.requires_grad();
         ctx->saved_data["num_poses"]        = (int64_t)poses_se3.size(0);
     }
-    // masks are not differentiable (the reference detaches them in RenderModule.cpp:74-102)
-    if (ctx) ctx->mark_non_differentiable(mask);
+    // With add_depth_to_network the output list carries L depth tensors behind the images
+    // (src/lib/rendering/PointRenderer.cu:1061-1066). The blend modes never write them: they are the zero-filled
+    // buffers of the cache (:402-470), which is what is returned here.
+    std::vector<torch::Tensor> depth;
+    if (info->params.add_depth_to_network)
+        for (int l = 0; l < L; ++l) depth.push_back(torch::zeros({B, 1, lay.layer_h[l], lay.layer_w[l]}, f32));
+    // masks are not differentiable (the reference detaches them in RenderModule.cpp:74-102); nor are the zero depths
+    if (ctx)
+    {
+        std::vector<torch::Tensor> constants = mask;
+        constants.insert(constants.end(), depth.begin(), depth.end());
+        ctx->mark_non_differentiable(constants);
+    }
+    out.insert(out.end(), depth.begin(), depth.end());
     out.insert(out.end(), mask.begin(), mask.end());
     return out;
 }
@@ -355,7 +395,6 @@ namespace vet_amd
 std::pair<std::vector<torch::Tensor>, std::vector<torch::Tensor>> PointRenderModule::forward(NeuralRenderInfo* nri)
 {
     TORCH_CHECK(nri, "PointRenderModule::forward: null NeuralRenderInfo");
-    TORCH_CHECK(!nri->params.add_depth_to_network, "add_depth_to_network is not available");
     nri->cache = cache.get();
     const bool with_environment = environment_map && enable_environment_map;
     TORCH_CHECK(!with_environment || nri->params.output_background_mask,
@@ -383,16 +422,22 @@ std::pair<std::vector<torch::Tensor>, std::vector<torch::Tensor>> PointRenderMod
     }
     const int L = nri->num_layers;
     std::vector<torch::Tensor> images(combined.begin(), combined.begin() + L);
-    std::vector<torch::Tensor> masks;
+    // RenderModule.cpp:76-100: then the depths (with add_depth_to_network), then the masks
+    const bool with_depth = nri->params.add_depth_to_network;
+    std::vector<torch::Tensor> depths, masks;
+    const int expected = L * (1 + (with_depth ? 1 : 0) + (nri->params.output_background_mask ? 1 : 0));
+    TORCH_CHECK((int)combined.size() == expected, "BlendPointCloud returned ", combined.size(), " tensors, expected ", expected);
+    if (with_depth) depths.assign(combined.begin() + L, combined.begin() + 2 * L);
     if (nri->params.output_background_mask)
     {
-        TORCH_CHECK((int)combined.size() == 2 * L, "BlendPointCloud returned ", combined.size(), " tensors, expected ", 2 * L);
-        masks.assign(combined.begin() + L, combined.end());
+        masks.assign(combined.begin() + (with_depth ? 2 : 1) * L, combined.end());
         for (auto& m : masks) m = m.detach();
     }
     if (super_sampling)
     {
+        // RenderModule.cpp:102-127 pools images, depths and masks alike
         for (auto& img : images) img = torch::avg_pool2d(img, {2, 2});
+        for (auto& d : depths) d = torch::avg_pool2d(d, {2, 2});
         for (auto& m : masks) m = torch::avg_pool2d(m, {2, 2});
         rescale(0.5f);
     }
@@ -429,6 +474,8 @@ std::pair<std::vector<torch::Tensor>, std::vector<torch::Tensor>> PointRenderMod
         TORCH_CHECK(!masks.empty(), "cat_masks_to_color needs output_background_mask");
         for (int i = 0; i < L; ++i) images[i] = torch::cat({images[i], masks[i]}, 1);
     }
+    if (with_depth)  // RenderModule.cpp:223-232
+        for (int i = 0; i < L; ++i) images[i] = torch::cat({images[i], depths[i]}, 1);
     TORCH_CHECK(images.front().size(2) == nri->images.front().h && images.front().size(3) == nri->images.front().w,
                 "PointRenderModule: output size does not match the view");
     return {images, masks};
@@ -464,6 +511,13 @@ SceneTensors LoadSceneCheckpoint(const std::string& prefix, torch::Device device
         {
             TORCH_CHECK(read_entry(ar, "t_position", st.t_position, false), "points.pth has no t_position");
             read_entry(ar, "t_index", st.t_index, true);
+            // what the rasterizer does not read is carried along for SaveSceneCheckpoint
+            read_entry(ar, "t_original_color", st.t_original_color, true);
+            read_entry(ar, "t_normal", st.t_normal, true);
+            read_entry(ar, "t_cell_bb_min", st.t_cell_bb_min, true);
+            read_entry(ar, "t_cell_bb_length", st.t_cell_bb_length, true);
+            read_entry(ar, "t_cell_value", st.t_cell_value, true);
+            read_entry(ar, "t_cell_access_count", st.t_cell_access_count, true);
             TORCH_CHECK(st.t_position.scalar_type() == torch::kFloat32 && st.t_position.dim() == 2 && st.t_position.size(1) == 4,
                         "t_position must be [N,4] float32");
             TORCH_CHECK(!st.t_index.defined() ||
@@ -505,8 +559,24 @@ void SaveSceneCheckpoint(const std::string& prefix, const SceneTensors& st)
     if (st.t_position.defined())
     {
         torch::serialize::OutputArchive ar;
+        // Every name NeuralPointCloudCudaImpl registers has to be there: torch::load of that module
+        // (src/lib/data/NeuralScene.cpp:349) reads them all and throws on a missing one. t_position, t_index and
+        // t_original_color are always registered (src/lib/rendering/NeuralPointCloudCuda.cpp:71-73); an index the bundle
+        // does not hold is the identity, colours it does not hold are written as zeros.
+        const int64_t n = st.t_position.size(0);
         ar.write("t_position", cpu(st.t_position), false);
-        if (st.t_index.defined()) ar.write("t_index", cpu(st.t_index), true);
+        ar.write("t_index", st.t_index.defined() ? cpu(st.t_index) : torch::arange(n, torch::kInt32).reshape({n, 1}), true);
+        ar.write("t_original_color", st.t_original_color.defined() ? cpu(st.t_original_color) : torch::zeros({n, 4}), true);
+        if (st.t_normal.defined()) ar.write("t_normal", cpu(st.t_normal), true);
+        if (st.t_cell_bb_min.defined())
+        {
+            TORCH_CHECK(st.t_cell_bb_length.defined() && st.t_cell_value.defined() && st.t_cell_access_count.defined(),
+                        "SaveSceneCheckpoint: the four cell tensors go together");
+            ar.write("t_cell_bb_min", cpu(st.t_cell_bb_min), true);
+            ar.write("t_cell_bb_length", cpu(st.t_cell_bb_length), true);
+            ar.write("t_cell_value", cpu(st.t_cell_value), true);
+            ar.write("t_cell_access_count", cpu(st.t_cell_access_count), true);
+        }
         ar.save_to(prefix + "points.pth");
     }
     if (st.texture.defined())
@@ -596,6 +666,29 @@ torch::Tensor MortonBlockShuffleOrder(torch::Tensor positions, int64_t block, ui
             o[w++] = keyed[(size_t)k].second;
     return out;
 }
+
+torch::Tensor SortBlocksByRadiusOrder(torch::Tensor radius, int64_t block)
+{
+    TORCH_CHECK(radius.dim() == 1 && !radius.is_cuda() && block >= 1, "SortBlocksByRadiusOrder: radius is a [N] CPU tensor");
+    const torch::Tensor r = radius.to(torch::kFloat32).contiguous();
+    const int64_t n       = r.size(0);
+    const float* rv       = r.data_ptr<float>();
+    torch::Tensor out     = torch::arange(n, torch::kInt64);
+    int64_t* o            = out.data_ptr<int64_t>();
+    // complete blocks only: n_blocks = NumVertices() / block_size, src/lib/data/SceneData.cpp:1007
+    for (int64_t b = 0; b < n / block; ++b)
+        std::stable_sort(o + b * block, o + (b + 1) * block, [rv](int64_t i1, int64_t i2) { return rv[i1] < rv[i2]; });
+    return out;
+}
+
+torch::Tensor ScenePreprocessOrder(torch::Tensor positions_radius, int64_t block, uint64_t seed)
+{
+    TORCH_CHECK(positions_radius.dim() == 2 && positions_radius.size(1) == 4 && !positions_radius.is_cuda(),
+                "ScenePreprocessOrder: positions_radius is a [N,4] CPU tensor (x, y, z, drop-out radius)");
+    const torch::Tensor first  = MortonBlockShuffleOrder(positions_radius, block, seed);
+    const torch::Tensor radius = positions_radius.select(1, 3).index_select(0, first);
+    return first.index_select(0, SortBlocksByRadiusOrder(radius, block));
+}
 }  // namespace vet_amd
 
 // ---- Python binding used by the tests: builds a NeuralRenderInfo from plain arguments and calls BlendPointCloud ----
@@ -665,13 +758,15 @@ std::vector<torch::Tensor> blend_point_cloud(torch::Tensor texture, torch::Tenso
         else if (k == "camera_gradient_normalization") p.camera_gradient_normalization = as_d() != 0;
         else if (k == "fused_confidence_scale") p.fused_confidence_scale = (float)as_d();
         else if (k == "fused_texture_abs") p.fused_texture_abs = as_d() != 0;
+        else if (k == "add_depth_to_network") p.add_depth_to_network = as_d() != 0;
+        else if (k == "dist_cutoff") p.dist_cutoff = (float)as_d();
         else if (k == "super_sampling") super_sampling = as_d() != 0;
         else if (k == "cat_masks_to_color") cat_masks_to_color = as_d() != 0;
         else if (k == "cat_env_to_color") cat_env_to_color = as_d() != 0;
         else if (k == "no_envmap_at_points") no_envmap_at_points = as_d() != 0;
         else TORCH_CHECK(false, "unknown RenderParams field ", k);
     }
-    if (super_sampling || cat_masks_to_color || !environment.is_none())
+    if (super_sampling || cat_masks_to_color || p.add_depth_to_network || !environment.is_none())
     {
         // through the caller glue of the reference (PointRenderModuleImpl::forward): images, then masks
         PointRenderModule module;
@@ -803,6 +898,12 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
                 else if (k == "tangent_poses") st.tangent_poses = t;
                 else if (k == "poses_se3") st.poses_se3 = t;
                 else if (k == "intrinsics") st.intrinsics = t;
+                else if (k == "t_original_color") st.t_original_color = t;
+                else if (k == "t_normal") st.t_normal = t;
+                else if (k == "t_cell_bb_min") st.t_cell_bb_min = t;
+                else if (k == "t_cell_bb_length") st.t_cell_bb_length = t;
+                else if (k == "t_cell_value") st.t_cell_value = t;
+                else if (k == "t_cell_access_count") st.t_cell_access_count = t;
                 else TORCH_CHECK(false, "unknown scene tensor ", k);
             }
             vet_amd::SaveSceneCheckpoint(prefix, st);
@@ -824,12 +925,33 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
             put("tangent_poses", st.tangent_poses);
             put("poses_se3", st.poses_se3);
             put("intrinsics", st.intrinsics);
+            put("t_original_color", st.t_original_color);
+            put("t_normal", st.t_normal);
+            put("t_cell_bb_min", st.t_cell_bb_min);
+            put("t_cell_bb_length", st.t_cell_bb_length);
+            put("t_cell_value", st.t_cell_value);
+            put("t_cell_access_count", st.t_cell_access_count);
             return d;
         },
         "NeuralScene::LoadCheckpoint of the reference for the tensors the rasterizer reads");
     m.def("morton_block_shuffle_order", &vet_amd::MortonBlockShuffleOrder, pybind11::arg("positions"),
           pybind11::arg("block") = 256, pybind11::arg("seed") = 0,
           "ReorderMorton64 + RandomBlockShuffle(block) of the reference's scene preprocessing, as a permutation");
+    m.def("sort_blocks_by_radius_order", &vet_amd::SortBlocksByRadiusOrder, pybind11::arg("radius"), pybind11::arg("block") = 256,
+          "SceneData::SortBlocksByRadius(block) of the reference's scene preprocessing, as a permutation");
+    m.def("scene_preprocess_order", &vet_amd::ScenePreprocessOrder, pybind11::arg("positions_radius"),
+          pybind11::arg("block") = 256, pybind11::arg("seed") = 0,
+          "ReorderMorton64 + RandomBlockShuffle + SortBlocksByRadius of the reference's scene preprocessing, as a permutation");
+    m.def(
+        "train_workspace_info",
+        []() {
+            pybind11::dict d;
+            d["defined"] = g_cache && g_cache->train_workspace.defined();
+            d["data_ptr"] = (g_cache && g_cache->train_workspace.defined()) ? (int64_t)(intptr_t)g_cache->train_workspace.data_ptr() : (int64_t)0;
+            d["bytes"]    = (g_cache && g_cache->train_workspace.defined()) ? g_cache->train_workspace.numel() : (int64_t)0;
+            return d;
+        },
+        "address and size of the workspace the binding's cache keeps for training steps (for the tests)");
     m.def("blend_point_cloud", &blend_point_cloud, pybind11::arg("texture"), pybind11::arg("background_color"),
           pybind11::arg("points"), pybind11::arg("pose_tangents"), pybind11::arg("intrinsics"), pybind11::arg("confidence"),
           pybind11::arg("poses_se3"), pybind11::arg("t_index"), pybind11::arg("views"), pybind11::arg("num_layers"),

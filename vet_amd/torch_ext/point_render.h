@@ -32,7 +32,9 @@ struct RenderParams
     int num_texture_channels           = -1;
     bool output_background_mask        = false;
     float output_background_mask_value = 0.f;
-    bool add_depth_to_network          = false;  // not produced by FULL_BLEND in the reference either (depth images stay zero)
+    bool add_depth_to_network          = false;  // the blend modes leave the depth images at zero, as the reference does
+    float dist_cutoff                  = 20.f;   // accepted and ignored: it only steers saiga's distortion model, and
+                                                 // cameras with non-zero distortion coefficients are refused
     float stability_cutoff_value       = 10000.f;
     bool need_point_gradient           = true;
     bool use_environment_map           = true;
@@ -64,6 +66,12 @@ struct SceneTensors
     torch::Tensor dynamic_refinement_t;       // scene->dynamic_refinement_t                [1] dummy
     torch::Tensor poses_se3;                  // scene->poses->poses_se3                    [F,8] f64
     torch::Tensor t_index;                    // scene->point_cloud_cuda->t_index           [N,1] i32, may be undefined
+    // Entries of the reference's point cloud module that the rasterizer does not read; kept so that a checkpoint that is
+    // loaded and saved again still holds every tensor NeuralPointCloudCudaImpl registers
+    // (src/lib/rendering/NeuralPointCloudCuda.cpp:53,71-73,84-87).
+    torch::Tensor t_original_color;           // buffer [N,4] f32, always registered by the reference
+    torch::Tensor t_normal;                   // buffer [N,1] i32 (10-bit packed), only with normals
+    torch::Tensor t_cell_bb_min, t_cell_bb_length, t_cell_value, t_cell_access_count;  // buffers, only with use_grid_loss
 };
 
 // The cell tensors of the point cloud (src/lib/rendering/NeuralPointCloudCuda.h:100-106).
@@ -86,6 +94,14 @@ class PointRendererCache
     PointRendererCache& operator=(const PointRendererCache&) = delete;
     vetrast_ctx* ctx = nullptr;
     torch::Tensor eval_workspace;
+    // The workspace of the last forward call that was saved for a backward pass. The next such call takes it again if
+    // nothing but this cache still holds it (the graph of that step has been released) and it is large enough: a
+    // training loop then runs in one workspace instead of allocating one per step.
+    torch::Tensor train_workspace;
+    // Cameras with non-zero distortion coefficients are refused (their model lives in saiga, which is not available). The
+    // coefficients sit in device memory, so checking them costs a blocking read: it is only repeated when the intrinsics
+    // tensor or its version counter changes. Throws if columns 5..12 of `intrinsics` [num_cameras,13] are not all zero.
+    void CheckIntrinsics(const torch::Tensor& intrinsics);
     // layers_cuda[l].weight of the reference's cache (src/lib/rendering/PointRenderer.h:131, written at
     // src/lib/rendering/RenderForward.cu:1355-1356): per layer [B,1,h_l,w_l], the transmittance left behind the last
     // blended fragment of every pixel. Only kept up to date by BlendPointCloud while keep_layer_weights is set.
@@ -100,6 +116,10 @@ class PointRendererCache
     void FillSceneGridWithLoss(int batch, const CellTensors& cells, const std::vector<ReducedImageInfo>& images,
                                torch::Tensor poses_se3, torch::Tensor intrinsics, torch::Tensor loss_img);
     torch::Tensor lift_workspace;
+
+   private:
+    const void* checked_intrinsics_ptr_ = nullptr;
+    int64_t checked_intrinsics_version_ = -1, checked_intrinsics_numel_ = -1;
 };
 
 class NeuralRenderInfo : public torch::CustomClassHolder
@@ -156,8 +176,9 @@ class MyAdam
     std::unique_ptr<PointRendererCache> cache_;
 };
 
-// Render the scene into a batch of images; every image is a pyramid of layers: L tensors [B,C,h_l,w_l], then L masks
-// [B,1,h_l,w_l] if output_background_mask.
+// Render the scene into a batch of images; every image is a pyramid of layers: L tensors [B,C,h_l,w_l], then L depth
+// tensors [B,1,h_l,w_l] if add_depth_to_network (all zero in the blend modes: the reference only fills them in its
+// depth-test mode, src/lib/rendering/PointRenderer.cu:1061-1066), then L masks [B,1,h_l,w_l] if output_background_mask.
 std::vector<torch::Tensor> BlendPointCloud(NeuralRenderInfo* info);
 
 // The caller of BlendPointCloud in VET: PointRenderModuleImpl::forward(NeuralRenderInfo*)
@@ -168,7 +189,8 @@ std::vector<torch::Tensor> BlendPointCloud(NeuralRenderInfo* info);
 // callback: it receives layers[l][b] = a clone of the [1,1,h_l,w_l] slice of the cache's weight tensor, as
 // EnvironmentMap::Sample2 does, and returns L tensors [B,C_env,h_l,w_l] that are appended as channels (cat_env_to_color)
 // or added to the images, masked to the pixels whose weight is at most 0.001 when no_envmap_at_points is on (:180-196,
-// literally: the reference zeroes the map where the weight EXCEEDS 0.001). add_depth_to_network is refused.
+// literally: the reference zeroes the map where the weight EXCEEDS 0.001). With add_depth_to_network the (zero) depth
+// tensors are appended to the images as a channel (:223-232).
 class PointRenderModule
 {
    public:
@@ -196,8 +218,10 @@ class PointRenderModule
 //   intrinsics.pth  parameter "intrinsics" [Ncam,13] f32                             (src/lib/data/NeuralStructure.cpp:96)
 // These two functions read and write exactly those entries into / from the tensor bundle the rasterizer takes, so a
 // scene trained by VET renders here and the other way round. Entries of the reference's modules that the rasterizer
-// does not read (normals, original colours, cell tensors, the environment map) are neither written nor required; a
-// missing file leaves the corresponding tensors undefined.
+// does not read are carried along: points.pth also holds the buffers "t_original_color" [N,4] f32 (always; torch::load
+// of the reference's module throws when a registered name is missing, so SaveSceneCheckpoint writes zeros when the bundle
+// has none), "t_normal" and the four "t_cell_*" tensors when the bundle has them. The environment map and the neural
+// camera have files of their own, which are not handled here. A missing file leaves the corresponding tensors undefined.
 SceneTensors LoadSceneCheckpoint(const std::string& prefix, torch::Device device = torch::kCPU);
 void SaveSceneCheckpoint(const std::string& prefix, const SceneTensors& scene);
 
@@ -209,5 +233,16 @@ void SaveSceneCheckpoint(const std::string& prefix, const SceneTensors& scene);
 // tensor; returns the permutation [N] int64 (new index -> old index). The Morton part is deterministic; the block
 // shuffle uses std::mt19937_64(seed) (saiga's generator is not part of the reference tree).
 torch::Tensor MortonBlockShuffleOrder(torch::Tensor positions, int64_t block = 256, uint64_t seed = 0);
+
+// SceneData::SortBlocksByRadius(256) (src/lib/data/SceneData.cpp:108,1005-1018), the step after the block shuffle:
+// inside every complete block of `block` consecutive points the points are sorted by their drop-out radius, ascending, so
+// that with drop_out_points_by_radius the points a layer drops are the leading lanes of every block. radius: [N] float
+// CPU tensor in the order the cloud is in; returns the permutation [N] int64 (new index -> old index). Points of equal
+// radius keep their order here (std::sort in the reference leaves it unspecified).
+torch::Tensor SortBlocksByRadiusOrder(torch::Tensor radius, int64_t block = 256);
+
+// All of src/lib/data/SceneData.cpp:105-108 for a cloud given as [N,4] (x, y, z, drop-out radius): Morton order, block
+// shuffle, blocks sorted by radius; the permutation [N] int64 (new index -> old index).
+torch::Tensor ScenePreprocessOrder(torch::Tensor positions_radius, int64_t block = 256, uint64_t seed = 0);
 
 }  // namespace vet_amd

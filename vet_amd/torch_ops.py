@@ -24,7 +24,9 @@ def blend_point_cloud(texture, background_color, points, pose_tangents, intrinsi
     """BlendPointCloud of the reference (src/lib/rendering/PointRenderer.h:53) on tensors; differentiable.
 
     views: list of (w, h, image_index, camera_index, camera_model, crop fx,fy,cx,cy,s, rot r00,r01,r10,r11).
-    Returns L tensors [B,C,h_l,w_l], then L masks if output_background_mask.
+    Returns L tensors [B,C,h_l,w_l], then L masks if output_background_mask (through the render module, i.e. with
+    super_sampling, cat_masks_to_color, add_depth_to_network or an environment: the images with their extra channels,
+    then the masks).
     environment: a callable standing in for the environment map of PointRenderModuleImpl::forward
     (src/lib/rendering/RenderModule.cpp:129-202): it gets layers[l][b] = the [1,1,h_l,w_l] per-pixel transmittance left
     behind the points and returns L tensors [B,C_env,h_l,w_l]; they are added to the images (masked with
@@ -55,6 +57,24 @@ def morton_block_shuffle_order(positions, block=256, seed=0):
     """The point order of the reference's scene preprocessing (ReorderMorton64 + RandomBlockShuffle(256),
     src/lib/data/SceneData.cpp:105-106) as a permutation [N] int64 of a [N,3] or [N,4] CPU tensor of positions."""
     return load().morton_block_shuffle_order(positions, int(block), int(seed))
+
+
+def sort_blocks_by_radius_order(radius, block=256):
+    """SceneData::SortBlocksByRadius(256) (src/lib/data/SceneData.cpp:108,1005-1018) as a permutation [N] int64: inside
+    every complete block the points sorted by drop-out radius, ascending. radius: [N] CPU tensor."""
+    return load().sort_blocks_by_radius_order(radius, int(block))
+
+
+def scene_preprocess_order(positions_radius, block=256, seed=0):
+    """All three steps of src/lib/data/SceneData.cpp:105-108 (Morton order, block shuffle, blocks sorted by radius) for a
+    [N,4] CPU tensor (x, y, z, drop-out radius), as a permutation [N] int64."""
+    return load().scene_preprocess_order(positions_radius, int(block), int(seed))
+
+
+def train_workspace_info():
+    """(data_ptr, bytes) of the workspace the binding's cache keeps between training steps; (0, 0) before the first."""
+    d = load().train_workspace_info()
+    return int(d["data_ptr"]), int(d["bytes"])
 
 
 def save_scene_checkpoint(prefix, **tensors):
