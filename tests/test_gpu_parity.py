@@ -82,6 +82,22 @@ def test_backward_matches_oracle(name, scene, overrides, rasterizer, oracle):
         assert err <= GRAD_TOL, key
 
 
+@pytest.mark.parametrize("mode", ["full", "fuzzy"])
+def test_position_heuristic_on_a_case_worked_out_by_hand(mode, rasterizer):
+    """The literal expectations of tests/helpers.py::hand_case, no oracle in between
+    (RenderBackward.cu:1346-1377; :729-1080 for FUZZY_BLEND)."""
+    from tests.helpers import check_hand_case, hand_case
+
+    scene, grad_out, expected = hand_case()
+    extra = dict(render_mode=abi.RENDER_FUZZY_BLEND, depth_accept_blend=0.01) if mode == "fuzzy" else {}
+    dev = DeviceScene(scene)
+    res = rasterizer.forward(dev, make_params(scene, need_point_gradient=1, **extra))
+    got = rasterizer.backward(res, [torch.from_numpy(g).cuda() for g in grad_out])
+    torch.cuda.synchronize()
+    check_hand_case(res.out[0].cpu().numpy(), got["points"].cpu().numpy(), got["point_count"].cpu().numpy(),
+                    expected[mode])
+
+
 def _backward_pair(scene, overrides, rasterizer, oracle, want_points=True):
     ref, dev, res, _ = _check_forward(scene, overrides, rasterizer, oracle)
     grad_out = scene.grad_out()

@@ -271,3 +271,24 @@ def test_threaded_oracle_agrees(oracle):
     gb = oracle.backward(b, go, num_threads=4)
     for k in ("texture", "confidence", "points"):
         assert np.allclose(ga[k], gb[k], rtol=1e-4, atol=1e-5 * max(1.0, np.abs(ga[k]).max()))
+
+
+@pytest.mark.parametrize("use_env", [0, 1])
+def test_suffix_sum_model_of_the_backward_pass_agrees_on_short_lists(oracle, use_env):
+    """The O(n) float64 model that the GPU test of long lists is checked against (tests/helpers.py) gives what the
+    oracle's literal O(n^2) loop gives (RenderBackward.cu:2987-3012), early exit, texture index and rim included."""
+    from tests.helpers import bilinear_backward_model, max_rel_err
+
+    scene = _scene(num_points=1500, seed=36, K=-1)
+    scene.confidence[:] = np.clip(scene.confidence * 1.6, 0, 0.98)  # so that the 0.001 cut triggers
+    rng = np.random.default_rng(8)
+    scene.index = rng.integers(0, 400, size=scene.num_points).astype(np.int32)
+    fwd = oracle.forward(scene, use_environment_map=use_env, need_point_gradient=1, **MODE)
+    grad_out = scene.grad_out()
+    got = oracle.backward(fwd, grad_out, want_points=True)
+    want = bilinear_backward_model(oracle, fwd, grad_out, use_env=bool(use_env))
+    full = np.diff(fwd.offsets[0].astype(np.int64))
+    assert (fwd.kept[0] < full).sum() > 20, "the early exit must be exercised"
+    np.testing.assert_array_equal(got["point_count"], want["point_count"])
+    for key in ("texture", "confidence", "points") + (() if use_env else ("background",)):
+        assert max_rel_err(got[key], want[key]) <= 1e-4, key

@@ -396,6 +396,19 @@ def test_position_gradient_chain_and_counts(oracle):
     assert np.all(g["points"][:, 3] == 0)
 
 
+@pytest.mark.parametrize("mode", ["full", "fuzzy"])
+def test_position_heuristic_on_a_case_worked_out_by_hand(mode, oracle):
+    """Literal numbers, not a second copy of the formula: two fragments in the centre pixel of a 7x7 image, their four
+    neighbours with known colours and upstream gradients (RenderBackward.cu:1346-1377; :729-1080 for FUZZY_BLEND)."""
+    from tests.helpers import check_hand_case, hand_case
+
+    scene, grad_out, expected = hand_case()
+    extra = dict(render_mode=abi.RENDER_FUZZY_BLEND, depth_accept_blend=0.01) if mode == "fuzzy" else {}
+    f = oracle.forward(scene, make_params(scene, need_point_gradient=1, **extra))
+    g = oracle.backward(f, grad_out)
+    check_hand_case(f.out[0], g["points"], g["point_count"], expected[mode])
+
+
 def test_point_gradient_normalization_modes(oracle):
     scene = synthetic.tiny_scene(num_points=900, K=4, seed=18)
     f = oracle.forward(scene, need_point_gradient=1)
