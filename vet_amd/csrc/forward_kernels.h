@@ -257,9 +257,9 @@ struct PackJob
 // cursor in a cache line of its own: appends to one cursor would queue up behind each other where many bins overflow
 // (a workgroup's segment has room for every hit the workgroups of that residue can produce). Bins are sized for an expected 1024 records at most, so the log stays empty or
 // short unless the cloud is far denser somewhere than on average.
-// A record is 16 bytes (key low, key high, pixel in bin, 0), or, where a point lands in one pixel per layer and point ids
-// fit 24 bits (`compact`), 8 bytes: (key high = depth bits, point id << 8 | pixel in bin). Half the bytes written here
-// and read again by the build pass.
+// A record is 16 bytes (key low, key high, pixel in bin, 0), or, where the low key word (point id; point id << 2 |
+// corner for the 2x2 splat) fits 24 bits (`compact`), 8 bytes: (key high = depth bits, key low << 8 | pixel in bin).
+// Half the bytes written here and read again by the build pass.
 struct ScatterTargets
 {
     uint4* primary;        // [bins][kPrimaryCap] records (uint2 records when compact)

@@ -148,10 +148,11 @@ inline int hits_of_mode(int render_mode)
     return render_mode == VETRAST_RENDER_BILINEAR_BLEND ? 4 : 1;
 }
 
-// Fragment records of 8 instead of 16 bytes: one hit per point and layer, point ids of 24 bits.
+// Fragment records of 8 instead of 16 bytes: the low key word (point id, or point id << 2 | corner of the 2x2 splat)
+// fits 24 bits.
 inline bool compact_records(int64_t N, int hits)
 {
-    return hits == 1 && N <= (int64_t)(1 << 24);
+    return N * hits <= (int64_t)(1 << 24);
 }
 
 inline int check_mode(int render_mode)

@@ -297,12 +297,11 @@ def config4(surface_points_n=4_000_000, sphere_points=500_000, seed=3, w=1920, h
         d /= np.maximum(np.linalg.norm(d, axis=1, keepdims=True), 1e-12)
         shells.append(r * d)
     xyz = np.concatenate([surf] + shells, axis=0)
-    if point_order == "vet_preprocess":
-        xyz = xyz[vet_preprocess_order(xyz, seed)]
     N = xyz.shape[0]
+    xyz, radius = ordered_cloud(xyz, point_radii(seed, N, 0.0), seed, point_order)
     pos = np.empty((N, 4), dtype=np.float32)
     pos[:, :3] = xyz.astype(np.float32)
-    pos[:, 3] = 0.01
+    pos[:, 3] = radius
     tex, conf, bg = _descriptors(seed, N)
     scale = w / 1920.0
     views = [ViewSpec(w, h, image_index=b) for b in range(num_views)]
@@ -319,10 +318,9 @@ def config5(num_points=10_000_000, seed=4, w=1920, h=1080, num_layers=4, K=16, p
     pos = np.empty((N, 4), dtype=np.float32)
     xyz = Stream(seed, "position").uniform(3 * N).reshape(N, 3) - 0.5
     xyz[:, 2] += 1.2
-    if point_order == "vet_preprocess":
-        xyz = xyz[vet_preprocess_order(xyz, seed)]
+    xyz, radius = ordered_cloud(xyz, point_radii(seed, N, 0.0), seed, point_order)
     pos[:, :3] = xyz.astype(np.float32)
-    pos[:, 3] = 0.01
+    pos[:, 3] = radius
     tex, conf, bg = _descriptors(seed, N)
     scale = w / 1920.0
     s = Scene("config5_depth_stress", pos, tex, conf, bg, _identity_pose((0, 0, 0)),
