@@ -124,7 +124,10 @@ def timed_samples(fn, warmup, steps, samples):
             "samples": [round(x, 5) for x in ms], "wall": wall}
 
 
-def run_scene(scene, backward, steps, warmup, samples, profile=True, render_mode=1, graph=False, **param_overrides):
+def run_scene(scene, backward, steps, warmup, samples, profile=True, render_mode=1, graph=False, processing_order=False,
+              **param_overrides):
+    """processing_order: hand the library a Morton order built on the device (vetrast_forward_args.point_order), as
+    the shim does for every cloud; its build time is reported, not part of the step."""
     import torch
 
     from vet_amd import abi
@@ -137,7 +140,14 @@ def run_scene(scene, backward, steps, warmup, samples, profile=True, render_mode
     lay = rast.layout(scene, render_mode)
     workspace = torch.empty(lay.total_bytes, dtype=torch.uint8, device="cuda")
     out = [torch.empty((B, Cn, h, w), dtype=torch.float32, device="cuda") for (w, h) in scene.layer_sizes()]
-    fwd = rast.forward(dev, params, save_for_backward=backward, workspace=workspace, out=out)
+    order, order_ms = None, None
+    if processing_order:
+        from vet_amd import torch_ops
+
+        d_pos = torch.from_numpy(scene.position).cuda()
+        order_ms = timed_samples(lambda: torch_ops.processing_order_on_device(d_pos), 2, 5, 3)["median"]
+        order = torch_ops.processing_order_on_device(d_pos)
+    fwd = rast.forward(dev, params, save_for_backward=backward, workspace=workspace, out=out, point_order=order)
     torch.cuda.synchronize()
     P = fwd.total_pixels()
     K = params.debug_max_list_length
@@ -170,7 +180,7 @@ def run_scene(scene, backward, steps, warmup, samples, profile=True, render_mode
     t_step = timed_samples(step, warmup, steps, samples)
     t_fwd = timed_samples(forward_only, 2, steps, samples) if backward else t_step
     res = {"step": t_step, "fwd": t_fwd, "ms_step": t_step["median"], "ms_fwd": t_fwd["median"],
-           "workspace_bytes": int(lay.total_bytes)}
+           "workspace_bytes": int(lay.total_bytes), "order_build_ms": order_ms}
     res.update(N=N, P=P, F=F, Fk=Fk, F_layers=F_layers, K=K, Cn=Cn, L=L, B=B, params=params)
     if graph:
         # the same step replayed from a HIP graph: no launch calls from the host between the kernels
@@ -495,10 +505,20 @@ def main():
         for order in ("vet_preprocess", "grown", "generated"):
             if order == args.point_order:
                 continue
-            r2 = run_scene(make(**dict(kw, point_order=order)), backward, **short)
+            sc2 = make(**dict(kw, point_order=order))
+            r2 = run_scene(sc2, backward, **short)
+            r2o = run_scene(sc2, backward, processing_order=True, **short)
             others.append({"point_order": order, "ms_per_step": round(r2["ms_step"], 5),
-                           "forward_ms": round(r2["ms_fwd"], 5)})
+                           "forward_ms": round(r2["ms_fwd"], 5),
+                           "with_processing_order": {"ms_per_step": round(r2o["ms_step"], 5),
+                                                     "forward_ms": round(r2o["ms_fwd"], 5)}})
         result["other_point_orders"] = others
+        r1o = run_scene(scene, backward, processing_order=True, **short)
+        result["processing_order"] = {
+            "what": "vetrast_forward_args.point_order = Morton order with shuffled 256-point blocks, built on the "
+                    "device by the shim (ProcessingOrderOnDevice) once per 1000 forward calls; results are the same bits",
+            "build_ms": round(r1o["order_build_ms"], 4),
+            "headline_order_ms_per_step": round(r1o["ms_step"], 5), "headline_order_forward_ms": round(r1o["ms_fwd"], 5)}
         if args.config in (2, 3):
             # log-normal radii, blocks sorted by radius as SortBlocksByRadius(256) leaves them, radius drop-out on
             sc = make(**dict(kw, radius_spread=0.5))

@@ -212,6 +212,14 @@ typedef struct vetrast_forward_args
      * (src/lib/rendering/RenderForward.cu:1355-1356), which PointRenderModuleImpl::forward hands to the environment map
      * (src/lib/rendering/RenderModule.cpp:132-196). NULL = not wanted. */
     float* out_weight[VETRAST_MAX_LAYERS];
+    /* Optional, device [N]: a permutation of 0..N-1, the order in which the binning pass walks the points (thread i
+     * takes point point_order[i]). Results do not depend on it, bit for bit; the time of the binning pass does: it
+     * groups the points of a wave by bin before it touches global counters, so it wants neighbours in the array to be
+     * neighbours in space. A cloud in the order of VET's preprocessing (src/lib/data/SceneData.cpp:105-108) needs none;
+     * one that has grown since (NeuralScene::AddNewPoints appends, src/lib/data/NeuralScene.cpp:1013) or comes in
+     * file order does. Point ids everywhere else (index, gradients, dropout) stay the caller's. NULL = array order.
+     * No counterpart in the reference. */
+    const int32_t* point_order;
 } vetrast_forward_args;
 
 /* Arguments of the backward pass. Replaces BlendPointCloudBackward's inputs and its seven returned tensors

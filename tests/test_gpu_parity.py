@@ -98,6 +98,32 @@ def test_position_heuristic_on_a_case_worked_out_by_hand(mode, rasterizer):
                     expected[mode])
 
 
+@pytest.mark.parametrize("mode", [abi.RENDER_FULL_BLEND, abi.RENDER_FUZZY_BLEND, abi.RENDER_BILINEAR_BLEND])
+def test_processing_order_changes_nothing(mode, rasterizer):
+    """vetrast_forward_args.point_order only tells the binning pass in which order to walk the points: lists, outputs
+    and gradients are the same bits for any permutation (several views, radius drop-out on; no texture index, whose
+    shared rows are summed with float atomics in arrival order)."""
+    scene = synthetic.tiny_scene(num_points=7000, K=8, seed=41, num_views=2)
+    rng = np.random.default_rng(11)
+    params = make_params(scene, need_point_gradient=1, render_mode=mode, drop_out_points_by_radius=1)
+    dev = DeviceScene(scene)
+    grad_out = [torch.from_numpy(g).cuda() for g in scene.grad_out()]
+    plain = rasterizer.forward(dev, params)
+    plain_g = {k: v.clone() for k, v in rasterizer.backward(plain, grad_out).items() if k != "_args"}
+    for perm in (rng.permutation(scene.num_points), np.arange(scene.num_points)[::-1].copy()):
+        order = torch.from_numpy(perm.astype(np.int32)).cuda()
+        res = rasterizer.forward(dev, params, point_order=order)
+        got = rasterizer.backward(res, grad_out)
+        torch.cuda.synchronize()
+        for b in range(2):
+            np.testing.assert_array_equal(res.offsets(b), plain.offsets(b))
+            np.testing.assert_array_equal(res.kept(b), plain.kept(b))
+        for a, b in zip(res.out, plain.out):
+            assert torch.equal(a, b)
+        for k, v in plain_g.items():
+            assert torch.equal(got[k], v), k
+
+
 def _backward_pair(scene, overrides, rasterizer, oracle, want_points=True):
     ref, dev, res, _ = _check_forward(scene, overrides, rasterizer, oracle)
     grad_out = scene.grad_out()

@@ -358,3 +358,50 @@ def test_training_steps_share_one_workspace():
     texture.grad = None
     sum(o.sum() for o in b).backward()
     np.testing.assert_array_equal(texture.grad.cpu().numpy() * 3, first_grad.cpu().numpy())
+
+
+def test_the_cache_keeps_a_processing_order_and_results_do_not_depend_on_it():
+    """The shim builds a Morton order on the device for the binning pass, rebuilds it when the number of points changes
+    and after `refresh` forward calls, and can be told not to; outputs and gradients are the same bits either way."""
+    from vet_amd import torch_ops
+
+    scene = synthetic.config2(num_points=30_000, w=320, h=180, point_order="grown")
+    cu = lambda a, rg=False: torch.from_numpy(np.ascontiguousarray(a)).cuda().requires_grad_(rg)
+    grads = [torch.from_numpy(g).cuda() for g in scene.grad_out()]
+
+    def run():
+        texture, confidence = cu(scene.texture, True), cu(scene.confidence.reshape(1, -1), True)
+        points = cu(scene.position, True)
+        B = scene.poses_se3.shape[0]
+        outs = torch_ops.blend_point_cloud(texture, cu(scene.background), points,
+                                           torch.zeros((B, 6), dtype=torch.float64, device="cuda"), cu(scene.intrinsics),
+                                           confidence, cu(scene.poses_se3), None, _views(scene), scene.num_layers,
+                                           train=True, use_environment_map=0, need_point_gradient=1,
+                                           drop_out_points_by_radius=0, debug_max_list_length=scene.max_list_length)
+        torch.autograd.backward(outs, grads)
+        return [o.detach().clone() for o in outs], [texture.grad, confidence.grad, points.grad]
+
+    try:
+        torch_ops.set_point_order_refresh(0)
+        plain_out, plain_grad = run()
+        assert torch_ops.point_order() is None
+        torch_ops.set_point_order_refresh(3)
+        out1, grad1 = run()
+        first = torch_ops.point_order()
+        assert first is not None and first.dtype == torch.int32 and first.numel() == scene.num_points
+        assert torch.equal(torch.sort(first.long()).values, torch.arange(scene.num_points, device="cuda"))
+        ptr = first.data_ptr()
+        run()
+        run()
+        assert torch_ops.point_order().data_ptr() == ptr, "kept for `refresh` calls"
+        run()
+        assert torch.equal(torch_ops.point_order(), first), "rebuilt from the same positions: the same order"
+        for a, b in zip(plain_out + plain_grad, out1 + grad1):
+            assert torch.equal(a, b)
+        # fewer points: a new order of the new length
+        scene.position, scene.texture, scene.confidence = scene.position[:20_000], scene.texture[:, :20_000].copy(), \
+            scene.confidence[:20_000]
+        run()
+        assert torch_ops.point_order().numel() == 20_000
+    finally:
+        torch_ops.set_point_order_refresh(1000)

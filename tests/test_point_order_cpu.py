@@ -110,3 +110,30 @@ def test_grown_cloud_order():
     b = np.sort(ordered.position.view([("", np.float32)] * 4).ravel())
     assert np.array_equal(a, b)
     assert not np.array_equal(s.position, ordered.position)
+
+
+def test_processing_order_on_device_is_a_permutation_with_compact_blocks():
+    """The order the shim builds for the binning pass (tensor operations, here on the CPU device): every point once,
+    and a 256-point block is a run of the Morton curve, i.e. small in space (random blocks span the scene)."""
+    import torch
+
+    from vet_amd import torch_ops
+
+    scene = synthetic.config2(num_points=60_000, point_order="generated")
+    xyz = scene.position[:, :3]
+    order = torch_ops.processing_order_on_device(torch.from_numpy(scene.position), 256, 3)
+    assert order.dtype == torch.int32 and tuple(order.shape) == (scene.num_points,)
+    o = order.numpy().astype(np.int64)
+    np.testing.assert_array_equal(np.sort(o), np.arange(scene.num_points))
+
+    def mean_block_diagonal(perm):
+        n = len(perm) // 256 * 256
+        b = xyz[perm[:n]].reshape(-1, 256, 3)
+        return float(np.linalg.norm(b.max(axis=1) - b.min(axis=1), axis=1).mean())
+
+    assert mean_block_diagonal(o) * 3 < mean_block_diagonal(np.random.default_rng(0).permutation(scene.num_points))
+    # deterministic for a seed, another seed shuffles the blocks differently
+    again = torch_ops.processing_order_on_device(torch.from_numpy(scene.position), 256, 3)
+    other = torch_ops.processing_order_on_device(torch.from_numpy(scene.position), 256, 4)
+    assert torch.equal(order, again) and not torch.equal(order, other)
+    assert torch_ops.processing_order_on_device(torch.zeros((0, 4))).numel() == 0

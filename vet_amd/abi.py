@@ -152,6 +152,7 @@ class ForwardArgs(C.Structure):
         ("workspace", C.c_void_p),
         ("workspace_bytes", C.c_size_t),
         ("out_weight", C.c_void_p * MAX_LAYERS),
+        ("point_order", C.c_void_p),
     ]
 
 

@@ -125,6 +125,7 @@ struct ViewPass
     int confidence_activation;  // 1: `confidence` holds raw values, the confidence is sigmoid(confidence_scale * raw)
     float confidence_scale;
     float2* projected;  // BILINEAR_BLEND: [N] image position of every visible point at layer 0, written by the scatter pass
+    const int32_t* point_order;  // [N] or null: the scatter pass's thread i takes point point_order[i]
 };
 
 struct Projected

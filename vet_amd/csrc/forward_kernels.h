@@ -312,21 +312,24 @@ template <int HITS>
 __global__ void __launch_bounds__(kBlock) bin_scatter_kernel(ViewPass a, uint32_t* __restrict__ bin_counts,
                                                               ScatterTargets out, PackJob pack)
 {
-    const int i    = blockIdx.x * blockDim.x + threadIdx.x;
+    const int slot = blockIdx.x * blockDim.x + threadIdx.x;
     const int lane = threadIdx.x & (kWave - 1);
-    // side job: texture row i, asked for first and stored last
-    const bool packs = pack.packed != nullptr && i < pack.N;
+    // the point this thread takes: the caller's processing order, if there is one (neighbours in a wave should be
+    // neighbours in space; ids in the records are the caller's either way)
+    const int i = (a.point_order != nullptr && slot < a.N) ? a.point_order[slot] : slot;
+    // side job: texture row `slot`, asked for first and stored last
+    const bool packs = pack.packed != nullptr && slot < pack.N;
     float row[4] = {0.f, 0.f, 0.f, 0.f}, row_confidence = 0.f;
     if (packs)
     {
 #pragma unroll
         for (int ci = 0; ci < VETRAST_MAX_CHANNELS; ++ci)
-            if (ci < pack.C) row[ci] = pack.texture[(size_t)ci * pack.N + i];
-        row_confidence = pack.confidence[i];
+            if (ci < pack.C) row[ci] = pack.texture[(size_t)ci * pack.N + slot];
+        row_confidence = pack.confidence[slot];
     }
     Projected p;
     p.ipx = p.ipy = p.z = p.radius = 0.f;
-    const bool visible = i < a.N && !point_is_skipped(a, i) && project_point(*a.view, a.position[i], p);
+    const bool visible = (uint32_t)i < (uint32_t)a.N && !point_is_skipped(a, i) && project_point(*a.view, a.position[i], p);
     float ipx = visible ? p.ipx : 0.f, ipy = visible ? p.ipy : 0.f, radius = visible ? p.radius : 0.f;
     const uint32_t depth_bits = __float_as_uint(p.z);
     bool dropped = !visible;  // from the layer on at which the splat radius falls under the threshold
@@ -452,8 +455,8 @@ __global__ void __launch_bounds__(kBlock) bin_scatter_kernel(ViewPass a, uint32_
             for (int ci = 0; ci < VETRAST_MAX_CHANNELS; ++ci) row[ci] = fabsf(row[ci]);
         }
         if (pack.confidence_activation) row_confidence = sigmoid_canon(pack.confidence_scale * row_confidence);
-        pack.packed[2 * (size_t)i]     = make_float4(row[0], row[1], row[2], row[3]);
-        pack.packed[2 * (size_t)i + 1] = make_float4(row_confidence, 0.f, 0.f, 0.f);
+        pack.packed[2 * (size_t)slot]     = make_float4(row[0], row[1], row[2], row[3]);
+        pack.packed[2 * (size_t)slot + 1] = make_float4(row_confidence, 0.f, 0.f, 0.f);
     }
 }
 

@@ -279,6 +279,7 @@ ViewPass make_view_pass(const vetrast_forward_args* a, const vetrast_workspace_l
     vp.stability_cutoff = a->params.stability_cutoff_value;
     vp.confidence_activation = a->params.confidence_activation;
     vp.confidence_scale      = a->params.confidence_scale;
+    vp.point_order = a->point_order;
     vp.projected = lay.projected_stride ? ws_ptr<float2>(a->workspace, lay.projected_base + lay.projected_stride * b) : nullptr;
     return vp;
 }

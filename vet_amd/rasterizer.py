@@ -225,7 +225,8 @@ class Rasterizer:
         return lay
 
     def forward(self, dev: DeviceScene, params: abi.Params = None, save_for_backward=True, workspace=None,
-                out=None, want_weight=False) -> ForwardResult:
+                out=None, want_weight=False, point_order=None) -> ForwardResult:
+        """point_order: optional int32 device tensor [N], a permutation: the order the binning pass walks the points in."""
         scene = dev.scene
         params = params or make_params(scene)
         lay = self.layout(scene, params.render_mode)
@@ -252,8 +253,11 @@ class Rasterizer:
                 args.out_weight[l] = weights[l].data_ptr()
         args.workspace = workspace.data_ptr()
         args.workspace_bytes = workspace.numel()
+        if point_order is not None:
+            assert point_order.dtype == torch.int32 and point_order.is_cuda and point_order.numel() == scene.num_points
+            args.point_order = point_order.data_ptr()
         abi.check(self.lib.vetrast_forward(self.ctx, C.byref(args), self._stream()), "forward")
-        return ForwardResult(out, masks, workspace, lay, args, (views, dev, params), weights)
+        return ForwardResult(out, masks, workspace, lay, args, (views, dev, params, point_order), weights)
 
     def backward(self, fwd: ForwardResult, grad_out: List[torch.Tensor], want_points=True, want_cameras=False,
                  **param_overrides):

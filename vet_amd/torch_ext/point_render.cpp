@@ -275,6 +275,8 @@ torch::autograd::variable_list PointRender::forward(torch::autograd::AutogradCon
     a.workspace         = workspace.data_ptr();
     a.workspace_bytes   = (size_t)workspace.numel();
     a.save_for_backward = need_backward ? 1 : 0;
+    const torch::Tensor& order = info->cache->PointOrderFor(points);
+    a.point_order              = order.defined() ? order.data_ptr<int32_t>() : nullptr;
     check_status(vetrast_forward(info->cache->ctx, &a, current_stream()), "forward");
 
     if (need_backward)
@@ -667,6 +669,62 @@ torch::Tensor MortonBlockShuffleOrder(torch::Tensor positions, int64_t block, ui
     return out;
 }
 
+torch::Tensor ProcessingOrderOnDevice(const torch::Tensor& positions, int64_t block, uint64_t seed)
+{
+    TORCH_CHECK(positions.dim() == 2 && positions.size(1) >= 3 && block >= 1,
+                "ProcessingOrderOnDevice: positions is a [N,3] or [N,4] tensor, block >= 1");
+    torch::NoGradGuard no_grad;
+    const int64_t n = positions.size(0);
+    auto i32        = torch::TensorOptions().device(positions.device()).dtype(torch::kInt32);
+    if (n == 0) return torch::empty({0}, i32);
+    const torch::Tensor p   = positions.detach().slice(1, 0, 3).to(torch::kFloat32);
+    const torch::Tensor lo  = std::get<0>(p.min(0)), hi = std::get<0>(p.max(0));
+    const torch::Tensor ext = (hi - lo).clamp_min(1e-30);
+    const torch::Tensor q   = ((p - lo) / ext * (float)((1 << 21) - 1)).floor().to(torch::kInt64);  // [N,3], 21 bits each
+    auto spread = [](torch::Tensor x) {  // bit k of x to bit 3 k
+        x = x.bitwise_or(x.bitwise_left_shift(32)).bitwise_and((int64_t)0x1f00000000ffffLL);
+        x = x.bitwise_or(x.bitwise_left_shift(16)).bitwise_and((int64_t)0x1f0000ff0000ffLL);
+        x = x.bitwise_or(x.bitwise_left_shift(8)).bitwise_and((int64_t)0x100f00f00f00f00fLL);
+        x = x.bitwise_or(x.bitwise_left_shift(4)).bitwise_and((int64_t)0x10c30c30c30c30c3LL);
+        x = x.bitwise_or(x.bitwise_left_shift(2)).bitwise_and((int64_t)0x1249249249249249LL);
+        return x;
+    };
+    const torch::Tensor code = spread(q.select(1, 0))
+                                   .bitwise_or(spread(q.select(1, 1)).bitwise_left_shift(1))
+                                   .bitwise_or(spread(q.select(1, 2)).bitwise_left_shift(2));
+    torch::Tensor order = code.argsort();
+    // whole blocks change places; what is left over behind the last whole block stays last, so that every block (a
+    // workgroup of the binning pass) remains one run of the curve
+    const int64_t blocks = n / block;
+    if (blocks > 1)
+    {
+        auto i64                  = torch::TensorOptions().device(positions.device()).dtype(torch::kInt64);
+        auto gen                  = at::detail::createCPUGenerator(seed);
+        const torch::Tensor perm  = torch::randperm(blocks, gen, torch::TensorOptions().dtype(torch::kInt64)).to(positions.device());
+        const torch::Tensor at    = (perm.unsqueeze(1) * block + torch::arange(block, i64).unsqueeze(0)).reshape({-1});
+        order                     = torch::cat({order.index_select(0, at), order.slice(0, blocks * block, n)});
+    }
+    return order.to(torch::kInt32);
+}
+
+const torch::Tensor& PointRendererCache::PointOrderFor(const torch::Tensor& points)
+{
+    if (point_order_refresh <= 0)
+    {
+        point_order = torch::Tensor();
+        return point_order;
+    }
+    const bool stale = !point_order.defined() || point_order.size(0) != points.size(0) ||
+                       point_order.device() != points.device() || point_order_age_ >= point_order_refresh;
+    if (stale)
+    {
+        point_order      = ProcessingOrderOnDevice(points, 256, 0);
+        point_order_age_ = 0;
+    }
+    ++point_order_age_;
+    return point_order;
+}
+
 torch::Tensor SortBlocksByRadiusOrder(torch::Tensor radius, int64_t block)
 {
     TORCH_CHECK(radius.dim() == 1 && !radius.is_cuda() && block >= 1, "SortBlocksByRadiusOrder: radius is a [N] CPU tensor");
@@ -942,6 +1000,21 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
     m.def("scene_preprocess_order", &vet_amd::ScenePreprocessOrder, pybind11::arg("positions_radius"),
           pybind11::arg("block") = 256, pybind11::arg("seed") = 0,
           "ReorderMorton64 + RandomBlockShuffle + SortBlocksByRadius of the reference's scene preprocessing, as a permutation");
+    m.def("processing_order_on_device", &vet_amd::ProcessingOrderOnDevice, pybind11::arg("positions"),
+          pybind11::arg("block") = 256, pybind11::arg("seed") = 0,
+          "Morton order with shuffled blocks, computed on the positions' device: int32 permutation for point_order");
+    m.def(
+        "set_point_order_refresh",
+        [](int64_t every) {
+            if (!g_cache) g_cache = std::make_shared<vet_amd::PointRendererCache>();
+            g_cache->point_order_refresh = every;
+            g_cache->point_order         = torch::Tensor();
+        },
+        "forward calls between rebuilds of the cache's processing order; 0 switches it off");
+    m.def(
+        "point_order",
+        []() { return (g_cache && g_cache->point_order.defined()) ? g_cache->point_order : torch::Tensor(); },
+        "the processing order the cache currently holds (undefined tensor: none)");
     m.def(
         "train_workspace_info",
         []() {

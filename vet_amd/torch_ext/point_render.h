@@ -102,6 +102,15 @@ class PointRendererCache
     // coefficients sit in device memory, so checking them costs a blocking read: it is only repeated when the intrinsics
     // tensor or its version counter changes. Throws if columns 5..12 of `intrinsics` [num_cameras,13] are not all zero.
     void CheckIntrinsics(const torch::Tensor& intrinsics);
+    // The order in which the binning pass walks the points (vetrast_forward_args.point_order): Morton order with shuffled
+    // 256-point blocks, built on the device from the positions, rebuilt when the number of points changes and every
+    // `point_order_refresh` forward calls (positions drift while they are optimised; the order only has to be roughly
+    // right). Results do not depend on it; a cloud that has grown since it was preprocessed (NeuralScene::AddNewPoints
+    // appends, src/lib/data/NeuralScene.cpp:1013) or that comes in file order renders up to twice as fast in the
+    // binning pass with it, one in VET's order loses nothing. 0: never build one, walk the array as it is.
+    int64_t point_order_refresh = 1000;
+    torch::Tensor point_order;  // int32 [N] on the points' device, or undefined
+    const torch::Tensor& PointOrderFor(const torch::Tensor& points);
     // layers_cuda[l].weight of the reference's cache (src/lib/rendering/PointRenderer.h:131, written at
     // src/lib/rendering/RenderForward.cu:1355-1356): per layer [B,1,h_l,w_l], the transmittance left behind the last
     // blended fragment of every pixel. Only kept up to date by BlendPointCloud while keep_layer_weights is set.
@@ -120,6 +129,7 @@ class PointRendererCache
    private:
     const void* checked_intrinsics_ptr_ = nullptr;
     int64_t checked_intrinsics_version_ = -1, checked_intrinsics_numel_ = -1;
+    int64_t point_order_age_ = 0;
 };
 
 class NeuralRenderInfo : public torch::CustomClassHolder
@@ -239,6 +249,9 @@ torch::Tensor MortonBlockShuffleOrder(torch::Tensor positions, int64_t block = 2
 // that with drop_out_points_by_radius the points a layer drops are the leading lanes of every block. radius: [N] float
 // CPU tensor in the order the cloud is in; returns the permutation [N] int64 (new index -> old index). Points of equal
 // radius keep their order here (std::sort in the reference leaves it unspecified).
+// The same kind of order (Morton code over the bounding box, then whole blocks shuffled) computed with tensor operations
+// on the device the positions are on, without a host round trip: int32 [N]. For vetrast_forward_args.point_order.
+torch::Tensor ProcessingOrderOnDevice(const torch::Tensor& positions, int64_t block = 256, uint64_t seed = 0);
 torch::Tensor SortBlocksByRadiusOrder(torch::Tensor radius, int64_t block = 256);
 
 // All of src/lib/data/SceneData.cpp:105-108 for a cloud given as [N,4] (x, y, z, drop-out radius): Morton order, block

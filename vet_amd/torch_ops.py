@@ -71,6 +71,22 @@ def scene_preprocess_order(positions_radius, block=256, seed=0):
     return load().scene_preprocess_order(positions_radius, int(block), int(seed))
 
 
+def processing_order_on_device(positions, block=256, seed=0):
+    """Morton order with shuffled blocks computed on the device of `positions`: int32 [N], for point_order."""
+    return load().processing_order_on_device(positions, block, seed)
+
+
+def set_point_order_refresh(every):
+    """Forward calls between rebuilds of the processing order the shim's cache keeps; 0 switches it off."""
+    load().set_point_order_refresh(int(every))
+
+
+def point_order():
+    """The processing order the shim's cache currently holds, or None."""
+    t = load().point_order()
+    return t if t is not None and t.numel() > 0 else None
+
+
 def train_workspace_info():
     """(data_ptr, bytes) of the workspace the binding's cache keeps between training steps; (0, 0) before the first."""
     d = load().train_workspace_info()
