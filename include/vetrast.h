@@ -170,10 +170,13 @@ typedef struct vetrast_workspace_layout
     size_t partial_base;   /* float [L][N][8]: backward scratch, gradient record of the fragment of point i in layer l */
     size_t background_partial_base; /* float [workgroups][8]: backward scratch, per-workgroup background-gradient sums */
     size_t camera_partial_base;     /* double [ceil(N/256)][12]: backward scratch, per-workgroup pose / intrinsics sums */
-    /* scratch shared by all views: the scatter pass writes the records of bin b to primary[b][rank] while rank < 2048;
+    /* scratch shared by all views: the scatter pass writes the records of a bin to the bin's own room while their rank
+     * is below the room's size (2048 records where about a thousand are expected per bin, 1024 where at most 512 are);
      * records beyond that go to a log of 256 segments (record + bin, rank in the slots array) and are filed into the
-     * compact array after the scan. log_cursor: per view, 256 uint32 64 bytes apart, entries in every segment. */
-    size_t primary_base;   /* uint32 [num_bins][2048][4], or [num_bins][2048][2] with the 8-byte records */
+     * compact array after the scan. log_cursor: per view, 256 uint32 64 bytes apart, entries in every segment.
+     * The log and the slots array only live inside a forward call: partial_base == log_base, the scratch of the
+     * backward call lies on top of them (forward_only_bytes covers the log, total_bytes both). */
+    size_t primary_base;   /* the rooms, layer after layer, bin after bin: 16-byte records, or 8-byte ones (see binned_base) */
     size_t log_base;       /* uint32 [256][ceil(ceil(N/256)/256)*256*L*hits][4] */
     size_t log_cursor_base;
     size_t last_key_base, last_key_stride;   /* per view, uint64 [P]: where cut_flags is 1, the key of the last fragment of

@@ -106,15 +106,26 @@ def test_workspace_layout_is_aligned_and_disjoint():
         ("transmittance", lay.transmittance_base, lay.transmittance_stride * B),
         ("weight", lay.weight_base, lay.weight_stride * B),
         ("packed", lay.packed_base, N * 32),
-        ("slots", lay.slots_base, log_records * 4),
-        ("log", lay.log_base, log_records * 16),
         ("log_cursor", lay.log_cursor_base, B * 256 * 64),
-        ("primary", lay.primary_base, lay.num_bins * 2048 * 8),
+        # rooms of 1024 records where at most 512 are expected per bin (layer 0: 2 M points over 8100 tiles), 2048 elsewhere
+        ("primary", lay.primary_base, (tiles[0] * 1024 + (tiles[1] + 4 * tiles[2] + 16 * tiles[3]) * 2048) * 8),
         ("views", lay.views_base, B * 128),
-        ("partial", lay.partial_base, N * L * 32),
-        ("background_partial", lay.background_partial_base, (P + 255) // 256 * 32),
-        ("camera_partial", lay.camera_partial_base, (N + 255) // 256 * 96),
     ]
+    # the scratch of the backward call lies on top of the overflow log, which only lives inside a forward call
+    forward_tail = [("log", lay.log_base, log_records * 16), ("slots", lay.slots_base, log_records * 4)]
+    backward_tail = [("partial", lay.partial_base, N * L * 32),
+                     ("background_partial", lay.background_partial_base, (P + 255) // 256 * 32),
+                     ("camera_partial", lay.camera_partial_base, (N + 255) // 256 * 96)]
+    head_end = max(b + sz for _, b, sz in regions)
+    for tail in (forward_tail, backward_tail):
+        assert min(b for _, b, _ in tail) >= head_end
+        srt = sorted(tail, key=lambda r: r[1])
+        for (n0, b0, s0), (n1, b1, _) in zip(srt, srt[1:]):
+            assert b0 + s0 <= b1, (n0, n1)
+        for name, base, size in tail:
+            assert base % 256 == 0 and base + size <= lay.total_bytes, name
+    assert lay.log_base == lay.partial_base
+    assert max(b + sz for _, b, sz in forward_tail) <= lay.forward_only_bytes
     assert lay.offsets_stride >= (P + 1) * 4 and lay.fragments_stride >= N * L * 8
     # 2 M points over 1080p: tiles at the two fine layers, 16x4 strips and single tile rows at the coarse ones
     assert lay.num_bins == tiles[0] + tiles[1] + 4 * tiles[2] + 16 * tiles[3]
@@ -125,7 +136,8 @@ def test_workspace_layout_is_aligned_and_disjoint():
     ordered = sorted(regions, key=lambda r: r[1])
     for (n0, b0, s0), (n1, b1, _) in zip(ordered, ordered[1:]):
         assert b0 + s0 <= b1, (n0, n1)
-    assert lay.forward_only_bytes <= lay.partial_base < lay.total_bytes
+    assert lay.partial_base < lay.forward_only_bytes <= lay.total_bytes
+    assert lay.total_bytes < 0.8e9 * B  # the diet: under 0.8 GB per view at 2 M points / 1080p / 4 layers
     # the log cursors sit right behind the bin counters (one zero-fill covers both); BILINEAR_BLEND adds `projected`
     assert lay.log_cursor_base == lay.bin_counts_base + lay.bin_counts_stride * B
     assert lay.projected_stride == 0

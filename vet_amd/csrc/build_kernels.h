@@ -26,14 +26,14 @@ namespace vetrast
 // on the 10 M point cloud.
 constexpr int kBuildPerThread = 4;
 constexpr int kBuildCap       = kBlock * kBuildPerThread;  // 1024 records = 8 KB of keys in LDS
-static_assert(kPrimaryCap >= kBuildCap, "a bin built in LDS must find all its records in its own room");
+static_assert(kPrimaryCapSmall >= kBuildCap, "a bin built in LDS must find all its records in its own room");
 constexpr int kStage          = 256;                       // descriptor records staged per round (8 KB)
 
 struct BuildPass
 {
     const uint32_t* bin_offsets;  // [bins + 1] exclusive scan of the bin counts
-    const uint4* primary;         // [bins][kPrimaryCap] fragment records, the first kPrimaryCap of every bin
-    const uint4* binned;          // compact array: record r >= kPrimaryCap of a bin sits at bin_offsets[bin] + r
+    const uint4* primary;         // the bins' rooms (LayerTable::room_base): the first room_cap[l] records of every bin
+    const uint4* binned;          // compact array: record r >= room_cap[l] of a bin sits at bin_offsets[bin] + r
     int compact_records;          // both hold 8-byte records (depth bits, point id << 8 | pixel in bin), see ScatterTargets
     uint32_t* offsets;    // [P + 1] per pixel: start of its list; [P] = fragments of the view
     uint64_t* fragments;
@@ -208,16 +208,18 @@ __global__ void __launch_bounds__(kBlock) bin_build_kernel(BuildPass a)
     // the same for every lane: tell the compiler, so that loops over the bin's records become scalar branches
     const uint32_t begin  = (uint32_t)__builtin_amdgcn_readfirstlane((int)a.bin_offsets[bin]);
     const uint32_t n      = (uint32_t)__builtin_amdgcn_readfirstlane((int)a.bin_offsets[bin + 1]) - begin;
+    const uint32_t room_cap = a.ly.room_cap[l];
+    const size_t room       = room_of_bin(a.ly, l, bin);
     // record r of the bin: its own room first, what did not fit there in the compact array; as (key low, key high,
     // pixel in bin, 0) whatever its form in memory
     auto record = [&](uint32_t r) {
-        const size_t at = r < (uint32_t)kPrimaryCap ? (size_t)bin * kPrimaryCap + r : (size_t)begin + r;
+        const size_t at = r < room_cap ? room + r : (size_t)begin + r;
         if (a.compact_records)
         {
-            const uint2 v = reinterpret_cast<const uint2*>(r < (uint32_t)kPrimaryCap ? a.primary : a.binned)[at];
+            const uint2 v = reinterpret_cast<const uint2*>(r < room_cap ? a.primary : a.binned)[at];
             return make_uint4(v.y >> 8, v.x, v.y & 0xFFu, 0u);
         }
-        return (r < (uint32_t)kPrimaryCap ? a.primary : a.binned)[at];
+        return (r < room_cap ? a.primary : a.binned)[at];
     };
     const bool in_lds     = n <= (uint32_t)kBuildCap;
     s_cnt[tid] = 0u;

@@ -16,7 +16,8 @@ constexpr int kBlendChunk     = 4;            // fragments a blend / backward th
 constexpr int kBackgroundRow  = 8;            // floats per workgroup row of background-gradient partial sums
 constexpr int kPreparedBackgroundOffset = 16;  // float index inside the flags block: the background as it is blended
 constexpr int kPackedFloats   = 8;            // interleaved record: 4 descriptor floats, confidence, 3 pad
-constexpr int kPrimaryCap     = 2048;         // fragment records every bin has room for (bins are sized for <= 1024 expected)
+constexpr int kPrimaryCap     = 2048;         // fragment records a bin has room for where about a thousand are expected
+constexpr int kPrimaryCapSmall = 1024;        // ... and where at most half of that is (a bin built in LDS holds <= 1024)
 constexpr int kLogSegments    = 256;          // the overflow log is cut into this many segments with a cursor each
 constexpr int kLogCursorStride = 16;          // uint32 between two cursors (64 bytes: one cursor per cache line)
 
@@ -56,7 +57,17 @@ struct LayerTable
     // of it, 16 = one row of it, 4), chosen per layer so that a bin is expected to hold about a thousand fragments.
     int bin_shift[VETRAST_MAX_LAYERS];
     uint32_t bin_base[VETRAST_MAX_LAYERS + 1];  // first bin of the layer; [L] = number of bins
+    // Every bin owns room for room_cap[l] fragment records (its first arrivals; later ones take the overflow path):
+    // the room of bin b of layer l starts at record room_base[l] + (b - bin_base[l]) * room_cap[l].
+    uint32_t room_cap[VETRAST_MAX_LAYERS];
+    uint32_t room_base[VETRAST_MAX_LAYERS + 1];  // [L] = records in all rooms
 };
+
+// First record of the room of `bin`, a bin of layer l.
+__host__ __device__ __forceinline__ size_t room_of_bin(const LayerTable& t, int l, uint32_t bin)
+{
+    return (size_t)t.room_base[l] + (size_t)(bin - t.bin_base[l]) * t.room_cap[l];
+}
 
 // Value of lane (lane ^ M) for the xor patterns a 64-wide bitonic network needs. Inside a row of 16 lanes the exchange
 // is a DPP move (register to register, a few cycles); only the four patterns that cross rows go through the LDS

@@ -251,7 +251,7 @@ struct PackJob
 };
 
 // Where the scatter pass puts a fragment record (64-bit key = depth bits << 32 | point id, pixel inside the bin).
-// Every bin owns room for kPrimaryCap records; a record whose rank inside its bin is beyond that is appended to a log
+// Every bin owns room for room_cap[layer] records; a record whose rank inside its bin is beyond that is appended to a log
 // (with its bin and rank), from where overflow_move_kernel brings it to the bin's place in the compact array once the
 // scan of the bin counts is known. The log is cut into segments, one per residue of the workgroup number, each with a
 // cursor in a cache line of its own: appends to one cursor would queue up behind each other where many bins overflow
@@ -262,7 +262,7 @@ struct PackJob
 // Half the bytes written here and read again by the build pass.
 struct ScatterTargets
 {
-    uint4* primary;        // [bins][kPrimaryCap] records (uint2 records when compact)
+    uint4* primary;        // the bins' rooms, LayerTable::room_base (uint2 records when compact)
     int compact;
     uint4* log;            // [kLogSegments][segment_capacity]: key low, key high, pixel in bin, bin
     uint32_t* log_rank;    // the same shape: rank of the logged record inside its bin
@@ -271,16 +271,17 @@ struct ScatterTargets
 };
 
 // One record to its bin; `valid` lanes carry one. Called by the whole wave (uniform control flow).
-__device__ __forceinline__ void store_record(const ScatterTargets& t, bool valid, uint32_t bin, uint32_t rank,
-                                             uint32_t low, uint32_t depth_bits, uint32_t in_bin, int lane)
+__device__ __forceinline__ void store_record(const ScatterTargets& t, const LayerTable& ly, int l, bool valid, uint32_t bin,
+                                             uint32_t rank, uint32_t low, uint32_t depth_bits, uint32_t in_bin, int lane)
 {
-    const bool over = valid && rank >= (uint32_t)kPrimaryCap;
+    const bool over = valid && rank >= ly.room_cap[l];
     if (valid && !over)
     {
+        const size_t at = room_of_bin(ly, l, bin) + rank;
         if (t.compact)
-            reinterpret_cast<uint2*>(t.primary)[(size_t)bin * kPrimaryCap + rank] = make_uint2(depth_bits, (low << 8) | in_bin);
+            reinterpret_cast<uint2*>(t.primary)[at] = make_uint2(depth_bits, (low << 8) | in_bin);
         else
-            t.primary[(size_t)bin * kPrimaryCap + rank] = make_uint4(low, depth_bits, in_bin, 0u);
+            t.primary[at] = make_uint4(low, depth_bits, in_bin, 0u);
     }
     const uint64_t m = __ballot(over);
     if (m != 0ull)  // rare
@@ -359,7 +360,7 @@ __global__ void __launch_bounds__(kBlock) bin_scatter_kernel(ViewPass a, uint32_
         {
             if (l >= a.ly.L) continue;
             const uint32_t group_base = (uint32_t)__shfl((int)base[l], (int)(who[l] & 0xFF), kWave);
-            store_record(out, (who[l] & 0x80000000u) != 0u, bins[l], group_base + ((who[l] >> 8) & 0xFFu), (uint32_t)i,
+            store_record(out, a.ly, l, (who[l] & 0x80000000u) != 0u, bins[l], group_base + ((who[l] >> 8) & 0xFFu), (uint32_t)i,
                          depth_bits, (who[l] >> 16) & 0xFFu, lane);
         }
     }
@@ -390,7 +391,7 @@ __global__ void __launch_bounds__(kBlock) bin_scatter_kernel(ViewPass a, uint32_
                 const uint32_t s = t == 0 ? start[0] : t == 1 ? start[1] : t == 2 ? start[2] : start[3];
                 const uint32_t r = t == 0 ? ranks[l][0] : t == 1 ? ranks[l][1] : t == 2 ? ranks[l][2] : ranks[l][3];
                 const uint32_t b = t == 0 ? bins[l][0] : t == 1 ? bins[l][1] : t == 2 ? bins[l][2] : bins[l][3];
-                store_record(out, (c & 1u) != 0u, b, s + ((r >> (8u * place)) & 0xFFu), ((uint32_t)i << 2) | (uint32_t)h,
+                store_record(out, a.ly, l, (c & 1u) != 0u, b, s + ((r >> (8u * place)) & 0xFFu), ((uint32_t)i << 2) | (uint32_t)h,
                              depth_bits, (in_bins[l] >> (8 * h)) & 0xFFu, lane);
             }
         };

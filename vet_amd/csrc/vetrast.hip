@@ -112,7 +112,7 @@ LayerTable make_layer_table(int w, int h, int L, int64_t N)
     LayerTable t;
     std::memset(&t, 0, sizeof(t));
     t.L           = L;
-    uint32_t tile = 0, bin = 0;
+    uint32_t tile = 0, bin = 0, room = 0;
     for (int l = 0; l < L; ++l)
     {
         t.w[l]         = w;
@@ -129,6 +129,9 @@ LayerTable make_layer_table(int w, int h, int L, int64_t N)
         while (shift > 2 && mean_len * (double)(1 << shift) > 1024.0) shift -= 2;
         t.bin_shift[l] = shift;
         t.bin_base[l]  = bin;
+        t.room_cap[l]  = mean_len * (double)(1 << shift) > 512.0 ? kPrimaryCap : kPrimaryCapSmall;
+        t.room_base[l] = room;
+        room += (tiles << (8 - shift)) * t.room_cap[l];
         bin += tiles << (8 - shift);
         w /= 2;
         h /= 2;
@@ -138,6 +141,7 @@ LayerTable make_layer_table(int w, int h, int L, int64_t N)
         t.tile_base[l] = tile;
         t.base[l]      = tile * kTilePixels;
         t.bin_base[l]  = bin;
+        t.room_base[l] = room;
     }
     return t;
 }
@@ -488,16 +492,12 @@ int vetrast_workspace_layout_for_mode(int32_t N, int32_t B, int32_t L, int32_t w
     const size_t record_bytes = compact_records(N, hits) ? sizeof(uint2) : sizeof(uint4);
     lay->binned_base = at;
     at += align_up(cap * record_bytes, kAlign);
-    lay->log_base = at;
-    at += align_up(log_records(N, L, hits) * sizeof(uint4), kAlign);
     lay->primary_base = at;
-    at += align_up(bins * (size_t)kPrimaryCap * record_bytes, kAlign);
+    at += align_up((size_t)t.room_base[L] * record_bytes, kAlign);
     lay->views_base = at;
     at += align_up((size_t)B * sizeof(DeviceView), kAlign);
     lay->packed_base = at;
     at += align_up((size_t)N * kPackedFloats * sizeof(float), kAlign);
-    lay->slots_base = at;
-    at += align_up(log_records(N, L, hits) * sizeof(uint32_t), kAlign);
     lay->weight_base   = at;
     lay->weight_stride = align_up(P * sizeof(float), kAlign);
     at += lay->weight_stride * B;
@@ -519,15 +519,22 @@ int vetrast_workspace_layout_for_mode(int32_t N, int32_t B, int32_t L, int32_t w
     lay->projected_base   = at;
     lay->projected_stride = hits == 4 ? align_up((size_t)N * sizeof(float2), kAlign) : 0;
     at += lay->projected_stride * B;
+    // The overflow log (written by the scatter pass, emptied by overflow_move_kernel before the build pass of the same
+    // view) is dead once the forward call is over: the scratch of the backward call lies on top of it.
+    const size_t shared_base = align_up(at, kAlign);
+    lay->log_base            = shared_base;
+    at                       = shared_base + align_up(log_records(N, L, hits) * sizeof(uint4), kAlign);
+    lay->slots_base          = at;
+    at += align_up(log_records(N, L, hits) * sizeof(uint32_t), kAlign);
     lay->forward_only_bytes = align_up(at, kAlign);
-    at                      = lay->forward_only_bytes;
+    at                      = shared_base;
     lay->partial_base       = at;
     at += align_up(cap * 8 * sizeof(float), kAlign);
     lay->background_partial_base = at;
     at += align_up((size_t)tile_grid(make_tile_map(t, nullptr, true)) * kBackgroundRow * sizeof(float), kAlign);
     lay->camera_partial_base = at;
     at += align_up(((size_t)N + kBlock - 1) / kBlock * kCameraRow * sizeof(double), kAlign);
-    lay->total_bytes = align_up(at, kAlign);
+    lay->total_bytes = std::max(align_up(at, kAlign), lay->forward_only_bytes);
     return VETRAST_OK;
 }
 
