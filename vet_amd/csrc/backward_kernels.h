@@ -418,6 +418,50 @@ struct FuzzyWalk
         for (int ci = 0; ci < C; ++ci) t[ci] = tt[ci];
     }
 
+    // The same for kChunk consecutive fragments e0 .. e0 + kChunk - 1 (those below n): all keys are asked for first, then
+    // all descriptor records, so that a chunk costs two memory round trips instead of two per fragment.
+    static constexpr int kChunk = 4;
+    __device__ __forceinline__ void elements(uint32_t e0, float (&t)[kChunk][C], float (&conf)[kChunk], float (&depth)[kChunk],
+                                             int (&id)[kChunk]) const
+    {
+        uint64_t key[kChunk];
+#pragma unroll
+        for (int u = 0; u < kChunk; ++u) key[u] = e0 + u < n ? list[e0 + u] : 0ull;
+        int ti[kChunk];
+#pragma unroll
+        for (int u = 0; u < kChunk; ++u)
+        {
+            const int point = (int)(uint32_t)key[u];
+            depth[u]        = __uint_as_float((uint32_t)(key[u] >> 32));
+            ti[u]           = -1;
+            id[u]           = -1;
+            if (e0 + u < n && (uint32_t)point < (uint32_t)a->N) ti[u] = a->index ? a->index[point] : point;
+            if ((uint32_t)ti[u] < (uint32_t)a->N)
+                id[u] = point;
+            else
+                ti[u] = -1;
+        }
+        float4 t4[kChunk], c4[kChunk];
+#pragma unroll
+        for (int u = 0; u < kChunk; ++u)
+        {
+            t4[u] = c4[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (ti[u] >= 0)
+            {
+                t4[u] = a->packed[2 * (size_t)ti[u]];
+                c4[u] = a->packed[2 * (size_t)ti[u] + 1];
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < kChunk; ++u)
+        {
+            const float tt[4] = {t4[u].x, t4[u].y, t4[u].z, t4[u].w};
+#pragma unroll
+            for (int ci = 0; ci < C; ++ci) t[u][ci] = tt[ci];
+            conf[u] = c4[u].x;
+        }
+    }
+
     __device__ __forceinline__ void begin_pass(int which)
     {
         pass     = which;
@@ -598,12 +642,14 @@ __global__ void __launch_bounds__(kBlock) blend_backward_fuzzy_kernel(BackwardPa
     for (int pass = 0; pass < 2; ++pass)
     {
         w.begin_pass(pass);
-        for (uint32_t i = 0; i < w.n; ++i)
+        for (uint32_t i0 = 0; i0 < w.n; i0 += FuzzyWalk<C>::kChunk)
         {
-            float t[C], conf, d;
-            int id;
-            w.element(i, t, conf, d, id);
-            w.consume(i, t, conf, d, id);
+            float t[FuzzyWalk<C>::kChunk][C], conf[FuzzyWalk<C>::kChunk], d[FuzzyWalk<C>::kChunk];
+            int id[FuzzyWalk<C>::kChunk];
+            w.elements(i0, t, conf, d, id);
+#pragma unroll
+            for (int u = 0; u < FuzzyWalk<C>::kChunk; ++u)
+                if (i0 + u < w.n) w.consume(i0 + u, t[u], conf[u], d[u], id[u]);
         }
         if (with_background)
         {
