@@ -38,6 +38,7 @@ def build_library(verbose=True):
 
 
 UBENCH_PATH = os.path.join(LIB_DIR, "ubench_atomics")
+ACCESS_FLOOR_PATH = os.path.join(LIB_DIR, "libaccess_floor.so")
 
 
 def build_microbenchmarks(verbose=True):
@@ -46,6 +47,11 @@ def build_microbenchmarks(verbose=True):
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
     cmd = [hipcc, "--offload-arch=gfx950", "-O3", "-std=c++17", "-Xclang", "-target-feature", "-Xclang",
            "-packed-fp32-ops", os.path.join(CSRC, "ubench", "atomics.hip"), "-o", UBENCH_PATH]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    subprocess.run(cmd, check=True)
+    cmd = [hipcc, "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared", "-Xclang", "-target-feature", "-Xclang",
+           "-packed-fp32-ops", os.path.join(CSRC, "ubench", "access_floor.hip"), "-o", ACCESS_FLOOR_PATH]
     if verbose:
         print(" ".join(cmd), flush=True)
     subprocess.run(cmd, check=True)

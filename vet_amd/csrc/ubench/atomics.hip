@@ -1,4 +1,4 @@
-// Throughput of scattered global atomics, loads and stores on one GPU: the figures the binning design rests on
+// Throughput of scattered global atomics, loads and stores (4, 8 and 32 bytes) on one GPU: the figures the binning design rests on
 // (one returning atomic per wave group and bin instead of one per fragment). A stand-alone program, not part of the
 // library: built by vet_amd/build.py next to it, run by `python bench.py --atomics-ubench`.
 //
@@ -38,6 +38,7 @@ enum Mode
     kLoad4,
     kStore8,
     kStore32,
+    kLoad32,
     kModes
 };
 
@@ -61,14 +62,19 @@ __global__ void scattered_ops(uint32_t* words, uint32_t num_words, uint32_t* out
             ((float4*)words)[(a >> 3) * 2]     = v;
             ((float4*)words)[(a >> 3) * 2 + 1] = v;
         }
+        if (MODE == kLoad32)
+        {
+            const float4 lo = ((const float4*)words)[(a >> 3) * 2], hi = ((const float4*)words)[(a >> 3) * 2 + 1];
+            acc += __float_as_uint(lo.x + hi.w);
+        }
     }
-    if (MODE == kAtomicReturning || MODE == kLoad4) out[i] = acc;
+    if (MODE == kAtomicReturning || MODE == kLoad4 || MODE == kLoad32) out[i] = acc;
 }
 
 int main()
 {
     const int n = 2000000, per_thread = 4;
-    const char* names[kModes] = {"atomic add, returning", "atomic add, no return", "store 4 B", "load 4 B", "store 8 B", "store 32 B"};
+    const char* names[kModes] = {"atomic add, returning", "atomic add, no return", "store 4 B", "load 4 B", "store 8 B", "store 32 B", "load 32 B"};
     const uint32_t sizes[]    = {32400u, 2754000u, 64000000u};
     uint32_t *words, *out;
     CK(hipMalloc(&words, (size_t)64000000u * 4));
@@ -92,7 +98,8 @@ int main()
                     case kStore4: hipLaunchKernelGGL(scattered_ops<kStore4>, g, b, 0, 0, words, num_words, out, n, per_thread); break;
                     case kLoad4: hipLaunchKernelGGL(scattered_ops<kLoad4>, g, b, 0, 0, words, num_words, out, n, per_thread); break;
                     case kStore8: hipLaunchKernelGGL(scattered_ops<kStore8>, g, b, 0, 0, words, num_words, out, n, per_thread); break;
-                    default: hipLaunchKernelGGL(scattered_ops<kStore32>, g, b, 0, 0, words, num_words, out, n, per_thread); break;
+                    case kStore32: hipLaunchKernelGGL(scattered_ops<kStore32>, g, b, 0, 0, words, num_words, out, n, per_thread); break;
+                    default: hipLaunchKernelGGL(scattered_ops<kLoad32>, g, b, 0, 0, words, num_words, out, n, per_thread); break;
                 }
                 CK(hipEventRecord(e1));
                 CK(hipEventSynchronize(e1));
