@@ -817,6 +817,7 @@ __global__ void __launch_bounds__(kBlock) gather_point_gradients_kernel(GatherPa
 #pragma unroll
     for (int ci = 0; ci < C; ++ci) gt[ci] = 0.f;
     float gc = 0.f, gx = 0.f, gy = 0.f, gz = 0.f, cnt = 0.f;
+    bool hit = false;   // the point has a blended fragment in this view
     float cam_sum[10];  // pose tangent (translation, rotation), fx, fy, cx, cy
 #pragma unroll
     for (int k = 0; k < 10; ++k) cam_sum[k] = 0.f;
@@ -860,6 +861,7 @@ __global__ void __launch_bounds__(kBlock) gather_point_gradients_kernel(GatherPa
 #pragma unroll
             for (int ci = 0; ci < C; ++ci) gt[ci] += r[ci];
             gc += r1.x;
+            hit = true;
             if (a.need_point_gradient && interior_pixel(x, y, ly.w[l], ly.h[l]))
             {
                 // ProjectPointPinholeBackward (src/lib/rendering/PointRendererHelper.h:317-372) for zero distortion, with
@@ -953,9 +955,13 @@ __global__ void __launch_bounds__(kBlock) gather_point_gradients_kernel(GatherPa
     }
     else if (a.accumulate)
     {
+        // a later view of the batch: rows of points the view does not see are left as they are
+        if (hit)
+        {
 #pragma unroll
-        for (int ci = 0; ci < C; ++ci) a.grad_texture[(size_t)ci * N + i] += gt[ci];
-        a.grad_confidence[i] += gc;
+            for (int ci = 0; ci < C; ++ci) a.grad_texture[(size_t)ci * N + i] += gt[ci];
+            a.grad_confidence[i] += gc;
+        }
     }
     else
     {
@@ -968,9 +974,12 @@ __global__ void __launch_bounds__(kBlock) gather_point_gradients_kernel(GatherPa
         float4* gp = reinterpret_cast<float4*>(a.grad_points) + i;
         if (a.accumulate)
         {
-            const float4 o = *gp;
-            *gp            = make_float4(o.x + gx, o.y + gy, o.z + gz, 0.f);
-            a.grad_point_count[i] += cnt;
+            if (cnt > 0.f)  // gx, gy, gz are sums over the cnt fragments that got a position gradient
+            {
+                const float4 o = *gp;
+                *gp            = make_float4(o.x + gx, o.y + gy, o.z + gz, 0.f);
+                a.grad_point_count[i] += cnt;
+            }
         }
         else
         {
