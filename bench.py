@@ -332,6 +332,44 @@ def time_lift_error(scene, steps, cpu_threads):
     return out
 
 
+def time_training_crops(steps, samples, render_mode):
+    """A batch as VET trains on it (configs/config.ini: batch_size 4, train_crop_size 512, no list cut, radius drop-out):
+    four 512x512 crops out of config 3's frame, radii spread log-normally. Timed without and with
+    vetrast_params.expected_fragments set to the per-layer fragment counts of the call before (what the shim does)."""
+    import torch
+
+    from vet_amd import abi, synthetic
+    from vet_amd.rasterizer import DeviceScene, Rasterizer, make_params
+
+    scene = synthetic.config3(radius_spread=0.5, K=-1)
+    scene.views = [synthetic.ViewSpec(512, 512, image_index=0, crop_transform=(1.0, 1.0, -float(ox), -float(oy), 0.0))
+                   for (ox, oy) in ((200, 100), (900, 300), (1300, 500), (600, 560))]
+    rast = Rasterizer()
+    dev = DeviceScene(scene)
+    grad_out = [torch.from_numpy(g).cuda() for g in scene.grad_out()]
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    out = {"what": "4 crops of 512x512 of config 3's frame in one call, K = -1, drop_out_points_by_radius, "
+                   "forward+backward, ms per batch", "render_mode": render_mode}
+    hint = [0.0] * 5
+    for name in ("ms_per_batch", "ms_per_batch_with_expected_fragments"):
+        params = make_params(scene, need_point_gradient=1, render_mode=render_mode, drop_out_points_by_radius=1,
+                             expected_fragments=hint)
+        fwd = rast.forward(dev, params)
+        bargs = rast.backward(fwd, grad_out)["_args"]
+
+        def step():
+            abi.check(rast.lib.vetrast_forward(rast.ctx, C.byref(fwd.args), stream), "forward")
+            abi.check(rast.lib.vetrast_backward(rast.ctx, C.byref(bargs), stream), "backward")
+
+        out[name] = round(timed_samples(step, 3, steps, samples)["median"], 5)
+        off, bases = fwd.offsets(0), fwd.layer_bases()
+        counts = [int(off[bases[l + 1]] - off[bases[l]]) for l in range(scene.num_layers)]
+        out["fragments_per_layer_of_view_0"] = counts
+        hint = [float(c) for c in counts] + [0.0] * (5 - len(counts))
+        del fwd, bargs
+    return out
+
+
 def time_access_floor(scene, steps, samples):
     """The bare access pattern of the per-pixel backward kernel on the frame's real lists (vet_amd/csrc/ubench/
     access_floor.hip): every list place streams its key and transmittance; with `gather` it also reads its point's
@@ -588,6 +626,8 @@ def main():
         result["calibration_kernel"] = {"kernel": "adam_step_kernel", "elements": n, "read_bytes": 16 * n,
                                         "write_bytes": 12 * n}
 
+    if extras and backward and args.config == 3:
+        result["training_crops"] = time_training_crops(max(10, args.steps // 2), 3, args.render_mode)
     if extras:
         result["lift_error"] = time_lift_error(scene, max(10, args.steps // 2), 0 if args.no_cpu_baseline else cpu_threads)
 

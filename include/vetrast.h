@@ -101,6 +101,13 @@ typedef struct vetrast_params
     int32_t texture_abs;                      /* 1: |texture| and |background| (PipelineParams::non_subzero_texture) */
     float depth_accept_blend;                 /* FUZZY_BLEND: depth range of a bucket, RenderParams::depth_accept_blend
                                                  (src/lib/data/Settings.h:42, default 0.01); must lie in (0, 1e4) */
+    /* A hint for speed only; results do not depend on it. The pixels of a layer are cut into bins sized so that a bin
+     * is expected to hold about a thousand fragments if EVERY point lands in the layer. A view that sees a part of the
+     * cloud (VET trains on 512x512 crops, configs/config.ini:27) or drops points by radius at the coarse layers then
+     * gets bins far too small. expected_fragments[l] > 0 says how many fragments ONE view is expected to leave in layer
+     * l (e.g. what the previous call left there: offsets[layer_pixel_base[l + 1]] - offsets[layer_pixel_base[l]]); the
+     * bins of that layer are sized for it. 0: every point. No counterpart in the reference. */
+    float expected_fragments[VETRAST_MAX_LAYERS];
 } vetrast_params;
 
 #define VETRAST_RENDER_FULL_BLEND 1

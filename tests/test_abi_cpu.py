@@ -30,7 +30,7 @@ def test_library_exports_every_declared_symbol():
 def test_struct_sizes_are_the_c_ones():
     # sizes the C compiler gives the structs of include/vetrast.h (LP64)
     assert C.sizeof(abi.View) == 5 * 4 + 9 * 4
-    assert C.sizeof(abi.Params) == 21 * 4
+    assert C.sizeof(abi.Params) == 21 * 4 + abi.MAX_LAYERS * 4
     assert C.sizeof(abi.LiftArgs) == 8 + 4 * 8 + 2 * 4 + 2 * 8 + C.sizeof(abi.View) + 8 + 4 * 4 + 2 * 8 == 160
     assert abi.LiftArgs.loss_image.offset % 8 == 0
     assert C.sizeof(abi.ForwardArgs) % 8 == 0

@@ -124,6 +124,36 @@ def test_processing_order_changes_nothing(mode, rasterizer):
             assert torch.equal(got[k], v), k
 
 
+@pytest.mark.parametrize("mode", [abi.RENDER_FULL_BLEND, abi.RENDER_BILINEAR_BLEND])
+def test_expected_fragments_hint_changes_nothing(mode, rasterizer):
+    """vetrast_params.expected_fragments only sizes the pixel bins: a crop that sees a part of the cloud gives the same
+    lists, images and gradients with the true counts, with counts far too small (records overflow their bins' rooms
+    and take the log path) and with counts far too large as with none."""
+    scene = synthetic.config2(num_points=120_000, w=480, h=270, K=8)
+    scene.views = [synthetic.ViewSpec(128, 96, crop_transform=(1.0, 1.0, -170.0, -90.0, 0.0)),
+                   synthetic.ViewSpec(128, 96, crop_transform=(1.0, 1.0, -20.0, -150.0, 0.0))]
+    dev = DeviceScene(scene)
+    grad_out = [torch.from_numpy(g).cuda() for g in scene.grad_out()]
+    plain = rasterizer.forward(dev, make_params(scene, need_point_gradient=1, render_mode=mode))
+    plain_g = {k: v.clone() for k, v in rasterizer.backward(plain, grad_out).items() if k != "_args"}
+    off, bases = plain.offsets(0), plain.layer_bases()
+    true_counts = [float(off[bases[l + 1]] - off[bases[l]]) for l in range(scene.num_layers)]
+    assert 0 < sum(true_counts) < 0.5 * scene.num_points * scene.num_layers, "the crop must see a part of the cloud only"
+    for hint in (true_counts, [1.0] * 4, [c * 50 for c in true_counts], [true_counts[0], 0.0, 3.0, 0.0]):
+        res = rasterizer.forward(dev, make_params(scene, need_point_gradient=1, render_mode=mode, expected_fragments=hint))
+        got = rasterizer.backward(res, grad_out)
+        torch.cuda.synchronize()
+        assert rasterizer.check_device_flags(res) == 0
+        for b in range(2):
+            np.testing.assert_array_equal(res.offsets(b), plain.offsets(b))
+            kept = kept_mask(plain.offsets(b), scene.max_list_length)  # what lies behind the cut is in no particular order
+            np.testing.assert_array_equal(res.fragments(b)[kept], plain.fragments(b)[kept])
+        for a, b in zip(res.out, plain.out):
+            assert torch.equal(a, b)
+        for k, v in plain_g.items():
+            assert torch.equal(got[k], v), k
+
+
 def _backward_pair(scene, overrides, rasterizer, oracle, want_points=True):
     ref, dev, res, _ = _check_forward(scene, overrides, rasterizer, oracle)
     grad_out = scene.grad_out()

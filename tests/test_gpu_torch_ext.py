@@ -405,3 +405,34 @@ def test_the_cache_keeps_a_processing_order_and_results_do_not_depend_on_it():
         assert torch_ops.point_order().numel() == 20_000
     finally:
         torch_ops.set_point_order_refresh(1000)
+
+
+def test_the_cache_sizes_bins_from_the_fragment_counts_of_earlier_calls():
+    """Crops that see a part of the cloud: the shim reads the per-layer fragment counts of a call back without blocking
+    and sizes the bins of later calls with them; images and gradients are the same bits with and without."""
+    from vet_amd import torch_ops
+
+    scene = synthetic.config2(num_points=60_000, w=480, h=270, K=8)
+    scene.views = [synthetic.ViewSpec(128, 96, crop_transform=(1.0, 1.0, -170.0, -90.0, 0.0))]
+    cu = lambda a, rg=False: torch.from_numpy(np.ascontiguousarray(a)).cuda().requires_grad_(rg)
+    grads = [torch.from_numpy(g).cuda() for g in scene.grad_out()]
+
+    def run(history):
+        texture, confidence = cu(scene.texture, True), cu(scene.confidence.reshape(1, -1), True)
+        outs = torch_ops.blend_point_cloud(texture, cu(scene.background), cu(scene.position),
+                                           torch.zeros((1, 6), dtype=torch.float64, device="cuda"), cu(scene.intrinsics),
+                                           confidence, cu(scene.poses_se3), None, _views(scene), scene.num_layers,
+                                           train=True, use_environment_map=0, need_point_gradient=0,
+                                           drop_out_points_by_radius=0, debug_max_list_length=scene.max_list_length,
+                                           size_bins_from_history=1 if history else 0)
+        torch.autograd.backward(outs, grads)
+        torch.cuda.synchronize()
+        return [o.detach().clone() for o in outs] + [texture.grad, confidence.grad]
+
+    plain = run(False)
+    first = run(True)   # nothing known yet: schedules the read-back
+    second = run(True)  # the copy has landed (run() synchronises): bins sized from it
+    hist = torch_ops.fragment_history()
+    assert len(hist) == scene.num_layers and 0 < sum(hist) < 0.5 * scene.num_points * scene.num_layers
+    for a, b, c in zip(plain, first, second):
+        assert torch.equal(a, b) and torch.equal(a, c)

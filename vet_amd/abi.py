@@ -63,6 +63,7 @@ class Params(C.Structure):
         ("confidence_scale", C.c_float),
         ("texture_abs", C.c_int32),
         ("depth_accept_blend", C.c_float),
+        ("expected_fragments", C.c_float * MAX_LAYERS),
     ]
 
 

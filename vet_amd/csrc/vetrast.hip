@@ -107,7 +107,7 @@ inline int grid_for(size_t n, int block = kBlock)
 }
 
 // N only steers the bin sizes: N / pixels bounds the mean list length of a layer from above without any device read.
-LayerTable make_layer_table(int w, int h, int L, int64_t N)
+LayerTable make_layer_table(int w, int h, int L, int64_t N, const float* expected_fragments = nullptr)
 {
     LayerTable t;
     std::memset(&t, 0, sizeof(t));
@@ -124,9 +124,19 @@ LayerTable make_layer_table(int w, int h, int L, int64_t N)
         const uint32_t tiles = (uint32_t)t.tiles_x[l] * (uint32_t)t.tiles_y[l];
         tile += tiles;
         // largest bin of 256, 64, 16 or 4 pixels expected to hold at most 1024 fragments
-        const double mean_len = (double)N / ((double)w * (double)h);
+        // Fragments the bins of the layer are sized for: every point, unless the caller knows how many a view leaves
+        // there. Then twice that number: the rule below was tuned on full frames, sized for every point, of which about
+        // half were in view (surfaces put a multiple of the mean into many bins).
+        double in_layer = (double)N;
+        if (expected_fragments && expected_fragments[l] > 0.f && 2.0 * (double)expected_fragments[l] < in_layer)
+            in_layer = 2.0 * (double)expected_fragments[l];
+        const double mean_len = in_layer / ((double)w * (double)h);
         int shift             = 8;
         while (shift > 2 && mean_len * (double)(1 << shift) > 1024.0) shift -= 2;
+        // ... and small enough for the layer to have a thousand bins where it has the pixels for them: every bin is one
+        // workgroup's chain of dependent steps, and a layer of a few dozen big bins (a coarse layer of a 512x512
+        // training crop) runs them on a few dozen compute units while the others wait
+        while (shift > 2 && (tiles << (8 - shift)) < 1024u) shift -= 2;
         t.bin_shift[l] = shift;
         t.bin_base[l]  = bin;
         t.room_cap[l]  = mean_len * (double)(1 << shift) > 512.0 ? kPrimaryCap : kPrimaryCapSmall;
@@ -143,6 +153,18 @@ LayerTable make_layer_table(int w, int h, int L, int64_t N)
         t.bin_base[l]  = bin;
         t.room_base[l] = room;
     }
+    return t;
+}
+
+// The layer table the kernels of a call work with: bins sized for the fragments the caller expects a view to leave in
+// every layer (vetrast_params.expected_fragments), but never more bins or more room than the table the workspace was
+// laid out for (every point in every layer), which smaller expectations cannot exceed: coarser bins are fewer, and a
+// bin's room at most doubles where its pixels quadruple.
+LayerTable make_call_layer_table(int w, int h, int L, int64_t hits_if_all_visible, const float* expected_fragments)
+{
+    const LayerTable full = make_layer_table(w, h, L, hits_if_all_visible);
+    const LayerTable t    = make_layer_table(w, h, L, hits_if_all_visible, expected_fragments);
+    if (t.bin_base[L] > full.bin_base[L] || t.room_base[L] > full.room_base[L]) return full;
     return t;
 }
 
@@ -555,7 +577,7 @@ int vetrast_forward(vetrast_ctx* ctx, const vetrast_forward_args* a, void* strea
     const vetrast_params& p = a->params;
     const int N = a->num_points, B = a->num_views, L = p.num_layers, C = p.num_texture_channels;
     const int hits      = hits_of_mode(p.render_mode);
-    const LayerTable ly = make_layer_table(a->views[0].w, a->views[0].h, L, (int64_t)N * hits);
+    const LayerTable ly = make_call_layer_table(a->views[0].w, a->views[0].h, L, (int64_t)N * hits, p.expected_fragments);
     const uint32_t bins = ly.bin_base[L];
     const size_t Tpad   = lay.bin_counts_stride / sizeof(uint32_t);
     void* ws            = a->workspace;
@@ -739,7 +761,7 @@ int vetrast_backward(vetrast_ctx* ctx, const vetrast_backward_args* g, void* str
     hipStream_t stream = (hipStream_t)stream_;
     const int N = a->num_points, B = a->num_views, L = p.num_layers, C = p.num_texture_channels;
     const int hits      = hits_of_mode(p.render_mode);
-    const LayerTable ly = make_layer_table(a->views[0].w, a->views[0].h, L, (int64_t)N * hits);
+    const LayerTable ly = make_call_layer_table(a->views[0].w, a->views[0].h, L, (int64_t)N * hits, p.expected_fragments);
     // fragments a pixel of layer l blends, bounded from above without a device read: all points land in the layer, the
     // top-K cut
     double list_bound[VETRAST_MAX_LAYERS] = {};

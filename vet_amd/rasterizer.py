@@ -41,6 +41,10 @@ def make_params(scene: Scene, **overrides) -> abi.Params:
     for k, v in {**scene.params, **overrides}.items():
         if not hasattr(p, k):
             raise AttributeError(f"vetrast_params has no field {k}")
+        if k == "expected_fragments":
+            for l, x in enumerate(v):
+                p.expected_fragments[l] = float(x)
+            continue
         setattr(p, k, v)
     return p
 

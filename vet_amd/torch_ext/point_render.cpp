@@ -8,6 +8,7 @@
 #include <fstream>
 #include <random>
 
+#include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
 #include <c10/hip/HIPStream.h>
 #include <torch/extension.h>
 
@@ -31,6 +32,7 @@ vetrast_params to_abi_params(const RenderParams& p, int num_layers)
     std::memset(&q, 0, sizeof(q));
     q.render_mode                      = p.render_mode;
     q.depth_accept_blend               = p.depth_accept_blend;
+    for (int l = 0; l < VETRAST_MAX_LAYERS; ++l) q.expected_fragments[l] = p.expected_fragments[l] > 0.f ? p.expected_fragments[l] : 0.f;
     q.num_texture_channels             = p.num_texture_channels;
     q.num_layers                       = num_layers;
     q.debug_max_list_length            = p.debug_max_list_length;
@@ -216,6 +218,9 @@ torch::autograd::variable_list PointRender::forward(torch::autograd::AutogradCon
     torch::Tensor dropout;
     if (info->train && info->params.dropout > 0) dropout = torch::empty({B, N}, f32).bernoulli_(info->params.dropout);
 
+    if (info->params.size_bins_from_history)
+        info->cache->ExpectedFragments(info->params.expected_fragments, N, L, info->images[0].w, info->images[0].h,
+                                       info->params.render_mode);
     // side inputs read through info->scene; they are saved with the graph so that backward does not touch the scene
     const torch::Tensor poses_se3 = info->scene->poses_se3;
     const torch::Tensor t_index   = info->scene->t_index;
@@ -278,6 +283,8 @@ torch::autograd::variable_list PointRender::forward(torch::autograd::AutogradCon
     const torch::Tensor& order = info->cache->PointOrderFor(points);
     a.point_order              = order.defined() ? order.data_ptr<int32_t>() : nullptr;
     check_status(vetrast_forward(info->cache->ctx, &a, current_stream()), "forward");
+    if (info->params.size_bins_from_history)
+        info->cache->NoteFragmentCounts(workspace, lay, N, L, info->images[0].w, info->images[0].h, a.params.render_mode);
 
     if (need_backward)
     {
@@ -707,6 +714,61 @@ torch::Tensor ProcessingOrderOnDevice(const torch::Tensor& positions, int64_t bl
     return order.to(torch::kInt32);
 }
 
+void PointRendererCache::PollFragmentCounts()
+{
+    if (!counts_pending_ || !counts_event_ || !counts_event_->query()) return;
+    const int32_t* v = counts_host_.data_ptr<int32_t>();
+    for (int l = 0; l < VETRAST_MAX_LAYERS; ++l) counts_[l] = l < pending_key_.L ? (float)(v[l + 1] - v[l]) : 0.f;
+    counts_key_     = pending_key_;
+    counts_valid_   = true;
+    counts_pending_ = false;
+}
+
+std::vector<float> PointRendererCache::FragmentHistory()
+{
+    PollFragmentCounts();
+    if (!counts_valid_) return {};
+    return std::vector<float>(counts_, counts_ + counts_key_.L);
+}
+
+void PointRendererCache::ExpectedFragments(float* expected, int64_t N, int L, int w, int h, int render_mode)
+{
+    PollFragmentCounts();
+    CountsKey key;
+    key.N = N, key.L = L, key.w = w, key.h = h, key.mode = render_mode;
+    const bool known = counts_valid_ && counts_key_ == key;
+    for (int l = 0; l < VETRAST_MAX_LAYERS; ++l) expected[l] = (known && l < L) ? counts_[l] + 1024.f : 0.f;
+}
+
+void PointRendererCache::NoteFragmentCounts(const torch::Tensor& workspace, const vetrast_workspace_layout& lay, int64_t N,
+                                            int L, int w, int h, int render_mode)
+{
+    CountsKey key;
+    key.N = N, key.L = L, key.w = w, key.h = h, key.mode = render_mode;
+    const bool known = counts_valid_ && counts_key_ == key;
+    ++calls_since_readback_;
+    if (counts_pending_ || (known && calls_since_readback_ < 16)) return;
+    calls_since_readback_ = 0;
+    torch::NoGradGuard no_grad;
+    const int64_t P = lay.layer_pixel_base[L];
+    if (!counts_index_.defined() || !(pending_key_ == key) || counts_index_.device() != workspace.device())
+    {
+        std::vector<int64_t> at((size_t)VETRAST_MAX_LAYERS + 1, P);
+        for (int l = 0; l <= L; ++l) at[(size_t)l] = lay.layer_pixel_base[l];
+        counts_index_ = torch::tensor(at, torch::TensorOptions().dtype(torch::kInt64)).to(workspace.device());
+    }
+    if (!counts_host_.defined())
+        counts_host_ = torch::empty({VETRAST_MAX_LAYERS + 1}, torch::TensorOptions().dtype(torch::kInt32).pinned_memory(true));
+    // view 0's exclusive scan of the per-pixel counts: the entry at a layer's first pixel is the number of fragments
+    // of the layers in front of it
+    const torch::Tensor scan = workspace.narrow(0, (int64_t)lay.offsets_base, (P + 1) * 4).view(torch::kInt32);
+    counts_host_.copy_(scan.index_select(0, counts_index_), /*non_blocking=*/true);
+    if (!counts_event_) counts_event_ = std::make_unique<c10::Event>(c10::DeviceType::CUDA);
+    counts_event_->record(c10::hip::getCurrentHIPStreamMasqueradingAsCUDA());
+    pending_key_    = key;
+    counts_pending_ = true;
+}
+
 const torch::Tensor& PointRendererCache::PointOrderFor(const torch::Tensor& points)
 {
     if (point_order_refresh <= 0)
@@ -812,6 +874,12 @@ std::vector<torch::Tensor> blend_point_cloud(torch::Tensor texture, torch::Tenso
         else if (k == "point_gradient_normalization") p.point_gradient_normalization = (int)as_d();
         else if (k == "render_mode") p.render_mode = (int)as_d();
         else if (k == "depth_accept_blend") p.depth_accept_blend = (float)as_d();
+        else if (k == "size_bins_from_history") p.size_bins_from_history = as_d() != 0.0;
+        else if (k == "expected_fragments")
+        {
+            auto v = item.second.cast<std::vector<double>>();
+            for (size_t l = 0; l < v.size() && l < (size_t)VETRAST_MAX_LAYERS; ++l) p.expected_fragments[l] = (float)v[l];
+        }
         else if (k == "K_gradient_factor") p.K_gradient_factor = (float)as_d();
         else if (k == "camera_gradient_normalization") p.camera_gradient_normalization = as_d() != 0;
         else if (k == "fused_confidence_scale") p.fused_confidence_scale = (float)as_d();
@@ -1011,6 +1079,9 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
             g_cache->point_order         = torch::Tensor();
         },
         "forward calls between rebuilds of the cache's processing order; 0 switches it off");
+    m.def(
+        "fragment_history", []() { return g_cache ? g_cache->FragmentHistory() : std::vector<float>(); },
+        "fragments per layer one view of a recent call left, as read back by the cache (empty: none yet)");
     m.def(
         "point_order",
         []() { return (g_cache && g_cache->point_order.defined()) ? g_cache->point_order : torch::Tensor(); },

@@ -40,6 +40,13 @@ struct RenderParams
     bool use_environment_map           = true;
     int render_mode                    = 1;  // 1 = FULL_BLEND, 2 = FUZZY_BLEND, 3 = BILINEAR_BLEND; mode 0 is not implemented
     float depth_accept_blend           = 0.01f;  // FUZZY_BLEND: depth range of a bucket
+    // Not in the reference. Hints for speed only (vetrast_params.expected_fragments): how many fragments one view is
+    // expected to leave in every layer, for sizing the pixel bins (0: every point lands in the layer, which is far too
+    // many for a 512x512 training crop or a layer most points drop out of by radius). With size_bins_from_history the
+    // cache fills the array from the fragment counts of earlier calls with the same image size, read back without
+    // blocking every few calls. Results do not depend on either.
+    bool size_bins_from_history        = true;
+    float expected_fragments[VETRAST_MAX_LAYERS] = {0.f, 0.f, 0.f, 0.f, 0.f};
     bool viewer_only                   = false;
     int debug_max_list_length          = -1;
     // Switches for two accidents of the reference implementation; the defaults reproduce it literally.
@@ -111,6 +118,14 @@ class PointRendererCache
     int64_t point_order_refresh = 1000;
     torch::Tensor point_order;  // int32 [N] on the points' device, or undefined
     const torch::Tensor& PointOrderFor(const torch::Tensor& points);
+    // Fragments per layer that a view of recent calls left, for RenderParams::expected_fragments: every 16th forward
+    // call copies the layer boundaries of view 0's scan to pinned host memory without blocking; the numbers are taken
+    // up by a later call once the copy has landed. Kept per image size, layer count, point count and render mode.
+    void ExpectedFragments(float* expected, int64_t N, int L, int w, int h, int render_mode);
+    void NoteFragmentCounts(const torch::Tensor& workspace, const vetrast_workspace_layout& lay, int64_t N, int L, int w,
+                            int h, int render_mode);
+    // what ExpectedFragments would work from right now (empty: nothing has been read back yet)
+    std::vector<float> FragmentHistory();
     // layers_cuda[l].weight of the reference's cache (src/lib/rendering/PointRenderer.h:131, written at
     // src/lib/rendering/RenderForward.cu:1355-1356): per layer [B,1,h_l,w_l], the transmittance left behind the last
     // blended fragment of every pixel. Only kept up to date by BlendPointCloud while keep_layer_weights is set.
@@ -130,6 +145,19 @@ class PointRendererCache
     const void* checked_intrinsics_ptr_ = nullptr;
     int64_t checked_intrinsics_version_ = -1, checked_intrinsics_numel_ = -1;
     int64_t point_order_age_ = 0;
+    struct CountsKey
+    {
+        int64_t N = -1;
+        int L = 0, w = 0, h = 0, mode = 0;
+        bool operator==(const CountsKey& o) const { return N == o.N && L == o.L && w == o.w && h == o.h && mode == o.mode; }
+    };
+    CountsKey counts_key_, pending_key_;
+    float counts_[VETRAST_MAX_LAYERS] = {0.f, 0.f, 0.f, 0.f, 0.f};
+    bool counts_valid_ = false, counts_pending_ = false;
+    int64_t calls_since_readback_ = 0;
+    torch::Tensor counts_host_, counts_index_;
+    std::unique_ptr<c10::Event> counts_event_;
+    void PollFragmentCounts();
 };
 
 class NeuralRenderInfo : public torch::CustomClassHolder

@@ -87,6 +87,11 @@ def point_order():
     return t if t is not None and t.numel() > 0 else None
 
 
+def fragment_history():
+    """Fragments per layer that one view of a recent call left, as the shim's cache has read them back ([] = none yet)."""
+    return list(load().fragment_history())
+
+
 def train_workspace_info():
     """(data_ptr, bytes) of the workspace the binding's cache keeps between training steps; (0, 0) before the first."""
     d = load().train_workspace_info()
