@@ -294,7 +294,7 @@ def time_lift_error(scene, steps, cpu_threads):
     error image. Reported beside the headline number, not part of it; the CPU oracle is timed on the same call."""
     import torch
 
-    from vet_amd import synthetic
+    from vet_amd import abi, synthetic
     from vet_amd.rasterizer import Rasterizer
 
     rast = Rasterizer()
@@ -309,7 +309,7 @@ def time_lift_error(scene, steps, cpu_threads):
     ws = rast.lift_error(d_mn, d_ln, val, cnt, view, d_pose, d_intr, d_img)
     torch.cuda.synchronize()
     pixels = int(cnt.sum().item())
-    queued = int(ws[128:132].view(torch.int32).item())
+    queued = int(ws[abi.LIFT_QUEUE_LENGTH_OFFSET:abi.LIFT_QUEUE_LENGTH_OFFSET + 4].view(torch.int32).item())
     calls = [1]
 
     def call():

@@ -34,12 +34,13 @@ typedef enum vetrast_status
     VETRAST_ERR_WORKSPACE_SMALL = -2, /* workspace_bytes below vetrast_forward_workspace_bytes() */
     VETRAST_ERR_HIP             = -3, /* a HIP runtime call failed; see vetrast_last_hip_error() */
     VETRAST_ERR_UNSUPPORTED     = -4, /* a reference feature outside the blending path (OCam, normals, ...) */
-    VETRAST_ERR_BAD_INPUT_DATA  = -5, /* device-side check failed (non-zero distortion), from vetrast_query_device_flags */
+    VETRAST_ERR_BAD_INPUT_DATA  = -5, /* device-side check failed (non-zero distortion that was not allowed), from
+                                         vetrast_query_device_flags */
     VETRAST_ERR_TOO_LARGE       = -6  /* size beyond the fixed maximum of an entry point that allocates nothing */
 } vetrast_status;
 
 /* Camera model tag of a view. Mirrors enum CameraModel, src/lib/data/SceneData.h:30-35.
- * Only PINHOLE_DISTORTION with all eight distortion coefficients equal to zero is implemented. */
+ * Only PINHOLE_DISTORTION is implemented; non-zero distortion coefficients need vetrast_params.allow_distortion. */
 #define VETRAST_CAMERA_PINHOLE_DISTORTION 0
 #define VETRAST_CAMERA_OCAM 1
 #define VETRAST_CAMERA_SPHERICAL 2
@@ -108,6 +109,20 @@ typedef struct vetrast_params
      * l (e.g. what the previous call left there: offsets[layer_pixel_base[l + 1]] - offsets[layer_pixel_base[l]]); the
      * bins of that layer are sized for it. 0: every point. No counterpart in the reference. */
     float expected_fragments[VETRAST_MAX_LAYERS];
+    /* Lens distortion. The reference distorts the normalised image point with saiga's distortNormalizedPoint
+     * (src/lib/rendering/PointRendererHelper.h:207,348), which is not part of its source tree; cameras with non-zero
+     * coefficients are therefore refused (VETRAST_ERR_BAD_INPUT_DATA through vetrast_query_device_flags) unless
+     * allow_distortion is set. With it, columns 5..12 of `intrinsics` are taken as k1 k2 k3 k4 k5 k6 p1 p2 (the order
+     * of src/lib/data/SceneData.cpp:464-478) of the rational model
+     *   x' = x (1 + k1 r^2 + k2 r^4 + k3 r^6) / (1 + k4 r^2 + k5 r^4 + k6 r^6) + 2 p1 x y + p2 (r^2 + 2 x^2)
+     *   y' = y (   same ratio   )                                              + p1 (r^2 + 2 y^2) + 2 p2 x y
+     * and the backward pass returns their gradient scaled as src/lib/rendering/RenderBackward.cu:1440-1455 scales it
+     * (k3 x 0.25, k4..k6 and p1, p2 x 0.1, everything x distortion_gradient_factor). PARITY WITH THE REFERENCE IS
+     * UNPINNED for such cameras: the formula is the published one the coefficient layout implies, not saiga's code,
+     * and RenderParams::dist_cutoff (points beyond the radius where the polynomial stops being monotonic are culled
+     * by saiga) is not applied. */
+    int32_t allow_distortion;
+    float distortion_gradient_factor;         /* RenderParams::distortion_gradient_factor, src/lib/data/Settings.h:54 */
 } vetrast_params;
 
 #define VETRAST_RENDER_FULL_BLEND 1
@@ -250,8 +265,8 @@ typedef struct vetrast_backward_args
     double* grad_pose;           /* device [F,6]: d/d(se3 tangent: translation, rotation) of pose row image_index; overwritten */
     float* grad_pose_count;      /* device [F]: fragments / 1024 per pose row; required with grad_pose */
     float* grad_intrinsics;      /* device [num_cameras,13]: fx,fy,cx,cy scaled by K_gradient_factor; the skew column is
-                                    zeroed as in the reference, and the 8 distortion columns stay 0 (their Jacobian is in
-                                    saiga, which is not available); overwritten */
+                                    zeroed as in the reference; the 8 distortion columns are filled where
+                                    vetrast_params.allow_distortion is set, else stay 0; overwritten */
     float* grad_intrinsics_count; /* device [num_cameras]: fragments / 1024 per camera row; required with grad_intrinsics */
 } vetrast_backward_args;
 
@@ -327,6 +342,9 @@ int vetrast_adam_step(vetrast_ctx* ctx, const vetrast_adam_args* args, void* str
 /* Byte offset inside the workspace of a uint32 that is 1 after the call if the camera row holds non-zero distortion
  * coefficients (they are ignored, as in vetrast_forward), else 0. */
 #define VETRAST_LIFT_FLAGS_OFFSET 192
+/* Byte offset inside the workspace of a uint32 that holds, after the call, how many cells were too large on screen for
+ * one wave and went through the shared path (a diagnostic; nothing has to read it). */
+#define VETRAST_LIFT_QUEUE_LENGTH_OFFSET 176
 typedef struct vetrast_lift_args
 {
     int64_t num_cells;

@@ -145,16 +145,19 @@ def backward(fwd: OracleForward, grad_out, want_points=True, want_cameras=False,
 
 
 def prepare_view(pose8, intrinsics13):
-    out = np.zeros(17, np.float32)
+    """Camera constants of a view: [0:12] rotation rows with the translation in the fourth column, [12:17] fx fy cx cy
+    s, [17:25] the distortion coefficients k1 k2 k3 k4 k5 k6 p1 p2, [25] 1 if any of them is not zero."""
+    out = np.zeros(26, np.float32)
     p = np.ascontiguousarray(pose8, np.float64)
     k = np.ascontiguousarray(intrinsics13, np.float32)
     load().vetref_prepare_view(_addr(p), _addr(k), _addr(out))
     return out
 
 
-def project_point(prepared17, view: abi.View, position4):
+def project_point(prepared26, view: abi.View, position4):
     out = np.zeros(4, np.float32)
-    m = np.ascontiguousarray(prepared17, np.float32)
+    m = np.ascontiguousarray(prepared26, np.float32)
+    assert m.size == 26
     p = np.ascontiguousarray(position4, np.float32)
     ok = load().vetref_project_point(_addr(m), C.byref(view), _addr(p), _addr(out))
     return bool(ok), out

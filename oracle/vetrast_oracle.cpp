@@ -21,6 +21,8 @@ struct Prepared
     float r[9];  // row-major rotation, world -> camera
     float t[3];
     float fx, fy, cx, cy, s;
+    float dist[8];  // k1 k2 k3 k4 k5 k6 p1 p2; used only when has_dist
+    bool has_dist;
 };
 
 struct Layers
@@ -75,7 +77,56 @@ Prepared prepare(const double* q, const float* intr)
     p.cx   = intr[2];
     p.cy   = intr[3];
     p.s    = intr[4];
+    p.has_dist = false;
+    for (int k = 0; k < 8; ++k)
+    {
+        p.dist[k] = intr[5 + k];
+        if (intr[5 + k] != 0.f) p.has_dist = true;
+    }
     return p;
+}
+
+// The 8-coefficient rational distortion model (k1 k2 k3 k4 k5 k6 p1 p2) on a normalised image point, every operation
+// rounded on its own. The reference calls saiga's distortNormalizedPoint here (rendering/PointRendererHelper.h:207),
+// which is not in its source tree: this is the published model its coefficient layout implies, parity unpinned.
+// J (optional): d(xd, yd) / d(x, y) row-major; Jd (optional): d(xd, yd) / d coefficient k as Jd[2 k], Jd[2 k + 1].
+inline void distort(const float* d, float x, float y, float& xd, float& yd, float* J = nullptr, float* Jd = nullptr)
+{
+    const float x2 = x * x, y2 = y * y, r2 = x2 + y2, xy2 = (2.f * x) * y;
+    const float u   = 1.f + r2 * (d[0] + r2 * (d[1] + r2 * d[2]));
+    const float v   = 1.f + r2 * (d[3] + r2 * (d[4] + r2 * d[5]));
+    const float iv  = 1.f / v;
+    const float rad = u * iv;
+    const float tx = d[6] * xy2 + d[7] * (r2 + 2.f * x2);
+    const float ty = d[6] * (r2 + 2.f * y2) + d[7] * xy2;
+    xd = x * rad + tx;
+    yd = y * rad + ty;
+    if (J)
+    {
+        const float du   = d[0] + r2 * (2.f * d[1] + (3.f * d[2]) * r2);  // du / d r2
+        const float dv   = d[3] + r2 * (2.f * d[4] + (3.f * d[5]) * r2);
+        const float drad = (du * v - u * dv) * (iv * iv);                  // d rad / d r2
+        const float rx = drad * (2.f * x), ry = drad * (2.f * y);          // d rad / dx, dy
+        J[0] = (rad + x * rx) + ((2.f * d[6]) * y + (6.f * d[7]) * x);
+        J[1] = x * ry + ((2.f * d[6]) * x + (2.f * d[7]) * y);
+        J[2] = y * rx + ((2.f * d[6]) * x + (2.f * d[7]) * y);
+        J[3] = (rad + y * ry) + ((6.f * d[6]) * y + (2.f * d[7]) * x);
+    }
+    if (Jd)
+    {
+        const float r4 = r2 * r2, r6 = r4 * r2;
+        const float a = iv, b = -(u * (iv * iv));
+        const float c[6] = {a * r2, a * r4, a * r6, b * r2, b * r4, b * r6};
+        for (int k = 0; k < 6; ++k)
+        {
+            Jd[2 * k]     = x * c[k];
+            Jd[2 * k + 1] = y * c[k];
+        }
+        Jd[12] = xy2;
+        Jd[13] = r2 + 2.f * y2;
+        Jd[14] = r2 + 2.f * x2;
+        Jd[15] = xy2;
+    }
 }
 
 bool distortion_is_zero(const float* intr)
@@ -101,8 +152,9 @@ bool project(const Prepared& c, const vetrast_view& v, const float* p4, Projecte
     const float vz = ((c.r[6] * x + c.r[7] * y) + c.r[8] * zz) + c.t[2];
     float z        = std::fmax(vz, 0.f);  // PointRendererHelper.h:191-192
     if (!(z > 0.f)) return false;        // z == 0 (also NaN)
-    const float nx = vx / vz;             // DivideByZ, PointRendererHelper.h:205
-    const float ny = vy / vz;
+    float nx = vx / vz;                   // DivideByZ, PointRendererHelper.h:205
+    float ny = vy / vz;
+    if (c.has_dist) distort(c.dist, nx, ny, nx, ny);  // distortNormalizedPoint, PointRendererHelper.h:207
     const float u  = (c.fx * nx + c.s * ny) + c.cx;  // K.normalizedToImage, PointRendererHelper.h:214
     const float w  = c.fy * ny + c.cy;
     const float* k = v.crop_transform;
@@ -303,7 +355,8 @@ int validate(const vetrast_forward_args* a)
         if (v.w != a->views[0].w || v.h != a->views[0].h || v.w < 1 || v.h < 1) return VETRAST_ERR_INVALID_ARG;
         if (v.image_index < 0 || v.image_index >= a->num_poses) return VETRAST_ERR_INVALID_ARG;
         if (v.camera_index < 0 || v.camera_index >= a->num_cameras) return VETRAST_ERR_INVALID_ARG;
-        if (!distortion_is_zero(a->intrinsics + 13 * (size_t)v.camera_index)) return VETRAST_ERR_BAD_INPUT_DATA;
+        if (!p.allow_distortion && !distortion_is_zero(a->intrinsics + 13 * (size_t)v.camera_index))
+            return VETRAST_ERR_BAD_INPUT_DATA;
     }
     return VETRAST_OK;
 }
@@ -358,9 +411,10 @@ struct PointGrad
     float gp[3];
     double gpose[6];
     float gk[5];
+    float gdis[8];
 };
 
-// ProjectPointPinholeBackward, rendering/PointRendererHelper.h:317-372, for zero distortion (J_p_dis = I), with the
+// ProjectPointPinholeBackward, rendering/PointRendererHelper.h:317-372 (J_p_dis = I for a camera without distortion), with the
 // crop transform scaled by 0.5^layer (all five coefficients, rendering/RenderBackward.cu:1381-1385 and :3100-3106):
 // image-space gradient (gxp, gyp) of layer l -> gradients of the point, the pose tangent and fx, fy, cx, cy, s.
 // J_point = R, J_p_div = [1/z 0 -x/z^2; 0 1/z -y/z^2].
@@ -371,6 +425,7 @@ inline PointGrad project_point_backward(const Prepared& cam, const vetrast_view&
     for (int k = 0; k < 3; ++k) o.gp[k] = 0.f;
     for (int k = 0; k < 6; ++k) o.gpose[k] = 0.0;
     for (int k = 0; k < 5; ++k) o.gk[k] = 0.f;
+    for (int k = 0; k < 8; ++k) o.gdis[k] = 0.f;
     const float scale = powf(0.5f, float(l));
     const float cfx = v.crop_transform[0] * scale, cfy = v.crop_transform[1] * scale, cs = v.crop_transform[4] * scale;
     const float px = p4[0], py = p4[1], pz = p4[2];
@@ -383,8 +438,19 @@ inline PointGrad project_point_backward(const Prepared& cam, const vetrast_view&
         const float br = v.crop_rotation[1] * gxp + v.crop_rotation[3] * gyp;
         const float a2 = cfx * ar;  // J_p_K2^T
         const float b2 = cs * ar + cfy * br;
-        const float d0 = cam.fx * a2;  // J_p_K1^T
-        const float d1 = cam.s * a2 + cam.fy * b2;
+        float d0 = cam.fx * a2;  // J_p_K1^T
+        float d1 = cam.s * a2 + cam.fy * b2;
+        float nx = vx / vz, ny = vy / vz;  // the point K is applied to
+        if (cam.has_dist)
+        {
+            // J_dis_dis^T and J_p_dis^T (rendering/PointRendererHelper.h:346-368)
+            float J[4], Jd[16], xd, yd;
+            distort(cam.dist, nx, ny, xd, yd, J, Jd);
+            for (int k = 0; k < 8; ++k) o.gdis[k] = Jd[2 * k] * d0 + Jd[2 * k + 1] * d1;
+            const float n0 = J[0] * d0 + J[2] * d1, n1 = J[1] * d0 + J[3] * d1;
+            d0 = n0, d1 = n1;
+            nx = xd, ny = yd;
+        }
         const float iz = 1.f / vz;
         const float e0 = iz * d0, e1 = iz * d1;
         const float e2 = (-vx * iz * iz) * d0 + (-vy * iz * iz) * d1;
@@ -400,7 +466,6 @@ inline PointGrad project_point_backward(const Prepared& cam, const vetrast_view&
         o.gpose[4] = vz * e0 - vx * e2;
         o.gpose[5] = vx * e1 - vy * e0;
         // J_k_K1^T grad_p_k2: image = (fx*nx + s*ny + cx, fy*ny + cy), columns fx, fy, cx, cy, s
-        const float nx = vx / vz, ny = vy / vz;
         o.gk[0] = nx * a2;
         o.gk[1] = ny * b2;
         o.gk[2] = a2;
@@ -441,7 +506,15 @@ inline void scatter_point_grad(const vetrast_backward_args* g, const vetrast_vie
         gk[4] *= 0;
         for (int k = 0; k < 5; ++k)
             atomic_add(&g->grad_intrinsics[13 * (size_t)v.camera_index + k], k_factor * gk[k], par);
-        // the eight distortion columns need saiga's distortion Jacobian: left at zero
+        // the eight distortion columns, scaled as rendering/RenderBackward.cu:1438-1455 scales them (zero for a camera
+        // without distortion)
+        if (g->fwd.params.allow_distortion)
+        {
+            const float w8[8] = {1.f, 1.f, 0.25f, 0.1f, 0.1f, 0.1f, 0.1f, 0.1f};
+            for (int k = 0; k < 8; ++k)
+                atomic_add(&g->grad_intrinsics[13 * (size_t)v.camera_index + 5 + k],
+                           g->fwd.params.distortion_gradient_factor * (pg.gdis[k] * w8[k]), par);
+        }
         atomic_add(&g->grad_intrinsics_count[v.camera_index], 1.f / 1024.f, par);
     }
 }
@@ -649,9 +722,13 @@ void fuzzy_pixel_value_gradients(const vetrast_backward_args* g, int N, int C, c
 
 }  // namespace
 
+// out26: rotation rows with the translation in the fourth column (12), fx fy cx cy s (5), the eight distortion
+// coefficients, and 1 if any of them is not zero
 extern "C" int vetref_prepare_view(const double* pose8, const float* intrinsics13, float* out17)
 {
     Prepared p = prepare(pose8, intrinsics13);
+    for (int k = 0; k < 8; ++k) out17[17 + k] = p.dist[k];
+    out17[25] = p.has_dist ? 1.f : 0.f;
     for (int r = 0; r < 3; ++r)
     {
         for (int c = 0; c < 3; ++c) out17[4 * r + c] = p.r[3 * r + c];
@@ -678,6 +755,8 @@ extern "C" int vetref_project_point(const float* m, const vetrast_view* view, co
     p.cx = m[14];
     p.cy = m[15];
     p.s  = m[16];
+    for (int k = 0; k < 8; ++k) p.dist[k] = m[17 + k];
+    p.has_dist = m[25] != 0.f;
     Projected o;
     if (!project(p, *view, position4, o)) return 0;
     ip_z_r[0] = o.ipx;

@@ -30,7 +30,7 @@ def test_library_exports_every_declared_symbol():
 def test_struct_sizes_are_the_c_ones():
     # sizes the C compiler gives the structs of include/vetrast.h (LP64)
     assert C.sizeof(abi.View) == 5 * 4 + 9 * 4
-    assert C.sizeof(abi.Params) == 21 * 4 + abi.MAX_LAYERS * 4
+    assert C.sizeof(abi.Params) == 21 * 4 + abi.MAX_LAYERS * 4 + 2 * 4
     assert C.sizeof(abi.LiftArgs) == 8 + 4 * 8 + 2 * 4 + 2 * 8 + C.sizeof(abi.View) + 8 + 4 * 4 + 2 * 8 == 160
     assert abi.LiftArgs.loss_image.offset % 8 == 0
     assert C.sizeof(abi.ForwardArgs) % 8 == 0
@@ -109,13 +109,13 @@ def test_workspace_layout_is_aligned_and_disjoint():
         ("log_cursor", lay.log_cursor_base, B * 256 * 64),
         # rooms of 1024 records where at most 512 are expected per bin (layer 0: 2 M points over 8100 tiles), 2048 elsewhere
         ("primary", lay.primary_base, (tiles[0] * 1024 + (tiles[1] + 4 * tiles[2] + 16 * tiles[3]) * 2048) * 8),
-        ("views", lay.views_base, B * 128),
+        ("views", lay.views_base, B * 160),
     ]
     # the scratch of the backward call lies on top of the overflow log, which only lives inside a forward call
     forward_tail = [("log", lay.log_base, log_records * 16), ("slots", lay.slots_base, log_records * 4)]
     backward_tail = [("partial", lay.partial_base, N * L * 32),
                      ("background_partial", lay.background_partial_base, (P + 255) // 256 * 32),
-                     ("camera_partial", lay.camera_partial_base, (N + 255) // 256 * 96)]
+                     ("camera_partial", lay.camera_partial_base, (N + 255) // 256 * 160)]
     head_end = max(b + sz for _, b, sz in regions)
     for tail in (forward_tail, backward_tail):
         assert min(b for _, b, _ in tail) >= head_end

@@ -24,7 +24,7 @@ def _run_both(rasterizer, oracle, mn, ln, view, poses, intr, img, border=abi.LIF
     ws = rasterizer.lift_error(dev[0], dev[1], dev[2], dev[3], view, dev[4], dev[5], dev[6], border_pixels=border)
     torch.cuda.synchronize()
     assert rasterizer.lift_flags(ws) == 0
-    queued = int(ws[128:132].view(torch.int32).item())
+    queued = int(ws[abi.LIFT_QUEUE_LENGTH_OFFSET:abi.LIFT_QUEUE_LENGTH_OFFSET + 4].view(torch.int32).item())
     return dev[2].cpu().numpy(), dev[3].cpu().numpy(), want_v, want_c, queued
 
 

@@ -1,0 +1,209 @@
+"""Pins the oracle's opt-in lens distortion (vetrast_params.allow_distortion).
+
+The reference distorts the normalised image point with saiga's distortNormalizedPoint
+(src/lib/rendering/PointRendererHelper.h:207,348), which is not in its source tree, and holds no test or vector for it:
+PARITY WITH THE REFERENCE IS UNPINNED for cameras with non-zero coefficients. What is pinned here is that the oracle
+implements the published 8-coefficient rational model that the coefficient layout k1 k2 k3 k4 k5 k6 p1 p2
+(src/lib/data/SceneData.cpp:464-478) implies: against a float64 statement of that model, closed-form special cases,
+and central differences for every gradient the distortion touches (point, pose, K, the eight coefficients with the
+scaling of src/lib/rendering/RenderBackward.cu:1438-1455).
+"""
+import numpy as np
+import pytest
+from scipy.spatial.transform import Rotation
+
+from tests.test_oracle_pinning import lists_of
+from vet_amd import abi, synthetic
+from vet_amd.rasterizer import make_params
+
+
+def distort64(d, n):
+    """OpenCV's rational model (k1 k2 k3 k4 k5 k6 p1 p2) on a normalised point, float64."""
+    k1, k2, k3, k4, k5, k6, p1, p2 = [float(v) for v in d]
+    x, y = float(n[0]), float(n[1])
+    r2 = x * x + y * y
+    rad = (1 + k1 * r2 + k2 * r2 ** 2 + k3 * r2 ** 3) / (1 + k4 * r2 + k5 * r2 ** 2 + k6 * r2 ** 3)
+    return np.array([x * rad + 2 * p1 * x * y + p2 * (r2 + 2 * x * x), y * rad + p1 * (r2 + 2 * y * y) + 2 * p2 * x * y])
+
+
+def project64_distorted(p, R, t, K5, d8, crop5, rot4, w, h):
+    v = R @ np.asarray(p[:3], dtype=np.float64) + t
+    n = distort64(d8, v[:2] / v[2])
+    u = K5[0] * n[0] + K5[4] * n[1] + K5[2]
+    vv = K5[1] * n[1] + K5[3]
+    x = crop5[0] * u + crop5[4] * vv + crop5[2]
+    y = crop5[1] * vv + crop5[3]
+    c = np.array([w // 2, h // 2], dtype=np.float64)
+    M = np.array([[rot4[0], rot4[1]], [rot4[2], rot4[3]]], dtype=np.float64)
+    return M @ (np.array([x, y]) - c) + c, v[2]
+
+
+def _coefficients(rng, scale=1.0):
+    return (np.array([0.12, -0.03, 0.004, 0.05, -0.01, 0.002, 0.004, -0.003]) * rng.uniform(0.5, 1.5, 8) * scale).astype(np.float32)
+
+
+def _view(rng):
+    view = abi.View()
+    view.w, view.h = 640, 480
+    ang = rng.normal() * 0.3
+    crop = [0.5 + rng.random(), 0.5 + rng.random(), rng.normal() * 20, rng.normal() * 20, rng.normal() * 0.1]
+    rot = [np.cos(ang), -np.sin(ang), np.sin(ang), np.cos(ang)]
+    view.crop_transform = (abi.C.c_float * 5)(*crop)
+    view.crop_rotation = (abi.C.c_float * 4)(*rot)
+    return view, np.array(crop, np.float32).astype(np.float64), np.array(rot, np.float32).astype(np.float64)
+
+
+def test_projection_matches_the_rational_model_in_float64(oracle):
+    rng = np.random.default_rng(41)
+    checked = 0
+    for trial in range(600):
+        q = rng.normal(size=4)
+        q /= np.linalg.norm(q)
+        pose = np.concatenate([q, rng.normal(size=3), [0.0]])
+        k = np.zeros(13, np.float32)
+        k[:5] = [400 + 300 * rng.random(), 400 + 300 * rng.random(), 300 + 50 * rng.random(), 200 + 50 * rng.random(), rng.normal() * 2]
+        k[5:] = _coefficients(rng)
+        view, crop, rot = _view(rng)
+        p = np.array([*rng.normal(size=3) * 2, 0.05], dtype=np.float32)
+        m = oracle.prepare_view(pose, k)
+        assert m[25] == 1 and np.array_equal(m[17:25], k[5:])
+        ok, got = oracle.project_point(m, view, p)
+        R = Rotation.from_quat(q).as_matrix()
+        ip, z = project64_distorted(p.astype(np.float64), R, pose[4:7], k[:5].astype(np.float64), k[5:].astype(np.float64), crop, rot, 640, 480)
+        assert ok == (z > 0)
+        n = (R @ p[:3].astype(np.float64) + pose[4:7])[:2] / z
+        if not ok or z < 0.05 or n @ n > 4.0:  # far outside any image the polynomial blows up the float32 error
+            continue
+        scale = max(1.0, abs(ip[0]), abs(ip[1]))
+        assert max(abs(got[0] - ip[0]), abs(got[1] - ip[1])) / scale * min(z, 1.0) < 3e-4
+        checked += 1
+    assert checked > 100
+
+
+def test_special_cases_in_closed_form(oracle):
+    """Zero coefficients: the bits of the path without distortion. k1 alone: x' = x (1 + k1 r^2). p1 alone:
+    x' = x + 2 p1 x y, y' = y + p1 (r^2 + 2 y^2). Identity pose, K = identity, so the image point IS the distorted one."""
+    pose = np.array([0, 0, 0, 1, 0, 0, 0, 0], dtype=np.float64)
+    view = abi.View()
+    view.w, view.h = 8, 8
+    view.crop_transform = (abi.C.c_float * 5)(1, 1, 0, 0, 0)
+    view.crop_rotation = (abi.C.c_float * 4)(1, 0, 0, 1)
+    k = np.zeros(13, np.float32)
+    k[:2] = 1.0
+    plain = oracle.prepare_view(pose, k)
+    p = np.array([0.5, -0.25, 2.0, 0.01], np.float32)  # normalised (0.25, -0.125), r^2 = 0.078125
+    _, base = oracle.project_point(plain, view, p)
+    # the point sits at (4, 4) + its normalised position after the rotation about the image centre: identity here
+    assert base[0] == 0.25 and base[1] == -0.125
+    forced = plain.copy()
+    forced[25] = 1.0  # distortion code path with all coefficients zero
+    _, same = oracle.project_point(forced, view, p)
+    np.testing.assert_array_equal(same, base)
+    k1 = k.copy()
+    k1[5] = 0.5
+    _, got = oracle.project_point(oracle.prepare_view(pose, k1), view, p)
+    np.testing.assert_allclose(got[:2], np.array([0.25, -0.125]) * (1 + 0.5 * 0.078125), rtol=1e-7)
+    p1 = k.copy()
+    p1[11] = 0.25
+    _, got = oracle.project_point(oracle.prepare_view(pose, p1), view, p)
+    np.testing.assert_allclose(got[:2], [0.25 + 2 * 0.25 * 0.25 * -0.125, -0.125 + 0.25 * (0.078125 + 2 * 0.015625)], rtol=1e-7)
+    k4 = k.copy()
+    k4[8] = 0.5  # denominator: x' = x / (1 + k4 r^2)
+    _, got = oracle.project_point(oracle.prepare_view(pose, k4), view, p)
+    np.testing.assert_allclose(got[:2], np.array([0.25, -0.125]) / (1 + 0.5 * 0.078125), rtol=3e-7)  # a reciprocal and a product
+
+
+def test_distorted_cameras_are_refused_unless_allowed(oracle):
+    scene = synthetic.tiny_scene(num_points=300, seed=42)
+    scene.intrinsics[0, 6] = 0.01
+    with pytest.raises(abi.VetrastError) as e:
+        oracle.forward(scene)
+    assert e.value.status == abi.ERR_BAD_INPUT_DATA
+    assert oracle.forward(scene, allow_distortion=1).status == 0
+
+
+def test_distortion_moves_the_fragments(oracle):
+    scene = synthetic.tiny_scene(num_points=2000, K=8, seed=43)
+    plain = oracle.forward(scene)
+    scene.intrinsics[0, 5:] = [0.3, -0.05, 0.0, 0.0, 0.0, 0.0, 0.01, -0.01]
+    bent = oracle.forward(scene, allow_distortion=1)
+    assert not np.array_equal(plain.offsets, bent.offsets)
+
+
+def test_gradients_match_central_differences(oracle):
+    """Point, pose, K and distortion gradients = sum over fragments of J^T dR/dp with J the central-difference
+    Jacobian of the float64 distorted projection; the eight distortion columns carry the reference's weights
+    (1, 1, 0.25, 0.1, 0.1, 0.1, 0.1, 0.1) x distortion_gradient_factor."""
+    scene = synthetic.tiny_scene(num_points=500, w=24, h=16, num_layers=2, K=3, seed=44)
+    ang = -0.15
+    scene.views[0].crop_transform = (1.05, 0.95, 0.5, 1.0, 0.02)
+    scene.views[0].crop_rotation = (np.cos(ang), -np.sin(ang), np.sin(ang), np.cos(ang))
+    scene.intrinsics[0, 4] = 0.2
+    scene.intrinsics[0, 5:] = [0.15, -0.04, 0.006, 0.05, -0.012, 0.002, 0.004, -0.003]
+    q = np.array([0.03, 0.04, -0.02, 1.0])
+    scene.poses_se3[0, :4] = q / np.linalg.norm(q)
+    factor = 0.25
+    params = make_params(scene, need_point_gradient=1, K_gradient_factor=0.5, allow_distortion=1,
+                         distortion_gradient_factor=factor)
+    f = oracle.forward(scene, params)
+    go = scene.grad_out()
+    g = oracle.backward(f, go, want_cameras=True)
+    lists = lists_of(f)
+    tex = scene.texture.astype(np.float64)
+    v = scene.views[0]
+    crop = np.array(v.crop_transform, np.float32).astype(np.float64)
+    rot = np.array(v.crop_rotation, np.float32).astype(np.float64)
+    K5 = scene.intrinsics[0, :5].astype(np.float64)
+    D8 = scene.intrinsics[0, 5:].astype(np.float64)
+    R0 = Rotation.from_quat(scene.poses_se3[0, :4]).as_matrix()
+    t0 = scene.poses_se3[0, 4:7].copy()
+    proj = lambda p, R=R0, t=t0, K=K5, D=D8: project64_distorted(p, R, t, K, D, crop, rot, v.w, v.h)[0]
+    want_points = np.zeros((scene.num_points, 3))
+    want_pose, want_k, want_d, n_frag = np.zeros(6), np.zeros(5), np.zeros(8), 0
+    Cn, eps = scene.num_channels, 1e-6
+    for (l, x, y), ids in lists.items():
+        w, h = f.sizes[l]
+        if min(x, y, w - 1 - x, h - 1 - y) <= 2:
+            continue
+        I, G = f.out[l][0].astype(np.float64), go[l][0].astype(np.float64)
+        for i in ids:
+            t = tex[:, i]
+            dx = 0.5 * (-(t - I[:, y, x - 1]) * G[:, y, x - 1] + (t - I[:, y, x + 1]) * G[:, y, x + 1]).sum() / Cn
+            dy = 0.5 * (-(t - I[:, y - 1, x]) * G[:, y - 1, x] + (t - I[:, y + 1, x]) * G[:, y + 1, x]).sum() / Cn
+            grad = (0.5 ** l) * np.array([dx, dy])
+            p = scene.position[i].astype(np.float64)
+            for k in range(3):
+                e = np.zeros(4)
+                e[k] = eps
+                want_points[i, k] += grad @ ((proj(p + e) - proj(p - e)) / (2 * eps))
+            for k in range(6):
+                ips = []
+                for sgn in (+1, -1):
+                    xi = np.zeros(6)
+                    xi[k] = sgn * eps
+                    Rw = Rotation.from_rotvec(xi[3:]).as_matrix()
+                    ips.append(proj(p, Rw @ R0, Rw @ t0 + xi[:3]))
+                want_pose[k] += grad @ ((ips[0] - ips[1]) / (2 * eps))
+            for k in range(4):
+                Kp, Km = K5.copy(), K5.copy()
+                Kp[k] += 1e-4
+                Km[k] -= 1e-4
+                want_k[k] += 0.5 * (grad @ ((proj(p, K=Kp) - proj(p, K=Km)) / 2e-4))
+            for k in range(8):
+                Dp, Dm = D8.copy(), D8.copy()
+                Dp[k] += 1e-5
+                Dm[k] -= 1e-5
+                want_d[k] += grad @ ((proj(p, D=Dp) - proj(p, D=Dm)) / 2e-5)
+            n_frag += 1
+    assert n_frag > 100
+    want_d *= factor * np.array([1, 1, 0.25, 0.1, 0.1, 0.1, 0.1, 0.1])
+    np.testing.assert_allclose(g["points"][:, :3], want_points, rtol=3e-3, atol=3e-4 * np.abs(want_points).max())
+    np.testing.assert_allclose(g["pose"][0], want_pose, rtol=3e-3, atol=3e-4 * np.abs(want_pose).max())
+    np.testing.assert_allclose(g["intrinsics"][0, :5], want_k, rtol=3e-3, atol=3e-4 * np.abs(want_k).max())
+    np.testing.assert_allclose(g["intrinsics"][0, 5:], want_d, rtol=3e-3, atol=3e-4 * np.abs(want_d).max())
+    assert np.abs(want_d).min() > 0
+    # without the switch the same zero-distortion scene leaves the eight columns at zero
+    scene.intrinsics[0, 5:] = 0
+    f0 = oracle.forward(scene, make_params(scene, need_point_gradient=1))
+    g0 = oracle.backward(f0, go, want_cameras=True)
+    assert np.all(g0["intrinsics"][0, 5:] == 0)

@@ -35,7 +35,7 @@ def _both(rasterizer, scene, mn, ln, img):
     ret = rasterizer.lift_error(d_mn, d_ln, got_v, got_c, scene.views[0], d_pose, d_intr, d_img, static_scratch=True)
     assert ret is None and torch.cuda.memory_allocated() == before
     torch.cuda.synchronize()
-    queued = int(ws[128:132].view(torch.int32).item())
+    queued = int(ws[abi.LIFT_QUEUE_LENGTH_OFFSET:abi.LIFT_QUEUE_LENGTH_OFFSET + 4].view(torch.int32).item())
     return got_v.cpu().numpy(), got_c.cpu().numpy(), want_v.cpu().numpy(), want_c.cpu().numpy(), c0, queued
 
 

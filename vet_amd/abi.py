@@ -64,6 +64,8 @@ class Params(C.Structure):
         ("texture_abs", C.c_int32),
         ("depth_accept_blend", C.c_float),
         ("expected_fragments", C.c_float * MAX_LAYERS),
+        ("allow_distortion", C.c_int32),
+        ("distortion_gradient_factor", C.c_float),
     ]
 
 
@@ -115,6 +117,7 @@ class AdamArgs(C.Structure):
 
 LIFT_BORDER_PIXELS = 32
 LIFT_FLAGS_OFFSET = 192
+LIFT_QUEUE_LENGTH_OFFSET = 176
 LIFT_STATIC_MAX_CELLS = 1 << 19
 
 

@@ -800,7 +800,8 @@ __device__ __forceinline__ float sign_of(float x)
     return x > 0.f ? 1.f : (x < 0.f ? -1.f : 0.f);  // torch's abs backward: grad * sign(x)
 }
 
-constexpr int kCameraRow = 12;  // doubles per workgroup row: 6 pose tangent, fx, fy, cx, cy, fragment count, pad
+constexpr int kCameraRow  = 20;  // doubles per workgroup row: 6 pose tangent, fx, fy, cx, cy, 8 distortion, fragment count, pad
+constexpr int kCameraSums = 18;  // of them sums of per-fragment terms
 
 // One thread per point: find the pixel the point fell into in every layer (the same projection as the scatter pass), decide
 // whether its fragment survived the top-K cut (its key is not larger than the K-th key of that pixel's sorted list), and
@@ -808,7 +809,7 @@ constexpr int kCameraRow = 12;  // doubles per workgroup row: 6 pose tangent, fx
 // descriptor and confidence sums are added with atomics (onto rows the host zero-filled).
 // HITS = 4 (BILINEAR_BLEND): a point has up to four fragments per layer, one per corner of its 2x2 pixels, with records
 // at partial[layer][corner][point].
-template <int C, int HITS>
+template <int C, int HITS, bool DISTORT = false>
 __global__ void __launch_bounds__(kBlock) gather_point_gradients_kernel(GatherPass a)
 {
     const int i      = blockIdx.x * blockDim.x + threadIdx.x;
@@ -818,9 +819,11 @@ __global__ void __launch_bounds__(kBlock) gather_point_gradients_kernel(GatherPa
     for (int ci = 0; ci < C; ++ci) gt[ci] = 0.f;
     float gc = 0.f, gx = 0.f, gy = 0.f, gz = 0.f, cnt = 0.f;
     bool hit = false;   // the point has a blended fragment in this view
-    float cam_sum[10];  // pose tangent (translation, rotation), fx, fy, cx, cy
+    // pose tangent (translation, rotation), fx, fy, cx, cy and, in the kernel for cameras with distortion, k1 .. p2
+    constexpr int kSums = DISTORT ? kCameraSums : 10;
+    float cam_sum[kSums];
 #pragma unroll
-    for (int k = 0; k < 10; ++k) cam_sum[k] = 0.f;
+    for (int k = 0; k < kSums; ++k) cam_sum[k] = 0.f;
     Projected p;
     const DeviceView& cam = *a.vp.view;
     const float4 wp       = alive ? a.vp.position[i] : make_float4(0.f, 0.f, 0.f, 0.f);
@@ -874,8 +877,23 @@ __global__ void __launch_bounds__(kBlock) gather_point_gradients_kernel(GatherPa
                 const float br = cam.rot[1] * gxp + cam.rot[3] * gyp;
                 const float a2 = cfx * ar;
                 const float b2 = cs * ar + cfy * br;
-                const float d0 = cam.fx * a2;
-                const float d1 = cam.s * a2 + cam.fy * b2;
+                float d0 = cam.fx * a2;
+                float d1 = cam.s * a2 + cam.fy * b2;
+                float nx = vx / vz, ny = vy / vz;  // the point K is applied to
+                if constexpr (DISTORT)
+                {
+                    if (cam.has_dist)
+                    {
+                        // J_dis_dis^T and J_p_dis^T of the distortion (src/lib/rendering/PointRendererHelper.h:346-368)
+                        float J[4], Jd[16], xd, yd;
+                        distort_point_jacobians(cam.dist, nx, ny, xd, yd, J, Jd);
+#pragma unroll
+                        for (int k = 0; k < 8; ++k) cam_sum[10 + k] += Jd[2 * k] * d0 + Jd[2 * k + 1] * d1;
+                        const float n0 = J[0] * d0 + J[2] * d1, n1 = J[1] * d0 + J[3] * d1;
+                        d0 = n0, d1 = n1;
+                        nx = xd, ny = yd;
+                    }
+                }
                 const float iz = 1.f / vz;
                 const float e0 = iz * d0, e1 = iz * d1;
                 const float e2 = (-vx * iz * iz) * d0 + (-vy * iz * iz) * d1;
@@ -894,8 +912,8 @@ __global__ void __launch_bounds__(kBlock) gather_point_gradients_kernel(GatherPa
                     cam_sum[3] += vy * e2 - vz * e1;
                     cam_sum[4] += vz * e0 - vx * e2;
                     cam_sum[5] += vx * e1 - vy * e0;
-                    cam_sum[6] += (vx / vz) * a2;
-                    cam_sum[7] += (vy / vz) * b2;
+                    cam_sum[6] += nx * a2;
+                    cam_sum[7] += ny * b2;
                     cam_sum[8] += a2;
                     cam_sum[9] += b2;
                 }
@@ -909,15 +927,15 @@ __global__ void __launch_bounds__(kBlock) gather_point_gradients_kernel(GatherPa
         __shared__ double cam_red[kBlock / kWave][kCameraRow];
         const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
 #pragma unroll
-        for (int k = 0; k < 11; ++k)
+        for (int k = 0; k <= kCameraSums; ++k)
         {
-            double v = (k < 10) ? (double)cam_sum[k] : (double)cnt;
+            double v = (k < kSums) ? (double)cam_sum[k < kSums ? k : 0] : (k == kCameraSums ? (double)cnt : 0.0);
 #pragma unroll
             for (int d = kWave / 2; d >= 1; d >>= 1) v += __shfl_xor(v, d, kWave);
             if (lane == 0) cam_red[wave][k] = v;
         }
         __syncthreads();
-        if (threadIdx.x < 11)
+        if (threadIdx.x <= kCameraSums)
             a.camera_partial[(size_t)blockIdx.x * kCameraRow + threadIdx.x] =
                 (cam_red[0][threadIdx.x] + cam_red[1][threadIdx.x]) + (cam_red[2][threadIdx.x] + cam_red[3][threadIdx.x]);
     }
@@ -1005,7 +1023,8 @@ __global__ void __launch_bounds__(kBlock) gather_point_gradients_kernel(GatherPa
 }
 
 // Adds the per-workgroup camera rows of one view to the pose row image_index (double) and the intrinsics row
-// camera_index (fx, fy, cx, cy times K_gradient_factor; skew and distortion columns stay zero), and the scaled fragment
+// camera_index (fx, fy, cx, cy times K_gradient_factor, the skew column stays zero; the distortion columns where
+// distortion is switched on), and the scaled fragment
 // count to both count arrays, as src/lib/rendering/RenderBackward.cu:1418-1459 does per fragment with atomics.
 __global__ void __launch_bounds__(kBlock) reduce_camera_kernel(const double* __restrict__ rows, int num_rows,
                                                                 int image_index, int camera_index, float k_factor,
@@ -1013,21 +1032,23 @@ __global__ void __launch_bounds__(kBlock) reduce_camera_kernel(const double* __r
                                                                 float* __restrict__ grad_pose_count,
                                                                 float* __restrict__ grad_intrinsics,
                                                                 float* __restrict__ grad_intrinsics_count,
-                                                                float pose_count_step)
+                                                                float pose_count_step, int with_distortion,
+                                                                float distortion_factor)
 {
+    constexpr int kTerms = kCameraSums + 1;
     __shared__ double red[kBlock / kWave][kCameraRow];
-    double acc[11];
+    double acc[kTerms];
 #pragma unroll
-    for (int k = 0; k < 11; ++k) acc[k] = 0.0;
+    for (int k = 0; k < kTerms; ++k) acc[k] = 0.0;
     for (int r = threadIdx.x; r < num_rows; r += kBlock)
     {
         const double* row = rows + (size_t)r * kCameraRow;
 #pragma unroll
-        for (int k = 0; k < 11; ++k) acc[k] += row[k];
+        for (int k = 0; k < kTerms; ++k) acc[k] += row[k];
     }
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
 #pragma unroll
-    for (int k = 0; k < 11; ++k)
+    for (int k = 0; k < kTerms; ++k)
     {
         double v = acc[k];
 #pragma unroll
@@ -1035,7 +1056,7 @@ __global__ void __launch_bounds__(kBlock) reduce_camera_kernel(const double* __r
         if (lane == 0) red[wave][k] = v;
     }
     __syncthreads();
-    if (threadIdx.x < 11)
+    if (threadIdx.x < kTerms)
     {
         const int k    = threadIdx.x;
         const double s = (red[0][k] + red[1][k]) + (red[2][k] + red[3][k]);
@@ -1047,6 +1068,15 @@ __global__ void __launch_bounds__(kBlock) reduce_camera_kernel(const double* __r
         {
             if (grad_intrinsics)
                 grad_intrinsics[13 * (size_t)camera_index + (k - 6)] += (float)((double)k_factor * s);
+        }
+        else if (k < kCameraSums)
+        {
+            // the distortion columns with the weights of src/lib/rendering/RenderBackward.cu:1440-1455:
+            // k3 x 0.25, k4..k6 and p1, p2 x 0.1, all x distortion_gradient_factor
+            const int c       = k - 10;
+            const double w8 = c < 2 ? 1.0 : c == 2 ? 0.25 : 0.1;
+            if (grad_intrinsics && with_distortion)
+                grad_intrinsics[13 * (size_t)camera_index + 5 + c] += (float)((double)distortion_factor * (s * w8));
         }
         else
         {

@@ -32,9 +32,11 @@ struct DeviceView
     float crop[5];            // fx, fy, cx, cy, s of the crop transform
     float rot[4];             // crop rotation r00 r01 r10 r11
     float ccx, ccy;           // (w/2, h/2) with integer halving
-    float pad[4];
+    float dist[8];            // k1 k2 k3 k4 k5 k6 p1 p2 of the rational distortion model; read only when has_dist
+    uint32_t has_dist;        // some coefficient is not zero and the caller has switched distortion on
+    float pad[3];
 };
-static_assert(sizeof(DeviceView) == 32 * 4, "DeviceView is 32 floats");
+static_assert(sizeof(DeviceView) == 40 * 4, "DeviceView is 40 floats");
 
 // Pixels are numbered tile by tile: every layer is cut into 16x16 pixel tiles (the last column and row of tiles may
 // hang over the image), tiles are numbered row-major inside a layer and layer after layer, and pixel (x, y) of layer l is
@@ -144,9 +146,62 @@ struct Projected
     float ipx, ipy, z, radius;
 };
 
+// The 8-coefficient rational distortion model (k1 k2 k3 k4 k5 k6 p1 p2) on a normalised image point, every operation
+// rounded on its own so that the CPU check of the same formula agrees bit for bit. The reference calls saiga's
+// distortNormalizedPoint here (src/lib/rendering/PointRendererHelper.h:207), which is not in its source tree: this is
+// the published model its coefficient layout implies.
+__device__ __forceinline__ void distort_point(const float* d, float x, float y, float& xd, float& yd)
+{
+    const float x2 = x * x, y2 = y * y, r2 = x2 + y2, xy2 = (2.f * x) * y;
+    const float u   = 1.f + r2 * (d[0] + r2 * (d[1] + r2 * d[2]));
+    const float v   = 1.f + r2 * (d[3] + r2 * (d[4] + r2 * d[5]));
+    const float iv  = 1.f / v;
+    const float rad = u * iv;
+    const float tx = d[6] * xy2 + d[7] * (r2 + 2.f * x2);
+    const float ty = d[6] * (r2 + 2.f * y2) + d[7] * xy2;
+    xd = x * rad + tx;
+    yd = y * rad + ty;
+}
+
+// The same with its Jacobians: J = d(xd, yd) / d(x, y) row-major, Jd[2 k], Jd[2 k + 1] = d(xd, yd) / d coefficient k.
+__device__ __forceinline__ void distort_point_jacobians(const float* d, float x, float y, float& xd, float& yd,
+                                                        float (&J)[4], float (&Jd)[16])
+{
+    const float x2 = x * x, y2 = y * y, r2 = x2 + y2, xy2 = (2.f * x) * y;
+    const float u   = 1.f + r2 * (d[0] + r2 * (d[1] + r2 * d[2]));
+    const float v   = 1.f + r2 * (d[3] + r2 * (d[4] + r2 * d[5]));
+    const float iv  = 1.f / v;
+    const float rad = u * iv;
+    const float tx = d[6] * xy2 + d[7] * (r2 + 2.f * x2);
+    const float ty = d[6] * (r2 + 2.f * y2) + d[7] * xy2;
+    xd = x * rad + tx;
+    yd = y * rad + ty;
+    const float du   = d[0] + r2 * (2.f * d[1] + (3.f * d[2]) * r2);  // du / d r2
+    const float dv   = d[3] + r2 * (2.f * d[4] + (3.f * d[5]) * r2);
+    const float drad = (du * v - u * dv) * (iv * iv);                  // d rad / d r2
+    const float rx = drad * (2.f * x), ry = drad * (2.f * y);
+    J[0] = (rad + x * rx) + ((2.f * d[6]) * y + (6.f * d[7]) * x);
+    J[1] = x * ry + ((2.f * d[6]) * x + (2.f * d[7]) * y);
+    J[2] = y * rx + ((2.f * d[6]) * x + (2.f * d[7]) * y);
+    J[3] = (rad + y * ry) + ((6.f * d[6]) * y + (2.f * d[7]) * x);
+    const float r4 = r2 * r2, r6 = r4 * r2;
+    const float a = iv, b = -(u * (iv * iv));
+    const float c[6] = {a * r2, a * r4, a * r6, b * r2, b * r4, b * r6};
+#pragma unroll
+    for (int k = 0; k < 6; ++k)
+    {
+        Jd[2 * k]     = x * c[k];
+        Jd[2 * k + 1] = y * c[k];
+    }
+    Jd[12] = xy2;
+    Jd[13] = r2 + 2.f * y2;
+    Jd[14] = r2 + 2.f * x2;
+    Jd[15] = xy2;
+}
+
 // Projection of one point: rigid transform, clamp z, divide, K, crop transform, rotation about the crop centre.
 // Follows ProjPoint / ProjectPointPinhole / rotateCropAroundCenter (src/lib/rendering/RenderForward.cu:110-158,
-// src/lib/rendering/PointRendererHelper.h:184-218) for zero distortion. Every operation is rounded on its own
+// src/lib/rendering/PointRendererHelper.h:184-218). Every operation is rounded on its own
 // (the file is compiled with -ffp-contract=off) so that the CPU check of the same formula agrees bit for bit.
 __device__ __forceinline__ bool project_point(const DeviceView& c, const float4 p, Projected& o)
 {
@@ -155,8 +210,9 @@ __device__ __forceinline__ bool project_point(const DeviceView& c, const float4 
     const float vz = ((c.r[6] * p.x + c.r[7] * p.y) + c.r[8] * p.z) + c.t[2];
     const float z  = fmaxf(vz, 0.f);
     if (!(z > 0.f)) return false;
-    const float nx  = vx / vz;
-    const float ny  = vy / vz;
+    float nx = vx / vz;
+    float ny = vy / vz;
+    if (c.has_dist) distort_point(c.dist, nx, ny, nx, ny);
     const float u   = (c.fx * nx + c.s * ny) + c.cx;
     const float v   = c.fy * ny + c.cy;
     const float ipx = (c.crop[0] * u + c.crop[4] * v) + c.crop[2];

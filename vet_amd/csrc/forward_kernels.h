@@ -81,16 +81,22 @@ __device__ __forceinline__ DeviceView make_device_view(const ViewSource& s, cons
     v.cy   = in[3];
     v.s    = in[4];
     distorted = false;
-    for (int j = 5; j < 13; ++j) distorted |= (in[j] != 0.f);
+    for (int j = 5; j < 13; ++j)
+    {
+        distorted |= (in[j] != 0.f);
+        v.dist[j - 5] = in[j];
+    }
+    v.has_dist = distorted ? 1u : 0u;
     for (int j = 0; j < 5; ++j) v.crop[j] = s.crop[j];
     for (int j = 0; j < 4; ++j) v.rot[j] = s.rot[j];
     v.ccx = (float)(s.w / 2);
     v.ccy = (float)(s.h / 2);
-    for (int j = 0; j < 4; ++j) v.pad[j] = 0.f;
+    for (int j = 0; j < 3; ++j) v.pad[j] = 0.f;
     return v;
 }
 
-// One thread per view fills its camera constants; non-zero distortion coefficients raise flag bit 0.
+// One thread per view fills its camera constants; non-zero distortion coefficients raise flag bit 0 unless the caller
+// has switched distortion on.
 // Workgroups beyond the first zero the per-bin counters of all views (n4 uint4 elements).
 __global__ void __launch_bounds__(kBlock) prepare_views_kernel(PrepareViewsArgs args, int first_view, int num_views,
                                                                 const double* __restrict__ poses_se3,
@@ -99,7 +105,7 @@ __global__ void __launch_bounds__(kBlock) prepare_views_kernel(PrepareViewsArgs 
                                                                 uint32_t* __restrict__ flags,
                                                                 uint4* __restrict__ counters4, size_t n4,
                                                                 const float* __restrict__ background, int channels,
-                                                                int texture_abs)
+                                                                int texture_abs, int allow_distortion)
 {
     if (blockIdx.x > 0)
     {
@@ -123,8 +129,12 @@ __global__ void __launch_bounds__(kBlock) prepare_views_kernel(PrepareViewsArgs 
     }
     if (k >= num_views) return;
     bool distorted = false;
-    const DeviceView v = make_device_view(args.src[k], poses_se3, intrinsics, distorted);
-    if (distorted) atomicOr(flags, 1u);
+    DeviceView v = make_device_view(args.src[k], poses_se3, intrinsics, distorted);
+    if (distorted && !allow_distortion)
+    {
+        atomicOr(flags, 1u);  // refused: the call renders the camera without distortion and says so
+        v.has_dist = 0u;
+    }
     views[first_view + k] = v;
 }
 

@@ -13,7 +13,9 @@ namespace vetrast
 {
 constexpr int kLiftWaveLimit = 4096;  // pixels a single wave rasterizes by itself: 64 rounds
 constexpr int kLiftChunk     = 4096;  // pixels per workgroup step of the shared path: 16 per thread
-constexpr int kLiftHeader    = 256;   // bytes in front of the queue: DeviceView (128), queue length (4)
+constexpr int kLiftHeader    = 256;   // bytes in front of the queue: DeviceView (160), queue length at 176, flag word at 192
+static_assert(sizeof(DeviceView) <= VETRAST_LIFT_QUEUE_LENGTH_OFFSET && VETRAST_LIFT_QUEUE_LENGTH_OFFSET + 4 <= VETRAST_LIFT_FLAGS_OFFSET,
+              "the header's three parts must not overlap");
 
 struct LiftPass
 {
@@ -40,6 +42,7 @@ __global__ void lift_prepare_kernel(ViewSource src, const double* __restrict__ p
     if (blockIdx.x != 0 || threadIdx.x != 0) return;
     bool distorted = false;
     *view          = make_device_view(src, poses_se3, intrinsics, distorted);
+    view->has_dist = 0u;  // cameras with distortion are refused here (the flag below)
     *queue_length  = 0u;
     *flags         = distorted ? 1u : 0u;
 }

@@ -6,6 +6,7 @@
 
 #include <cmath>
 #include <cstring>
+#include <type_traits>
 #include <mutex>
 #include <new>
 #include <vector>
@@ -383,7 +384,7 @@ void launch_lift(const vetrast_lift_args* a, char* ws, hipStream_t stream)
     lp.width        = a->width;
     lp.border       = a->border_pixels;
     lp.view         = reinterpret_cast<const DeviceView*>(ws);
-    lp.queue_length = reinterpret_cast<uint32_t*>(ws + sizeof(DeviceView));
+    lp.queue_length = reinterpret_cast<uint32_t*>(ws + VETRAST_LIFT_QUEUE_LENGTH_OFFSET);
     lp.queue        = reinterpret_cast<uint2*>(ws + kLiftHeader);
     lp.sums = reinterpret_cast<double*>(ws + kLiftHeader + align_up((size_t)a->num_cells * sizeof(uint2), kAlign));
     lp.starts = reinterpret_cast<unsigned long long*>(reinterpret_cast<char*>(lp.sums) +
@@ -610,7 +611,7 @@ int vetrast_forward(vetrast_ctx* ctx, const vetrast_forward_args* a, void* strea
             }
             hipLaunchKernelGGL(prepare_views_kernel, dim3(1 + (first == 0 ? zero_blocks : 0)), dim3(kBlock), 0, stream, pv,
                                first, cnt, a->poses_se3, a->intrinsics, views, flags, counters4, n4, a->background, C,
-                               p.texture_abs);
+                               p.texture_abs, p.allow_distortion);
         }
     }
 
@@ -907,22 +908,27 @@ int vetrast_backward(vetrast_ctx* ctx, const vetrast_backward_args* g, void* str
             gp.confidence_scale      = p.confidence_scale;
             gp.texture_abs           = p.texture_abs;
             const dim3 grid(grid_for(N)), blk(kBlock);
+            // cameras with distortion switched on take the variant that carries the distortion Jacobians
+            auto launch = [&](auto c_tag, auto hits_tag) {
+                constexpr int kC = decltype(c_tag)::value, kHits = decltype(hits_tag)::value;
+                if (p.allow_distortion)
+                    hipLaunchKernelGGL((gather_point_gradients_kernel<kC, kHits, true>), grid, blk, 0, stream, gp);
+                else
+                    hipLaunchKernelGGL((gather_point_gradients_kernel<kC, kHits, false>), grid, blk, 0, stream, gp);
+            };
+            auto with_channels = [&](auto hits_tag) {
+                switch (C)
+                {
+                    case 1: launch(std::integral_constant<int, 1>{}, hits_tag); break;
+                    case 2: launch(std::integral_constant<int, 2>{}, hits_tag); break;
+                    case 3: launch(std::integral_constant<int, 3>{}, hits_tag); break;
+                    default: launch(std::integral_constant<int, 4>{}, hits_tag); break;
+                }
+            };
             if (hits == 1)
-                switch (C)
-                {
-                    case 1: hipLaunchKernelGGL((gather_point_gradients_kernel<1, 1>), grid, blk, 0, stream, gp); break;
-                    case 2: hipLaunchKernelGGL((gather_point_gradients_kernel<2, 1>), grid, blk, 0, stream, gp); break;
-                    case 3: hipLaunchKernelGGL((gather_point_gradients_kernel<3, 1>), grid, blk, 0, stream, gp); break;
-                    default: hipLaunchKernelGGL((gather_point_gradients_kernel<4, 1>), grid, blk, 0, stream, gp); break;
-                }
+                with_channels(std::integral_constant<int, 1>{});
             else
-                switch (C)
-                {
-                    case 1: hipLaunchKernelGGL((gather_point_gradients_kernel<1, 4>), grid, blk, 0, stream, gp); break;
-                    case 2: hipLaunchKernelGGL((gather_point_gradients_kernel<2, 4>), grid, blk, 0, stream, gp); break;
-                    case 3: hipLaunchKernelGGL((gather_point_gradients_kernel<3, 4>), grid, blk, 0, stream, gp); break;
-                    default: hipLaunchKernelGGL((gather_point_gradients_kernel<4, 4>), grid, blk, 0, stream, gp); break;
-                }
+                with_channels(std::integral_constant<int, 4>{});
         }
         if (want_camera)
         {
@@ -930,7 +936,7 @@ int vetrast_backward(vetrast_ctx* ctx, const vetrast_backward_args* g, void* str
             hipLaunchKernelGGL(reduce_camera_kernel, dim3(1), dim3(kBlock), 0, stream, camera_rows, grid_for(N),
                                a->views[b].image_index, a->views[b].camera_index, p.K_gradient_factor, g->grad_pose,
                                g->grad_pose_count, g->grad_intrinsics, g->grad_intrinsics_count,
-                               hits == 1 ? 1.f / 1024.f : 1.f);
+                               hits == 1 ? 1.f / 1024.f : 1.f, p.allow_distortion, p.distortion_gradient_factor);
         }
         if (N == 0)
         {

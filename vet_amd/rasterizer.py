@@ -38,6 +38,8 @@ def make_params(scene: Scene, **overrides) -> abi.Params:
     p.confidence_scale = 10.0
     p.texture_abs = 0
     p.depth_accept_blend = 0.01
+    p.allow_distortion = 0
+    p.distortion_gradient_factor = 0.005
     for k, v in {**scene.params, **overrides}.items():
         if not hasattr(p, k):
             raise AttributeError(f"vetrast_params has no field {k}")

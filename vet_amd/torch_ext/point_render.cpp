@@ -48,6 +48,8 @@ vetrast_params to_abi_params(const RenderParams& p, int num_layers)
     q.quirk_background_confidence_leak = p.quirk_background_confidence_leak ? 1 : 0;
     q.point_gradient_normalization     = p.point_gradient_normalization;
     q.K_gradient_factor                = p.K_gradient_factor;
+    q.allow_distortion                 = p.allow_distortion ? 1 : 0;
+    q.distortion_gradient_factor       = p.distortion_gradient_factor;
     q.camera_gradient_normalization    = p.camera_gradient_normalization ? 1 : 0;
     q.confidence_activation            = p.fused_confidence_scale > 0.f ? 1 : 0;
     q.confidence_scale                 = p.fused_confidence_scale;
@@ -212,7 +214,7 @@ torch::autograd::variable_list PointRender::forward(torch::autograd::AutogradCon
     const int B = (int)info->images.size(), L = info->num_layers, C = (int)texture.size(0);
     const int64_t N = points.size(0);
     auto f32        = torch::TensorOptions().device(points.device()).dtype(torch::kFloat32);
-    info->cache->CheckIntrinsics(intrinsics);
+    if (!info->params.allow_distortion) info->cache->CheckIntrinsics(intrinsics);
 
     // dropout mask per view, PointRenderer.cu:461-468 (the mask is 1 where a point is dropped)
     torch::Tensor dropout;
@@ -881,6 +883,8 @@ std::vector<torch::Tensor> blend_point_cloud(torch::Tensor texture, torch::Tenso
             for (size_t l = 0; l < v.size() && l < (size_t)VETRAST_MAX_LAYERS; ++l) p.expected_fragments[l] = (float)v[l];
         }
         else if (k == "K_gradient_factor") p.K_gradient_factor = (float)as_d();
+        else if (k == "distortion_gradient_factor") p.distortion_gradient_factor = (float)as_d();
+        else if (k == "allow_distortion") p.allow_distortion = as_d() != 0.0;
         else if (k == "camera_gradient_normalization") p.camera_gradient_normalization = as_d() != 0;
         else if (k == "fused_confidence_scale") p.fused_confidence_scale = (float)as_d();
         else if (k == "fused_texture_abs") p.fused_texture_abs = as_d() != 0;

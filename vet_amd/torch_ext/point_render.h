@@ -28,6 +28,11 @@ struct RenderParams
     float dropout                      = 0.25f;
     float drop_out_radius_threshold    = 0.6f;
     float K_gradient_factor            = 0.5f;
+    float distortion_gradient_factor   = 0.005f;  // src/lib/data/Settings.h:54
+    // Not in the reference: cameras with non-zero distortion coefficients are refused unless this is set; with it they
+    // are rendered with the published 8-coefficient rational model (vetrast_params.allow_distortion; parity with
+    // saiga's distortNormalizedPoint unpinned, dist_cutoff not applied).
+    bool allow_distortion              = false;
     bool drop_out_points_by_radius     = true;
     int num_texture_channels           = -1;
     bool output_background_mask        = false;
