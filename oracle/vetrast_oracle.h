@@ -18,6 +18,11 @@
  *   projection        pinned by the reference's own host restatements of the pinhole model
  *                     (src/lib/data/SceneData.cpp:28-36,1020-1049) for zero distortion and by brute-force checks;
  *                     the bit pattern of saiga's TransformPoint / DivideByZ is PARITY UNPINNED (saiga is not vendored)
+ *   lens distortion   (params.allow_distortion) PARITY UNPINNED: the reference calls saiga's distortNormalizedPoint
+ *                     (rendering/PointRendererHelper.h:207,348), whose source is not in its tree, and holds no vector
+ *                     for it. The oracle states the published 8-coefficient rational model the coefficient layout
+ *                     implies; what pins THAT (a float64 statement, closed forms, central differences of every
+ *                     gradient) is in tests/test_oracle_distortion.py. dist_cutoff is not applied.
  *   count/scan/fill   pinned by brute force and by the reference's own invariant counters == counts
  *   sort              pinned against a generic sort of (depth, id) pairs; the id tie-break refines the reference's
  *                     depth-only order
