@@ -23,6 +23,16 @@ def _levels(scene, step=0.25, seed=5):
     return scene
 
 
+def _far(scene, depth=95000.0):
+    """Moves the points out along their viewing rays (the tiny scene's camera looks down z from z = -2)."""
+    z = scene.position[:, 2].astype(np.float64) + 2.0
+    scale = (z + depth) / z
+    scene.position[:, 0] = (scene.position[:, 0] * scale).astype(np.float32)
+    scene.position[:, 1] = (scene.position[:, 1] * scale).astype(np.float32)
+    scene.position[:, 2] = (z + depth - 2.0).astype(np.float32)
+    return scene
+
+
 def _scenes():
     yield "tiny_K4", synthetic.tiny_scene(), {}
     yield "tiny_levels_K8", _levels(synthetic.tiny_scene(num_points=6000, K=8, seed=81)), {}
@@ -33,6 +43,19 @@ def _scenes():
         {"use_environment_map": 1}
     yield "wide_depth_range", synthetic.tiny_scene(num_points=5000, K=12, seed=86), {"depth_accept_blend": 0.3}
     yield "odd_size_5_layers", _levels(synthetic.tiny_scene(num_points=9000, w=83, h=61, num_layers=5, K=6, seed=87)), {}
+    # a depth range that covers the nearest fragments from zero (they join the bucket that is open from the start,
+    # RenderBackward.cu:706-714), one that covers all fragments, and one that also covers the background element at
+    # depth 1e5 (the largest range the library takes is 1e4, so the points are moved out to 95 000); each with short
+    # lists and with lists too long for the kernel that lays fragments out densely
+    yield "range_reaches_zero_K8", synthetic.tiny_scene(num_points=3000, K=8, seed=90), {"depth_accept_blend": 2.0}
+    yield "range_reaches_zero_nocut", synthetic.tiny_scene(num_points=30000, K=-1, seed=91), {"depth_accept_blend": 2.0}
+    yield "one_bucket_K8", synthetic.tiny_scene(num_points=3000, K=8, seed=92), {"depth_accept_blend": 9.0e3}
+    yield "one_bucket_nocut", synthetic.tiny_scene(num_points=30000, K=-1, seed=93), {"depth_accept_blend": 9.0e3}
+    yield "background_in_last_bucket_K8", _far(synthetic.tiny_scene(num_points=3000, K=8, seed=95)), \
+        {"depth_accept_blend": 9.0e3}
+    yield "background_in_last_bucket_nocut", _far(synthetic.tiny_scene(num_points=30000, K=-1, seed=96)), \
+        {"depth_accept_blend": 9.0e3}
+    yield "single_fragments_K1", _levels(synthetic.tiny_scene(num_points=6000, K=1, seed=94)), {}
     yield "config1", synthetic.config1(), {"depth_accept_blend": 0.05}
     yield "config2_200k", synthetic.config2(num_points=200_000), {"depth_accept_blend": 0.05}
 

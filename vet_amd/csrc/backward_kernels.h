@@ -7,6 +7,8 @@
 // reference issues per fragment and channel (src/lib/rendering/RenderBackward.cu:1152,1157,1177,1405-1407), were the
 // single largest cost on MI355X; without them the gradients are also reproducible run to run.
 #pragma once
+#include <type_traits>
+
 #include "common.h"
 
 namespace vetrast
@@ -558,6 +560,9 @@ struct FuzzyWalk
             start    = i;
             first_id = id;
         }
+        // (the first element of a list joins the bucket that is open from the start when its depth is within the range
+        // of zero: it is that bucket's first element all the same)
+        if (m == 0) first_id = id;
         acc_conf += conf;
 #pragma unroll
         for (int ci = 0; ci < C; ++ci) acc_t[ci] += t[ci];
@@ -589,55 +594,373 @@ struct FuzzyWalk
     }
 };
 
+// Value the lane D places below (above) in the same row of 16 lanes holds; the lane's own value where the row has no
+// such lane. DPP register moves; every lane of the wave must be active.
+template <int D>
+__device__ __forceinline__ float row_below(float v)
+{
+    return __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(v), __float_as_int(v), 0x110 + D, 0xF, 0xF, false));
+}
+template <int D>
+__device__ __forceinline__ float row_above(float v)
+{
+    return __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(v), __float_as_int(v), 0x100 + D, 0xF, 0xF, false));
+}
+
+// What the FUZZY_BLEND backward kernels know about a pixel before they look at its fragments.
+struct FuzzyPixel
+{
+    uint32_t n, off;  // fragments after the cut, place of the first one
+    bool do_point;
+    float g[4], ax[4], ay[4], bx, by;  // upstream gradient; position heuristic in slope / offset form
+};
+
+template <int C>
+__device__ __forceinline__ FuzzyPixel fuzzy_pixel(const BackwardPass& a, const TilePixel& px)
+{
+    FuzzyPixel f;
+    f.n = f.off = 0, f.do_point = false, f.bx = f.by = 0.f;
+#pragma unroll
+    for (int ci = 0; ci < 4; ++ci) f.g[ci] = f.ax[ci] = f.ay[ci] = 0.f;
+    if (!px.active) return f;
+    const int l = px.l, lw = a.ly.w[l], lh = a.ly.h[l];
+    const size_t plane   = (size_t)lw * lh;
+    const uint32_t local = px.local;
+    const float* G       = a.grad_out[l];
+#pragma unroll
+    for (int ci = 0; ci < C; ++ci) f.g[ci] = G[ci * plane + local];
+    f.off = a.offsets[px.q];
+    f.n   = a.offsets[px.q + 1] - f.off;
+    if (a.K > 0) f.n = min(f.n, (uint32_t)a.K);
+    f.do_point = a.need_point_gradient && f.n > 0 && interior_pixel(px.x, px.y, lw, lh);
+    if (f.do_point)
+    {
+        // see blend_backward_kernel
+        const float* I = a.out[l];
+#pragma unroll
+        for (int ci = 0; ci < C; ++ci)
+        {
+            const float* Ic = I + ci * plane + local;
+            const float* Gc = G + ci * plane + local;
+            const float Ix0 = Ic[-1], Ix1 = Ic[1], Iy0 = Ic[-lw], Iy1 = Ic[lw];
+            const float Gx0 = Gc[-1], Gx1 = Gc[1], Gy0 = Gc[-lw], Gy1 = Gc[lw];
+            f.ax[ci] = 0.5f * (Gx1 - Gx0);
+            f.ay[ci] = 0.5f * (Gy1 - Gy0);
+            f.bx += 0.5f * (Ix0 * Gx0 - Ix1 * Gx1);
+            f.by += 0.5f * (Iy0 * Gy0 - Iy1 * Gy1);
+        }
+    }
+    return f;
+}
+
+// Lists of up to kFuzzyDense fragments are laid out densely, one lane per FRAGMENT, as in blend_backward_kernel; what is
+// different here is that a fragment's gradient depends on its whole bucket (means over the bucket's elements) and on
+// all buckets of its pixel (transmittance in front, bucket terms behind), so a pixel's fragments must sit in one step
+// of 64 lanes. Every pixel gets a slot of 1, 2, 4, 8 or 16 lanes (its list length rounded up to a power of two), the
+// slots are handed out largest first, which keeps each aligned to its own size: no slot crosses a row of 16 lanes,
+// the sums over a bucket, the transmittance product and the suffix sum of the bucket terms are shift-and-combine steps
+// inside a row (register moves), and steps need no carries between them. Only the bucket boundaries are a sequential
+// rule (a bucket starts where the depth leaves the range of the bucket's FIRST element), and that rule needs the
+// depths alone: all lanes of a slot run it together over the slot's depths. Sums and products are combined pairwise
+// instead of front to back, which moves the results by rounding only. The slots of a step are at most as long as its
+// first one, and the step's code is compiled once per slot length so that shorter slots take fewer combine steps.
+// Longer lists are left to blend_backward_fuzzy_walk_kernel; the workgroup says in column 7 of its background row
+// whether it has any.
+constexpr int kFuzzyDense     = 16;
+constexpr int kFuzzyWalkColumn = 7;
+
 template <int C>
 __global__ void __launch_bounds__(kBlock) blend_backward_fuzzy_kernel(BackwardPass a, float depth_accept)
 {
     constexpr int kWaves = kBlock / kWave;
-    __shared__ float red[kWaves][C + 1];
+    __shared__ uint32_t s_off[kWaves][kWave];
+    __shared__ uint16_t s_slot[kWaves][kWave];
+    __shared__ uint8_t s_n[kWaves][kWave];
+    __shared__ uint8_t s_point[kWaves][kWave];
+    __shared__ float4 s_g[kWaves][kWave];
+    __shared__ float4 s_ax[kWaves][kWave];
+    __shared__ float4 s_ay[kWaves][kWave];
+    __shared__ float2 s_bxy[kWaves][kWave];
+    __shared__ uint8_t s_item[kWaves][kWaveItems];
+    __shared__ float red[kWaves][C + 2];
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
     const TilePixel px = tile_pixel(a.tiles, a.ly);
-    const int l        = px.l;
-    FuzzyWalk<C> w;
-    w.a = &a, w.list = a.fragments, w.partial_l = a.partial + 2 * (size_t)l * a.N, w.n = 0, w.bx = w.by = 0.f;
-    w.do_point = false, w.depth_accept = depth_accept, w.total = w.prefix = 0.0;
+    float4* partial_l  = a.partial + 2 * (size_t)px.l * a.N;
+    const bool with_background = !a.use_environment_map;  // every list ends with the background element
+    float bg_grad[C];
 #pragma unroll
-    for (int ci = 0; ci < C; ++ci) w.g[ci] = w.ax[ci] = w.ay[ci] = w.bg_grad[ci] = 0.f;
-    bool with_background = false;  // the list ends with the background element
-
-    if (px.active)
+    for (int ci = 0; ci < C; ++ci) bg_grad[ci] = 0.f;
+    uint32_t n;
     {
-        const int lw = a.ly.w[l], lh = a.ly.h[l];
-        const size_t plane   = (size_t)lw * lh;
-        const uint32_t local = px.local;
-        const float* G       = a.grad_out[l];
+        const FuzzyPixel f = fuzzy_pixel<C>(a, px);
+        n                  = f.n;
+        // an empty list: the background is the only bucket, one element of confidence 1 with nothing in front of it
+        if (px.active && n == 0 && with_background)
 #pragma unroll
-        for (int ci = 0; ci < C; ++ci) w.g[ci] = G[ci * plane + local];
-        const uint32_t off = a.offsets[px.q];
-        uint32_t n         = a.offsets[px.q + 1] - off;
-        if (a.K > 0) n = min(n, (uint32_t)a.K);
-        w.n               = n;
-        w.list            = a.fragments + off;
-        with_background   = !a.use_environment_map;
-
-        // position heuristic of this pixel in slope / offset form (see blend_backward_kernel)
-        w.do_point = a.need_point_gradient && n > 0 && interior_pixel(px.x, px.y, lw, lh);
-        if (w.do_point)
+            for (int ci = 0; ci < C; ++ci) bg_grad[ci] = f.g[ci];
+        s_off[wave][lane]   = f.off;
+        s_point[wave][lane] = f.do_point ? 1 : 0;
+        s_g[wave][lane]     = make_float4(f.g[0], f.g[1], f.g[2], f.g[3]);
+        if (f.do_point)
         {
-            const float* I = a.out[l];
-#pragma unroll
-            for (int ci = 0; ci < C; ++ci)
-            {
-                const float* Ic = I + ci * plane + local;
-                const float* Gc = G + ci * plane + local;
-                const float Ix0 = Ic[-1], Ix1 = Ic[1], Iy0 = Ic[-lw], Iy1 = Ic[lw];
-                const float Gx0 = Gc[-1], Gx1 = Gc[1], Gy0 = Gc[-lw], Gy1 = Gc[lw];
-                w.ax[ci] = 0.5f * (Gx1 - Gx0);
-                w.ay[ci] = 0.5f * (Gy1 - Gy0);
-                w.bx += 0.5f * (Ix0 * Gx0 - Ix1 * Gx1);
-                w.by += 0.5f * (Iy0 * Gy0 - Iy1 * Gy1);
-            }
+            s_ax[wave][lane]  = make_float4(f.ax[0], f.ax[1], f.ax[2], f.ax[3]);
+            s_ay[wave][lane]  = make_float4(f.ay[0], f.ay[1], f.ay[2], f.ay[3]);
+            s_bxy[wave][lane] = make_float2(f.bx, f.by);
         }
     }
+    const bool dense = n > 0 && n <= (uint32_t)kFuzzyDense;
+    s_n[wave][lane]  = (uint8_t)(dense ? n : 0);
+
+    // ---- slots, largest first ---------------------------------------------------------------------------------------
+    const uint32_t size = dense ? (n > 1 ? 1u << (32 - __clz((int)n - 1)) : 1u) : 0u;
+    uint32_t slot = 0, total = 0;
+#pragma unroll
+    for (uint32_t cls = kFuzzyDense; cls >= 1; cls >>= 1)
+    {
+        const uint64_t members = __ballot(size == cls);
+        if (size == cls) slot = total + cls * (uint32_t)__popcll(members & ((1ull << lane) - 1ull));
+        total += cls * (uint32_t)__popcll(members);
+    }
+    s_slot[wave][lane] = (uint16_t)slot;
+    for (uint32_t j = 0; j < size; ++j) s_item[wave][slot + j] = j < n ? (uint8_t)lane : (uint8_t)255;
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+
+    // One step: 64 lanes, slots of at most BOUND lanes.
+    auto step = [&](uint32_t k0, auto bound_constant) {
+        constexpr uint32_t BOUND = decltype(bound_constant)::value;
+        const uint32_t k = k0 + lane;
+        const int p      = k < total ? (int)s_item[wave][k] : 255;
+        const bool item  = p != 255;
+        uint32_t np = 0, j = 0;
+        int first = lane;  // first lane of the slot
+        float depth = 0.f, conf = 0.f;
+        float t[4]  = {0.f, 0.f, 0.f, 0.f};
+        float g[4]  = {0.f, 0.f, 0.f, 0.f};
+        int id = -1;
+        if (item)
+        {
+            np    = s_n[wave][p];
+            j     = k - s_slot[wave][p];
+            first = lane - (int)j;
+            const uint64_t key = a.fragments[s_off[wave][p] + j];
+            depth              = __uint_as_float((uint32_t)(key >> 32));
+            const int point    = (int)(uint32_t)key;
+            int ti             = -1;
+            // guards the gathers; never false for a workspace the forward pass wrote. An element that fails them
+            // counts as a fragment with a zero descriptor and confidence and gets no record, as in the walk.
+            if ((uint32_t)point < (uint32_t)a.N) ti = a.index ? a.index[point] : point;
+            if ((uint32_t)ti < (uint32_t)a.N)
+            {
+                const float4 t4 = a.packed[2 * (size_t)ti];
+                conf            = a.packed[2 * (size_t)ti + 1].x;
+                t[0] = t4.x, t[1] = t4.y, t[2] = t4.z, t[3] = t4.w;
+                id = point;
+            }
+            const float4 g4 = s_g[wave][p];
+            g[0] = g4.x, g[1] = g4.y, g[2] = g4.z, g[3] = g4.w;
+        }
+        // bucket boundaries (src/lib/rendering/RenderBackward.cu:706-714): element 0 opens the first bucket whether or
+        // not it resets the range
+        float last_min = 0.f;
+        uint32_t heads = 1u;
+        if constexpr (BOUND > 1)
+        {
+            float d[BOUND];
+#pragma unroll
+            for (uint32_t i = 0; i < BOUND; ++i) d[i] = __shfl(depth, (first + (int)i) & (kWave - 1), kWave);
+#pragma unroll
+            for (uint32_t i = 0; i < BOUND; ++i)
+                if (i < np && !(d[i] - last_min < depth_accept))
+                {
+                    last_min = d[i];
+                    heads |= 1u << i;
+                }
+        }
+        else if (!(depth - last_min < depth_accept))
+            last_min = depth;
+        // The background (depth MAX_DEPTH_CONST = 1e5, src/lib/rendering/RenderConstants.h:30) is a bucket of its own
+        // unless the last bucket's range reaches that far: then it is one more element of that bucket.
+        const bool bg_joins = with_background && (100000.f - last_min < depth_accept);
+
+        const uint32_t head  = 31u - (uint32_t)__clz((int)(heads & ((2u << j) - 1u)));  // first element of this bucket
+        const uint32_t later = heads >> (j + 1u);
+        const uint32_t next  = later ? j + (uint32_t)__ffs((int)later) : np;  // first element of the next bucket
+        const uint32_t dist  = j - head;
+        const bool opens     = item && dist == 0u;
+        const bool in_last   = item && next == np;
+        const float inv      = 1.f / (float)(item ? next - head + (bg_joins && in_last ? 1u : 0u) : 1u);
+
+        // sums over the bucket: inclusive scan from the bucket's first lane, the last lane of the bucket has the sums
+        float sums[C + 1];
+        sums[C] = conf;
+#pragma unroll
+        for (int ci = 0; ci < C; ++ci) sums[ci] = t[ci];
+        if constexpr (BOUND > 1)
+        {
+            const int last_lane = item ? first + (int)next - 1 : lane;
+#pragma unroll
+            for (int v = 0; v <= C; ++v)
+            {
+                float x = sums[v], o;
+                o = row_below<1>(x); if (dist >= 1u) x += o;
+                if constexpr (BOUND > 2) { o = row_below<2>(x); if (dist >= 2u) x += o; }
+                if constexpr (BOUND > 4) { o = row_below<4>(x); if (dist >= 4u) x += o; }
+                if constexpr (BOUND > 8) { o = row_below<8>(x); if (dist >= 8u) x += o; }
+                sums[v] = __shfl(x, last_lane, kWave);
+            }
+        }
+        if (bg_joins && in_last)
+        {
+            sums[C] += 1.f;
+#pragma unroll
+            for (int ci = 0; ci < C; ++ci) sums[ci] += a.background[ci];
+        }
+        const float bconf = sums[C] * inv;
+        float dot = 0.f;
+#pragma unroll
+        for (int ci = 0; ci < C; ++ci) dot += (sums[ci] * inv) * g[ci];
+        // transmittance in front of the bucket: product of (1 - mean confidence) over the buckets before it
+        float P = opens ? 1.f - bconf : 1.f;
+        float A = 1.f, A_end = P;
+        if constexpr (BOUND > 1)
+        {
+            float o;
+            o = row_below<1>(P); if (j >= 1u) P *= o;
+            if constexpr (BOUND > 2) { o = row_below<2>(P); if (j >= 2u) P *= o; }
+            if constexpr (BOUND > 4) { o = row_below<4>(P); if (j >= 4u) P *= o; }
+            if constexpr (BOUND > 8) { o = row_below<8>(P); if (j >= 8u) P *= o; }
+            const float P_before = __shfl(P, (item && head > 0u) ? first + (int)head - 1 : lane, kWave);
+            A_end                = __shfl(P, item ? first + (int)np - 1 : lane, kWave);  // behind the last bucket
+            if (head > 0u) A = P_before;
+        }
+        // bucket terms behind this bucket (the background's included): suffix sum over the slot
+        float x = 0.f;
+#pragma unroll
+        for (int ci = 0; ci < C; ++ci) x += ((g[ci] * (sums[ci] * inv)) * A) * bconf;
+        float S = 0.f;
+        if constexpr (BOUND > 1)
+        {
+            float Q = opens ? x : 0.f, o;
+            o = row_above<1>(Q); if (j + 1u < np) Q += o;
+            if constexpr (BOUND > 2) { o = row_above<2>(Q); if (j + 2u < np) Q += o; }
+            if constexpr (BOUND > 4) { o = row_above<4>(Q); if (j + 4u < np) Q += o; }
+            if constexpr (BOUND > 8) { o = row_above<8>(Q); if (j + 8u < np) Q += o; }
+            const float Q_next = __shfl(Q, (item && next < np) ? first + (int)next : lane, kWave);
+            if (next < np) S = Q_next;
+        }
+        if (with_background && !bg_joins)
+        {
+            float xb = 0.f;
+#pragma unroll
+            for (int ci = 0; ci < C; ++ci) xb += ((g[ci] * a.background[ci]) * A_end) * 1.f;
+            S += xb;
+        }
+        if (with_background && item && j + 1u == np)
+        {
+            // the background's share: an element of the last bucket, or a bucket of its own behind all others
+            const float scale = bg_joins ? A * bconf : A_end * 1.f;
+            const float share = bg_joins ? inv : 1.f;
+#pragma unroll
+            for (int ci = 0; ci < C; ++ci) bg_grad[ci] += (scale * g[ci]) * share;
+        }
+        float4 rec_lo = make_float4(0.f, 0.f, 0.f, 0.f), rec_hi = rec_lo;
+        const bool give = item && id >= 0;
+        if (give)
+        {
+            const float gconf = (dot * A) * inv - S / ((1.f - bconf) + 1e-9f);
+            float gt[4]       = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int ci = 0; ci < C; ++ci) gt[ci] = ((A * bconf) * g[ci]) * inv;
+            float gp0 = 0.f, gp1 = 0.f;
+            if (s_point[wave][p] & 1)
+            {
+                // the position part of an element's record depends on its own descriptor, not on the bucket's
+                const float4 ax4 = s_ax[wave][p], ay4 = s_ay[wave][p];
+                const float2 b2  = s_bxy[wave][p];
+                const float ax[4] = {ax4.x, ax4.y, ax4.z, ax4.w}, ay[4] = {ay4.x, ay4.y, ay4.z, ay4.w};
+                float dR_dpx = b2.x, dR_dpy = b2.y;
+#pragma unroll
+                for (int ci = 0; ci < C; ++ci)
+                {
+                    dR_dpx += t[ci] * ax[ci];
+                    dR_dpy += t[ci] * ay[ci];
+                }
+                gp0 = dR_dpx / (float)C;
+                gp1 = dR_dpy / (float)C;
+            }
+            rec_lo = make_float4(gt[0], gt[1], gt[2], gt[3]);
+            rec_hi = make_float4(gconf, gp0, gp1, 0.f);
+        }
+        {
+            // record stores, two lanes per record (see blend_backward_kernel)
+            const int odd         = lane & 1;
+            const int own         = give ? id : -1;
+            const int other       = pair_other(own);
+            const float4 o_lo     = pair_other(rec_lo);
+            const float4 o_hi     = pair_other(rec_hi);
+            const int id_first    = odd ? other : own;
+            const int id_second   = odd ? own : other;
+            const float4 v_first  = odd ? o_hi : rec_lo;
+            const float4 v_second = odd ? rec_hi : o_lo;
+            if (id_first >= 0) partial_l[2 * (size_t)id_first + odd] = v_first;
+            if (id_second >= 0) partial_l[2 * (size_t)id_second + odd] = v_second;
+        }
+    };
+    for (uint32_t k0 = 0; k0 < total; k0 += kWave)
+    {
+        // the first slot of a step is its longest
+        const uint32_t n0 = (uint32_t)__builtin_amdgcn_readfirstlane((int)s_n[wave][s_item[wave][k0]]);
+        if (n0 > 8)
+            step(k0, std::integral_constant<uint32_t, 16>{});
+        else if (n0 > 4)
+            step(k0, std::integral_constant<uint32_t, 8>{});
+        else if (n0 > 2)
+            step(k0, std::integral_constant<uint32_t, 4>{});
+        else if (n0 > 1)
+            step(k0, std::integral_constant<uint32_t, 2>{});
+        else
+            step(k0, std::integral_constant<uint32_t, 1>{});
+    }
+
+#pragma unroll
+    for (int ci = 0; ci < C; ++ci)
+    {
+        const float s = wave_sum(bg_grad[ci]);
+        if (lane == 0) red[wave][ci] = s;
+    }
+    {
+        const bool longer = __ballot(n > (uint32_t)kFuzzyDense) != 0ull;
+        if (lane == 0) red[wave][C] = 0.f;  // no background-confidence leak in this mode (guarded, RenderBackward.cu:643)
+        if (lane == 0) red[wave][C + 1] = longer ? 1.f : 0.f;
+    }
+    __syncthreads();
+    float* row = a.background_partial + (size_t)blockIdx.x * kBackgroundRow;
+    if (threadIdx.x <= C) row[threadIdx.x] = (red[0][threadIdx.x] + red[1][threadIdx.x]) + (red[2][threadIdx.x] + red[3][threadIdx.x]);
+    if (threadIdx.x == C + 1)
+        row[kFuzzyWalkColumn] = (red[0][C + 1] + red[1][C + 1]) + (red[2][C + 1] + red[3][C + 1]);
+}
+
+// The lists blend_backward_fuzzy_kernel left out (more than kFuzzyDense fragments): one lane per pixel walks its list
+// (FuzzyWalk). Same grid; a workgroup without such a list leaves at once. Launched where the list cut allows such lists.
+template <int C>
+__global__ void __launch_bounds__(kBlock) blend_backward_fuzzy_walk_kernel(BackwardPass a, float depth_accept)
+{
+    constexpr int kWaves = kBlock / kWave;
+    __shared__ float red[kWaves][C];
+    float* row = a.background_partial + (size_t)blockIdx.x * kBackgroundRow;
+    if (row[kFuzzyWalkColumn] == 0.f) return;
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    const TilePixel px = tile_pixel(a.tiles, a.ly);
+    const FuzzyPixel f = fuzzy_pixel<C>(a, px);
+    const bool walk    = f.n > (uint32_t)kFuzzyDense;
+    FuzzyWalk<C> w;
+    w.a = &a, w.list = a.fragments + f.off, w.partial_l = a.partial + 2 * (size_t)px.l * a.N, w.n = walk ? f.n : 0u;
+    w.do_point = f.do_point, w.depth_accept = depth_accept, w.total = w.prefix = 0.0;
+    w.bx = f.bx, w.by = f.by;
+#pragma unroll
+    for (int ci = 0; ci < C; ++ci) w.g[ci] = f.g[ci], w.ax[ci] = f.ax[ci], w.ay[ci] = f.ay[ci], w.bg_grad[ci] = 0.f;
 #pragma unroll 1
     for (int pass = 0; pass < 2; ++pass)
     {
@@ -651,7 +974,7 @@ __global__ void __launch_bounds__(kBlock) blend_backward_fuzzy_kernel(BackwardPa
             for (int u = 0; u < FuzzyWalk<C>::kChunk; ++u)
                 if (i0 + u < w.n) w.consume(i0 + u, t[u], conf[u], d[u], id[u]);
         }
-        if (with_background)
+        if (walk && !a.use_environment_map)
         {
             float t[C], conf, d;
             int id;
@@ -660,18 +983,14 @@ __global__ void __launch_bounds__(kBlock) blend_backward_fuzzy_kernel(BackwardPa
         }
         w.end_pass();
     }
-
 #pragma unroll
     for (int ci = 0; ci < C; ++ci)
     {
         const float s = wave_sum(w.bg_grad[ci]);
         if (lane == 0) red[wave][ci] = s;
     }
-    if (lane == 0) red[wave][C] = 0.f;  // no background-confidence leak in this mode (guarded, RenderBackward.cu:643)
     __syncthreads();
-    if (threadIdx.x <= C)
-        a.background_partial[(size_t)blockIdx.x * kBackgroundRow + threadIdx.x] =
-            (red[0][threadIdx.x] + red[1][threadIdx.x]) + (red[2][threadIdx.x] + red[3][threadIdx.x]);
+    if (threadIdx.x < C) row[threadIdx.x] += (red[0][threadIdx.x] + red[1][threadIdx.x]) + (red[2][threadIdx.x] + red[3][threadIdx.x]);
 }
 
 // Sums the per-workgroup background rows of one view (one workgroup, fixed order, so the result is reproducible) and

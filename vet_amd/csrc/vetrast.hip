@@ -850,6 +850,7 @@ int vetrast_backward(vetrast_ctx* ctx, const vetrast_backward_args* g, void* str
             }
             const dim3 grid(tile_grid(tiles)), blk(kBlock);
             if (p.render_mode == VETRAST_RENDER_FUZZY_BLEND)
+            {
                 switch (C)
                 {
                     case 1: hipLaunchKernelGGL(blend_backward_fuzzy_kernel<1>, grid, blk, 0, stream, bp, p.depth_accept_blend); break;
@@ -857,6 +858,16 @@ int vetrast_backward(vetrast_ctx* ctx, const vetrast_backward_args* g, void* str
                     case 3: hipLaunchKernelGGL(blend_backward_fuzzy_kernel<3>, grid, blk, 0, stream, bp, p.depth_accept_blend); break;
                     default: hipLaunchKernelGGL(blend_backward_fuzzy_kernel<4>, grid, blk, 0, stream, bp, p.depth_accept_blend); break;
                 }
+                // lists longer than the dense kernel lays out exist only where the cut allows them
+                if (bp.K <= 0 || bp.K > kFuzzyDense)
+                    switch (C)
+                    {
+                        case 1: hipLaunchKernelGGL(blend_backward_fuzzy_walk_kernel<1>, grid, blk, 0, stream, bp, p.depth_accept_blend); break;
+                        case 2: hipLaunchKernelGGL(blend_backward_fuzzy_walk_kernel<2>, grid, blk, 0, stream, bp, p.depth_accept_blend); break;
+                        case 3: hipLaunchKernelGGL(blend_backward_fuzzy_walk_kernel<3>, grid, blk, 0, stream, bp, p.depth_accept_blend); break;
+                        default: hipLaunchKernelGGL(blend_backward_fuzzy_walk_kernel<4>, grid, blk, 0, stream, bp, p.depth_accept_blend); break;
+                    }
+            }
             else if (hits == 1)
                 switch (C)
                 {
