@@ -436,3 +436,30 @@ def test_the_cache_sizes_bins_from_the_fragment_counts_of_earlier_calls():
     assert len(hist) == scene.num_layers and 0 < sum(hist) < 0.5 * scene.num_points * scene.num_layers
     for a, b, c in zip(plain, first, second):
         assert torch.equal(a, b) and torch.equal(a, c)
+
+
+@pytest.mark.parametrize("render_mode", [1, 3], ids=["full_blend", "bilinear_blend"])
+def test_adapter_templates_render_like_the_binding(render_mode):
+    """vet_adapter.h, instantiated with stand-ins that carry the member names of VET's NeuralScene, ReducedImageInfo
+    (Eigen-style crop_rotation(r, c), enum camera model), RenderParams and NeuralRenderInfo, hands the shim the same
+    call as the tensor binding: images and masks are equal bit for bit, a rotated and scaled crop included."""
+    from vet_amd import torch_ops
+
+    scene = synthetic.tiny_scene(num_points=4000, K=6, seed=61, num_views=2)
+    views = [list(v) for v in _views(scene)]
+    c, s_ = np.cos(0.3), np.sin(0.3)
+    views[1][5:10] = [0.9, 0.9, 1.5, -0.75, 0.0]   # crop_transform fx, fy, cx, cy, s
+    views[1][10:14] = [c, -s_, s_, c]              # crop_rotation, row-major
+    cu = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
+    args = (cu(scene.texture), cu(scene.background), cu(scene.position),
+            torch.zeros((scene.poses_se3.shape[0], 6), dtype=torch.float64, device="cuda"), cu(scene.intrinsics),
+            cu(scene.confidence.reshape(1, -1)), cu(scene.poses_se3))
+    want = torch_ops.blend_point_cloud(*args, None, views, scene.num_layers, train=False, use_environment_map=0,
+                                       dropout=0, render_mode=render_mode, debug_max_list_length=6,
+                                       output_background_mask=1)
+    got = torch_ops.adapter_selftest(*args, views, scene.num_layers, render_mode=render_mode, max_list_length=6,
+                                     output_background_mask=True)
+    assert len(got) == len(want) == 2 * scene.num_layers
+    for a, b in zip(got, want):
+        assert torch.equal(a, b)
+    assert float(got[0][1].abs().max()) > 0  # the rotated crop shows points

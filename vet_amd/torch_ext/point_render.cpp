@@ -1,6 +1,7 @@
 // libtorch host side of the MI355X blending point rasterizer: autograd Function with the reference's argument order,
 // calling the C ABI of include/vetrast.h. See point_render.h for the reference lines each piece mirrors.
 #include "point_render.h"
+#include "vet_adapter.h"
 
 #include <algorithm>
 #include <cmath>
@@ -975,6 +976,116 @@ void MyAdam::zero_grad()
 }
 }  // namespace vet_amd
 
+// ---- self test of vet_adapter.h ------------------------------------------------------------------------------------
+// Stand-ins with the member names and spellings of the reference's types (module holders with operator->, an
+// Eigen-style operator()(row, col), an enum class for the camera model, bool / int / float members of RenderParams under
+// the reference's names and defaults), so that the adapter's templates are compiled and run without VET's headers.
+namespace reference_stand_ins
+{
+enum class CameraModel : int { PINHOLE_DISTORTION = 0, OCAM = 1, SPHERICAL = 2 };
+struct IntrinsicsPinholef { float fx = 1, fy = 1, cx = 0, cy = 0, s = 0; };
+struct Mat2f
+{
+    float m[4] = {1, 0, 0, 1};  // column-major, as Eigen stores it
+    float operator()(int r, int c) const { return m[c * 2 + r]; }
+};
+struct ReducedImageInfo
+{
+    int w = 0, h = 0;
+    int image_index  = -1;
+    int camera_index = -1;
+    CameraModel camera_model_type = CameraModel::PINHOLE_DISTORTION;
+    IntrinsicsPinholef crop_transform;
+    Mat2f crop_rotation;
+};
+struct RenderParams  // src/lib/data/Settings.h:19-93, the members the adapter reads
+{
+    bool check_normal = false;
+    float dropout = 0.25, depth_accept_blend = 0.01;
+    float drop_out_radius_threshold = 0.6;
+    bool drop_out_points_by_radius  = true;
+    float distortion_gradient_factor = 0.005, K_gradient_factor = 0.5;
+    int num_texture_channels = -1;
+    float dist_cutoff = 20.f;
+    bool output_background_mask = false;
+    float output_background_mask_value = 0;
+    bool add_depth_to_network = false;
+    float stability_cutoff_value = 10000.f;
+    bool need_point_gradient = true, use_environment_map = true;
+    int render_mode = 1;
+    bool viewer_only = false;
+    int debug_max_list_length = -1;
+};
+struct TextureImpl { torch::Tensor texture, background_color, confidence_value_of_point; };
+struct PointCloudImpl { torch::Tensor t_position, t_index, t_original_color, t_normal; };
+struct PosesImpl { torch::Tensor tangent_poses, poses_se3; };
+struct IntrinsicsImpl { torch::Tensor intrinsics; };
+struct NeuralScene
+{
+    std::shared_ptr<PointCloudImpl> point_cloud_cuda = std::make_shared<PointCloudImpl>();
+    std::shared_ptr<TextureImpl> texture             = std::make_shared<TextureImpl>();
+    std::shared_ptr<PosesImpl> poses                 = std::make_shared<PosesImpl>();
+    std::shared_ptr<IntrinsicsImpl> intrinsics       = std::make_shared<IntrinsicsImpl>();
+    torch::Tensor dynamic_refinement_t;
+};
+struct NeuralRenderInfo
+{
+    NeuralScene* scene = nullptr;
+    std::vector<ReducedImageInfo> images;
+    RenderParams params;
+    int num_layers = 1;
+    bool train = false;
+    int current_epoch = 0;
+    void* timer_system = nullptr;
+    void* cache = nullptr;
+};
+}  // namespace reference_stand_ins
+
+// Renders through vet_adapter.h from stand-ins filled with the given tensors; `views` as for blend_point_cloud. The
+// caller compares the result with blend_point_cloud's for the same input.
+std::vector<torch::Tensor> adapter_selftest(torch::Tensor texture, torch::Tensor background_color, torch::Tensor points,
+                                            torch::Tensor pose_tangents, torch::Tensor intrinsics, torch::Tensor confidence,
+                                            torch::Tensor poses_se3, std::vector<std::vector<double>> views, int num_layers,
+                                            int render_mode, int max_list_length, bool output_background_mask)
+{
+    namespace ref = reference_stand_ins;
+    if (!g_cache) g_cache = std::make_shared<vet_amd::PointRendererCache>();
+    ref::NeuralScene scene;
+    scene.texture->texture                   = texture;
+    scene.texture->background_color          = background_color;
+    scene.texture->confidence_value_of_point = confidence;
+    scene.point_cloud_cuda->t_position       = points;
+    scene.poses->tangent_poses               = pose_tangents;
+    scene.poses->poses_se3                   = poses_se3;
+    scene.intrinsics->intrinsics             = intrinsics;
+    scene.dynamic_refinement_t               = torch::zeros({1}, points.options());
+    ref::NeuralRenderInfo info;
+    info.scene      = &scene;
+    info.num_layers = num_layers;
+    info.train      = false;
+    for (auto& v : views)
+    {
+        TORCH_CHECK(v.size() == 14, "a view is (w, h, image_index, camera_index, camera_model, crop[5], rot[4])");
+        ref::ReducedImageInfo r;
+        r.w = (int)v[0], r.h = (int)v[1], r.image_index = (int)v[2], r.camera_index = (int)v[3];
+        r.camera_model_type = static_cast<ref::CameraModel>((int)v[4]);
+        r.crop_transform.fx = (float)v[5], r.crop_transform.fy = (float)v[6], r.crop_transform.cx = (float)v[7];
+        r.crop_transform.cy = (float)v[8], r.crop_transform.s = (float)v[9];
+        // row-major in `views`, column-major in the stand-in, as in Eigen
+        r.crop_rotation.m[0] = (float)v[10], r.crop_rotation.m[2] = (float)v[11];
+        r.crop_rotation.m[1] = (float)v[12], r.crop_rotation.m[3] = (float)v[13];
+        info.images.push_back(r);
+    }
+    info.params.dropout                = 0.f;
+    info.params.num_texture_channels   = (int)texture.size(0);
+    info.params.use_environment_map    = false;
+    info.params.render_mode            = render_mode;
+    info.params.debug_max_list_length  = max_list_length;
+    info.params.output_background_mask = output_background_mask;
+    vet_amd::SceneTensors bundle;
+    return vet_amd::BlendPointCloudOf(&info, g_cache.get(), &bundle);
+}
+
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
 {
     pybind11::class_<vet_amd::MyAdam>(m, "MyAdam")
@@ -1100,6 +1211,11 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
             return d;
         },
         "address and size of the workspace the binding's cache keeps for training steps (for the tests)");
+    m.def("adapter_selftest", &adapter_selftest, pybind11::arg("texture"), pybind11::arg("background_color"),
+          pybind11::arg("points"), pybind11::arg("pose_tangents"), pybind11::arg("intrinsics"), pybind11::arg("confidence"),
+          pybind11::arg("poses_se3"), pybind11::arg("views"), pybind11::arg("num_layers"), pybind11::arg("render_mode") = 1,
+          pybind11::arg("max_list_length") = -1, pybind11::arg("output_background_mask") = false,
+          "renders through vet_adapter.h from stand-ins that have the member names of the reference's types");
     m.def("blend_point_cloud", &blend_point_cloud, pybind11::arg("texture"), pybind11::arg("background_color"),
           pybind11::arg("points"), pybind11::arg("pose_tangents"), pybind11::arg("intrinsics"), pybind11::arg("confidence"),
           pybind11::arg("poses_se3"), pybind11::arg("t_index"), pybind11::arg("views"), pybind11::arg("num_layers"),

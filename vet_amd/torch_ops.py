@@ -39,6 +39,16 @@ def blend_point_cloud(texture, background_color, points, pose_tangents, intrinsi
                                     {k: float(v) for k, v in params.items()}, environment)
 
 
+def adapter_selftest(texture, background_color, points, pose_tangents, intrinsics, confidence, poses_se3, views,
+                     num_layers, render_mode=1, max_list_length=-1, output_background_mask=False):
+    """Renders through vet_amd/torch_ext/vet_adapter.h (the templates that turn the reference's NeuralScene,
+    ReducedImageInfo, RenderParams and NeuralRenderInfo into the shim's types), instantiated with stand-ins that have the
+    reference's member names. Same result as blend_point_cloud(..., use_environment_map=0, dropout=0)."""
+    return load().adapter_selftest(texture, background_color, points, pose_tangents, intrinsics, confidence, poses_se3,
+                                   [list(map(float, v)) for v in views], int(num_layers), int(render_mode),
+                                   int(max_list_length), bool(output_background_mask))
+
+
 def MyAdam(groups, beta1=0.9, beta2=0.999, eps=1e-8, weight_decay=0.0):
     """The reference's texture optimiser (torch::optim::MyAdam, src/lib/models/my_adam.cpp) with one fused kernel per
     tensor and step. groups: list of (list of float32 CUDA parameter tensors, learning rate)."""
