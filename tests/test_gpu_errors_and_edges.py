@@ -126,11 +126,14 @@ def test_nonzero_distortion_raises_the_device_flag(rasterizer):
     assert rasterizer.check_device_flags(res) == abi.OK
 
 
-def test_forward_backward_can_be_captured_in_a_hip_graph(rasterizer, oracle):
+@pytest.mark.parametrize("mode,K", [(abi.RENDER_FULL_BLEND, 16), (abi.RENDER_FUZZY_BLEND, -1), (abi.RENDER_BILINEAR_BLEND, 16)],
+                         ids=["full", "fuzzy_no_cut", "bilinear"])
+def test_forward_backward_can_be_captured_in_a_hip_graph(mode, K, rasterizer, oracle):
     """The library only launches kernels (no memsets, allocations or host reads), so a whole step replays from a
-    graph; every replay is compared with the eager result, with eager work in between."""
-    scene = synthetic.config2(num_points=60_000, w=480, h=270)
-    params = make_params(scene, need_point_gradient=1)
+    graph; every replay is compared with the eager result, with eager work in between. (FUZZY_BLEND without a list cut
+    also launches the kernel that walks the lists too long for the dense layout.)"""
+    scene = synthetic.config2(num_points=60_000, w=480, h=270, K=K)
+    params = make_params(scene, need_point_gradient=1, render_mode=mode, depth_accept_blend=0.05)
     dev = DeviceScene(scene)
     eager = rasterizer.forward(dev, params)
     go = [torch.from_numpy(g).cuda() for g in scene.grad_out()]
