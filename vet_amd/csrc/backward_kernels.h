@@ -1146,7 +1146,11 @@ __global__ void __launch_bounds__(kBlock) gather_point_gradients_kernel(GatherPa
     Projected p;
     const DeviceView& cam = *a.vp.view;
     const float4 wp       = alive ? a.vp.position[i] : make_float4(0.f, 0.f, 0.f, 0.f);
-    if (alive && !point_is_skipped(a.vp, i) && project_point(cam, wp, p))
+    // (a position further outside the image than the coarsest layer's border pixels reach has no fragment in any
+    // layer, see bin_scatter_kernel: most of the cloud, for a crop)
+    const float reach = (float)(1 << (a.vp.ly.L - 1)) + 1.f;
+    if (alive && !point_is_skipped(a.vp, i) && project_point(cam, wp, p) && p.ipx >= -reach &&
+        p.ipx <= (float)a.vp.ly.w[0] + reach && p.ipy >= -reach && p.ipy <= (float)a.vp.ly.h[0] + reach)
     {
         // view-space position again, for the projection Jacobian (same expressions as project_point)
         const float vx = ((cam.r[0] * wp.x + cam.r[1] * wp.y) + cam.r[2] * wp.z) + cam.t[0];

@@ -343,7 +343,15 @@ __global__ void __launch_bounds__(kBlock) bin_scatter_kernel(ViewPass a, uint32_
     const bool visible = (uint32_t)i < (uint32_t)a.N && !point_is_skipped(a, i) && project_point(*a.view, a.position[i], p);
     float ipx = visible ? p.ipx : 0.f, ipy = visible ? p.ipy : 0.f, radius = visible ? p.radius : 0.f;
     const uint32_t depth_bits = __float_as_uint(p.z);
-    bool dropped = !visible;  // from the layer on at which the splat radius falls under the threshold
+    // A position further outside the image than the reach of the coarsest layer's border pixels hits no pixel of any
+    // layer (layer l halves the coordinates l times, exactly; its pixel 0 reaches down to -2^l in layer-0 units with the
+    // 2x2 splat, its last pixel not beyond the image size plus 2^l). A crop leaves most of the cloud out there: where
+    // that is so for a whole wave, the wave skips the layers altogether.
+    const float reach = (float)(1 << (a.ly.L - 1)) + 1.f;
+    const bool inside = visible && ipx >= -reach && ipx <= (float)a.ly.w[0] + reach && ipy >= -reach &&
+                        ipy <= (float)a.ly.h[0] + reach;
+    const bool any_inside = __ballot(inside) != 0ull;
+    bool dropped = !inside;  // also from the layer on at which the splat radius falls under the threshold
     if constexpr (HITS == 1)
     {
         // Layer by layer: group the wave's hits by bin and issue the group's atomic right away. The atomics of a wave
@@ -355,7 +363,7 @@ __global__ void __launch_bounds__(kBlock) bin_scatter_kernel(ViewPass a, uint32_
         for (int l = 0; l < VETRAST_MAX_LAYERS; ++l, radius *= 0.5f, ipx *= 0.5f, ipy *= 0.5f)
         {
             base[l] = 0, who[l] = 0, bins[l] = 0;
-            if (l >= a.ly.L) continue;
+            if (l >= a.ly.L || !any_inside) continue;
             if (a.drop_by_radius && radius < a.radius_threshold) dropped = true;
             uint32_t tile = 0, in_tile = 0, bin = 0, in_bin = 0;
             const bool has = !dropped && layer_hit<HITS>(a.ly, l, ipx, ipy, 0, tile, in_tile);
@@ -368,7 +376,7 @@ __global__ void __launch_bounds__(kBlock) bin_scatter_kernel(ViewPass a, uint32_
 #pragma unroll
         for (int l = 0; l < VETRAST_MAX_LAYERS; ++l)
         {
-            if (l >= a.ly.L) continue;
+            if (l >= a.ly.L || !any_inside) continue;
             const uint32_t group_base = (uint32_t)__shfl((int)base[l], (int)(who[l] & 0xFF), kWave);
             store_record(out, a.ly, l, (who[l] & 0x80000000u) != 0u, bins[l], group_base + ((who[l] >> 8) & 0xFFu), (uint32_t)i,
                          depth_bits, (who[l] >> 16) & 0xFFu, lane);
@@ -378,7 +386,7 @@ __global__ void __launch_bounds__(kBlock) bin_scatter_kernel(ViewPass a, uint32_
     {
         // The blend and its backward pass form a fragment's bilinear weight from the point's image position; they
         // read it from here (8 bytes) instead of projecting the point again for every one of its fragments.
-        if (visible) a.projected[i] = make_float2(p.ipx, p.ipy);
+        if (inside) a.projected[i] = make_float2(p.ipx, p.ipy);
         // The four pixels of a point mostly lie in one bin or two. Per layer the hits of a lane are therefore taken
         // bin by bin: in every turn a lane brings all its remaining hits that share the bin of its first remaining
         // hit, as one entry of that weight, so a layer takes as many grouping turns as the lane with the most
@@ -411,7 +419,7 @@ __global__ void __launch_bounds__(kBlock) bin_scatter_kernel(ViewPass a, uint32_
             code[l] = 0, in_bins[l] = 0;
 #pragma unroll
             for (int t = 0; t < kTurns; ++t) base[l][t] = 0, leader[l][t] = 0, ranks[l][t] = 0, bins[l][t] = 0;
-            if (l < a.ly.L)
+            if (l < a.ly.L && any_inside)
             {
                 if (a.drop_by_radius && radius < a.radius_threshold) dropped = true;
                 uint32_t bin[HITS];
@@ -454,9 +462,9 @@ __global__ void __launch_bounds__(kBlock) bin_scatter_kernel(ViewPass a, uint32_
                     if (has && g.leader == lane) base[l][t] = atomicAdd(&bin_counts[key], g.total);
                 }
             }
-            if (l >= 1 && l - 1 < a.ly.L) store_layer(l - 1);
+            if (l >= 1 && l - 1 < a.ly.L && any_inside) store_layer(l - 1);
         }
-        if (VETRAST_MAX_LAYERS - 1 < a.ly.L) store_layer(VETRAST_MAX_LAYERS - 1);
+        if (VETRAST_MAX_LAYERS - 1 < a.ly.L && any_inside) store_layer(VETRAST_MAX_LAYERS - 1);
     }
     if (packs)
     {
