@@ -298,8 +298,14 @@ def time_lift_error(scene, steps, cpu_threads):
     from vet_amd.rasterizer import Rasterizer
 
     rast = Rasterizer()
+    # 0.25 m cells; a scene whose box would need more than four million of them (config 4's outdoor scene: the grid is
+    # built on the host) gets cells twice as large until it does not
     cell_size = 0.25
-    mn, ln = synthetic.cell_grid(scene.position[:, :3], cell_size)
+    xyz = scene.position[:, :3]
+    extent = (xyz.max(axis=0) - xyz.min(axis=0)).astype(np.float64) + 0.02
+    while float(np.prod(np.ceil(extent / cell_size))) > 4e6:
+        cell_size *= 2.0
+    mn, ln = synthetic.cell_grid(xyz, cell_size)
     view = scene.views[0]
     img = synthetic.error_image(5, 3, view.h, view.w)
     to_dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
