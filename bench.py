@@ -634,6 +634,9 @@ def main():
 
     if extras and backward and args.config == 3:
         result["training_crops"] = time_training_crops(max(10, args.steps // 2), 3, args.render_mode)
+        if args.render_mode == 1:
+            # the same batch in the mode VET's shipped configuration trains in
+            result["training_crops_bilinear"] = time_training_crops(max(10, args.steps // 2), 3, 3)
     if extras:
         result["lift_error"] = time_lift_error(scene, max(10, args.steps // 2), 0 if args.no_cpu_baseline else cpu_threads)
 
