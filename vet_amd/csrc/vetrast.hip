@@ -771,8 +771,11 @@ int vetrast_backward(vetrast_ctx* ctx, const vetrast_backward_args* g, void* str
         list_bound[l] = (double)N * hits / ((double)ly.w[l] * ly.h[l]);
         if (p.debug_max_list_length > 0) list_bound[l] = std::min(list_bound[l], (double)p.debug_max_list_length);
     }
-    // (the FUZZY_BLEND kernel walks a pixel's list in one thread and wants every lane to carry a pixel)
-    const TileMap tiles = make_tile_map(ly, p.render_mode == VETRAST_RENDER_FUZZY_BLEND ? nullptr : list_bound);
+    // (FUZZY_BLEND: where the cut lets every list into the dense layout; the kernel that walks longer lists one lane
+    // per pixel wants every lane to carry a pixel)
+    const bool fuzzy_walks = p.render_mode == VETRAST_RENDER_FUZZY_BLEND &&
+                             (p.debug_max_list_length <= 0 || p.debug_max_list_length > kFuzzyDense);
+    const TileMap tiles = make_tile_map(ly, fuzzy_walks ? nullptr : list_bound);
     void* ws            = a->workspace;
 
     // The per-point kernel overwrites every gradient row in the first view, so the zeros_like fills of
