@@ -39,6 +39,9 @@ def _scenes():
     yield "tiny_levels_nocut_3ch", _levels(synthetic.tiny_scene(num_points=5000, K=-1, channels=3, seed=82)), {}
     yield "tiny_long_lists_levels", _levels(synthetic.tiny_scene(num_points=40000, K=0, seed=83)), {}
     yield "tiny_long_lists_K16", _levels(synthetic.tiny_scene(num_points=40000, K=16, seed=84)), {}
+    # the backward pass takes lists beyond 16 fragments one lane per pixel while the cut is at most 64, else a wave per list
+    yield "tiny_long_lists_K40", _levels(synthetic.tiny_scene(num_points=40000, K=40, seed=97)), {}
+    yield "tiny_long_lists_K100", _levels(synthetic.tiny_scene(num_points=40000, K=100, seed=98)), {}
     yield "tiny_2views_envmap", _levels(synthetic.tiny_scene(num_points=3000, K=8, num_views=2, seed=85)), \
         {"use_environment_map": 1}
     yield "wide_depth_range", synthetic.tiny_scene(num_points=5000, K=12, seed=86), {"depth_accept_blend": 0.3}
@@ -48,7 +51,10 @@ def _scenes():
     # depth 1e5 (the largest range the library takes is 1e4, so the points are moved out to 95 000); each with short
     # lists and with lists too long for the kernel that lays fragments out densely
     yield "range_reaches_zero_K8", synthetic.tiny_scene(num_points=3000, K=8, seed=90), {"depth_accept_blend": 2.0}
-    yield "range_reaches_zero_nocut", synthetic.tiny_scene(num_points=30000, K=-1, seed=91), {"depth_accept_blend": 2.0}
+    # (8 000 points: buckets of up to some two hundred elements. With 30 000 the oracle's own float32 sums over buckets
+    # of 800 elements, added front to back as the reference adds them, are 2e-6 off a float64 evaluation of the same
+    # formulas, which is beyond the bar below for the smallest gradients; the library's pairwise sums are not.)
+    yield "range_reaches_zero_nocut", synthetic.tiny_scene(num_points=8000, K=-1, seed=91), {"depth_accept_blend": 2.0}
     yield "one_bucket_K8", synthetic.tiny_scene(num_points=3000, K=8, seed=92), {"depth_accept_blend": 9.0e3}
     yield "one_bucket_nocut", synthetic.tiny_scene(num_points=30000, K=-1, seed=93), {"depth_accept_blend": 9.0e3}
     yield "background_in_last_bucket_K8", _far(synthetic.tiny_scene(num_points=3000, K=8, seed=95)), \
@@ -165,3 +171,79 @@ def test_depth_range_is_checked(rasterizer):
             rasterizer.forward(dev, make_params(scene, depth_accept_blend=bad, **MODE))
         assert e.value.status == abi.ERR_INVALID_ARG
     rasterizer.forward(dev, make_params(scene, depth_accept_blend=0.0))  # ignored by the other modes
+
+
+def _float64_model(scene, res, grad_out, depth_accept):
+    """BlendBackwardsFuzzy's value gradients (src/lib/rendering/RenderBackward.cu:570-727) evaluated in float64 from the
+    lists the forward pass left: bucket boundaries by the float32 comparison the kernels make, everything else (bucket
+    means, transmittance chain, bucket terms, the sum of the later buckets' terms) in double precision. One view, no
+    texture index, no environment map. Returns (d texture [C,N], d confidence [N], d background [C])."""
+    N, C = scene.num_points, scene.num_channels
+    off, keys = res.offsets(0), res.fragments(0)
+    depth32 = (keys >> np.uint64(32)).astype(np.uint32).view(np.float32)
+    pid = (keys & np.uint64(0xFFFFFFFF)).astype(np.int64)
+    conf, tex = scene.confidence.astype(np.float64), scene.texture.astype(np.float64)
+    bg = scene.background.astype(np.float64)
+    g_tex, g_conf, g_bg = np.zeros((C, N)), np.zeros(N), np.zeros(C)
+    accept = np.float32(depth_accept)
+    bases = res.layer_bases()
+    for l, (w, h) in enumerate(scene.layer_sizes()):
+        G = grad_out[l][0].astype(np.float64).reshape(C, -1)
+        for local in range(w * h):
+            q = bases[l] + local
+            lo, hi = int(off[q]), int(off[q + 1])
+            g = G[:, local]
+            d, ids = depth32[lo:hi], pid[lo:hi]
+            heads, last_min = [], np.float32(0.0)
+            for i in range(hi - lo):
+                if not (np.float32(d[i] - last_min) < accept):
+                    last_min = d[i]
+                    heads.append(i)
+                elif i == 0:
+                    heads.append(0)
+            joins = hi > lo and bool(np.float32(np.float32(100000.0) - last_min) < accept)  # background into the last bucket
+            A, terms, buckets = 1.0, [], []
+            for b, s_ in enumerate(heads):
+                e_ = heads[b + 1] if b + 1 < len(heads) else hi - lo
+                last = b + 1 == len(heads)
+                m = e_ - s_ + (1 if last and joins else 0)
+                bc = (conf[ids[s_:e_]].sum() + (1.0 if last and joins else 0.0)) / m
+                tb = (tex[:, ids[s_:e_]].sum(axis=1) + (bg if last and joins else 0.0)) / m
+                dot = float((tb * g).sum())
+                buckets.append((s_, e_, m, bc, dot, A, last and joins))
+                terms.append(dot * A * bc)
+                A *= 1.0 - bc
+            total = sum(terms) + (0.0 if joins else float((g * bg).sum()) * A)
+            if not joins:
+                g_bg += A * g
+            prefix = 0.0
+            for (s_, e_, m, bc, dot, Ab, with_bg), x in zip(buckets, terms):
+                prefix += x
+                np.add.at(g_conf, ids[s_:e_], dot * Ab / m - (total - prefix) / ((1.0 - bc) + 1e-9))
+                np.add.at(g_tex, (slice(None), ids[s_:e_]), (Ab * bc / m) * g[:, None])
+                if with_bg:
+                    g_bg += (Ab * bc / m) * g
+    return g_tex, g_conf, g_bg
+
+
+def test_long_buckets_against_a_float64_evaluation(rasterizer, oracle):
+    """Lists of hundreds to thousands of fragments in two or three buckets per pixel. The oracle adds a bucket's
+    confidences and descriptors up front to back in float32, as the reference does; over 800 elements that sum alone is
+    a few 1e-6 off. The library combines pairwise. Both are compared with the same formulas in float64: the library
+    must agree within half the bar the oracle comparisons use (observed 2e-5, the oracle 2e-4)."""
+    scene = synthetic.tiny_scene(num_points=30000, K=-1, seed=91)
+    params = make_params(scene, depth_accept_blend=2.0, need_point_gradient=0, **MODE)
+    dev = DeviceScene(scene)
+    res = rasterizer.forward(dev, params, save_for_backward=True)
+    grad_out = scene.grad_out()
+    got = rasterizer.backward(res, [torch.from_numpy(g).cuda() for g in grad_out], want_points=False)
+    torch.cuda.synchronize()
+    assert int(np.diff(res.offsets(0)).max()) > 1000, "the scene is meant to have very long lists"
+    m_tex, m_conf, m_bg = _float64_model(scene, res, grad_out, 2.0)
+    want = oracle.backward(oracle.forward(scene, params), grad_out, want_points=False)
+    for key, model in (("texture", m_tex), ("confidence", m_conf), ("background", m_bg)):
+        lib_err = max_rel_err(got[key].cpu().numpy().astype(np.float64), model)
+        oracle_err = max_rel_err(want[key].astype(np.float64), model)
+        print(f"  {key}: library vs float64 {lib_err:.2e}, oracle vs float64 {oracle_err:.2e}", flush=True)
+        assert lib_err <= 5e-5, key
+        assert oracle_err <= 1e-3, key

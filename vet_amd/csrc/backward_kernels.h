@@ -666,11 +666,18 @@ __device__ __forceinline__ FuzzyPixel fuzzy_pixel(const BackwardPass& a, const T
 // first one, and the step's code is compiled once per slot length so that shorter slots take fewer combine steps.
 // Longer lists are left to blend_backward_fuzzy_walk_kernel; the workgroup says in column 7 of its background row
 // whether it has any.
-constexpr int kFuzzyDense     = 16;
-constexpr int kFuzzyWalkColumn = 7;
+constexpr int kFuzzyDense      = 16;
+// Lists beyond the dense layout: `walk_max` (a kernel argument) is the longest list blend_backward_fuzzy_walk_kernel
+// takes, one lane per pixel; longer ones go to blend_backward_fuzzy_long_kernel, the whole wave per list. The walk is
+// the faster of the two while all lists are short (a cut of up to kFuzzyWalkCut: 64 pixels advance together), the
+// wave-per-list kernel where some are long (no cut: the longest list alone would keep one lane busy for a millisecond),
+// and running both one after the other costs more than either, so the host picks one by the cut.
+constexpr int kFuzzyWalkCut    = 64;
+constexpr int kFuzzyWalkColumn = 7;   // background row, column 7: the workgroup has a list for the walk kernel
+constexpr int kFuzzyLongColumn = 6;   // ... column 6: one for the wave-per-list kernel
 
 template <int C>
-__global__ void __launch_bounds__(kBlock) blend_backward_fuzzy_kernel(BackwardPass a, float depth_accept)
+__global__ void __launch_bounds__(kBlock) blend_backward_fuzzy_kernel(BackwardPass a, float depth_accept, uint32_t walk_max)
 {
     constexpr int kWaves = kBlock / kWave;
     __shared__ uint32_t s_off[kWaves][kWave];
@@ -682,7 +689,7 @@ __global__ void __launch_bounds__(kBlock) blend_backward_fuzzy_kernel(BackwardPa
     __shared__ float4 s_ay[kWaves][kWave];
     __shared__ float2 s_bxy[kWaves][kWave];
     __shared__ uint8_t s_item[kWaves][kWaveItems];
-    __shared__ float red[kWaves][C + 2];
+    __shared__ float red[kWaves][C + 3];
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
     const TilePixel px = tile_pixel(a.tiles, a.ly);
     float4* partial_l  = a.partial + 2 * (size_t)px.l * a.N;
@@ -931,21 +938,25 @@ __global__ void __launch_bounds__(kBlock) blend_backward_fuzzy_kernel(BackwardPa
         if (lane == 0) red[wave][ci] = s;
     }
     {
-        const bool longer = __ballot(n > (uint32_t)kFuzzyDense) != 0ull;
+        const bool longer = __ballot(n > (uint32_t)kFuzzyDense && n <= walk_max) != 0ull;
+        const bool longest = __ballot(n > max(walk_max, (uint32_t)kFuzzyDense)) != 0ull;
         if (lane == 0) red[wave][C] = 0.f;  // no background-confidence leak in this mode (guarded, RenderBackward.cu:643)
         if (lane == 0) red[wave][C + 1] = longer ? 1.f : 0.f;
+        if (lane == 0) red[wave][C + 2] = longest ? 1.f : 0.f;
     }
     __syncthreads();
     float* row = a.background_partial + (size_t)blockIdx.x * kBackgroundRow;
     if (threadIdx.x <= C) row[threadIdx.x] = (red[0][threadIdx.x] + red[1][threadIdx.x]) + (red[2][threadIdx.x] + red[3][threadIdx.x]);
     if (threadIdx.x == C + 1)
         row[kFuzzyWalkColumn] = (red[0][C + 1] + red[1][C + 1]) + (red[2][C + 1] + red[3][C + 1]);
+    if (threadIdx.x == C + 2)
+        row[kFuzzyLongColumn] = (red[0][C + 2] + red[1][C + 2]) + (red[2][C + 2] + red[3][C + 2]);
 }
 
 // The lists blend_backward_fuzzy_kernel left out (more than kFuzzyDense fragments): one lane per pixel walks its list
 // (FuzzyWalk). Same grid; a workgroup without such a list leaves at once. Launched where the list cut allows such lists.
 template <int C>
-__global__ void __launch_bounds__(kBlock) blend_backward_fuzzy_walk_kernel(BackwardPass a, float depth_accept)
+__global__ void __launch_bounds__(kBlock) blend_backward_fuzzy_walk_kernel(BackwardPass a, float depth_accept, uint32_t walk_max)
 {
     constexpr int kWaves = kBlock / kWave;
     __shared__ float red[kWaves][C];
@@ -954,7 +965,7 @@ __global__ void __launch_bounds__(kBlock) blend_backward_fuzzy_walk_kernel(Backw
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
     const TilePixel px = tile_pixel(a.tiles, a.ly);
     const FuzzyPixel f = fuzzy_pixel<C>(a, px);
-    const bool walk    = f.n > (uint32_t)kFuzzyDense;
+    const bool walk    = f.n > (uint32_t)kFuzzyDense && f.n <= walk_max;
     FuzzyWalk<C> w;
     w.a = &a, w.list = a.fragments + f.off, w.partial_l = a.partial + 2 * (size_t)px.l * a.N, w.n = walk ? f.n : 0u;
     w.do_point = f.do_point, w.depth_accept = depth_accept, w.total = w.prefix = 0.0;
@@ -987,6 +998,305 @@ __global__ void __launch_bounds__(kBlock) blend_backward_fuzzy_walk_kernel(Backw
     for (int ci = 0; ci < C; ++ci)
     {
         const float s = wave_sum(w.bg_grad[ci]);
+        if (lane == 0) red[wave][ci] = s;
+    }
+    __syncthreads();
+    if (threadIdx.x < C) row[threadIdx.x] += (red[0][threadIdx.x] + red[1][threadIdx.x]) + (red[2][threadIdx.x] + red[3][threadIdx.x]);
+}
+
+// The lists blend_backward_fuzzy_kernel left out (more than kFuzzyDense fragments), one after the other, each by the
+// whole wave: 64 consecutive fragments per step, front to back, one lane per fragment. The bucket boundaries of a step
+// are found by a loop over its depths that every lane runs alike (the rule is sequential, but it needs the depths
+// only); sums over a bucket, the transmittance product over the buckets in front and the running sum of the bucket
+// terms are scans over the lanes. What crosses a step boundary is carried in registers: the open bucket (sums, number
+// of elements, first element), the depth its range started at, the transmittance in front of it and the sum of the
+// bucket terms so far. A bucket's gradient needs the sum of the terms of all LATER buckets, so the list is processed
+// twice: the first pass only adds up the terms, the second has the total and writes. The elements of a bucket that was
+// still open at the end of their step get the position part of their record there and the bucket's part when it
+// closes, from a loop over their keys. Same grid as the dense kernel; a workgroup without such a list leaves at once.
+template <int C>
+__global__ void __launch_bounds__(kBlock) blend_backward_fuzzy_long_kernel(BackwardPass a, float depth_accept, uint32_t walk_max)
+{
+    constexpr int kWaves = kBlock / kWave;
+    __shared__ float red[kWaves][C];
+    float* row = a.background_partial + (size_t)blockIdx.x * kBackgroundRow;
+    if (row[kFuzzyLongColumn] == 0.f) return;
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    const TilePixel px = tile_pixel(a.tiles, a.ly);
+    const FuzzyPixel f = fuzzy_pixel<C>(a, px);
+    float4* partial_l  = a.partial + 2 * (size_t)px.l * a.N;  // the layer is the same for the whole workgroup
+    const bool with_background = !a.use_environment_map;
+    float bg_grad[C];  // summed over the wave at the end: every lane adds what it computes for lane 0's sake once
+#pragma unroll
+    for (int ci = 0; ci < C; ++ci) bg_grad[ci] = 0.f;
+    auto everywhere = [&](float v, int src) { return __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(v), src)); };
+
+    uint64_t todo = __ballot(f.n > max(walk_max, (uint32_t)kFuzzyDense));
+    while (todo != 0ull)
+    {
+        const int src = __ffsll((unsigned long long)todo) - 1;
+        todo &= todo - 1ull;
+        // the pixel, the same on every lane
+        const uint32_t n       = (uint32_t)__builtin_amdgcn_readlane((int)f.n, src);
+        const uint64_t* list   = a.fragments + (uint32_t)__builtin_amdgcn_readlane((int)f.off, src);
+        const bool do_point    = __builtin_amdgcn_readlane((int)f.do_point, src) != 0;
+        float g[4], ax[4], ay[4];
+#pragma unroll
+        for (int ci = 0; ci < 4; ++ci) g[ci] = everywhere(f.g[ci], src), ax[ci] = everywhere(f.ax[ci], src), ay[ci] = everywhere(f.ay[ci], src);
+        const float bx = everywhere(f.bx, src), by = everywhere(f.by, src);
+
+        double total = 0.0;
+#pragma unroll 1
+        for (int pass = 0; pass < 2; ++pass)
+        {
+            // carried from step to step (the same on every lane)
+            float open_sums[C + 1];
+#pragma unroll
+            for (int v = 0; v <= C; ++v) open_sums[v] = 0.f;
+            uint32_t open_m = 0, open_start = 0;
+            float last_min = 0.f, A_front = 1.f;  // transmittance in front of the open bucket
+            double prefix  = 0.0;                 // bucket terms of the closed buckets
+#pragma unroll 1
+            for (uint32_t begin = 0; begin < n; begin += kWave)
+            {
+                const uint32_t valid = min((uint32_t)kWave, n - begin);
+                const bool last_step = begin + kWave >= n;
+                const bool has       = (uint32_t)lane < valid;
+                float depth = 0.f, conf = 0.f;
+                float t[4]  = {0.f, 0.f, 0.f, 0.f};
+                int id = -1;
+                if (has)
+                {
+                    const uint64_t key = list[begin + lane];
+                    depth              = __uint_as_float((uint32_t)(key >> 32));
+                    const int point    = (int)(uint32_t)key;
+                    int ti             = -1;
+                    if ((uint32_t)point < (uint32_t)a.N) ti = a.index ? a.index[point] : point;
+                    if ((uint32_t)ti < (uint32_t)a.N)
+                    {
+                        const float4 t4 = a.packed[2 * (size_t)ti];
+                        conf            = a.packed[2 * (size_t)ti + 1].x;
+                        t[0] = t4.x, t[1] = t4.y, t[2] = t4.z, t[3] = t4.w;
+                        id = point;
+                    }
+                }
+                // ---- bucket boundaries of this step (src/lib/rendering/RenderBackward.cu:706-714); element 0 of the
+                // list opens the first bucket whether or not it resets the range
+                uint64_t heads = begin == 0 ? 1ull : 0ull;
+                for (uint32_t i = 0; i < valid; ++i)
+                {
+                    const float di = everywhere(depth, (int)i);
+                    if (!(di - last_min < depth_accept))
+                    {
+                        last_min = di;
+                        heads |= 1ull << i;
+                    }
+                }
+                // the background (depth 1e5) behind the last fragment: one more element of the last bucket if that
+                // bucket's range reaches it, else a bucket of its own
+                const bool bg_joins = last_step && with_background && (100000.f - last_min < depth_accept);
+
+                // ---- a bucket that was open and has no element in this step closes in front of it
+                if (open_m != 0u && (heads & 1ull))
+                {
+                    const float inv   = 1.f / (float)open_m;
+                    const float bconf = open_sums[C] * inv;
+                    float dot = 0.f, x = 0.f;
+#pragma unroll
+                    for (int ci = 0; ci < C; ++ci)
+                    {
+                        const float tb = open_sums[ci] * inv;
+                        dot += tb * g[ci];
+                        x += ((g[ci] * tb) * A_front) * bconf;
+                    }
+                    if (pass == 0)
+                        total += (double)x;
+                    else
+                    {
+                        prefix += (double)x;
+                        const float S     = (float)(total - prefix);
+                        const float gconf = (dot * A_front) * inv - S / ((1.f - bconf) + 1e-9f);
+                        float gt[4]       = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                        for (int ci = 0; ci < C; ++ci) gt[ci] = ((A_front * bconf) * g[ci]) * inv;
+                        for (uint32_t e = open_start + lane; e < begin; e += kWave)
+                        {
+                            const int point = (int)(uint32_t)list[e];
+                            int ti          = -1;
+                            if ((uint32_t)point < (uint32_t)a.N) ti = a.index ? a.index[point] : point;
+                            if ((uint32_t)ti >= (uint32_t)a.N) continue;
+                            partial_l[2 * (size_t)point] = make_float4(gt[0], gt[1], gt[2], gt[3]);
+                            reinterpret_cast<float*>(&partial_l[2 * (size_t)point + 1])[0] = gconf;
+                        }
+                    }
+                    A_front = (1.f - bconf) * A_front;
+                    open_m  = 0u;
+#pragma unroll
+                    for (int v = 0; v <= C; ++v) open_sums[v] = 0.f;
+                }
+
+                // ---- this lane's bucket inside the step
+                const uint64_t upto  = heads & (lane == kWave - 1 ? ~0ull : (2ull << lane) - 1ull);
+                const bool joined    = upto == 0ull;  // belongs to the bucket that was open when the step began
+                const uint32_t first = joined ? 0u : 63u - (uint32_t)__clzll((long long)upto);
+                const uint64_t later = lane == kWave - 1 ? 0ull : heads >> (lane + 1);
+                uint32_t next        = later ? (uint32_t)lane + (uint32_t)__ffsll((unsigned long long)later) : valid;
+                next                 = min(next, valid);
+                const uint32_t dist  = (uint32_t)lane - first;
+                const bool closes    = has && (next < valid || last_step);  // the bucket ends in this step
+                const bool tail      = has && next == valid;                // the last bucket of the step
+                // sums over the bucket's elements of this step: inclusive scan from its first lane, read at its last
+                float sums[C + 1];
+                sums[C] = conf;
+#pragma unroll
+                for (int ci = 0; ci < C; ++ci) sums[ci] = t[ci];
+                const int last_lane = has ? (int)next - 1 : lane;
+#pragma unroll
+                for (int v = 0; v <= C; ++v)
+                {
+                    float x = sums[v];
+#pragma unroll
+                    for (int d = 1; d < kWave; d <<= 1)
+                    {
+                        const float o = __shfl_up(x, d, kWave);
+                        if (dist >= (uint32_t)d) x += o;
+                    }
+                    sums[v] = __shfl(x, last_lane, kWave);
+                    if (joined) sums[v] = open_sums[v] + sums[v];
+                }
+                uint32_t m = has ? (next - first) + (joined ? open_m : 0u) : 1u;
+                if (bg_joins && tail)
+                {
+                    sums[C] += 1.f;
+#pragma unroll
+                    for (int ci = 0; ci < C; ++ci) sums[ci] += a.background[ci];
+                    m += 1u;
+                }
+                const float inv   = 1.f / (float)m;
+                const float bconf = sums[C] * inv;
+                float dot = 0.f;
+#pragma unroll
+                for (int ci = 0; ci < C; ++ci) dot += (sums[ci] * inv) * g[ci];
+                // transmittance in front: product of (1 - mean confidence) over the buckets that close in this step in
+                // front of this one, times what was in front of the step
+                const bool closing_lane = closes && lane == last_lane;
+                float P = closing_lane ? 1.f - bconf : 1.f;
+#pragma unroll
+                for (int d = 1; d < kWave; d <<= 1)
+                {
+                    const float o = __shfl_up(P, d, kWave);
+                    if (lane >= d) P *= o;
+                }
+                const float P_before = __shfl(P, first > 0u ? (int)first - 1 : lane, kWave);
+                const float A        = first > 0u ? A_front * P_before : A_front;
+                const float P_end    = everywhere(P, (int)valid - 1);  // over all buckets that close in this step
+                float x = 0.f;
+#pragma unroll
+                for (int ci = 0; ci < C; ++ci) x += ((g[ci] * (sums[ci] * inv)) * A) * bconf;
+                // running sum of the terms of the buckets that close in this step
+                float X = closing_lane ? x : 0.f;
+#pragma unroll
+                for (int d = 1; d < kWave; d <<= 1)
+                {
+                    const float o = __shfl_up(X, d, kWave);
+                    if (lane >= d) X += o;
+                }
+                const float X_end = everywhere(X, (int)valid - 1);
+                if (pass == 1)
+                {
+                    const float X_mine = __shfl(X, last_lane, kWave);  // terms up to and including this lane's bucket
+                    float gp0 = 0.f, gp1 = 0.f;
+                    if (has && id >= 0 && do_point)
+                    {
+                        float dR_dpx = bx, dR_dpy = by;
+#pragma unroll
+                        for (int ci = 0; ci < C; ++ci)
+                        {
+                            dR_dpx += t[ci] * ax[ci];
+                            dR_dpy += t[ci] * ay[ci];
+                        }
+                        gp0 = dR_dpx / (float)C;
+                        gp1 = dR_dpy / (float)C;
+                    }
+                    const float S     = (float)(total - (prefix + (double)X_mine));
+                    const float gconf = (dot * A) * inv - S / ((1.f - bconf) + 1e-9f);
+                    float gt[4]       = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                    for (int ci = 0; ci < C; ++ci) gt[ci] = ((A * bconf) * g[ci]) * inv;
+                    if (has && id >= 0)
+                    {
+                        if (closes)
+                        {
+                            partial_l[2 * (size_t)id]     = make_float4(gt[0], gt[1], gt[2], gt[3]);
+                            partial_l[2 * (size_t)id + 1] = make_float4(gconf, gp0, gp1, 0.f);
+                        }
+                        else
+                        {
+                            // the bucket stays open: its part of the record follows when it closes
+                            float* rec = reinterpret_cast<float*>(&partial_l[2 * (size_t)id + 1]);
+                            rec[1] = gp0, rec[2] = gp1, rec[3] = 0.f;
+                        }
+                    }
+                    // the elements an earlier step left with a bucket that closes here
+                    const bool joined_closes = open_m != 0u && __builtin_amdgcn_readlane((int)(closes && joined), 0) != 0;
+                    if (joined_closes)
+                    {
+                        float gt0[4];
+#pragma unroll
+                        for (int ci = 0; ci < 4; ++ci) gt0[ci] = everywhere(gt[ci], 0);
+                        const float gconf0 = everywhere(gconf, 0);
+                        for (uint32_t e = open_start + lane; e < begin; e += kWave)
+                        {
+                            const int point = (int)(uint32_t)list[e];
+                            int ti          = -1;
+                            if ((uint32_t)point < (uint32_t)a.N) ti = a.index ? a.index[point] : point;
+                            if ((uint32_t)ti >= (uint32_t)a.N) continue;
+                            partial_l[2 * (size_t)point] = make_float4(gt0[0], gt0[1], gt0[2], gt0[3]);
+                            reinterpret_cast<float*>(&partial_l[2 * (size_t)point + 1])[0] = gconf0;
+                        }
+                    }
+                    if (last_step && with_background && lane == (int)valid - 1)
+                    {
+                        // the background's share: an element of the last bucket, or a bucket of its own behind all
+                        const float scale = bg_joins ? A * bconf : (A_front * P_end) * 1.f;
+                        const float share = bg_joins ? inv : 1.f;
+#pragma unroll
+                        for (int ci = 0; ci < C; ++ci) bg_grad[ci] += (scale * g[ci]) * share;
+                    }
+                }
+                // ---- what the next step inherits
+                if (pass == 0)
+                    total += (double)X_end;
+                else
+                    prefix += (double)X_end;
+                if (last_step)
+                {
+                    if (pass == 0 && with_background && !bg_joins)
+                    {
+                        float xb = 0.f;
+#pragma unroll
+                        for (int ci = 0; ci < C; ++ci) xb += ((g[ci] * a.background[ci]) * (A_front * P_end)) * 1.f;
+                        total += (double)xb;
+                    }
+                }
+                else
+                {
+                    // the last bucket of the step stays open (valid = 64 here)
+                    const bool all_joined   = heads == 0ull;
+                    const uint32_t open_pos = all_joined ? 0u : 63u - (uint32_t)__clzll((long long)heads);
+#pragma unroll
+                    for (int v = 0; v <= C; ++v) open_sums[v] = everywhere(sums[v], kWave - 1);
+                    open_m     = (uint32_t)kWave - open_pos + (all_joined ? open_m : 0u);
+                    open_start = all_joined ? open_start : begin + open_pos;
+                    A_front    = A_front * P_end;
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int ci = 0; ci < C; ++ci)
+    {
+        const float s = wave_sum(bg_grad[ci]);
         if (lane == 0) red[wave][ci] = s;
     }
     __syncthreads();

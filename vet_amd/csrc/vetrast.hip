@@ -771,11 +771,7 @@ int vetrast_backward(vetrast_ctx* ctx, const vetrast_backward_args* g, void* str
         list_bound[l] = (double)N * hits / ((double)ly.w[l] * ly.h[l]);
         if (p.debug_max_list_length > 0) list_bound[l] = std::min(list_bound[l], (double)p.debug_max_list_length);
     }
-    // (FUZZY_BLEND: where the cut lets every list into the dense layout; the kernel that walks longer lists one lane
-    // per pixel wants every lane to carry a pixel)
-    const bool fuzzy_walks = p.render_mode == VETRAST_RENDER_FUZZY_BLEND &&
-                             (p.debug_max_list_length <= 0 || p.debug_max_list_length > kFuzzyDense);
-    const TileMap tiles = make_tile_map(ly, fuzzy_walks ? nullptr : list_bound);
+    const TileMap tiles = make_tile_map(ly, list_bound);
     void* ws            = a->workspace;
 
     // The per-point kernel overwrites every gradient row in the first view, so the zeros_like fills of
@@ -854,22 +850,26 @@ int vetrast_backward(vetrast_ctx* ctx, const vetrast_backward_args* g, void* str
             const dim3 grid(tile_grid(tiles)), blk(kBlock);
             if (p.render_mode == VETRAST_RENDER_FUZZY_BLEND)
             {
+                // Lists of more than kFuzzyDense fragments exist only where the cut allows them. With a cut of up to
+                // kFuzzyWalkCut they are walked one lane per pixel; otherwise each is taken by a whole wave.
+                const bool beyond_dense = bp.K <= 0 || bp.K > kFuzzyDense;
+                const bool walks        = bp.K > kFuzzyDense && bp.K <= kFuzzyWalkCut;
+                const uint32_t walk_max = walks ? (uint32_t)bp.K : (uint32_t)kFuzzyDense;
+                auto launch = [&](auto channels) {
+                    constexpr int kC = decltype(channels)::value;
+                    hipLaunchKernelGGL(blend_backward_fuzzy_kernel<kC>, grid, blk, 0, stream, bp, p.depth_accept_blend, walk_max);
+                    if (beyond_dense && walks)
+                        hipLaunchKernelGGL(blend_backward_fuzzy_walk_kernel<kC>, grid, blk, 0, stream, bp, p.depth_accept_blend, walk_max);
+                    if (beyond_dense && !walks)
+                        hipLaunchKernelGGL(blend_backward_fuzzy_long_kernel<kC>, grid, blk, 0, stream, bp, p.depth_accept_blend, walk_max);
+                };
                 switch (C)
                 {
-                    case 1: hipLaunchKernelGGL(blend_backward_fuzzy_kernel<1>, grid, blk, 0, stream, bp, p.depth_accept_blend); break;
-                    case 2: hipLaunchKernelGGL(blend_backward_fuzzy_kernel<2>, grid, blk, 0, stream, bp, p.depth_accept_blend); break;
-                    case 3: hipLaunchKernelGGL(blend_backward_fuzzy_kernel<3>, grid, blk, 0, stream, bp, p.depth_accept_blend); break;
-                    default: hipLaunchKernelGGL(blend_backward_fuzzy_kernel<4>, grid, blk, 0, stream, bp, p.depth_accept_blend); break;
+                    case 1: launch(std::integral_constant<int, 1>{}); break;
+                    case 2: launch(std::integral_constant<int, 2>{}); break;
+                    case 3: launch(std::integral_constant<int, 3>{}); break;
+                    default: launch(std::integral_constant<int, 4>{}); break;
                 }
-                // lists longer than the dense kernel lays out exist only where the cut allows them
-                if (bp.K <= 0 || bp.K > kFuzzyDense)
-                    switch (C)
-                    {
-                        case 1: hipLaunchKernelGGL(blend_backward_fuzzy_walk_kernel<1>, grid, blk, 0, stream, bp, p.depth_accept_blend); break;
-                        case 2: hipLaunchKernelGGL(blend_backward_fuzzy_walk_kernel<2>, grid, blk, 0, stream, bp, p.depth_accept_blend); break;
-                        case 3: hipLaunchKernelGGL(blend_backward_fuzzy_walk_kernel<3>, grid, blk, 0, stream, bp, p.depth_accept_blend); break;
-                        default: hipLaunchKernelGGL(blend_backward_fuzzy_walk_kernel<4>, grid, blk, 0, stream, bp, p.depth_accept_blend); break;
-                    }
             }
             else if (hits == 1)
                 switch (C)
