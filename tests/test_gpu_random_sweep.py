@@ -106,11 +106,7 @@ def test_random_case(seed, rasterizer, oracle):
         g, w_ = got[key].cpu().numpy(), want[key]
         assert np.all(np.isfinite(g)), key
         err = max_rel_err(g, w_) if np.abs(w_).max() > 0 else float(np.abs(g).max())
-        # FUZZY_BLEND with lists beyond the top-16 cut: buckets of hundreds of elements, which the oracle adds up front
-        # to back in float32 as the reference does and the library pairwise; the oracle's sums are the less exact
-        # ones (tests/test_gpu_fuzzy.py::test_long_buckets_against_a_float64_evaluation)
-        long_buckets = over["render_mode"] == 2 and not 0 < scene.max_list_length <= 16
-        assert err <= (3e-4 if long_buckets else 1e-4), (key, err)
+        assert err <= 1e-4, (key, err)
 
 
 def _draw_clustered(seed):
@@ -175,8 +171,6 @@ def test_random_clustered_case(seed, rasterizer, oracle):
     for l in range(scene.num_layers):
         np.testing.assert_array_equal(res.out[l].cpu().numpy(), ref.out[l], err_msg=f"layer {l}")
     tol = 1e-4  # also for uncut lists of tens of thousands of fragments
-    if over["render_mode"] == abi.RENDER_FUZZY_BLEND and not 0 < scene.max_list_length <= 16:
-        tol = 3e-4  # the oracle's front-to-back float32 sums over long buckets, see test_random_case
     grad_out = scene.grad_out()
     want = oracle.backward(ref, grad_out, num_threads=8)
     got = rasterizer.backward(res, [torch.from_numpy(g).cuda() for g in grad_out])

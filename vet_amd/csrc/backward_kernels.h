@@ -1193,18 +1193,23 @@ __global__ void __launch_bounds__(kBlock) blend_backward_fuzzy_long_kernel(Backw
                 float x = 0.f;
 #pragma unroll
                 for (int ci = 0; ci < C; ++ci) x += ((g[ci] * (sums[ci] * inv)) * A) * bconf;
-                // running sum of the terms of the buckets that close in this step
+                // Terms of the buckets that close in this step, summed from the back: a bucket needs the terms of the
+                // buckets BEHIND it, and taking them as (all) - (those in front) would cancel to rounding noise deep in
+                // a list, where what is left behind is a millionth of what lies in front.
                 float X = closing_lane ? x : 0.f;
 #pragma unroll
                 for (int d = 1; d < kWave; d <<= 1)
                 {
-                    const float o = __shfl_up(X, d, kWave);
-                    if (lane >= d) X += o;
+                    const float o = __shfl_down(X, d, kWave);
+                    if (lane + d < kWave) X += o;
                 }
-                const float X_end = everywhere(X, (int)valid - 1);
+                const float X_end = everywhere(X, 0);  // all of them
                 if (pass == 1)
                 {
-                    const float X_mine = __shfl(X, last_lane, kWave);  // terms up to and including this lane's bucket
+                    // behind this lane's bucket inside the step
+                    // (the exchange is made by every lane, then the lanes with nothing behind them drop what they got)
+                    const float X_next   = __shfl(X, min(last_lane + 1, kWave - 1), kWave);
+                    const float X_behind = last_lane + 1 < kWave ? X_next : 0.f;
                     float gp0 = 0.f, gp1 = 0.f;
                     if (has && id >= 0 && do_point)
                     {
@@ -1218,7 +1223,8 @@ __global__ void __launch_bounds__(kBlock) blend_backward_fuzzy_long_kernel(Backw
                         gp0 = dR_dpx / (float)C;
                         gp1 = dR_dpy / (float)C;
                     }
-                    const float S     = (float)(total - (prefix + (double)X_mine));
+                    // ... and behind the step: both sums are made of the same float terms, so this difference is exact
+                    const float S     = X_behind + (float)(total - (prefix + (double)X_end));
                     const float gconf = (dot * A) * inv - S / ((1.f - bconf) + 1e-9f);
                     float gt[4]       = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
