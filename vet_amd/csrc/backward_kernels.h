@@ -673,6 +673,14 @@ constexpr int kFuzzyDense      = 16;
 // wave-per-list kernel where some are long (no cut: the longest list alone would keep one lane busy for a millisecond),
 // and running both one after the other costs more than either, so the host picks one by the cut.
 constexpr int kFuzzyWalkCut    = 64;
+// The wave-per-list kernel is launched kFuzzyReplicas times over (grid.y): replica r takes every kFuzzyReplicas-th long
+// list of a wave's pixels. Long lists cluster (where a surface is seen edge-on a whole strip of pixels holds hundreds
+// of fragments each), and a wave takes its lists one after the other. Replica 0 adds its background sums to the row
+// the dense kernel left for the workgroup; the others write rows of their own, which fold_background_rows_kernel adds up
+// into kFuzzyFoldRows rows right behind the per-workgroup ones, so that the sum over the rows stays short:
+// [workgroups] [kFuzzyFoldRows] [replica 1: workgroups] [replica 2: workgroups] ...
+constexpr int kFuzzyReplicas   = 4;
+constexpr int kFuzzyFoldRows   = 256;
 constexpr int kFuzzyWalkColumn = 7;   // background row, column 7: the workgroup has a list for the walk kernel
 constexpr int kFuzzyLongColumn = 6;   // ... column 6: one for the wave-per-list kernel
 
@@ -1019,8 +1027,15 @@ __global__ void __launch_bounds__(kBlock) blend_backward_fuzzy_long_kernel(Backw
 {
     constexpr int kWaves = kBlock / kWave;
     __shared__ float red[kWaves][C];
-    float* row = a.background_partial + (size_t)blockIdx.x * kBackgroundRow;
-    if (row[kFuzzyLongColumn] == 0.f) return;
+    const uint32_t replica = blockIdx.y;
+    float* row      = a.background_partial + (size_t)blockIdx.x * kBackgroundRow;
+    float* row_mine = replica == 0u ? row
+                                    : a.background_partial + ((size_t)kFuzzyFoldRows + (size_t)replica * gridDim.x + blockIdx.x) * kBackgroundRow;
+    if (row[kFuzzyLongColumn] == 0.f)
+    {
+        if (replica != 0u && threadIdx.x < (uint32_t)kBackgroundRow) row_mine[threadIdx.x] = 0.f;
+        return;
+    }
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
     const TilePixel px = tile_pixel(a.tiles, a.ly);
     const FuzzyPixel f = fuzzy_pixel<C>(a, px);
@@ -1032,10 +1047,11 @@ __global__ void __launch_bounds__(kBlock) blend_backward_fuzzy_long_kernel(Backw
     auto everywhere = [&](float v, int src) { return __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(v), src)); };
 
     uint64_t todo = __ballot(f.n > max(walk_max, (uint32_t)kFuzzyDense));
-    while (todo != 0ull)
+    for (uint32_t turn = 0; todo != 0ull; ++turn)
     {
         const int src = __ffsll((unsigned long long)todo) - 1;
         todo &= todo - 1ull;
+        if (turn % (uint32_t)kFuzzyReplicas != replica) continue;
         // the pixel, the same on every lane
         const uint32_t n       = (uint32_t)__builtin_amdgcn_readlane((int)f.n, src);
         const uint64_t* list   = a.fragments + (uint32_t)__builtin_amdgcn_readlane((int)f.off, src);
@@ -1306,7 +1322,36 @@ __global__ void __launch_bounds__(kBlock) blend_backward_fuzzy_long_kernel(Backw
         if (lane == 0) red[wave][ci] = s;
     }
     __syncthreads();
-    if (threadIdx.x < C) row[threadIdx.x] += (red[0][threadIdx.x] + red[1][threadIdx.x]) + (red[2][threadIdx.x] + red[3][threadIdx.x]);
+    if (threadIdx.x < (uint32_t)kBackgroundRow)
+    {
+        const float sum = threadIdx.x < C ? (red[0][threadIdx.x] + red[1][threadIdx.x]) + (red[2][threadIdx.x] + red[3][threadIdx.x]) : 0.f;
+        if (replica == 0u)
+        {
+            if (threadIdx.x < C) row[threadIdx.x] += sum;
+        }
+        else
+            row_mine[threadIdx.x] = sum;
+    }
+}
+
+// Adds `num_rows` rows of kBackgroundRow floats up into kFuzzyFoldRows rows: workgroup j takes rows j, j + 256, ... in a
+// fixed order (32 threads per column, each every 32nd of the workgroup's rows, then the 32 partial sums one after the other).
+__global__ void __launch_bounds__(kBlock) fold_background_rows_kernel(const float* __restrict__ rows, int num_rows,
+                                                                      float* __restrict__ folded)
+{
+    __shared__ float part[kBlock / kBackgroundRow][kBackgroundRow];
+    const int column = threadIdx.x % kBackgroundRow, sub = threadIdx.x / kBackgroundRow;
+    float sum = 0.f;
+    for (int r = blockIdx.x + kFuzzyFoldRows * sub; r < num_rows; r += kFuzzyFoldRows * (kBlock / kBackgroundRow))
+        sum += rows[(size_t)r * kBackgroundRow + column];
+    part[sub][column] = sum;
+    __syncthreads();
+    if (threadIdx.x < (uint32_t)kBackgroundRow)
+    {
+        float total = 0.f;
+        for (int k = 0; k < kBlock / kBackgroundRow; ++k) total += part[k][threadIdx.x];
+        folded[(size_t)blockIdx.x * kBackgroundRow + threadIdx.x] = total;
+    }
 }
 
 // Sums the per-workgroup background rows of one view (one workgroup, fixed order, so the result is reproducible) and

@@ -554,7 +554,8 @@ int vetrast_workspace_layout_for_mode(int32_t N, int32_t B, int32_t L, int32_t w
     lay->partial_base       = at;
     at += align_up(cap * 8 * sizeof(float), kAlign);
     lay->background_partial_base = at;
-    at += align_up((size_t)tile_grid(make_tile_map(t, nullptr, true)) * kBackgroundRow * sizeof(float), kAlign);
+    // (the FUZZY_BLEND kernel that takes a wave per list keeps rows per replica and kFuzzyFoldRows rows they are folded into)
+    at += align_up(((size_t)tile_grid(make_tile_map(t, nullptr, true)) * kFuzzyReplicas + kFuzzyFoldRows) * kBackgroundRow * sizeof(float), kAlign);
     lay->camera_partial_base = at;
     at += align_up(((size_t)N + kBlock - 1) / kBlock * kCameraRow * sizeof(double), kAlign);
     lay->total_bytes = std::max(align_up(at, kAlign), lay->forward_only_bytes);
@@ -813,6 +814,8 @@ int vetrast_backward(vetrast_ctx* ctx, const vetrast_backward_args* g, void* str
     double* camera_rows            = ws_ptr<double>(ws, lay.camera_partial_base);
     float4* partial        = ws_ptr<float4>(ws, lay.partial_base);
     float* background_rows = ws_ptr<float>(ws, lay.background_partial_base);
+    const bool fuzzy_long  = p.render_mode == VETRAST_RENDER_FUZZY_BLEND &&
+                            (p.debug_max_list_length <= 0 || p.debug_max_list_length > kFuzzyWalkCut);
     for (int b = 0; b < B; ++b)
     {
         uint32_t* offsets   = ws_ptr<uint32_t>(ws, lay.offsets_base + lay.offsets_stride * b);
@@ -861,7 +864,15 @@ int vetrast_backward(vetrast_ctx* ctx, const vetrast_backward_args* g, void* str
                     if (beyond_dense && walks)
                         hipLaunchKernelGGL(blend_backward_fuzzy_walk_kernel<kC>, grid, blk, 0, stream, bp, p.depth_accept_blend, walk_max);
                     if (beyond_dense && !walks)
-                        hipLaunchKernelGGL(blend_backward_fuzzy_long_kernel<kC>, grid, blk, 0, stream, bp, p.depth_accept_blend, walk_max);
+                    {
+                        hipLaunchKernelGGL(blend_backward_fuzzy_long_kernel<kC>, dim3(grid.x, kFuzzyReplicas), blk, 0, stream, bp,
+                                           p.depth_accept_blend, walk_max);
+                        // the rows of replicas 1 .. into kFuzzyFoldRows rows behind the per-workgroup ones
+                        hipLaunchKernelGGL(fold_background_rows_kernel, dim3(kFuzzyFoldRows), blk, 0, stream,
+                                           bp.background_partial + ((size_t)kFuzzyFoldRows + grid.x) * kBackgroundRow,
+                                           (int)((kFuzzyReplicas - 1) * grid.x),
+                                           bp.background_partial + (size_t)grid.x * kBackgroundRow);
+                    }
                 };
                 switch (C)
                 {
@@ -908,7 +919,8 @@ int vetrast_backward(vetrast_ctx* ctx, const vetrast_backward_args* g, void* str
             gp.camera_partial      = want_camera ? camera_rows : nullptr;
             gp.accumulate          = (add_to_rows || b > 0) ? 1 : 0;
             gp.background_rows       = background_rows;
-            gp.num_background_rows   = (int)tile_grid(tiles);
+            // (with the folded rows of the FUZZY_BLEND kernel that takes a wave per list, where it ran)
+            gp.num_background_rows   = (int)tile_grid(tiles) + (fuzzy_long ? kFuzzyFoldRows : 0);
             gp.grad_background       = g->grad_background;
             gp.add_leak = (p.quirk_background_confidence_leak && !p.use_environment_map && hits == 1 &&
                            p.render_mode != VETRAST_RENDER_FUZZY_BLEND)
@@ -956,7 +968,7 @@ int vetrast_backward(vetrast_ctx* ctx, const vetrast_backward_args* g, void* str
         {
             ScopeTimer tm(ctx, stream, VETRAST_SCOPE_BACKWARD_GATHER);
             hipLaunchKernelGGL(reduce_background_kernel, dim3(1), dim3(kReduceBlock), 0, stream, background_rows,
-                               (int)(tile_grid(tiles)), C, g->grad_background, g->grad_confidence,
+                               (int)(tile_grid(tiles)) + (fuzzy_long ? kFuzzyFoldRows : 0), C, g->grad_background, g->grad_confidence,
                                0, b > 0 ? 1 : 0, p.texture_abs ? a->background : nullptr);
         }
     }
