@@ -39,8 +39,12 @@ def _scenes():
     yield "tiny_levels_nocut_3ch", _levels(synthetic.tiny_scene(num_points=5000, K=-1, channels=3, seed=82)), {}
     yield "tiny_long_lists_levels", _levels(synthetic.tiny_scene(num_points=40000, K=0, seed=83)), {}
     yield "tiny_long_lists_K16", _levels(synthetic.tiny_scene(num_points=40000, K=16, seed=84)), {}
-    # the backward pass takes lists beyond 16 fragments one lane per pixel while the cut is at most 64, else a wave per list
+    # a cut of 17 to 64 lays lists of up to 64 fragments out densely, in slots of 32 and 64 lanes that span rows of the
+    # wave (more slots than a wave's table holds at once: it goes through them in batches); beyond that cut lists of
+    # more than 16 fragments are taken a wave per list
+    yield "tiny_long_lists_K24", _levels(synthetic.tiny_scene(num_points=40000, K=24, seed=99)), {}
     yield "tiny_long_lists_K40", _levels(synthetic.tiny_scene(num_points=40000, K=40, seed=97)), {}
+    yield "tiny_long_lists_K64_3ch", _levels(synthetic.tiny_scene(num_points=40000, K=64, channels=3, seed=100)), {}
     yield "tiny_long_lists_K100", _levels(synthetic.tiny_scene(num_points=40000, K=100, seed=98)), {}
     yield "tiny_2views_envmap", _levels(synthetic.tiny_scene(num_points=3000, K=8, num_views=2, seed=85)), \
         {"use_environment_map": 1}
@@ -60,6 +64,10 @@ def _scenes():
     yield "background_in_last_bucket_K8", _far(synthetic.tiny_scene(num_points=3000, K=8, seed=95)), \
         {"depth_accept_blend": 9.0e3}
     yield "background_in_last_bucket_nocut", _far(synthetic.tiny_scene(num_points=30000, K=-1, seed=96)), \
+        {"depth_accept_blend": 9.0e3}
+    yield "range_reaches_zero_K48", synthetic.tiny_scene(num_points=8000, K=48, seed=101), {"depth_accept_blend": 2.0}
+    yield "one_bucket_K64", synthetic.tiny_scene(num_points=30000, K=64, seed=102), {"depth_accept_blend": 9.0e3}
+    yield "background_in_last_bucket_K32", _far(synthetic.tiny_scene(num_points=30000, K=32, seed=103)), \
         {"depth_accept_blend": 9.0e3}
     yield "single_fragments_K1", _levels(synthetic.tiny_scene(num_points=6000, K=1, seed=94)), {}
     yield "config1", synthetic.config1(), {"depth_accept_blend": 0.05}

@@ -357,242 +357,16 @@ __global__ void __launch_bounds__(kBlock) blend_backward_kernel(BackwardPass a)
 }
 
 // FUZZY_BLEND, per-pixel part of the backward pass: BlendBackwardsFuzzy<C>, src/lib/rendering/RenderBackward.cu:570-1080.
-// One lane per pixel walks its (cut) list front to back. Fragments are collected into a bucket while their depth
-// stays within depth_accept of the bucket's first one (every bucket, unlike the forward kernel, which only averages
-// the nearest one); the background, at depth 1e5, ends up in a bucket of its own. With the bucket's mean confidence c,
-// mean descriptor t, m elements and the transmittance A in front of it:
+// Fragments are collected into a bucket while their depth stays within depth_accept of the bucket's first one (every
+// bucket, unlike the forward kernel, which only averages the nearest one); the background, at depth 1e5, ends up in a
+// bucket of its own. With the bucket's mean confidence c, mean descriptor t, m elements and the transmittance A in
+// front of it:
 //   d tex_e[ci] = (A * c * g[ci]) / m,   d conf_e = (A * (t . g)) / m  -  S_b / (1 - c + 1e-9)
 // for each of its elements e, where S_b is the sum over all LATER buckets b' of sum_ci g[ci] t'[ci] A' c' (the
 // reference hands every element in front of a bucket the bucket's whole term, :654-672). The reference walks all
-// elements in front for every bucket; here the list is walked twice, first for the total of the bucket terms, then
-// with a running prefix, so that S_b = total - prefix. The position part (:729-1080) is the neighbour-difference
-// heuristic of the FULL_BLEND kernel. Records go to partial[layer][point] as there: the position part of an element's
-// record when the element is met in the second pass, the rest when its bucket closes, for which only the keys of the
-// bucket's elements are read again (gathering the descriptor records a third time cost a third of the kernel).
-
-// State of one pixel's walk over its list (one of the two passes at a time).
-template <int C>
-struct FuzzyWalk
-{
-    // the pixel
-    const BackwardPass* a;
-    const uint64_t* list;
-    float4* partial_l;
-    uint32_t n;  // fragments (after the cut)
-    float g[C], ax[C], ay[C], bx, by;
-    bool do_point;
-    float depth_accept;
-    float bg_grad[C];
-    double total, prefix;
-    // the pass
-    int pass;
-    float last_min, acc_conf, A, acc_t[C];
-    uint32_t m, start;
-    int first_id;  // point of the open bucket's first element
-
-    // Descriptor and confidence of list element e from memory; the background is the element behind the last fragment.
-    __device__ __forceinline__ void element(uint32_t e, float (&t)[C], float& conf, float& depth, int& id) const
-    {
-        id = -1;
-        if (e >= n)
-        {
-#pragma unroll
-            for (int ci = 0; ci < C; ++ci) t[ci] = a->background[ci];
-            conf  = 1.f;
-            depth = 100000.f;  // MAX_DEPTH_CONST, src/lib/rendering/RenderConstants.h:30
-            return;
-        }
-        const uint64_t key = list[e];
-        depth              = __uint_as_float((uint32_t)(key >> 32));
-        const int point    = (int)(uint32_t)key;
-        int ti             = -1;
-        if ((uint32_t)point < (uint32_t)a->N) ti = a->index ? a->index[point] : point;
-        float4 t4 = make_float4(0.f, 0.f, 0.f, 0.f);
-        conf      = 0.f;
-        if ((uint32_t)ti < (uint32_t)a->N)
-        {
-            t4   = a->packed[2 * (size_t)ti];
-            conf = a->packed[2 * (size_t)ti + 1].x;
-            id   = point;
-        }
-        const float tt[4] = {t4.x, t4.y, t4.z, t4.w};
-#pragma unroll
-        for (int ci = 0; ci < C; ++ci) t[ci] = tt[ci];
-    }
-
-    // The same for kChunk consecutive fragments e0 .. e0 + kChunk - 1 (those below n): all keys are asked for first, then
-    // all descriptor records, so that a chunk costs two memory round trips instead of two per fragment.
-    static constexpr int kChunk = 4;
-    __device__ __forceinline__ void elements(uint32_t e0, float (&t)[kChunk][C], float (&conf)[kChunk], float (&depth)[kChunk],
-                                             int (&id)[kChunk]) const
-    {
-        uint64_t key[kChunk];
-#pragma unroll
-        for (int u = 0; u < kChunk; ++u) key[u] = e0 + u < n ? list[e0 + u] : 0ull;
-        int ti[kChunk];
-#pragma unroll
-        for (int u = 0; u < kChunk; ++u)
-        {
-            const int point = (int)(uint32_t)key[u];
-            depth[u]        = __uint_as_float((uint32_t)(key[u] >> 32));
-            ti[u]           = -1;
-            id[u]           = -1;
-            if (e0 + u < n && (uint32_t)point < (uint32_t)a->N) ti[u] = a->index ? a->index[point] : point;
-            if ((uint32_t)ti[u] < (uint32_t)a->N)
-                id[u] = point;
-            else
-                ti[u] = -1;
-        }
-        float4 t4[kChunk], c4[kChunk];
-#pragma unroll
-        for (int u = 0; u < kChunk; ++u)
-        {
-            t4[u] = c4[u] = make_float4(0.f, 0.f, 0.f, 0.f);
-            if (ti[u] >= 0)
-            {
-                t4[u] = a->packed[2 * (size_t)ti[u]];
-                c4[u] = a->packed[2 * (size_t)ti[u] + 1];
-            }
-        }
-#pragma unroll
-        for (int u = 0; u < kChunk; ++u)
-        {
-            const float tt[4] = {t4[u].x, t4[u].y, t4[u].z, t4[u].w};
-#pragma unroll
-            for (int ci = 0; ci < C; ++ci) t[u][ci] = tt[ci];
-            conf[u] = c4[u].x;
-        }
-    }
-
-    __device__ __forceinline__ void begin_pass(int which)
-    {
-        pass     = which;
-        last_min = 0.f, acc_conf = 0.f, A = 1.f;
-#pragma unroll
-        for (int ci = 0; ci < C; ++ci) acc_t[ci] = 0.f;
-        m = 0, start = 0, first_id = -1;
-    }
-
-    // closes the bucket [start, start + m)
-    __device__ __forceinline__ void close_bucket()
-    {
-        const float inv  = 1.f / (float)m;
-        const float conf = acc_conf * inv;
-        float tb[C];
-        float dot = 0.f, x = 0.f;
-#pragma unroll
-        for (int ci = 0; ci < C; ++ci)
-        {
-            tb[ci] = acc_t[ci] * inv;
-            dot += tb[ci] * g[ci];
-            x += ((g[ci] * tb[ci]) * A) * conf;
-        }
-        if (pass == 0)
-            total += (double)x;
-        else
-        {
-            prefix += (double)x;
-            const float S      = (float)(total - prefix);
-            const float galpha = dot * A;
-            const float gconf  = galpha * inv - S / ((1.f - conf) + 1e-9f);
-            float gt[4]        = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-            for (int ci = 0; ci < C; ++ci) gt[ci] = ((A * conf) * g[ci]) * inv;
-            // every element of the bucket gets the bucket's descriptor and confidence gradient; the position part of
-            // its record was written when the element was consumed. Only the point ids are needed here: the keys are
-            // read again (neighbouring places, in cache), eight at a time so that the loads overlap, not the
-            // descriptor records.
-            auto give = [&](int id) {
-                partial_l[2 * (size_t)id] = make_float4(gt[0], gt[1], gt[2], gt[3]);
-                reinterpret_cast<float*>(&partial_l[2 * (size_t)id + 1])[0] = gconf;
-            };
-            if (m == 1)
-            {
-                if (start >= n)
-                {
-#pragma unroll
-                    for (int ci = 0; ci < C; ++ci) bg_grad[ci] += gt[ci];
-                }
-                else if (first_id >= 0)
-                    give(first_id);
-            }
-            else
-                for (uint32_t e0 = start; e0 < start + m; e0 += 8)
-                {
-                    int point[8];
-#pragma unroll
-                    for (int u = 0; u < 8; ++u)
-                    {
-                        const uint32_t e = e0 + u;
-                        point[u]         = (e < start + m && e < n) ? (int)(uint32_t)list[e] : -1;
-                    }
-#pragma unroll
-                    for (int u = 0; u < 8; ++u)
-                    {
-                        const uint32_t e = e0 + u;
-                        if (e >= start + m) break;
-                        if (e >= n)
-                        {
-#pragma unroll
-                            for (int ci = 0; ci < C; ++ci) bg_grad[ci] += gt[ci];
-                            continue;
-                        }
-                        int ti = -1;
-                        if ((uint32_t)point[u] < (uint32_t)a->N) ti = a->index ? a->index[point[u]] : point[u];
-                        if ((uint32_t)ti < (uint32_t)a->N) give(point[u]);
-                    }
-                }
-        }
-        A = (1.f - conf) * A;
-    }
-
-    // list element i joins the open bucket or starts the next one
-    __device__ __forceinline__ void consume(uint32_t i, const float (&t)[C], float conf, float d, int id)
-    {
-        if (!(d - last_min < depth_accept))
-        {
-            if (i != 0) close_bucket();
-            acc_conf = 0.f;
-            m        = 0;
-#pragma unroll
-            for (int ci = 0; ci < C; ++ci) acc_t[ci] = 0.f;
-            last_min = d;
-            start    = i;
-            first_id = id;
-        }
-        // (the first element of a list joins the bucket that is open from the start when its depth is within the range
-        // of zero: it is that bucket's first element all the same)
-        if (m == 0) first_id = id;
-        acc_conf += conf;
-#pragma unroll
-        for (int ci = 0; ci < C; ++ci) acc_t[ci] += t[ci];
-        ++m;
-        if (pass == 1 && id >= 0)
-        {
-            // the position part of the element's record does not depend on its bucket
-            float gp0 = 0.f, gp1 = 0.f;
-            if (do_point)
-            {
-                float dR_dpx = bx, dR_dpy = by;
-#pragma unroll
-                for (int ci = 0; ci < C; ++ci)
-                {
-                    dR_dpx += t[ci] * ax[ci];
-                    dR_dpy += t[ci] * ay[ci];
-                }
-                gp0 = dR_dpx / (float)C;
-                gp1 = dR_dpy / (float)C;
-            }
-            float* rec = reinterpret_cast<float*>(&partial_l[2 * (size_t)id + 1]);
-            rec[1] = gp0, rec[2] = gp1, rec[3] = 0.f;
-        }
-    }
-
-    __device__ __forceinline__ void end_pass()
-    {
-        if (m > 0) close_bucket();
-    }
-};
+// elements in front for every bucket, one thread per pixel; here the fragments of a pixel sit on neighbouring lanes and
+// S_b is a sum from the back. The position part (:729-1080) is the neighbour-difference heuristic of the FULL_BLEND
+// kernel. Records go to partial[layer][point] as there.
 
 // Value the lane D places below (above) in the same row of 16 lanes holds; the lane's own value where the row has no
 // such lane. DPP register moves; every lane of the wave must be active.
@@ -656,23 +430,23 @@ __device__ __forceinline__ FuzzyPixel fuzzy_pixel(const BackwardPass& a, const T
 // Lists of up to kFuzzyDense fragments are laid out densely, one lane per FRAGMENT, as in blend_backward_kernel; what is
 // different here is that a fragment's gradient depends on its whole bucket (means over the bucket's elements) and on
 // all buckets of its pixel (transmittance in front, bucket terms behind), so a pixel's fragments must sit in one step
-// of 64 lanes. Every pixel gets a slot of 1, 2, 4, 8 or 16 lanes (its list length rounded up to a power of two), the
-// slots are handed out largest first, which keeps each aligned to its own size: no slot crosses a row of 16 lanes,
-// the sums over a bucket, the transmittance product and the suffix sum of the bucket terms are shift-and-combine steps
-// inside a row (register moves), and steps need no carries between them. Only the bucket boundaries are a sequential
-// rule (a bucket starts where the depth leaves the range of the bucket's FIRST element), and that rule needs the
-// depths alone: all lanes of a slot run it together over the slot's depths. Sums and products are combined pairwise
-// instead of front to back, which moves the results by rounding only. The slots of a step are at most as long as its
-// first one, and the step's code is compiled once per slot length so that shorter slots take fewer combine steps.
-// Longer lists are left to blend_backward_fuzzy_walk_kernel; the workgroup says in column 7 of its background row
-// whether it has any.
-constexpr int kFuzzyDense      = 16;
-// Lists beyond the dense layout: `walk_max` (a kernel argument) is the longest list blend_backward_fuzzy_walk_kernel
-// takes, one lane per pixel; longer ones go to blend_backward_fuzzy_long_kernel, the whole wave per list. The walk is
-// the faster of the two while all lists are short (a cut of up to kFuzzyWalkCut: 64 pixels advance together), the
-// wave-per-list kernel where some are long (no cut: the longest list alone would keep one lane busy for a millisecond),
-// and running both one after the other costs more than either, so the host picks one by the cut.
-constexpr int kFuzzyWalkCut    = 64;
+// of 64 lanes. Every pixel gets a slot of 1, 2, 4 ... 64 lanes (its list length rounded up to a power of two), the
+// slots are handed out largest first, which keeps each aligned to its own size, and steps need no carries between
+// them. A slot of up to kFuzzyNarrow lanes lies inside a row of 16 lanes: the sums over a bucket, the transmittance
+// product and the sum of the bucket terms behind are shift-and-combine steps inside the row (register moves), and
+// the step's code is compiled once per slot length so that shorter slots take fewer of them (the slots of a step
+// are at most as long as its first). Slots of 32 and 64 lanes span rows: the same steps through the LDS crossbar, two
+// more of them. Only the bucket boundaries are a sequential rule (a bucket starts where the depth leaves the range of
+// the bucket's FIRST element), and that rule needs the depths alone: all lanes of a slot run it together over the
+// slot's depths. Sums and products are combined pairwise instead of front to back, which moves the results by
+// rounding only. The table that says which pixel a lane's fragment belongs to holds kWaveItems slots; a wave whose
+// pixels need more goes through it in batches. Longer lists are left to blend_backward_fuzzy_long_kernel; the
+// workgroup says in column kFuzzyLongColumn of its background row whether it has any.
+constexpr int kFuzzyDense      = 64;  // longest list of the dense layout
+constexpr int kFuzzyNarrow     = 16;  // longest slot that lies inside a row of 16 lanes
+// The kernel is compiled for DENSE = kFuzzyNarrow (no slot spans rows: fewer registers, more waves per SIMD) and for
+// DENSE = kFuzzyDense; the host takes the narrow one where the cut keeps every list that short.
+constexpr int kFuzzyLongColumn = 6;   // background row, column 6: the workgroup has a list for the wave-per-list kernel
 // The wave-per-list kernel is launched kFuzzyReplicas times over (grid.y): replica r takes every kFuzzyReplicas-th long
 // list of a wave's pixels. Long lists cluster (where a surface is seen edge-on a whole strip of pixels holds hundreds
 // of fragments each), and a wave takes its lists one after the other. Replica 0 adds its background sums to the row
@@ -681,11 +455,9 @@ constexpr int kFuzzyWalkCut    = 64;
 // [workgroups] [kFuzzyFoldRows] [replica 1: workgroups] [replica 2: workgroups] ...
 constexpr int kFuzzyReplicas   = 4;
 constexpr int kFuzzyFoldRows   = 256;
-constexpr int kFuzzyWalkColumn = 7;   // background row, column 7: the workgroup has a list for the walk kernel
-constexpr int kFuzzyLongColumn = 6;   // ... column 6: one for the wave-per-list kernel
 
-template <int C>
-__global__ void __launch_bounds__(kBlock) blend_backward_fuzzy_kernel(BackwardPass a, float depth_accept, uint32_t walk_max)
+template <int C, int DENSE>
+__global__ void __launch_bounds__(kBlock) blend_backward_fuzzy_kernel(BackwardPass a, float depth_accept)
 {
     constexpr int kWaves = kBlock / kWave;
     __shared__ uint32_t s_off[kWaves][kWave];
@@ -723,21 +495,23 @@ __global__ void __launch_bounds__(kBlock) blend_backward_fuzzy_kernel(BackwardPa
             s_bxy[wave][lane] = make_float2(f.bx, f.by);
         }
     }
-    const bool dense = n > 0 && n <= (uint32_t)kFuzzyDense;
+    const bool dense = n > 0 && n <= (uint32_t)DENSE;
     s_n[wave][lane]  = (uint8_t)(dense ? n : 0);
 
     // ---- slots, largest first ---------------------------------------------------------------------------------------
     const uint32_t size = dense ? (n > 1 ? 1u << (32 - __clz((int)n - 1)) : 1u) : 0u;
     uint32_t slot = 0, total = 0;
 #pragma unroll
-    for (uint32_t cls = kFuzzyDense; cls >= 1; cls >>= 1)
+    for (uint32_t cls = DENSE; cls >= 1; cls >>= 1)
     {
         const uint64_t members = __ballot(size == cls);
         if (size == cls) slot = total + cls * (uint32_t)__popcll(members & ((1ull << lane) - 1ull));
         total += cls * (uint32_t)__popcll(members);
     }
     s_slot[wave][lane] = (uint16_t)slot;
-    for (uint32_t j = 0; j < size; ++j) s_item[wave][slot + j] = j < n ? (uint8_t)lane : (uint8_t)255;
+    // the item table holds kWaveItems slots at a time: those from batch0 on (all of them unless slots span rows)
+    constexpr bool kBatched = DENSE * kWave > kWaveItems;
+    uint32_t batch0         = 0;
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
@@ -746,7 +520,7 @@ __global__ void __launch_bounds__(kBlock) blend_backward_fuzzy_kernel(BackwardPa
     auto step = [&](uint32_t k0, auto bound_constant) {
         constexpr uint32_t BOUND = decltype(bound_constant)::value;
         const uint32_t k = k0 + lane;
-        const int p      = k < total ? (int)s_item[wave][k] : 255;
+        const int p      = k < total ? (int)s_item[wave][k - batch0] : 255;
         const bool item  = p != 255;
         uint32_t np = 0, j = 0;
         int first = lane;  // first lane of the slot
@@ -764,7 +538,7 @@ __global__ void __launch_bounds__(kBlock) blend_backward_fuzzy_kernel(BackwardPa
             const int point    = (int)(uint32_t)key;
             int ti             = -1;
             // guards the gathers; never false for a workspace the forward pass wrote. An element that fails them
-            // counts as a fragment with a zero descriptor and confidence and gets no record, as in the walk.
+            // counts as a fragment with a zero descriptor and confidence and gets no record.
             if ((uint32_t)point < (uint32_t)a.N) ti = a.index ? a.index[point] : point;
             if ((uint32_t)ti < (uint32_t)a.N)
             {
@@ -923,20 +697,219 @@ __global__ void __launch_bounds__(kBlock) blend_backward_fuzzy_kernel(BackwardPa
             if (id_second >= 0) partial_l[2 * (size_t)id_second + odd] = v_second;
         }
     };
-    for (uint32_t k0 = 0; k0 < total; k0 += kWave)
+    // The same for slots of 32 or 64 lanes, which span rows: the combine steps go through the LDS crossbar instead of
+    // register moves inside a row, and two more of them reach across the slot. `bound`: the length of the step's first slot.
+    auto step_wide = [&](uint32_t k0, uint32_t bound) {
+        const uint32_t k = k0 + lane;
+        const int p      = k < total ? (int)s_item[wave][k - batch0] : 255;
+        const bool item  = p != 255;
+        uint32_t np = 0, j = 0;
+        int first = lane;  // first lane of the slot
+        float depth = 0.f, conf = 0.f;
+        float t[4]  = {0.f, 0.f, 0.f, 0.f};
+        float g[4]  = {0.f, 0.f, 0.f, 0.f};
+        int id = -1;
+        if (item)
+        {
+            np    = s_n[wave][p];
+            j     = k - s_slot[wave][p];
+            first = lane - (int)j;
+            const uint64_t key = a.fragments[s_off[wave][p] + j];
+            depth              = __uint_as_float((uint32_t)(key >> 32));
+            const int point    = (int)(uint32_t)key;
+            int ti             = -1;
+            // guards the gathers; never false for a workspace the forward pass wrote. An element that fails them
+            // counts as a fragment with a zero descriptor and confidence and gets no record.
+            if ((uint32_t)point < (uint32_t)a.N) ti = a.index ? a.index[point] : point;
+            if ((uint32_t)ti < (uint32_t)a.N)
+            {
+                const float4 t4 = a.packed[2 * (size_t)ti];
+                conf            = a.packed[2 * (size_t)ti + 1].x;
+                t[0] = t4.x, t[1] = t4.y, t[2] = t4.z, t[3] = t4.w;
+                id = point;
+            }
+            const float4 g4 = s_g[wave][p];
+            g[0] = g4.x, g[1] = g4.y, g[2] = g4.z, g[3] = g4.w;
+        }
+        // bucket boundaries (src/lib/rendering/RenderBackward.cu:706-714): element 0 opens the first bucket whether or
+        // not it resets the range
+        float last_min = 0.f;
+        uint64_t heads = 1ull;
+        for (uint32_t i = 0; i < bound; ++i)
+        {
+            const float di = __shfl(depth, (first + (int)i) & (kWave - 1), kWave);
+            if (i < np && !(di - last_min < depth_accept))
+            {
+                last_min = di;
+                heads |= 1ull << i;
+            }
+        }
+        // The background (depth MAX_DEPTH_CONST = 1e5, src/lib/rendering/RenderConstants.h:30) is a bucket of its own
+        // unless the last bucket's range reaches that far: then it is one more element of that bucket.
+        const bool bg_joins = with_background && (100000.f - last_min < depth_accept);
+
+        const uint32_t head  = 63u - (uint32_t)__clzll((long long)(heads & (j >= 63u ? ~0ull : (2ull << j) - 1ull)));  // first element of this bucket
+        const uint64_t later = j >= 63u ? 0ull : heads >> (j + 1u);
+        const uint32_t next  = later ? j + (uint32_t)__ffsll((unsigned long long)later) : np;  // first element of the next bucket
+        const uint32_t dist  = j - head;
+        const bool opens     = item && dist == 0u;
+        const bool in_last   = item && next == np;
+        const float inv      = 1.f / (float)(item ? next - head + (bg_joins && in_last ? 1u : 0u) : 1u);
+
+        // sums over the bucket: inclusive scan from the bucket's first lane, the last lane of the bucket has the sums
+        float sums[C + 1];
+        sums[C] = conf;
+#pragma unroll
+        for (int ci = 0; ci < C; ++ci) sums[ci] = t[ci];
+        {
+            const int last_lane = item ? first + (int)next - 1 : lane;
+#pragma unroll
+            for (int v = 0; v <= C; ++v)
+            {
+                float x = sums[v];
+#pragma unroll
+                for (int d = 1; d < kWave; d <<= 1)
+                {
+                    const float o = __shfl_up(x, d, kWave);
+                    if (dist >= (uint32_t)d) x += o;
+                }
+                sums[v] = __shfl(x, last_lane, kWave);
+            }
+        }
+        if (bg_joins && in_last)
+        {
+            sums[C] += 1.f;
+#pragma unroll
+            for (int ci = 0; ci < C; ++ci) sums[ci] += a.background[ci];
+        }
+        const float bconf = sums[C] * inv;
+        float dot = 0.f;
+#pragma unroll
+        for (int ci = 0; ci < C; ++ci) dot += (sums[ci] * inv) * g[ci];
+        // transmittance in front of the bucket: product of (1 - mean confidence) over the buckets before it
+        float P = opens ? 1.f - bconf : 1.f;
+        float A = 1.f, A_end = P;
+        {
+#pragma unroll
+            for (int d = 1; d < kWave; d <<= 1)
+            {
+                const float o = __shfl_up(P, d, kWave);
+                if (j >= (uint32_t)d) P *= o;
+            }
+            const float P_before = __shfl(P, (item && head > 0u) ? first + (int)head - 1 : lane, kWave);
+            A_end                = __shfl(P, item ? first + (int)np - 1 : lane, kWave);  // behind the last bucket
+            if (head > 0u) A = P_before;
+        }
+        // bucket terms behind this bucket (the background's included): suffix sum over the slot
+        float x = 0.f;
+#pragma unroll
+        for (int ci = 0; ci < C; ++ci) x += ((g[ci] * (sums[ci] * inv)) * A) * bconf;
+        float S = 0.f;
+        {
+            float Q = opens ? x : 0.f;
+#pragma unroll
+            for (int d = 1; d < kWave; d <<= 1)
+            {
+                const float o = __shfl_down(Q, d, kWave);
+                if (j + (uint32_t)d < np) Q += o;
+            }
+            const float Q_next = __shfl(Q, (item && next < np) ? first + (int)next : lane, kWave);
+            if (next < np) S = Q_next;
+        }
+        if (with_background && !bg_joins)
+        {
+            float xb = 0.f;
+#pragma unroll
+            for (int ci = 0; ci < C; ++ci) xb += ((g[ci] * a.background[ci]) * A_end) * 1.f;
+            S += xb;
+        }
+        if (with_background && item && j + 1u == np)
+        {
+            // the background's share: an element of the last bucket, or a bucket of its own behind all others
+            const float scale = bg_joins ? A * bconf : A_end * 1.f;
+            const float share = bg_joins ? inv : 1.f;
+#pragma unroll
+            for (int ci = 0; ci < C; ++ci) bg_grad[ci] += (scale * g[ci]) * share;
+        }
+        float4 rec_lo = make_float4(0.f, 0.f, 0.f, 0.f), rec_hi = rec_lo;
+        const bool give = item && id >= 0;
+        if (give)
+        {
+            const float gconf = (dot * A) * inv - S / ((1.f - bconf) + 1e-9f);
+            float gt[4]       = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int ci = 0; ci < C; ++ci) gt[ci] = ((A * bconf) * g[ci]) * inv;
+            float gp0 = 0.f, gp1 = 0.f;
+            if (s_point[wave][p] & 1)
+            {
+                // the position part of an element's record depends on its own descriptor, not on the bucket's
+                const float4 ax4 = s_ax[wave][p], ay4 = s_ay[wave][p];
+                const float2 b2  = s_bxy[wave][p];
+                const float ax[4] = {ax4.x, ax4.y, ax4.z, ax4.w}, ay[4] = {ay4.x, ay4.y, ay4.z, ay4.w};
+                float dR_dpx = b2.x, dR_dpy = b2.y;
+#pragma unroll
+                for (int ci = 0; ci < C; ++ci)
+                {
+                    dR_dpx += t[ci] * ax[ci];
+                    dR_dpy += t[ci] * ay[ci];
+                }
+                gp0 = dR_dpx / (float)C;
+                gp1 = dR_dpy / (float)C;
+            }
+            rec_lo = make_float4(gt[0], gt[1], gt[2], gt[3]);
+            rec_hi = make_float4(gconf, gp0, gp1, 0.f);
+        }
+        {
+            // record stores, two lanes per record (see blend_backward_kernel)
+            const int odd         = lane & 1;
+            const int own         = give ? id : -1;
+            const int other       = pair_other(own);
+            const float4 o_lo     = pair_other(rec_lo);
+            const float4 o_hi     = pair_other(rec_hi);
+            const int id_first    = odd ? other : own;
+            const int id_second   = odd ? own : other;
+            const float4 v_first  = odd ? o_hi : rec_lo;
+            const float4 v_second = odd ? rec_hi : o_lo;
+            if (id_first >= 0) partial_l[2 * (size_t)id_first + odd] = v_first;
+            if (id_second >= 0) partial_l[2 * (size_t)id_second + odd] = v_second;
+        }
+    };
+    for (uint32_t b0 = 0; b0 < total; b0 += kWaveItems)
     {
-        // the first slot of a step is its longest
-        const uint32_t n0 = (uint32_t)__builtin_amdgcn_readfirstlane((int)s_n[wave][s_item[wave][k0]]);
-        if (n0 > 8)
-            step(k0, std::integral_constant<uint32_t, 16>{});
-        else if (n0 > 4)
-            step(k0, std::integral_constant<uint32_t, 8>{});
-        else if (n0 > 2)
-            step(k0, std::integral_constant<uint32_t, 4>{});
-        else if (n0 > 1)
-            step(k0, std::integral_constant<uint32_t, 2>{});
-        else
-            step(k0, std::integral_constant<uint32_t, 1>{});
+        if constexpr (kBatched) batch0 = b0;
+        if (kBatched && batch0 != 0u)
+        {
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();  // every lane is done with the table of the batch before
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        }
+        // slots are aligned to their size and the table's size is a multiple of every size: none lies across two batches
+        if (size != 0u && slot >= batch0 && slot < batch0 + (uint32_t)kWaveItems)
+            for (uint32_t j = 0; j < size; ++j) s_item[wave][slot - batch0 + j] = j < n ? (uint8_t)lane : (uint8_t)255;
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        const uint32_t batch_end = min(total, batch0 + (uint32_t)kWaveItems);
+        for (uint32_t k0 = batch0; k0 < batch_end; k0 += kWave)
+        {
+            // the first slot of a step is its longest
+            const uint32_t n0 = (uint32_t)__builtin_amdgcn_readfirstlane((int)s_n[wave][s_item[wave][k0 - batch0]]);
+            if (DENSE > kFuzzyNarrow && n0 > (uint32_t)kFuzzyNarrow)
+            {
+                if constexpr (DENSE > kFuzzyNarrow) step_wide(k0, n0 > 32u ? 64u : 32u);
+            }
+            else if (n0 > 8)
+                step(k0, std::integral_constant<uint32_t, 16>{});
+            else if (n0 > 4)
+                step(k0, std::integral_constant<uint32_t, 8>{});
+            else if (n0 > 2)
+                step(k0, std::integral_constant<uint32_t, 4>{});
+            else if (n0 > 1)
+                step(k0, std::integral_constant<uint32_t, 2>{});
+            else
+                step(k0, std::integral_constant<uint32_t, 1>{});
+        }
+        if constexpr (!kBatched) break;
     }
 
 #pragma unroll
@@ -946,73 +919,18 @@ __global__ void __launch_bounds__(kBlock) blend_backward_fuzzy_kernel(BackwardPa
         if (lane == 0) red[wave][ci] = s;
     }
     {
-        const bool longer = __ballot(n > (uint32_t)kFuzzyDense && n <= walk_max) != 0ull;
-        const bool longest = __ballot(n > max(walk_max, (uint32_t)kFuzzyDense)) != 0ull;
+        const bool longest = __ballot(n > (uint32_t)DENSE) != 0ull;
         if (lane == 0) red[wave][C] = 0.f;  // no background-confidence leak in this mode (guarded, RenderBackward.cu:643)
-        if (lane == 0) red[wave][C + 1] = longer ? 1.f : 0.f;
-        if (lane == 0) red[wave][C + 2] = longest ? 1.f : 0.f;
+        if (lane == 0) red[wave][C + 1] = longest ? 1.f : 0.f;
     }
     __syncthreads();
     float* row = a.background_partial + (size_t)blockIdx.x * kBackgroundRow;
     if (threadIdx.x <= C) row[threadIdx.x] = (red[0][threadIdx.x] + red[1][threadIdx.x]) + (red[2][threadIdx.x] + red[3][threadIdx.x]);
     if (threadIdx.x == C + 1)
-        row[kFuzzyWalkColumn] = (red[0][C + 1] + red[1][C + 1]) + (red[2][C + 1] + red[3][C + 1]);
-    if (threadIdx.x == C + 2)
-        row[kFuzzyLongColumn] = (red[0][C + 2] + red[1][C + 2]) + (red[2][C + 2] + red[3][C + 2]);
+        row[kFuzzyLongColumn] = (red[0][C + 1] + red[1][C + 1]) + (red[2][C + 1] + red[3][C + 1]);
 }
 
-// The lists blend_backward_fuzzy_kernel left out (more than kFuzzyDense fragments): one lane per pixel walks its list
-// (FuzzyWalk). Same grid; a workgroup without such a list leaves at once. Launched where the list cut allows such lists.
-template <int C>
-__global__ void __launch_bounds__(kBlock) blend_backward_fuzzy_walk_kernel(BackwardPass a, float depth_accept, uint32_t walk_max)
-{
-    constexpr int kWaves = kBlock / kWave;
-    __shared__ float red[kWaves][C];
-    float* row = a.background_partial + (size_t)blockIdx.x * kBackgroundRow;
-    if (row[kFuzzyWalkColumn] == 0.f) return;
-    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
-    const TilePixel px = tile_pixel(a.tiles, a.ly);
-    const FuzzyPixel f = fuzzy_pixel<C>(a, px);
-    const bool walk    = f.n > (uint32_t)kFuzzyDense && f.n <= walk_max;
-    FuzzyWalk<C> w;
-    w.a = &a, w.list = a.fragments + f.off, w.partial_l = a.partial + 2 * (size_t)px.l * a.N, w.n = walk ? f.n : 0u;
-    w.do_point = f.do_point, w.depth_accept = depth_accept, w.total = w.prefix = 0.0;
-    w.bx = f.bx, w.by = f.by;
-#pragma unroll
-    for (int ci = 0; ci < C; ++ci) w.g[ci] = f.g[ci], w.ax[ci] = f.ax[ci], w.ay[ci] = f.ay[ci], w.bg_grad[ci] = 0.f;
-#pragma unroll 1
-    for (int pass = 0; pass < 2; ++pass)
-    {
-        w.begin_pass(pass);
-        for (uint32_t i0 = 0; i0 < w.n; i0 += FuzzyWalk<C>::kChunk)
-        {
-            float t[FuzzyWalk<C>::kChunk][C], conf[FuzzyWalk<C>::kChunk], d[FuzzyWalk<C>::kChunk];
-            int id[FuzzyWalk<C>::kChunk];
-            w.elements(i0, t, conf, d, id);
-#pragma unroll
-            for (int u = 0; u < FuzzyWalk<C>::kChunk; ++u)
-                if (i0 + u < w.n) w.consume(i0 + u, t[u], conf[u], d[u], id[u]);
-        }
-        if (walk && !a.use_environment_map)
-        {
-            float t[C], conf, d;
-            int id;
-            w.element(w.n, t, conf, d, id);  // the background behind the last fragment
-            w.consume(w.n, t, conf, d, id);
-        }
-        w.end_pass();
-    }
-#pragma unroll
-    for (int ci = 0; ci < C; ++ci)
-    {
-        const float s = wave_sum(w.bg_grad[ci]);
-        if (lane == 0) red[wave][ci] = s;
-    }
-    __syncthreads();
-    if (threadIdx.x < C) row[threadIdx.x] += (red[0][threadIdx.x] + red[1][threadIdx.x]) + (red[2][threadIdx.x] + red[3][threadIdx.x]);
-}
-
-// The lists blend_backward_fuzzy_kernel left out (more than kFuzzyDense fragments), one after the other, each by the
+// The lists blend_backward_fuzzy_kernel left out (more than `dense_max` fragments), one after the other, each by the
 // whole wave: 64 consecutive fragments per step, front to back, one lane per fragment. The bucket boundaries of a step
 // are found by a loop over its depths that every lane runs alike (the rule is sequential, but it needs the depths
 // only); sums over a bucket, the transmittance product over the buckets in front and the running sum of the bucket
@@ -1023,7 +941,7 @@ __global__ void __launch_bounds__(kBlock) blend_backward_fuzzy_walk_kernel(Backw
 // still open at the end of their step get the position part of their record there and the bucket's part when it
 // closes, from a loop over their keys. Same grid as the dense kernel; a workgroup without such a list leaves at once.
 template <int C>
-__global__ void __launch_bounds__(kBlock) blend_backward_fuzzy_long_kernel(BackwardPass a, float depth_accept, uint32_t walk_max)
+__global__ void __launch_bounds__(kBlock) blend_backward_fuzzy_long_kernel(BackwardPass a, float depth_accept, uint32_t dense_max)
 {
     constexpr int kWaves = kBlock / kWave;
     __shared__ float red[kWaves][C];
@@ -1046,7 +964,7 @@ __global__ void __launch_bounds__(kBlock) blend_backward_fuzzy_long_kernel(Backw
     for (int ci = 0; ci < C; ++ci) bg_grad[ci] = 0.f;
     auto everywhere = [&](float v, int src) { return __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(v), src)); };
 
-    uint64_t todo = __ballot(f.n > max(walk_max, (uint32_t)kFuzzyDense));
+    uint64_t todo = __ballot(f.n > dense_max);
     for (uint32_t turn = 0; todo != 0ull; ++turn)
     {
         const int src = __ffsll((unsigned long long)todo) - 1;

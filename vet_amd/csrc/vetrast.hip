@@ -815,7 +815,7 @@ int vetrast_backward(vetrast_ctx* ctx, const vetrast_backward_args* g, void* str
     float4* partial        = ws_ptr<float4>(ws, lay.partial_base);
     float* background_rows = ws_ptr<float>(ws, lay.background_partial_base);
     const bool fuzzy_long  = p.render_mode == VETRAST_RENDER_FUZZY_BLEND &&
-                            (p.debug_max_list_length <= 0 || p.debug_max_list_length > kFuzzyWalkCut);
+                            (p.debug_max_list_length <= 0 || p.debug_max_list_length > kFuzzyDense);
     for (int b = 0; b < B; ++b)
     {
         uint32_t* offsets   = ws_ptr<uint32_t>(ws, lay.offsets_base + lay.offsets_stride * b);
@@ -853,20 +853,21 @@ int vetrast_backward(vetrast_ctx* ctx, const vetrast_backward_args* g, void* str
             const dim3 grid(tile_grid(tiles)), blk(kBlock);
             if (p.render_mode == VETRAST_RENDER_FUZZY_BLEND)
             {
-                // Lists of more than kFuzzyDense fragments exist only where the cut allows them. With a cut of up to
-                // kFuzzyWalkCut they are walked one lane per pixel; otherwise each is taken by a whole wave.
+                // Lists of more than kFuzzyDense fragments exist only where the cut allows them; each is taken by a whole
+                // wave, in a second kernel.
                 const bool beyond_dense = bp.K <= 0 || bp.K > kFuzzyDense;
-                const bool walks        = bp.K > kFuzzyDense && bp.K <= kFuzzyWalkCut;
-                const uint32_t walk_max = walks ? (uint32_t)bp.K : (uint32_t)kFuzzyDense;
+                // With longer lists about, the narrow dense kernel in front of it is as fast as the wide one (measured).
+                const bool wide = !beyond_dense && bp.K > kFuzzyNarrow;
                 auto launch = [&](auto channels) {
                     constexpr int kC = decltype(channels)::value;
-                    hipLaunchKernelGGL(blend_backward_fuzzy_kernel<kC>, grid, blk, 0, stream, bp, p.depth_accept_blend, walk_max);
-                    if (beyond_dense && walks)
-                        hipLaunchKernelGGL(blend_backward_fuzzy_walk_kernel<kC>, grid, blk, 0, stream, bp, p.depth_accept_blend, walk_max);
-                    if (beyond_dense && !walks)
+                    if (wide)
+                        hipLaunchKernelGGL((blend_backward_fuzzy_kernel<kC, kFuzzyDense>), grid, blk, 0, stream, bp, p.depth_accept_blend);
+                    else
+                        hipLaunchKernelGGL((blend_backward_fuzzy_kernel<kC, kFuzzyNarrow>), grid, blk, 0, stream, bp, p.depth_accept_blend);
+                    if (beyond_dense)
                     {
                         hipLaunchKernelGGL(blend_backward_fuzzy_long_kernel<kC>, dim3(grid.x, kFuzzyReplicas), blk, 0, stream, bp,
-                                           p.depth_accept_blend, walk_max);
+                                           p.depth_accept_blend, (uint32_t)(wide ? kFuzzyDense : kFuzzyNarrow));
                         // the rows of replicas 1 .. into kFuzzyFoldRows rows behind the per-workgroup ones
                         hipLaunchKernelGGL(fold_background_rows_kernel, dim3(kFuzzyFoldRows), blk, 0, stream,
                                            bp.background_partial + ((size_t)kFuzzyFoldRows + grid.x) * kBackgroundRow,
