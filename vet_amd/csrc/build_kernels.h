@@ -353,22 +353,32 @@ __global__ void __launch_bounds__(kBlock) bin_build_kernel(BuildPass a)
             if ((uint32_t)tid < pixels)
             {
                 const uint32_t lo = max(start, base), hi = min(start + keep, base + (uint32_t)kStage);
-                for (uint32_t r = lo; r < hi && !saturated; ++r)
+                uint32_t r = lo;
+                if constexpr (FUZZY)
+                {
+                    // The nearest bucket, in a loop of its own, so that the loop below is FULL_BLEND's (which the
+                    // compiler unrolls, with the stage reads of several fragments in flight). What is stored is the
+                    // transmittance in front of the bucket the fragment joins.
+                    for (; r < hi && fuzzy.open; ++r)
+                    {
+                        const float4 t4 = s_stage[r - base][0];
+                        const float2 cd = *reinterpret_cast<const float2*>(&s_stage[r - base][1]);  // confidence, depth
+                        const float t[4] = {t4.x, t4.y, t4.z, t4.w};
+                        const bool joined = fuzzy.take(cd.y, cd.x, t, a.depth_accept, T, color);
+                        s_T[2 * r + 1] = T;
+                        ++used;
+                        if (joined) continue;
+                        const float Tc = T * cd.x;
+#pragma unroll
+                        for (int ci = 0; ci < C; ++ci) color[ci] = Tc * t[ci] + color[ci];
+                        T = (1.f - cd.x) * T;
+                    }
+                }
+                for (; r < hi && !saturated; ++r)
                 {
                     const float4 t4 = s_stage[r - base][0];
-                    const float2 cd = *reinterpret_cast<const float2*>(&s_stage[r - base][1]);  // confidence, depth
-                    const float cf  = cd.x;
+                    const float cf  = s_stage[r - base][1].x;
                     const float t[4] = {t4.x, t4.y, t4.z, t4.w};
-                    if constexpr (FUZZY)
-                    {
-                        // what is stored is the transmittance in front of the bucket the fragment joins
-                        if (fuzzy.open && fuzzy.take(cd.y, cf, t, a.depth_accept, T, color))
-                        {
-                            s_T[2 * r + 1] = T;
-                            ++used;
-                            continue;
-                        }
-                    }
                     s_T[2 * r + 1]  = T;
                     const float Tc   = T * cf;
 #pragma unroll
@@ -482,21 +492,29 @@ __global__ void __launch_bounds__(kBlock) bin_build_kernel(BuildPass a)
                 if ((uint32_t)tid < pixels)
                 {
                     const uint32_t lo = max(start, base), hi = min(start + keep, base + (uint32_t)kStage);
-                    for (uint32_t r = lo; r < hi && !saturated; ++r)
+                    uint32_t r = lo;
+                    if constexpr (FUZZY)
+                    {
+                        for (; r < hi && fuzzy.open; ++r)  // the nearest bucket, as above
+                        {
+                            const float4 t4 = s_stage[r - base][0];
+                            const float2 cd = *reinterpret_cast<const float2*>(&s_stage[r - base][1]);  // confidence, depth
+                            const float t[4] = {t4.x, t4.y, t4.z, t4.w};
+                            const bool joined = fuzzy.take(cd.y, cd.x, t, a.depth_accept, T, color);
+                            if (a.transmittance) a.transmittance[begin + r] = T;
+                            ++used;
+                            if (joined) continue;
+                            const float Tc = T * cd.x;
+#pragma unroll
+                            for (int ci = 0; ci < C; ++ci) color[ci] = Tc * t[ci] + color[ci];
+                            T = (1.f - cd.x) * T;
+                        }
+                    }
+                    for (; r < hi && !saturated; ++r)
                     {
                         const float4 t4 = s_stage[r - base][0];
-                        const float2 cd = *reinterpret_cast<const float2*>(&s_stage[r - base][1]);  // confidence, depth
-                        const float cf  = cd.x;
+                        const float cf  = s_stage[r - base][1].x;
                         const float t[4] = {t4.x, t4.y, t4.z, t4.w};
-                        if constexpr (FUZZY)
-                        {
-                            if (fuzzy.open && fuzzy.take(cd.y, cf, t, a.depth_accept, T, color))
-                            {
-                                if (a.transmittance) a.transmittance[begin + r] = T;
-                                ++used;
-                                continue;
-                            }
-                        }
                         if (a.transmittance) a.transmittance[begin + r] = T;
                         const float Tc = T * cf;
 #pragma unroll
