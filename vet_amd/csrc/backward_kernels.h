@@ -932,12 +932,14 @@ __global__ void __launch_bounds__(kBlock) blend_backward_fuzzy_kernel(BackwardPa
 
 // The lists blend_backward_fuzzy_kernel left out (more than `dense_max` fragments), one after the other, each by the
 // whole wave: 64 consecutive fragments per step, front to back, one lane per fragment. The bucket boundaries of a step
-// are found by a loop over its depths that every lane runs alike (the rule is sequential, but it needs the depths
-// only); sums over a bucket, the transmittance product over the buckets in front and the running sum of the bucket
+// are found by a loop over its buckets that every lane runs alike (the rule is sequential, but it needs the depths
+// only: all lanes test their depth against the open range at once, the first that fails opens the next bucket); sums
+// over a bucket, the transmittance product over the buckets in front and the running sum of the bucket
 // terms are scans over the lanes. What crosses a step boundary is carried in registers: the open bucket (sums, number
 // of elements, first element), the depth its range started at, the transmittance in front of it and the sum of the
 // bucket terms so far. A bucket's gradient needs the sum of the terms of all LATER buckets, so the list is processed
-// twice: the first pass only adds up the terms, the second has the total and writes. The elements of a bucket that was
+// twice: the first pass only adds up the terms, the second has the total and writes (a list of up to 64 fragments has
+// its total inside its one step and is processed once). The elements of a bucket that was
 // still open at the end of their step get the position part of their record there and the bucket's part when it
 // closes, from a loop over their keys. Same grid as the dense kernel; a workgroup without such a list leaves at once.
 template <int C>
@@ -979,9 +981,11 @@ __global__ void __launch_bounds__(kBlock) blend_backward_fuzzy_long_kernel(Backw
         for (int ci = 0; ci < 4; ++ci) g[ci] = everywhere(f.g[ci], src), ax[ci] = everywhere(f.ax[ci], src), ay[ci] = everywhere(f.ay[ci], src);
         const float bx = everywhere(f.bx, src), by = everywhere(f.by, src);
 
+        // A list that fits one step needs no first pass: the total is known inside the step.
+        const bool one_step = n <= (uint32_t)kWave;
         double total = 0.0;
 #pragma unroll 1
-        for (int pass = 0; pass < 2; ++pass)
+        for (int pass = one_step ? 1 : 0; pass < 2; ++pass)
         {
             // carried from step to step (the same on every lane)
             float open_sums[C + 1];
@@ -1016,15 +1020,15 @@ __global__ void __launch_bounds__(kBlock) blend_backward_fuzzy_long_kernel(Backw
                 }
                 // ---- bucket boundaries of this step (src/lib/rendering/RenderBackward.cu:706-714); element 0 of the
                 // list opens the first bucket whether or not it resets the range
+                // One trip per bucket, not per element: the elements that do not fit the open range are found by all
+                // lanes at once, the first of them opens the next bucket and sets the next range.
                 uint64_t heads = begin == 0 ? 1ull : 0ull;
-                for (uint32_t i = 0; i < valid; ++i)
+                for (uint64_t beyond = __ballot(has && !(depth - last_min < depth_accept)); beyond != 0ull;)
                 {
-                    const float di = everywhere(depth, (int)i);
-                    if (!(di - last_min < depth_accept))
-                    {
-                        last_min = di;
-                        heads |= 1ull << i;
-                    }
+                    const int i = __ffsll((unsigned long long)beyond) - 1;
+                    heads |= 1ull << i;
+                    last_min = everywhere(depth, i);
+                    beyond   = __ballot(has && lane > i && !(depth - last_min < depth_accept));
                 }
                 // the background (depth 1e5) behind the last fragment: one more element of the last bucket if that
                 // bucket's range reaches it, else a bucket of its own
@@ -1138,6 +1142,18 @@ __global__ void __launch_bounds__(kBlock) blend_backward_fuzzy_long_kernel(Backw
                     if (lane + d < kWave) X += o;
                 }
                 const float X_end = everywhere(X, 0);  // all of them
+                if (one_step)
+                {
+                    // what the first pass would have left, from the same terms in the same order
+                    total = (double)X_end;
+                    if (with_background && !bg_joins)
+                    {
+                        float xb = 0.f;
+#pragma unroll
+                        for (int ci = 0; ci < C; ++ci) xb += ((g[ci] * a.background[ci]) * (A_front * P_end)) * 1.f;
+                        total += (double)xb;
+                    }
+                }
                 if (pass == 1)
                 {
                     // behind this lane's bucket inside the step
