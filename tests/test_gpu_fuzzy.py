@@ -39,9 +39,9 @@ def _scenes():
     yield "tiny_levels_nocut_3ch", _levels(synthetic.tiny_scene(num_points=5000, K=-1, channels=3, seed=82)), {}
     yield "tiny_long_lists_levels", _levels(synthetic.tiny_scene(num_points=40000, K=0, seed=83)), {}
     yield "tiny_long_lists_K16", _levels(synthetic.tiny_scene(num_points=40000, K=16, seed=84)), {}
-    # a cut of 17 to 64 lays lists of up to 64 fragments out densely, in slots of 32 and 64 lanes that span rows of the
+    # a cut of 17 to 32 lays lists of up to 32 fragments out densely, in slots of 32 lanes that span two rows of the
     # wave (more slots than a wave's table holds at once: it goes through them in batches); beyond that cut lists of
-    # more than 16 fragments are taken a wave per list
+    # more than 16 fragments are taken a wave per list (those of up to 64 in one pass, longer ones in two)
     yield "tiny_long_lists_K24", _levels(synthetic.tiny_scene(num_points=40000, K=24, seed=99)), {}
     yield "tiny_long_lists_K40", _levels(synthetic.tiny_scene(num_points=40000, K=40, seed=97)), {}
     yield "tiny_long_lists_K64_3ch", _levels(synthetic.tiny_scene(num_points=40000, K=64, channels=3, seed=100)), {}
@@ -65,7 +65,8 @@ def _scenes():
         {"depth_accept_blend": 9.0e3}
     yield "background_in_last_bucket_nocut", _far(synthetic.tiny_scene(num_points=30000, K=-1, seed=96)), \
         {"depth_accept_blend": 9.0e3}
-    yield "range_reaches_zero_K48", synthetic.tiny_scene(num_points=8000, K=48, seed=101), {"depth_accept_blend": 2.0}
+    yield "range_reaches_zero_K28", synthetic.tiny_scene(num_points=8000, K=28, seed=101), {"depth_accept_blend": 2.0}
+    yield "range_reaches_zero_K48", synthetic.tiny_scene(num_points=8000, K=48, seed=104), {"depth_accept_blend": 2.0}
     yield "one_bucket_K64", synthetic.tiny_scene(num_points=30000, K=64, seed=102), {"depth_accept_blend": 9.0e3}
     yield "background_in_last_bucket_K32", _far(synthetic.tiny_scene(num_points=30000, K=32, seed=103)), \
         {"depth_accept_blend": 9.0e3}

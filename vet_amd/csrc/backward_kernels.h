@@ -430,22 +430,24 @@ __device__ __forceinline__ FuzzyPixel fuzzy_pixel(const BackwardPass& a, const T
 // Lists of up to kFuzzyDense fragments are laid out densely, one lane per FRAGMENT, as in blend_backward_kernel; what is
 // different here is that a fragment's gradient depends on its whole bucket (means over the bucket's elements) and on
 // all buckets of its pixel (transmittance in front, bucket terms behind), so a pixel's fragments must sit in one step
-// of 64 lanes. Every pixel gets a slot of 1, 2, 4 ... 64 lanes (its list length rounded up to a power of two), the
+// of 64 lanes. Every pixel gets a slot of 1, 2, 4 ... 32 lanes (its list length rounded up to a power of two), the
 // slots are handed out largest first, which keeps each aligned to its own size, and steps need no carries between
 // them. A slot of up to kFuzzyNarrow lanes lies inside a row of 16 lanes: the sums over a bucket, the transmittance
 // product and the sum of the bucket terms behind are shift-and-combine steps inside the row (register moves), and
 // the step's code is compiled once per slot length so that shorter slots take fewer of them (the slots of a step
-// are at most as long as its first). Slots of 32 and 64 lanes span rows: the same steps through the LDS crossbar, two
+// are at most as long as its first). A slot of 32 lanes spans two rows: the same steps through the LDS crossbar, one
 // more of them. Only the bucket boundaries are a sequential rule (a bucket starts where the depth leaves the range of
 // the bucket's FIRST element), and that rule needs the depths alone: all lanes of a slot run it together over the
 // slot's depths. Sums and products are combined pairwise instead of front to back, which moves the results by
 // rounding only. The table that says which pixel a lane's fragment belongs to holds kWaveItems slots; a wave whose
 // pixels need more goes through it in batches. Longer lists are left to blend_backward_fuzzy_long_kernel; the
 // workgroup says in column kFuzzyLongColumn of its background row whether it has any.
-constexpr int kFuzzyDense      = 64;  // longest list of the dense layout
+constexpr int kFuzzyDense      = 32;  // longest list of the dense layout
 constexpr int kFuzzyNarrow     = 16;  // longest slot that lies inside a row of 16 lanes
 // The kernel is compiled for DENSE = kFuzzyNarrow (no slot spans rows: fewer registers, more waves per SIMD) and for
-// DENSE = kFuzzyDense; the host takes the narrow one where the cut keeps every list that short.
+// DENSE = kFuzzyDense; the host takes the narrow one where the cut keeps every list that short, and also where lists
+// beyond kFuzzyDense may exist: those go to blend_backward_fuzzy_long_kernel, which then is the faster one for the lists
+// of 17 to 32 fragments as well (measured; slots of 64 lanes lost against it too).
 constexpr int kFuzzyLongColumn = 6;   // background row, column 6: the workgroup has a list for the wave-per-list kernel
 // The wave-per-list kernel is launched kFuzzyReplicas times over (grid.y): replica r takes every kFuzzyReplicas-th long
 // list of a wave's pixels. Long lists cluster (where a surface is seen edge-on a whole strip of pixels holds hundreds
@@ -697,8 +699,8 @@ __global__ void __launch_bounds__(kBlock) blend_backward_fuzzy_kernel(BackwardPa
             if (id_second >= 0) partial_l[2 * (size_t)id_second + odd] = v_second;
         }
     };
-    // The same for slots of 32 or 64 lanes, which span rows: the combine steps go through the LDS crossbar instead of
-    // register moves inside a row, and two more of them reach across the slot. `bound`: the length of the step's first slot.
+    // The same for slots that span rows (DENSE lanes at most): the combine steps go through the LDS crossbar instead of
+    // register moves inside a row, and more of them reach across the slot. `bound`: the length of the step's first slot.
     auto step_wide = [&](uint32_t k0, uint32_t bound) {
         const uint32_t k = k0 + lane;
         const int p      = k < total ? (int)s_item[wave][k - batch0] : 255;
@@ -768,7 +770,7 @@ __global__ void __launch_bounds__(kBlock) blend_backward_fuzzy_kernel(BackwardPa
             {
                 float x = sums[v];
 #pragma unroll
-                for (int d = 1; d < kWave; d <<= 1)
+                for (int d = 1; d < DENSE; d <<= 1)  // no slot is longer
                 {
                     const float o = __shfl_up(x, d, kWave);
                     if (dist >= (uint32_t)d) x += o;
@@ -791,7 +793,7 @@ __global__ void __launch_bounds__(kBlock) blend_backward_fuzzy_kernel(BackwardPa
         float A = 1.f, A_end = P;
         {
 #pragma unroll
-            for (int d = 1; d < kWave; d <<= 1)
+            for (int d = 1; d < DENSE; d <<= 1)  // no slot is longer
             {
                 const float o = __shfl_up(P, d, kWave);
                 if (j >= (uint32_t)d) P *= o;
@@ -808,7 +810,7 @@ __global__ void __launch_bounds__(kBlock) blend_backward_fuzzy_kernel(BackwardPa
         {
             float Q = opens ? x : 0.f;
 #pragma unroll
-            for (int d = 1; d < kWave; d <<= 1)
+            for (int d = 1; d < DENSE; d <<= 1)  // no slot is longer
             {
                 const float o = __shfl_down(Q, d, kWave);
                 if (j + (uint32_t)d < np) Q += o;

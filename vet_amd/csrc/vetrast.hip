@@ -856,7 +856,7 @@ int vetrast_backward(vetrast_ctx* ctx, const vetrast_backward_args* g, void* str
                 // Lists of more than kFuzzyDense fragments exist only where the cut allows them; each is taken by a whole
                 // wave, in a second kernel.
                 const bool beyond_dense = bp.K <= 0 || bp.K > kFuzzyDense;
-                // With longer lists about, the narrow dense kernel in front of it is as fast as the wide one (measured).
+                // With longer lists about, the narrow dense kernel in front of that one is faster than the wide one (measured).
                 const bool wide = !beyond_dense && bp.K > kFuzzyNarrow;
                 auto launch = [&](auto channels) {
                     constexpr int kC = decltype(channels)::value;
