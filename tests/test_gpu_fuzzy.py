@@ -46,6 +46,11 @@ def _scenes():
     yield "tiny_long_lists_K40", _levels(synthetic.tiny_scene(num_points=40000, K=40, seed=97)), {}
     yield "tiny_long_lists_K64_3ch", _levels(synthetic.tiny_scene(num_points=40000, K=64, channels=3, seed=100)), {}
     yield "tiny_long_lists_K100", _levels(synthetic.tiny_scene(num_points=40000, K=100, seed=98)), {}
+    # the lengths either side of a change of method: 17 (first slot of 32 lanes), 33 (first list for the wave-per-list
+    # kernel under a cut beyond 32), 65 (first list of two steps: one element in the second)
+    yield "tiny_long_lists_K17", _levels(synthetic.tiny_scene(num_points=40000, K=17, seed=105)), {}
+    yield "tiny_long_lists_K33", _levels(synthetic.tiny_scene(num_points=40000, K=33, seed=106)), {}
+    yield "tiny_long_lists_K65", _levels(synthetic.tiny_scene(num_points=40000, K=65, seed=107)), {}
     yield "tiny_2views_envmap", _levels(synthetic.tiny_scene(num_points=3000, K=8, num_views=2, seed=85)), \
         {"use_environment_map": 1}
     yield "wide_depth_range", synthetic.tiny_scene(num_points=5000, K=12, seed=86), {"depth_accept_blend": 0.3}
@@ -68,6 +73,7 @@ def _scenes():
     yield "range_reaches_zero_K28", synthetic.tiny_scene(num_points=8000, K=28, seed=101), {"depth_accept_blend": 2.0}
     yield "range_reaches_zero_K48", synthetic.tiny_scene(num_points=8000, K=48, seed=104), {"depth_accept_blend": 2.0}
     yield "one_bucket_K64", synthetic.tiny_scene(num_points=30000, K=64, seed=102), {"depth_accept_blend": 9.0e3}
+    yield "one_bucket_K65", synthetic.tiny_scene(num_points=30000, K=65, seed=108), {"depth_accept_blend": 9.0e3}
     yield "background_in_last_bucket_K32", _far(synthetic.tiny_scene(num_points=30000, K=32, seed=103)), \
         {"depth_accept_blend": 9.0e3}
     yield "single_fragments_K1", _levels(synthetic.tiny_scene(num_points=6000, K=1, seed=94)), {}
