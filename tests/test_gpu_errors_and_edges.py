@@ -283,13 +283,16 @@ def test_two_contexts_on_two_streams_do_not_disturb_each_other(rasterizer, oracl
                 assert torch.equal(grads[k], v), (k, frame)
 
 
-def test_empty_cloud(rasterizer):
+@pytest.mark.parametrize("mode", ["full", "fuzzy_no_cut", "bilinear"])
+def test_empty_cloud(rasterizer, mode):
     """num_points = 0 (the buffers exist, they are just not read): every pixel shows the background, the background
     gradient is the plain sum of the incoming gradients, nothing else is touched or launched on the points."""
-    print("[case] empty cloud", flush=True)
+    print(f"[case] empty cloud, {mode}", flush=True)
     scene = synthetic.tiny_scene(num_points=8, w=40, h=24, num_layers=3, seed=58)
     dev = DeviceScene(scene)
-    params = make_params(scene, need_point_gradient=1)
+    over = {"full": {}, "bilinear": {"render_mode": abi.RENDER_BILINEAR_BLEND},
+            "fuzzy_no_cut": {"render_mode": abi.RENDER_FUZZY_BLEND, "depth_accept_blend": 0.05, "debug_max_list_length": -1}}[mode]
+    params = make_params(scene, need_point_gradient=1, **over)
     full = rasterizer.forward(dev, params)  # sizes the workspace and the outputs
     torch.cuda.synchronize()
     args = full.args
