@@ -13,6 +13,22 @@
 
 namespace vetrast
 {
+// Small accumulators of the call (pose and intrinsics gradients and their counts) that have to start at zero: the first
+// workgroup of the first view's per-pixel kernel clears them, which is in front of every kernel that adds to them in
+// stream order and saves the launches of a fill kernel each.
+struct ClearJob
+{
+    uint32_t* ptr[4];
+    uint32_t count[4];  // 32-bit words; 0 = nothing to clear
+};
+__device__ __forceinline__ void clear_small_accumulators(const ClearJob& job)
+{
+    if (blockIdx.x != 0 || blockIdx.y != 0) return;
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+        for (uint32_t i = threadIdx.x; i < job.count[k]; i += blockDim.x) job.ptr[k][i] = 0u;
+}
+
 struct BackwardPass
 {
     const uint32_t* offsets;
@@ -36,6 +52,7 @@ struct BackwardPass
     int use_environment_map;
     int need_point_gradient;
     int quirk_background_confidence_leak;
+    ClearJob clear;
 };
 
 // Sum over the 64 lanes (xor butterfly, widest step first); every lane gets the total. The four steps inside a row of
@@ -101,6 +118,7 @@ __global__ void __launch_bounds__(kBlock) blend_backward_kernel(BackwardPass a)
     __shared__ uint8_t s_item[kWaves][kWaveItems];
     __shared__ float red[kWaves][C + 1];
 
+    clear_small_accumulators(a.clear);
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
     const TilePixel px = tile_pixel(a.tiles, a.ly);
     const int l        = px.l;
@@ -472,6 +490,7 @@ __global__ void __launch_bounds__(kBlock) blend_backward_fuzzy_kernel(BackwardPa
     __shared__ float2 s_bxy[kWaves][kWave];
     __shared__ uint8_t s_item[kWaves][kWaveItems];
     __shared__ float red[kWaves][C + 3];
+    clear_small_accumulators(a.clear);
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
     const TilePixel px = tile_pixel(a.tiles, a.ly);
     float4* partial_l  = a.partial + 2 * (size_t)px.l * a.N;

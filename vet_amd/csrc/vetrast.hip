@@ -779,6 +779,8 @@ int vetrast_backward(vetrast_ctx* ctx, const vetrast_backward_args* g, void* str
     // PointRenderer.cu:267-277 are only needed where rows are added to with atomics: with a texture index
     // indirection, where several points may share a row.
     const bool add_to_rows = a->index != nullptr;
+    ClearJob clear          = {};
+    constexpr size_t kClearByKernel = 16384;  // words one workgroup clears in passing
     {
         ScopeTimer tm(ctx, stream, VETRAST_SCOPE_BACKWARD_PREPARE);
         auto zero = [&](float* ptr, size_t n) {
@@ -786,15 +788,33 @@ int vetrast_backward(vetrast_ctx* ctx, const vetrast_backward_args* g, void* str
             hipLaunchKernelGGL(fill_u32_kernel, dim3(std::min(grid_for(n), 8192)), dim3(kBlock), 0, stream,
                                reinterpret_cast<uint32_t*>(ptr), n, 0u);
         };
+        // the pose and intrinsics accumulators: by the first view's per-pixel kernel where they are small (ClearJob)
+        const size_t pose_words = (size_t)12 * a->num_poses, camera_words = (size_t)13 * a->num_cameras;
         if (g->grad_pose)
         {
-            zero(reinterpret_cast<float*>(g->grad_pose), (size_t)12 * a->num_poses);
-            zero(g->grad_pose_count, (size_t)a->num_poses);
+            if (pose_words <= kClearByKernel)
+            {
+                clear.ptr[0] = reinterpret_cast<uint32_t*>(g->grad_pose), clear.count[0] = (uint32_t)pose_words;
+                clear.ptr[1] = reinterpret_cast<uint32_t*>(g->grad_pose_count), clear.count[1] = (uint32_t)a->num_poses;
+            }
+            else
+            {
+                zero(reinterpret_cast<float*>(g->grad_pose), pose_words);
+                zero(g->grad_pose_count, (size_t)a->num_poses);
+            }
         }
         if (g->grad_intrinsics)
         {
-            zero(g->grad_intrinsics, (size_t)13 * a->num_cameras);
-            zero(g->grad_intrinsics_count, (size_t)a->num_cameras);
+            if (camera_words <= kClearByKernel)
+            {
+                clear.ptr[2] = reinterpret_cast<uint32_t*>(g->grad_intrinsics), clear.count[2] = (uint32_t)camera_words;
+                clear.ptr[3] = reinterpret_cast<uint32_t*>(g->grad_intrinsics_count), clear.count[3] = (uint32_t)a->num_cameras;
+            }
+            else
+            {
+                zero(g->grad_intrinsics, camera_words);
+                zero(g->grad_intrinsics_count, (size_t)a->num_cameras);
+            }
         }
         if (add_to_rows)
         {
@@ -841,6 +861,7 @@ int vetrast_backward(vetrast_ctx* ctx, const vetrast_backward_args* g, void* str
             bp.use_environment_map              = p.use_environment_map;
             bp.need_point_gradient              = want_image_gradient ? 1 : 0;
             bp.quirk_background_confidence_leak = p.quirk_background_confidence_leak;
+            bp.clear                            = b == 0 ? clear : ClearJob{};
             for (int l = 0; l < VETRAST_MAX_LAYERS; ++l)
             {
                 bp.grad_out[l] = nullptr;
