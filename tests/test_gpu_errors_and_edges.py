@@ -318,3 +318,36 @@ def test_empty_cloud(rasterizer, mode):
     exact = sum(x.astype(np.float64).sum(axis=(0, 2, 3)) for x in scene.grad_out())
     assert max_rel_err(gb.cpu().numpy(), exact) <= 1e-5
     assert not gt.any() and not gc.any()
+
+
+@pytest.mark.parametrize("num_poses", [2, 40, 3000])
+def test_camera_accumulators_are_cleared(rasterizer, oracle, num_poses):
+    """The pose and intrinsics gradients are sums over the views of a call and are cleared inside the call: by the first
+    per-pixel kernel where they are small, by a fill kernel of their own where they are not (3 000 pose rows). The call
+    is replayed onto outputs full of NaN; rows no view uses must come back as exact zeros."""
+    print(f"[case] camera accumulators, {num_poses} pose rows", flush=True)
+    scene = synthetic.tiny_scene(num_points=4000, num_views=2, seed=61)
+    have = scene.poses_se3.shape[0]
+    if num_poses > have:
+        scene.poses_se3 = np.ascontiguousarray(np.concatenate(
+            [scene.poses_se3, np.tile(scene.poses_se3[:1], (num_poses - have, 1))]))
+    params = make_params(scene, need_point_gradient=1)
+    dev = DeviceScene(scene)
+    res = rasterizer.forward(dev, params, save_for_backward=True)
+    grad_out = scene.grad_out()
+    got = rasterizer.backward(res, [torch.from_numpy(x).cuda() for x in grad_out], want_cameras=True)
+    torch.cuda.synchronize()
+    for key in ("pose", "pose_count", "intrinsics", "intrinsics_count"):
+        got[key].fill_(float("nan"))
+    abi.check(rasterizer.lib.vetrast_backward(rasterizer.ctx, C.byref(got["_args"]), None), "backward again")
+    torch.cuda.synchronize()
+    want = oracle.backward(oracle.forward(scene, params), grad_out, want_points=True, want_cameras=True)
+    used = sorted({v.image_index for v in scene.views})
+    pose = got["pose"].cpu().numpy()
+    assert np.isfinite(pose).all() and np.isfinite(got["intrinsics"].cpu().numpy()).all()
+    unused = np.setdiff1d(np.arange(pose.shape[0]), used)
+    assert not pose[unused].any() and not got["pose_count"].cpu().numpy()[unused].any()
+    np.testing.assert_array_equal(got["pose_count"].cpu().numpy(), want["pose_count"])
+    np.testing.assert_array_equal(got["intrinsics_count"].cpu().numpy(), want["intrinsics_count"])
+    assert max_rel_err(pose, want["pose"]) <= 1e-3
+    assert max_rel_err(got["intrinsics"].cpu().numpy(), want["intrinsics"]) <= 1e-3
