@@ -376,45 +376,6 @@ def time_training_crops(steps, samples, render_mode):
     return out
 
 
-def time_access_floor(scene, steps, samples):
-    """The bare access pattern of the per-pixel backward kernel on the frame's real lists (vet_amd/csrc/ubench/
-    access_floor.hip): every list place streams its key and transmittance; with `gather` it also reads its point's
-    32-byte descriptor record, with `scatter` it stores a 32-byte record at the point's place. No arithmetic, no
-    per-pixel data: the time of the memory accesses alone."""
-    import torch
-
-    from vet_amd.rasterizer import DeviceScene, Rasterizer, make_params
-
-    path = os.path.join(ROOT, "vet_amd", "lib", "libaccess_floor.so")
-    if not os.path.exists(path):
-        raise FileNotFoundError(f"{path} is not built (python -m vet_amd.build)")
-    lib = C.CDLL(path)
-    rast = Rasterizer()
-    fwd = rast.forward(DeviceScene(scene), make_params(scene, need_point_gradient=1))
-    torch.cuda.synchronize()
-    off = fwd.offsets(0)
-    F, N = int(off[-1]), scene.num_points
-    kept = int(np.minimum(np.diff(off), scene.max_list_length).sum()) if scene.max_list_length > 0 else F
-    bases = fwd.layer_bases()
-    firsts = [int(off[bases[l]]) if l < scene.num_layers else F for l in range(1, 4)]
-    frags = torch.from_numpy(fwd.fragments(0).astype(np.uint64).view(np.int64)).cuda()
-    trans = torch.from_numpy(fwd.transmittance(0).astype(np.float32)).cuda()
-    packed = torch.randn(N * 8, device="cuda")
-    partial = torch.empty(4 * N * 8, device="cuda")
-    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
-    ptr = lambda t: C.c_void_p(t.data_ptr())
-    out = {"list_places": F, "of_them_blended": kept,
-           "what": "one thread per list place of the frame's real lists: stream key + transmittance, gather the point's "
-                   "32-byte descriptor record, store a 32-byte record at the point's place; no arithmetic"}
-    for name, what in (("stream_only", 0), ("gather", 1), ("scatter", 2), ("gather_and_scatter", 3)):
-        def run():
-            rc = lib.access_floor_run(ptr(frags), ptr(trans), ptr(packed), ptr(partial), F, N, firsts[0], firsts[1],
-                                      firsts[2], what, stream)
-            assert rc == 0, rc
-        out[name + "_us"] = round(timed_samples(run, 3, steps, samples)["median"] * 1e3, 1)
-    return out
-
-
 def host_threads(requested):
     """Threads for the CPU legs: every core this process may run on, within the worker limit the box sets for a job
     (OMP_NUM_THREADS where the environment has it). Returns (threads, cores visible, limit or None)."""
@@ -447,11 +408,6 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--lift-only", action="store_true",
                     help="time only the error lifting on the configuration's scene and print its object")
-    ap.add_argument("--atomics-ubench", action="store_true",
-                    help="run the stand-alone microbenchmark of scattered atomics / loads / stores and print its table")
-    ap.add_argument("--access-floor", action="store_true",
-                    help="time the bare gather / scatter pattern of the per-pixel backward kernel on the frame's real lists "
-                         "and print its object")
     ap.add_argument("--cpu-threads", type=int, default=0,
                     help="0 = every core this process may use, within the box's worker limit (OMP_NUM_THREADS)")
     args = ap.parse_args()
@@ -459,15 +415,6 @@ def main():
         print("bench.py: this build runs the rasterizer on ONE GPU (views of a batch are rendered back to back); "
               "--gpus N with N > 1 is not available", file=sys.stderr)
         sys.exit(2)
-
-    if args.atomics_ubench:
-        import subprocess
-
-        exe = os.path.join(ROOT, "vet_amd", "lib", "ubench_atomics")
-        if not os.path.exists(exe):
-            print(f"bench.py: {exe} is not built (python -m vet_amd.build)", file=sys.stderr)
-            sys.exit(2)
-        sys.exit(subprocess.run([exe]).returncode)  # a child process; this one has not touched the GPU
 
     import torch
 
@@ -484,9 +431,6 @@ def main():
     backward = args.config != 2
     scene = make(**kw)
     cpu_threads, cores_visible, cores_limit = host_threads(args.cpu_threads)
-    if args.access_floor:
-        print(json.dumps({"access_floor": time_access_floor(scene, args.steps, args.samples)}))
-        return
     if args.lift_only:
         print(json.dumps({"lift_error": time_lift_error(scene, args.steps, 0 if args.no_cpu_baseline else cpu_threads)}))
         return

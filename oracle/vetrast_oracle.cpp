@@ -418,8 +418,11 @@ struct PointGrad
 // crop transform scaled by 0.5^layer (all five coefficients, rendering/RenderBackward.cu:1381-1385 and :3100-3106):
 // image-space gradient (gxp, gyp) of layer l -> gradients of the point, the pose tangent and fx, fy, cx, cy, s.
 // J_point = R, J_p_div = [1/z 0 -x/z^2; 0 1/z -y/z^2].
+// with_distortion: the camera model carries the distortion step (vetrast_params.allow_distortion), so its Jacobians
+// take part even where every coefficient is zero: d(xd, yd)/d(x, y) is then exactly the identity and the coefficient
+// gradients J_dis_dis^T (rendering/PointRendererHelper.h:346-368) are not zero (x r^2 and so on).
 inline PointGrad project_point_backward(const Prepared& cam, const vetrast_view& v, int l, const float* p4, float gxp,
-                                        float gyp)
+                                        float gyp, bool with_distortion)
 {
     PointGrad o;
     for (int k = 0; k < 3; ++k) o.gp[k] = 0.f;
@@ -441,7 +444,7 @@ inline PointGrad project_point_backward(const Prepared& cam, const vetrast_view&
         float d0 = cam.fx * a2;  // J_p_K1^T
         float d1 = cam.s * a2 + cam.fy * b2;
         float nx = vx / vz, ny = vy / vz;  // the point K is applied to
-        if (cam.has_dist)
+        if (cam.has_dist || with_distortion)
         {
             // J_dis_dis^T and J_p_dis^T (rendering/PointRendererHelper.h:346-368)
             float J[4], Jd[16], xd, yd;
@@ -615,7 +618,7 @@ void bilinear_pixel_backward(const vetrast_backward_args* g, const Scene& s, int
         const float gxp    = J[blend_index][0] * grad_blend_single;
         const float gyp    = J[blend_index][1] * grad_blend_single;
         const int point_id = get_point_id(full_buffer_pos);
-        const PointGrad pg = project_point_backward(cam, v, l, a->position + 4 * (size_t)point_id, gxp, gyp);
+        const PointGrad pg = project_point_backward(cam, v, l, a->position + 4 * (size_t)point_id, gxp, gyp, a->params.allow_distortion != 0);
         scatter_point_grad(g, v, point_id, pg, 1.f, pr.K_gradient_factor, par);  // pose count +1 here (:3146)
     }
 }
@@ -1158,7 +1161,7 @@ extern "C" int vetref_backward(const vetrast_backward_args* g, const uint32_t* o
                         }
                         const float gxp = dR_dpx / float(C), gyp = dR_dpy / float(C);  // :1374
                         const PointGrad pg =
-                            project_point_backward(cam, v, l, a->position + 4 * (size_t)point_id, gxp, gyp);
+                            project_point_backward(cam, v, l, a->position + 4 * (size_t)point_id, gxp, gyp, a->params.allow_distortion != 0);
                         scatter_point_grad(g, v, point_id, pg, 1.f / 1024.f, pr.K_gradient_factor, par);
                     }
                 }

@@ -67,19 +67,33 @@ def test_without_the_switch_the_camera_is_refused(rasterizer):
     assert rasterizer.check_device_flags(res) == abi.OK
 
 
-def test_zero_coefficients_with_the_switch_on_are_the_plain_camera(rasterizer):
+def test_zero_coefficients_with_the_switch_on_are_the_plain_camera(rasterizer, oracle):
+    """All coefficients zero, switch on: the same images and the same gradients bit for bit as with the switch off (the
+    distortion Jacobian is exactly the identity there), except the eight distortion columns of the intrinsics gradient,
+    which hold J_dis_dis^T (src/lib/rendering/PointRendererHelper.h:346-368) and are not zero: checked against the
+    oracle, whose values tests/test_oracle_distortion.py pins against central differences."""
     scene = synthetic.tiny_scene(num_points=4000, K=8, seed=53)
     dev = DeviceScene(scene)
-    grad_out = [torch.from_numpy(g).cuda() for g in scene.grad_out()]
+    go = scene.grad_out()
+    grad_out = [torch.from_numpy(g).cuda() for g in go]
     plain = rasterizer.forward(dev, make_params(scene, need_point_gradient=1))
     plain_g = {k: v.clone() for k, v in rasterizer.backward(plain, grad_out, want_cameras=True).items() if k != "_args"}
-    on = rasterizer.forward(dev, make_params(scene, need_point_gradient=1, allow_distortion=1))
+    params = make_params(scene, need_point_gradient=1, allow_distortion=1)
+    on = rasterizer.forward(dev, params)
     on_g = rasterizer.backward(on, grad_out, want_cameras=True)
     torch.cuda.synchronize()
     for a, b in zip(plain.out, on.out):
         assert torch.equal(a, b)
     for k, v in plain_g.items():
-        assert torch.equal(on_g[k], v), k
+        if k == "intrinsics":
+            assert torch.equal(on_g[k][:, :5], v[:, :5]), k
+            assert not v[:, 5:].any()
+        else:
+            assert torch.equal(on_g[k], v), k
+    want = oracle.backward(oracle.forward(scene, params), go, want_cameras=True)
+    got = on_g["intrinsics"].cpu().numpy()
+    assert np.abs(got[0, 5:]).min() > 0
+    assert max_rel_err(got[:, 5:], want["intrinsics"][:, 5:]) <= 1e-4
 
 
 def test_through_the_shim(oracle):

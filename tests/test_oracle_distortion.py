@@ -130,16 +130,21 @@ def test_distortion_moves_the_fragments(oracle):
     assert not np.array_equal(plain.offsets, bent.offsets)
 
 
-def test_gradients_match_central_differences(oracle):
+@pytest.mark.parametrize("coefficients", [[0.15, -0.04, 0.006, 0.05, -0.012, 0.002, 0.004, -0.003], [0.0] * 8],
+                         ids=["bent", "all_zero"])
+def test_gradients_match_central_differences(coefficients, oracle):
     """Point, pose, K and distortion gradients = sum over fragments of J^T dR/dp with J the central-difference
     Jacobian of the float64 distorted projection; the eight distortion columns carry the reference's weights
-    (1, 1, 0.25, 0.1, 0.1, 0.1, 0.1, 0.1) x distortion_gradient_factor."""
+    (1, 1, 0.25, 0.1, 0.1, 0.1, 0.1, 0.1) x distortion_gradient_factor. With the switch on that also holds for a
+    camera whose coefficients are all zero (ProjectPointPinholeBackward returns J_dis_dis^T whatever their values,
+    src/lib/rendering/PointRendererHelper.h:346-368): the derivative with respect to k1 at k1 = 0 is x r^2, not 0, so
+    such a camera can start to learn its distortion."""
     scene = synthetic.tiny_scene(num_points=500, w=24, h=16, num_layers=2, K=3, seed=44)
     ang = -0.15
     scene.views[0].crop_transform = (1.05, 0.95, 0.5, 1.0, 0.02)
     scene.views[0].crop_rotation = (np.cos(ang), -np.sin(ang), np.sin(ang), np.cos(ang))
     scene.intrinsics[0, 4] = 0.2
-    scene.intrinsics[0, 5:] = [0.15, -0.04, 0.006, 0.05, -0.012, 0.002, 0.004, -0.003]
+    scene.intrinsics[0, 5:] = coefficients
     q = np.array([0.03, 0.04, -0.02, 1.0])
     scene.poses_se3[0, :4] = q / np.linalg.norm(q)
     factor = 0.25

@@ -37,27 +37,6 @@ def build_library(verbose=True):
     return LIB_PATH
 
 
-UBENCH_PATH = os.path.join(LIB_DIR, "ubench_atomics")
-ACCESS_FLOOR_PATH = os.path.join(LIB_DIR, "libaccess_floor.so")
-
-
-def build_microbenchmarks(verbose=True):
-    """Stand-alone measurement programs (vet_amd/csrc/ubench): nothing in the library depends on them."""
-    os.makedirs(LIB_DIR, exist_ok=True)
-    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
-    cmd = [hipcc, "--offload-arch=gfx950", "-O3", "-std=c++17", "-Xclang", "-target-feature", "-Xclang",
-           "-packed-fp32-ops", os.path.join(CSRC, "ubench", "atomics.hip"), "-o", UBENCH_PATH]
-    if verbose:
-        print(" ".join(cmd), flush=True)
-    subprocess.run(cmd, check=True)
-    cmd = [hipcc, "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared", "-Xclang", "-target-feature", "-Xclang",
-           "-packed-fp32-ops", os.path.join(CSRC, "ubench", "access_floor.hip"), "-o", ACCESS_FLOOR_PATH]
-    if verbose:
-        print(" ".join(cmd), flush=True)
-    subprocess.run(cmd, check=True)
-    return UBENCH_PATH
-
-
 TORCH_EXT_PATH = os.path.join(LIB_DIR, "vetrast_torch.so")
 
 
@@ -92,6 +71,4 @@ if __name__ == "__main__":
     if "--lib-only" not in sys.argv:
         build_torch_extension()
         print("built", TORCH_EXT_PATH)
-        build_microbenchmarks()
-        print("built", UBENCH_PATH)
     sys.exit(0)

@@ -1521,17 +1521,18 @@ __global__ void __launch_bounds__(kBlock) gather_point_gradients_kernel(GatherPa
                 float nx = vx / vz, ny = vy / vz;  // the point K is applied to
                 if constexpr (DISTORT)
                 {
-                    if (cam.has_dist)
-                    {
-                        // J_dis_dis^T and J_p_dis^T of the distortion (src/lib/rendering/PointRendererHelper.h:346-368)
-                        float J[4], Jd[16], xd, yd;
-                        distort_point_jacobians(cam.dist, nx, ny, xd, yd, J, Jd);
+                    // J_dis_dis^T and J_p_dis^T of the distortion (src/lib/rendering/PointRendererHelper.h:346-368). The
+                    // kernel is compiled in this form for callers that have switched distortion on, whatever the
+                    // coefficients are: where all of them are zero J is exactly the identity (the other gradients keep
+                    // their bits) and the coefficient gradients are not zero (x r^2 and so on), so such a camera can
+                    // start to learn its distortion.
+                    float J[4], Jd[16], xd, yd;
+                    distort_point_jacobians(cam.dist, nx, ny, xd, yd, J, Jd);
 #pragma unroll
-                        for (int k = 0; k < 8; ++k) cam_sum[10 + k] += Jd[2 * k] * d0 + Jd[2 * k + 1] * d1;
-                        const float n0 = J[0] * d0 + J[2] * d1, n1 = J[1] * d0 + J[3] * d1;
-                        d0 = n0, d1 = n1;
-                        nx = xd, ny = yd;
-                    }
+                    for (int k = 0; k < 8; ++k) cam_sum[10 + k] += Jd[2 * k] * d0 + Jd[2 * k + 1] * d1;
+                    const float n0 = J[0] * d0 + J[2] * d1, n1 = J[1] * d0 + J[3] * d1;
+                    d0 = n0, d1 = n1;
+                    nx = xd, ny = yd;
                 }
                 const float iz = 1.f / vz;
                 const float e0 = iz * d0, e1 = iz * d1;
