@@ -206,47 +206,6 @@ typedef struct vetrast_workspace_layout
     size_t projected_base, projected_stride; /* per view, float [N][2], BILINEAR_BLEND only (stride 0 otherwise): image
                                                 position of every visible point at layer 0, from which the blend and its
                                                 backward pass form the bilinear weights */
-    /* ---- The region-major path. A FULL_BLEND call whose cloud is expected to leave a few hundred points per 16x16
-     * pixels of layer 0 (vetrast_forward_uses_regions says whether a call does) keeps its lists in another form, in
-     * the same workspace: the arrays above are then not written, the ones below are (all zero for the other modes).
-     * A REGION is 16x16 pixels of layer 0 plus the 8x8, 4x4, 2x2, 1 pixels of the coarser layers over the same area;
-     * pixel (x, y) of layer l has the number
-     *   q = region_pixels * ((y >> (4 - l)) * regions_x + (x >> (4 - l)))
-     *       + region_layer_first[l] + ((y & (s - 1)) << (4 - l)) + (x & (s - 1)),   s = 16 >> l.
-     * The pass over the points leaves one 32-byte record per point and region the point touches in the region's room
-     * (region_room records each): uint32 [8] = pixel numbers inside the region of the layers it hits there (8, 6, 4,
-     * 2, 0 bits from bit 0, 8, 14, 18, 20), depth bits, point id | layer mask << 27, confidence, descriptor [4].
-     * bin_counts_base then holds, per view, uint32 [num_regions]: records per region. A region with at most
-     * region_room records keeps its lists as slots (uint16 at region_list_slot_base: index of the record in the
-     * region's room); a region with more (a HEAVY region) as keys (uint64 at region_list_key_base, depth bits << 32 |
-     * point id, every list sorted in full). The list of pixel q holds count(q) places from place first(region) +
-     * start(q) on, where first = region * num_layers * region_room and (start, count) = (pixel_info[q].x & 0xFFFF,
-     * pixel_info[q].x >> 16) for a region built from slots, first = region_info[region].x and (start, count) =
-     * heavy_pixel[q] for a heavy one; the first min(count, K) places are the sorted fragments that were blended. */
-    int32_t region_pixels;                            /* pixels of a region over all layers */
-    int32_t region_room;                              /* records a region has room for */
-    int32_t region_layer_first[VETRAST_MAX_LAYERS + 1];
-    int32_t regions_x;                                /* regions per row = ceil(w / 16) */
-    int32_t reserved2;
-    int64_t num_regions;                              /* regions of one view */
-    size_t region_counters_base;                      /* per view, uint32 [16], 64 bytes apart: [0] list places handed out
-                                                         to heavy regions */
-    size_t region_views_base;                         /* prepared per-view camera constants */
-    size_t region_rooms_base, region_rooms_stride;    /* per view, uint32 [num_regions][region_room][8] */
-    size_t region_info_base, region_info_stride;      /* per view, uint32 [num_regions][2]: first list place, list places */
-    size_t region_pixel_info_base, region_pixel_info_stride;   /* per view, uint32 [num_regions * region_pixels][2]:
-                                                                  start | count << 16, bits of the final transmittance */
-    size_t region_heavy_pixel_base, region_heavy_pixel_stride; /* per view, uint32 [num_regions * region_pixels][2]:
-                                                                  start, count of the pixels of heavy regions */
-    size_t region_list_slot_base, region_list_slot_stride;     /* per view, uint16 [num_regions * L * region_room] */
-    size_t region_list_T_base, region_list_T_stride;           /* per view, float, the same places: transmittance in front
-                                                                  of every blended fragment */
-    size_t region_list_key_base, region_list_key_stride;       /* per view, uint64 [fragment_capacity] (heavy regions) */
-    size_t region_heavy_T_base, region_heavy_T_stride;         /* per view, float [fragment_capacity], the same places */
-    size_t region_log_base;                /* uint32 [256][segment][4]: records beyond a region's room (forward scratch) */
-    size_t region_partial_base;            /* float [L][N][8]: backward scratch, on top of the log */
-    size_t region_background_partial_base; /* float [num_regions][8] */
-    size_t region_camera_partial_base;     /* double [ceil(N/256)][20] */
 } vetrast_workspace_layout;
 
 /* Arguments of the forward pass. Replaces the inputs PointRender::forward receives
@@ -328,12 +287,6 @@ int vetrast_workspace_layout_for(int32_t num_points, int32_t num_views, int32_t 
 int vetrast_workspace_layout_for_mode(int32_t num_points, int32_t num_views, int32_t num_layers, int32_t w, int32_t h,
                                       int32_t render_mode, vetrast_workspace_layout* layout);
 size_t vetrast_forward_workspace_bytes(int32_t num_points, int32_t num_views, int32_t num_layers, int32_t w, int32_t h);
-
-/* 1 if a forward call with these arguments keeps its lists in the region-major form of vetrast_workspace_layout, 0 if
- * in the per-layer form, negative on invalid arguments. Only readers of the workspace need to know; results do not
- * depend on it. Pure host arithmetic on num_points, the image size, the layers, the render mode and
- * params.expected_fragments. */
-int vetrast_forward_uses_regions(const vetrast_forward_args* args);
 
 /* Forward: project, count, scan, fill, per-pixel sort by (depth bits, point id), top-K cut, front-to-back blend.
  * Replaces BlendPointCloudForward in FULL_BLEND mode (src/lib/rendering/PointRenderer.cu:657-1069). */

@@ -126,8 +126,8 @@ def test_processing_order_changes_nothing(mode, rasterizer):
 
 @pytest.mark.parametrize("mode", [abi.RENDER_FULL_BLEND, abi.RENDER_BILINEAR_BLEND])
 def test_expected_fragments_hint_changes_nothing(mode, rasterizer):
-    """vetrast_params.expected_fragments only sizes the pixel bins (and decides whether FULL_BLEND builds its lists
-    region by region): a crop that sees a part of the cloud gives the same lists, images and gradients with the true counts, with counts far too small (records overflow their bins' rooms
+    """vetrast_params.expected_fragments only sizes the pixel bins: a crop that sees a part of the cloud gives the same
+    lists, images and gradients with the true counts, with counts far too small (records overflow their bins' rooms
     and take the log path) and with counts far too large as with none."""
     scene = synthetic.config2(num_points=120_000, w=480, h=270, K=8)
     scene.views = [synthetic.ViewSpec(128, 96, crop_transform=(1.0, 1.0, -170.0, -90.0, 0.0)),
@@ -151,14 +151,7 @@ def test_expected_fragments_hint_changes_nothing(mode, rasterizer):
         for a, b in zip(res.out, plain.out):
             assert torch.equal(a, b)
         for k, v in plain_g.items():
-            if res.regions == plain.regions:
-                assert torch.equal(got[k], v), k
-            else:
-                # FULL_BLEND keeps its lists region by region where the hint says that a region holds a few hundred
-                # records, per layer otherwise: the same fragments, but a point's gradient terms are added up in
-                # another order (per region and then over the regions, instead of layer after layer): the bar between
-                # the two is the one each of them is held to against the CPU check
-                assert k == "point_count" and torch.equal(got[k], v) or max_rel_err(got[k].cpu().numpy(), v.cpu().numpy()) <= 1e-4, k
+            assert torch.equal(got[k], v), k
 
 
 def _backward_pair(scene, overrides, rasterizer, oracle, want_points=True):

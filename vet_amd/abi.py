@@ -102,25 +102,6 @@ class WorkspaceLayout(C.Structure):
         ("primary_base", C.c_size_t), ("log_base", C.c_size_t), ("log_cursor_base", C.c_size_t),
         ("last_key_base", C.c_size_t), ("last_key_stride", C.c_size_t),
         ("projected_base", C.c_size_t), ("projected_stride", C.c_size_t),
-        # the region-major path
-        ("region_pixels", C.c_int32), ("region_room", C.c_int32),
-        ("region_layer_first", C.c_int32 * (MAX_LAYERS + 1)),
-        ("regions_x", C.c_int32), ("reserved2", C.c_int32),
-        ("num_regions", C.c_int64),
-        ("region_counters_base", C.c_size_t),
-        ("region_views_base", C.c_size_t),
-        ("region_rooms_base", C.c_size_t), ("region_rooms_stride", C.c_size_t),
-        ("region_info_base", C.c_size_t), ("region_info_stride", C.c_size_t),
-        ("region_pixel_info_base", C.c_size_t), ("region_pixel_info_stride", C.c_size_t),
-        ("region_heavy_pixel_base", C.c_size_t), ("region_heavy_pixel_stride", C.c_size_t),
-        ("region_list_slot_base", C.c_size_t), ("region_list_slot_stride", C.c_size_t),
-        ("region_list_T_base", C.c_size_t), ("region_list_T_stride", C.c_size_t),
-        ("region_list_key_base", C.c_size_t), ("region_list_key_stride", C.c_size_t),
-        ("region_heavy_T_base", C.c_size_t), ("region_heavy_T_stride", C.c_size_t),
-        ("region_log_base", C.c_size_t),
-        ("region_partial_base", C.c_size_t),
-        ("region_background_partial_base", C.c_size_t),
-        ("region_camera_partial_base", C.c_size_t),
     ]
 
 
@@ -205,7 +186,6 @@ SYMBOLS = {
     "vetrast_workspace_layout_for_mode": (C.c_int, [C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_int32,
                                                     C.POINTER(WorkspaceLayout)]),
     "vetrast_forward_workspace_bytes": (C.c_size_t, [C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_int32]),
-    "vetrast_forward_uses_regions": (C.c_int, [C.POINTER(ForwardArgs)]),
     "vetrast_forward": (C.c_int, [C.c_void_p, C.POINTER(ForwardArgs), C.c_void_p]),
     "vetrast_backward": (C.c_int, [C.c_void_p, C.POINTER(BackwardArgs), C.c_void_p]),
     "vetrast_adam_step": (C.c_int, [C.c_void_p, C.POINTER(AdamArgs), C.c_void_p]),

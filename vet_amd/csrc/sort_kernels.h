@@ -11,8 +11,6 @@
 // sorts by depth only and leaves lists beyond 4096 entries partly unsorted (:290). Here the order is total
 // (depth, then point id) and exact for every length.
 #pragma once
-#include <type_traits>
-
 #include "common.h"
 
 namespace vetrast
@@ -24,67 +22,58 @@ __device__ __forceinline__ uint64_t shfl_u64(uint64_t v, int src)
     return ((uint64_t)hi << 32) | lo;
 }
 
-// The order of the keys. Every sorting routine below takes it as an argument: KeyLess is the order of the 64-bit keys
-// as numbers, (depth bits, point id); a caller whose keys carry something else than the point id in their low word
-// hands over an order that looks the id up where two depths are equal.
-struct KeyLess
-{
-    __device__ __forceinline__ bool operator()(uint64_t a, uint64_t b) const { return a < b; }
-};
-
 // One compare-exchange stage with partner lane ^ M: lanes for which keep_min holds keep the smaller key of the pair.
-template <int M, class Less>
-__device__ __forceinline__ uint64_t exchange(uint64_t key, int lane, bool keep_min, const Less& less)
+template <int M>
+__device__ __forceinline__ uint64_t exchange(uint64_t key, int lane, bool keep_min)
 {
     const uint32_t lo    = lane_xor<M>((uint32_t)key, lane);
     const uint32_t hi    = lane_xor<M>((uint32_t)(key >> 32), lane);
     const uint64_t other = ((uint64_t)hi << 32) | lo;
-    const bool take      = keep_min ? less(other, key) : less(key, other);
+    const bool take      = keep_min ? (other < key) : (other > key);
     return take ? other : key;
 }
 
-template <int K2, int J, class Less>
-__device__ __forceinline__ uint64_t halving_steps(uint64_t key, int lane, const Less& less)
+template <int K2, int J>
+__device__ __forceinline__ uint64_t halving_steps(uint64_t key, int lane)
 {
     if constexpr (J >= 1)
     {
-        key = exchange<J>(key, lane, (lane & J) == 0, less);
-        key = halving_steps<K2, (J >> 1)>(key, lane, less);
+        key = exchange<J>(key, lane, (lane & J) == 0);
+        key = halving_steps<K2, (J >> 1)>(key, lane);
     }
     return key;
 }
 
-template <int K2, int MAXK, class Less>
-__device__ __forceinline__ uint64_t bitonic_stages(uint64_t key, int lane, const Less& less)
+template <int K2, int MAXK>
+__device__ __forceinline__ uint64_t bitonic_stages(uint64_t key, int lane)
 {
     if constexpr (K2 <= MAXK)
     {
-        key = exchange<K2 - 1>(key, lane, (lane & (K2 >> 1)) == 0, less);  // mirror step inside every block of K2 lanes
-        key = halving_steps<K2, (K2 >> 2)>(key, lane, less);
-        key = bitonic_stages<K2 * 2, MAXK>(key, lane, less);
+        key = exchange<K2 - 1>(key, lane, (lane & (K2 >> 1)) == 0);  // mirror step inside every block of K2 lanes
+        key = halving_steps<K2, (K2 >> 2)>(key, lane);
+        key = bitonic_stages<K2 * 2, MAXK>(key, lane);
     }
     return key;
 }
 
 // Ascending bitonic sort of every aligned group of 2^LOG lanes (all-ascending form: a mirror step, then halving
 // steps), LOG = 1..6.
-template <int LOG, class Less = KeyLess>
-__device__ __forceinline__ uint64_t bitonic_sort_groups(uint64_t key, int lane, const Less& less = Less())
+template <int LOG>
+__device__ __forceinline__ uint64_t bitonic_sort_groups(uint64_t key, int lane)
 {
-    return bitonic_stages<2, (1 << LOG)>(key, lane, less);
+    return bitonic_stages<2, (1 << LOG)>(key, lane);
 }
 
 // Halving steps only: sorts a bitonic sequence held by the 64 lanes.
-template <class Less = KeyLess>
-__device__ __forceinline__ uint64_t bitonic_merge64(uint64_t key, int lane, const Less& less = Less())
+__device__ __forceinline__ uint64_t bitonic_merge64(uint64_t key, int lane)
 {
-    return halving_steps<64, 32>(key, lane, less);
+    return halving_steps<64, 32>(key, lane);
 }
 
 // Sort `count` lists of class LOG (2^(LOG-1) < n <= 2^LOG) found in the wave; src_lane[r] is the lane that owns the r-th.
-template <int LOG, class Less>
+template <int LOG>
 __device__ __forceinline__ void sort_class(uint64_t* fragments, const uint8_t* src_lane, int count,
-                                           uint32_t off, uint32_t n, int lane, int K, const Less& less)
+                                           uint32_t off, uint32_t n, int lane, int K)
 {
     constexpr int m        = 1 << LOG;
     constexpr int per_pass = kWave >> LOG;
@@ -98,18 +87,7 @@ __device__ __forceinline__ void sort_class(uint64_t* fragments, const uint8_t* s
         uint32_t nn      = __shfl(n, src, kWave);
         if (!valid) nn = 0;
         uint64_t key = ((uint32_t)e < nn) ? fragments[o + e] : kInfKey;
-        if constexpr (std::is_same<Less, KeyLess>::value)
-            key = bitonic_sort_groups<LOG>(key, lane, less);
-        else
-        {
-            // An order that differs from the keys' own only where two high words (depths) are equal: sort by the keys
-            // as numbers, which is cheaper, and only where two neighbours of a sorted list then share a depth (rare)
-            // run the network again with the caller's order.
-            key                  = bitonic_sort_groups<LOG>(key, lane, KeyLess());
-            const uint32_t hi    = (uint32_t)(key >> 32);
-            const uint32_t after = (uint32_t)__shfl_down((int)hi, 1, kWave);
-            if (__ballot((uint32_t)e + 1u < nn && hi == after) != 0ull) key = bitonic_sort_groups<LOG>(key, lane, less);
-        }
+        key          = bitonic_sort_groups<LOG>(key, lane);
         const uint32_t keep = (K > 0) ? min(nn, (uint32_t)K) : nn;
         if ((uint32_t)e < keep) fragments[o + e] = key;
     }
@@ -118,28 +96,26 @@ __device__ __forceinline__ void sort_class(uint64_t* fragments, const uint8_t* s
 // K smallest keys (K <= 64) of a list longer than 64, sorted, written to its first K places. The wave keeps the 64
 // smallest keys seen so far in sorted order; a chunk of 64 further keys is looked at only if one of them beats the
 // current K-th smallest.
-template <class Less>
-__device__ __forceinline__ void select_smallest(uint64_t* list, uint32_t n, int lane, int K, const Less& less)
+__device__ __forceinline__ void select_smallest(uint64_t* list, uint32_t n, int lane, int K)
 {
     uint64_t best = list[lane];  // n > 64
-    best          = bitonic_sort_groups<6>(best, lane, less);
+    best          = bitonic_sort_groups<6>(best, lane);
     for (uint32_t base = kWave; base < n; base += kWave)
     {
         const uint64_t v   = (base + lane < n) ? list[base + lane] : kInfKey;
         const uint64_t thr = shfl_u64(best, K - 1);
-        if (__ballot(less(v, thr)) == 0ull) continue;
-        const uint64_t sorted = bitonic_sort_groups<6>(v, lane, less);
+        if (__ballot(v < thr) == 0ull) continue;
+        const uint64_t sorted = bitonic_sort_groups<6>(v, lane);
         const uint64_t mirror = shfl_u64(sorted, kWave - 1 - lane);
-        best                  = less(mirror, best) ? mirror : best;  // 64 smallest of the 128, a bitonic sequence
-        best                  = bitonic_merge64(best, lane, less);
+        best                  = (mirror < best) ? mirror : best;  // 64 smallest of the 128, a bitonic sequence
+        best                  = bitonic_merge64(best, lane);
     }
     if (lane < K) list[lane] = best;
 }
 
 // In-place bitonic sort of a list of any length in global memory by one wave; places beyond n act as +infinity and
 // are never touched. Slow path: only lists longer than 64 with no usable cut come here.
-template <class Less>
-__device__ __forceinline__ void sort_in_memory(uint64_t* list, uint32_t n, int lane, const Less& less)
+__device__ __forceinline__ void sort_in_memory(uint64_t* list, uint32_t n, int lane)
 {
     uint32_t m = 1;
     while (m < n) m <<= 1;
@@ -154,7 +130,7 @@ __device__ __forceinline__ void sort_in_memory(uint64_t* list, uint32_t n, int l
             if (j < n)
             {
                 const uint64_t a = list[i], b = list[j];
-                if (less(b, a))
+                if (b < a)
                 {
                     list[i] = b;
                     list[j] = a;
@@ -170,7 +146,7 @@ __device__ __forceinline__ void sort_in_memory(uint64_t* list, uint32_t n, int l
                 if (j < n)
                 {
                     const uint64_t a = list[i], b = list[j];
-                    if (less(b, a))
+                    if (b < a)
                     {
                         list[i] = b;
                         list[j] = a;
@@ -187,8 +163,8 @@ __device__ __forceinline__ void sort_in_memory(uint64_t* list, uint32_t n, int l
 // merged pairwise, level by level, in the all-ascending form of the bitonic network: the mirror step and the halving
 // steps over 64 or more places pair whole chunks register against register (the mirror step with the partner chunk
 // reversed across the wave), the last six halving steps of a level run inside every chunk. One load and one store per key.
-template <int CH, class Less>
-__device__ __forceinline__ void sort_in_registers(uint64_t* list, uint32_t n, int lane, const Less& less)
+template <int CH>
+__device__ __forceinline__ void sort_in_registers(uint64_t* list, uint32_t n, int lane)
 {
     uint64_t c[CH];
 #pragma unroll
@@ -198,7 +174,7 @@ __device__ __forceinline__ void sort_in_registers(uint64_t* list, uint32_t n, in
         c[q]               = idx < n ? list[idx] : kInfKey;
     }
 #pragma unroll
-    for (int q = 0; q < CH; ++q) c[q] = bitonic_sort_groups<6>(c[q], lane, less);
+    for (int q = 0; q < CH; ++q) c[q] = bitonic_sort_groups<6>(c[q], lane);
     auto reversed = [&](uint64_t v) {
         const uint32_t lo = lane_xor<63>((uint32_t)v, lane), hi = lane_xor<63>((uint32_t)(v >> 32), lane);
         return ((uint64_t)hi << 32) | lo;
@@ -212,8 +188,7 @@ __device__ __forceinline__ void sort_in_registers(uint64_t* list, uint32_t n, in
             {
                 const int p        = q - (q % w) + (w - 1 - (q % w));
                 const uint64_t r   = reversed(c[p]);
-                const bool lt      = less(r, c[q]);
-                const uint64_t mn  = lt ? r : c[q], mx = lt ? c[q] : r;
+                const uint64_t mn  = r < c[q] ? r : c[q], mx = r < c[q] ? c[q] : r;
                 c[q]               = mn;
                 c[p]               = reversed(mx);
             }
@@ -224,12 +199,11 @@ __device__ __forceinline__ void sort_in_registers(uint64_t* list, uint32_t n, in
                 if ((q & d) == 0)
                 {
                     const uint64_t x = c[q], y = c[q + d];
-                    const bool lt    = less(y, x);
-                    c[q]             = lt ? y : x;
-                    c[q + d]         = lt ? x : y;
+                    c[q]             = y < x ? y : x;
+                    c[q + d]         = y < x ? x : y;
                 }
 #pragma unroll
-        for (int q = 0; q < CH; ++q) c[q] = bitonic_merge64(c[q], lane, less);
+        for (int q = 0; q < CH; ++q) c[q] = bitonic_merge64(c[q], lane);
     }
 #pragma unroll
     for (int q = 0; q < CH; ++q)
@@ -245,9 +219,8 @@ constexpr uint32_t kRegisterSortKeys = 256;  // longest list sort_wave_lists sor
 // (n = 0 for lanes without a list). `fragments` may point to global memory or to LDS. Lists that have to be sorted in
 // full and hold more than kRegisterSortKeys and up to `skip_longer` keys are left alone: the caller sorts them by other
 // means.
-template <class Less = KeyLess>
 __device__ __forceinline__ void sort_wave_lists(uint64_t* fragments, uint8_t* src_lane, uint32_t off, uint32_t n,
-                                                int lane, int K, uint32_t skip_longer = 0, const Less& less = Less())
+                                                int lane, int K, uint32_t skip_longer = 0)
 {
     // class = ceil(log2(n)) for 2 <= n <= 64, 0 for n <= 1 (nothing to do), 7 for n > 64
     int cls = 0;
@@ -269,12 +242,12 @@ __device__ __forceinline__ void sort_wave_lists(uint64_t* fragments, uint8_t* sr
         const int count = __popcll(mask);
         switch (c)
         {
-            case 1: sort_class<1>(fragments, src_lane, count, off, n, lane, K, less); break;
-            case 2: sort_class<2>(fragments, src_lane, count, off, n, lane, K, less); break;
-            case 3: sort_class<3>(fragments, src_lane, count, off, n, lane, K, less); break;
-            case 4: sort_class<4>(fragments, src_lane, count, off, n, lane, K, less); break;
-            case 5: sort_class<5>(fragments, src_lane, count, off, n, lane, K, less); break;
-            default: sort_class<6>(fragments, src_lane, count, off, n, lane, K, less); break;
+            case 1: sort_class<1>(fragments, src_lane, count, off, n, lane, K); break;
+            case 2: sort_class<2>(fragments, src_lane, count, off, n, lane, K); break;
+            case 3: sort_class<3>(fragments, src_lane, count, off, n, lane, K); break;
+            case 4: sort_class<4>(fragments, src_lane, count, off, n, lane, K); break;
+            case 5: sort_class<5>(fragments, src_lane, count, off, n, lane, K); break;
+            default: sort_class<6>(fragments, src_lane, count, off, n, lane, K); break;
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
@@ -289,15 +262,15 @@ __device__ __forceinline__ void sort_wave_lists(uint64_t* fragments, uint8_t* sr
         const uint32_t o  = __shfl(off, src, kWave);
         const uint32_t nn = __shfl(n, src, kWave);
         if (K > 0 && K <= kWave)
-            select_smallest(fragments + o, nn, lane, K, less);
+            select_smallest(fragments + o, nn, lane, K);
         else if (nn <= 2 * kWave)
-            sort_in_registers<2>(fragments + o, nn, lane, less);
+            sort_in_registers<2>(fragments + o, nn, lane);
         else if (nn <= kRegisterSortKeys)
-            sort_in_registers<4>(fragments + o, nn, lane, less);
+            sort_in_registers<4>(fragments + o, nn, lane);
         else if (nn <= skip_longer)
             continue;  // the caller sorts lists of this length with the whole workgroup
         else
-            sort_in_memory(fragments + o, nn, lane, less);
+            sort_in_memory(fragments + o, nn, lane);
     }
 }
 

@@ -17,7 +17,6 @@
 #include "build_kernels.h"
 #include "backward_kernels.h"
 #include "lift_kernels.h"
-#include "region_kernels.h"
 
 using namespace vetrast;
 
@@ -291,52 +290,6 @@ uint32_t tile_grid(const TileMap& m)
     return m.regions_per_xcd * m.groups_per_region * kXcds;
 }
 
-// ---- the region-major path (region_kernels.h) ---------------------------------------------------------------------
-RegionTable make_region_table(int w, int h, int L)
-{
-    RegionTable t;
-    std::memset(&t, 0, sizeof(t));
-    t.L         = L;
-    t.regions_x = (uint32_t)(w + kRegion - 1) / kRegion;
-    t.regions   = t.regions_x * ((uint32_t)(h + kRegion - 1) / kRegion);
-    uint32_t px = 0;
-    for (int l = 0; l < L; ++l)
-    {
-        t.w[l]     = w;
-        t.h[l]     = h;
-        t.first[l] = px;
-        px += 1u << (2 * (kRegionLog - l));
-        w /= 2;
-        h /= 2;
-    }
-    for (int l = L; l <= VETRAST_MAX_LAYERS; ++l) t.first[l] = px;
-    t.ppr = px;
-    return t;
-}
-
-// The log of the region path: a workgroup of the scatter pass appends to the segment of its number; a point leaves at
-// most min(L, 4) records (one per region it touches).
-uint32_t region_log_segment_records(int64_t N, int L)
-{
-    const int64_t groups = (N + kBlock - 1) / kBlock;
-    return (uint32_t)((groups + kLogSegments - 1) / kLogSegments * kBlock * std::min(L, 4));
-}
-
-// Whether a call takes the region-major path: FULL_BLEND, and a cloud that is expected to leave a region (16x16 pixels
-// of layer 0 and what lies over them in the coarser layers) a few hundred records, so that all but a few regions fit
-// their room. The points a view sees are bounded by N, or by twice the fragments the caller expects in layer 0; a
-// point near a region's border leaves a record in the neighbouring region too (about 1.45 records per point).
-bool region_path(int64_t N, int w, int h, int L, int render_mode, const float* expected_fragments)
-{
-    if (render_mode != VETRAST_RENDER_FULL_BLEND) return false;
-    if (N >= ((int64_t)1 << kRegionIdBits) || L - 1 > kRegionLog) return false;
-    double seen = (double)N;
-    if (expected_fragments && expected_fragments[0] > 0.f && 2.0 * (double)expected_fragments[0] < seen)
-        seen = 2.0 * (double)expected_fragments[0];
-    const double regions = (double)((w + kRegion - 1) / kRegion) * (double)((h + kRegion - 1) / kRegion);
-    return 1.45 * seen / regions <= 400.0;
-}
-
 ViewPass make_view_pass(const vetrast_forward_args* a, const vetrast_workspace_layout& lay, const LayerTable& ly, int b)
 {
     ViewPass vp;
@@ -459,210 +412,6 @@ void launch_lift(const vetrast_lift_args* a, char* ws, hipStream_t stream)
                        dim3(kBlock), 0, stream, lp);
 }
 
-// The per-view launches of the region-major path: the pass over the points, then one workgroup per region.
-void forward_regions(vetrast_ctx* ctx, const vetrast_forward_args* a, const vetrast_workspace_layout& lay,
-                     const LayerTable& ly, hipStream_t stream)
-{
-    const vetrast_params& p = a->params;
-    const int N = a->num_points, B = a->num_views, L = p.num_layers, C = p.num_texture_channels;
-    void* ws             = a->workspace;
-    const RegionTable rt = make_region_table(a->views[0].w, a->views[0].h, L);
-    for (int b = 0; b < B; ++b)
-    {
-        ViewPass vp = make_view_pass(a, lay, ly, b);
-        vp.view     = ws_ptr<DeviceView>(ws, lay.region_views_base) + b;
-        uint32_t* region_count = ws_ptr<uint32_t>(ws, lay.bin_counts_base + lay.bin_counts_stride * b);
-        uint4* rooms           = ws_ptr<uint4>(ws, lay.region_rooms_base + lay.region_rooms_stride * b);
-        uint32_t* log_cursor   = ws_ptr<uint32_t>(ws, lay.log_cursor_base) + (size_t)b * kLogSegments * kLogCursorStride;
-        if (N > 0)
-        {
-            ScopeTimer tm(ctx, stream, VETRAST_SCOPE_COUNT);
-            RegionTargets t;
-            t.region_count     = region_count;
-            t.rooms            = rooms;
-            t.log              = ws_ptr<uint4>(ws, lay.region_log_base);
-            t.log_cursor       = log_cursor;
-            t.segment_capacity = region_log_segment_records(N, L);
-            t.texture          = a->texture;
-            t.confidence       = a->confidence;
-            t.C                = C;
-            t.texture_abs      = p.texture_abs;
-            hipLaunchKernelGGL(region_scatter_kernel, dim3(grid_for(N)), dim3(kBlock), 0, stream, vp, rt, t);
-        }
-        {
-            ScopeTimer tm(ctx, stream, VETRAST_SCOPE_BUILD);
-            RegionPass rp;
-            rp.rt               = rt;
-            rp.region_count     = region_count;
-            rp.rooms            = rooms;
-            rp.log              = ws_ptr<uint4>(ws, lay.region_log_base);
-            rp.log_cursor       = log_cursor;
-            rp.segment_capacity = region_log_segment_records(N, L);
-            rp.counters         = ws_ptr<uint32_t>(ws, lay.region_counters_base) + (size_t)b * kRegionCounterWords;
-            rp.region_info      = ws_ptr<uint2>(ws, lay.region_info_base + lay.region_info_stride * b);
-            rp.pixel_info       = ws_ptr<uint2>(ws, lay.region_pixel_info_base + lay.region_pixel_info_stride * b);
-            rp.heavy_pixel      = ws_ptr<uint2>(ws, lay.region_heavy_pixel_base + lay.region_heavy_pixel_stride * b);
-            rp.list_slot        = ws_ptr<uint16_t>(ws, lay.region_list_slot_base + lay.region_list_slot_stride * b);
-            rp.list_key         = ws_ptr<uint64_t>(ws, lay.region_list_key_base + lay.region_list_key_stride * b);
-            rp.list_T = a->save_for_backward ? ws_ptr<float>(ws, lay.region_list_T_base + lay.region_list_T_stride * b) : nullptr;
-            rp.heavy_T = a->save_for_backward ? ws_ptr<float>(ws, lay.region_heavy_T_base + lay.region_heavy_T_stride * b) : nullptr;
-            rp.list_places      = (uint32_t)(L * kRegionRoom);
-            rp.list_capacity         = (uint32_t)lay.fragment_capacity;
-            rp.texture               = a->texture;
-            rp.confidence            = a->confidence;
-            rp.index                 = a->index;
-            rp.N                     = N;
-            rp.C                     = C;
-            rp.confidence_activation = p.confidence_activation;
-            rp.confidence_scale      = p.confidence_scale;
-            rp.texture_abs           = p.texture_abs;
-            rp.background            = ws_ptr<const float>(ws, lay.flags_base) + kPreparedBackgroundOffset;
-            rp.K                     = p.debug_max_list_length;
-            rp.use_environment_map   = p.use_environment_map;
-            rp.mask_value            = p.output_background_mask_value;
-            for (int l = 0; l < VETRAST_MAX_LAYERS; ++l)
-            {
-                rp.out[l] = rp.out_mask[l] = rp.out_weight[l] = nullptr;
-                if (l >= L) continue;
-                const size_t plane = (size_t)rt.w[l] * rt.h[l];
-                rp.out[l]          = a->out[l] + (size_t)b * C * plane;
-                if (p.output_background_mask) rp.out_mask[l] = a->out_mask[l] + (size_t)b * plane;
-                if (a->out_weight[l]) rp.out_weight[l] = a->out_weight[l] + (size_t)b * plane;
-            }
-            const dim3 g(rt.regions, L + 1), blk(kBlock);  // planes: see region_forward_kernel
-            switch (C)
-            {
-                case 1: hipLaunchKernelGGL(region_forward_kernel<1>, g, blk, 0, stream, rp); break;
-                case 2: hipLaunchKernelGGL(region_forward_kernel<2>, g, blk, 0, stream, rp); break;
-                case 3: hipLaunchKernelGGL(region_forward_kernel<3>, g, blk, 0, stream, rp); break;
-                default: hipLaunchKernelGGL(region_forward_kernel<4>, g, blk, 0, stream, rp); break;
-            }
-        }
-    }
-}
-
-// The per-view launches of the backward pass of the region-major path.
-void backward_regions(vetrast_ctx* ctx, const vetrast_backward_args* g, const vetrast_workspace_layout& lay,
-                      const LayerTable& ly, const ClearJob& clear, bool want_camera, bool want_image_gradient,
-                      bool add_to_rows, hipStream_t stream)
-{
-    const vetrast_forward_args* a = &g->fwd;
-    const vetrast_params& p       = a->params;
-    const int N = a->num_points, B = a->num_views, L = p.num_layers, C = p.num_texture_channels;
-    void* ws               = a->workspace;
-    const RegionTable rt   = make_region_table(a->views[0].w, a->views[0].h, L);
-    float4* partial        = ws_ptr<float4>(ws, lay.region_partial_base);
-    float* background_rows = ws_ptr<float>(ws, lay.region_background_partial_base);
-    double* camera_rows    = ws_ptr<double>(ws, lay.region_camera_partial_base);
-    for (int b = 0; b < B; ++b)
-    {
-        uint32_t* region_count = ws_ptr<uint32_t>(ws, lay.bin_counts_base + lay.bin_counts_stride * b);
-        {
-            ScopeTimer tm(ctx, stream, VETRAST_SCOPE_BACKWARD_BLEND);
-            RegionBackwardPass bp;
-            bp.rt           = rt;
-            bp.region_count = region_count;
-            bp.rooms        = ws_ptr<uint4>(ws, lay.region_rooms_base + lay.region_rooms_stride * b);
-            bp.region_info  = ws_ptr<uint2>(ws, lay.region_info_base + lay.region_info_stride * b);
-            bp.pixel_info   = ws_ptr<uint2>(ws, lay.region_pixel_info_base + lay.region_pixel_info_stride * b);
-            bp.heavy_pixel  = ws_ptr<uint2>(ws, lay.region_heavy_pixel_base + lay.region_heavy_pixel_stride * b);
-            bp.list_slot    = ws_ptr<uint16_t>(ws, lay.region_list_slot_base + lay.region_list_slot_stride * b);
-            bp.list_key     = ws_ptr<uint64_t>(ws, lay.region_list_key_base + lay.region_list_key_stride * b);
-            bp.list_T       = ws_ptr<float>(ws, lay.region_list_T_base + lay.region_list_T_stride * b);
-            bp.heavy_T      = ws_ptr<float>(ws, lay.region_heavy_T_base + lay.region_heavy_T_stride * b);
-            bp.list_places  = (uint32_t)(L * kRegionRoom);
-            bp.texture      = a->texture;
-            bp.confidence   = a->confidence;
-            bp.index        = a->index;
-            bp.N            = N;
-            bp.C            = C;
-            bp.confidence_activation = p.confidence_activation;
-            bp.confidence_scale      = p.confidence_scale;
-            bp.texture_abs           = p.texture_abs;
-            bp.background            = ws_ptr<const float>(ws, lay.flags_base) + kPreparedBackgroundOffset;
-            bp.partial               = partial;
-            bp.background_partial    = background_rows;
-            bp.K                     = p.debug_max_list_length;
-            bp.use_environment_map   = p.use_environment_map;
-            bp.need_point_gradient   = want_image_gradient ? 1 : 0;
-            bp.quirk_background_confidence_leak = p.quirk_background_confidence_leak;
-            bp.clear                 = b == 0 ? clear : ClearJob{};
-            for (int l = 0; l < VETRAST_MAX_LAYERS; ++l)
-            {
-                bp.grad_out[l] = nullptr;
-                bp.out[l]      = nullptr;
-                if (l >= L) continue;
-                const size_t plane = (size_t)rt.w[l] * rt.h[l];
-                bp.grad_out[l]     = g->grad_out[l] + (size_t)b * C * plane;
-                bp.out[l]          = a->out[l] + (size_t)b * C * plane;
-            }
-            const dim3 grid(rt.regions, kRegionPlanes), blk(kBlock);
-            switch (C)
-            {
-                case 1: hipLaunchKernelGGL(region_backward_kernel<1>, grid, blk, 0, stream, bp); break;
-                case 2: hipLaunchKernelGGL(region_backward_kernel<2>, grid, blk, 0, stream, bp); break;
-                case 3: hipLaunchKernelGGL(region_backward_kernel<3>, grid, blk, 0, stream, bp); break;
-                default: hipLaunchKernelGGL(region_backward_kernel<4>, grid, blk, 0, stream, bp); break;
-            }
-        }
-        if (N > 0)
-        {
-            ScopeTimer tm(ctx, stream, VETRAST_SCOPE_BACKWARD_GATHER);
-            RegionGatherPass gp;
-            gp.vp                    = make_view_pass(a, lay, ly, b);
-            gp.vp.view               = ws_ptr<DeviceView>(ws, lay.region_views_base) + b;
-            gp.rt                    = rt;
-            gp.region_count          = region_count;
-            gp.partial               = partial;
-            gp.grad_texture          = g->grad_texture;
-            gp.grad_confidence       = g->grad_confidence;
-            gp.grad_points           = g->grad_points;
-            gp.grad_point_count      = g->grad_point_count;
-            gp.camera_partial        = want_camera ? camera_rows : nullptr;
-            gp.need_point_gradient   = want_image_gradient ? 1 : 0;
-            gp.accumulate            = (add_to_rows || b > 0) ? 1 : 0;
-            gp.background_rows       = background_rows;
-            gp.num_background_rows   = (int)rt.regions;
-            gp.grad_background       = g->grad_background;
-            gp.add_leak              = (p.quirk_background_confidence_leak && !p.use_environment_map) ? 1 : 0;
-            gp.background_accumulate = b > 0 ? 1 : 0;
-            gp.texture_raw           = a->texture;
-            gp.background_raw        = a->background;
-            gp.texture_abs           = p.texture_abs;
-            const dim3 grid(grid_for(N)), blk(kBlock);
-            auto launch = [&](auto c_tag) {
-                constexpr int kC = decltype(c_tag)::value;
-                if (p.allow_distortion)
-                    hipLaunchKernelGGL((region_gather_kernel<kC, true>), grid, blk, 0, stream, gp);
-                else
-                    hipLaunchKernelGGL((region_gather_kernel<kC, false>), grid, blk, 0, stream, gp);
-            };
-            switch (C)
-            {
-                case 1: launch(std::integral_constant<int, 1>{}); break;
-                case 2: launch(std::integral_constant<int, 2>{}); break;
-                case 3: launch(std::integral_constant<int, 3>{}); break;
-                default: launch(std::integral_constant<int, 4>{}); break;
-            }
-        }
-        if (want_camera)
-        {
-            ScopeTimer tm(ctx, stream, VETRAST_SCOPE_BACKWARD_GATHER);
-            hipLaunchKernelGGL(reduce_camera_kernel, dim3(1), dim3(kBlock), 0, stream, camera_rows, grid_for(N),
-                               a->views[b].image_index, a->views[b].camera_index, p.K_gradient_factor, g->grad_pose,
-                               g->grad_pose_count, g->grad_intrinsics, g->grad_intrinsics_count, 1.f / 1024.f,
-                               p.allow_distortion, p.distortion_gradient_factor);
-        }
-        if (N == 0)
-        {
-            ScopeTimer tm(ctx, stream, VETRAST_SCOPE_BACKWARD_GATHER);
-            hipLaunchKernelGGL(reduce_background_kernel, dim3(1), dim3(kReduceBlock), 0, stream, background_rows,
-                               (int)rt.regions, C, g->grad_background, g->grad_confidence, 0, b > 0 ? 1 : 0,
-                               p.texture_abs ? a->background : nullptr);
-        }
-    }
-}
-
 }  // namespace
 
 extern "C" {
@@ -758,8 +507,6 @@ int vetrast_workspace_layout_for_mode(int32_t N, int32_t B, int32_t L, int32_t w
     at += lay->bin_counts_stride * B;
     lay->log_cursor_base = at;  // right behind the bin counters: one zero-fill covers both
     at += log_cursor_bytes(B);
-    lay->region_counters_base = at;  // ... and these
-    at += align_up((size_t)B * kRegionCounterWords * sizeof(uint32_t), kAlign);
     lay->scan_partials_base = at;
     at += align_up((Tpad / kScanPerBlock) * sizeof(uint32_t), kAlign);
     lay->offsets_base   = at;
@@ -812,47 +559,6 @@ int vetrast_workspace_layout_for_mode(int32_t N, int32_t B, int32_t L, int32_t w
     lay->camera_partial_base = at;
     at += align_up(((size_t)N + kBlock - 1) / kBlock * kCameraRow * sizeof(double), kAlign);
     lay->total_bytes = std::max(align_up(at, kAlign), lay->forward_only_bytes);
-    if (render_mode == VETRAST_RENDER_FULL_BLEND && (int64_t)N < ((int64_t)1 << kRegionIdBits))
-    {
-        // The arrays of the region-major path lie over those of the per-layer path (a call uses one form or the other)
-        // from the per-view arrays on; both share the counters in front of them.
-        const RegionTable rt = make_region_table(w, h, L);
-        lay->region_pixels   = (int32_t)rt.ppr;
-        lay->region_room     = kRegionRoom;
-        for (int l = 0; l <= VETRAST_MAX_LAYERS; ++l) lay->region_layer_first[l] = (int32_t)rt.first[l];
-        lay->regions_x   = (int32_t)rt.regions_x;
-        lay->num_regions = (int64_t)rt.regions;
-        // (the region counters use the bin counters' array: a view has fewer regions than bins)
-        size_t rat = lay->offsets_base;
-        lay->region_views_base = rat;
-        rat += align_up((size_t)B * sizeof(DeviceView), kAlign);
-        auto per_view = [&](size_t& base, size_t& stride, size_t bytes) {
-            base   = rat;
-            stride = align_up(bytes, kAlign);
-            rat += stride * B;
-        };
-        const size_t Pq = (size_t)rt.regions * rt.ppr;
-        per_view(lay->region_rooms_base, lay->region_rooms_stride, (size_t)rt.regions * kRegionRoom * 2 * sizeof(uint4));
-        per_view(lay->region_info_base, lay->region_info_stride, (size_t)rt.regions * sizeof(uint2));
-        per_view(lay->region_pixel_info_base, lay->region_pixel_info_stride, Pq * sizeof(uint2));
-        per_view(lay->region_heavy_pixel_base, lay->region_heavy_pixel_stride, Pq * sizeof(uint2));
-        const size_t places = (size_t)rt.regions * L * kRegionRoom;  // a region owns one place per record and layer
-        per_view(lay->region_list_slot_base, lay->region_list_slot_stride, places * sizeof(uint16_t));
-        per_view(lay->region_list_T_base, lay->region_list_T_stride, places * sizeof(float));
-        per_view(lay->region_list_key_base, lay->region_list_key_stride, cap * sizeof(uint64_t));
-        per_view(lay->region_heavy_T_base, lay->region_heavy_T_stride, cap * sizeof(float));
-        lay->region_log_base = rat;
-        const size_t log_end = rat + align_up((size_t)region_log_segment_records(N, L) * kLogSegments * sizeof(uint4), kAlign);
-        const size_t region_forward_only = log_end;
-        lay->region_partial_base = rat;
-        rat += align_up(cap * 8 * sizeof(float), kAlign);
-        lay->region_background_partial_base = rat;
-        rat += align_up((size_t)rt.regions * kBackgroundRow * sizeof(float), kAlign);
-        lay->region_camera_partial_base = rat;
-        rat += align_up(((size_t)N + kBlock - 1) / kBlock * kCameraRow * sizeof(double), kAlign);
-        lay->forward_only_bytes = std::max(lay->forward_only_bytes, region_forward_only);
-        lay->total_bytes        = std::max(lay->total_bytes, std::max(align_up(rat, kAlign), region_forward_only));
-    }
     return VETRAST_OK;
 }
 
@@ -861,17 +567,6 @@ size_t vetrast_forward_workspace_bytes(int32_t N, int32_t B, int32_t L, int32_t 
     vetrast_workspace_layout lay;
     if (vetrast_workspace_layout_for(N, B, L, w, h, &lay) != VETRAST_OK) return 0;
     return lay.total_bytes;
-}
-
-int vetrast_forward_uses_regions(const vetrast_forward_args* a)
-{
-    if (!a || !a->views || a->num_views < 1) return VETRAST_ERR_INVALID_ARG;
-    const vetrast_params& p = a->params;
-    int st = check_mode(p.render_mode);
-    if (st != VETRAST_OK) return st;
-    st = check_dims(a->num_points, a->num_views, p.num_layers, a->views[0].w, a->views[0].h, hits_of_mode(p.render_mode));
-    if (st != VETRAST_OK) return st;
-    return region_path(a->num_points, a->views[0].w, a->views[0].h, p.num_layers, p.render_mode, p.expected_fragments) ? 1 : 0;
 }
 
 int vetrast_forward(vetrast_ctx* ctx, const vetrast_forward_args* a, void* stream_)
@@ -892,13 +587,12 @@ int vetrast_forward(vetrast_ctx* ctx, const vetrast_forward_args* a, void* strea
     float4* packed      = ws_ptr<float4>(ws, lay.packed_base);
     uint32_t* slots     = ws_ptr<uint32_t>(ws, lay.slots_base);
     uint32_t* partials  = ws_ptr<uint32_t>(ws, lay.scan_partials_base);
-    const bool regions  = region_path(N, a->views[0].w, a->views[0].h, L, p.render_mode, p.expected_fragments);
-    DeviceView* views   = ws_ptr<DeviceView>(ws, regions ? lay.region_views_base : lay.views_base);
+    DeviceView* views   = ws_ptr<DeviceView>(ws, lay.views_base);
 
     {
         ScopeTimer tm(ctx, stream, VETRAST_SCOPE_PREPARE);
         // per-bin counters of all views (contiguous) start at zero; InitializeData, PointRenderer.cu:402-470
-        const size_t n4  = (Tpad * B * sizeof(uint32_t) + log_cursor_bytes(B) + (size_t)B * kRegionCounterWords * sizeof(uint32_t)) / sizeof(uint4);
+        const size_t n4  = (Tpad * B * sizeof(uint32_t) + log_cursor_bytes(B)) / sizeof(uint4);
         uint4* counters4 = ws_ptr<uint4>(ws, lay.bin_counts_base);
         const int zero_blocks = std::min(grid_for(n4), 1024);
         for (int first = 0; first < B; first += 16)
@@ -922,12 +616,6 @@ int vetrast_forward(vetrast_ctx* ctx, const vetrast_forward_args* a, void* strea
         }
     }
 
-    if (regions)
-    {
-        forward_regions(ctx, a, lay, ly, stream);
-        VET_HIP(ctx, hipGetLastError());
-        return VETRAST_OK;
-    }
     for (int b = 0; b < B; ++b)
     {
         const ViewPass vp   = make_view_pass(a, lay, ly, b);
@@ -1143,14 +831,12 @@ int vetrast_backward(vetrast_ctx* ctx, const vetrast_backward_args* g, void* str
     // (src/lib/rendering/RenderBackward.cu:1183, 1401-1459)
     const bool want_camera         = p.need_point_gradient && (g->grad_pose || g->grad_intrinsics) && N > 0;
     const bool want_image_gradient = p.need_point_gradient && (g->grad_points || g->grad_pose || g->grad_intrinsics);
-    const bool regions = region_path(N, a->views[0].w, a->views[0].h, L, p.render_mode, p.expected_fragments);
-    if (regions) backward_regions(ctx, g, lay, ly, clear, want_camera, want_image_gradient, add_to_rows, stream);
     double* camera_rows            = ws_ptr<double>(ws, lay.camera_partial_base);
     float4* partial        = ws_ptr<float4>(ws, lay.partial_base);
     float* background_rows = ws_ptr<float>(ws, lay.background_partial_base);
     const bool fuzzy_long  = p.render_mode == VETRAST_RENDER_FUZZY_BLEND &&
                             (p.debug_max_list_length <= 0 || p.debug_max_list_length > kFuzzyDense);
-    for (int b = 0; b < B && !regions; ++b)
+    for (int b = 0; b < B; ++b)
     {
         uint32_t* offsets   = ws_ptr<uint32_t>(ws, lay.offsets_base + lay.offsets_stride * b);
         uint64_t* fragments = ws_ptr<uint64_t>(ws, lay.fragments_base + lay.fragments_stride * b);

@@ -95,7 +95,6 @@ class ForwardResult:
     args: abi.ForwardArgs
     keep: tuple  # objects that must outlive `args`
     out_weight: Optional[List[torch.Tensor]] = None  # [B,1,h,w] per layer, only with want_weight
-    regions: bool = False  # the call kept its lists in the region-major form (vetrast_forward_uses_regions)
 
     def _view_array(self, base, stride, b, dtype, count):
         nbytes = count * torch.empty((), dtype=dtype).element_size()
@@ -134,77 +133,6 @@ class ForwardResult:
             self._pixel_map = np.concatenate(parts)
         return self._pixel_map
 
-    # ---- the region-major form of the lists (see vetrast_workspace_layout in include/vetrast.h) ------------------
-    def _region_pixel_map(self):
-        """int64 [total_pixels]: region-major pixel number of every image-order pixel."""
-        if getattr(self, "_rmap", None) is None:
-            lay, parts = self.layout, []
-            ppr, rx = int(lay.region_pixels), int(lay.regions_x)
-            for l in range(self.num_layers()):
-                w, h = int(lay.layer_w[l]), int(lay.layer_h[l])
-                sl = 4 - l
-                y, x = np.meshgrid(np.arange(h, dtype=np.int64), np.arange(w, dtype=np.int64), indexing="ij")
-                q = ppr * ((y >> sl) * rx + (x >> sl)) + int(lay.region_layer_first[l]) + \
-                    ((y & ((1 << sl) - 1)) << sl) + (x & ((1 << sl) - 1))
-                parts.append(q.reshape(-1))
-            self._rmap = np.concatenate(parts)
-        return self._rmap
-
-    def _region_view(self, b):
-        """What the region-major path left for view b, as numpy arrays in image order: per-pixel counts, first list
-        place, final transmittance, and whether the pixel's region is a heavy one."""
-        cache = getattr(self, "_rview", None)
-        if cache is None:
-            cache = self._rview = {}
-        if b not in cache:
-            lay = self.layout
-            regions, ppr = int(lay.num_regions), int(lay.region_pixels)
-            rc = self._view_array(lay.bin_counts_base, lay.bin_counts_stride, b, torch.int32, regions).cpu().numpy()
-            heavy = (rc.astype(np.int64) & 0xFFFFFFFF) > int(lay.region_room)
-            info = self._view_array(lay.region_info_base, lay.region_info_stride, b, torch.int32, 2 * regions)
-            info = (info.cpu().numpy().astype(np.int64) & 0xFFFFFFFF).reshape(regions, 2)
-            pix = self._view_array(lay.region_pixel_info_base, lay.region_pixel_info_stride, b, torch.int32,
-                                   2 * regions * ppr).cpu().numpy().reshape(regions * ppr, 2)
-            m = self._region_pixel_map()
-            region_of = m // ppr
-            word = pix[m, 0].astype(np.int64) & 0xFFFFFFFF
-            start, count = word & 0xFFFF, word >> 16
-            if heavy.any():
-                hp = self._view_array(lay.region_heavy_pixel_base, lay.region_heavy_pixel_stride, b, torch.int32,
-                                      2 * regions * ppr).cpu().numpy().reshape(regions * ppr, 2)
-                hv = heavy[region_of]
-                start = np.where(hv, hp[m, 0].astype(np.int64) & 0xFFFFFFFF, start)
-                count = np.where(hv, hp[m, 1].astype(np.int64) & 0xFFFFFFFF, count)
-            off = np.concatenate([[0], np.cumsum(count)]).astype(np.int64)
-            # a region built from slots owns L * region_room list places; a heavy one drew its places from a cursor
-            own = region_of * (self.num_layers() * int(lay.region_room))
-            first_place = np.where(heavy[region_of], info[region_of, 0], own) + start
-            src = np.repeat(first_place - off[:-1], count) + np.arange(off[-1], dtype=np.int64)
-            cache[b] = dict(off=off, src=src, weight=np.ascontiguousarray(pix[m, 1]).view(np.float32),
-                            region_of_fragment=np.repeat(region_of, count), heavy=heavy)
-        return cache[b]
-
-    def _region_fragments(self, b):
-        lay, v = self.layout, self._region_view(b)
-        cap, room = int(lay.fragment_capacity), int(lay.region_room)
-        places = int(lay.num_regions) * self.num_layers() * room
-        src, reg = v["src"], v["region_of_fragment"]
-        keys = np.zeros(len(src), dtype=np.uint64)
-        hv = v["heavy"][reg] if len(src) else np.zeros(0, dtype=bool)
-        if hv.any():
-            lk = self._view_array(lay.region_list_key_base, lay.region_list_key_stride, b, torch.int64, cap)
-            keys[hv] = lk.cpu().numpy().view(np.uint64)[src[hv]]
-        if (~hv).any():
-            slots = self._view_array(lay.region_list_slot_base, lay.region_list_slot_stride, b, torch.int16, places)
-            slots = slots.cpu().numpy().view(np.uint16)[src[~hv]].astype(np.int64)
-            rooms = self._view_array(lay.region_rooms_base, lay.region_rooms_stride, b, torch.int32,
-                                     int(lay.num_regions) * room * 8).cpu().numpy().reshape(-1, 8)
-            rec = rooms[reg[~hv] * room + slots]
-            depth = rec[:, 1].astype(np.int64) & 0xFFFFFFFF
-            ids = rec[:, 2].astype(np.int64) & ((1 << 27) - 1)
-            keys[~hv] = ((depth << 32) | ids).astype(np.uint64)
-        return keys
-
     def device_offsets(self, b=0):
         """int64 numpy copy of the list starts [device_pixels + 1] of view b, in workspace pixel order."""
         t = self._view_array(self.layout.offsets_base, self.layout.offsets_stride, b, torch.int32,
@@ -222,33 +150,16 @@ class ForwardResult:
 
     def offsets(self, b=0):
         """int64 exclusive scan [P+1] of the per-pixel fragment counts of view b, image order."""
-        if self.regions:
-            return self._region_view(b)["off"]
         return self._gather_index(b)[0]
 
     def fragments(self, b=0):
         """uint64 fragment keys of view b, the lists concatenated in image order."""
-        if self.regions:
-            return self._region_fragments(b)
         _, src = self._gather_index(b)
         t = self._view_array(self.layout.fragments_base, self.layout.fragments_stride, b, torch.int64,
                              int(self.layout.fragment_capacity))
         return t.cpu().numpy().view(np.uint64)[src]
 
     def transmittance(self, b=0):
-        if self.regions:
-            lay, v = self.layout, self._region_view(b)
-            src, hv = v["src"], v["heavy"][v["region_of_fragment"]]
-            res = np.zeros(len(src), dtype=np.float32)
-            if (~hv).any():
-                places = int(lay.num_regions) * self.num_layers() * int(lay.region_room)
-                t = self._view_array(lay.region_list_T_base, lay.region_list_T_stride, b, torch.float32, places)
-                res[~hv] = t.cpu().numpy()[src[~hv]]
-            if hv.any():
-                t = self._view_array(lay.region_heavy_T_base, lay.region_heavy_T_stride, b, torch.float32,
-                                     int(lay.fragment_capacity))
-                res[hv] = t.cpu().numpy()[src[hv]]
-            return res
         _, src = self._gather_index(b)
         t = self._view_array(self.layout.transmittance_base, self.layout.transmittance_stride, b, torch.float32,
                              int(self.layout.fragment_capacity))
@@ -263,8 +174,6 @@ class ForwardResult:
         return t.cpu().numpy().astype(np.int64)[self.pixel_map()]
 
     def weight(self, b=0):
-        if self.regions:
-            return self._region_view(b)["weight"]
         t = self._view_array(self.layout.weight_base, self.layout.weight_stride, b, torch.float32,
                              self.device_pixels())
         return t.cpu().numpy()[self.pixel_map()]
@@ -354,8 +263,7 @@ class Rasterizer:
             assert point_order.dtype == torch.int32 and point_order.is_cuda and point_order.numel() == scene.num_points
             args.point_order = point_order.data_ptr()
         abi.check(self.lib.vetrast_forward(self.ctx, C.byref(args), self._stream()), "forward")
-        regions = self.lib.vetrast_forward_uses_regions(C.byref(args)) == 1
-        return ForwardResult(out, masks, workspace, lay, args, (views, dev, params, point_order), weights, regions)
+        return ForwardResult(out, masks, workspace, lay, args, (views, dev, params, point_order), weights)
 
     def backward(self, fwd: ForwardResult, grad_out: List[torch.Tensor], want_points=True, want_cameras=False,
                  **param_overrides):

@@ -287,8 +287,7 @@ torch::autograd::variable_list PointRender::forward(torch::autograd::AutogradCon
     a.point_order              = order.defined() ? order.data_ptr<int32_t>() : nullptr;
     check_status(vetrast_forward(info->cache->ctx, &a, current_stream()), "forward");
     if (info->params.size_bins_from_history)
-        info->cache->NoteFragmentCounts(workspace, lay, N, L, info->images[0].w, info->images[0].h, a.params.render_mode,
-                                        vetrast_forward_uses_regions(&a) == 1);
+        info->cache->NoteFragmentCounts(workspace, lay, N, L, info->images[0].w, info->images[0].h, a.params.render_mode);
 
     if (need_backward)
     {
@@ -745,7 +744,7 @@ void PointRendererCache::ExpectedFragments(float* expected, int64_t N, int L, in
 }
 
 void PointRendererCache::NoteFragmentCounts(const torch::Tensor& workspace, const vetrast_workspace_layout& lay, int64_t N,
-                                            int L, int w, int h, int render_mode, bool regions)
+                                            int L, int w, int h, int render_mode)
 {
     CountsKey key;
     key.N = N, key.L = L, key.w = w, key.h = h, key.mode = render_mode;
@@ -763,33 +762,10 @@ void PointRendererCache::NoteFragmentCounts(const torch::Tensor& workspace, cons
     }
     if (!counts_host_.defined())
         counts_host_ = torch::empty({VETRAST_MAX_LAYERS + 1}, torch::TensorOptions().dtype(torch::kInt32).pinned_memory(true));
-    if (regions)
-    {
-        // A call that keeps its lists region by region leaves, per pixel, a word with the length of the pixel's list in
-        // its upper half (pixels numbered region by region, a region's pixels layer after layer): view 0's lengths
-        // added up per layer and brought to the running sums the other form leaves. (The pixels of the few regions
-        // that hold more records than their room keep their lengths elsewhere; as a hint the sums do without them.)
-        const int64_t regions = lay.num_regions, ppr = lay.region_pixels;
-        const torch::Tensor words = workspace.narrow(0, (int64_t)lay.region_pixel_info_base, regions * ppr * 8)
-                                        .view(torch::kInt32)
-                                        .view({regions, ppr, 2})
-                                        .select(2, 0);
-        std::vector<torch::Tensor> sums = {torch::zeros({1}, words.options().dtype(torch::kInt64))};
-        for (int l = 0; l < VETRAST_MAX_LAYERS; ++l)
-        {
-            const int64_t a = lay.region_layer_first[l < L ? l : L], b = lay.region_layer_first[l < L ? l + 1 : L];
-            sums.push_back(b > a ? words.slice(1, a, b).bitwise_right_shift(16).bitwise_and(0xFFFF).sum().reshape({1}) + sums.back()
-                                 : sums.back());
-        }
-        counts_host_.copy_(torch::cat(sums).to(torch::kInt32), /*non_blocking=*/true);
-    }
-    else
-    {
-        // view 0's exclusive scan of the per-pixel counts: the entry at a layer's first pixel is the number of
-        // fragments of the layers in front of it
-        const torch::Tensor scan = workspace.narrow(0, (int64_t)lay.offsets_base, (P + 1) * 4).view(torch::kInt32);
-        counts_host_.copy_(scan.index_select(0, counts_index_), /*non_blocking=*/true);
-    }
+    // view 0's exclusive scan of the per-pixel counts: the entry at a layer's first pixel is the number of fragments
+    // of the layers in front of it
+    const torch::Tensor scan = workspace.narrow(0, (int64_t)lay.offsets_base, (P + 1) * 4).view(torch::kInt32);
+    counts_host_.copy_(scan.index_select(0, counts_index_), /*non_blocking=*/true);
     if (!counts_event_) counts_event_ = std::make_unique<c10::Event>(c10::DeviceType::CUDA);
     counts_event_->record(c10::hip::getCurrentHIPStreamMasqueradingAsCUDA());
     pending_key_    = key;

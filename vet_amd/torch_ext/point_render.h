@@ -128,7 +128,7 @@ class PointRendererCache
     // up by a later call once the copy has landed. Kept per image size, layer count, point count and render mode.
     void ExpectedFragments(float* expected, int64_t N, int L, int w, int h, int render_mode);
     void NoteFragmentCounts(const torch::Tensor& workspace, const vetrast_workspace_layout& lay, int64_t N, int L, int w,
-                            int h, int render_mode, bool regions);
+                            int h, int render_mode);
     // what ExpectedFragments would work from right now (empty: nothing has been read back yet)
     std::vector<float> FragmentHistory();
     // layers_cuda[l].weight of the reference's cache (src/lib/rendering/PointRenderer.h:131, written at
