@@ -183,7 +183,9 @@ typedef struct vetrast_workspace_layout
     size_t views_base;     /* prepared per-view camera constants */
     size_t scan_partials_base;
     int64_t num_bins;      /* bins of one view: runs of 256 / 64 / 16 / 4 consecutive pixel numbers, chosen per layer from N */
-    size_t bin_counts_base, bin_counts_stride; /* per view, uint32 [num_bins+1 padded]: fragments per bin, then their exclusive scan */
+    size_t bin_counts_base, bin_counts_stride; /* per view, uint32 [2][num_bins+1 padded]: fragments per bin, and their
+                                                  exclusive scan (in place of the counts where a view has more than
+                                                  15 360 bins) */
     size_t binned_base;    /* uint32 [N*L*hits][4]: compact array of fragment records (key low, key high, pixel in bin, 0),
                               only used for the records beyond a bin's own room; scratch. In FULL_BLEND / FUZZY_BLEND with
                               N <= 2^24 a record is uint32 [2]: (depth bits, point id << 8 | pixel in bin) */

@@ -1585,7 +1585,7 @@ __global__ void __launch_bounds__(kBlock) gather_point_gradients_kernel(GatherPa
         const int row = a.vp.index ? a.vp.index[i] : i;
         if ((uint32_t)row < (uint32_t)N)
         {
-            if (a.confidence_activation)
+            if (a.confidence_activation && hit)  // (a point without a fragment has no gradient, and its row may not be packed)
             {
                 const float s = a.packed[2 * (size_t)row + 1].x;  // d sigmoid(k x) / dx = k s (1 - s)
                 gc            = gc * ((a.confidence_scale * s) * (1.f - s));
@@ -1653,7 +1653,7 @@ __global__ void __launch_bounds__(kBlock) gather_point_gradients_kernel(GatherPa
         float leak_factor = 1.f;
         if (a.confidence_activation && a.add_leak)
         {
-            const float s0 = a.packed[1].x;
+            const float s0 = sigmoid_canon(a.confidence_scale * a.vp.confidence[0]);  // (row 0 may not be packed)
             leak_factor    = (a.confidence_scale * s0) * (1.f - s0);
         }
         sum_background_rows<kBlock>(a.background_rows, a.num_background_rows, C, a.grad_background, a.grad_confidence,

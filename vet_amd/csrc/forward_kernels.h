@@ -163,7 +163,8 @@ __device__ __forceinline__ bool point_is_skipped(const ViewPass& a, int i)
 //      bins per layer: the wave groups its hits by bin with ballots and issues one returning atomic per distinct bin,
 //      which counts the bin and gives every hit its arrival rank inside it; the fragment record goes straight to
 //      place `rank` of the room the bin owns (no second projection pass).
-//   2. exclusive scan over the bin counts (overflow_move_kernel then files the few records that did not fit a bin's room).
+//   2. exclusive scan over the bin counts; the few records that did not fit a bin's room are filed behind it (the same
+//      launch, scan_move_kernel, where a view has at most kScanMoveMax bins; overflow_move_kernel otherwise).
 //   3. bin_build_kernel: one workgroup per bin counts the pixels, scans them, scatters the keys and sorts the lists, all
 //      in LDS. Pixels are numbered tile by tile, so the scan of the bin counts IS the start of every bin's lists and no
 //      scan over the pixels is needed.
@@ -258,6 +259,7 @@ struct PackJob
     int confidence_activation;
     float confidence_scale;
     int texture_abs;
+    int visible_only;  // pack the rows of the points that can leave a fragment in this view only (see bin_scatter_kernel)
 };
 
 // Where the scatter pass puts a fragment record (64-bit key = depth bits << 32 | point id, pixel inside the bin).
@@ -328,16 +330,6 @@ __global__ void __launch_bounds__(kBlock) bin_scatter_kernel(ViewPass a, uint32_
     // the point this thread takes: the caller's processing order, if there is one (neighbours in a wave should be
     // neighbours in space; ids in the records are the caller's either way)
     const int i = (a.point_order != nullptr && slot < a.N) ? a.point_order[slot] : slot;
-    // side job: texture row `slot`, asked for first and stored last
-    const bool packs = pack.packed != nullptr && slot < pack.N;
-    float row[4] = {0.f, 0.f, 0.f, 0.f}, row_confidence = 0.f;
-    if (packs)
-    {
-#pragma unroll
-        for (int ci = 0; ci < VETRAST_MAX_CHANNELS; ++ci)
-            if (ci < pack.C) row[ci] = pack.texture[(size_t)ci * pack.N + slot];
-        row_confidence = pack.confidence[slot];
-    }
     Projected p;
     p.ipx = p.ipy = p.z = p.radius = 0.f;
     const bool visible = (uint32_t)i < (uint32_t)a.N && !point_is_skipped(a, i) && project_point(*a.view, a.position[i], p);
@@ -351,6 +343,18 @@ __global__ void __launch_bounds__(kBlock) bin_scatter_kernel(ViewPass a, uint32_
     const bool inside = visible && ipx >= -reach && ipx <= (float)a.ly.w[0] + reach && ipy >= -reach &&
                         ipy <= (float)a.ly.h[0] + reach;
     const bool any_inside = __ballot(inside) != 0ull;
+    // side job: texture row `slot`, asked for here and stored last. Only fragments ever read a row, so a call with one
+    // view, no texture index and no processing order (row, point and thread then are the same number) leaves out the
+    // rows of the points outside the view: half of the cloud for a full frame, most of it for a crop.
+    const bool packs = pack.packed != nullptr && slot < pack.N && (!pack.visible_only || inside);
+    float row[4] = {0.f, 0.f, 0.f, 0.f}, row_confidence = 0.f;
+    if (packs)
+    {
+#pragma unroll
+        for (int ci = 0; ci < VETRAST_MAX_CHANNELS; ++ci)
+            if (ci < pack.C) row[ci] = pack.texture[(size_t)ci * pack.N + slot];
+        row_confidence = pack.confidence[slot];
+    }
     bool dropped = !inside;  // also from the layer on at which the splat radius falls under the threshold
     if constexpr (HITS == 1)
     {
@@ -575,23 +579,32 @@ __global__ void __launch_bounds__(kBlock) scan_apply_kernel(uint4* __restrict__ 
     }
 }
 
-// The same scan in one launch by one workgroup of 1024 threads, for up to 16 K counts (a 1080p frame has some ten
-// thousand bins): thread t owns the 16 consecutive counts [16 t, 16 t + 16). The array is zero padded to a multiple of
-// 4096 counts, so whole uint4 loads never leave it.
-constexpr int kScanSmallBlock = 1024;
-constexpr int kScanSmallMax   = kScanSmallBlock * kScanPerThread;
+// Scan and move in one launch, for up to kScanMoveMax counts: one workgroup per segment of the overflow log. Every
+// workgroup whose segment holds entries scans the bin counts into LDS for itself and files its entries with them;
+// workgroup 0 scans in any case and writes the result to `offsets` (the counts stay as they are, so that the other
+// workgroups may read them meanwhile). As a rule the log is empty: 255 workgroups leave at once and the launch is the
+// scan alone, where the two kernels cost a launch (and a dependency on the one before) each.
+constexpr int kScanMoveMax = 60 * kBlock;  // 61 440 bytes of LDS
 
-__global__ void __launch_bounds__(kScanSmallBlock) scan_small_kernel(uint4* __restrict__ counts4, uint32_t n)
+__global__ void __launch_bounds__(kBlock) scan_move_kernel(const uint4* __restrict__ counts4, uint32_t n,
+                                                            uint4* __restrict__ offsets4, ScatterTargets in,
+                                                            uint4* __restrict__ binned, uint32_t capacity)
 {
-    __shared__ uint32_t wave_tot[kScanSmallBlock / kWave];
-    const bool mine_any = (uint32_t)threadIdx.x * kScanPerThread < n;
-    uint4* mine         = counts4 + threadIdx.x * (kScanPerThread / 4);
-    uint4 v[kScanPerThread / 4];
+    __shared__ uint32_t s_off[kScanMoveMax];
+    __shared__ uint32_t wave_tot[kBlock / kWave];
+    const uint32_t segment = blockIdx.x;
+    // (workgroup 0 scans whatever its segment holds: it asks for its cursor and for the counts at once)
+    const uint32_t entries = min(in.log_cursor[segment * kLogCursorStride], in.segment_capacity);
+    if (segment != 0u && entries == 0u) return;
+    constexpr int kPer = kScanMoveMax / kBlock;  // 60 consecutive counts per thread, as 15 16-byte loads
+    const uint4* src   = counts4 + threadIdx.x * (kPer / 4);
+    uint4 v[kPer / 4];
     uint32_t sum = 0;
 #pragma unroll
-    for (int k = 0; k < kScanPerThread / 4; ++k)
+    for (int k = 0; k < kPer / 4; ++k)
     {
-        v[k] = mine_any ? mine[k] : make_uint4(0u, 0u, 0u, 0u);
+        // (the array is zero padded to a multiple of 4096 counts, so whole loads never leave it)
+        v[k] = (uint32_t)threadIdx.x * kPer + 4 * k < n ? src[k] : make_uint4(0u, 0u, 0u, 0u);
         sum += (v[k].x + v[k].y) + (v[k].z + v[k].w);
     }
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
@@ -600,9 +613,9 @@ __global__ void __launch_bounds__(kScanSmallBlock) scan_small_kernel(uint4* __re
     __syncthreads();
     uint32_t run = incl - sum;
     for (int k = 0; k < wave; ++k) run += wave_tot[k];
-    if (!mine_any) return;
+    uint4* dst = offsets4 + threadIdx.x * (kPer / 4);
 #pragma unroll
-    for (int k = 0; k < kScanPerThread / 4; ++k)
+    for (int k = 0; k < kPer / 4; ++k)
     {
         uint4 o;
         o.x = run;
@@ -613,7 +626,21 @@ __global__ void __launch_bounds__(kScanSmallBlock) scan_small_kernel(uint4* __re
         run += v[k].z;
         o.w = run;
         run += v[k].w;
-        mine[k] = o;
+        if (segment == 0u && (uint32_t)threadIdx.x * kPer + 4 * k < n) dst[k] = o;
+        if (entries != 0u) reinterpret_cast<uint4*>(s_off)[threadIdx.x * (kPer / 4) + k] = o;
+    }
+    if (entries == 0u) return;
+    __syncthreads();
+    const size_t first = (size_t)segment * in.segment_capacity;
+    for (uint32_t e = threadIdx.x; e < entries; e += blockDim.x)
+    {
+        const uint4 rec    = in.log[first + e];
+        const uint32_t pos = (rec.w < (uint32_t)kScanMoveMax ? s_off[rec.w] : capacity) + in.log_rank[first + e];
+        if (pos >= capacity) continue;  // guard: never true
+        if (in.compact)
+            reinterpret_cast<uint2*>(binned)[pos] = make_uint2(rec.y, (rec.x << 8) | rec.z);
+        else
+            binned[pos] = make_uint4(rec.x, rec.y, rec.z, 0u);
     }
 }
 

@@ -503,7 +503,7 @@ int vetrast_workspace_layout_for_mode(int32_t N, int32_t B, int32_t L, int32_t w
     lay->flags_base        = at;
     at += kAlign;
     lay->bin_counts_base   = at;
-    lay->bin_counts_stride = Tpad * sizeof(uint32_t);
+    lay->bin_counts_stride = 2 * Tpad * sizeof(uint32_t);  // the counts, and behind them room for their scan
     at += lay->bin_counts_stride * B;
     lay->log_cursor_base = at;  // right behind the bin counters: one zero-fill covers both
     at += log_cursor_bytes(B);
@@ -581,7 +581,7 @@ int vetrast_forward(vetrast_ctx* ctx, const vetrast_forward_args* a, void* strea
     const int hits      = hits_of_mode(p.render_mode);
     const LayerTable ly = make_call_layer_table(a->views[0].w, a->views[0].h, L, (int64_t)N * hits, p.expected_fragments);
     const uint32_t bins = ly.bin_base[L];
-    const size_t Tpad   = lay.bin_counts_stride / sizeof(uint32_t);
+    const size_t Tpad   = lay.bin_counts_stride / sizeof(uint32_t) / 2;  // counts per view; as many words behind them
     void* ws            = a->workspace;
     uint32_t* flags     = ws_ptr<uint32_t>(ws, lay.flags_base);
     float4* packed      = ws_ptr<float4>(ws, lay.packed_base);
@@ -592,7 +592,7 @@ int vetrast_forward(vetrast_ctx* ctx, const vetrast_forward_args* a, void* strea
     {
         ScopeTimer tm(ctx, stream, VETRAST_SCOPE_PREPARE);
         // per-bin counters of all views (contiguous) start at zero; InitializeData, PointRenderer.cu:402-470
-        const size_t n4  = (Tpad * B * sizeof(uint32_t) + log_cursor_bytes(B)) / sizeof(uint4);
+        const size_t n4  = (2 * Tpad * B * sizeof(uint32_t) + log_cursor_bytes(B)) / sizeof(uint4);
         uint4* counters4 = ws_ptr<uint4>(ws, lay.bin_counts_base);
         const int zero_blocks = std::min(grid_for(n4), 1024);
         for (int first = 0; first < B; first += 16)
@@ -642,6 +642,7 @@ int vetrast_forward(vetrast_ctx* ctx, const vetrast_forward_args* a, void* strea
         pack.confidence_activation = p.confidence_activation;
         pack.confidence_scale      = p.confidence_scale;
         pack.texture_abs           = p.texture_abs;
+        pack.visible_only          = (B == 1 && a->index == nullptr && a->point_order == nullptr) ? 1 : 0;
         uint8_t* list_is_cut     = ws_ptr<uint8_t>(ws, lay.cut_flags_base + lay.cut_flags_stride * b);
         if (N > 0)
         {
@@ -651,11 +652,17 @@ int vetrast_forward(vetrast_ctx* ctx, const vetrast_forward_args* a, void* strea
             else
                 hipLaunchKernelGGL(bin_scatter_kernel<4>, dim3(grid_for(N)), dim3(kBlock), 0, stream, vp, bin_counts, targets, pack);
         }
+        // Where the bins of a view are few enough, one launch scans their counts and files the logged records (the
+        // scan lands behind the counts); otherwise the scan runs in place and the move kernel follows.
+        const bool scan_and_move = bins + 1 <= (uint32_t)kScanMoveMax;
+        const uint32_t* bin_offsets = scan_and_move ? bin_counts + Tpad : bin_counts;
         {
             ScopeTimer tm(ctx, stream, VETRAST_SCOPE_SCAN);
-            if (bins + 1 <= (uint32_t)kScanSmallMax)
-                hipLaunchKernelGGL(scan_small_kernel, dim3(1), dim3(kScanSmallBlock), 0, stream,
-                                   reinterpret_cast<uint4*>(bin_counts), bins + 1);
+            if (scan_and_move)
+                hipLaunchKernelGGL(scan_move_kernel, dim3(kLogSegments), dim3(kBlock), 0, stream,
+                                   reinterpret_cast<const uint4*>(bin_counts), bins + 1,
+                                   reinterpret_cast<uint4*>(bin_counts + Tpad), targets, binned,
+                                   (uint32_t)lay.fragment_capacity);
             else
             {
                 const int blocks = (int)(Tpad / kScanPerBlock);
@@ -665,7 +672,7 @@ int vetrast_forward(vetrast_ctx* ctx, const vetrast_forward_args* a, void* strea
                                    reinterpret_cast<uint4*>(bin_counts), partials);
             }
         }
-        if (N > 0)
+        if (N > 0 && !scan_and_move)
         {
             ScopeTimer tm(ctx, stream, VETRAST_SCOPE_FILL);
             // the few records beyond their bin's own room, if any
@@ -689,7 +696,7 @@ int vetrast_forward(vetrast_ctx* ctx, const vetrast_forward_args* a, void* strea
         {
             ScopeTimer tm(ctx, stream, VETRAST_SCOPE_BUILD);
             BuildPass bp;
-            bp.bin_offsets         = bin_counts;
+            bp.bin_offsets         = bin_offsets;
             bp.primary             = targets.primary;
             bp.binned              = binned;
             bp.compact_records     = targets.compact;
