@@ -247,6 +247,14 @@ typedef struct vetrast_forward_args
      * file order does. Point ids everywhere else (index, gradients, dropout) stay the caller's. NULL = array order.
      * No counterpart in the reference. */
     const int32_t* point_order;
+    /* Optional, device float [N][8], 32-byte aligned: the descriptor records vetrast_pack_descriptors wrote from THIS
+     * texture and confidence under THESE params (num_texture_channels, confidence_activation, confidence_scale,
+     * texture_abs). The call then reads a fragment's descriptor and confidence from it and leaves out the interleave
+     * it otherwise does on the side in every call: for callers that render a scene more than once between changes of
+     * its texture (a viewer; evaluation). The caller vouches that the records are current; vetrast_backward reads the
+     * same array. NULL = the call interleaves for itself, into the workspace. No counterpart in the reference, which
+     * reads the planar tensors per channel (src/lib/rendering/RenderForward.cu:1338-1342). */
+    const float* packed_descriptors;
 } vetrast_forward_args;
 
 /* Arguments of the backward pass. Replaces BlendPointCloudBackward's inputs and its seven returned tensors
@@ -303,6 +311,21 @@ int vetrast_backward(vetrast_ctx* ctx, const vetrast_backward_args* args, void* 
  * distortion model is not available, so such input is flagged instead of guessed). */
 int vetrast_query_device_flags(vetrast_ctx* ctx, const void* workspace, const vetrast_workspace_layout* layout,
                                void* stream);
+
+/* Writes the descriptor records of vetrast_forward_args.packed_descriptors: row i = texture[0..C-1][i] (|.| with
+ * texture_abs), then confidence[i] (sigmoid(confidence_scale * .) with confidence_activation), then zeros; the steps
+ * of NeuralPointTextureImpl::PrepareTexture / PrepareConfidence (src/lib/models/NeuralTexture.h:38-55) and the
+ * interleave in one pass. Of `params` only those four members are read. One streaming kernel, 52 bytes per point. */
+typedef struct vetrast_pack_args
+{
+    int32_t num_points;
+    const float* texture;    /* device [C,N] */
+    const float* confidence; /* device [N] */
+    vetrast_params params;
+    float* packed;           /* device [N][8], 32-byte aligned; fully overwritten */
+} vetrast_pack_args;
+size_t vetrast_packed_descriptor_bytes(int32_t num_points);
+int vetrast_pack_descriptors(vetrast_ctx* ctx, const vetrast_pack_args* args, void* stream);
 
 /* One Adam step on a flat float tensor, the update MyAdam::step applies to texture_raw, confidence_raw and
  * background_color_raw after every batch (src/lib/models/my_adam.cpp:25-104 = torch's Adam without amsgrad; options as

@@ -44,7 +44,7 @@ def test_every_struct_field_sits_where_the_c_compiler_puts_it(tmp_path):
 
     pairs = [("vetrast_view", abi.View), ("vetrast_params", abi.Params), ("vetrast_workspace_layout", abi.WorkspaceLayout),
              ("vetrast_forward_args", abi.ForwardArgs), ("vetrast_backward_args", abi.BackwardArgs),
-             ("vetrast_adam_args", abi.AdamArgs), ("vetrast_lift_args", abi.LiftArgs)]
+             ("vetrast_adam_args", abi.AdamArgs), ("vetrast_lift_args", abi.LiftArgs), ("vetrast_pack_args", abi.PackArgs)]
     lines = ['#include <stdio.h>', '#include <stddef.h>', '#include "vetrast.h"', 'int main(void) {']
     for cname, mirror in pairs:
         lines.append(f'printf("{cname} size %zu\\n", sizeof({cname}));')

@@ -279,26 +279,46 @@ def _plain_call(scene, torch_ops, texture=None, confidence=None, intrinsics=None
 
 def test_cameras_with_distortion_are_refused_by_the_shim():
     """Non-zero distortion coefficients (columns 5..12 of the intrinsics) must not render as an undistorted pinhole
-    through the drop-in seam: BlendPointCloud and FillSceneGridWithLoss throw. The check is repeated when the tensor
-    changes in place."""
+    through the drop-in seam: BlendPointCloud and FillSceneGridWithLoss throw. A tensor the cache has not seen is read
+    back (blocking) and refused before anything renders. A tensor it knows is never read back again: when it changes in
+    place, the call that follows renders, the status word that call raised on the device travels to the host behind it,
+    and the next call throws."""
     from vet_amd import torch_ops
 
     scene = synthetic.tiny_scene(num_points=1000, K=8, seed=36)
+    fresh = torch.from_numpy(scene.intrinsics.copy()).cuda()
+    fresh[0, 7] = 1e-3
+    with pytest.raises(RuntimeError, match="distortion"):
+        _plain_call(scene, torch_ops, intrinsics=fresh)  # unknown tensor: refused at once
+
     intr = torch.from_numpy(scene.intrinsics.copy()).cuda()
     outs = _plain_call(scene, torch_ops, intrinsics=intr)  # zero coefficients: fine
     assert len(outs) == scene.num_layers
     intr[0, 7] = 1e-3  # k3, changed in place: same storage, new version
+    assert len(_plain_call(scene, torch_ops, intrinsics=intr)) == scene.num_layers  # not read back: renders, flagged
+    torch.cuda.synchronize()
     with pytest.raises(RuntimeError, match="distortion"):
         _plain_call(scene, torch_ops, intrinsics=intr)
     mn, ln = synthetic.cell_grid(scene.position[:, :3], 0.5)
     dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
     value = torch.zeros((len(mn), 1), device="cuda")
     count = torch.zeros((len(mn), 1), dtype=torch.int32, device="cuda")
-    with pytest.raises(RuntimeError, match="distortion"):
+    with pytest.raises(RuntimeError, match="distortion"):  # after a refusal the tensor itself is checked again
         torch_ops.fill_scene_grid_with_loss(0, dev(mn), dev(ln), value, count, _views(scene), dev(scene.poses_se3), intr,
                                             torch.zeros((3, scene.views[0].h, scene.views[0].w), device="cuda"))
     assert int(count.sum()) == 0
     intr[0, 7] = 0.0
+    assert len(_plain_call(scene, torch_ops, intrinsics=intr)) == scene.num_layers
+
+    # a write that leaves the tensor's version counter alone (as one through a raw pointer does) is found by the
+    # look at the status word that every 64th call asks for
+    with torch.autograd._unsafe_preserve_version_counter(intr):
+        intr[0, 5] = 2e-3
+    with pytest.raises(RuntimeError, match="distortion"):
+        for _ in range(70):
+            _plain_call(scene, torch_ops, intrinsics=intr)
+            torch.cuda.synchronize()
+    intr[0, 5] = 0.0
     assert len(_plain_call(scene, torch_ops, intrinsics=intr)) == scene.num_layers
 
 

@@ -31,10 +31,14 @@ def _both(rasterizer, scene, mn, ln, img):
     want_v, want_c = dev(v0), dev(c0)
     ws = rasterizer.lift_error(d_mn, d_ln, want_v, want_c, scene.views[0], d_pose, d_intr, d_img)
     got_v, got_c = dev(v0), dev(c0)
-    before = torch.cuda.memory_allocated()
-    ret = rasterizer.lift_error(d_mn, d_ln, got_v, got_c, scene.views[0], d_pose, d_intr, d_img, static_scratch=True)
-    assert ret is None and torch.cuda.memory_allocated() == before
+    # Nothing is allocated: neither through torch's caching allocator nor straight from the device (free bytes as
+    # hipMemGetInfo reports them, which a hipMalloc inside the library would lower).
     torch.cuda.synchronize()
+    before, free_before = torch.cuda.memory_allocated(), torch.cuda.mem_get_info()[0]
+    ret = rasterizer.lift_error(d_mn, d_ln, got_v, got_c, scene.views[0], d_pose, d_intr, d_img, static_scratch=True)
+    torch.cuda.synchronize()
+    assert ret is None and torch.cuda.memory_allocated() == before
+    assert torch.cuda.mem_get_info()[0] >= free_before, "the device lost free memory during the call"
     queued = int(ws[abi.LIFT_QUEUE_LENGTH_OFFSET:abi.LIFT_QUEUE_LENGTH_OFFSET + 4].view(torch.int32).item())
     return got_v.cpu().numpy(), got_c.cpu().numpy(), want_v.cpu().numpy(), want_c.cpu().numpy(), c0, queued
 

@@ -115,6 +115,15 @@ class AdamArgs(C.Structure):
     ]
 
 
+class PackArgs(C.Structure):
+    _fields_ = [
+        ("num_points", C.c_int32),
+        ("texture", C.c_void_p), ("confidence", C.c_void_p),
+        ("params", Params),
+        ("packed", C.c_void_p),
+    ]
+
+
 LIFT_BORDER_PIXELS = 32
 LIFT_FLAGS_OFFSET = 192
 LIFT_QUEUE_LENGTH_OFFSET = 176
@@ -157,6 +166,7 @@ class ForwardArgs(C.Structure):
         ("workspace_bytes", C.c_size_t),
         ("out_weight", C.c_void_p * MAX_LAYERS),
         ("point_order", C.c_void_p),
+        ("packed_descriptors", C.c_void_p),
     ]
 
 
@@ -188,6 +198,8 @@ SYMBOLS = {
     "vetrast_forward_workspace_bytes": (C.c_size_t, [C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_int32]),
     "vetrast_forward": (C.c_int, [C.c_void_p, C.POINTER(ForwardArgs), C.c_void_p]),
     "vetrast_backward": (C.c_int, [C.c_void_p, C.POINTER(BackwardArgs), C.c_void_p]),
+    "vetrast_packed_descriptor_bytes": (C.c_size_t, [C.c_int32]),
+    "vetrast_pack_descriptors": (C.c_int, [C.c_void_p, C.POINTER(PackArgs), C.c_void_p]),
     "vetrast_adam_step": (C.c_int, [C.c_void_p, C.POINTER(AdamArgs), C.c_void_p]),
     "vetrast_lift_workspace_bytes": (C.c_size_t, [C.c_int64]),
     "vetrast_lift_error": (C.c_int, [C.c_void_p, C.POINTER(LiftArgs), C.c_void_p]),

@@ -606,8 +606,8 @@ __global__ void __launch_bounds__(kBlock) bin_build_kernel(BuildPass a)
         a.list_is_cut[q] = used < c ? 1 : 0;
         // ... and that key itself (the sorted keys of this bin went out to the fragment buffer before the blend)
         if (used < c) a.last_key[q] = used ? a.fragments[begin + start + used - 1u] : 0ull;
-        const uint32_t in_layer = q - a.ly.base[l];
-        const uint32_t tile     = in_layer / kTilePixels;
+        // a bin lies inside one tile: the tile's coordinates are the same for the whole workgroup (scalar arithmetic)
+        const uint32_t tile = (q0 - a.ly.base[l]) / kTilePixels;
         const uint32_t ty = tile / (uint32_t)a.ly.tiles_x[l], tx = tile - ty * (uint32_t)a.ly.tiles_x[l];
         const int x = (int)(tx * kTile + (q & (kTile - 1))), y = (int)(ty * kTile + ((q / kTile) & (kTile - 1)));
         if (x < a.ly.w[l] && y < a.ly.h[l])

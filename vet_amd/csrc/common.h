@@ -368,18 +368,20 @@ __device__ __forceinline__ TilePixel tile_pixel(const TileMap& tm, const LayerTa
     uint32_t t            = slot % tm.groups_per_region;  // workgroup inside the region, coarsest layer first
     if (region >= tm.regions) return r;
     // layer L-1 has 1 tile per region, L-2 has 4, L-3 has 16, ...; split[l] workgroups per tile
-    int l          = tm.L - 1;
-    uint32_t side  = 1;  // tiles per region side in layer l
-    while (t >= side * side * tm.split[l])
+    int l            = tm.L - 1;
+    uint32_t side_log = 0;  // tiles per region side in layer l: 1 << side_log
+    while (t >= tm.split[l] << (2 * side_log))
     {
-        t -= side * side * tm.split[l];
-        side <<= 1;
+        t -= tm.split[l] << (2 * side_log);
+        ++side_log;
         --l;
     }
-    const uint32_t strip = t % tm.split[l];  // 16x4 strip of the tile, if the layer is split
-    t /= tm.split[l];
+    // split is 1 or 4 and the side a power of two: shifts and masks instead of divisions by run-time values
+    const uint32_t split_log = tm.split[l] == 1 ? 0u : 2u;
+    const uint32_t strip     = t & (tm.split[l] - 1u);  // 16x4 strip of the tile, if the layer is split
+    t >>= split_log;
     const uint32_t ry = region / tm.regions_x, rx = region - ry * tm.regions_x;
-    const uint32_t ty = ry * side + t / side, tx = rx * side + (t & (side - 1));
+    const uint32_t ty = (ry << side_log) + (t >> side_log), tx = (rx << side_log) + (t & ((1u << side_log) - 1u));
     r.l = l;
     if (tx >= (uint32_t)ly.tiles_x[l] || ty >= (uint32_t)ly.tiles_y[l]) return r;
     uint32_t in_tile = threadIdx.x;  // 16 * (row of the tile) + column

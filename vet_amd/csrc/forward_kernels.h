@@ -262,6 +262,19 @@ struct PackJob
     int visible_only;  // pack the rows of the points that can leave a fragment in this view only (see bin_scatter_kernel)
 };
 
+// The record of texture row `slot` from its raw values.
+__device__ __forceinline__ void store_packed_row(const PackJob& pack, int slot, float (&row)[4], float row_confidence)
+{
+    if (pack.texture_abs)
+    {
+#pragma unroll
+        for (int ci = 0; ci < VETRAST_MAX_CHANNELS; ++ci) row[ci] = fabsf(row[ci]);
+    }
+    if (pack.confidence_activation) row_confidence = sigmoid_canon(pack.confidence_scale * row_confidence);
+    pack.packed[2 * (size_t)slot]     = make_float4(row[0], row[1], row[2], row[3]);
+    pack.packed[2 * (size_t)slot + 1] = make_float4(row_confidence, 0.f, 0.f, 0.f);
+}
+
 // Where the scatter pass puts a fragment record (64-bit key = depth bits << 32 | point id, pixel inside the bin).
 // Every bin owns room for room_cap[layer] records; a record whose rank inside its bin is beyond that is appended to a log
 // (with its bin and rank), from where overflow_move_kernel brings it to the bin's place in the compact array once the
@@ -470,17 +483,20 @@ __global__ void __launch_bounds__(kBlock) bin_scatter_kernel(ViewPass a, uint32_
         }
         if (VETRAST_MAX_LAYERS - 1 < a.ly.L && any_inside) store_layer(VETRAST_MAX_LAYERS - 1);
     }
-    if (packs)
-    {
-        if (pack.texture_abs)
-        {
+    if (packs) store_packed_row(pack, slot, row, row_confidence);
+}
+
+// The interleave as a launch of its own, for a caller that keeps the records across calls while texture and confidence
+// stay as they are (vetrast_pack_descriptors): every row, whatever a view sees.
+__global__ void __launch_bounds__(kBlock) pack_descriptors_kernel(PackJob pack)
+{
+    const int slot = blockIdx.x * blockDim.x + threadIdx.x;
+    if (slot >= pack.N) return;
+    float row[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int ci = 0; ci < VETRAST_MAX_CHANNELS; ++ci) row[ci] = fabsf(row[ci]);
-        }
-        if (pack.confidence_activation) row_confidence = sigmoid_canon(pack.confidence_scale * row_confidence);
-        pack.packed[2 * (size_t)slot]     = make_float4(row[0], row[1], row[2], row[3]);
-        pack.packed[2 * (size_t)slot + 1] = make_float4(row_confidence, 0.f, 0.f, 0.f);
-    }
+    for (int ci = 0; ci < VETRAST_MAX_CHANNELS; ++ci)
+        if (ci < pack.C) row[ci] = pack.texture[(size_t)ci * pack.N + slot];
+    store_packed_row(pack, slot, row, pack.confidence[slot]);
 }
 
 // Brings the logged records (rank beyond the bin's own room) to the bin's place in the compact array:

@@ -238,6 +238,7 @@ int validate_forward(const vetrast_forward_args* a, vetrast_workspace_layout* la
         if (p.output_background_mask && !for_backward && !a->out_mask[l]) return VETRAST_ERR_INVALID_ARG;
     }
     if (((uintptr_t)a->workspace % kAlign) != 0 || ((uintptr_t)a->position % 16) != 0) return VETRAST_ERR_INVALID_ARG;
+    if (((uintptr_t)a->packed_descriptors % 32) != 0) return VETRAST_ERR_INVALID_ARG;
     st = vetrast_workspace_layout_for_mode(a->num_points, a->num_views, p.num_layers, w, h, p.render_mode, lay);
     if (st != VETRAST_OK) return st;
     const size_t need = a->save_for_backward ? lay->total_bytes : lay->forward_only_bytes;
@@ -584,7 +585,10 @@ int vetrast_forward(vetrast_ctx* ctx, const vetrast_forward_args* a, void* strea
     const size_t Tpad   = lay.bin_counts_stride / sizeof(uint32_t) / 2;  // counts per view; as many words behind them
     void* ws            = a->workspace;
     uint32_t* flags     = ws_ptr<uint32_t>(ws, lay.flags_base);
-    float4* packed      = ws_ptr<float4>(ws, lay.packed_base);
+    // the caller's descriptor records where it keeps them current itself, else the workspace's, written by this call
+    const bool own_pack  = a->packed_descriptors == nullptr;
+    float4* packed       = own_pack ? ws_ptr<float4>(ws, lay.packed_base)
+                                    : reinterpret_cast<float4*>(const_cast<float*>(a->packed_descriptors));
     uint32_t* slots     = ws_ptr<uint32_t>(ws, lay.slots_base);
     uint32_t* partials  = ws_ptr<uint32_t>(ws, lay.scan_partials_base);
     DeviceView* views   = ws_ptr<DeviceView>(ws, lay.views_base);
@@ -636,7 +640,7 @@ int vetrast_forward(vetrast_ctx* ctx, const vetrast_forward_args* a, void* strea
         PackJob pack;
         pack.texture               = a->texture;
         pack.confidence            = a->confidence;
-        pack.packed                = b == 0 ? packed : nullptr;
+        pack.packed                = (b == 0 && own_pack) ? packed : nullptr;
         pack.N                     = N;
         pack.C                     = C;
         pack.confidence_activation = p.confidence_activation;
@@ -857,7 +861,8 @@ int vetrast_backward(vetrast_ctx* ctx, const vetrast_backward_args* g, void* str
             bp.transmittance    = ws_ptr<float>(ws, lay.transmittance_base + lay.transmittance_stride * b);
             bp.weight           = ws_ptr<float>(ws, lay.weight_base + lay.weight_stride * b);
             bp.index            = a->index;
-            bp.packed           = ws_ptr<float4>(ws, lay.packed_base);
+            bp.packed           = a->packed_descriptors ? reinterpret_cast<const float4*>(a->packed_descriptors)
+                                                        : ws_ptr<float4>(ws, lay.packed_base);
             bp.background       = ws_ptr<const float>(ws, lay.flags_base) + kPreparedBackgroundOffset;
             bp.partial          = partial;
             bp.background_partial = background_rows;
@@ -956,7 +961,8 @@ int vetrast_backward(vetrast_ctx* ctx, const vetrast_backward_args* g, void* str
                               ? 1
                               : 0;
             gp.background_accumulate = b > 0 ? 1 : 0;
-            gp.packed                = ws_ptr<float4>(ws, lay.packed_base);
+            gp.packed                = a->packed_descriptors ? reinterpret_cast<const float4*>(a->packed_descriptors)
+                                                             : ws_ptr<float4>(ws, lay.packed_base);
             gp.texture_raw           = a->texture;
             gp.background_raw        = a->background;
             gp.confidence_activation = p.confidence_activation;
@@ -1015,6 +1021,36 @@ int vetrast_backward(vetrast_ctx* ctx, const vetrast_backward_args* g, void* str
                            g->grad_pose_count, a->num_poses, g->grad_intrinsics, g->grad_intrinsics_count,
                            a->num_cameras);
     }
+    VET_HIP(ctx, hipGetLastError());
+    return VETRAST_OK;
+}
+
+size_t vetrast_packed_descriptor_bytes(int32_t num_points)
+{
+    return num_points > 0 ? (size_t)num_points * 2 * sizeof(float4) : 0;
+}
+
+int vetrast_pack_descriptors(vetrast_ctx* ctx, const vetrast_pack_args* a, void* stream_)
+{
+    if (!ctx || !a || a->num_points < 0) return VETRAST_ERR_INVALID_ARG;
+    const int C = a->params.num_texture_channels;
+    if (C < 1 || C > VETRAST_MAX_CHANNELS) return VETRAST_ERR_INVALID_ARG;
+    if (a->num_points == 0) return VETRAST_OK;
+    if (!a->texture || !a->confidence || !a->packed) return VETRAST_ERR_INVALID_ARG;
+    if (reinterpret_cast<uintptr_t>(a->packed) % (2 * sizeof(float4)) != 0) return VETRAST_ERR_INVALID_ARG;
+    PackJob pack;
+    pack.texture               = a->texture;
+    pack.confidence            = a->confidence;
+    pack.packed                = reinterpret_cast<float4*>(a->packed);
+    pack.N                     = a->num_points;
+    pack.C                     = C;
+    pack.confidence_activation = a->params.confidence_activation;
+    pack.confidence_scale      = a->params.confidence_scale;
+    pack.texture_abs           = a->params.texture_abs;
+    pack.visible_only          = 0;
+    hipStream_t stream         = (hipStream_t)stream_;
+    ScopeTimer tm(ctx, stream, VETRAST_SCOPE_PACK);
+    hipLaunchKernelGGL(pack_descriptors_kernel, dim3(grid_for(a->num_points)), dim3(kBlock), 0, stream, pack);
     VET_HIP(ctx, hipGetLastError());
     return VETRAST_OK;
 }

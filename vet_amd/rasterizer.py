@@ -231,8 +231,10 @@ class Rasterizer:
         return lay
 
     def forward(self, dev: DeviceScene, params: abi.Params = None, save_for_backward=True, workspace=None,
-                out=None, want_weight=False, point_order=None) -> ForwardResult:
-        """point_order: optional int32 device tensor [N], a permutation: the order the binning pass walks the points in."""
+                out=None, want_weight=False, point_order=None, packed=None) -> ForwardResult:
+        """point_order: optional int32 device tensor [N], a permutation: the order the binning pass walks the points in.
+        packed: optional float32 device tensor [N,8] from pack_descriptors: the call reads the descriptor records from
+        it instead of interleaving them itself."""
         scene = dev.scene
         params = params or make_params(scene)
         lay = self.layout(scene, params.render_mode)
@@ -262,8 +264,27 @@ class Rasterizer:
         if point_order is not None:
             assert point_order.dtype == torch.int32 and point_order.is_cuda and point_order.numel() == scene.num_points
             args.point_order = point_order.data_ptr()
+        if packed is not None:
+            assert packed.dtype == torch.float32 and packed.is_cuda and packed.is_contiguous()
+            assert packed.numel() == 8 * scene.num_points
+            args.packed_descriptors = packed.data_ptr()
         abi.check(self.lib.vetrast_forward(self.ctx, C.byref(args), self._stream()), "forward")
-        return ForwardResult(out, masks, workspace, lay, args, (views, dev, params, point_order), weights)
+        return ForwardResult(out, masks, workspace, lay, args, (views, dev, params, point_order, packed), weights)
+
+    def pack_descriptors(self, dev: DeviceScene, params: abi.Params, out=None) -> torch.Tensor:
+        """The descriptor records [N,8] of the scene's texture and confidence under `params` (vetrast_pack_descriptors),
+        for forward(..., packed=...)."""
+        n = dev.scene.num_points
+        assert self.lib.vetrast_packed_descriptor_bytes(n) == 32 * n
+        if out is None:
+            out = torch.empty((n, 8), dtype=torch.float32, device=dev.device)
+        a = abi.PackArgs()
+        a.num_points = n
+        a.texture, a.confidence = dev.ptr("texture"), dev.ptr("confidence")
+        C.memmove(C.byref(a.params), C.byref(params), C.sizeof(abi.Params))
+        a.packed = out.data_ptr()
+        abi.check(self.lib.vetrast_pack_descriptors(self.ctx, C.byref(a), self._stream()), "pack_descriptors")
+        return out
 
     def backward(self, fwd: ForwardResult, grad_out: List[torch.Tensor], want_points=True, want_cameras=False,
                  **param_overrides):

@@ -129,24 +129,106 @@ PointRendererCache::~PointRendererCache()
     vetrast_destroy(ctx);
 }
 
+static const char* kDistortionRefused =
+    "a camera has non-zero distortion coefficients (columns 5..12 of intrinsics): the distortion model of the "
+    "reference lives in saiga and is not implemented; such cameras are refused rather than rendered as "
+    "undistorted pinholes (RenderParams::allow_distortion switches the published rational model on)";
+
+void PointRendererCache::PollDeviceFlags()
+{
+    if (!flags_pending_ || !flags_event_ || !flags_event_->query()) return;
+    flags_pending_ = false;
+    if (flags_host_.data_ptr<int32_t>()[0] & 1)
+    {
+        checked_intrinsics_ptr_ = nullptr;  // the next call checks the tensor itself again, and blocks for it
+        TORCH_CHECK(false, "an earlier forward call rendered with these intrinsics: ", kDistortionRefused);
+    }
+}
+
 void PointRendererCache::CheckIntrinsics(const torch::Tensor& intrinsics)
 {
     TORCH_CHECK(intrinsics.defined() && intrinsics.dim() == 2 && intrinsics.size(1) == 13,
                 "intrinsics must be [num_cameras,13]");
+    PollDeviceFlags();
     const void* ptr       = intrinsics.data_ptr();
     const int64_t version = (int64_t)intrinsics._version();
-    if (ptr == checked_intrinsics_ptr_ && version == checked_intrinsics_version_ &&
-        intrinsics.numel() == checked_intrinsics_numel_)
+    const auto held = checked_intrinsics_storage_.lock();
+    if (ptr == checked_intrinsics_ptr_ && intrinsics.numel() == checked_intrinsics_numel_ && held &&
+        held.get() == intrinsics.storage().unsafeGetStorageImpl())
+    {
+        // known memory: no read here; ask for the device's own verdict on this call where the contents may have changed
+        if (version != checked_intrinsics_version_ || ++calls_since_flags_ >= 64) flags_wanted_ = true;
+        checked_intrinsics_version_ = version;
         return;
-    // blocking: one device -> host read per change of the tensor
+    }
+    // blocking: one device -> host read per intrinsics tensor
     const bool distorted = intrinsics.detach().slice(1, 5, 13).ne(0).any().item<bool>();
-    TORCH_CHECK(!distorted,
-                "a camera has non-zero distortion coefficients (columns 5..12 of intrinsics): the distortion model of the "
-                "reference lives in saiga and is not implemented; such cameras are refused rather than rendered as "
-                "undistorted pinholes");
+    TORCH_CHECK(!distorted, kDistortionRefused);
     checked_intrinsics_ptr_     = ptr;
+    checked_intrinsics_storage_ = intrinsics.storage().getWeakStorageImpl();
     checked_intrinsics_version_ = version;
     checked_intrinsics_numel_   = intrinsics.numel();
+    flags_wanted_               = false;
+    calls_since_flags_          = 0;
+}
+
+void PointRendererCache::NoteDeviceFlags(const torch::Tensor& workspace, const vetrast_workspace_layout& lay)
+{
+    if (!flags_wanted_ || flags_pending_) return;
+    torch::NoGradGuard no_grad;
+    if (!flags_host_.defined())
+        flags_host_ = torch::zeros({4}, torch::TensorOptions().dtype(torch::kInt32).pinned_memory(true));
+    flags_host_.copy_(workspace.narrow(0, (int64_t)lay.flags_base, 16).view(torch::kInt32), /*non_blocking=*/true);
+    if (!flags_event_) flags_event_ = std::make_unique<c10::Event>(c10::DeviceType::CUDA);
+    flags_event_->record(c10::hip::getCurrentHIPStreamMasqueradingAsCUDA());
+    flags_pending_     = true;
+    flags_wanted_      = false;
+    calls_since_flags_ = 0;
+}
+
+torch::Tensor PointRendererCache::KeptDescriptorsFor(const torch::Tensor& texture, const torch::Tensor& confidence,
+                                                     const vetrast_params& params)
+{
+    if (!keep_packed_descriptors) return torch::Tensor();
+    PackKey key;
+    key.texture            = texture.data_ptr();
+    key.confidence         = confidence.data_ptr();
+    key.texture_storage    = texture.storage().unsafeGetStorageImpl();
+    key.confidence_storage = confidence.storage().unsafeGetStorageImpl();
+    key.texture_version    = (int64_t)texture._version();
+    key.confidence_version = (int64_t)confidence._version();
+    key.N                  = confidence.numel();
+    key.C                  = params.num_texture_channels;
+    key.activation         = params.confidence_activation;
+    key.texture_abs        = params.texture_abs;
+    key.scale              = params.confidence_scale;
+    const bool alive       = pack_texture_storage_.lock() && pack_confidence_storage_.lock();
+    if (!(alive && key == pack_key_))
+    {
+        // first sight of these tensors in this state: remember them, interleave inside the call
+        pack_key_                = key;
+        pack_texture_storage_    = texture.storage().getWeakStorageImpl();
+        pack_confidence_storage_ = confidence.storage().getWeakStorageImpl();
+        packed_valid_            = false;
+        return torch::Tensor();
+    }
+    if (!packed_valid_)
+    {
+        // records a backward pass may still read (saved with its graph) are left alone
+        if (!packed_.defined() || packed_.use_count() > 1 || packed_.size(0) != key.N || packed_.device() != texture.device())
+            packed_ = torch::empty({key.N, 8}, texture.options().requires_grad(false));
+        vetrast_pack_args a;
+        std::memset(&a, 0, sizeof(a));
+        a.num_points = (int32_t)key.N;
+        a.texture    = texture.data_ptr<float>();
+        a.confidence = confidence.data_ptr<float>();
+        a.params     = params;
+        a.packed     = packed_.data_ptr<float>();
+        check_status(vetrast_pack_descriptors(ctx, &a, c10::hip::getCurrentHIPStream().stream()), "pack_descriptors");
+        packed_valid_ = true;
+    }
+    ++calls_with_kept_descriptors;
+    return packed_;
 }
 
 void PointRendererCache::FillSceneGridWithLoss(int batch, const CellTensors& cells,
@@ -233,6 +315,8 @@ torch::autograd::variable_list PointRender::forward(torch::autograd::AutogradCon
     check_status(vetrast_workspace_layout_for_mode(a.num_points, B, L, info->images[0].w, info->images[0].h,
                                                    a.params.render_mode, &lay),
                  "layout");
+    const torch::Tensor kept_pack = info->cache->KeptDescriptorsFor(texture, confidence, a.params);
+    if (kept_pack.defined()) a.packed_descriptors = kept_pack.data_ptr<float>();
 
     const bool need_backward =
         ctx != nullptr && (texture.requires_grad() || background_color.requires_grad() || points.requires_grad() ||
@@ -286,6 +370,7 @@ torch::autograd::variable_list PointRender::forward(torch::autograd::AutogradCon
     const torch::Tensor& order = info->cache->PointOrderFor(points);
     a.point_order              = order.defined() ? order.data_ptr<int32_t>() : nullptr;
     check_status(vetrast_forward(info->cache->ctx, &a, current_stream()), "forward");
+    if (!info->params.allow_distortion) info->cache->NoteDeviceFlags(workspace, lay);
     if (info->params.size_bins_from_history)
         info->cache->NoteFragmentCounts(workspace, lay, N, L, info->images[0].w, info->images[0].h, a.params.render_mode);
 
@@ -297,7 +382,9 @@ torch::autograd::variable_list PointRender::forward(torch::autograd::AutogradCon
         saved.insert(saved.end(), out.begin(), out.end());
         if (dropout.defined()) saved.push_back(dropout);
         if (t_index.defined()) saved.push_back(t_index);
+        if (kept_pack.defined()) saved.push_back(kept_pack);
         ctx->save_for_backward(saved);
+        ctx->saved_data["has_kept_pack"] = kept_pack.defined();
         ctx->saved_data["has_dropout"] = dropout.defined();
         ctx->saved_data["has_index"]   = t_index.defined();
         ctx->saved_data["points_need_grad"] = points.requires_grad();
@@ -333,7 +420,8 @@ torch::autograd::variable_list PointRender::backward(torch::autograd::AutogradCo
     const bool has_dropout   = ctx->saved_data["has_dropout"].toBool();
     const bool has_index     = ctx->saved_data["has_index"].toBool();
     constexpr int kFixed     = 7;
-    TORCH_CHECK((int)saved.size() == kFixed + L + (has_dropout ? 1 : 0) + (has_index ? 1 : 0),
+    const bool has_kept_pack = ctx->saved_data["has_kept_pack"].toBool();
+    TORCH_CHECK((int)saved.size() == kFixed + L + (has_dropout ? 1 : 0) + (has_index ? 1 : 0) + (has_kept_pack ? 1 : 0),
                 "unexpected number of saved tensors");  // PointRenderer.cu:1163-1164
     TORCH_CHECK((int)grad_output.size() >= L, "expected one upstream gradient per layer");  // PointRenderer.cu:1158-1159
     torch::Tensor workspace = saved[0], texture = saved[1], background_color = saved[2], points = saved[3],
@@ -356,6 +444,7 @@ torch::autograd::variable_list PointRender::backward(torch::autograd::AutogradCo
     g.fwd.workspace         = workspace.data_ptr();
     g.fwd.workspace_bytes   = (size_t)workspace.numel();
     g.fwd.save_for_backward = 1;
+    if (has_kept_pack) g.fwd.packed_descriptors = saved.back().data_ptr<float>();
 
     // zeros_like of each gradient tensor (PointRenderer.cu:267-277); the library overwrites them.
     torch::Tensor g_texture    = torch::empty_like(texture);
@@ -739,8 +828,8 @@ void PointRendererCache::ExpectedFragments(float* expected, int64_t N, int L, in
     PollFragmentCounts();
     CountsKey key;
     key.N = N, key.L = L, key.w = w, key.h = h, key.mode = render_mode;
-    const bool known = counts_valid_ && counts_key_ == key;
-    for (int l = 0; l < VETRAST_MAX_LAYERS; ++l) expected[l] = (known && l < L) ? counts_[l] + 1024.f : 0.f;
+    if (!(counts_valid_ && counts_key_ == key)) return;  // no history for such calls yet: the caller's own hints stand
+    for (int l = 0; l < VETRAST_MAX_LAYERS; ++l) expected[l] = l < L ? counts_[l] + 1024.f : 0.f;
 }
 
 void PointRendererCache::NoteFragmentCounts(const torch::Tensor& workspace, const vetrast_workspace_layout& lay, int64_t N,
@@ -965,6 +1054,9 @@ void MyAdam::step(bool zero_grad)
             a.weight_decay = weight_decay_;
             a.zero_grad    = zero_grad ? 1 : 0;
             check_status(vetrast_adam_step(cache_->ctx, &a, c10::hip::getCurrentHIPStream().stream()), "adam_step");
+            // the kernel wrote through raw pointers: tell everyone who keys on the version counters
+            p.unsafeGetTensorImpl()->bump_version();
+            if (zero_grad) grad.unsafeGetTensorImpl()->bump_version();
         }
 }
 
@@ -1201,6 +1293,16 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
         "point_order",
         []() { return (g_cache && g_cache->point_order.defined()) ? g_cache->point_order : torch::Tensor(); },
         "the processing order the cache currently holds (undefined tensor: none)");
+    m.def(
+        "kept_descriptor_calls", []() { return g_cache ? g_cache->calls_with_kept_descriptors : (int64_t)0; },
+        "forward calls of the binding's cache so far that read descriptor records kept from an earlier call");
+    m.def(
+        "set_keep_packed_descriptors",
+        [](bool keep) {
+            if (!g_cache) g_cache = std::make_shared<vet_amd::PointRendererCache>();
+            g_cache->keep_packed_descriptors = keep;
+        },
+        "whether the binding's cache keeps descriptor records across calls while texture and confidence stay unchanged");
     m.def(
         "train_workspace_info",
         []() {

@@ -110,10 +110,14 @@ class PointRendererCache
     // nothing but this cache still holds it (the graph of that step has been released) and it is large enough: a
     // training loop then runs in one workspace instead of allocating one per step.
     torch::Tensor train_workspace;
-    // Cameras with non-zero distortion coefficients are refused (their model lives in saiga, which is not available). The
-    // coefficients sit in device memory, so checking them costs a blocking read: it is only repeated when the intrinsics
-    // tensor or its version counter changes. Throws if columns 5..12 of `intrinsics` [num_cameras,13] are not all zero.
+    // Cameras with non-zero distortion coefficients are refused unless RenderParams::allow_distortion is set. The
+    // coefficients sit in device memory. The first call for an intrinsics tensor (its memory and size) reads columns
+    // 5..12 of `intrinsics` [num_cameras,13] back, which blocks, and throws if they are not all zero. Later calls never
+    // block: when the tensor's version counter has moved (an optimiser step), and every 64th call whatever the counter
+    // says (writes through a raw pointer leave it alone), NoteDeviceFlags copies the status word that the forward call
+    // raises on the device to pinned memory behind the call, and the next call that finds the copy landed throws.
     void CheckIntrinsics(const torch::Tensor& intrinsics);
+    void NoteDeviceFlags(const torch::Tensor& workspace, const vetrast_workspace_layout& lay);
     // The order in which the binning pass walks the points (vetrast_forward_args.point_order): Morton order with shuffled
     // 256-point blocks, built on the device from the positions, rebuilt when the number of points changes and every
     // `point_order_refresh` forward calls (positions drift while they are optimised; the order only has to be roughly
@@ -123,6 +127,16 @@ class PointRendererCache
     int64_t point_order_refresh = 1000;
     torch::Tensor point_order;  // int32 [N] on the points' device, or undefined
     const torch::Tensor& PointOrderFor(const torch::Tensor& points);
+    // Descriptor records kept across calls (vetrast_forward_args.packed_descriptors). A forward call that finds texture
+    // and confidence as the call before left them (same storage, same version counters, same activation settings)
+    // packs them once with vetrast_pack_descriptors; the calls after it read those records, until one of the tensors
+    // changes: a viewer or an evaluation loop renders a scene many times between changes. A training step, whose
+    // optimiser moves the tensors every step, never gets that far and interleaves inside the call. Writers that go
+    // around the version counter must bump it (vet_amd::MyAdam does). false: never keep records.
+    bool keep_packed_descriptors = true;
+    torch::Tensor KeptDescriptorsFor(const torch::Tensor& texture, const torch::Tensor& confidence,
+                                     const vetrast_params& params);
+    int64_t calls_with_kept_descriptors = 0;  // forward calls so far that read kept records
     // Fragments per layer that a view of recent calls left, for RenderParams::expected_fragments: every 16th forward
     // call copies the layer boundaries of view 0's scan to pinned host memory without blocking; the numbers are taken
     // up by a later call once the copy has landed. Kept per image size, layer count, point count and render mode.
@@ -147,9 +161,37 @@ class PointRendererCache
     torch::Tensor lift_workspace;
 
    private:
+    // the storage is held weakly: while it is, no other tensor's memory can pass for it at the same address
     const void* checked_intrinsics_ptr_ = nullptr;
+    c10::weak_intrusive_ptr<c10::StorageImpl> checked_intrinsics_storage_{c10::intrusive_ptr<c10::StorageImpl>()};
     int64_t checked_intrinsics_version_ = -1, checked_intrinsics_numel_ = -1;
+    bool flags_wanted_ = false, flags_pending_ = false;
+    int64_t calls_since_flags_ = 0;
+    torch::Tensor flags_host_;
+    std::unique_ptr<c10::Event> flags_event_;
+    void PollDeviceFlags();
     int64_t point_order_age_ = 0;
+    struct PackKey
+    {
+        const void *texture = nullptr, *confidence = nullptr;
+        const void *texture_storage = nullptr, *confidence_storage = nullptr;
+        int64_t texture_version = -1, confidence_version = -1, N = -1;
+        int C = 0, activation = 0, texture_abs = 0;
+        float scale = 0.f;
+        bool operator==(const PackKey& o) const
+        {
+            return texture == o.texture && confidence == o.confidence && texture_storage == o.texture_storage &&
+                   confidence_storage == o.confidence_storage && texture_version == o.texture_version &&
+                   confidence_version == o.confidence_version && N == o.N && C == o.C && activation == o.activation &&
+                   texture_abs == o.texture_abs && scale == o.scale;
+        }
+    };
+    PackKey pack_key_;
+    // held weakly so that the storages the key names cannot be freed and their addresses handed to other tensors
+    c10::weak_intrusive_ptr<c10::StorageImpl> pack_texture_storage_{c10::intrusive_ptr<c10::StorageImpl>()};
+    c10::weak_intrusive_ptr<c10::StorageImpl> pack_confidence_storage_{c10::intrusive_ptr<c10::StorageImpl>()};
+    bool packed_valid_ = false;
+    torch::Tensor packed_;
     struct CountsKey
     {
         int64_t N = -1;

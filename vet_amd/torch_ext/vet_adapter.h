@@ -114,7 +114,8 @@ c10::intrusive_ptr<NeuralRenderInfo> RenderInfoOf(const InfoT& info, PointRender
 }
 
 // BlendPointCloud(NeuralRenderInfo*) of the reference (src/lib/rendering/RenderInfo.cpp:18-47) on the reference's own
-// info object: L images, then L masks with output_background_mask, then L depth images with add_depth_to_network.
+// info object: L images, then L depth images with add_depth_to_network, then L masks with output_background_mask
+// (the order of src/lib/rendering/PointRenderer.cu:1061-1066).
 template <class InfoT>
 std::vector<torch::Tensor> BlendPointCloudOf(InfoT* info, PointRendererCache* cache, SceneTensors* bundle)
 {

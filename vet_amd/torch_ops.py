@@ -102,6 +102,16 @@ def fragment_history():
     return list(load().fragment_history())
 
 
+def kept_descriptor_calls():
+    """Forward calls of the shim's cache so far that read descriptor records kept from an earlier call."""
+    return int(load().kept_descriptor_calls())
+
+
+def set_keep_packed_descriptors(keep):
+    """Whether the shim's cache keeps descriptor records across calls while texture and confidence stay unchanged."""
+    load().set_keep_packed_descriptors(bool(keep))
+
+
 def train_workspace_info():
     """(data_ptr, bytes) of the workspace the binding's cache keeps between training steps; (0, 0) before the first."""
     d = load().train_workspace_info()
