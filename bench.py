@@ -208,6 +208,7 @@ def run_scene(scene, backward, steps, warmup, samples, profile=True, render_mode
 
         res["kept_descriptors"] = {
             "ms_per_step": round(timed_samples(kept_step, 3, steps, samples)["median"], 5),
+            "plain_step_timed_right_after_ms": round(timed_samples(step, 3, steps, samples)["median"], 5),
             "forward_ms": round(timed_samples(kept_forward, 3, steps, samples)["median"], 5),
             "pack_ms": round(timed_samples(lambda: rast.pack_descriptors(dev, params, out=packed), 3, steps, samples)["median"], 5),
             "what": "the same step with vetrast_forward_args.packed_descriptors set (records written once by "

@@ -409,6 +409,7 @@ def test_the_cache_keeps_a_processing_order_and_results_do_not_depend_on_it():
         out1, grad1 = run()
         first = torch_ops.point_order()
         assert first is not None and first.dtype == torch.int32 and first.numel() == scene.num_points
+        assert torch_ops.point_order_in_use(), "a fifth of this cloud was appended unsorted: the order pays"
         assert torch.equal(torch.sort(first.long()).values, torch.arange(scene.num_points, device="cuda"))
         ptr = first.data_ptr()
         run()
@@ -423,6 +424,26 @@ def test_the_cache_keeps_a_processing_order_and_results_do_not_depend_on_it():
             scene.confidence[:20_000]
         run()
         assert torch_ops.point_order().numel() == 20_000
+    finally:
+        torch_ops.set_point_order_refresh(1000)
+
+
+def test_a_cloud_in_preprocessed_order_goes_without_the_order_array():
+    """The cache compares how far apart the 64 points of a wave lie in array order and in the order it has built; a
+    cloud that comes in the order of VET's preprocessing (src/lib/data/SceneData.cpp:105-106) is as good as it is, so
+    its calls are not handed the array; one in the generator's raw order is."""
+    from vet_amd import torch_ops
+
+    try:
+        torch_ops.set_point_order_refresh(1000)
+        for order, used in (("vet_preprocess", False), ("generated", True), ("vet_preprocess", False)):
+            # (2 000 points on each of the generator's 200 surfaces: a run of 64 of them spans its whole surface)
+            scene = synthetic.config2(num_points=400_000, w=320, h=180, point_order=order)
+            assert len(_plain_call(scene, torch_ops)) == scene.num_layers
+            assert torch_ops.point_order() is not None and torch_ops.point_order_in_use() == used, order
+            scene = synthetic.config2(num_points=409_600, w=320, h=180, point_order=order)  # another size: rebuilt
+            _plain_call(scene, torch_ops)
+            assert torch_ops.point_order_in_use() == used, order
     finally:
         torch_ops.set_point_order_refresh(1000)
 

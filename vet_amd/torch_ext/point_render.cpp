@@ -874,9 +874,28 @@ const torch::Tensor& PointRendererCache::PointOrderFor(const torch::Tensor& poin
     {
         point_order      = ProcessingOrderOnDevice(points, 256, 0);
         point_order_age_ = 0;
+        // Is the array's own order as good? What the binning pass wants is that the 64 points of a wave lie close
+        // together: the summed extent of the runs of 64 points, in array order and in the new order. A cloud in the
+        // order of VET's preprocessing passes as it is and the call then goes without the order array (one index
+        // read and one position gather per point less, and single-view calls may leave the descriptor rows of points
+        // outside the view alone). One blocking read per rebuild, which costs milliseconds anyway.
+        torch::NoGradGuard no_grad;
+        const int64_t runs = points.size(0) / 64;
+        point_order_in_use = true;
+        if (runs > 0)
+        {
+            auto extent = [&](const torch::Tensor& xyz) {
+                const torch::Tensor r = xyz.narrow(0, 0, runs * 64).view({runs, 64, 3});
+                return (std::get<0>(r.max(1)) - std::get<0>(r.min(1))).sum().item<double>();
+            };
+            const torch::Tensor xyz = points.detach().narrow(1, 0, 3);
+            const double as_is      = extent(xyz);
+            const double ordered    = extent(xyz.index_select(0, point_order.to(torch::kInt64)));
+            point_order_in_use      = ordered < 0.8 * as_is;
+        }
     }
     ++point_order_age_;
-    return point_order;
+    return point_order_in_use ? point_order : no_point_order_;
 }
 
 torch::Tensor SortBlocksByRadiusOrder(torch::Tensor radius, int64_t block)
@@ -1293,6 +1312,9 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
         "point_order",
         []() { return (g_cache && g_cache->point_order.defined()) ? g_cache->point_order : torch::Tensor(); },
         "the processing order the cache currently holds (undefined tensor: none)");
+    m.def(
+        "point_order_in_use", []() { return g_cache && g_cache->point_order.defined() && g_cache->point_order_in_use; },
+        "whether forward calls are handed the cache's processing order (false: the array's own order is as good)");
     m.def(
         "kept_descriptor_calls", []() { return g_cache ? g_cache->calls_with_kept_descriptors : (int64_t)0; },
         "forward calls of the binding's cache so far that read descriptor records kept from an earlier call");

@@ -126,6 +126,9 @@ class PointRendererCache
     // binning pass with it, one in VET's order loses nothing. 0: never build one, walk the array as it is.
     int64_t point_order_refresh = 1000;
     torch::Tensor point_order;  // int32 [N] on the points' device, or undefined
+    // false: the array's own order keeps the 64 points of a wave as close together as the built order would (checked
+    // at every rebuild), and calls go without an order array
+    bool point_order_in_use = true;
     const torch::Tensor& PointOrderFor(const torch::Tensor& points);
     // Descriptor records kept across calls (vetrast_forward_args.packed_descriptors). A forward call that finds texture
     // and confidence as the call before left them (same storage, same version counters, same activation settings)
@@ -171,6 +174,7 @@ class PointRendererCache
     std::unique_ptr<c10::Event> flags_event_;
     void PollDeviceFlags();
     int64_t point_order_age_ = 0;
+    torch::Tensor no_point_order_;  // stays undefined
     struct PackKey
     {
         const void *texture = nullptr, *confidence = nullptr;

@@ -97,6 +97,11 @@ def point_order():
     return t if t is not None and t.numel() > 0 else None
 
 
+def point_order_in_use():
+    """Whether forward calls are handed the processing order (False: the array's own order is as good)."""
+    return bool(load().point_order_in_use())
+
+
 def fragment_history():
     """Fragments per layer that one view of a recent call left, as the shim's cache has read them back ([] = none yet)."""
     return list(load().fragment_history())
