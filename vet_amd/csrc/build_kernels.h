@@ -195,7 +195,8 @@ __global__ void __launch_bounds__(kBlock) bin_build_kernel(BuildPass a)
     __shared__ uint64_t s_block_sorted[kBlock / kWave];  // pixels whose lists the whole workgroup sorts, a mask per wave
     __shared__ uint64_t s_keys[kBuildCap];
     __shared__ uint8_t s_pix[kBuildCap];       // pixel (inside the bin) of every list place
-    __shared__ float4 s_stage[kStage][2];      // descriptor, confidence of the staged fragments
+    __shared__ float4 s_stage[2][kStage];      // descriptors, then confidences (and depths) of the staged fragments: two
+                                               // planes, so that the lanes of a store or load are 16 bytes apart
     const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
     const uint32_t bin = a.num_bins - 1u - blockIdx.x;  // coarse layers first
     int l              = 0;
@@ -346,8 +347,8 @@ __global__ void __launch_bounds__(kBlock) bin_build_kernel(BuildPass a)
                 }
                 // FUZZY_BLEND buckets by depth: it rides along in the stage (the key's depth half is still intact here)
                 if constexpr (FUZZY) c4.y = __uint_as_float(s_id[2 * r + 1]);
-                s_stage[r - base][0] = t4;
-                s_stage[r - base][1] = c4;
+                s_stage[0][r - base] = t4;
+                s_stage[1][r - base] = c4;
             }
             __syncthreads();
             if ((uint32_t)tid < pixels)
@@ -361,8 +362,8 @@ __global__ void __launch_bounds__(kBlock) bin_build_kernel(BuildPass a)
                     // transmittance in front of the bucket the fragment joins.
                     for (; r < hi && fuzzy.open; ++r)
                     {
-                        const float4 t4 = s_stage[r - base][0];
-                        const float2 cd = *reinterpret_cast<const float2*>(&s_stage[r - base][1]);  // confidence, depth
+                        const float4 t4 = s_stage[0][r - base];
+                        const float2 cd = *reinterpret_cast<const float2*>(&s_stage[1][r - base]);  // confidence, depth
                         const float t[4] = {t4.x, t4.y, t4.z, t4.w};
                         const bool joined = fuzzy.take(cd.y, cd.x, t, a.depth_accept, T, color);
                         s_T[2 * r + 1] = T;
@@ -376,8 +377,8 @@ __global__ void __launch_bounds__(kBlock) bin_build_kernel(BuildPass a)
                 }
                 for (; r < hi && !saturated; ++r)
                 {
-                    const float4 t4 = s_stage[r - base][0];
-                    const float cf  = s_stage[r - base][1].x;
+                    const float4 t4 = s_stage[0][r - base];
+                    const float cf  = s_stage[1][r - base].x;
                     const float t[4] = {t4.x, t4.y, t4.z, t4.w};
                     s_T[2 * r + 1]  = T;
                     const float Tc   = T * cf;
@@ -485,8 +486,8 @@ __global__ void __launch_bounds__(kBlock) bin_build_kernel(BuildPass a)
                         c4.x = fragment_alpha<BILINEAR>(a, l, low, c4.x);
                     }
                     if constexpr (FUZZY) c4.y = __uint_as_float((uint32_t)(k64 >> 32));
-                    s_stage[r - base][0] = t4;
-                    s_stage[r - base][1] = c4;
+                    s_stage[0][r - base] = t4;
+                    s_stage[1][r - base] = c4;
                 }
                 __syncthreads();
                 if ((uint32_t)tid < pixels)
@@ -497,8 +498,8 @@ __global__ void __launch_bounds__(kBlock) bin_build_kernel(BuildPass a)
                     {
                         for (; r < hi && fuzzy.open; ++r)  // the nearest bucket, as above
                         {
-                            const float4 t4 = s_stage[r - base][0];
-                            const float2 cd = *reinterpret_cast<const float2*>(&s_stage[r - base][1]);  // confidence, depth
+                            const float4 t4 = s_stage[0][r - base];
+                            const float2 cd = *reinterpret_cast<const float2*>(&s_stage[1][r - base]);  // confidence, depth
                             const float t[4] = {t4.x, t4.y, t4.z, t4.w};
                             const bool joined = fuzzy.take(cd.y, cd.x, t, a.depth_accept, T, color);
                             if (a.transmittance) a.transmittance[begin + r] = T;
@@ -512,8 +513,8 @@ __global__ void __launch_bounds__(kBlock) bin_build_kernel(BuildPass a)
                     }
                     for (; r < hi && !saturated; ++r)
                     {
-                        const float4 t4 = s_stage[r - base][0];
-                        const float cf  = s_stage[r - base][1].x;
+                        const float4 t4 = s_stage[0][r - base];
+                        const float cf  = s_stage[1][r - base].x;
                         const float t[4] = {t4.x, t4.y, t4.z, t4.w};
                         if (a.transmittance) a.transmittance[begin + r] = T;
                         const float Tc = T * cf;
