@@ -173,9 +173,10 @@ def test_the_binding_keeps_records_only_while_the_tensors_stand_still(oracle):
     torch_ops.set_keep_packed_descriptors(True)
 
 
-def test_gradients_through_kept_records_in_the_binding(oracle):
-    """Two forward+backward passes on unchanged leaves (gradient accumulation without an optimiser step in between):
-    the second reads kept records, in its backward pass too, and adds the same gradients again."""
+def test_the_binding_keeps_records_for_calls_without_a_backward_pass_only(oracle):
+    """Forward calls that are saved for a backward pass interleave inside the call whatever the tensors did since the
+    last call (gradient accumulation over unchanged leaves gives the same gradients every time); calls under no_grad
+    on the same leaves read kept records from the second one on, with the same images."""
     from vet_amd import torch_ops
 
     scene = synthetic.tiny_scene(num_points=3000, K=8, seed=76)
@@ -183,14 +184,21 @@ def test_gradients_through_kept_records_in_the_binding(oracle):
     texture = cu(scene.texture).requires_grad_(True)
     confidence = cu(scene.confidence.reshape(1, -1)).requires_grad_(True)
     torch_ops.set_keep_packed_descriptors(True)
-    grads = []
+    grads, images = [], []
     calls = torch_ops.kept_descriptor_calls()
     for k in range(3):
         texture.grad = confidence.grad = None
         outs = _plain_call(scene, torch_ops, texture=texture, confidence=confidence, train=True)
         sum((o * o).sum() for o in outs).backward()
         grads.append((texture.grad.clone(), confidence.grad.clone()))
-    assert torch_ops.kept_descriptor_calls() == calls + 2
+        images.append([o.detach().clone() for o in outs])
+    assert torch_ops.kept_descriptor_calls() == calls
     for gt, gc in grads[1:]:
         assert torch.equal(gt, grads[0][0]) and torch.equal(gc, grads[0][1])
     assert float(grads[0][0].abs().sum()) > 0
+    with torch.no_grad():
+        for k in range(3):
+            outs = _plain_call(scene, torch_ops, texture=texture, confidence=confidence)
+            for a, b in zip(outs, images[0]):
+                assert torch.equal(a, b)
+    assert torch_ops.kept_descriptor_calls() == calls + 2

@@ -15,8 +15,9 @@ pytestmark = pytest.mark.gpu
 
 @pytest.mark.parametrize("render_mode", [abi.RENDER_FULL_BLEND, abi.RENDER_BILINEAR_BLEND])
 @pytest.mark.parametrize("with_index", [False, True])
-def test_fused_preparation_matches_oracle(render_mode, with_index, rasterizer, oracle):
-    scene = _raw_scene(51, num_points=6000, K=8, num_views=2)
+@pytest.mark.parametrize("num_views", [1, 2])  # (a call with one view interleaves the rows of visible points only)
+def test_fused_preparation_matches_oracle(render_mode, with_index, num_views, rasterizer, oracle):
+    scene = _raw_scene(51, num_points=6000, K=8, num_views=num_views)
     if with_index:
         scene.index = np.random.default_rng(3).integers(0, 1200, size=scene.num_points).astype(np.int32)
     params = make_params(scene, need_point_gradient=1, render_mode=render_mode, quirk_background_confidence_leak=1,
@@ -24,7 +25,7 @@ def test_fused_preparation_matches_oracle(render_mode, with_index, rasterizer, o
     ref = oracle.forward(scene, params)
     res = rasterizer.forward(DeviceScene(scene), params)
     torch.cuda.synchronize()
-    for b in range(2):
+    for b in range(num_views):
         np.testing.assert_array_equal(res.offsets(b), ref.offsets[b].astype(np.int64))
         np.testing.assert_array_equal(res.weight(b), ref.weight[b])
     for l in range(scene.num_layers):

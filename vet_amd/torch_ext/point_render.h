@@ -130,12 +130,13 @@ class PointRendererCache
     // at every rebuild), and calls go without an order array
     bool point_order_in_use = true;
     const torch::Tensor& PointOrderFor(const torch::Tensor& points);
-    // Descriptor records kept across calls (vetrast_forward_args.packed_descriptors). A forward call that finds texture
-    // and confidence as the call before left them (same storage, same version counters, same activation settings)
-    // packs them once with vetrast_pack_descriptors; the calls after it read those records, until one of the tensors
-    // changes: a viewer or an evaluation loop renders a scene many times between changes. A training step, whose
-    // optimiser moves the tensors every step, never gets that far and interleaves inside the call. Writers that go
-    // around the version counter must bump it (vet_amd::MyAdam does). false: never keep records.
+    // Descriptor records kept across calls (vetrast_forward_args.packed_descriptors), for forward calls that no
+    // backward pass follows. Such a call that finds texture and confidence as the one before left them (same storage,
+    // same version counters, same activation settings) packs them once with vetrast_pack_descriptors; the calls after
+    // it read those records, until one of the tensors changes: a viewer or an evaluation loop renders a scene many
+    // times between changes. Calls that are saved for a backward pass always interleave inside the call (that also
+    // warms the cache for the backward pass's gathers, which is worth more than the interleave costs). Writers that
+    // go around the version counter must bump it (vet_amd::MyAdam does). false: never keep records.
     bool keep_packed_descriptors = true;
     torch::Tensor KeptDescriptorsFor(const torch::Tensor& texture, const torch::Tensor& confidence,
                                      const vetrast_params& params);
@@ -219,6 +220,9 @@ class NeuralRenderInfo : public torch::CustomClassHolder
     RenderParams params;
     int num_layers           = 1;
     bool train               = false;
+    // Set by BlendPointCloud: whether autograd was recording when the call was made. Under torch::NoGradGuard nothing
+    // is saved for a backward pass, whatever the leaves require.
+    bool grad_mode           = true;
     int current_epoch        = 0;
     void* timer_system       = nullptr;  // accepted for signature parity; per-kernel times come from vetrast_scope_times
     PointRendererCache* cache = nullptr;
