@@ -102,6 +102,9 @@ class WorkspaceLayout(C.Structure):
         ("primary_base", C.c_size_t), ("log_base", C.c_size_t), ("log_cursor_base", C.c_size_t),
         ("last_key_base", C.c_size_t), ("last_key_stride", C.c_size_t),
         ("projected_base", C.c_size_t), ("projected_stride", C.c_size_t),
+        ("view_lanes", C.c_int32), ("reserved2", C.c_int32),
+        ("binned_stride", C.c_size_t), ("primary_stride", C.c_size_t), ("scan_partials_stride", C.c_size_t),
+        ("lane_scratch_stride", C.c_size_t),
     ]
 
 

@@ -1413,13 +1413,20 @@ struct GatherPass
     double* camera_partial;   // [workgroups][kCameraRow] per-workgroup pose / intrinsics sums, or null
     int K;
     int need_point_gradient;
-    int accumulate;  // 0: overwrite the gradient rows (first view), 1: add to them (further views)
+    // One launch takes a round of up to kViewLanes views: the pointers above are those of the round's first view, view
+    // v of the round lies v * the stride behind them (per-view arrays of the workspace; the record and background-row
+    // arrays of the view's lane; a camera-row block per view). A point's position is read once for all of them and its
+    // gradient rows are written once.
+    int view_count;
+    size_t dropout_stride, flags_stride, last_key_stride, kept_stride;  // elements of the respective arrays
+    size_t partial_stride, background_rows_stride, camera_partial_stride;
+    int accumulate;  // 0: overwrite the gradient rows (the call's first round), 1: add to them (further rounds)
     // background gradient: workgroup 0 also sums the rows the per-pixel kernel left (hidden behind the other workgroups)
     const float* background_rows;
     int num_background_rows;
     float* grad_background;
     int add_leak;
-    int background_accumulate;
+    int background_accumulate;  // for the round's first view; the others always add
     // chain rule of the fused preparation steps (confidence = sigmoid(scale * raw), texture = |raw|, background = |raw|):
     // the gradients written are those of the raw tensors
     const float4* packed;      // prepared confidence of a row: packed[2 * row + 1].x
@@ -1444,28 +1451,44 @@ constexpr int kCameraSums = 18;  // of them sums of per-fragment terms
 // descriptor and confidence sums are added with atomics (onto rows the host zero-filled).
 // HITS = 4 (BILINEAR_BLEND): a point has up to four fragments per layer, one per corner of its 2x2 pixels, with records
 // at partial[layer][corner][point].
-template <int C, int HITS, bool DISTORT = false>
+// MANY: the launch takes a round of several views (a.view_count of them); otherwise one view, and the loop over the
+// views and its address arithmetic fold away (the kernel then needs 58 registers instead of 71 to 77, and it lives
+// off the number of waves in flight).
+template <int C, int HITS, bool DISTORT = false, bool MANY = false>
 __global__ void __launch_bounds__(kBlock) gather_point_gradients_kernel(GatherPass a)
 {
+    const int view_count = MANY ? a.view_count : 1;
     const int i      = blockIdx.x * blockDim.x + threadIdx.x;
     const bool alive = i < a.vp.N;
+    const int N      = a.vp.N;
+    // sums over the fragments of the point in all views of the round
     float gt[C];
 #pragma unroll
     for (int ci = 0; ci < C; ++ci) gt[ci] = 0.f;
     float gc = 0.f, gx = 0.f, gy = 0.f, gz = 0.f, cnt = 0.f;
-    bool hit = false;   // the point has a blended fragment in this view
-    // pose tangent (translation, rotation), fx, fy, cx, cy and, in the kernel for cameras with distortion, k1 .. p2
+    bool hit = false;   // the point has a blended fragment in one of the views
     constexpr int kSums = DISTORT ? kCameraSums : 10;
+    const float4 wp     = alive ? a.vp.position[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+    // skipped in every view alike (viewer cut-off), or in this view (drop-out mask)
+    const bool never = !alive || point_is_skipped_in_all_views(a.vp, i);
+  for (int view = 0; view < view_count; ++view)
+  {
+    const float* dropout       = a.vp.dropout ? a.vp.dropout + (size_t)view * a.dropout_stride : nullptr;
+    const uint8_t* list_is_cut = a.list_is_cut + (size_t)view * a.flags_stride;
+    const uint64_t* last_key   = a.last_key + (size_t)view * a.last_key_stride;
+    const float4* partial      = a.partial + (size_t)view * a.partial_stride;
+    // pose tangent (translation, rotation), fx, fy, cx, cy and, in the kernel for cameras with distortion, k1 .. p2:
+    // per view
     float cam_sum[kSums];
 #pragma unroll
     for (int k = 0; k < kSums; ++k) cam_sum[k] = 0.f;
+    float view_cnt = 0.f;
     Projected p;
-    const DeviceView& cam = *a.vp.view;
-    const float4 wp       = alive ? a.vp.position[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+    const DeviceView& cam = a.vp.view[view];
     // (a position further outside the image than the coarsest layer's border pixels reach has no fragment in any
     // layer, see bin_scatter_kernel: most of the cloud, for a crop)
     const float reach = (float)(1 << (a.vp.ly.L - 1)) + 1.f;
-    if (alive && !point_is_skipped(a.vp, i) && project_point(cam, wp, p) && p.ipx >= -reach &&
+    if (!never && !(dropout && dropout[i] == 1.f) && project_point(cam, wp, p) && p.ipx >= -reach &&
         p.ipx <= (float)a.vp.ly.w[0] + reach && p.ipy >= -reach && p.ipy <= (float)a.vp.ly.h[0] + reach)
     {
         // view-space position again, for the projection Jacobian (same expressions as project_point)
@@ -1491,14 +1514,14 @@ __global__ void __launch_bounds__(kBlock) gather_point_gradients_kernel(GatherPa
             // cut, saturation) the last blended key has to be looked up.
             // (FULL_BLEND without a cut never sets the flag; the K > 0 test keeps a corrupted flag byte from turning
             // K <= 0 into an index.)
-            if (a.list_is_cut[q] && (HITS != 1 || a.K > 0))
+            if (list_is_cut[q] && (HITS != 1 || a.K > 0))
             {
                 const uint64_t key = depth_key | (HITS == 1 ? (uint32_t)i : (((uint32_t)i << 2) | (uint32_t)h));
-                if (key > a.last_key[q]) continue;  // 0 where no fragment was blended: every key is beyond it
+                if (key > last_key[q]) continue;  // 0 where no fragment was blended: every key is beyond it
             }
             const size_t rec = (size_t)(l * HITS + h) * a.vp.N + i;
-            const float4 r0  = a.partial[2 * rec];
-            const float4 r1  = a.partial[2 * rec + 1];
+            const float4 r0  = partial[2 * rec];
+            const float4 r1  = partial[2 * rec + 1];
             const float r[4] = {r0.x, r0.y, r0.z, r0.w};
 #pragma unroll
             for (int ci = 0; ci < C; ++ci) gt[ci] += r[ci];
@@ -1541,6 +1564,7 @@ __global__ void __launch_bounds__(kBlock) gather_point_gradients_kernel(GatherPa
                 gy += (cam.r[1] * e0 + cam.r[4] * e1) + cam.r[7] * e2;
                 gz += (cam.r[2] * e0 + cam.r[5] * e1) + cam.r[8] * e2;
                 cnt += 1.f;
+                view_cnt += 1.f;
                 if (a.camera_partial)
                 {
                     // pose: J_pose^T e with J_pose = [I | -[view_p]x] (tangent = translation, rotation; applied on the
@@ -1569,17 +1593,18 @@ __global__ void __launch_bounds__(kBlock) gather_point_gradients_kernel(GatherPa
 #pragma unroll
         for (int k = 0; k <= kCameraSums; ++k)
         {
-            double v = (k < kSums) ? (double)cam_sum[k < kSums ? k : 0] : (k == kCameraSums ? (double)cnt : 0.0);
+            double v = (k < kSums) ? (double)cam_sum[k < kSums ? k : 0] : (k == kCameraSums ? (double)view_cnt : 0.0);
 #pragma unroll
             for (int d = kWave / 2; d >= 1; d >>= 1) v += __shfl_xor(v, d, kWave);
             if (lane == 0) cam_red[wave][k] = v;
         }
         __syncthreads();
         if (threadIdx.x <= kCameraSums)
-            a.camera_partial[(size_t)blockIdx.x * kCameraRow + threadIdx.x] =
+            a.camera_partial[(size_t)view * a.camera_partial_stride + (size_t)blockIdx.x * kCameraRow + threadIdx.x] =
                 (cam_red[0][threadIdx.x] + cam_red[1][threadIdx.x]) + (cam_red[2][threadIdx.x] + cam_red[3][threadIdx.x]);
+        __syncthreads();  // (the next view of the round uses the array again)
     }
-    const int N = a.vp.N;
+  }
     if (alive && (a.confidence_activation || a.texture_abs))
     {
         const int row = a.vp.index ? a.vp.index[i] : i;
@@ -1656,9 +1681,14 @@ __global__ void __launch_bounds__(kBlock) gather_point_gradients_kernel(GatherPa
             const float s0 = sigmoid_canon(a.confidence_scale * a.vp.confidence[0]);  // (row 0 may not be packed)
             leak_factor    = (a.confidence_scale * s0) * (1.f - s0);
         }
-        sum_background_rows<kBlock>(a.background_rows, a.num_background_rows, C, a.grad_background, a.grad_confidence,
-                                    a.add_leak, a.background_accumulate, a.vp.index != nullptr,
-                                    a.texture_abs ? a.background_raw : nullptr, leak_factor);
+        for (int v = 0; v < view_count; ++v)
+        {
+            sum_background_rows<kBlock>(a.background_rows + (size_t)v * a.background_rows_stride, a.num_background_rows, C,
+                                        a.grad_background, a.grad_confidence, a.add_leak,
+                                        (v > 0 || a.background_accumulate) ? 1 : 0, a.vp.index != nullptr,
+                                        a.texture_abs ? a.background_raw : nullptr, leak_factor);
+            __syncthreads();
+        }
     }
 }
 

@@ -138,9 +138,9 @@ __global__ void __launch_bounds__(kBlock) prepare_views_kernel(PrepareViewsArgs 
     views[first_view + k] = v;
 }
 
-__device__ __forceinline__ bool point_is_skipped(const ViewPass& a, int i)
+// The viewer's confidence cut-off: the same verdict in every view of a call.
+__device__ __forceinline__ bool point_is_skipped_in_all_views(const ViewPass& a, int i)
 {
-    if (a.dropout && a.dropout[i] == 1.f) return true;
     if (a.viewer_only)
     {
         const int ti = a.index ? a.index[i] : i;
@@ -149,6 +149,12 @@ __device__ __forceinline__ bool point_is_skipped(const ViewPass& a, int i)
         if (c < a.stability_cutoff) return true;
     }
     return false;
+}
+
+__device__ __forceinline__ bool point_is_skipped(const ViewPass& a, int i)
+{
+    if (a.dropout && a.dropout[i] == 1.f) return true;  // this view's drop-out mask
+    return point_is_skipped_in_all_views(a, i);
 }
 
 // ---- binning ---------------------------------------------------------------------------------------------------------

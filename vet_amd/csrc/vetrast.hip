@@ -35,6 +35,10 @@ struct vetrast_ctx
     float acc_ms[VETRAST_SCOPE_COUNT_]      = {};
     int32_t acc_launches[VETRAST_SCOPE_COUNT_] = {};
     char* lift_scratch = nullptr;  // this device's copy of the file-scope scratch array (vetrast_lift_error_static)
+    // Calls with several views run them side by side on these streams (default priority), forked from and joined with
+    // the caller's stream by events; see ViewLanes below.
+    hipStream_t lane_stream[kViewLanes] = {nullptr, nullptr, nullptr, nullptr};  // [0] stays unused
+    std::vector<hipEvent_t> sync_events;  // ordering events (no timing), reused from call to call
 };
 
 namespace
@@ -264,6 +268,12 @@ uint32_t log_segment_records(int64_t N, int L, int hits)
 size_t log_records(int64_t N, int L, int hits) { return (size_t)log_segment_records(N, L, hits) * kLogSegments; }
 size_t log_cursor_bytes(int B) { return (size_t)B * kLogSegments * kLogCursorStride * sizeof(uint32_t); }
 
+// Per-workgroup pose / intrinsics rows one view's per-point backward pass leaves.
+size_t camera_rows_bytes(int64_t N)
+{
+    return align_up(((size_t)N + kBlock - 1) / kBlock * kCameraRow * sizeof(double), kAlign);
+}
+
 TileMap make_tile_map(const LayerTable& ly, const double* list_bound = nullptr, bool split_all = false)
 {
     TileMap m;
@@ -436,6 +446,15 @@ int vetrast_create(vetrast_ctx** out_ctx)
         vetrast_destroy(ctx);
         return VETRAST_ERR_HIP;
     }
+    // (lane 0 is the caller's stream: three streams of the context's own, so that a call stays within the four
+    // hardware queues a process has by default)
+    for (int k = 1; k < kViewLanes; ++k)
+        if (hipStreamCreateWithFlags(&ctx->lane_stream[k], hipStreamNonBlocking) != hipSuccess)
+        {
+            ctx->lane_stream[k] = nullptr;
+            vetrast_destroy(ctx);
+            return VETRAST_ERR_HIP;
+        }
     *out_ctx = ctx;
     return VETRAST_OK;
 }
@@ -443,6 +462,9 @@ int vetrast_create(vetrast_ctx** out_ctx)
 void vetrast_destroy(vetrast_ctx* ctx)
 {
     if (!ctx) return;
+    for (auto ls : ctx->lane_stream)
+        if (ls) (void)hipStreamDestroy(ls);
+    for (auto e : ctx->sync_events) (void)hipEventDestroy(e);
     for (auto& s : ctx->spans)
     {
         (void)hipEventDestroy(s.start);
@@ -508,16 +530,22 @@ int vetrast_workspace_layout_for_mode(int32_t N, int32_t B, int32_t L, int32_t w
     at += lay->bin_counts_stride * B;
     lay->log_cursor_base = at;  // right behind the bin counters: one zero-fill covers both
     at += log_cursor_bytes(B);
-    lay->scan_partials_base = at;
-    at += align_up((Tpad / kScanPerBlock) * sizeof(uint32_t), kAlign);
+    // scratch that exists once per lane (views that run side by side), see vetrast_workspace_layout::view_lanes
+    const int lanes            = std::min(B, kViewLanes);
+    lay->view_lanes            = lanes;
+    lay->scan_partials_base    = at;
+    lay->scan_partials_stride  = align_up((Tpad / kScanPerBlock) * sizeof(uint32_t), kAlign);
+    at += lay->scan_partials_stride * lanes;
     lay->offsets_base   = at;
     lay->offsets_stride = align_up((P + 1) * sizeof(uint32_t), kAlign);
     at += lay->offsets_stride * B;
     const size_t record_bytes = compact_records(N, hits) ? sizeof(uint2) : sizeof(uint4);
-    lay->binned_base = at;
-    at += align_up(cap * record_bytes, kAlign);
-    lay->primary_base = at;
-    at += align_up((size_t)t.room_base[L] * record_bytes, kAlign);
+    lay->binned_base   = at;
+    lay->binned_stride = align_up(cap * record_bytes, kAlign);
+    at += lay->binned_stride * lanes;
+    lay->primary_base   = at;
+    lay->primary_stride = align_up((size_t)t.room_base[L] * record_bytes, kAlign);
+    at += lay->primary_stride * lanes;
     lay->views_base = at;
     at += align_up((size_t)B * sizeof(DeviceView), kAlign);
     lay->packed_base = at;
@@ -545,20 +573,25 @@ int vetrast_workspace_layout_for_mode(int32_t N, int32_t B, int32_t L, int32_t w
     at += lay->projected_stride * B;
     // The overflow log (written by the scatter pass, emptied by overflow_move_kernel before the build pass of the same
     // view) is dead once the forward call is over: the scratch of the backward call lies on top of it.
+    // One such block per lane, lane_scratch_stride apart.
     const size_t shared_base = align_up(at, kAlign);
     lay->log_base            = shared_base;
     at                       = shared_base + align_up(log_records(N, L, hits) * sizeof(uint4), kAlign);
     lay->slots_base          = at;
     at += align_up(log_records(N, L, hits) * sizeof(uint32_t), kAlign);
-    lay->forward_only_bytes = align_up(at, kAlign);
-    at                      = shared_base;
-    lay->partial_base       = at;
+    const size_t forward_block = align_up(at, kAlign) - shared_base;
+    at                         = shared_base;
+    lay->partial_base          = at;
     at += align_up(cap * 8 * sizeof(float), kAlign);
     lay->background_partial_base = at;
     // (the FUZZY_BLEND kernel that takes a wave per list keeps rows per replica and kFuzzyFoldRows rows they are folded into)
     at += align_up(((size_t)tile_grid(make_tile_map(t, nullptr, true)) * kFuzzyReplicas + kFuzzyFoldRows) * kBackgroundRow * sizeof(float), kAlign);
-    lay->camera_partial_base = at;
-    at += align_up(((size_t)N + kBlock - 1) / kBlock * kCameraRow * sizeof(double), kAlign);
+    const size_t backward_block = align_up(at, kAlign) - shared_base;
+    lay->lane_scratch_stride    = std::max(forward_block, backward_block);
+    lay->forward_only_bytes     = shared_base + lay->lane_scratch_stride * (lanes - 1) + forward_block;
+    at                          = shared_base + lay->lane_scratch_stride * lanes;
+    lay->camera_partial_base = at;  // (a block of rows per view of a round, see camera_rows_bytes)
+    at += camera_rows_bytes(N) * lanes;
     lay->total_bytes = std::max(align_up(at, kAlign), lay->forward_only_bytes);
     return VETRAST_OK;
 }
@@ -569,6 +602,69 @@ size_t vetrast_forward_workspace_bytes(int32_t N, int32_t B, int32_t L, int32_t 
     if (vetrast_workspace_layout_for(N, B, L, w, h, &lay) != VETRAST_OK) return 0;
     return lay.total_bytes;
 }
+
+namespace
+{
+// The views of one call side by side. View b runs on lane b % lanes: a stream of the context's own that has waited
+// for the caller's stream (fork) and that the caller's stream waits for in the end (join), ordered by events, so the
+// call behaves like one stream's worth of work to the caller and can be captured into a graph with it. Kernels of
+// small views (training crops) leave most of the chip idle on their own and are chains of dependent launches; four of
+// them at a time fill it. With one view everything stays on the caller's stream.
+struct ViewLanes
+{
+    vetrast_ctx* ctx;
+    hipStream_t main;
+    int lanes;
+    size_t used = 0;
+    hipError_t err = hipSuccess;
+
+    ViewLanes(vetrast_ctx* c, hipStream_t m, int n) : ctx(c), main(m), lanes(n > 1 ? n : 1) {}
+    void check(hipError_t e)
+    {
+        if (e != hipSuccess && err == hipSuccess) err = e;
+    }
+    hipEvent_t event()
+    {
+        if (used == ctx->sync_events.size())
+        {
+            hipEvent_t e = nullptr;
+            check(hipEventCreateWithFlags(&e, hipEventDisableTiming));
+            if (!e) return nullptr;
+            ctx->sync_events.push_back(e);
+        }
+        return ctx->sync_events[used++];
+    }
+    // lane 0 is the caller's stream itself: its views need no hand-over, and the call stays within four streams
+    hipStream_t stream(int b) const { return (lanes > 1 && b % lanes != 0) ? ctx->lane_stream[b % lanes] : main; }
+    int lane(int b) const { return lanes > 1 ? b % lanes : 0; }
+    // an event that stands for everything enqueued on `s` so far
+    hipEvent_t mark(hipStream_t s)
+    {
+        hipEvent_t e = event();
+        if (e) check(hipEventRecord(e, s));
+        return e;
+    }
+    void wait(hipStream_t waiter, hipEvent_t e)
+    {
+        if (e) check(hipStreamWaitEvent(waiter, e, 0));
+    }
+    void after(hipStream_t waiter, hipStream_t done)
+    {
+        if (waiter != done) wait(waiter, mark(done));
+    }
+    void fork()
+    {
+        if (lanes < 2) return;
+        hipEvent_t e = mark(main);
+        for (int k = 1; k < lanes; ++k) wait(ctx->lane_stream[k], e);
+    }
+    void join()
+    {
+        if (lanes < 2) return;
+        for (int k = 1; k < lanes; ++k) after(main, ctx->lane_stream[k]);
+    }
+};
+}  // namespace
 
 int vetrast_forward(vetrast_ctx* ctx, const vetrast_forward_args* a, void* stream_)
 {
@@ -589,9 +685,9 @@ int vetrast_forward(vetrast_ctx* ctx, const vetrast_forward_args* a, void* strea
     const bool own_pack  = a->packed_descriptors == nullptr;
     float4* packed       = own_pack ? ws_ptr<float4>(ws, lay.packed_base)
                                     : reinterpret_cast<float4*>(const_cast<float*>(a->packed_descriptors));
-    uint32_t* slots     = ws_ptr<uint32_t>(ws, lay.slots_base);
-    uint32_t* partials  = ws_ptr<uint32_t>(ws, lay.scan_partials_base);
     DeviceView* views   = ws_ptr<DeviceView>(ws, lay.views_base);
+    hipStream_t caller  = stream;
+    ViewLanes lanes(ctx, caller, lay.view_lanes);
 
     {
         ScopeTimer tm(ctx, stream, VETRAST_SCOPE_PREPARE);
@@ -620,19 +716,26 @@ int vetrast_forward(vetrast_ctx* ctx, const vetrast_forward_args* a, void* strea
         }
     }
 
+    lanes.fork();
+    hipEvent_t packed_ready = nullptr;  // the first view's scatter pass has interleaved the descriptors
     for (int b = 0; b < B; ++b)
     {
+        // this view's lane: its stream, its copy of the scratch
+        stream               = lanes.stream(b);
+        const size_t lane    = (size_t)lanes.lane(b);
+        uint32_t* slots      = ws_ptr<uint32_t>(ws, lay.slots_base + lay.lane_scratch_stride * lane);
+        uint32_t* partials   = ws_ptr<uint32_t>(ws, lay.scan_partials_base + lay.scan_partials_stride * lane);
         const ViewPass vp   = make_view_pass(a, lay, ly, b);
         uint32_t* offsets   = ws_ptr<uint32_t>(ws, lay.offsets_base + lay.offsets_stride * b);
         uint64_t* fragments = ws_ptr<uint64_t>(ws, lay.fragments_base + lay.fragments_stride * b);
         float* trans        = ws_ptr<float>(ws, lay.transmittance_base + lay.transmittance_stride * b);
         float* weight       = ws_ptr<float>(ws, lay.weight_base + lay.weight_stride * b);
         uint32_t* bin_counts     = ws_ptr<uint32_t>(ws, lay.bin_counts_base + lay.bin_counts_stride * b);
-        uint4* binned            = ws_ptr<uint4>(ws, lay.binned_base);
+        uint4* binned            = ws_ptr<uint4>(ws, lay.binned_base + lay.binned_stride * lane);
         ScatterTargets targets;
-        targets.primary      = ws_ptr<uint4>(ws, lay.primary_base);
+        targets.primary      = ws_ptr<uint4>(ws, lay.primary_base + lay.primary_stride * lane);
         targets.compact      = compact_records(N, hits) ? 1 : 0;
-        targets.log          = ws_ptr<uint4>(ws, lay.log_base);
+        targets.log          = ws_ptr<uint4>(ws, lay.log_base + lay.lane_scratch_stride * lane);
         targets.log_rank     = slots;
         targets.log_cursor   = ws_ptr<uint32_t>(ws, lay.log_cursor_base) + (size_t)b * kLogSegments * kLogCursorStride;
         targets.segment_capacity = log_segment_records(N, L, hits);
@@ -656,6 +759,7 @@ int vetrast_forward(vetrast_ctx* ctx, const vetrast_forward_args* a, void* strea
             else
                 hipLaunchKernelGGL(bin_scatter_kernel<4>, dim3(grid_for(N)), dim3(kBlock), 0, stream, vp, bin_counts, targets, pack);
         }
+        if (b == 0 && lanes.lanes > 1 && own_pack) packed_ready = lanes.mark(stream);
         // Where the bins of a view are few enough, one launch scans their counts and files the logged records (the
         // scan lands behind the counts); otherwise the scan runs in place and the move kernel follows.
         const bool scan_and_move = bins + 1 <= (uint32_t)kScanMoveMax;
@@ -697,6 +801,8 @@ int vetrast_forward(vetrast_ctx* ctx, const vetrast_forward_args* a, void* strea
             if (p.output_background_mask) out_mask[l] = a->out_mask[l] + (size_t)b * plane;
             if (a->out_weight[l]) out_weight[l] = a->out_weight[l] + (size_t)b * plane;
         }
+        // the build pass reads the descriptor records: the first view of every other lane waits for them
+        if (b > 0 && b < lanes.lanes) lanes.wait(stream, packed_ready);
         {
             ScopeTimer tm(ctx, stream, VETRAST_SCOPE_BUILD);
             BuildPass bp;
@@ -751,6 +857,8 @@ int vetrast_forward(vetrast_ctx* ctx, const vetrast_forward_args* a, void* strea
                 }
         }
     }
+    lanes.join();
+    VET_HIP(ctx, lanes.err);
     VET_HIP(ctx, hipGetLastError());
     return VETRAST_OK;
 }
@@ -843,14 +951,25 @@ int vetrast_backward(vetrast_ctx* ctx, const vetrast_backward_args* g, void* str
     const bool want_camera         = p.need_point_gradient && (g->grad_pose || g->grad_intrinsics) && N > 0;
     const bool want_image_gradient = p.need_point_gradient && (g->grad_points || g->grad_pose || g->grad_intrinsics);
     double* camera_rows            = ws_ptr<double>(ws, lay.camera_partial_base);
-    float4* partial        = ws_ptr<float4>(ws, lay.partial_base);
-    float* background_rows = ws_ptr<float>(ws, lay.background_partial_base);
     const bool fuzzy_long  = p.render_mode == VETRAST_RENDER_FUZZY_BLEND &&
                             (p.debug_max_list_length <= 0 || p.debug_max_list_length > kFuzzyDense);
-    for (int b = 0; b < B; ++b)
-    {
+    // The per-pixel kernels of up to view_lanes views run side by side, each into its lane's record array; the
+    // per-point kernels add to the same gradient rows, so they stay on the caller's stream, one view after the other,
+    // each behind its view's per-pixel kernel; a lane's next per-pixel kernel waits for the per-point kernel that
+    // reads what the last one left.
+    hipStream_t caller = stream;
+    ViewLanes lanes(ctx, caller, lay.view_lanes);
+    lanes.fork();
+    std::vector<hipEvent_t> gathered((size_t)B, nullptr);
+    // the per-pixel part of view b, on its lane
+    auto per_pixel = [&](int b) {
+        const size_t lane      = (size_t)lanes.lane(b);
+        float4* partial        = ws_ptr<float4>(ws, lay.partial_base + lay.lane_scratch_stride * lane);
+        float* background_rows = ws_ptr<float>(ws, lay.background_partial_base + lay.lane_scratch_stride * lane);
         uint32_t* offsets   = ws_ptr<uint32_t>(ws, lay.offsets_base + lay.offsets_stride * b);
         uint64_t* fragments = ws_ptr<uint64_t>(ws, lay.fragments_base + lay.fragments_stride * b);
+        stream = lanes.stream(b);
+        if (lanes.lanes > 1 && b >= lanes.lanes) lanes.wait(stream, gathered[(size_t)(b - lanes.lanes)]);
         {
             ScopeTimer tm(ctx, stream, VETRAST_SCOPE_BACKWARD_BLEND);
             BackwardPass bp;
@@ -933,6 +1052,18 @@ int vetrast_backward(vetrast_ctx* ctx, const vetrast_backward_args* g, void* str
                     default: hipLaunchKernelGGL((blend_backward_kernel<4, true>), grid, blk, 0, stream, bp); break;
                 }
         }
+    };
+    // the per-point part of the views [b, last) of a round: one launch on the caller's stream, behind the round's
+    // per-pixel kernels
+    auto per_point = [&](int b, int last) {
+        const size_t lane      = (size_t)lanes.lane(b);
+        float4* partial        = ws_ptr<float4>(ws, lay.partial_base + lay.lane_scratch_stride * lane);
+        float* background_rows = ws_ptr<float>(ws, lay.background_partial_base + lay.lane_scratch_stride * lane);
+        uint32_t* offsets   = ws_ptr<uint32_t>(ws, lay.offsets_base + lay.offsets_stride * b);
+        uint64_t* fragments = ws_ptr<uint64_t>(ws, lay.fragments_base + lay.fragments_stride * b);
+        (void)offsets, (void)fragments;
+        for (int v = b; v < last; ++v) lanes.after(caller, lanes.stream(v));
+        stream = caller;
         if (N > 0)
         {
             ScopeTimer tm(ctx, stream, VETRAST_SCOPE_BACKWARD_GATHER);
@@ -951,6 +1082,14 @@ int vetrast_backward(vetrast_ctx* ctx, const vetrast_backward_args* g, void* str
             gp.K                   = p.debug_max_list_length;
             gp.need_point_gradient = want_image_gradient ? 1 : 0;
             gp.camera_partial      = want_camera ? camera_rows : nullptr;
+            gp.view_count          = last - b;
+            gp.dropout_stride      = (size_t)N;
+            gp.flags_stride        = lay.cut_flags_stride;
+            gp.last_key_stride     = lay.last_key_stride / sizeof(uint64_t);
+            gp.kept_stride         = lay.kept_stride / sizeof(uint32_t);
+            gp.partial_stride      = lay.lane_scratch_stride / sizeof(float4);
+            gp.background_rows_stride = lay.lane_scratch_stride / sizeof(float);
+            gp.camera_partial_stride  = camera_rows_bytes(N) / sizeof(double);
             gp.accumulate          = (add_to_rows || b > 0) ? 1 : 0;
             gp.background_rows       = background_rows;
             // (with the folded rows of the FUZZY_BLEND kernel that takes a wave per list, where it ran)
@@ -972,7 +1111,14 @@ int vetrast_backward(vetrast_ctx* ctx, const vetrast_backward_args* g, void* str
             // cameras with distortion switched on take the variant that carries the distortion Jacobians
             auto launch = [&](auto c_tag, auto hits_tag) {
                 constexpr int kC = decltype(c_tag)::value, kHits = decltype(hits_tag)::value;
-                if (p.allow_distortion)
+                if (gp.view_count > 1)
+                {
+                    if (p.allow_distortion)
+                        hipLaunchKernelGGL((gather_point_gradients_kernel<kC, kHits, true, true>), grid, blk, 0, stream, gp);
+                    else
+                        hipLaunchKernelGGL((gather_point_gradients_kernel<kC, kHits, false, true>), grid, blk, 0, stream, gp);
+                }
+                else if (p.allow_distortion)
                     hipLaunchKernelGGL((gather_point_gradients_kernel<kC, kHits, true>), grid, blk, 0, stream, gp);
                 else
                     hipLaunchKernelGGL((gather_point_gradients_kernel<kC, kHits, false>), grid, blk, 0, stream, gp);
@@ -991,22 +1137,41 @@ int vetrast_backward(vetrast_ctx* ctx, const vetrast_backward_args* g, void* str
             else
                 with_channels(std::integral_constant<int, 4>{});
         }
-        if (want_camera)
+        for (int v = b; want_camera && v < last; ++v)
         {
             ScopeTimer tm(ctx, stream, VETRAST_SCOPE_BACKWARD_GATHER);
-            hipLaunchKernelGGL(reduce_camera_kernel, dim3(1), dim3(kBlock), 0, stream, camera_rows, grid_for(N),
-                               a->views[b].image_index, a->views[b].camera_index, p.K_gradient_factor, g->grad_pose,
+            hipLaunchKernelGGL(reduce_camera_kernel, dim3(1), dim3(kBlock), 0, stream,
+                               camera_rows + (size_t)(v - b) * (camera_rows_bytes(N) / sizeof(double)), grid_for(N),
+                               a->views[v].image_index, a->views[v].camera_index, p.K_gradient_factor, g->grad_pose,
                                g->grad_pose_count, g->grad_intrinsics, g->grad_intrinsics_count,
                                hits == 1 ? 1.f / 1024.f : 1.f, p.allow_distortion, p.distortion_gradient_factor);
         }
-        if (N == 0)
+        for (int v = b; N == 0 && v < last; ++v)
         {
             ScopeTimer tm(ctx, stream, VETRAST_SCOPE_BACKWARD_GATHER);
-            hipLaunchKernelGGL(reduce_background_kernel, dim3(1), dim3(kReduceBlock), 0, stream, background_rows,
+            hipLaunchKernelGGL(reduce_background_kernel, dim3(1), dim3(kReduceBlock), 0, stream,
+                               background_rows + (size_t)(v - b) * (lay.lane_scratch_stride / sizeof(float)),
                                (int)(tile_grid(tiles)) + (fuzzy_long ? kFuzzyFoldRows : 0), C, g->grad_background, g->grad_confidence,
-                               0, b > 0 ? 1 : 0, p.texture_abs ? a->background : nullptr);
+                               0, v > 0 ? 1 : 0, p.texture_abs ? a->background : nullptr);
         }
+        if (lanes.lanes > 1 && last < B)
+        {
+            // the next round's per-pixel kernels overwrite the lanes' record arrays
+            const hipEvent_t e = lanes.mark(caller);
+            for (int v = b; v < last; ++v) gathered[(size_t)v] = e;
+        }
+    };
+    // Views in rounds of one per lane: first the per-pixel kernels of the round (side by side), then its per-point
+    // kernels. (Enqueued in this order, no per-pixel kernel waits in a hardware queue behind a per-point kernel of
+    // another view.)
+    for (int first = 0; first < B; first += lanes.lanes)
+    {
+        const int last = std::min(B, first + lanes.lanes);
+        for (int b = first; b < last; ++b) per_pixel(b);
+        per_point(first, last);
     }
+    stream = caller;  // (every lane's last kernel has been waited for above)
+    VET_HIP(ctx, lanes.err);
     if (g->grad_points && p.point_gradient_normalization != 0 && N > 0)
     {
         ScopeTimer tm(ctx, stream, VETRAST_SCOPE_BACKWARD_POST);
