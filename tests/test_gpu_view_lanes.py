@@ -66,6 +66,37 @@ def test_many_views_match_the_oracle(render_mode, num_views, rasterizer, oracle)
     assert np.abs(want["pose"]).sum() > 0 and got["pose_count"].cpu().numpy().min() > 0
 
 
+@pytest.mark.parametrize("render_mode", MODES)
+@pytest.mark.parametrize("num_views", [1, 3, 6])
+def test_hints_that_switch_the_record_layout_change_nothing(render_mode, num_views, rasterizer, oracle):
+    """Where the caller expects its views to see a small part of the cloud (vetrast_params.expected_fragments), the
+    backward pass keeps a point's gradient records next to each other instead of layer after layer. The same call
+    without hints, with hints that say "most of the cloud" and with hints that say "next to nothing" (which also makes
+    the bins overflow): images the same bits, gradients against the oracle and against each other."""
+    scene = _scene(num_views, 60 + num_views)
+    go = scene.grad_out()
+    results = []
+    for hint in (0.0, 0.9 * scene.num_points, 25.0):
+        params = make_params(scene, need_point_gradient=1, render_mode=render_mode, depth_accept_blend=0.05)
+        for l in range(scene.num_layers):
+            params.expected_fragments[l] = hint
+        res = rasterizer.forward(DeviceScene(scene), params)
+        got = rasterizer.backward(res, [torch.from_numpy(g).cuda() for g in go], want_cameras=True)
+        torch.cuda.synchronize()
+        results.append((res, got, params))
+    ref = oracle.forward(scene, results[0][2])
+    want = oracle.backward(ref, go, want_cameras=True)
+    for res, got, _ in results:
+        for l in range(scene.num_layers):
+            np.testing.assert_array_equal(res.out[l].cpu().numpy(), ref.out[l])
+        for key in ("texture", "confidence", "background", "points", "pose", "intrinsics"):
+            err = max_rel_err(got[key].cpu().numpy(), want[key])
+            assert err <= (3e-4 if key in ("pose", "intrinsics") else 1e-4), (key, err)
+    # one record per fragment whatever the layout: the per-point sums are the same additions in the same order
+    for key in ("texture", "confidence", "points", "point_count"):
+        assert torch.equal(results[0][1][key], results[2][1][key]), key
+
+
 def test_a_call_of_many_views_equals_its_views_one_by_one(rasterizer):
     """Seven views in one call against seven calls of one view: images and lists bit for bit, and the gradients of the
     big call equal the sum of the single calls' gradients to rounding (the rows are added in view order either way)."""

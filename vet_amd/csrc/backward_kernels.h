@@ -43,7 +43,8 @@ struct BackwardPass
     const float* background;
     const float* grad_out[VETRAST_MAX_LAYERS];  // already offset to this view
     const float* out[VETRAST_MAX_LAYERS];       // forward result, already offset to this view
-    float4* partial;          // [L][hits][N] records of 2 float4: (d tex0..3), (d conf, d image x, d image y, 0)
+    float4* partial;          // records of 2 float4: (d tex0..3), (d conf, d image x, d image y, 0), at gradient_record
+    int point_major_records;  // layout of the record array, see gradient_record
     float* background_partial;  // [workgroups][8]: per-workgroup sums of d background[0..C) and of the leak term
     LayerTable ly;
     TileMap tiles;
@@ -200,7 +201,7 @@ __global__ void __launch_bounds__(kBlock) blend_backward_kernel(BackwardPass a)
     uint32_t max_n = n;
 #pragma unroll
     for (int d = kWave / 2; d >= 1; d >>= 1) max_n = max(max_n, (uint32_t)__shfl_xor((int)max_n, d, kWave));
-    float4* partial_l = a.partial + 2 * (size_t)l * (BILINEAR ? 4 : 1) * a.N;
+    float4* partial_l = a.partial;  // (records are addressed by gradient_record)
     // Windows run from the deepest list places to the nearest. Where only a few pixels of the wave still have fragments
     // that deep (uncut lists of hundreds of fragments at a handful of pixels), a window of 16 places would fill a
     // quarter of the lanes or less and every window costs a dependent chain of memory round trips, so the window is
@@ -337,7 +338,7 @@ __global__ void __launch_bounds__(kBlock) blend_backward_kernel(BackwardPass a)
                 // Record stores, two lanes per record: first the even lane's record (even lane its low half, odd lane
                 // the high half), then the odd lane's, so that each instruction issues one 32-byte request per record.
                 const int odd        = lane & 1;
-                const int own        = ti >= 0 ? (BILINEAR ? corner * a.N + id : id) : -1;
+                const int own        = ti >= 0 ? (int)gradient_record(a.point_major_records, a.N, a.ly.L, BILINEAR ? 4 : 1, l, corner, id) : -1;
                 const int other      = pair_other(own);
                 const float4 o_lo    = pair_other(rec_lo);
                 const float4 o_hi    = pair_other(rec_hi);
@@ -345,7 +346,7 @@ __global__ void __launch_bounds__(kBlock) blend_backward_kernel(BackwardPass a)
                 const int id_second  = odd ? own : other;
                 const float4 v_first = odd ? o_hi : rec_lo;
                 const float4 v_second = odd ? rec_hi : o_lo;
-                // own/other are record numbers: the point id, in BILINEAR_BLEND behind the corner's block of N records
+                // own/other are record numbers
                 if (id_first >= 0) partial_l[2 * (size_t)id_first + odd] = v_first;
                 if (id_second >= 0) partial_l[2 * (size_t)id_second + odd] = v_second;
             }
@@ -493,7 +494,7 @@ __global__ void __launch_bounds__(kBlock) blend_backward_fuzzy_kernel(BackwardPa
     clear_small_accumulators(a.clear);
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
     const TilePixel px = tile_pixel(a.tiles, a.ly);
-    float4* partial_l  = a.partial + 2 * (size_t)px.l * a.N;
+    float4* partial_l  = a.partial;  // (records are addressed by gradient_record)
     const bool with_background = !a.use_environment_map;  // every list ends with the background element
     float bg_grad[C];
 #pragma unroll
@@ -706,7 +707,7 @@ __global__ void __launch_bounds__(kBlock) blend_backward_fuzzy_kernel(BackwardPa
         {
             // record stores, two lanes per record (see blend_backward_kernel)
             const int odd         = lane & 1;
-            const int own         = give ? id : -1;
+            const int own         = give ? (int)gradient_record(a.point_major_records, a.N, a.ly.L, 1, px.l, 0, id) : -1;
             const int other       = pair_other(own);
             const float4 o_lo     = pair_other(rec_lo);
             const float4 o_hi     = pair_other(rec_hi);
@@ -883,7 +884,7 @@ __global__ void __launch_bounds__(kBlock) blend_backward_fuzzy_kernel(BackwardPa
         {
             // record stores, two lanes per record (see blend_backward_kernel)
             const int odd         = lane & 1;
-            const int own         = give ? id : -1;
+            const int own         = give ? (int)gradient_record(a.point_major_records, a.N, a.ly.L, 1, px.l, 0, id) : -1;
             const int other       = pair_other(own);
             const float4 o_lo     = pair_other(rec_lo);
             const float4 o_hi     = pair_other(rec_hi);
@@ -980,7 +981,7 @@ __global__ void __launch_bounds__(kBlock) blend_backward_fuzzy_long_kernel(Backw
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
     const TilePixel px = tile_pixel(a.tiles, a.ly);
     const FuzzyPixel f = fuzzy_pixel<C>(a, px);
-    float4* partial_l  = a.partial + 2 * (size_t)px.l * a.N;  // the layer is the same for the whole workgroup
+    float4* partial_l  = a.partial;  // (records are addressed by gradient_record)
     const bool with_background = !a.use_environment_map;
     float bg_grad[C];  // summed over the wave at the end: every lane adds what it computes for lane 0's sake once
 #pragma unroll
@@ -1084,8 +1085,8 @@ __global__ void __launch_bounds__(kBlock) blend_backward_fuzzy_long_kernel(Backw
                             int ti          = -1;
                             if ((uint32_t)point < (uint32_t)a.N) ti = a.index ? a.index[point] : point;
                             if ((uint32_t)ti >= (uint32_t)a.N) continue;
-                            partial_l[2 * (size_t)point] = make_float4(gt[0], gt[1], gt[2], gt[3]);
-                            reinterpret_cast<float*>(&partial_l[2 * (size_t)point + 1])[0] = gconf;
+                            partial_l[2 * gradient_record(a.point_major_records, a.N, a.ly.L, 1, px.l, 0, point)] = make_float4(gt[0], gt[1], gt[2], gt[3]);
+                            reinterpret_cast<float*>(&partial_l[2 * gradient_record(a.point_major_records, a.N, a.ly.L, 1, px.l, 0, point) + 1])[0] = gconf;
                         }
                     }
                     A_front = (1.f - bconf) * A_front;
@@ -1204,13 +1205,13 @@ __global__ void __launch_bounds__(kBlock) blend_backward_fuzzy_long_kernel(Backw
                     {
                         if (closes)
                         {
-                            partial_l[2 * (size_t)id]     = make_float4(gt[0], gt[1], gt[2], gt[3]);
-                            partial_l[2 * (size_t)id + 1] = make_float4(gconf, gp0, gp1, 0.f);
+                            partial_l[2 * gradient_record(a.point_major_records, a.N, a.ly.L, 1, px.l, 0, id)]     = make_float4(gt[0], gt[1], gt[2], gt[3]);
+                            partial_l[2 * gradient_record(a.point_major_records, a.N, a.ly.L, 1, px.l, 0, id) + 1] = make_float4(gconf, gp0, gp1, 0.f);
                         }
                         else
                         {
                             // the bucket stays open: its part of the record follows when it closes
-                            float* rec = reinterpret_cast<float*>(&partial_l[2 * (size_t)id + 1]);
+                            float* rec = reinterpret_cast<float*>(&partial_l[2 * gradient_record(a.point_major_records, a.N, a.ly.L, 1, px.l, 0, id) + 1]);
                             rec[1] = gp0, rec[2] = gp1, rec[3] = 0.f;
                         }
                     }
@@ -1228,8 +1229,8 @@ __global__ void __launch_bounds__(kBlock) blend_backward_fuzzy_long_kernel(Backw
                             int ti          = -1;
                             if ((uint32_t)point < (uint32_t)a.N) ti = a.index ? a.index[point] : point;
                             if ((uint32_t)ti >= (uint32_t)a.N) continue;
-                            partial_l[2 * (size_t)point] = make_float4(gt0[0], gt0[1], gt0[2], gt0[3]);
-                            reinterpret_cast<float*>(&partial_l[2 * (size_t)point + 1])[0] = gconf0;
+                            partial_l[2 * gradient_record(a.point_major_records, a.N, a.ly.L, 1, px.l, 0, point)] = make_float4(gt0[0], gt0[1], gt0[2], gt0[3]);
+                            reinterpret_cast<float*>(&partial_l[2 * gradient_record(a.point_major_records, a.N, a.ly.L, 1, px.l, 0, point) + 1])[0] = gconf0;
                         }
                     }
                     if (last_step && with_background && lane == (int)valid - 1)
@@ -1417,6 +1418,7 @@ struct GatherPass
     // v of the round lies v * the stride behind them (per-view arrays of the workspace; the record and background-row
     // arrays of the view's lane; a camera-row block per view). A point's position is read once for all of them and its
     // gradient rows are written once.
+    int point_major_records;  // layout of the record array, see gradient_record
     int view_count;
     size_t dropout_stride, flags_stride, last_key_stride, kept_stride;  // elements of the respective arrays
     size_t partial_stride, background_rows_stride, camera_partial_stride;
@@ -1519,7 +1521,7 @@ __global__ void __launch_bounds__(kBlock) gather_point_gradients_kernel(GatherPa
                 const uint64_t key = depth_key | (HITS == 1 ? (uint32_t)i : (((uint32_t)i << 2) | (uint32_t)h));
                 if (key > last_key[q]) continue;  // 0 where no fragment was blended: every key is beyond it
             }
-            const size_t rec = (size_t)(l * HITS + h) * a.vp.N + i;
+            const size_t rec = gradient_record(a.point_major_records, a.vp.N, ly.L, HITS, l, h, i);
             const float4 r0  = partial[2 * rec];
             const float4 r1  = partial[2 * rec + 1];
             const float r[4] = {r0.x, r0.y, r0.z, r0.w};

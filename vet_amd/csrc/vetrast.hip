@@ -953,6 +953,20 @@ int vetrast_backward(vetrast_ctx* ctx, const vetrast_backward_args* g, void* str
     double* camera_rows            = ws_ptr<double>(ws, lay.camera_partial_base);
     const bool fuzzy_long  = p.render_mode == VETRAST_RENDER_FUZZY_BLEND &&
                             (p.debug_max_list_length <= 0 || p.debug_max_list_length > kFuzzyDense);
+    // Layout of the gradient records (gradient_record): point after point where the caller expects the views to see a
+    // small part of the cloud (a third of the fragments every point in every layer would leave, or less), layer after
+    // layer otherwise and where nothing is known.
+    int point_major_records = 0;
+    {
+        double expected = 0.0;
+        bool known      = true;
+        for (int l = 0; l < L; ++l)
+        {
+            known = known && p.expected_fragments[l] > 0.f;
+            expected += p.expected_fragments[l];
+        }
+        point_major_records = (known && expected < (double)N * hits * L / 3.0) ? 1 : 0;
+    }
     // The per-pixel kernels of up to view_lanes views run side by side, each into its lane's record array; the
     // per-point kernels add to the same gradient rows, so they stay on the caller's stream, one view after the other,
     // each behind its view's per-pixel kernel; a lane's next per-pixel kernel waits for the per-point kernel that
@@ -984,6 +998,7 @@ int vetrast_backward(vetrast_ctx* ctx, const vetrast_backward_args* g, void* str
                                                         : ws_ptr<float4>(ws, lay.packed_base);
             bp.background       = ws_ptr<const float>(ws, lay.flags_base) + kPreparedBackgroundOffset;
             bp.partial          = partial;
+            bp.point_major_records = point_major_records;
             bp.background_partial = background_rows;
             bp.ly               = ly;
             bp.tiles            = tiles;
@@ -1082,6 +1097,7 @@ int vetrast_backward(vetrast_ctx* ctx, const vetrast_backward_args* g, void* str
             gp.K                   = p.debug_max_list_length;
             gp.need_point_gradient = want_image_gradient ? 1 : 0;
             gp.camera_partial      = want_camera ? camera_rows : nullptr;
+            gp.point_major_records = point_major_records;
             gp.view_count          = last - b;
             gp.dropout_stride      = (size_t)N;
             gp.flags_stride        = lay.cut_flags_stride;
