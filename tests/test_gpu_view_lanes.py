@@ -142,7 +142,9 @@ def test_a_call_of_several_rounds_replays_from_a_hip_graph(render_mode, rasteriz
     torch.cuda.synchronize()
     want_out = [o.clone() for o in eager.out]
     want_g = {k: v.clone() for k, v in eager_g.items() if k != "_args"}
-    lib, ctx = rasterizer.lib, rasterizer.ctx
+    # a context whose very first calls are the captured ones (it must not have to create anything while it is captured)
+    fresh = Rasterizer()
+    lib, ctx = fresh.lib, fresh.ctx
     side = torch.cuda.Stream()
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.stream(side):

@@ -455,6 +455,18 @@ int vetrast_create(vetrast_ctx** out_ctx)
             vetrast_destroy(ctx);
             return VETRAST_ERR_HIP;
         }
+    // ordering events for calls with several views, made here so that a call that is being captured into a graph
+    // creates nothing (a call of up to some forty views gets by with these; more are made when needed)
+    for (int k = 0; k < 64; ++k)
+    {
+        hipEvent_t ev = nullptr;
+        if (hipEventCreateWithFlags(&ev, hipEventDisableTiming) != hipSuccess)
+        {
+            vetrast_destroy(ctx);
+            return VETRAST_ERR_HIP;
+        }
+        ctx->sync_events.push_back(ev);
+    }
     *out_ctx = ctx;
     return VETRAST_OK;
 }
