@@ -286,10 +286,10 @@ def time_fused_steps(scene, render_mode, steps, samples):
             "adam_frac_of_hbm_peak": round(adam_bytes / 1e6 / ms_adam / HBM_PEAK_GBS, 4)}
 
 
-def time_shim_path(scene, render_mode, steps, samples):
+def time_shim_path(scene, render_mode, steps, samples, **overrides):
     """The same frame through the libtorch shim as a trainer calls it: BlendPointCloud with train = true, then
     autograd's backward with the upstream gradients; workspace and output allocation, the autograd graph and the
-    gradient tensors torch allocates are all inside the timed region."""
+    gradient tensors torch allocates are all inside the timed region. `overrides`: RenderParams members by name."""
     import torch
 
     from vet_amd import torch_ops
@@ -308,12 +308,15 @@ def time_shim_path(scene, render_mode, steps, samples):
     def step():
         for t in leaves:
             t.grad = None
+        kw = dict(train=True, use_environment_map=0, need_point_gradient=1, drop_out_points_by_radius=0,
+                  debug_max_list_length=scene.max_list_length, render_mode=render_mode)
+        kw.update(overrides)
         outs = torch_ops.blend_point_cloud(texture, background, points, tangents, intrinsics, confidence, poses, index,
-                                           views, scene.num_layers, train=True, use_environment_map=0,
-                                           need_point_gradient=1, drop_out_points_by_radius=0,
-                                           debug_max_list_length=scene.max_list_length, render_mode=render_mode)
+                                           views, scene.num_layers, **kw)
         torch.autograd.backward(outs[:scene.num_layers], grads)
 
+    for _ in range(40):  # (the cache reads the fragment counts of a call back every 16th call and sizes bins from them)
+        step()
     t = timed_samples(step, 3, steps, samples)
     _, ws_bytes = torch_ops.train_workspace_info()
     return {"ms_per_step": round(t["median"], 5), "p10": round(t["p10"], 5), "p90": round(t["p90"], 5),
@@ -406,6 +409,11 @@ def time_training_crops(steps, samples, render_mode):
         out["fragments_per_layer_of_view_0"] = counts
         hint = [float(c) for c in counts] + [0.0] * (5 - len(counts))
         del fwd, bargs
+    del dev
+    torch.cuda.empty_cache()
+    # the same batch as a trainer issues it: through the libtorch shim, which sizes the bins from its own history
+    out["ms_per_batch_through_the_shim"] = time_shim_path(scene, render_mode, steps, samples, drop_out_points_by_radius=1,
+                                                          debug_max_list_length=-1)["ms_per_step"]
     return out
 
 

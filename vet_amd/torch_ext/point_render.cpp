@@ -891,7 +891,9 @@ const torch::Tensor& PointRendererCache::PointOrderFor(const torch::Tensor& poin
             const torch::Tensor xyz = points.detach().narrow(1, 0, 3);
             const double as_is      = extent(xyz);
             const double ordered    = extent(xyz.index_select(0, point_order.to(torch::kInt64)));
-            point_order_in_use      = ordered < 0.8 * as_is;
+            // (blocks whose points VET has sorted by radius come out at 0.5 to 0.6 and are faster as they are; a
+            // cloud with a fifth of its points appended unsorted at 0.22, the generator's order at 0.33)
+            point_order_in_use      = ordered < 0.4 * as_is;
         }
     }
     ++point_order_age_;
