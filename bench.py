@@ -453,7 +453,7 @@ def main():
                     help="0 = every core this process may use, within the box's worker limit (OMP_NUM_THREADS)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
-        print("bench.py: this build runs the rasterizer on ONE GPU (views of a batch are rendered back to back); "
+        print("bench.py: this build runs the rasterizer on ONE GPU (the views of a batch share it); "
               "--gpus N with N > 1 is not available", file=sys.stderr)
         sys.exit(2)
 
