@@ -104,7 +104,7 @@ constexpr int kWaveItems  = kWave * kWindow;    // item table of a wave
 // 2 away from the border only, d conf_j = weight_j * d alpha_j and the position gradient is the analytic
 // d weight_j / d position * confidence_j * d alpha_j. A record goes to partial[layer][corner][point].
 template <int C, bool BILINEAR>
-__global__ void __launch_bounds__(kBlock) blend_backward_kernel(BackwardPass a)
+__device__ __forceinline__ void blend_backward(const BackwardPass& a)
 {
     constexpr int kWaves = kBlock / kWave;
     __shared__ uint32_t s_off[kWaves][kWave];
@@ -375,6 +375,18 @@ __global__ void __launch_bounds__(kBlock) blend_backward_kernel(BackwardPass a)
             (red[0][threadIdx.x] + red[1][threadIdx.x]) + (red[2][threadIdx.x] + red[3][threadIdx.x]);
 }
 
+template <int C, bool BILINEAR>
+__global__ void __launch_bounds__(kBlock) blend_backward_kernel(BackwardPass a)
+{
+    blend_backward<C, BILINEAR>(a);
+}
+
+template <int C, bool BILINEAR>
+__global__ void __launch_bounds__(kBlock) blend_backward_views_kernel(PerView<BackwardPass> views)
+{
+    blend_backward<C, BILINEAR>(views.v[blockIdx.y]);
+}
+
 // FUZZY_BLEND, per-pixel part of the backward pass: BlendBackwardsFuzzy<C>, src/lib/rendering/RenderBackward.cu:570-1080.
 // Fragments are collected into a bucket while their depth stays within depth_accept of the bucket's first one (every
 // bucket, unlike the forward kernel, which only averages the nearest one); the background, at depth 1e5, ends up in a
@@ -478,7 +490,7 @@ constexpr int kFuzzyReplicas   = 4;
 constexpr int kFuzzyFoldRows   = 256;
 
 template <int C, int DENSE>
-__global__ void __launch_bounds__(kBlock) blend_backward_fuzzy_kernel(BackwardPass a, float depth_accept)
+__device__ __forceinline__ void blend_backward_fuzzy(const BackwardPass& a, float depth_accept)
 {
     constexpr int kWaves = kBlock / kWave;
     __shared__ uint32_t s_off[kWaves][kWave];
@@ -952,6 +964,18 @@ __global__ void __launch_bounds__(kBlock) blend_backward_fuzzy_kernel(BackwardPa
         row[kFuzzyLongColumn] = (red[0][C + 1] + red[1][C + 1]) + (red[2][C + 1] + red[3][C + 1]);
 }
 
+template <int C, int DENSE>
+__global__ void __launch_bounds__(kBlock) blend_backward_fuzzy_kernel(BackwardPass a, float depth_accept)
+{
+    blend_backward_fuzzy<C, DENSE>(a, depth_accept);
+}
+
+template <int C, int DENSE>
+__global__ void __launch_bounds__(kBlock) blend_backward_fuzzy_views_kernel(PerView<BackwardPass> views, float depth_accept)
+{
+    blend_backward_fuzzy<C, DENSE>(views.v[blockIdx.y], depth_accept);
+}
+
 // The lists blend_backward_fuzzy_kernel left out (more than `dense_max` fragments), one after the other, each by the
 // whole wave: 64 consecutive fragments per step, front to back, one lane per fragment. The bucket boundaries of a step
 // are found by a loop over its buckets that every lane runs alike (the rule is sequential, but it needs the depths
@@ -965,7 +989,7 @@ __global__ void __launch_bounds__(kBlock) blend_backward_fuzzy_kernel(BackwardPa
 // still open at the end of their step get the position part of their record there and the bucket's part when it
 // closes, from a loop over their keys. Same grid as the dense kernel; a workgroup without such a list leaves at once.
 template <int C>
-__global__ void __launch_bounds__(kBlock) blend_backward_fuzzy_long_kernel(BackwardPass a, float depth_accept, uint32_t dense_max)
+__device__ __forceinline__ void blend_backward_fuzzy_long(const BackwardPass& a, float depth_accept, uint32_t dense_max)
 {
     constexpr int kWaves = kBlock / kWave;
     __shared__ float red[kWaves][C];
@@ -1290,10 +1314,23 @@ __global__ void __launch_bounds__(kBlock) blend_backward_fuzzy_long_kernel(Backw
     }
 }
 
+template <int C>
+__global__ void __launch_bounds__(kBlock) blend_backward_fuzzy_long_kernel(BackwardPass a, float depth_accept, uint32_t dense_max)
+{
+    blend_backward_fuzzy_long<C>(a, depth_accept, dense_max);
+}
+
+// (blockIdx.y is the replica here)
+template <int C>
+__global__ void __launch_bounds__(kBlock) blend_backward_fuzzy_long_views_kernel(PerView<BackwardPass> views, float depth_accept,
+                                                                                 uint32_t dense_max)
+{
+    blend_backward_fuzzy_long<C>(views.v[blockIdx.z], depth_accept, dense_max);
+}
+
 // Adds `num_rows` rows of kBackgroundRow floats up into kFuzzyFoldRows rows: workgroup j takes rows j, j + 256, ... in a
 // fixed order (32 threads per column, each every 32nd of the workgroup's rows, then the 32 partial sums one after the other).
-__global__ void __launch_bounds__(kBlock) fold_background_rows_kernel(const float* __restrict__ rows, int num_rows,
-                                                                      float* __restrict__ folded)
+__device__ __forceinline__ void fold_background_rows(const float* __restrict__ rows, int num_rows, float* __restrict__ folded)
 {
     __shared__ float part[kBlock / kBackgroundRow][kBackgroundRow];
     const int column = threadIdx.x % kBackgroundRow, sub = threadIdx.x / kBackgroundRow;
@@ -1308,6 +1345,25 @@ __global__ void __launch_bounds__(kBlock) fold_background_rows_kernel(const floa
         for (int k = 0; k < kBlock / kBackgroundRow; ++k) total += part[k][threadIdx.x];
         folded[(size_t)blockIdx.x * kBackgroundRow + threadIdx.x] = total;
     }
+}
+
+__global__ void __launch_bounds__(kBlock) fold_background_rows_kernel(const float* __restrict__ rows, int num_rows,
+                                                                      float* __restrict__ folded)
+{
+    fold_background_rows(rows, num_rows, folded);
+}
+
+struct FoldArgs
+{
+    const float* rows;
+    int num_rows;
+    float* folded;
+};
+
+__global__ void __launch_bounds__(kBlock) fold_background_rows_views_kernel(PerView<FoldArgs> views)
+{
+    const FoldArgs& v = views.v[blockIdx.y];
+    fold_background_rows(v.rows, v.num_rows, v.folded);
 }
 
 // Sums the per-workgroup background rows of one view (one workgroup, fixed order, so the result is reproducible) and

@@ -184,8 +184,8 @@ __device__ __forceinline__ void block_sort_in_lds(uint64_t* list, uint32_t n, ui
     __syncthreads();
 }
 
-template <int C, bool BILINEAR, bool FUZZY = false>
-__global__ void __launch_bounds__(kBlock) bin_build_kernel(BuildPass a)
+template <int C, bool BILINEAR, bool FUZZY>
+__device__ __forceinline__ void bin_build(const BuildPass& a)
 {
     static_assert(!(BILINEAR && FUZZY), "one blend rule at a time");
     __shared__ uint32_t s_cnt[kTilePixels];
@@ -626,6 +626,18 @@ __global__ void __launch_bounds__(kBlock) bin_build_kernel(BuildPass a)
             if (a.out_weight[l]) a.out_weight[l][local] = T;
         }
     }
+}
+
+template <int C, bool BILINEAR, bool FUZZY = false>
+__global__ void __launch_bounds__(kBlock) bin_build_kernel(BuildPass a)
+{
+    bin_build<C, BILINEAR, FUZZY>(a);
+}
+
+template <int C, bool BILINEAR, bool FUZZY = false>
+__global__ void __launch_bounds__(kBlock) bin_build_views_kernel(PerView<BuildPass> views)
+{
+    bin_build<C, BILINEAR, FUZZY>(views.v[blockIdx.y]);
 }
 
 }  // namespace vetrast

@@ -18,7 +18,7 @@ constexpr int kPreparedBackgroundOffset = 16;  // float index inside the flags b
 constexpr int kPackedFloats   = 8;            // interleaved record: 4 descriptor floats, confidence, 3 pad
 constexpr int kPrimaryCap     = 2048;         // fragment records a bin has room for where about a thousand are expected
 constexpr int kPrimaryCapSmall = 1024;        // ... and where at most half of that is (a bin built in LDS holds <= 1024)
-constexpr int kViewLanes      = 4;            // views of one call that run side by side (each with scratch of its own)
+constexpr int kViewLanes      = 4;            // views of one call that share a launch (each with scratch of its own)
 constexpr int kLogSegments    = 256;          // the overflow log is cut into this many segments with a cursor each
 constexpr int kLogCursorStride = 16;          // uint32 between two cursors (64 bytes: one cursor per cache line)
 
@@ -123,6 +123,15 @@ __device__ __forceinline__ uint32_t wave_inclusive_scan(uint32_t v, int /*lane*/
 }
 
 // Launch descriptor shared by the forward kernels of one view.
+// Several views of a call in one launch: the arguments of every view travel side by side as the kernel argument and
+// blockIdx.y (blockIdx.z where a kernel uses y itself) picks the view. Small views (training crops) leave most of the
+// chip idle on their own and are chains of dependent launches; four of them at a time fill it.
+template <class Args>
+struct PerView
+{
+    Args v[kViewLanes];
+};
+
 struct ViewPass
 {
     const float4* position;

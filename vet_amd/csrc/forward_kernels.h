@@ -341,8 +341,8 @@ __device__ __forceinline__ void store_record(const ScatterTargets& t, const Laye
 // (BILINEAR_BLEND), each of which is a fragment of its own with its own bin; the low key word is then
 // point id << 2 | corner.
 template <int HITS>
-__global__ void __launch_bounds__(kBlock) bin_scatter_kernel(ViewPass a, uint32_t* __restrict__ bin_counts,
-                                                              ScatterTargets out, PackJob pack)
+__device__ __forceinline__ void bin_scatter(const ViewPass& a, uint32_t* __restrict__ bin_counts,
+                                            const ScatterTargets& out, const PackJob& pack)
 {
     const int slot = blockIdx.x * blockDim.x + threadIdx.x;
     const int lane = threadIdx.x & (kWave - 1);
@@ -492,6 +492,31 @@ __global__ void __launch_bounds__(kBlock) bin_scatter_kernel(ViewPass a, uint32_
     if (packs) store_packed_row(pack, slot, row, row_confidence);
 }
 
+template <int HITS>
+__global__ void __launch_bounds__(kBlock) bin_scatter_kernel(ViewPass a, uint32_t* __restrict__ bin_counts,
+                                                              ScatterTargets out, PackJob pack)
+{
+    bin_scatter<HITS>(a, bin_counts, out, pack);
+}
+
+struct ScatterArgs
+{
+    ViewPass view;
+    uint32_t* bin_counts;
+    ScatterTargets out;
+    PackJob pack;
+};
+
+// (A thread that took its point through the views of a round one after the other would read the point arrays once
+// instead of once per view; measured, that is slower: the pass waits for its atomics, not for memory, and fewer,
+// longer threads hide less of that.)
+template <int HITS>
+__global__ void __launch_bounds__(kBlock) bin_scatter_views_kernel(PerView<ScatterArgs> views)
+{
+    const ScatterArgs& v = views.v[blockIdx.y];
+    bin_scatter<HITS>(v.view, v.bin_counts, v.out, v.pack);
+}
+
 // The interleave as a launch of its own, for a caller that keeps the records across calls while texture and confidence
 // stay as they are (vetrast_pack_descriptors): every row, whatever a view sees.
 __global__ void __launch_bounds__(kBlock) pack_descriptors_kernel(PackJob pack)
@@ -507,8 +532,8 @@ __global__ void __launch_bounds__(kBlock) pack_descriptors_kernel(PackJob pack)
 
 // Brings the logged records (rank beyond the bin's own room) to the bin's place in the compact array:
 // binned[bin_offsets[bin] + rank]. Runs after the scan of the bin counts; the log is empty as a rule.
-__global__ void __launch_bounds__(kBlock) overflow_move_kernel(ScatterTargets in, const uint32_t* __restrict__ bin_offsets,
-                                                                uint4* __restrict__ binned, uint32_t capacity)
+__device__ __forceinline__ void overflow_move(const ScatterTargets& in, const uint32_t* __restrict__ bin_offsets,
+                                              uint4* __restrict__ binned, uint32_t capacity)
 {
     for (uint32_t segment = blockIdx.x; segment < (uint32_t)kLogSegments; segment += gridDim.x)
     {
@@ -525,6 +550,30 @@ __global__ void __launch_bounds__(kBlock) overflow_move_kernel(ScatterTargets in
                 binned[pos] = make_uint4(rec.x, rec.y, rec.z, 0u);
         }
     }
+}
+
+__global__ void __launch_bounds__(kBlock) overflow_move_kernel(ScatterTargets in, const uint32_t* __restrict__ bin_offsets,
+                                                                uint4* __restrict__ binned, uint32_t capacity)
+{
+    overflow_move(in, bin_offsets, binned, capacity);
+}
+
+// What the scan and move kernels of one view work on.
+struct ScanArgs
+{
+    uint32_t* bin_counts;     // the counts; the scan-and-move kernel leaves its result `scanned_behind` words behind
+    uint32_t scanned_behind;  // them, the two-launch scan in place
+    uint32_t n;               // counts (scan and move in one launch)
+    uint32_t* partials;       // one word per 4096 counts (scan in two launches)
+    ScatterTargets in;
+    uint4* binned;
+    uint32_t capacity;
+};
+
+__global__ void __launch_bounds__(kBlock) overflow_move_views_kernel(PerView<ScanArgs> views)
+{
+    const ScanArgs& v = views.v[blockIdx.y];
+    overflow_move(v.in, v.bin_counts, v.binned, v.capacity);
 }
 
 // ---- exclusive scan of the per-tile counts, in place, in two launches --------------------------------------------
@@ -544,8 +593,7 @@ __device__ __forceinline__ uint32_t block_reduce_sum(uint32_t v, uint32_t* lds4)
     return total;
 }
 
-__global__ void __launch_bounds__(kBlock) scan_partials_kernel(const uint4* __restrict__ counts4,
-                                                                uint32_t* __restrict__ partials)
+__device__ __forceinline__ void scan_partials(const uint4* __restrict__ counts4, uint32_t* __restrict__ partials)
 {
     __shared__ uint32_t lds4[4];
     const uint4* src = counts4 + (size_t)blockIdx.x * (kScanPerBlock / 4);
@@ -560,8 +608,19 @@ __global__ void __launch_bounds__(kBlock) scan_partials_kernel(const uint4* __re
     if (threadIdx.x == 0) partials[blockIdx.x] = total;
 }
 
-__global__ void __launch_bounds__(kBlock) scan_apply_kernel(uint4* __restrict__ counts4,
-                                                             const uint32_t* __restrict__ partials)
+__global__ void __launch_bounds__(kBlock) scan_partials_kernel(const uint4* __restrict__ counts4,
+                                                                uint32_t* __restrict__ partials)
+{
+    scan_partials(counts4, partials);
+}
+
+__global__ void __launch_bounds__(kBlock) scan_partials_views_kernel(PerView<ScanArgs> views)
+{
+    const ScanArgs& v = views.v[blockIdx.y];
+    scan_partials(reinterpret_cast<const uint4*>(v.bin_counts), v.partials);
+}
+
+__device__ __forceinline__ void scan_apply(uint4* __restrict__ counts4, const uint32_t* __restrict__ partials)
 {
     __shared__ uint32_t lds4[4];
     __shared__ uint32_t wave_tot[4];
@@ -601,6 +660,18 @@ __global__ void __launch_bounds__(kBlock) scan_apply_kernel(uint4* __restrict__ 
     }
 }
 
+__global__ void __launch_bounds__(kBlock) scan_apply_kernel(uint4* __restrict__ counts4,
+                                                             const uint32_t* __restrict__ partials)
+{
+    scan_apply(counts4, partials);
+}
+
+__global__ void __launch_bounds__(kBlock) scan_apply_views_kernel(PerView<ScanArgs> views)
+{
+    const ScanArgs& v = views.v[blockIdx.y];
+    scan_apply(reinterpret_cast<uint4*>(v.bin_counts), v.partials);
+}
+
 // Scan and move in one launch, for up to kScanMoveMax counts: one workgroup per segment of the overflow log. Every
 // workgroup whose segment holds entries scans the bin counts into LDS for itself and files its entries with them;
 // workgroup 0 scans in any case and writes the result to `offsets` (the counts stay as they are, so that the other
@@ -608,9 +679,8 @@ __global__ void __launch_bounds__(kBlock) scan_apply_kernel(uint4* __restrict__ 
 // scan alone, where the two kernels cost a launch (and a dependency on the one before) each.
 constexpr int kScanMoveMax = 60 * kBlock;  // 61 440 bytes of LDS
 
-__global__ void __launch_bounds__(kBlock) scan_move_kernel(const uint4* __restrict__ counts4, uint32_t n,
-                                                            uint4* __restrict__ offsets4, ScatterTargets in,
-                                                            uint4* __restrict__ binned, uint32_t capacity)
+__device__ __forceinline__ void scan_move(const uint4* __restrict__ counts4, uint32_t n, uint4* __restrict__ offsets4,
+                                          const ScatterTargets& in, uint4* __restrict__ binned, uint32_t capacity)
 {
     __shared__ uint32_t s_off[kScanMoveMax];
     __shared__ uint32_t wave_tot[kBlock / kWave];
@@ -664,6 +734,20 @@ __global__ void __launch_bounds__(kBlock) scan_move_kernel(const uint4* __restri
         else
             binned[pos] = make_uint4(rec.x, rec.y, rec.z, 0u);
     }
+}
+
+__global__ void __launch_bounds__(kBlock) scan_move_kernel(const uint4* __restrict__ counts4, uint32_t n,
+                                                            uint4* __restrict__ offsets4, ScatterTargets in,
+                                                            uint4* __restrict__ binned, uint32_t capacity)
+{
+    scan_move(counts4, n, offsets4, in, binned, capacity);
+}
+
+__global__ void __launch_bounds__(kBlock) scan_move_views_kernel(PerView<ScanArgs> views)
+{
+    const ScanArgs& v = views.v[blockIdx.y];
+    scan_move(reinterpret_cast<const uint4*>(v.bin_counts), v.n,
+              reinterpret_cast<uint4*>(v.bin_counts + v.scanned_behind), v.in, v.binned, v.capacity);
 }
 
 // Front-to-back blend of one pixel's sorted list read from memory: out += (T*c)*t, T = (1-c)*T, in exactly this order

@@ -723,8 +723,6 @@ int vetrast_forward(vetrast_ctx* ctx, const vetrast_forward_args* a, void* strea
     float4* packed       = own_pack ? ws_ptr<float4>(ws, lay.packed_base)
                                     : reinterpret_cast<float4*>(const_cast<float*>(a->packed_descriptors));
     DeviceView* views   = ws_ptr<DeviceView>(ws, lay.views_base);
-    hipStream_t caller  = stream;
-    ViewLanes lanes(ctx, caller, lay.view_lanes);
 
     {
         ScopeTimer tm(ctx, stream, VETRAST_SCOPE_PREPARE);
@@ -753,111 +751,69 @@ int vetrast_forward(vetrast_ctx* ctx, const vetrast_forward_args* a, void* strea
         }
     }
 
-    lanes.fork();
-    hipEvent_t packed_ready = nullptr;  // the first view's scatter pass has interleaved the descriptors
-    for (int b = 0; b < B; ++b)
+    // Views in rounds of up to view_lanes: every kernel takes the views of a round in one launch (each view with the
+    // scratch of its lane).
+    const int lanes          = std::max(1, lay.view_lanes);
+    const bool scan_and_move = bins + 1 <= (uint32_t)kScanMoveMax;
+    for (int first = 0; first < B; first += lanes)
     {
-        // this view's lane: its stream, its copy of the scratch
-        stream               = lanes.stream(b);
-        const size_t lane    = (size_t)lanes.lane(b);
-        uint32_t* slots      = ws_ptr<uint32_t>(ws, lay.slots_base + lay.lane_scratch_stride * lane);
-        uint32_t* partials   = ws_ptr<uint32_t>(ws, lay.scan_partials_base + lay.scan_partials_stride * lane);
-        const ViewPass vp   = make_view_pass(a, lay, ly, b);
-        uint32_t* offsets   = ws_ptr<uint32_t>(ws, lay.offsets_base + lay.offsets_stride * b);
-        uint64_t* fragments = ws_ptr<uint64_t>(ws, lay.fragments_base + lay.fragments_stride * b);
-        float* trans        = ws_ptr<float>(ws, lay.transmittance_base + lay.transmittance_stride * b);
-        float* weight       = ws_ptr<float>(ws, lay.weight_base + lay.weight_stride * b);
-        uint32_t* bin_counts     = ws_ptr<uint32_t>(ws, lay.bin_counts_base + lay.bin_counts_stride * b);
-        uint4* binned            = ws_ptr<uint4>(ws, lay.binned_base + lay.binned_stride * lane);
-        ScatterTargets targets;
-        targets.primary      = ws_ptr<uint4>(ws, lay.primary_base + lay.primary_stride * lane);
-        targets.compact      = compact_records(N, hits) ? 1 : 0;
-        targets.log          = ws_ptr<uint4>(ws, lay.log_base + lay.lane_scratch_stride * lane);
-        targets.log_rank     = slots;
-        targets.log_cursor   = ws_ptr<uint32_t>(ws, lay.log_cursor_base) + (size_t)b * kLogSegments * kLogCursorStride;
-        targets.segment_capacity = log_segment_records(N, L, hits);
-        // the scatter pass of the first view also interleaves the descriptors (PrepareTexture / PrepareConfidence included)
-        PackJob pack;
-        pack.texture               = a->texture;
-        pack.confidence            = a->confidence;
-        pack.packed                = (b == 0 && own_pack) ? packed : nullptr;
-        pack.N                     = N;
-        pack.C                     = C;
-        pack.confidence_activation = p.confidence_activation;
-        pack.confidence_scale      = p.confidence_scale;
-        pack.texture_abs           = p.texture_abs;
-        pack.visible_only          = (B == 1 && a->index == nullptr && a->point_order == nullptr) ? 1 : 0;
-        uint8_t* list_is_cut     = ws_ptr<uint8_t>(ws, lay.cut_flags_base + lay.cut_flags_stride * b);
-        if (N > 0)
+        const int last = std::min(B, first + lanes), count = last - first;
+        const bool one = count == 1;
+        PerView<ScatterArgs> scatter;
+        PerView<ScanArgs> scan;
+        PerView<BuildPass> build;
+        for (int b = first; b < last; ++b)
         {
-            ScopeTimer tm(ctx, stream, VETRAST_SCOPE_COUNT);
-            if (hits == 1)
-                hipLaunchKernelGGL(bin_scatter_kernel<1>, dim3(grid_for(N)), dim3(kBlock), 0, stream, vp, bin_counts, targets, pack);
-            else
-                hipLaunchKernelGGL(bin_scatter_kernel<4>, dim3(grid_for(N)), dim3(kBlock), 0, stream, vp, bin_counts, targets, pack);
-        }
-        if (b == 0 && lanes.lanes > 1 && own_pack) packed_ready = lanes.mark(stream);
-        // Where the bins of a view are few enough, one launch scans their counts and files the logged records (the
-        // scan lands behind the counts); otherwise the scan runs in place and the move kernel follows.
-        const bool scan_and_move = bins + 1 <= (uint32_t)kScanMoveMax;
-        const uint32_t* bin_offsets = scan_and_move ? bin_counts + Tpad : bin_counts;
-        {
-            ScopeTimer tm(ctx, stream, VETRAST_SCOPE_SCAN);
-            if (scan_and_move)
-                hipLaunchKernelGGL(scan_move_kernel, dim3(kLogSegments), dim3(kBlock), 0, stream,
-                                   reinterpret_cast<const uint4*>(bin_counts), bins + 1,
-                                   reinterpret_cast<uint4*>(bin_counts + Tpad), targets, binned,
-                                   (uint32_t)lay.fragment_capacity);
-            else
-            {
-                const int blocks = (int)(Tpad / kScanPerBlock);
-                hipLaunchKernelGGL(scan_partials_kernel, dim3(blocks), dim3(kBlock), 0, stream,
-                                   reinterpret_cast<const uint4*>(bin_counts), partials);
-                hipLaunchKernelGGL(scan_apply_kernel, dim3(blocks), dim3(kBlock), 0, stream,
-                                   reinterpret_cast<uint4*>(bin_counts), partials);
-            }
-        }
-        if (N > 0 && !scan_and_move)
-        {
-            ScopeTimer tm(ctx, stream, VETRAST_SCOPE_FILL);
-            // the few records beyond their bin's own room, if any
-            hipLaunchKernelGGL(overflow_move_kernel, dim3(256), dim3(kBlock), 0, stream, targets, bin_counts, binned,
-                               (uint32_t)lay.fragment_capacity);
-        }
-        float* out[VETRAST_MAX_LAYERS];
-        float* out_mask[VETRAST_MAX_LAYERS];
-        float* out_weight[VETRAST_MAX_LAYERS];
-        for (int l = 0; l < VETRAST_MAX_LAYERS; ++l)
-        {
-            out[l]        = nullptr;
-            out_mask[l]   = nullptr;
-            out_weight[l] = nullptr;
-            if (l >= L) continue;
-            const size_t plane = (size_t)ly.w[l] * ly.h[l];
-            out[l]             = a->out[l] + (size_t)b * C * plane;
-            if (p.output_background_mask) out_mask[l] = a->out_mask[l] + (size_t)b * plane;
-            if (a->out_weight[l]) out_weight[l] = a->out_weight[l] + (size_t)b * plane;
-        }
-        // the build pass reads the descriptor records: the first view of every other lane waits for them
-        if (b > 0 && b < lanes.lanes) lanes.wait(stream, packed_ready);
-        {
-            ScopeTimer tm(ctx, stream, VETRAST_SCOPE_BUILD);
-            BuildPass bp;
-            bp.bin_offsets         = bin_offsets;
+            const size_t lane = (size_t)(b - first);
+            ScatterArgs& sc   = scatter.v[lane];
+            sc.view           = make_view_pass(a, lay, ly, b);
+            sc.bin_counts     = ws_ptr<uint32_t>(ws, lay.bin_counts_base + lay.bin_counts_stride * b);
+            ScatterTargets& targets  = sc.out;
+            targets.primary          = ws_ptr<uint4>(ws, lay.primary_base + lay.primary_stride * lane);
+            targets.compact          = compact_records(N, hits) ? 1 : 0;
+            targets.log              = ws_ptr<uint4>(ws, lay.log_base + lay.lane_scratch_stride * lane);
+            targets.log_rank         = ws_ptr<uint32_t>(ws, lay.slots_base + lay.lane_scratch_stride * lane);
+            targets.log_cursor       = ws_ptr<uint32_t>(ws, lay.log_cursor_base) + (size_t)b * kLogSegments * kLogCursorStride;
+            targets.segment_capacity = log_segment_records(N, L, hits);
+            // the scatter pass of the first view also interleaves the descriptors (PrepareTexture / PrepareConfidence included)
+            PackJob& pack              = sc.pack;
+            pack.texture               = a->texture;
+            pack.confidence            = a->confidence;
+            pack.packed                = (b == 0 && own_pack) ? packed : nullptr;
+            pack.N                     = N;
+            pack.C                     = C;
+            pack.confidence_activation = p.confidence_activation;
+            pack.confidence_scale      = p.confidence_scale;
+            pack.texture_abs           = p.texture_abs;
+            pack.visible_only          = (B == 1 && a->index == nullptr && a->point_order == nullptr) ? 1 : 0;
+
+            // Where the bins of a view are few enough, one launch scans their counts and files the logged records (the
+            // scan lands behind the counts); otherwise the scan runs in place and the move kernel follows.
+            ScanArgs& sa      = scan.v[lane];
+            sa.bin_counts     = sc.bin_counts;
+            sa.scanned_behind = (uint32_t)Tpad;
+            sa.n              = bins + 1;
+            sa.partials       = ws_ptr<uint32_t>(ws, lay.scan_partials_base + lay.scan_partials_stride * lane);
+            sa.in             = targets;
+            sa.binned         = ws_ptr<uint4>(ws, lay.binned_base + lay.binned_stride * lane);
+            sa.capacity       = (uint32_t)lay.fragment_capacity;
+
+            BuildPass& bp          = build.v[lane];
+            bp.bin_offsets         = scan_and_move ? sc.bin_counts + Tpad : sc.bin_counts;
             bp.primary             = targets.primary;
-            bp.binned              = binned;
+            bp.binned              = sa.binned;
             bp.compact_records     = targets.compact;
-            bp.offsets             = offsets;
-            bp.fragments           = fragments;
-            bp.list_is_cut         = list_is_cut;
+            bp.offsets             = ws_ptr<uint32_t>(ws, lay.offsets_base + lay.offsets_stride * b);
+            bp.fragments           = ws_ptr<uint64_t>(ws, lay.fragments_base + lay.fragments_stride * b);
+            bp.list_is_cut         = ws_ptr<uint8_t>(ws, lay.cut_flags_base + lay.cut_flags_stride * b);
             bp.last_key            = ws_ptr<uint64_t>(ws, lay.last_key_base + lay.last_key_stride * b);
             bp.kept                = ws_ptr<uint32_t>(ws, lay.kept_base + lay.kept_stride * b);
-            bp.projected           = vp.projected;
+            bp.projected           = sc.view.projected;
             bp.index               = a->index;
             bp.packed              = packed;
             bp.background          = reinterpret_cast<const float*>(flags) + kPreparedBackgroundOffset;
-            bp.transmittance       = a->save_for_backward ? trans : nullptr;
-            bp.weight              = weight;
+            bp.transmittance       = a->save_for_backward ? ws_ptr<float>(ws, lay.transmittance_base + lay.transmittance_stride * b) : nullptr;
+            bp.weight              = ws_ptr<float>(ws, lay.weight_base + lay.weight_stride * b);
             bp.ly                  = ly;
             bp.num_bins            = bins;
             bp.N                   = N;
@@ -866,36 +822,99 @@ int vetrast_forward(vetrast_ctx* ctx, const vetrast_forward_args* a, void* strea
             bp.mask_value          = p.output_background_mask_value;
             bp.depth_accept        = p.depth_accept_blend;
             for (int l = 0; l < VETRAST_MAX_LAYERS; ++l)
-                bp.out[l] = out[l], bp.out_mask[l] = out_mask[l], bp.out_weight[l] = out_weight[l];
-            const dim3 g(bins), blk(kBlock);
-            if (p.render_mode == VETRAST_RENDER_FUZZY_BLEND)
-                switch (C)
-                {
-                    case 1: hipLaunchKernelGGL((bin_build_kernel<1, false, true>), g, blk, 0, stream, bp); break;
-                    case 2: hipLaunchKernelGGL((bin_build_kernel<2, false, true>), g, blk, 0, stream, bp); break;
-                    case 3: hipLaunchKernelGGL((bin_build_kernel<3, false, true>), g, blk, 0, stream, bp); break;
-                    default: hipLaunchKernelGGL((bin_build_kernel<4, false, true>), g, blk, 0, stream, bp); break;
-                }
+            {
+                bp.out[l] = bp.out_mask[l] = bp.out_weight[l] = nullptr;
+                if (l >= L) continue;
+                const size_t plane = (size_t)ly.w[l] * ly.h[l];
+                bp.out[l]          = a->out[l] + (size_t)b * C * plane;
+                if (p.output_background_mask) bp.out_mask[l] = a->out_mask[l] + (size_t)b * plane;
+                if (a->out_weight[l]) bp.out_weight[l] = a->out_weight[l] + (size_t)b * plane;
+            }
+        }
+        const dim3 blk(kBlock);
+        const unsigned views_y = (unsigned)count;
+        if (N > 0)
+        {
+            ScopeTimer tm(ctx, stream, VETRAST_SCOPE_COUNT);
+            const ScatterArgs& sc = scatter.v[0];
+            const dim3 g(grid_for(N)), gv(grid_for(N), views_y);
+            if (hits == 1 && one)
+                hipLaunchKernelGGL(bin_scatter_kernel<1>, g, blk, 0, stream, sc.view, sc.bin_counts, sc.out, sc.pack);
             else if (hits == 1)
-                switch (C)
-                {
-                    case 1: hipLaunchKernelGGL((bin_build_kernel<1, false>), g, blk, 0, stream, bp); break;
-                    case 2: hipLaunchKernelGGL((bin_build_kernel<2, false>), g, blk, 0, stream, bp); break;
-                    case 3: hipLaunchKernelGGL((bin_build_kernel<3, false>), g, blk, 0, stream, bp); break;
-                    default: hipLaunchKernelGGL((bin_build_kernel<4, false>), g, blk, 0, stream, bp); break;
-                }
+                hipLaunchKernelGGL(bin_scatter_views_kernel<1>, gv, blk, 0, stream, scatter);
+            else if (one)
+                hipLaunchKernelGGL(bin_scatter_kernel<4>, g, blk, 0, stream, sc.view, sc.bin_counts, sc.out, sc.pack);
             else
+                hipLaunchKernelGGL(bin_scatter_views_kernel<4>, gv, blk, 0, stream, scatter);
+        }
+        {
+            ScopeTimer tm(ctx, stream, VETRAST_SCOPE_SCAN);
+            const ScanArgs& sa = scan.v[0];
+            if (scan_and_move)
+            {
+                if (one)
+                    hipLaunchKernelGGL(scan_move_kernel, dim3(kLogSegments), blk, 0, stream,
+                                       reinterpret_cast<const uint4*>(sa.bin_counts), sa.n,
+                                       reinterpret_cast<uint4*>(sa.bin_counts + Tpad), sa.in, sa.binned, sa.capacity);
+                else
+                    hipLaunchKernelGGL(scan_move_views_kernel, dim3(kLogSegments, views_y), blk, 0, stream, scan);
+            }
+            else
+            {
+                const unsigned blocks = (unsigned)(Tpad / kScanPerBlock);
+                if (one)
+                {
+                    hipLaunchKernelGGL(scan_partials_kernel, dim3(blocks), blk, 0, stream,
+                                       reinterpret_cast<const uint4*>(sa.bin_counts), sa.partials);
+                    hipLaunchKernelGGL(scan_apply_kernel, dim3(blocks), blk, 0, stream,
+                                       reinterpret_cast<uint4*>(sa.bin_counts), sa.partials);
+                }
+                else
+                {
+                    hipLaunchKernelGGL(scan_partials_views_kernel, dim3(blocks, views_y), blk, 0, stream, scan);
+                    hipLaunchKernelGGL(scan_apply_views_kernel, dim3(blocks, views_y), blk, 0, stream, scan);
+                }
+            }
+        }
+        if (N > 0 && !scan_and_move)
+        {
+            ScopeTimer tm(ctx, stream, VETRAST_SCOPE_FILL);
+            // the few records beyond their bin's own room, if any
+            const ScanArgs& sa = scan.v[0];
+            if (one)
+                hipLaunchKernelGGL(overflow_move_kernel, dim3(256), blk, 0, stream, sa.in, sa.bin_counts, sa.binned, sa.capacity);
+            else
+                hipLaunchKernelGGL(overflow_move_views_kernel, dim3(256, views_y), blk, 0, stream, scan);
+        }
+        {
+            ScopeTimer tm(ctx, stream, VETRAST_SCOPE_BUILD);
+            const BuildPass& bp = build.v[0];
+            const dim3 g(bins), gv(bins, views_y);
+            auto launch = [&](auto channels, auto bilinear, auto fuzzy) {
+                constexpr int kC         = decltype(channels)::value;
+                constexpr bool kBilinear = decltype(bilinear)::value, kFuzzy = decltype(fuzzy)::value;
+                if (one)
+                    hipLaunchKernelGGL((bin_build_kernel<kC, kBilinear, kFuzzy>), g, blk, 0, stream, bp);
+                else
+                    hipLaunchKernelGGL((bin_build_views_kernel<kC, kBilinear, kFuzzy>), gv, blk, 0, stream, build);
+            };
+            auto with_channels = [&](auto bilinear, auto fuzzy) {
                 switch (C)
                 {
-                    case 1: hipLaunchKernelGGL((bin_build_kernel<1, true>), g, blk, 0, stream, bp); break;
-                    case 2: hipLaunchKernelGGL((bin_build_kernel<2, true>), g, blk, 0, stream, bp); break;
-                    case 3: hipLaunchKernelGGL((bin_build_kernel<3, true>), g, blk, 0, stream, bp); break;
-                    default: hipLaunchKernelGGL((bin_build_kernel<4, true>), g, blk, 0, stream, bp); break;
+                    case 1: launch(std::integral_constant<int, 1>{}, bilinear, fuzzy); break;
+                    case 2: launch(std::integral_constant<int, 2>{}, bilinear, fuzzy); break;
+                    case 3: launch(std::integral_constant<int, 3>{}, bilinear, fuzzy); break;
+                    default: launch(std::integral_constant<int, 4>{}, bilinear, fuzzy); break;
                 }
+            };
+            if (p.render_mode == VETRAST_RENDER_FUZZY_BLEND)
+                with_channels(std::false_type{}, std::true_type{});
+            else if (hits == 1)
+                with_channels(std::false_type{}, std::false_type{});
+            else
+                with_channels(std::true_type{}, std::false_type{});
         }
     }
-    lanes.join();
-    VET_HIP(ctx, lanes.err);
     VET_HIP(ctx, hipGetLastError());
     return VETRAST_OK;
 }
@@ -1004,79 +1023,102 @@ int vetrast_backward(vetrast_ctx* ctx, const vetrast_backward_args* g, void* str
         }
         point_major_records = (known && expected < (double)N * hits * L / 3.0) ? 1 : 0;
     }
-    // The per-pixel kernels of up to view_lanes views run side by side, each into its lane's record array; the
-    // per-point kernels add to the same gradient rows, so they stay on the caller's stream, one view after the other,
-    // each behind its view's per-pixel kernel; a lane's next per-pixel kernel waits for the per-point kernel that
-    // reads what the last one left.
-    hipStream_t caller = stream;
-    ViewLanes lanes(ctx, caller, lay.view_lanes);
-    lanes.fork();
-    std::vector<hipEvent_t> gathered((size_t)B, nullptr);
-    // the per-pixel part of view b, on its lane
-    auto per_pixel = [&](int b) {
-        const size_t lane      = (size_t)lanes.lane(b);
-        float4* partial        = ws_ptr<float4>(ws, lay.partial_base + lay.lane_scratch_stride * lane);
-        float* background_rows = ws_ptr<float>(ws, lay.background_partial_base + lay.lane_scratch_stride * lane);
-        uint32_t* offsets   = ws_ptr<uint32_t>(ws, lay.offsets_base + lay.offsets_stride * b);
-        uint64_t* fragments = ws_ptr<uint64_t>(ws, lay.fragments_base + lay.fragments_stride * b);
-        stream = lanes.stream(b);
-        if (lanes.lanes > 1 && b >= lanes.lanes) lanes.wait(stream, gathered[(size_t)(b - lanes.lanes)]);
+    // Views in rounds of up to view_lanes: the per-pixel kernel takes the views of a round in one launch, each into its
+    // lane's record array, and the per-point kernel behind it reads them all, again in one launch (the views add to
+    // the same gradient rows).
+    const int lanes = std::max(1, lay.view_lanes);
+    const float4* packed = a->packed_descriptors ? reinterpret_cast<const float4*>(a->packed_descriptors)
+                                                 : ws_ptr<float4>(ws, lay.packed_base);
+    const int background_rows_count = (int)tile_grid(tiles) + (fuzzy_long ? kFuzzyFoldRows : 0);
+    for (int first = 0; first < B; first += lanes)
+    {
+        const int last = std::min(B, first + lanes), count = last - first;
+        float4* partial        = ws_ptr<float4>(ws, lay.partial_base);
+        float* background_rows = ws_ptr<float>(ws, lay.background_partial_base);
         {
             ScopeTimer tm(ctx, stream, VETRAST_SCOPE_BACKWARD_BLEND);
-            BackwardPass bp;
-            bp.offsets          = offsets;
-            bp.kept             = ws_ptr<uint32_t>(ws, lay.kept_base + lay.kept_stride * b);
-            bp.projected        = lay.projected_stride ? ws_ptr<float2>(ws, lay.projected_base + lay.projected_stride * b) : nullptr;
-            bp.fragments        = fragments;
-            bp.transmittance    = ws_ptr<float>(ws, lay.transmittance_base + lay.transmittance_stride * b);
-            bp.weight           = ws_ptr<float>(ws, lay.weight_base + lay.weight_stride * b);
-            bp.index            = a->index;
-            bp.packed           = a->packed_descriptors ? reinterpret_cast<const float4*>(a->packed_descriptors)
-                                                        : ws_ptr<float4>(ws, lay.packed_base);
-            bp.background       = ws_ptr<const float>(ws, lay.flags_base) + kPreparedBackgroundOffset;
-            bp.partial          = partial;
-            bp.point_major_records = point_major_records;
-            bp.background_partial = background_rows;
-            bp.ly               = ly;
-            bp.tiles            = tiles;
-            bp.N                = N;
-            bp.K                = p.debug_max_list_length;
-            bp.use_environment_map              = p.use_environment_map;
-            bp.need_point_gradient              = want_image_gradient ? 1 : 0;
-            bp.quirk_background_confidence_leak = p.quirk_background_confidence_leak;
-            bp.clear                            = b == 0 ? clear : ClearJob{};
-            for (int l = 0; l < VETRAST_MAX_LAYERS; ++l)
+            PerView<BackwardPass> views;
+            for (int b = first; b < last; ++b)
             {
-                bp.grad_out[l] = nullptr;
-                bp.out[l]      = nullptr;
-                if (l >= L) continue;
-                const size_t plane = (size_t)ly.w[l] * ly.h[l];
-                bp.grad_out[l]     = g->grad_out[l] + (size_t)b * C * plane;
-                bp.out[l]          = a->out[l] + (size_t)b * C * plane;
+                const size_t lane = (size_t)(b - first);
+                BackwardPass& bp  = views.v[lane];
+                bp.offsets          = ws_ptr<uint32_t>(ws, lay.offsets_base + lay.offsets_stride * b);
+                bp.kept             = ws_ptr<uint32_t>(ws, lay.kept_base + lay.kept_stride * b);
+                bp.projected        = lay.projected_stride ? ws_ptr<float2>(ws, lay.projected_base + lay.projected_stride * b) : nullptr;
+                bp.fragments        = ws_ptr<uint64_t>(ws, lay.fragments_base + lay.fragments_stride * b);
+                bp.transmittance    = ws_ptr<float>(ws, lay.transmittance_base + lay.transmittance_stride * b);
+                bp.weight           = ws_ptr<float>(ws, lay.weight_base + lay.weight_stride * b);
+                bp.index            = a->index;
+                bp.packed           = packed;
+                bp.background       = ws_ptr<const float>(ws, lay.flags_base) + kPreparedBackgroundOffset;
+                bp.partial          = ws_ptr<float4>(ws, lay.partial_base + lay.lane_scratch_stride * lane);
+                bp.point_major_records = point_major_records;
+                bp.background_partial  = ws_ptr<float>(ws, lay.background_partial_base + lay.lane_scratch_stride * lane);
+                bp.ly               = ly;
+                bp.tiles            = tiles;
+                bp.N                = N;
+                bp.K                = p.debug_max_list_length;
+                bp.use_environment_map              = p.use_environment_map;
+                bp.need_point_gradient              = want_image_gradient ? 1 : 0;
+                bp.quirk_background_confidence_leak = p.quirk_background_confidence_leak;
+                bp.clear                            = b == 0 ? clear : ClearJob{};
+                for (int l = 0; l < VETRAST_MAX_LAYERS; ++l)
+                {
+                    bp.grad_out[l] = nullptr;
+                    bp.out[l]      = nullptr;
+                    if (l >= L) continue;
+                    const size_t plane = (size_t)ly.w[l] * ly.h[l];
+                    bp.grad_out[l]     = g->grad_out[l] + (size_t)b * C * plane;
+                    bp.out[l]          = a->out[l] + (size_t)b * C * plane;
+                }
             }
-            const dim3 grid(tile_grid(tiles)), blk(kBlock);
+            const BackwardPass& bp = views.v[0];
+            const unsigned tiles_x = tile_grid(tiles);
+            const dim3 grid(tiles_x), grid_views(tiles_x, (unsigned)count), blk(kBlock);
+            const bool one = count == 1;
             if (p.render_mode == VETRAST_RENDER_FUZZY_BLEND)
             {
                 // Lists of more than kFuzzyDense fragments exist only where the cut allows them; each is taken by a whole
                 // wave, in a second kernel.
                 const bool beyond_dense = bp.K <= 0 || bp.K > kFuzzyDense;
                 // With longer lists about, the narrow dense kernel in front of that one is faster than the wide one (measured).
-                const bool wide = !beyond_dense && bp.K > kFuzzyNarrow;
+                const bool wide    = !beyond_dense && bp.K > kFuzzyNarrow;
+                const float accept = p.depth_accept_blend;
                 auto launch = [&](auto channels) {
                     constexpr int kC = decltype(channels)::value;
-                    if (wide)
-                        hipLaunchKernelGGL((blend_backward_fuzzy_kernel<kC, kFuzzyDense>), grid, blk, 0, stream, bp, p.depth_accept_blend);
+                    if (wide && one)
+                        hipLaunchKernelGGL((blend_backward_fuzzy_kernel<kC, kFuzzyDense>), grid, blk, 0, stream, bp, accept);
+                    else if (wide)
+                        hipLaunchKernelGGL((blend_backward_fuzzy_views_kernel<kC, kFuzzyDense>), grid_views, blk, 0, stream, views, accept);
+                    else if (one)
+                        hipLaunchKernelGGL((blend_backward_fuzzy_kernel<kC, kFuzzyNarrow>), grid, blk, 0, stream, bp, accept);
                     else
-                        hipLaunchKernelGGL((blend_backward_fuzzy_kernel<kC, kFuzzyNarrow>), grid, blk, 0, stream, bp, p.depth_accept_blend);
+                        hipLaunchKernelGGL((blend_backward_fuzzy_views_kernel<kC, kFuzzyNarrow>), grid_views, blk, 0, stream, views, accept);
                     if (beyond_dense)
                     {
-                        hipLaunchKernelGGL(blend_backward_fuzzy_long_kernel<kC>, dim3(grid.x, kFuzzyReplicas), blk, 0, stream, bp,
-                                           p.depth_accept_blend, (uint32_t)(wide ? kFuzzyDense : kFuzzyNarrow));
+                        const uint32_t dense_max = (uint32_t)(wide ? kFuzzyDense : kFuzzyNarrow);
                         // the rows of replicas 1 .. into kFuzzyFoldRows rows behind the per-workgroup ones
-                        hipLaunchKernelGGL(fold_background_rows_kernel, dim3(kFuzzyFoldRows), blk, 0, stream,
-                                           bp.background_partial + ((size_t)kFuzzyFoldRows + grid.x) * kBackgroundRow,
-                                           (int)((kFuzzyReplicas - 1) * grid.x),
-                                           bp.background_partial + (size_t)grid.x * kBackgroundRow);
+                        PerView<FoldArgs> folds;
+                        for (int k = 0; k < count; ++k)
+                        {
+                            folds.v[k].rows     = views.v[k].background_partial + ((size_t)kFuzzyFoldRows + tiles_x) * kBackgroundRow;
+                            folds.v[k].num_rows = (int)((kFuzzyReplicas - 1) * tiles_x);
+                            folds.v[k].folded   = views.v[k].background_partial + (size_t)tiles_x * kBackgroundRow;
+                        }
+                        if (one)
+                        {
+                            hipLaunchKernelGGL(blend_backward_fuzzy_long_kernel<kC>, dim3(tiles_x, kFuzzyReplicas), blk, 0, stream, bp,
+                                               accept, dense_max);
+                            hipLaunchKernelGGL(fold_background_rows_kernel, dim3(kFuzzyFoldRows), blk, 0, stream, folds.v[0].rows,
+                                               folds.v[0].num_rows, folds.v[0].folded);
+                        }
+                        else
+                        {
+                            hipLaunchKernelGGL(blend_backward_fuzzy_long_views_kernel<kC>, dim3(tiles_x, kFuzzyReplicas, (unsigned)count),
+                                               blk, 0, stream, views, accept, dense_max);
+                            hipLaunchKernelGGL(fold_background_rows_views_kernel, dim3(kFuzzyFoldRows, (unsigned)count), blk, 0,
+                                               stream, folds);
+                        }
                     }
                 };
                 switch (C)
@@ -1087,45 +1129,41 @@ int vetrast_backward(vetrast_ctx* ctx, const vetrast_backward_args* g, void* str
                     default: launch(std::integral_constant<int, 4>{}); break;
                 }
             }
-            else if (hits == 1)
-                switch (C)
-                {
-                    case 1: hipLaunchKernelGGL((blend_backward_kernel<1, false>), grid, blk, 0, stream, bp); break;
-                    case 2: hipLaunchKernelGGL((blend_backward_kernel<2, false>), grid, blk, 0, stream, bp); break;
-                    case 3: hipLaunchKernelGGL((blend_backward_kernel<3, false>), grid, blk, 0, stream, bp); break;
-                    default: hipLaunchKernelGGL((blend_backward_kernel<4, false>), grid, blk, 0, stream, bp); break;
-                }
             else
-                switch (C)
-                {
-                    case 1: hipLaunchKernelGGL((blend_backward_kernel<1, true>), grid, blk, 0, stream, bp); break;
-                    case 2: hipLaunchKernelGGL((blend_backward_kernel<2, true>), grid, blk, 0, stream, bp); break;
-                    case 3: hipLaunchKernelGGL((blend_backward_kernel<3, true>), grid, blk, 0, stream, bp); break;
-                    default: hipLaunchKernelGGL((blend_backward_kernel<4, true>), grid, blk, 0, stream, bp); break;
-                }
+            {
+                auto launch = [&](auto channels, auto bilinear) {
+                    constexpr int kC         = decltype(channels)::value;
+                    constexpr bool kBilinear = decltype(bilinear)::value;
+                    if (one)
+                        hipLaunchKernelGGL((blend_backward_kernel<kC, kBilinear>), grid, blk, 0, stream, bp);
+                    else
+                        hipLaunchKernelGGL((blend_backward_views_kernel<kC, kBilinear>), grid_views, blk, 0, stream, views);
+                };
+                auto with_channels = [&](auto bilinear) {
+                    switch (C)
+                    {
+                        case 1: launch(std::integral_constant<int, 1>{}, bilinear); break;
+                        case 2: launch(std::integral_constant<int, 2>{}, bilinear); break;
+                        case 3: launch(std::integral_constant<int, 3>{}, bilinear); break;
+                        default: launch(std::integral_constant<int, 4>{}, bilinear); break;
+                    }
+                };
+                if (hits == 1)
+                    with_channels(std::false_type{});
+                else
+                    with_channels(std::true_type{});
+            }
         }
-    };
-    // the per-point part of the views [b, last) of a round: one launch on the caller's stream, behind the round's
-    // per-pixel kernels
-    auto per_point = [&](int b, int last) {
-        const size_t lane      = (size_t)lanes.lane(b);
-        float4* partial        = ws_ptr<float4>(ws, lay.partial_base + lay.lane_scratch_stride * lane);
-        float* background_rows = ws_ptr<float>(ws, lay.background_partial_base + lay.lane_scratch_stride * lane);
-        uint32_t* offsets   = ws_ptr<uint32_t>(ws, lay.offsets_base + lay.offsets_stride * b);
-        uint64_t* fragments = ws_ptr<uint64_t>(ws, lay.fragments_base + lay.fragments_stride * b);
-        (void)offsets, (void)fragments;
-        for (int v = b; v < last; ++v) lanes.after(caller, lanes.stream(v));
-        stream = caller;
         if (N > 0)
         {
             ScopeTimer tm(ctx, stream, VETRAST_SCOPE_BACKWARD_GATHER);
             GatherPass gp;
-            gp.vp                  = make_view_pass(a, lay, ly, b);
-            gp.offsets             = offsets;
-            gp.fragments           = fragments;
-            gp.list_is_cut         = ws_ptr<uint8_t>(ws, lay.cut_flags_base + lay.cut_flags_stride * b);
-            gp.last_key            = ws_ptr<uint64_t>(ws, lay.last_key_base + lay.last_key_stride * b);
-            gp.kept                = ws_ptr<uint32_t>(ws, lay.kept_base + lay.kept_stride * b);
+            gp.vp                  = make_view_pass(a, lay, ly, first);
+            gp.offsets             = ws_ptr<uint32_t>(ws, lay.offsets_base + lay.offsets_stride * first);
+            gp.fragments           = ws_ptr<uint64_t>(ws, lay.fragments_base + lay.fragments_stride * first);
+            gp.list_is_cut         = ws_ptr<uint8_t>(ws, lay.cut_flags_base + lay.cut_flags_stride * first);
+            gp.last_key            = ws_ptr<uint64_t>(ws, lay.last_key_base + lay.last_key_stride * first);
+            gp.kept                = ws_ptr<uint32_t>(ws, lay.kept_base + lay.kept_stride * first);
             gp.partial             = partial;
             gp.grad_texture        = g->grad_texture;
             gp.grad_confidence     = g->grad_confidence;
@@ -1135,7 +1173,7 @@ int vetrast_backward(vetrast_ctx* ctx, const vetrast_backward_args* g, void* str
             gp.need_point_gradient = want_image_gradient ? 1 : 0;
             gp.camera_partial      = want_camera ? camera_rows : nullptr;
             gp.point_major_records = point_major_records;
-            gp.view_count          = last - b;
+            gp.view_count          = count;
             gp.dropout_stride      = (size_t)N;
             gp.flags_stride        = lay.cut_flags_stride;
             gp.last_key_stride     = lay.last_key_stride / sizeof(uint64_t);
@@ -1143,18 +1181,17 @@ int vetrast_backward(vetrast_ctx* ctx, const vetrast_backward_args* g, void* str
             gp.partial_stride      = lay.lane_scratch_stride / sizeof(float4);
             gp.background_rows_stride = lay.lane_scratch_stride / sizeof(float);
             gp.camera_partial_stride  = camera_rows_bytes(N) / sizeof(double);
-            gp.accumulate          = (add_to_rows || b > 0) ? 1 : 0;
+            gp.accumulate          = (add_to_rows || first > 0) ? 1 : 0;
             gp.background_rows       = background_rows;
             // (with the folded rows of the FUZZY_BLEND kernel that takes a wave per list, where it ran)
-            gp.num_background_rows   = (int)tile_grid(tiles) + (fuzzy_long ? kFuzzyFoldRows : 0);
+            gp.num_background_rows   = background_rows_count;
             gp.grad_background       = g->grad_background;
             gp.add_leak = (p.quirk_background_confidence_leak && !p.use_environment_map && hits == 1 &&
                            p.render_mode != VETRAST_RENDER_FUZZY_BLEND)
                               ? 1
                               : 0;
-            gp.background_accumulate = b > 0 ? 1 : 0;
-            gp.packed                = a->packed_descriptors ? reinterpret_cast<const float4*>(a->packed_descriptors)
-                                                             : ws_ptr<float4>(ws, lay.packed_base);
+            gp.background_accumulate = first > 0 ? 1 : 0;
+            gp.packed                = packed;
             gp.texture_raw           = a->texture;
             gp.background_raw        = a->background;
             gp.confidence_activation = p.confidence_activation;
@@ -1190,41 +1227,24 @@ int vetrast_backward(vetrast_ctx* ctx, const vetrast_backward_args* g, void* str
             else
                 with_channels(std::integral_constant<int, 4>{});
         }
-        for (int v = b; want_camera && v < last; ++v)
+        for (int v = first; want_camera && v < last; ++v)
         {
             ScopeTimer tm(ctx, stream, VETRAST_SCOPE_BACKWARD_GATHER);
             hipLaunchKernelGGL(reduce_camera_kernel, dim3(1), dim3(kBlock), 0, stream,
-                               camera_rows + (size_t)(v - b) * (camera_rows_bytes(N) / sizeof(double)), grid_for(N),
+                               camera_rows + (size_t)(v - first) * (camera_rows_bytes(N) / sizeof(double)), grid_for(N),
                                a->views[v].image_index, a->views[v].camera_index, p.K_gradient_factor, g->grad_pose,
                                g->grad_pose_count, g->grad_intrinsics, g->grad_intrinsics_count,
                                hits == 1 ? 1.f / 1024.f : 1.f, p.allow_distortion, p.distortion_gradient_factor);
         }
-        for (int v = b; N == 0 && v < last; ++v)
+        for (int v = first; N == 0 && v < last; ++v)
         {
             ScopeTimer tm(ctx, stream, VETRAST_SCOPE_BACKWARD_GATHER);
             hipLaunchKernelGGL(reduce_background_kernel, dim3(1), dim3(kReduceBlock), 0, stream,
-                               background_rows + (size_t)(v - b) * (lay.lane_scratch_stride / sizeof(float)),
-                               (int)(tile_grid(tiles)) + (fuzzy_long ? kFuzzyFoldRows : 0), C, g->grad_background, g->grad_confidence,
-                               0, v > 0 ? 1 : 0, p.texture_abs ? a->background : nullptr);
+                               background_rows + (size_t)(v - first) * (lay.lane_scratch_stride / sizeof(float)),
+                               background_rows_count, C, g->grad_background, g->grad_confidence, 0, v > 0 ? 1 : 0,
+                               p.texture_abs ? a->background : nullptr);
         }
-        if (lanes.lanes > 1 && last < B)
-        {
-            // the next round's per-pixel kernels overwrite the lanes' record arrays
-            const hipEvent_t e = lanes.mark(caller);
-            for (int v = b; v < last; ++v) gathered[(size_t)v] = e;
-        }
-    };
-    // Views in rounds of one per lane: first the per-pixel kernels of the round (side by side), then its per-point
-    // kernels. (Enqueued in this order, no per-pixel kernel waits in a hardware queue behind a per-point kernel of
-    // another view.)
-    for (int first = 0; first < B; first += lanes.lanes)
-    {
-        const int last = std::min(B, first + lanes.lanes);
-        for (int b = first; b < last; ++b) per_pixel(b);
-        per_point(first, last);
     }
-    stream = caller;  // (every lane's last kernel has been waited for above)
-    VET_HIP(ctx, lanes.err);
     if (g->grad_points && p.point_gradient_normalization != 0 && N > 0)
     {
         ScopeTimer tm(ctx, stream, VETRAST_SCOPE_BACKWARD_POST);
