@@ -498,15 +498,10 @@ def main():
     for k in ("PREPARE", "PACK", "SCAN", "BACKWARD_PREPARE", "BACKWARD_POST"):
         if r["per_step_ms"].get(k, 0.0) > 0:
             kernels[k] = {"ms": round(r["per_step_ms"][k], 5), "alg_MB": 0.0, "GBps": None, "frac": None}
-    if B > 1:
-        # the views of a call run side by side: a scope's launches overlap those of other scopes and views, so its time
-        # says how long its kernels were under way, not what share of the step they are, and no rate follows from it
-        for k in kernels:
-            kernels[k]["GBps"] = kernels[k]["frac"] = None
     dominant = max(alg.keys(), key=lambda k: r["per_step_ms"].get(k, 0.0))
     dom_ms = r["per_launch_ms"][dominant]
     dom_launches = max(1.0, r["launches_per_step"].get(dominant, 1.0))
-    dom_bytes = alg[dominant] / dom_launches  # one launch handles one view
+    dom_bytes = alg[dominant] / dom_launches  # (one launch takes up to four views of a call)
     achieved = dom_bytes / 1e6 / dom_ms if dom_ms > 0 else 0.0
     total_alg = sum(alg.values())
 
@@ -552,9 +547,6 @@ def main():
         },
         "forward_ms": round(ms_fwd, 5),
         "backward_ms": round(ms_step - ms_fwd, 5) if backward else None,
-        "kernels_note": ("the views of the call run side by side (up to four at a time): per-scope times overlap and add "
-                         "up to more than the step; the roofline object's launch time is that of a kernel sharing the "
-                         "chip with the other views' kernels") if B > 1 else None,
         "step_algorithmic_MB": round(total_alg / 1e6, 3),
         "step_GBps": round(total_alg / 1e6 / ms_step, 1),
         "step_frac_of_hbm_peak": round(total_alg / 1e6 / ms_step / HBM_PEAK_GBS, 4),

@@ -6,12 +6,8 @@
  * on; all `host` pointers are ordinary host memory that only has to stay valid for the duration of the call.
  * Every entry point returns 0 on success or a negative vetrast_status, never aborts, never allocates device
  * memory behind the caller's back (the caller owns inputs, outputs and the workspace) and, unless stated
- * otherwise, only enqueues work that is ordered like work on the given stream (pass the hipStream_t as `void*`,
- * NULL = default stream): whatever was enqueued on that stream before the call comes first, whatever is enqueued
- * after it sees the call's results. vetrast_forward and vetrast_backward with more than one view run a part of that
- * work on up to three streams the library keeps per device (default priority, shared by all contexts) that wait for
- * the given stream at the start of the call and that the given stream waits for at its end, by events; a call that
- * is captured into a HIP graph takes them into the capture and out again. A context serves one host thread at a time.
+ * otherwise, only enqueues work on the given stream (pass the hipStream_t as `void*`, NULL = default stream).
+ * A context serves one host thread at a time.
  *
  * The reference has no C ABI; its seam is the libtorch function
  *   std::vector<torch::Tensor> BlendPointCloud(NeuralRenderInfo*)          src/lib/rendering/PointRenderer.h:53
@@ -213,11 +209,10 @@ typedef struct vetrast_workspace_layout
     size_t projected_base, projected_stride; /* per view, float [N][2], BILINEAR_BLEND only (stride 0 otherwise): image
                                                 position of every visible point at layer 0, from which the blend and its
                                                 backward pass form the bilinear weights */
-    /* A call with several views runs up to view_lanes = min(num_views, 4) of them side by side (view b on lane
-     * b % view_lanes, lane 0 on the caller's stream, the others on streams of the library's own between a fork from
-     * and a join with the caller's stream), so the scratch that used to be shared by all views exists once per lane: lane k's copy of binned,
-     * primary and scan_partials lies k * the stride behind the base, its copy of the log / slots / partial /
-     * background_partial block k * lane_scratch_stride behind theirs. */
+    /* A call with several views takes them view_lanes = min(num_views, 4) at a time: every kernel of the call is one
+     * launch for the views of such a round (view b of the call on lane b % view_lanes), so the scratch that one view
+     * needs exists once per lane: lane k's copy of binned, primary and scan_partials lies k * the stride behind the
+     * base, its copy of the log / slots / partial / background_partial block k * lane_scratch_stride behind theirs. */
     int32_t view_lanes;
     int32_t reserved2;
     size_t binned_stride, primary_stride, scan_partials_stride, lane_scratch_stride;

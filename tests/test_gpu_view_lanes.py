@@ -1,8 +1,8 @@
-"""GPU tests of calls with several views, whose views the library runs side by side.
+"""GPU tests of calls with several views, whose views share the library's launches.
 
-Up to four views of a call run at the same time, each on a lane (a stream of the library's own, forked from and joined
-with the caller's stream, with its own copy of the scratch the views used to share); further views follow in rounds;
-the per-point backward kernel takes a whole round in one launch. None of that may show in the results: the cases here
+Up to four views of a call go through every kernel together: one launch per kernel for such a round, each view on a lane
+(its own copy of the scratch that one view needs); further views follow in rounds; the per-point backward kernel adds
+a round's views up inside its threads. None of that may show in the results: the cases here
 hold calls of 2 to 9 views (short rounds, exact rounds, several rounds) against the oracle in all three render modes
 with camera gradients, drop-out masks and an index indirection, compare a call of many views with the same views given
 one per call, capture such a call in a HIP graph and replay it, and run two contexts on two streams at once.
@@ -130,9 +130,8 @@ def test_a_call_of_many_views_equals_its_views_one_by_one(rasterizer):
 
 @pytest.mark.parametrize("render_mode", [abi.RENDER_FULL_BLEND, abi.RENDER_BILINEAR_BLEND])
 def test_a_call_of_several_rounds_replays_from_a_hip_graph(render_mode, rasterizer):
-    """Six views (a round of four and a round of two) with camera gradients, captured on a side stream: the lanes'
-    streams join the capture through the events that order them and leave it again before it ends; every replay gives
-    the bits of the eager call, with eager calls in between."""
+    """Six views (a round of four and a round of two) with camera gradients, captured on a side stream: every replay
+    gives the bits of the eager call, with eager calls in between."""
     scene = _scene(6, 95, num_points=20_000)
     params = make_params(scene, need_point_gradient=1, render_mode=render_mode)
     dev = DeviceScene(scene)
@@ -165,13 +164,13 @@ def test_a_call_of_several_rounds_replays_from_a_hip_graph(render_mode, rasteriz
             assert torch.equal(a, b), f"replay {replay}"
         for k, v in want_g.items():
             assert torch.equal(eager_g[k], v), (k, replay)
-        again = rasterizer.forward(dev, params)  # eager work between replays, through the same lanes
+        again = rasterizer.forward(dev, params)  # eager work between replays, in the same workspace
         torch.cuda.synchronize()
         assert torch.equal(again.out[0], want_out[0])
 
 
 def test_two_contexts_with_lanes_on_two_streams(oracle):
-    """Two contexts, each with lanes of its own, issue calls of five views on two caller streams at the same time."""
+    """Two contexts issue calls of five views on two caller streams at the same time (each call has its own workspace)."""
     scenes = [_scene(5, 97), _scene(5, 98)]
     rasts = [Rasterizer(), Rasterizer()]
     streams = [torch.cuda.Stream(), torch.cuda.Stream()]

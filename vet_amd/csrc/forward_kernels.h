@@ -340,18 +340,13 @@ __device__ __forceinline__ void store_record(const ScatterTargets& t, const Laye
 // HITS = 1: a point lands in the pixel it rounds to (FULL_BLEND); HITS = 4: in the 2x2 pixels around it
 // (BILINEAR_BLEND), each of which is a fragment of its own with its own bin; the low key word is then
 // point id << 2 | corner.
+// This is the part of the pass behind the projection: thread `slot` has point i, which is `visible` at p in this view.
 template <int HITS>
-__device__ __forceinline__ void bin_scatter(const ViewPass& a, uint32_t* __restrict__ bin_counts,
-                                            const ScatterTargets& out, const PackJob& pack)
+__device__ __forceinline__ void scatter_projected(const ViewPass& a, uint32_t* __restrict__ bin_counts,
+                                                  const ScatterTargets& out, const PackJob& pack, int slot, int i, bool visible,
+                                                  const Projected& p)
 {
-    const int slot = blockIdx.x * blockDim.x + threadIdx.x;
     const int lane = threadIdx.x & (kWave - 1);
-    // the point this thread takes: the caller's processing order, if there is one (neighbours in a wave should be
-    // neighbours in space; ids in the records are the caller's either way)
-    const int i = (a.point_order != nullptr && slot < a.N) ? a.point_order[slot] : slot;
-    Projected p;
-    p.ipx = p.ipy = p.z = p.radius = 0.f;
-    const bool visible = (uint32_t)i < (uint32_t)a.N && !point_is_skipped(a, i) && project_point(*a.view, a.position[i], p);
     float ipx = visible ? p.ipx : 0.f, ipy = visible ? p.ipy : 0.f, radius = visible ? p.radius : 0.f;
     const uint32_t depth_bits = __float_as_uint(p.z);
     // A position further outside the image than the reach of the coarsest layer's border pixels hits no pixel of any
@@ -492,6 +487,21 @@ __device__ __forceinline__ void bin_scatter(const ViewPass& a, uint32_t* __restr
     if (packs) store_packed_row(pack, slot, row, row_confidence);
 }
 
+// The pass for one view: fetch, projection, and the above.
+template <int HITS>
+__device__ __forceinline__ void bin_scatter(const ViewPass& a, uint32_t* __restrict__ bin_counts,
+                                            const ScatterTargets& out, const PackJob& pack)
+{
+    const int slot = blockIdx.x * blockDim.x + threadIdx.x;
+    // the point this thread takes: the caller's processing order, if there is one (neighbours in a wave should be
+    // neighbours in space; ids in the records are the caller's either way)
+    const int i = (a.point_order != nullptr && slot < a.N) ? a.point_order[slot] : slot;
+    Projected p;
+    p.ipx = p.ipy = p.z = p.radius = 0.f;
+    const bool visible = (uint32_t)i < (uint32_t)a.N && !point_is_skipped(a, i) && project_point(*a.view, a.position[i], p);
+    scatter_projected<HITS>(a, bin_counts, out, pack, slot, i, visible, p);
+}
+
 template <int HITS>
 __global__ void __launch_bounds__(kBlock) bin_scatter_kernel(ViewPass a, uint32_t* __restrict__ bin_counts,
                                                               ScatterTargets out, PackJob pack)
@@ -507,9 +517,10 @@ struct ScatterArgs
     PackJob pack;
 };
 
-// (A thread that took its point through the views of a round one after the other would read the point arrays once
-// instead of once per view; measured, that is slower: the pass waits for its atomics, not for memory, and fewer,
-// longer threads hide less of that.)
+// The views of a round, one per blockIdx.y. (One pass over the points for all views of the round, each thread taking
+// its point through one view after the other, reads the point arrays once instead of once per view; measured on four
+// training crops it is slower by a fifth to a half, also with the fetch shared and only the projection repeated: the
+// pass waits for its atomics, not for memory, and more, shorter threads hide more of that.)
 template <int HITS>
 __global__ void __launch_bounds__(kBlock) bin_scatter_views_kernel(PerView<ScatterArgs> views)
 {

@@ -35,10 +35,6 @@ struct vetrast_ctx
     float acc_ms[VETRAST_SCOPE_COUNT_]      = {};
     int32_t acc_launches[VETRAST_SCOPE_COUNT_] = {};
     char* lift_scratch = nullptr;  // this device's copy of the file-scope scratch array (vetrast_lift_error_static)
-    // Calls with several views run them side by side on these streams (default priority; shared by all contexts of the
-    // device), forked from and joined with the caller's stream by events; see ViewLanes below.
-    hipStream_t lane_stream[kViewLanes] = {nullptr, nullptr, nullptr, nullptr};  // the device's lane streams; [0] stays unused
-    std::vector<hipEvent_t> sync_events;  // ordering events (no timing), reused from call to call
 };
 
 namespace
@@ -333,35 +329,6 @@ constexpr int kMaxDevices = 64;
 std::mutex g_scratch_mutex;
 char* g_scratch_ptr[kMaxDevices] = {};
 
-// The lane streams (see ViewLanes): three per device for the whole process, made when the first context on the device
-// is, and kept until the process ends. All contexts share them: a process has four hardware queues by default, streams
-// are dealt to them in turn, and lane streams of its own for every context would soon sit on the queue of the
-// caller's stream or of each other, which puts the views of a call back in line (measured: the batch of four training
-// crops 0.59 ms with the lanes on queues of their own, 0.71 ms with a second context's lanes). Calls of two contexts
-// that are under way at the same time share the lanes correctly (events order each call's own work).
-std::mutex g_lane_mutex;
-hipStream_t g_lane_stream[kMaxDevices][kViewLanes] = {};
-
-hipError_t lane_streams_of_device(int device, hipStream_t (&out)[kViewLanes])
-{
-    if (device < 0 || device >= kMaxDevices) return hipErrorInvalidDevice;
-    std::lock_guard<std::mutex> lock(g_lane_mutex);
-    for (int k = 1; k < kViewLanes; ++k)  // (lane 0 is the caller's stream)
-    {
-        if (!g_lane_stream[device][k])
-        {
-            hipError_t e = hipStreamCreateWithFlags(&g_lane_stream[device][k], hipStreamNonBlocking);
-            if (e != hipSuccess)
-            {
-                g_lane_stream[device][k] = nullptr;
-                return e;
-            }
-        }
-        out[k] = g_lane_stream[device][k];
-    }
-    return hipSuccess;
-}
-
 // Address of the scratch array on `device`, which must be the current device. hipSuccess and a non-null pointer on
 // success.
 hipError_t scratch_of_device(int device, char** out)
@@ -475,25 +442,6 @@ int vetrast_create(vetrast_ctx** out_ctx)
         vetrast_destroy(ctx);
         return VETRAST_ERR_HIP;
     }
-    // (lane 0 is the caller's stream; three more, so that a call stays within the four hardware queues a process has
-    // by default)
-    if (lane_streams_of_device(ctx->device, ctx->lane_stream) != hipSuccess)
-    {
-        vetrast_destroy(ctx);
-        return VETRAST_ERR_HIP;
-    }
-    // ordering events for calls with several views, made here so that a call that is being captured into a graph
-    // creates nothing (a call of up to some forty views gets by with these; more are made when needed)
-    for (int k = 0; k < 64; ++k)
-    {
-        hipEvent_t ev = nullptr;
-        if (hipEventCreateWithFlags(&ev, hipEventDisableTiming) != hipSuccess)
-        {
-            vetrast_destroy(ctx);
-            return VETRAST_ERR_HIP;
-        }
-        ctx->sync_events.push_back(ev);
-    }
     *out_ctx = ctx;
     return VETRAST_OK;
 }
@@ -501,7 +449,6 @@ int vetrast_create(vetrast_ctx** out_ctx)
 void vetrast_destroy(vetrast_ctx* ctx)
 {
     if (!ctx) return;
-    for (auto e : ctx->sync_events) (void)hipEventDestroy(e);
     for (auto& s : ctx->spans)
     {
         (void)hipEventDestroy(s.start);
@@ -642,65 +589,18 @@ size_t vetrast_forward_workspace_bytes(int32_t N, int32_t B, int32_t L, int32_t 
 
 namespace
 {
-// The views of one call side by side. View b runs on lane b % lanes: a stream of the context's own that has waited
-// for the caller's stream (fork) and that the caller's stream waits for in the end (join), ordered by events, so the
-// call behaves like one stream's worth of work to the caller and can be captured into a graph with it. Kernels of
-// small views (training crops) leave most of the chip idle on their own and are chains of dependent launches; four of
-// them at a time fill it. With one view everything stays on the caller's stream.
-struct ViewLanes
+// Whether the caller expects a view of the call to see a small part of the cloud: a third of the fragments every
+// point in every layer would leave, or less. False where it has not said (expected_fragments).
+bool views_see_little(const vetrast_params& p, int N, int hits)
 {
-    vetrast_ctx* ctx;
-    hipStream_t main;
-    int lanes;
-    size_t used = 0;
-    hipError_t err = hipSuccess;
-
-    ViewLanes(vetrast_ctx* c, hipStream_t m, int n) : ctx(c), main(m), lanes(n > 1 ? n : 1) {}
-    void check(hipError_t e)
+    double expected = 0.0;
+    for (int l = 0; l < p.num_layers; ++l)
     {
-        if (e != hipSuccess && err == hipSuccess) err = e;
+        if (!(p.expected_fragments[l] > 0.f)) return false;
+        expected += p.expected_fragments[l];
     }
-    hipEvent_t event()
-    {
-        if (used == ctx->sync_events.size())
-        {
-            hipEvent_t e = nullptr;
-            check(hipEventCreateWithFlags(&e, hipEventDisableTiming));
-            if (!e) return nullptr;
-            ctx->sync_events.push_back(e);
-        }
-        return ctx->sync_events[used++];
-    }
-    // lane 0 is the caller's stream itself: its views need no hand-over, and the call stays within four streams
-    hipStream_t stream(int b) const { return (lanes > 1 && b % lanes != 0) ? ctx->lane_stream[b % lanes] : main; }
-    int lane(int b) const { return lanes > 1 ? b % lanes : 0; }
-    // an event that stands for everything enqueued on `s` so far
-    hipEvent_t mark(hipStream_t s)
-    {
-        hipEvent_t e = event();
-        if (e) check(hipEventRecord(e, s));
-        return e;
-    }
-    void wait(hipStream_t waiter, hipEvent_t e)
-    {
-        if (e) check(hipStreamWaitEvent(waiter, e, 0));
-    }
-    void after(hipStream_t waiter, hipStream_t done)
-    {
-        if (waiter != done) wait(waiter, mark(done));
-    }
-    void fork()
-    {
-        if (lanes < 2) return;
-        hipEvent_t e = mark(main);
-        for (int k = 1; k < lanes; ++k) wait(ctx->lane_stream[k], e);
-    }
-    void join()
-    {
-        if (lanes < 2) return;
-        for (int k = 1; k < lanes; ++k) after(main, ctx->lane_stream[k]);
-    }
-};
+    return expected < (double)N * hits * p.num_layers / 3.0;
+}
 }  // namespace
 
 int vetrast_forward(vetrast_ctx* ctx, const vetrast_forward_args* a, void* stream_)
@@ -1010,19 +910,8 @@ int vetrast_backward(vetrast_ctx* ctx, const vetrast_backward_args* g, void* str
     const bool fuzzy_long  = p.render_mode == VETRAST_RENDER_FUZZY_BLEND &&
                             (p.debug_max_list_length <= 0 || p.debug_max_list_length > kFuzzyDense);
     // Layout of the gradient records (gradient_record): point after point where the caller expects the views to see a
-    // small part of the cloud (a third of the fragments every point in every layer would leave, or less), layer after
-    // layer otherwise and where nothing is known.
-    int point_major_records = 0;
-    {
-        double expected = 0.0;
-        bool known      = true;
-        for (int l = 0; l < L; ++l)
-        {
-            known = known && p.expected_fragments[l] > 0.f;
-            expected += p.expected_fragments[l];
-        }
-        point_major_records = (known && expected < (double)N * hits * L / 3.0) ? 1 : 0;
-    }
+    // small part of the cloud, layer after layer otherwise and where nothing is known.
+    const int point_major_records = views_see_little(p, N, hits) ? 1 : 0;
     // Views in rounds of up to view_lanes: the per-pixel kernel takes the views of a round in one launch, each into its
     // lane's record array, and the per-point kernel behind it reads them all, again in one launch (the views add to
     // the same gradient rows).
