@@ -97,6 +97,47 @@ def test_hints_that_switch_the_record_layout_change_nothing(render_mode, num_vie
         assert torch.equal(results[0][1][key], results[2][1][key]), key
 
 
+@pytest.mark.parametrize("render_mode", [abi.RENDER_FULL_BLEND, abi.RENDER_BILINEAR_BLEND])
+def test_views_that_see_little_interleave_the_rows_they_need(render_mode, rasterizer, oracle):
+    """With hints that say "a small part of the cloud" (and neither texture index nor processing order) every view's
+    scatter pass interleaves the descriptor rows of the points it sees instead of the first view's taking all rows.
+    Five crops (two rounds) into a workspace filled with NaN bit patterns beforehand: whatever row a fragment or a
+    gradient needs has been written by this call; rows of points that no view sees stay untouched."""
+    scene = synthetic.tiny_scene(num_points=6000, w=96, h=64, num_layers=3, K=8, seed=99)
+    scene.views = [synthetic.ViewSpec(32, 24, image_index=0, crop_transform=(1.0, 1.0, -float(ox), -float(oy), 0.0))
+                   for (ox, oy) in ((0, 0), (40, 10), (64, 40), (20, 30), (50, 0))]
+    params = make_params(scene, need_point_gradient=1, render_mode=render_mode)
+    for l in range(scene.num_layers):
+        params.expected_fragments[l] = 40.0
+    dev = DeviceScene(scene)
+    first = rasterizer.forward(dev, params)  # (for the size of the workspace)
+    workspace = torch.full_like(first.workspace, 0xFF)
+    res = rasterizer.forward(dev, params, workspace=workspace)
+    go = scene.grad_out()
+    got = rasterizer.backward(res, [torch.from_numpy(g).cuda() for g in go])
+    torch.cuda.synchronize()
+    assert rasterizer.check_device_flags(res) == 0
+    ref = oracle.forward(scene, params)
+    want = oracle.backward(ref, go)
+    for l in range(scene.num_layers):
+        np.testing.assert_array_equal(res.out[l].cpu().numpy(), ref.out[l])
+    for key in ("texture", "confidence", "background", "points"):
+        assert max_rel_err(got[key].cpu().numpy(), want[key]) <= 1e-4, key
+    rows = res.workspace[res.layout.packed_base:res.layout.packed_base + 32 * scene.num_points].view(torch.float32)
+    rows = rows.reshape(scene.num_points, 8).cpu().numpy()
+    written = ~np.isnan(rows[:, 0])
+    assert 0 < written.sum() < scene.num_points  # some rows, not all of them
+    np.testing.assert_array_equal(rows[written, :scene.num_channels], scene.texture.T[written])
+    seen = np.zeros(scene.num_points, dtype=bool)
+    for b in range(len(scene.views)):
+        frag = res.fragments(b)
+        ids = (frag & np.uint64(0xFFFFFFFF)).astype(np.int64)
+        if render_mode == abi.RENDER_BILINEAR_BLEND:
+            ids >>= 2
+        seen[ids[: int(res.offsets(b)[-1])]] = True
+    assert not (seen & ~written).any()
+
+
 def test_a_call_of_many_views_equals_its_views_one_by_one(rasterizer):
     """Seven views in one call against seven calls of one view: images and lists bit for bit, and the gradients of the
     big call equal the sum of the single calls' gradients to rounding (the rows are added in view order either way)."""

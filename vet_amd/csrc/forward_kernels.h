@@ -520,7 +520,9 @@ struct ScatterArgs
 // The views of a round, one per blockIdx.y. (One pass over the points for all views of the round, each thread taking
 // its point through one view after the other, reads the point arrays once instead of once per view; measured on four
 // training crops it is slower by a fifth to a half, also with the fetch shared and only the projection repeated: the
-// pass waits for its atomics, not for memory, and more, shorter threads hide more of that.)
+// pass waits for its atomics, not for memory, and more, shorter threads hide more of that. Workgroups of the views
+// taking turns, instead of all of one view before those of the next, is slower as well, by a tenth for crops and by
+// half for full frames.)
 template <int HITS>
 __global__ void __launch_bounds__(kBlock) bin_scatter_views_kernel(PerView<ScatterArgs> views)
 {

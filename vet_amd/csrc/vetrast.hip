@@ -655,6 +655,12 @@ int vetrast_forward(vetrast_ctx* ctx, const vetrast_forward_args* a, void* strea
     // scratch of its lane).
     const int lanes          = std::max(1, lay.view_lanes);
     const bool scan_and_move = bins + 1 <= (uint32_t)kScanMoveMax;
+    // The descriptor interleave rides on the scatter pass of the first view, which takes every row; or, where row,
+    // point and thread are the same number (no texture index, no processing order), on that of every view, each for
+    // the rows of the points it sees (only fragments ever read a row; views that see the same point write the same
+    // bytes): with one view, and with several where the caller expects each to see little of the cloud.
+    const bool rows_of_visible_points =
+        a->index == nullptr && a->point_order == nullptr && (B == 1 || views_see_little(p, N, hits));
     for (int first = 0; first < B; first += lanes)
     {
         const int last = std::min(B, first + lanes), count = last - first;
@@ -679,13 +685,13 @@ int vetrast_forward(vetrast_ctx* ctx, const vetrast_forward_args* a, void* strea
             PackJob& pack              = sc.pack;
             pack.texture               = a->texture;
             pack.confidence            = a->confidence;
-            pack.packed                = (b == 0 && own_pack) ? packed : nullptr;
+            pack.packed                = (own_pack && (b == 0 || rows_of_visible_points)) ? packed : nullptr;
             pack.N                     = N;
             pack.C                     = C;
             pack.confidence_activation = p.confidence_activation;
             pack.confidence_scale      = p.confidence_scale;
             pack.texture_abs           = p.texture_abs;
-            pack.visible_only          = (B == 1 && a->index == nullptr && a->point_order == nullptr) ? 1 : 0;
+            pack.visible_only          = rows_of_visible_points ? 1 : 0;
 
             // Where the bins of a view are few enough, one launch scans their counts and files the logged records (the
             // scan lands behind the counts); otherwise the scan runs in place and the move kernel follows.
