@@ -514,7 +514,7 @@ int vetrast_workspace_layout_for_mode(int32_t N, int32_t B, int32_t L, int32_t w
     at += lay->bin_counts_stride * B;
     lay->log_cursor_base = at;  // right behind the bin counters: one zero-fill covers both
     at += log_cursor_bytes(B);
-    // scratch that exists once per lane (views that run side by side), see vetrast_workspace_layout::view_lanes
+    // scratch that exists once per lane (the views that share a launch), see vetrast_workspace_layout::view_lanes
     const int lanes            = std::min(B, kViewLanes);
     lay->view_lanes            = lanes;
     lay->scan_partials_base    = at;
