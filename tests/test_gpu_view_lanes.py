@@ -97,6 +97,31 @@ def test_hints_that_switch_the_record_layout_change_nothing(render_mode, num_vie
         assert torch.equal(results[0][1][key], results[2][1][key]), key
 
 
+@pytest.mark.parametrize("max_list_length", [-1, 48])
+def test_uncut_fuzzy_lists_of_several_views(max_list_length, rasterizer, oracle):
+    """FUZZY_BLEND without a cut (or a cut beyond what the dense backward kernel takes): lists of more than 32 fragments
+    go to the kernel that gives a wave to each list, whose grid already uses y for its replicas (the view is z there),
+    and the replicas' background rows are folded per view. Five views = a round of four and a round of one."""
+    scene = _scene(5, 70, num_points=20_000)
+    scene.max_list_length = max_list_length
+    params = make_params(scene, need_point_gradient=1, render_mode=abi.RENDER_FUZZY_BLEND, depth_accept_blend=0.05)
+    assert params.debug_max_list_length == max_list_length
+    res = rasterizer.forward(DeviceScene(scene), params)
+    go = scene.grad_out()
+    got = rasterizer.backward(res, [torch.from_numpy(g).cuda() for g in go], want_cameras=True)
+    torch.cuda.synchronize()
+    assert rasterizer.check_device_flags(res) == 0
+    ref = oracle.forward(scene, params)
+    lengths = np.diff(ref.offsets[4].astype(np.int64))
+    assert lengths.max() > 64  # long lists exist, in the last view too
+    want = oracle.backward(ref, go, want_cameras=True)
+    for l in range(scene.num_layers):
+        np.testing.assert_array_equal(res.out[l].cpu().numpy(), ref.out[l])
+    for key in ("texture", "confidence", "background", "points", "pose", "intrinsics"):
+        err = max_rel_err(got[key].cpu().numpy(), want[key])
+        assert err <= (3e-4 if key in ("pose", "intrinsics") else 1e-4), (key, err)
+
+
 @pytest.mark.parametrize("render_mode", [abi.RENDER_FULL_BLEND, abi.RENDER_BILINEAR_BLEND])
 def test_views_that_see_little_interleave_the_rows_they_need(render_mode, rasterizer, oracle):
     """With hints that say "a small part of the cloud" (and neither texture index nor processing order) every view's
