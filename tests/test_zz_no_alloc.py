@@ -3,6 +3,8 @@ against vetrast_lift_error with a caller-owned workspace: per-cell pixel counts 
 relative (a cell's float terms are summed in double and rounded once on both paths; for cells on the shared path only
 the order of the double additions differs between two runs). Two calls in a row share the one scratch array, the second
 on a smaller grid, so stale queue entries, sums and prefix sums of the first call would show."""
+import gc
+
 import numpy as np
 import pytest
 import torch
@@ -33,11 +35,15 @@ def _both(rasterizer, scene, mn, ln, img):
     got_v, got_c = dev(v0), dev(c0)
     # Nothing is allocated: neither through torch's caching allocator nor straight from the device (free bytes as
     # hipMemGetInfo reports them, which a hipMalloc inside the library would lower).
+    # (Tensors of earlier tests that the garbage collector frees meanwhile lower the bytes in use, so the check is on
+    # the allocator's count of allocations, which only ever goes up.)
+    gc.collect()
     torch.cuda.synchronize()
-    before, free_before = torch.cuda.memory_allocated(), torch.cuda.mem_get_info()[0]
+    allocations = lambda: torch.cuda.memory_stats()["allocation.all.allocated"]
+    before, free_before = allocations(), torch.cuda.mem_get_info()[0]
     ret = rasterizer.lift_error(d_mn, d_ln, got_v, got_c, scene.views[0], d_pose, d_intr, d_img, static_scratch=True)
     torch.cuda.synchronize()
-    assert ret is None and torch.cuda.memory_allocated() == before
+    assert ret is None and allocations() == before, "a tensor was allocated during the call"
     assert torch.cuda.mem_get_info()[0] >= free_before, "the device lost free memory during the call"
     queued = int(ws[abi.LIFT_QUEUE_LENGTH_OFFSET:abi.LIFT_QUEUE_LENGTH_OFFSET + 4].view(torch.int32).item())
     return got_v.cpu().numpy(), got_c.cpu().numpy(), want_v.cpu().numpy(), want_c.cpu().numpy(), c0, queued

@@ -665,9 +665,9 @@ int vetrast_forward(vetrast_ctx* ctx, const vetrast_forward_args* a, void* strea
     {
         const int last = std::min(B, first + lanes), count = last - first;
         const bool one = count == 1;
-        PerView<ScatterArgs> scatter;
-        PerView<ScanArgs> scan;
-        PerView<BuildPass> build;
+        PerView<ScatterArgs> scatter{};
+        PerView<ScanArgs> scan{};
+        PerView<BuildPass> build{};
         for (int b = first; b < last; ++b)
         {
             const size_t lane = (size_t)(b - first);
@@ -932,7 +932,7 @@ int vetrast_backward(vetrast_ctx* ctx, const vetrast_backward_args* g, void* str
         float* background_rows = ws_ptr<float>(ws, lay.background_partial_base);
         {
             ScopeTimer tm(ctx, stream, VETRAST_SCOPE_BACKWARD_BLEND);
-            PerView<BackwardPass> views;
+            PerView<BackwardPass> views{};
             for (int b = first; b < last; ++b)
             {
                 const size_t lane = (size_t)(b - first);
@@ -993,7 +993,7 @@ int vetrast_backward(vetrast_ctx* ctx, const vetrast_backward_args* g, void* str
                     {
                         const uint32_t dense_max = (uint32_t)(wide ? kFuzzyDense : kFuzzyNarrow);
                         // the rows of replicas 1 .. into kFuzzyFoldRows rows behind the per-workgroup ones
-                        PerView<FoldArgs> folds;
+                        PerView<FoldArgs> folds{};
                         for (int k = 0; k < count; ++k)
                         {
                             folds.v[k].rows     = views.v[k].background_partial + ((size_t)kFuzzyFoldRows + tiles_x) * kBackgroundRow;
