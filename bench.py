@@ -547,6 +547,9 @@ def main():
         },
         "forward_ms": round(ms_fwd, 5),
         "backward_ms": round(ms_step - ms_fwd, 5) if backward else None,
+        "kernels_note": ("the byte model counts every view's pass over the point arrays; the per-point backward kernel "
+                         "takes the (up to four) views of a launch in one pass over them, so its rate against the model can "
+                         "exceed what the memory delivers") if B > 1 else None,
         "step_algorithmic_MB": round(total_alg / 1e6, 3),
         "step_GBps": round(total_alg / 1e6 / ms_step, 1),
         "step_frac_of_hbm_peak": round(total_alg / 1e6 / ms_step / HBM_PEAK_GBS, 4),
