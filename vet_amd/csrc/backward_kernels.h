@@ -227,22 +227,41 @@ __device__ __forceinline__ void blend_backward(const BackwardPass& a)
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 
-        for (int k0 = (int)((total - 1) / kWave) * kWave; total > 0 && k0 >= 0; k0 -= kWave)
-        {
+        // BILINEAR_BLEND asks for the key and the transmittance of a step's fragments one step ahead: they only depend
+        // on the item table, and the step's own chain (key -> descriptor record and position -> arithmetic -> store)
+        // is then one memory round trip shorter (per-pixel backward kernel of a 1080p frame 247 -> 237 us). With one
+        // fragment per point and layer it gains nothing at one view and costs 4 % at four (measured), so there the
+        // step asks for its own.
+        int p_next = -1;
+        uint32_t low_next = 0;
+        float T_next      = 0.f;
+        auto fetch = [&](int k0) {
             const uint32_t k = (uint32_t)k0 + lane;
-            const bool valid = k < total;
-            const int p      = valid ? (int)s_item[wave][k] : -1;  // lane of the pixel this fragment belongs to
-            float x = 0.f, T = 0.f, c = 0.f, dot = 0.f;
+            p_next           = k < total ? (int)s_item[wave][k] : -1;  // lane of the pixel this fragment belongs to
+            if (p_next >= 0)
+            {
+                const uint32_t pos = s_off[wave][p_next] + jw + (k - s_base[wave][p_next]);
+                low_next           = (uint32_t)a.fragments[pos];
+                T_next             = a.transmittance[pos];
+            }
+        };
+        const int k_first = total > 0 ? (int)((total - 1) / kWave) * kWave : -1;
+        if (BILINEAR && k_first >= 0) fetch(k_first);
+        for (int k0 = k_first; k0 >= 0; k0 -= kWave)
+        {
+            if constexpr (!BILINEAR) fetch(k0);
+            const int p        = p_next;
+            const bool valid   = p >= 0;
+            const uint32_t low = low_next;
+            float x = 0.f, T = T_next, c = 0.f, dot = 0.f;
+            if (BILINEAR && k0 >= kWave) fetch(k0 - kWave);
             float t[4] = {0.f, 0.f, 0.f, 0.f};
             float4 g4  = make_float4(0.f, 0.f, 0.f, 0.f);
             int id = -1, ti = -1, corner = 0;
             if (valid)
             {
-                const uint32_t pos = s_off[wave][p] + jw + (k - s_base[wave][p]);
-                const uint32_t low = (uint32_t)a.fragments[pos];
                 id                 = BILINEAR ? (int)(low >> 2) : (int)low;
                 corner             = BILINEAR ? (int)(low & 3u) : 0;
-                T                  = a.transmittance[pos];
                 // guards the gathers; never false for a workspace the forward pass wrote
                 if ((uint32_t)id < (uint32_t)a.N) ti = a.index ? a.index[id] : id;
                 if ((uint32_t)ti >= (uint32_t)a.N) ti = -1;
